@@ -1,0 +1,353 @@
+"""CPU oracle for the ringattention hot path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, loop for loop, the algorithm of the reference's
+``ringattention/ringattention_jax.py`` with torch-CPU tensors.  It exists to
+check the HIP kernels; nothing in the shipped package may import it.  Only the
+tests, the smoke entry and the ``cpu_baseline`` leg of the benchmark use it.
+
+How the oracle itself is pinned (the reference ships no tests or golden
+vectors, and JAX/flax are not importable where this was written):
+
+* forward (``blockwise_attention_fwd`` / ``ring_attention_fwd``): checked in
+  float64 against ``dense_attention`` below, an independent un-chunked softmax
+  whose mask is built from global positions, on sweeps of chunk sizes, ring
+  sizes, causal block sizes, segment ids, biases and cache_idx values.
+* backward: checked against ``torch.autograd`` of ``dense_attention`` and
+  against float64 finite differences.
+* ``below_or_on_diag``: exhaustive integer tables against the brute-force
+  "tile holds an unmasked pair" test where they must agree, and against the
+  enumerated off-by-one cases where they must not.
+* ``chunk_attention_bias``: case enumeration (bias / segment / causal / all),
+  the ``min(bias, 0)`` clamp and the two ``finfo.min`` constants.
+* ``blockwise_feedforward``: equals the un-chunked feed-forward; SwiGLU
+  backward is torch autograd.
+
+Parity unpinned (would need the reference's own runtime): the dropout mask
+bits (``jax.random`` stream) - dropout is refused - and XLA-CPU's exact
+summation order / its bf16 rounding of intermediate einsum results, both far
+below the stated tolerances.
+
+Layout: q/k/v/out/grads ``(B, S, H, D)``; softmax statistics ``(B, H, S)``.
+"""
+import math
+
+import torch
+
+_FINFO_MIN = {
+    torch.float32: torch.finfo(torch.float32).min,    # -3.4028235e38
+    torch.bfloat16: torch.finfo(torch.bfloat16).min,  # -3.3895314e38
+    torch.float16: torch.finfo(torch.float16).min,    # -65504
+    torch.float64: torch.finfo(torch.float64).min,
+}
+
+
+def finfo_min(dtype):
+    return _FINFO_MIN[dtype]
+
+
+def below_or_on_diag(r, r_blk_size, c, c_blk_size, causal_block_size):
+    """ringattention_jax.py:324-331.  Pure integer predicate on global chunk indices."""
+    cq = max(causal_block_size, r_blk_size)
+    ck = max(causal_block_size, c_blk_size)
+    r = r // (cq // r_blk_size)
+    c = c // (ck // c_blk_size)
+    return ((r + 1) * cq - 1) > (c * ck)
+
+
+def _dynamic_slice_start(start, size, dim):
+    # lax.dynamic_slice clamps the start so the slice stays in range.
+    return max(0, min(start, dim - size))
+
+
+def chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
+                         causal_block_size, dtype, query_chunk_idx, key_chunk_idx,
+                         work_dtype=torch.float32):
+    """ringattention_jax.py:272-322 without the dropout branch (:311-321).
+
+    Returns the additive tile, broadcastable to (B, H, qc, kc), holding values
+    representable in ``dtype`` but stored in ``work_dtype``.
+    """
+    query_offset = query_chunk_idx * query_chunk_size
+    key_offset = key_chunk_idx * key_chunk_size
+    fmin = finfo_min(dtype)
+    chunk_bias = torch.zeros((1, 1, 1, 1), dtype=work_dtype)
+    if bias is not None:                                                   # :278-283
+        qs = min(bias.shape[-2], query_chunk_size)
+        ks = min(bias.shape[-1], key_chunk_size)
+        k0 = _dynamic_slice_start(key_offset, ks, bias.shape[-1])
+        chunk_bias = bias[:, :, 0:qs, k0:k0 + ks].to(work_dtype)
+    if segment_ids is not None:                                            # :285-299
+        q0 = _dynamic_slice_start(query_offset, query_chunk_size, segment_ids.shape[1])
+        k0 = _dynamic_slice_start(key_offset, key_chunk_size, segment_ids.shape[1])
+        q_seg = segment_ids[:, q0:q0 + query_chunk_size]
+        k_seg = segment_ids[:, k0:k0 + key_chunk_size]
+        neq = ~torch.eq(q_seg[:, :, None], k_seg[:, None, :])
+        seg_bias = neq[:, None].to(work_dtype) * fmin
+        chunk_bias = torch.minimum(chunk_bias, seg_bias)
+    if causal_block_size is not None:                                      # :301-309
+        q_idx = (torch.arange(query_chunk_size).reshape(-1, 1) + query_offset) // causal_block_size
+        k_idx = (torch.arange(key_chunk_size).reshape(1, -1) + key_offset) // causal_block_size
+        causal = (q_idx < k_idx).to(work_dtype) * fmin
+        chunk_bias = torch.minimum(chunk_bias, causal.reshape(1, 1, *causal.shape))
+    # :322  .astype(dtype): round to the kwargs dtype, then carry on in work_dtype
+    if dtype in (torch.bfloat16, torch.float16):
+        chunk_bias = chunk_bias.to(dtype).to(work_dtype)
+    return chunk_bias
+
+
+def _check_no_dropout(deterministic, attn_pdrop):
+    if (not deterministic) and attn_pdrop > 0.0:
+        raise NotImplementedError("attention dropout draws from the jax.random stream; not restated")
+
+
+def blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_start, bias, segment_ids,
+                            causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
+                            dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
+                            precision=None, prevent_cse=True, cache_idx=None):
+    """ringattention_jax.py:99-179.  q/k/v already in the working dtype; returns the new carry."""
+    _check_no_dropout(deterministic, attn_pdrop)
+    batch, q_len, num_heads, dim = q.shape
+    kv_len = k.shape[1]
+    num_q = q_len // query_chunk_size
+    num_kv = kv_len // key_chunk_size
+    wd = q.dtype
+    numerator, denominator, max_score = (x.clone() for x in carry)
+    scale = math.sqrt(dim)                                                  # :118
+    for qi in range(num_q):                                                 # :171
+        qs = slice(qi * query_chunk_size, (qi + 1) * query_chunk_size)
+        q_chunk = q[:, qs]
+        num_c = numerator[:, qs]
+        den_c = denominator[:, :, qs]
+        max_c = max_score[:, :, qs]
+        for ki in range(num_kv):                                            # :166-168
+            if causal_block_size is not None and not below_or_on_diag(
+                    q_chunk_idx_start + qi, query_chunk_size,
+                    k_chunk_idx_start + ki, key_chunk_size, causal_block_size):
+                continue                                                    # :158-164 identity
+            ks = slice(ki * key_chunk_size, (ki + 1) * key_chunk_size)
+            k_chunk, v_chunk = k[:, ks], v[:, ks].to(wd)
+            w = torch.einsum('bqhd,bkhd->bhqk', q_chunk, k_chunk) / scale   # :134
+            w = w + chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
+                                         causal_block_size, dtype, q_chunk_idx_start + qi,
+                                         k_chunk_idx_start + ki, work_dtype=wd)  # :135-136
+            new_max = torch.maximum(max_c, w.max(dim=-1).values)            # :138
+            e = torch.exp(w - new_max[..., None])                           # :140
+            ev = torch.einsum('bhqk,bkhd->bqhd', e, v_chunk)                # :141
+            corr = torch.exp(max_c - new_max)                               # :142
+            num_c = num_c * corr.permute(0, 2, 1)[..., None] + ev           # :143
+            den_c = den_c * corr + e.sum(dim=-1)                            # :144
+            max_c = new_max
+        numerator[:, qs] = num_c
+        denominator[:, :, qs] = den_c
+        max_score[:, :, qs] = max_c
+    return numerator, denominator, max_score
+
+
+def blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_start, bias, segment_ids,
+                            causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
+                            dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
+                            precision=None, prevent_cse=True, cache_idx=None):
+    """ringattention_jax.py:181-270.  Adds this block's gradients into the incoming dq/dk/dv."""
+    _check_no_dropout(deterministic, attn_pdrop)
+    batch, q_len, num_heads, dim = q.shape
+    kv_len = k.shape[1]
+    num_q = q_len // query_chunk_size
+    num_kv = kv_len // key_chunk_size
+    wd = q.dtype
+    dq, dk, dv, output, denominator, max_score = carry
+    dq, dk, dv = dq.clone(), dk.clone(), dv.clone()
+    g = g.to(wd)
+    scale = math.sqrt(dim)
+    for qi in range(num_q):                                                 # :263
+        qs = slice(qi * query_chunk_size, (qi + 1) * query_chunk_size)
+        q_chunk, g_chunk = q[:, qs], g[:, qs]
+        den_c, max_c = denominator[:, :, qs], max_score[:, :, qs]
+        dl_part = torch.einsum('bqhd,bqhd->bhq', g_chunk, output[:, qs].to(wd))[..., None]  # :218
+        dq_c = dq[:, qs]
+        for ki in range(num_kv):                                            # :259-261
+            if causal_block_size is not None and not below_or_on_diag(
+                    q_chunk_idx_start + qi, query_chunk_size,
+                    k_chunk_idx_start + ki, key_chunk_size, causal_block_size):
+                continue                                                    # :246-257 zero dk/dv part
+            ks = slice(ki * key_chunk_size, (ki + 1) * key_chunk_size)
+            k_chunk, v_chunk = k[:, ks], v[:, ks].to(wd)
+            w = torch.einsum('bqhd,bkhd->bhqk', q_chunk, k_chunk) / scale   # :223
+            w = w + chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
+                                         causal_block_size, dtype, q_chunk_idx_start + qi,
+                                         k_chunk_idx_start + ki, work_dtype=wd)  # :224-225
+            p = torch.exp(w - max_c[..., None]) / den_c[..., None]          # :226
+            ds = torch.einsum('bqhd,bkhd->bhqk', g_chunk, v_chunk)          # :228
+            dl = (ds - dl_part) * p                                         # :229
+            dq_c = dq_c + torch.einsum('bhqk,bkhd->bqhd', dl, k_chunk) / scale      # :230
+            dk[:, ks] += torch.einsum('bqhd,bhqk->bkhd', q_chunk, dl) / scale       # :231,:262
+            dv[:, ks] += torch.einsum('bhqk,bqhd->bkhd', p, g_chunk)                # :232,:262
+        dq[:, qs] = dq_c
+    return dq, dk, dv
+
+
+def _work_dtype(q, float32_logits, compute_dtype):
+    if compute_dtype is not None:
+        return compute_dtype
+    return torch.float32 if (float32_logits or q.dtype == torch.float32) else torch.float32
+
+
+def ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, float32_logits,
+                       blockwise_kwargs, compute_dtype=None):
+    """ringattention_jax.py:17-53 executed for every device of a ring of ``axis_size``.
+
+    q/k/v are the *global* arrays (what the caller of shard_map holds); device i
+    owns the i-th contiguous slice of the sequence axis.  ``attn_bias`` and
+    ``segment_ids`` are replicated.  The ppermute (:47) is replaced by indexing
+    the shard that would have arrived at step idx, which is (i - idx) % N (:36).
+    Returns (out in v.dtype, residuals) with residuals in the working dtype.
+    """
+    wd = _work_dtype(q, float32_logits, compute_dtype)
+    n = axis_size
+    qw, kw = q.to(wd), k.to(wd)                                            # :18-19
+    batch, q_total, num_heads, dim = q.shape
+    kv_total = k.shape[1]
+    q_len, kv_len = q_total // n, kv_total // n
+    qc, kc = blockwise_kwargs["query_chunk_size"], blockwise_kwargs["key_chunk_size"]
+    outs, dens, maxs = [], [], []
+    for dev in range(n):
+        q_d = qw[:, dev * q_len:(dev + 1) * q_len]
+        num = torch.zeros((batch, q_len, num_heads, dim), dtype=wd)         # :22
+        den = torch.zeros((batch, num_heads, q_len), dtype=wd)              # :23
+        mx = torch.full((batch, num_heads, q_len), -math.inf, dtype=wd)     # :49
+        for idx in range(n):                                                # :50-51
+            if cache_idx is None:
+                q_start = dev * (q_len // qc)                               # :32-33
+            else:
+                q_start = cache_idx // qc                                   # :35
+            k_blk = (dev - idx) % n                                         # :36
+            k_start = k_blk * (kv_len // kc)                                # :37
+            ksl = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            num, den, mx = blockwise_attention_fwd(
+                q_d, kw[:, ksl], v[:, ksl], (num, den, mx), q_start, k_start,
+                bias=attn_bias, segment_ids=segment_ids, cache_idx=cache_idx, **blockwise_kwargs)
+        outs.append(num / den.permute(0, 2, 1)[..., None])                  # :52
+        dens.append(den)
+        maxs.append(mx)
+    output = torch.cat(outs, dim=1)
+    denominator = torch.cat(dens, dim=2)
+    max_score = torch.cat(maxs, dim=2)
+    res = (output, qw, kw, v, attn_bias, segment_ids, cache_idx, denominator, max_score)
+    return output.to(v.dtype), res
+
+
+def ring_attention_bwd(axis_size, float32_logits, blockwise_kwargs, res, g):
+    """ringattention_jax.py:55-90 for every device of the ring; returns global dq, dk, dv."""
+    output, q, k, v, attn_bias, segment_ids, cache_idx, denominator, max_score = res
+    wd = q.dtype
+    n = axis_size
+    batch, q_total, num_heads, dim = q.shape
+    kv_total = k.shape[1]
+    q_len, kv_len = q_total // n, kv_total // n
+    qc, kc = blockwise_kwargs["query_chunk_size"], blockwise_kwargs["key_chunk_size"]
+    dq = torch.zeros_like(q)                                               # :61
+    dk = torch.zeros_like(k)                                               # :62
+    dv = torch.zeros(v.shape, dtype=wd)                                    # :63
+    for dev in range(n):
+        qsl = slice(dev * q_len, (dev + 1) * q_len)
+        for idx in range(n):                                                # :88
+            q_start = dev * (q_len // qc) if cache_idx is None else cache_idx // qc   # :69-73
+            k_blk = (dev - idx) % n                                         # :74
+            k_start = k_blk * (kv_len // kc)                                # :75
+            ksl = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            # dk/dv partials travel with their K/V shard (:85-86): accumulate at the shard's home.
+            dq_d, dk_s, dv_s = blockwise_attention_bwd(
+                q[:, qsl], k[:, ksl], v[:, ksl], g[:, qsl],
+                (dq[:, qsl], dk[:, ksl], dv[:, ksl], output[:, qsl], denominator[:, :, qsl],
+                 max_score[:, :, qsl]),
+                q_start, k_start, bias=attn_bias, segment_ids=segment_ids, cache_idx=cache_idx,
+                **blockwise_kwargs)
+            dq[:, qsl], dk[:, ksl], dv[:, ksl] = dq_d, dk_s, dv_s
+    return dq, dk, dv
+
+
+def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, float32_logits,
+                   blockwise_kwargs, compute_dtype=None):
+    """Forward value only (ringattention_jax.py:92-95)."""
+    return ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, float32_logits,
+                              blockwise_kwargs, compute_dtype)[0]
+
+
+def dense_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, blockwise_kwargs,
+                    compute_dtype=torch.float64):
+    """Independent closed form: softmax(Q K^T / sqrt(D) + B_eff) V on the global arrays.
+
+    B_eff is built from global positions, not chunk by chunk: pairs in tiles the
+    skip predicate drops are -inf; pairs masked by segment/causal inside a tile
+    that runs are finfo(dtype).min; the rest get the bias, clamped to <= 0
+    whenever a mask feature is on (the minimum() of ringattention_jax.py:299,309).
+    Differentiable with torch.autograd.
+    """
+    wd = compute_dtype
+    qc, kc = blockwise_kwargs["query_chunk_size"], blockwise_kwargs["key_chunk_size"]
+    cbs = blockwise_kwargs["causal_block_size"]
+    dtype = blockwise_kwargs.get("dtype", torch.float32)
+    fmin = finfo_min(dtype)
+    batch, q_total, num_heads, dim = q.shape
+    kv_total = k.shape[1]
+    n = axis_size
+    q_len = q_total // n
+    # global positions of every local query row / key column
+    loc_q = torch.arange(q_total) % q_len
+    dev_q = torch.arange(q_total) // q_len
+    if cache_idx is None:
+        q_chunk = dev_q * (q_len // qc) + loc_q // qc
+    else:
+        q_chunk = cache_idx // qc + loc_q // qc
+    g_q = q_chunk * qc + loc_q % qc
+    g_k = torch.arange(kv_total)
+    k_chunk = g_k // kc
+    logits = torch.einsum('bqhd,bkhd->bhqk', q.to(wd), k.to(wd)) / math.sqrt(dim)
+    any_mask = (segment_ids is not None) or (cbs is not None)
+    add = torch.zeros((1, 1, 1, 1), dtype=wd)
+    if attn_bias is not None:
+        b = attn_bias.to(wd)
+        if b.shape[-2] != 1:
+            # the reference always slices query rows 0:qc of the bias (:281)
+            b = b[:, :, (loc_q % qc), :]
+        if b.shape[-1] == 1:
+            b = b.expand(*b.shape[:3], kv_total)
+        add = b
+        if any_mask:
+            add = torch.clamp(add, max=0.0)
+    add = add.expand(-1, -1, q_total if add.shape[2] != 1 else 1, kv_total if add.shape[3] != 1 else 1)
+    if dtype in (torch.bfloat16, torch.float16):
+        add = add.to(dtype).to(wd)
+    masked = torch.zeros((1, 1, q_total, kv_total), dtype=torch.bool)
+    if segment_ids is not None:
+        masked = masked | (segment_ids[:, g_q][:, None, :, None] != segment_ids[:, g_k][:, None, None, :])
+    if cbs is not None:
+        masked = masked | ((g_q // cbs)[:, None] < (g_k // cbs)[None, :])[None, None]
+    logits = logits + add
+    logits = torch.where(masked, torch.full((), fmin, dtype=wd), logits)
+    if cbs is not None:
+        cq, ck = max(cbs, qc), max(cbs, kc)
+        r = q_chunk // (cq // qc)
+        c = k_chunk // (ck // kc)
+        run = ((r[:, None] + 1) * cq - 1) > (c[None, :] * ck)
+        logits = torch.where(run[None, None], logits, torch.full((), -math.inf, dtype=wd))
+    p = torch.softmax(logits, dim=-1)      # all -inf rows -> NaN, as 0/0 in the reference (:52)
+    return torch.einsum('bhqk,bkhd->bqhd', p, v.to(wd))
+
+
+def swiglu(x, w1, w2, w3):
+    """The caller-side SwiGLU MLP the reference's blockwise_feedforward is used with:
+    w2( silu(x w1) * (x w3) ), weights stored (in, out)."""
+    a = x @ w1
+    b = x @ w3
+    return (torch.nn.functional.silu(a) * b) @ w2
+
+
+def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), policy=None, pre_remat=True):
+    """ringattention_jax.py:333-352.  'b (c n) d -> b c n d' with c=chunk_size, scanned over n:
+    each step feeds chunk_size tokens {ci*n + j : ci} to ``feedforward``."""
+    b, s, d = inputs.shape
+    n = s // chunk_size
+    x = inputs.reshape(b, chunk_size, n, d)                                 # :339
+    outs = [feedforward(x[:, :, j, :]) for j in range(n)]                   # :340-350
+    out = torch.stack(outs, dim=2)
+    return out.reshape(b, s, out.shape[-1])                                 # :351

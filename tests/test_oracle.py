@@ -1,0 +1,337 @@
+"""Pins the CPU oracle against what the mathematics fixes: an independent dense softmax in
+float64, torch.autograd / finite differences for the backward, exhaustive integer tables for the
+skip predicate, and case enumeration for the bias builder."""
+import itertools
+import math
+
+import pytest
+import torch
+
+from oracle import ringattention_oracle as O
+
+F64 = torch.float64
+
+
+def kwargs(qc, kc, cbs=1, dtype=torch.float32):
+    return dict(causal_block_size=cbs, deterministic=True, dropout_rng=None, attn_pdrop=0.0,
+                query_chunk_size=qc, key_chunk_size=kc, dtype=dtype, policy=None, precision=None,
+                prevent_cse=True)
+
+
+def make(B, S, H, D, seed=0, dtype=F64, Skv=None):
+    g = torch.Generator().manual_seed(seed)
+    Skv = S if Skv is None else Skv
+    q = torch.randn(B, S, H, D, generator=g, dtype=dtype)
+    k = torch.randn(B, Skv, H, D, generator=g, dtype=dtype)
+    v = torch.randn(B, Skv, H, D, generator=g, dtype=dtype)
+    return q, k, v
+
+
+def seg_ids(B, S, seed=1, mean=7):
+    g = torch.Generator().manual_seed(seed)
+    out = torch.zeros(B, S, dtype=torch.int32)
+    for b in range(B):
+        pos, doc = 0, 0
+        while pos < S:
+            ln = int(torch.randint(1, 2 * mean, (1,), generator=g))
+            out[b, pos:pos + ln] = doc
+            pos += ln
+            doc += 1
+    return out
+
+
+# ----------------------------------------------------------------------------- predicate
+
+def brute_tile_has_unmasked(r, qc, c, kc, cbs):
+    for i in range(r * qc, (r + 1) * qc):
+        for j in range(c * kc, (c + 1) * kc):
+            if not (i // cbs < j // cbs):
+                return True
+    return False
+
+
+@pytest.mark.parametrize("blk", [2, 3, 4, 8])
+@pytest.mark.parametrize("cbs", [1, 2, 4, 8, 16])
+def test_predicate_equal_chunks_matches_bruteforce(blk, cbs):
+    if cbs > blk and cbs % blk:
+        pytest.skip("causal block must be a multiple of the chunk")
+    if cbs < blk and blk % cbs:
+        pytest.skip("chunk must be a multiple of the causal block")
+    for r in range(12):
+        for c in range(12):
+            assert bool(O.below_or_on_diag(r, blk, c, blk, cbs)) == brute_tile_has_unmasked(r, blk, c, blk, cbs), (r, c)
+
+
+def test_predicate_off_by_one_cases():
+    # chunk sizes (1,1): the strict '>' drops every diagonal tile
+    for r in range(8):
+        assert not O.below_or_on_diag(r, 1, r, 1, 1)
+        if r:
+            assert O.below_or_on_diag(r, 1, r - 1, 1, 1)
+    # decode shape (1,512): the query's own key chunk runs unless q_pos % 512 == 0
+    for pos in [0, 1, 511, 512, 513, 1024, 1500]:
+        own = pos // 512
+        assert bool(O.below_or_on_diag(pos, 1, own, 512, 1)) == (pos % 512 != 0)
+        if own:
+            assert O.below_or_on_diag(pos, 1, own - 1, 512, 1)
+        assert not O.below_or_on_diag(pos, 1, own + 1, 512, 1)
+
+
+def test_predicate_closed_form_unequal_chunks():
+    # with cbs=1 the predicate is "last row of the q chunk is strictly past the first key of the k chunk"
+    for qc, kc in [(2, 4), (4, 2), (8, 2), (2, 8), (3, 5)]:
+        for r in range(10):
+            for c in range(10):
+                assert bool(O.below_or_on_diag(r, qc, c, kc, 1)) == ((r + 1) * qc - 1 > c * kc)
+
+
+# ----------------------------------------------------------------------------- bias builder
+
+def test_chunk_bias_cases():
+    qc, kc = 4, 4
+    bias = torch.tensor([0.5, -1.0, 2.0, -3.0, 1.0, -0.25, 0.0, 4.0]).reshape(1, 1, 1, 8)
+    seg = torch.tensor([[0, 0, 0, 1, 1, 1, 2, 2]], dtype=torch.int32)
+    fmin32 = torch.finfo(torch.float32).min
+    # bias only: passed through unclamped, sliced at the global key offset
+    t = O.chunk_attention_bias(qc, kc, bias, None, None, torch.float32, 0, 1)
+    assert torch.equal(t, bias[..., 4:8])
+    # nothing at all: a single zero
+    t = O.chunk_attention_bias(qc, kc, None, None, None, torch.float32, 1, 0)
+    assert t.shape == (1, 1, 1, 1) and float(t) == 0.0
+    # causal only, diagonal tile
+    t = O.chunk_attention_bias(qc, kc, None, None, 1, torch.float32, 1, 1)
+    exp = torch.triu(torch.ones(4, 4), diagonal=1) * fmin32
+    assert torch.equal(t[0, 0], exp)
+    # segment + bias: allowed -> min(bias, 0), masked -> finfo.min
+    t = O.chunk_attention_bias(qc, kc, bias, seg, None, torch.float32, 0, 1)
+    for i in range(4):
+        for j in range(4):
+            if seg[0, i] == seg[0, 4 + j]:
+                assert float(t[0, 0, i, j]) == min(float(bias[0, 0, 0, 4 + j]), 0.0)
+            else:
+                assert float(t[0, 0, i, j]) == fmin32
+    # everything, bf16 kwargs dtype: mask value is the bf16 minimum and the bias is rounded to bf16
+    b2 = torch.tensor([-1.001, -2.003, 0.3, -0.7]).reshape(1, 1, 1, 4)
+    t = O.chunk_attention_bias(qc, kc, b2, seg[:, :4], 1, torch.bfloat16, 0, 0)
+    assert float(t[0, 0, 0, 1]) == torch.finfo(torch.bfloat16).min
+    assert float(t[0, 0, 1, 0]) == float(torch.tensor(-1.001).bfloat16())
+    assert float(t[0, 0, 2, 2]) == 0.0   # positive bias clamped
+    assert abs(torch.finfo(torch.bfloat16).min - (-3.3895314e38)) < 1e32
+    assert abs(torch.finfo(torch.float32).min - (-3.4028235e38)) < 1e31
+
+
+def test_chunk_bias_causal_block_size():
+    t = O.chunk_attention_bias(4, 4, None, None, 2, torch.float32, 1, 1)
+    # positions 4..7, blocks of 2: (4,5) see (4,5); (6,7) see (4..7)
+    exp_masked = torch.tensor([[0, 0, 1, 1], [0, 0, 1, 1], [0, 0, 0, 0], [0, 0, 0, 0]], dtype=torch.bool)
+    assert torch.equal(t[0, 0] != 0, exp_masked)
+
+
+# ----------------------------------------------------------------------------- forward vs dense
+
+FWD_CASES = [
+    # B,S,H,D,qc,kc,cbs,N,use_bias,use_seg
+    (1, 32, 2, 8, 8, 8, 1, 1, False, False),
+    (2, 32, 2, 8, 8, 8, 1, 1, True, True),
+    (1, 32, 1, 4, 4, 8, 1, 1, True, False),
+    (1, 32, 1, 4, 8, 4, 1, 2, False, True),
+    (2, 48, 2, 8, 4, 4, 1, 3, True, True),
+    (1, 64, 2, 8, 8, 8, 1, 4, True, True),
+    (1, 64, 1, 8, 8, 8, 4, 2, True, True),
+    (1, 64, 1, 8, 4, 4, 8, 2, False, False),
+    (1, 64, 1, 8, 16, 8, 2, 1, True, False),
+    (1, 32, 2, 8, 8, 8, None, 1, True, True),
+    (1, 32, 2, 8, 8, 8, None, 2, True, False),
+    (1, 32, 2, 8, 8, 8, None, 1, False, False),
+    (1, 16, 1, 4, 2, 2, 1, 1, False, False),
+]
+
+
+@pytest.mark.parametrize("case", FWD_CASES)
+def test_forward_matches_dense(case):
+    B, S, H, D, qc, kc, cbs, N, use_bias, use_seg = case
+    q, k, v = make(B, S, H, D, seed=S + H)
+    g = torch.Generator().manual_seed(5)
+    bias = torch.randn(B, 1, 1, S, generator=g, dtype=F64) if use_bias else None
+    seg = seg_ids(B, S) if use_seg else None
+    kw = kwargs(qc, kc, cbs)
+    out, res = O.ring_attention_fwd(q, k, v, bias, seg, None, N, True, kw, compute_dtype=F64)
+    ref = O.dense_attention(q, k, v, bias, seg, None, N, kw)
+    assert torch.allclose(out, ref, atol=1e-12, rtol=1e-10)
+    # softmax statistics: den * exp(max) is the dense partition function
+    assert torch.isfinite(res[-1]).all() and (res[-2] > 0).all()
+
+
+def test_forward_ring_and_chunk_invariance():
+    q, k, v = make(1, 64, 2, 8, seed=3)
+    seg = seg_ids(1, 64)
+    base = O.ring_attention(q, k, v, None, seg, None, 1, True, kwargs(8, 8), compute_dtype=F64)
+    for N, qc, kc in [(2, 8, 8), (4, 8, 8), (8, 8, 8), (1, 16, 4), (2, 4, 16), (1, 2, 32)]:
+        o = O.ring_attention(q, k, v, None, seg, None, N, True, kwargs(qc, kc), compute_dtype=F64)
+        assert torch.allclose(o, base, atol=1e-12), (N, qc, kc)
+
+
+def test_rows_sum_to_one_and_head_batch_equivariance():
+    q, k, v = make(2, 32, 3, 8, seed=9)
+    ones = torch.ones_like(v)
+    o = O.ring_attention(q, k, ones, None, None, None, 2, True, kwargs(8, 8), compute_dtype=F64)
+    assert torch.allclose(o, ones, atol=1e-13)
+    perm_b, perm_h = [1, 0], [2, 0, 1]
+    o1 = O.ring_attention(q, k, v, None, None, None, 2, True, kwargs(8, 8), compute_dtype=F64)
+    o2 = O.ring_attention(q[perm_b][:, :, perm_h], k[perm_b][:, :, perm_h], v[perm_b][:, :, perm_h],
+                          None, None, None, 2, True, kwargs(8, 8), compute_dtype=F64)
+    assert torch.equal(o1[perm_b][:, :, perm_h], o2)
+
+
+def test_positive_bias_is_clamped_only_with_masks():
+    q, k, v = make(1, 16, 1, 4, seed=2)
+    bias = torch.full((1, 1, 1, 16), 3.0, dtype=F64)
+    bias[..., ::2] = -1.0
+    kw_nomask = kwargs(4, 4, None)
+    a = O.ring_attention(q, k, v, bias, None, None, 1, True, kw_nomask, compute_dtype=F64)
+    b = O.ring_attention(q, k, v, torch.clamp(bias, max=0.0), None, None, 1, True, kw_nomask, compute_dtype=F64)
+    assert not torch.allclose(a, b)
+    kw = kwargs(4, 4, 1)
+    a = O.ring_attention(q, k, v, bias, None, None, 1, True, kw, compute_dtype=F64)
+    b = O.ring_attention(q, k, v, torch.clamp(bias, max=0.0), None, None, 1, True, kw, compute_dtype=F64)
+    assert torch.equal(a, b)
+
+
+def test_masked_keys_are_bitwise_isolated():
+    q, k, v = make(1, 32, 2, 8, seed=4, dtype=torch.float32)
+    kw = kwargs(8, 8, 1)
+    a = O.ring_attention(q, k, v, None, None, None, 2, True, kw)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, 20:] += 100.0
+    v2[:, 20:] -= 50.0
+    b = O.ring_attention(q, k2, v2, None, None, None, 2, True, kw)
+    assert torch.equal(a[:, :20], b[:, :20])
+
+
+def test_fully_masked_then_real_is_annihilated_exactly():
+    # key chunk 0 belongs to another segment: the row first sees uniform weights, then exactly none of it
+    q, k, v = make(1, 8, 1, 4, seed=6, dtype=torch.float32)
+    seg = torch.tensor([[0, 0, 0, 0, 1, 1, 1, 1]], dtype=torch.int32)
+    kw = kwargs(4, 4, 1)
+    a = O.ring_attention(q, k, v, None, seg, None, 1, True, kw)
+    b = O.ring_attention(q[:, 4:], k[:, 4:], v[:, 4:], None, None, None, 1, True, kw)
+    assert torch.equal(a[:, 4:], b)
+
+
+# ----------------------------------------------------------------------------- decode (cache_idx)
+
+@pytest.mark.parametrize("cache_idx", [1, 5, 8, 13, 16, 23])
+def test_decode_matches_dense_and_prefill_row(cache_idx):
+    L, kc = 32, 8
+    q, k, v = make(2, L, 2, 8, seed=11)
+    kw = kwargs(1, kc, 1)
+    q1 = q[:, cache_idx:cache_idx + 1]
+    out = O.ring_attention(q1, k, v, None, None, cache_idx, 1, True, kw, compute_dtype=F64)
+    ref = O.dense_attention(q1, k, v, None, None, cache_idx, 1, kw)
+    assert torch.allclose(out, ref, atol=1e-12)
+    # keys attended: 0..cache_idx, minus the own chunk when cache_idx % kc == 0 (the strict '>')
+    last = cache_idx if cache_idx % kc else cache_idx - 1
+    w = torch.einsum('bqhd,bkhd->bhqk', q1, k[:, :last + 1]) / math.sqrt(8)
+    exp = torch.einsum('bhqk,bkhd->bqhd', torch.softmax(w, -1), v[:, :last + 1])
+    assert torch.allclose(out, exp, atol=1e-12)
+    if cache_idx % kc:
+        pre = O.ring_attention(q, k, v, None, None, None, 1, True, kwargs(8, kc, 1), compute_dtype=F64)
+        assert torch.allclose(out[:, 0], pre[:, cache_idx], atol=1e-12)
+
+
+def test_decode_at_zero_is_nan():
+    q, k, v = make(1, 8, 1, 4, seed=1)
+    out = O.ring_attention(q[:, :1], k, v, None, None, 0, 1, True, kwargs(1, 4, 1), compute_dtype=F64)
+    assert torch.isnan(out).all()
+
+
+# ----------------------------------------------------------------------------- backward
+
+BWD_CASES = [
+    (1, 32, 2, 8, 8, 8, 1, 1, False, False),
+    (2, 32, 2, 8, 8, 8, 1, 2, True, True),
+    (1, 48, 1, 4, 4, 8, 1, 3, True, False),
+    (1, 64, 2, 8, 8, 4, 4, 2, True, True),
+    (1, 32, 2, 8, 8, 8, None, 2, True, True),
+    (1, 32, 1, 8, 16, 8, 1, 1, False, True),
+]
+
+
+@pytest.mark.parametrize("case", BWD_CASES)
+def test_backward_matches_autograd_of_dense(case):
+    B, S, H, D, qc, kc, cbs, N, use_bias, use_seg = case
+    q, k, v = make(B, S, H, D, seed=S)
+    gen = torch.Generator().manual_seed(8)
+    g = torch.randn(B, S, H, D, generator=gen, dtype=F64)
+    bias = torch.randn(B, 1, 1, S, generator=gen, dtype=F64) if use_bias else None
+    seg = seg_ids(B, S) if use_seg else None
+    kw = kwargs(qc, kc, cbs)
+    _, res = O.ring_attention_fwd(q, k, v, bias, seg, None, N, True, kw, compute_dtype=F64)
+    dq, dk, dv = O.ring_attention_bwd(N, True, kw, res, g)
+    qa, ka, va = (x.clone().requires_grad_(True) for x in (q, k, v))
+    ref = O.dense_attention(qa, ka, va, bias, seg, None, N, kw)
+    ref.backward(g)
+    for a, b in ((dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
+        assert torch.allclose(a, b, atol=1e-11, rtol=1e-9)
+
+
+def test_backward_finite_differences():
+    q, k, v = make(1, 8, 1, 4, seed=21)
+    gen = torch.Generator().manual_seed(3)
+    g = torch.randn(1, 8, 1, 4, generator=gen, dtype=F64)
+    kw = kwargs(4, 4, 1)
+    _, res = O.ring_attention_fwd(q, k, v, None, None, None, 2, True, kw, compute_dtype=F64)
+    dq, dk, dv = O.ring_attention_bwd(2, True, kw, res, g)
+
+    def f(q_, k_, v_):
+        return float((O.ring_attention(q_, k_, v_, None, None, None, 2, True, kw, compute_dtype=F64) * g).sum())
+    eps = 1e-6
+    for which, grad in ((0, dq), (1, dk), (2, dv)):
+        for idx in [(0, 1, 0, 2), (0, 5, 0, 0), (0, 7, 0, 3)]:
+            args = [q.clone(), k.clone(), v.clone()]
+            args[which][idx] += eps
+            up = f(*args)
+            args[which][idx] -= 2 * eps
+            dn = f(*args)
+            assert abs((up - dn) / (2 * eps) - float(grad[idx])) < 1e-6
+
+
+def test_backward_adds_into_incoming_gradients():
+    q, k, v = make(1, 16, 1, 4, seed=5)
+    kw = kwargs(4, 4, 1)
+    _, res = O.ring_attention_fwd(q, k, v, None, None, None, 1, True, kw, compute_dtype=F64)
+    out, qw, kw_, vv, _, _, _, den, mx = res
+    g = torch.ones_like(q)
+    z = torch.zeros_like(q)
+    a = O.blockwise_attention_bwd(qw, kw_, vv, g, (z, z, z, out, den, mx), 0, 0, None, None, **kw)
+    one = torch.ones_like(q)
+    b = O.blockwise_attention_bwd(qw, kw_, vv, g, (one, 2 * one, 3 * one, out, den, mx), 0, 0, None, None, **kw)
+    for i, (x, y) in enumerate(zip(a, b)):
+        assert torch.allclose(x + (i + 1), y, atol=1e-13)
+
+
+# ----------------------------------------------------------------------------- feed-forward
+
+def test_blockwise_feedforward_equals_unchunked_and_uses_strided_groups():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 24, 8, generator=g, dtype=F64)
+    w1, w3 = torch.randn(8, 20, generator=g, dtype=F64), torch.randn(8, 20, generator=g, dtype=F64)
+    w2 = torch.randn(20, 8, generator=g, dtype=F64)
+    seen = []
+
+    def ff(h):
+        seen.append(h.clone())
+        return O.swiglu(h, w1, w2, w3)
+    y = O.blockwise_feedforward(ff, x, 6)
+    assert torch.allclose(y, O.swiglu(x, w1, w2, w3), atol=1e-12)
+    assert len(seen) == 4 and seen[0].shape == (2, 6, 8)
+    # step j gets tokens {ci * n + j}: a strided set, n = S / chunk_size
+    assert torch.equal(seen[1], x[:, 1::4])
+
+
+def test_dropout_is_refused():
+    q, k, v = make(1, 8, 1, 4)
+    kw = kwargs(4, 4, 1)
+    kw.update(deterministic=False, attn_pdrop=0.1)
+    with pytest.raises(NotImplementedError):
+        O.ring_attention(q, k, v, None, None, None, 1, True, kw)
