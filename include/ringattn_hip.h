@@ -1,0 +1,171 @@
+/*
+ * C-ABI of libringattn_hip.so: the per-device hot path of ring attention with
+ * blockwise transformers, written for MI355X (gfx950).
+ *
+ * Every entry point enqueues work on the caller's HIP stream and returns; none
+ * allocates, frees, retains a pointer or synchronises the device.  All pointers
+ * are device pointers owned by the caller.  Return value: RA_OK or an RA_ERR_*
+ * code; ra_last_error() gives the text of the calling thread's last failure.
+ *
+ * Tensor layout (the reference's, ringattention/ringattention_jax.py:20-23):
+ *   q, k, v, out, gradients, numerator      (B, S, H, D), D contiguous, head stride D
+ *   denominator, max_score, delta           (B, H, S),    S contiguous
+ * Sequence and batch strides are explicit (in elements) so that a ring shard can
+ * be a slice of the caller's global array.
+ */
+#ifndef RINGATTN_HIP_H_
+#define RINGATTN_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* ra_stream_t; /* == hipStream_t */
+
+enum { RA_OK = 0, RA_ERR_INVALID = 1, RA_ERR_UNSUPPORTED = 2, RA_ERR_LAUNCH = 3 };
+enum { RA_F32 = 0, RA_BF16 = 1 };
+
+/* kernel family selector (ra_attn_*_params.impl) */
+enum {
+  RA_IMPL_AUTO = 0,    /* MFMA kernels when the shape allows, else the generic ones */
+  RA_IMPL_GENERIC = 1, /* fp32 vector-ALU kernels: any chunk sizes, fp32 or bf16 inputs */
+  RA_IMPL_MFMA = 2     /* bf16 MFMA kernels only; RA_ERR_UNSUPPORTED if the shape does not fit */
+};
+
+/*
+ * The additive-bias / mask description of one (ring step, device):
+ * what _chunk_attention_bias (ringattention_jax.py:272-322) and below_or_on_diag
+ * (:324-331) take, in global chunk coordinates.
+ */
+typedef struct ra_mask {
+  const float* bias;          /* nullable; values already rounded to blockwise_kwargs["dtype"] */
+  int64_t bias_stride_b;      /* element strides; 0 broadcasts that axis */
+  int64_t bias_stride_h;
+  int64_t bias_stride_q;      /* indexed by the row INSIDE the query chunk (:281 slices rows 0:qc) */
+  int64_t bias_stride_k;      /* indexed by the GLOBAL key position (:281) */
+  const int32_t* segment_ids; /* nullable; (B or 1, seg_len), indexed by GLOBAL positions (:286-295) */
+  int64_t seg_stride_b;
+  int32_t seg_len;
+  int32_t causal_block_size;  /* 0 = None */
+  int32_t query_chunk_size;
+  int32_t key_chunk_size;
+  int32_t q_chunk_idx_start;  /* :33 ; ignored when cache_idx is given */
+  int32_t k_chunk_idx_start;  /* :37 */
+  const int32_t* cache_idx;   /* nullable device scalar: q_chunk_idx_start = *cache_idx / query_chunk_size (:35) */
+  float mask_min;             /* finfo(blockwise_kwargs["dtype"]).min (:298,:308) */
+  int32_t skip_masked_tiles;  /* 1: kernels may also skip sub-tiles whose every pair is masked; exact
+                                 unless a query row has no unmasked key at all in the whole ring */
+} ra_mask;
+
+/* _blockwise_attention_fwd (ringattention_jax.py:99-179): one ring step on one device.
+ * Updates the carry (numerator, denominator, max_score) in place. */
+typedef struct ra_attn_fwd_params {
+  const void* q; const void* k; const void* v;
+  int32_t dtype;              /* RA_F32 | RA_BF16, of q, k and v */
+  int32_t B, Sq, Skv, H, D;
+  int64_t q_stride_b, q_stride_s;     /* elements */
+  int64_t kv_stride_b, kv_stride_s;
+  float* numerator;  int64_t num_stride_b, num_stride_s;   /* (B,Sq,H,D) fp32 */
+  float* denominator; float* max_score;                    /* (B,H,Sq) fp32 */
+  int64_t stat_stride_b, stat_stride_h;
+  ra_mask mask;
+  int32_t impl;
+  int32_t carry_is_initial;   /* 1: the carry holds (0, 0, -inf) by definition; kernels need not read it */
+} ra_attn_fwd_params;
+
+/* _blockwise_attention_bwd (ringattention_jax.py:181-270): adds this step's gradients into the
+ * fp32 accumulators dq (Sq side) and dk, dv (Skv side). */
+typedef struct ra_attn_bwd_params {
+  const void* q; const void* k; const void* v; const void* g;   /* g: cotangent of out, same dtype */
+  int32_t dtype;
+  int32_t B, Sq, Skv, H, D;
+  int64_t q_stride_b, q_stride_s;     /* q and g */
+  int64_t kv_stride_b, kv_stride_s;
+  const float* delta;                 /* (B,H,Sq): sum_d g*out (:218), from ra_attn_bwd_delta */
+  const float* denominator; const float* max_score;
+  int64_t stat_stride_b, stat_stride_h;
+  float* dq; int64_t dq_stride_b, dq_stride_s;
+  float* dk; float* dv; int64_t dkv_stride_b, dkv_stride_s;
+  ra_mask mask;
+  int32_t impl;
+} ra_attn_bwd_params;
+
+/* Carry initialisation (ringattention_jax.py:22-23,:49): numerator = 0, denominator = 0, max = -inf. */
+int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s,
+                       float* denominator, float* max_score, int64_t stat_stride_b, int64_t stat_stride_h,
+                       int32_t B, int32_t Sq, int32_t H, int32_t D, ra_stream_t stream);
+
+/* _blockwise_attention_fwd, ringattention_jax.py:99-179 (called at :38-46). */
+int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream);
+
+/* output = numerator / denominator, cast (ringattention_jax.py:52-53).  out_dtype RA_F32|RA_BF16. */
+int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_stride_s,
+                     const float* denominator, int64_t stat_stride_b, int64_t stat_stride_h,
+                     void* out, int32_t out_dtype, int64_t out_stride_b, int64_t out_stride_s,
+                     int32_t B, int32_t Sq, int32_t H, int32_t D, ra_stream_t stream);
+
+/* delta[b,h,s] = sum_d g*out (ringattention_jax.py:218).  g, out: same dtype, same strides. */
+int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t stride_b, int64_t stride_s,
+                      float* delta, int64_t stat_stride_b, int64_t stat_stride_h,
+                      int32_t B, int32_t Sq, int32_t H, int32_t D, ra_stream_t stream);
+
+/* _blockwise_attention_bwd, ringattention_jax.py:181-270 (called at :76-84). */
+int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream);
+
+/*
+ * Decode: the cache_idx path (ringattention_jax.py:31-35 with q_len == 1): one query token per
+ * batch row against the whole KV cache buffer, streamed once.  Same mask semantics as above with
+ * query_chunk_size == 1.  workspace: ra_decode_workspace_bytes() bytes of device memory.
+ */
+typedef struct ra_decode_params {
+  const void* q;              /* (B,1,H,D) */
+  const void* k; const void* v;   /* (B,L,H,D) cache buffers */
+  void* out;                  /* (B,1,H,D), same dtype */
+  int32_t dtype;
+  int32_t B, L, H, D;
+  int64_t q_stride_b, kv_stride_b, kv_stride_s, out_stride_b;
+  ra_mask mask;               /* query_chunk_size must be 1; cache_idx pointer or q_chunk_idx_start */
+  void* workspace; size_t workspace_bytes;
+  int32_t num_splits;         /* 0 = choose */
+} ra_decode_params;
+
+size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int32_t num_splits);
+int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream);
+
+/*
+ * SwiGLU feed-forward on one chunk of tokens, the body that blockwise_feedforward
+ * (ringattention_jax.py:333-352) scans: y = (silu(x w1) * (x w3)) w2, bf16, fp32 accumulation.
+ * x (T,d) ; w1,w3 (d,f) ; w2 (f,d) ; row-major.  a,b (T,f) bf16 are written by the forward
+ * (pre-activations, recomputed or kept by the caller) and read by the backward.
+ */
+typedef struct ra_swiglu_params {
+  int32_t T, d, f;
+  const void* x; const void* w1; const void* w2; const void* w3;
+  void* a; void* b; void* h;      /* (T,f) bf16 scratch: x w1, x w3, silu(a)*b */
+  void* y;                        /* (T,d) bf16 */
+  /* backward only */
+  const void* dy;                 /* (T,d) */
+  void* dx;                       /* (T,d) */
+  float* dw1; float* dw2; float* dw3;   /* fp32 accumulators, added into (weights are broadcast
+                                           over the scan, so their gradients sum over chunks) */
+  void* da; void* db;             /* (T,f) bf16 scratch */
+} ra_swiglu_params;
+
+int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream);
+int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream);
+
+/* C (M,N) = op(A) op(B), bf16 inputs, fp32 accumulation.  trans_a: A is stored (K,M); trans_b: B is
+ * stored (N,K).  c_dtype RA_BF16 (overwrite) or RA_F32 (accumulate when beta_one != 0). */
+int ra_gemm_bf16(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K,
+                 int32_t trans_a, int32_t trans_b, int32_t c_dtype, int32_t beta_one, ra_stream_t stream);
+
+const char* ra_last_error(void);
+int ra_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RINGATTN_HIP_H_ */

@@ -1,0 +1,20 @@
+"""MI355X-native ring attention hot path.
+
+Exports the names of the reference package (ringattention/__init__.py:26-27 binds ``ringattention``
+per backend; here there is one backend, the gfx950 HIP kernels):
+
+    ringattention, ringattention_jax, blockwise_feedforward
+
+plus ``ring_axis`` to declare the size of the (virtual) sequence-parallel ring, ``SwiGLU`` and
+``decode_attention``.
+"""
+from .ringattention_hip import (ring_attention, ring_axis, axis_size, below_or_on_diag, run_prefix_keys,
+                                _blockwise_attention_fwd, _blockwise_attention_bwd)
+from .feedforward import blockwise_feedforward, SwiGLU, gemm_bf16
+from .decode import decode_attention
+
+ringattention = ring_attention
+ringattention_jax = ring_attention
+
+__all__ = ["ringattention", "ringattention_jax", "ring_attention", "blockwise_feedforward", "ring_axis",
+           "axis_size", "SwiGLU", "decode_attention", "below_or_on_diag"]

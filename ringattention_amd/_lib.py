@@ -1,0 +1,115 @@
+"""ctypes binding of libringattn_hip.so (the C-ABI declared in include/ringattn_hip.h).
+
+The library is the only compute path: loading fails loudly when it has not been built, and
+nothing here falls back to torch ops.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libringattn_hip.so")
+
+RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
+RA_F32, RA_BF16 = 0, 1
+RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
+
+i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
+
+
+class RaMask(C.Structure):
+    _fields_ = [
+        ("bias", vp), ("bias_stride_b", i64), ("bias_stride_h", i64), ("bias_stride_q", i64),
+        ("bias_stride_k", i64), ("segment_ids", vp), ("seg_stride_b", i64), ("seg_len", i32),
+        ("causal_block_size", i32), ("query_chunk_size", i32), ("key_chunk_size", i32),
+        ("q_chunk_idx_start", i32), ("k_chunk_idx_start", i32), ("cache_idx", vp), ("mask_min", f32),
+        ("skip_masked_tiles", i32),
+    ]
+
+
+class RaAttnFwdParams(C.Structure):
+    _fields_ = [
+        ("q", vp), ("k", vp), ("v", vp), ("dtype", i32),
+        ("B", i32), ("Sq", i32), ("Skv", i32), ("H", i32), ("D", i32),
+        ("q_stride_b", i64), ("q_stride_s", i64), ("kv_stride_b", i64), ("kv_stride_s", i64),
+        ("numerator", vp), ("num_stride_b", i64), ("num_stride_s", i64),
+        ("denominator", vp), ("max_score", vp), ("stat_stride_b", i64), ("stat_stride_h", i64),
+        ("mask", RaMask), ("impl", i32), ("carry_is_initial", i32),
+    ]
+
+
+class RaAttnBwdParams(C.Structure):
+    _fields_ = [
+        ("q", vp), ("k", vp), ("v", vp), ("g", vp), ("dtype", i32),
+        ("B", i32), ("Sq", i32), ("Skv", i32), ("H", i32), ("D", i32),
+        ("q_stride_b", i64), ("q_stride_s", i64), ("kv_stride_b", i64), ("kv_stride_s", i64),
+        ("delta", vp), ("denominator", vp), ("max_score", vp), ("stat_stride_b", i64), ("stat_stride_h", i64),
+        ("dq", vp), ("dq_stride_b", i64), ("dq_stride_s", i64),
+        ("dk", vp), ("dv", vp), ("dkv_stride_b", i64), ("dkv_stride_s", i64),
+        ("mask", RaMask), ("impl", i32),
+    ]
+
+
+class RaDecodeParams(C.Structure):
+    _fields_ = [
+        ("q", vp), ("k", vp), ("v", vp), ("out", vp), ("dtype", i32),
+        ("B", i32), ("L", i32), ("H", i32), ("D", i32),
+        ("q_stride_b", i64), ("kv_stride_b", i64), ("kv_stride_s", i64), ("out_stride_b", i64),
+        ("mask", RaMask), ("workspace", vp), ("workspace_bytes", C.c_size_t), ("num_splits", i32),
+    ]
+
+
+class RaSwigluParams(C.Structure):
+    _fields_ = [
+        ("T", i32), ("d", i32), ("f", i32),
+        ("x", vp), ("w1", vp), ("w2", vp), ("w3", vp),
+        ("a", vp), ("b", vp), ("h", vp), ("y", vp),
+        ("dy", vp), ("dx", vp), ("dw1", vp), ("dw2", vp), ("dw3", vp), ("da", vp), ("db", vp),
+    ]
+
+
+# every symbol include/ringattn_hip.h declares: (name, restype, argtypes)
+SYMBOLS = {
+    "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
+    "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
+    "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),
+    "ra_attn_bwd_delta": (C.c_int, [vp, vp, i32, i64, i64, vp, i64, i64, i32, i32, i32, i32, vp]),
+    "ra_attn_bwd_block": (C.c_int, [C.POINTER(RaAttnBwdParams), vp]),
+    "ra_decode_workspace_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
+    "ra_decode_fwd": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
+    "ra_swiglu_fwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
+    "ra_swiglu_bwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
+    "ra_gemm_bf16": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp]),
+    "ra_last_error": (C.c_char_p, []),
+    "ra_version": (C.c_int, []),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library once; raise if it is missing (there is no fallback path)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            "ringattention_amd: %s is missing. Build it with `python -m ringattention_amd.build` "
+            "(hipcc, gfx950); there is no non-HIP fallback." % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc == RA_OK:
+        return
+    msg = load().ra_last_error().decode()
+    if rc == RA_ERR_UNSUPPORTED:
+        raise NotImplementedError("%s: %s" % (what, msg))
+    if rc == RA_ERR_INVALID:
+        raise ValueError("%s: %s" % (what, msg))
+    raise RuntimeError("%s: %s (code %d)" % (what, msg, rc))

@@ -1,0 +1,171 @@
+// extern "C" surface of libringattn_hip.so: argument validation, kernel-family
+// dispatch and per-thread error text.  Declarations: include/ringattn_hip.h.
+#include <stdarg.h>
+#include <stdio.h>
+#include "common.hpp"
+
+namespace ra {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int attn_fwd_generic(const ra_attn_fwd_params* p, hipStream_t s);
+int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s);
+int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s);     // RA_ERR_UNSUPPORTED if shape does not fit
+int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s);
+bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p);
+bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p);
+int carry_init(float*, int64_t, int64_t, float*, float*, int64_t, int64_t, int, int, int, int, hipStream_t);
+int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, void*, int, int64_t, int64_t, int,
+             int, int, int, hipStream_t);
+int bwd_delta(const void*, const void*, int, int64_t, int64_t, float*, int64_t, int64_t, int, int, int, int,
+              hipStream_t);
+int decode_pick_splits(int B, int L, int H, int D, int dtype);
+int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
+int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
+int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s);
+int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
+              int beta_one, hipStream_t s);
+
+static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
+  RA_REQUIRE(m.query_chunk_size > 0 && m.key_chunk_size > 0, RA_ERR_INVALID, "%s: chunk sizes must be positive", who);
+  RA_REQUIRE(Sq % m.query_chunk_size == 0, RA_ERR_INVALID, "%s: q_len %d is not a multiple of query_chunk_size %d",
+             who, Sq, m.query_chunk_size);
+  RA_REQUIRE(Skv % m.key_chunk_size == 0, RA_ERR_INVALID, "%s: kv_len %d is not a multiple of key_chunk_size %d",
+             who, Skv, m.key_chunk_size);
+  RA_REQUIRE(m.causal_block_size >= 0, RA_ERR_INVALID, "%s: causal_block_size must be >= 0 (0 = None)", who);
+  if (m.causal_block_size > 0) {
+    const int cbs = m.causal_block_size;
+    RA_REQUIRE((cbs <= m.query_chunk_size || cbs % m.query_chunk_size == 0) &&
+                   (cbs <= m.key_chunk_size || cbs % m.key_chunk_size == 0),
+               RA_ERR_INVALID, "%s: causal_block_size %d larger than a chunk must be a multiple of it", who, cbs);
+  }
+  RA_REQUIRE(m.q_chunk_idx_start >= 0 && m.k_chunk_idx_start >= 0, RA_ERR_INVALID, "%s: negative chunk start", who);
+  if (m.segment_ids) RA_REQUIRE(m.seg_len > 0, RA_ERR_INVALID, "%s: segment_ids given with seg_len 0", who);
+  return RA_OK;
+}
+
+}  // namespace ra
+
+using namespace ra;
+
+extern "C" {
+
+const char* ra_last_error(void) { return g_err; }
+int ra_version(void) { return 1; }
+
+int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s, float* denominator,
+                       float* max_score, int64_t stat_stride_b, int64_t stat_stride_h, int32_t B, int32_t Sq,
+                       int32_t H, int32_t D, ra_stream_t stream) {
+  RA_REQUIRE(numerator && denominator && max_score, RA_ERR_INVALID, "carry_init: null pointer");
+  RA_REQUIRE(B > 0 && Sq > 0 && H > 0 && D > 0, RA_ERR_INVALID, "carry_init: empty shape");
+  return carry_init(numerator, num_stride_b, num_stride_s, denominator, max_score, stat_stride_b, stat_stride_h, B,
+                    Sq, H, D, (hipStream_t)stream);
+}
+
+int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "attn_fwd_block: null params");
+  RA_REQUIRE(p->q && p->k && p->v && p->numerator && p->denominator && p->max_score, RA_ERR_INVALID,
+             "attn_fwd_block: null tensor");
+  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_fwd_block: dtype %d", p->dtype);
+  RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_fwd_block: empty shape");
+  RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_fwd_block: B and H must be <= 65535");
+  if (int rc = check_mask(p->mask, p->Sq, p->Skv, "attn_fwd_block")) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (p->impl == RA_IMPL_GENERIC) return attn_fwd_generic(p, s);
+  if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, s);
+  RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
+             "attn_fwd_block: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128");
+  return attn_fwd_generic(p, s);
+}
+
+int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_stride_s, const float* denominator,
+                     int64_t stat_stride_b, int64_t stat_stride_h, void* out, int32_t out_dtype,
+                     int64_t out_stride_b, int64_t out_stride_s, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                     ra_stream_t stream) {
+  RA_REQUIRE(numerator && denominator && out, RA_ERR_INVALID, "finalize: null pointer");
+  RA_REQUIRE(out_dtype == RA_F32 || out_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "finalize: dtype %d", out_dtype);
+  RA_REQUIRE(B > 0 && Sq > 0 && H > 0 && D > 0 && B <= 65535, RA_ERR_INVALID, "finalize: bad shape");
+  return finalize(numerator, num_stride_b, num_stride_s, denominator, stat_stride_b, stat_stride_h, out, out_dtype,
+                  out_stride_b, out_stride_s, B, Sq, H, D, (hipStream_t)stream);
+}
+
+int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t stride_b, int64_t stride_s, float* delta,
+                      int64_t stat_stride_b, int64_t stat_stride_h, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                      ra_stream_t stream) {
+  RA_REQUIRE(g && out && delta, RA_ERR_INVALID, "bwd_delta: null pointer");
+  RA_REQUIRE(dtype == RA_F32 || dtype == RA_BF16, RA_ERR_UNSUPPORTED, "bwd_delta: dtype %d", dtype);
+  RA_REQUIRE(B > 0 && Sq > 0 && H > 0 && D > 0 && B <= 65535, RA_ERR_INVALID, "bwd_delta: bad shape");
+  return bwd_delta(g, out, dtype, stride_b, stride_s, delta, stat_stride_b, stat_stride_h, B, Sq, H, D,
+                   (hipStream_t)stream);
+}
+
+int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "attn_bwd_block: null params");
+  RA_REQUIRE(p->q && p->k && p->v && p->g && p->delta && p->denominator && p->max_score && p->dq && p->dk && p->dv,
+             RA_ERR_INVALID, "attn_bwd_block: null tensor");
+  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_bwd_block: dtype %d", p->dtype);
+  RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_bwd_block: empty shape");
+  RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_bwd_block: B and H must be <= 65535");
+  if (int rc = check_mask(p->mask, p->Sq, p->Skv, "attn_bwd_block")) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (p->impl == RA_IMPL_GENERIC) return attn_bwd_generic(p, s);
+  if (attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, s);
+  RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
+             "attn_bwd_block: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128");
+  return attn_bwd_generic(p, s);
+}
+
+size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int32_t num_splits) {
+  if (B <= 0 || L <= 0 || H <= 0 || D <= 0) return 0;
+  int ns = num_splits > 0 ? num_splits : 256;   // upper bound of the automatic choice
+  return (size_t)B * H * ns * (D + 2) * sizeof(float);
+}
+
+int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "decode_fwd: null params");
+  RA_REQUIRE(p->q && p->k && p->v && p->out && p->workspace, RA_ERR_INVALID, "decode_fwd: null tensor");
+  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "decode_fwd: dtype %d", p->dtype);
+  RA_REQUIRE(p->B > 0 && p->L > 0 && p->H > 0 && p->D > 0 && p->B <= 65535, RA_ERR_INVALID, "decode_fwd: bad shape");
+  RA_REQUIRE(p->mask.query_chunk_size == 1, RA_ERR_INVALID,
+             "decode_fwd: one query token needs query_chunk_size == 1 (q_len // query_chunk_size chunks)");
+  if (int rc = check_mask(p->mask, 1, p->L, "decode_fwd")) return rc;
+  int ns = p->num_splits > 0 ? p->num_splits : decode_pick_splits(p->B, p->L, p->H, p->D, p->dtype);
+  RA_REQUIRE(ns <= 256, RA_ERR_INVALID, "decode_fwd: num_splits %d > 256", ns);
+  size_t need = (size_t)p->B * p->H * ns * (p->D + 2) * sizeof(float);
+  RA_REQUIRE(p->workspace_bytes >= need, RA_ERR_INVALID, "decode_fwd: workspace %zu bytes < %zu needed",
+             p->workspace_bytes, need);
+  return decode_fwd(p, ns, (hipStream_t)stream);
+}
+
+int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "swiglu_fwd: null params");
+  RA_REQUIRE(p->x && p->w1 && p->w2 && p->w3 && p->a && p->b && p->h && p->y, RA_ERR_INVALID, "swiglu_fwd: null tensor");
+  RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_fwd: empty shape");
+  return swiglu_fwd(p, (hipStream_t)stream);
+}
+
+int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "swiglu_bwd: null params");
+  RA_REQUIRE(p->x && p->w1 && p->w2 && p->w3 && p->a && p->b && p->h && p->dy && p->dx && p->dw1 && p->dw2 &&
+                 p->dw3 && p->da && p->db,
+             RA_ERR_INVALID, "swiglu_bwd: null tensor");
+  RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_bwd: empty shape");
+  return swiglu_bwd(p, (hipStream_t)stream);
+}
+
+int ra_gemm_bf16(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,
+                 int32_t trans_b, int32_t c_dtype, int32_t beta_one, ra_stream_t stream) {
+  RA_REQUIRE(A && Bm && C, RA_ERR_INVALID, "gemm_bf16: null pointer");
+  RA_REQUIRE(M > 0 && N > 0 && K > 0, RA_ERR_INVALID, "gemm_bf16: empty shape");
+  RA_REQUIRE(c_dtype == RA_F32 || c_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "gemm_bf16: c_dtype %d", c_dtype);
+  return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,457 @@
+// Generic blockwise-attention kernels: fp32 arithmetic on the vector ALU, one
+// query row (or one key row) per lane, K/V (or Q/dO) tiles broadcast from LDS.
+// They accept any chunk sizes, fp32 or bf16 inputs and any supported head size,
+// and evaluate the reference's mask element by element; the MFMA kernels are
+// checked against them at sizes the CPU oracle cannot reach.
+//
+// Semantics follow ringattention_jax.py:130-145 (forward tile), :220-233
+// (backward tile), :272-322 (bias / mask) and :324-331 (skip predicate).
+#include "common.hpp"
+
+namespace ra {
+
+struct GenericArgs {
+  const void* q; const void* k; const void* v; const void* g;
+  int B, Sq, Skv, H, D;
+  int64_t q_sb, q_ss, kv_sb, kv_ss;
+  float* num; int64_t num_sb, num_ss;
+  float* den; float* mx; const float* delta;
+  int64_t st_sb, st_sh;
+  float* dq; int64_t dq_sb, dq_ss;
+  float* dk; float* dv; int64_t dkv_sb, dkv_ss;
+  MaskView mv;
+  const int32_t* cache_idx;
+  int carry_is_initial;
+};
+
+__device__ __forceinline__ MaskView resolve_mask(const GenericArgs& a) {
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;   // ringattention_jax.py:35
+  return mv;
+}
+
+// per-row constants of the mask
+struct RowInfo {
+  int kend;        // keys [0,kend) of this shard are in chunks that run for this row
+  long long gq_blk;
+  int seg;
+  int64_t bias_off;
+};
+
+__device__ __forceinline__ RowInfo row_info(const MaskView& mv, int b, int h, int row, int skv) {
+  RowInfo r;
+  int qi = row / mv.qc;
+  r.kend = mv.run_prefix_keys(qi, skv);
+  long long gq = mv.global_q(row);
+  r.gq_blk = mv.cbs > 0 ? gq / mv.cbs : 0;
+  r.seg = 0;
+  if (mv.seg) {
+    int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, row % mv.qc);
+    r.seg = mv.seg[(int64_t)b * mv.seg_sb + idx];
+  }
+  r.bias_off = (int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(row % mv.qc) * mv.bias_sq;
+  return r;
+}
+
+// logit of (row, local key kj) given the raw dot product; -inf when the pair's tile does not run
+__device__ __forceinline__ float logit(const MaskView& mv, const RowInfo& r, float dot, float scale, int kj,
+                                       int seg_k) {
+  if (kj >= r.kend) return RA_NEG_INF;
+  long long gk = mv.global_k(kj);
+  float add = 0.f;
+  if (mv.bias) {
+    add = mv.bias[r.bias_off + gk * mv.bias_sk];
+    if (mv.any_mask) add = fminf(add, 0.f);                       // minimum(), :299,:309
+  }
+  bool masked = (mv.cbs > 0 && r.gq_blk < gk / mv.cbs) || (mv.seg && r.seg != seg_k);
+  if (masked) add = mv.mask_min;
+  return dot / scale + add;                                       // :134-136
+}
+
+template <typename T, int D>
+__device__ __forceinline__ void stage_rows(float* dst, const T* src, int64_t stride_s, int row0, int nrows,
+                                           int limit, int tid, int nthreads) {
+  // dst[r*D + d] = src[(row0+r)*stride_s + d] for r < nrows, zero past limit
+  for (int i = tid; i < nrows * D; i += nthreads) {
+    int r = i / D, d = i % D;
+    int row = row0 + r;
+    dst[i] = row < limit ? load_f32<T>(src + (int64_t)row * stride_s + d) : 0.f;
+  }
+}
+
+constexpr int GEN_ROWS = 64;   // rows per workgroup = one wavefront
+constexpr int GEN_TK = 16;     // keys (or query rows) staged per step
+
+// ------------------------------------------------------------------ forward
+template <typename T, int D>
+__global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs a) {
+  __shared__ float Ks[GEN_TK * D];
+  __shared__ float Vs[GEN_TK * D];
+  __shared__ int seg_k[GEN_TK];
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, b = blockIdx.z, h = blockIdx.y;
+  const int row = blockIdx.x * GEN_ROWS + tid;
+  const bool valid = row < a.Sq;
+  const int rrow = valid ? row : a.Sq - 1;
+  const T* qp = (const T*)a.q + (int64_t)b * a.q_sb + (int64_t)rrow * a.q_ss + (int64_t)h * D;
+  const T* kbase = (const T*)a.k + (int64_t)b * a.kv_sb + (int64_t)h * D;
+  const T* vbase = (const T*)a.v + (int64_t)b * a.kv_sb + (int64_t)h * D;
+  float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)rrow * a.num_ss + (int64_t)h * D;
+  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rrow;
+  const float scale = sqrtf((float)D);                            // :118
+
+  float q[D], acc[D];
+#pragma unroll
+  for (int d = 0; d < D; d++) q[d] = load_f32<T>(qp + d);
+  float m = RA_NEG_INF, l = 0.f;
+  if (a.carry_is_initial) {
+#pragma unroll
+    for (int d = 0; d < D; d++) acc[d] = 0.f;
+  } else {
+#pragma unroll
+    for (int d = 0; d < D; d++) acc[d] = nump[d];
+    m = a.mx[st]; l = a.den[st];
+  }
+  RowInfo ri = row_info(mv, b, h, rrow, a.Skv);
+  if (!valid) ri.kend = 0;
+  int kend_wg = ri.kend;
+  for (int off = 32; off > 0; off >>= 1) kend_wg = max(kend_wg, __shfl_xor(kend_wg, off));
+
+  for (int k0 = 0; k0 < kend_wg; k0 += GEN_TK) {
+    __syncthreads();
+    stage_rows<T, D>(Ks, kbase, a.kv_ss, k0, GEN_TK, a.Skv, tid, GEN_ROWS);
+    stage_rows<T, D>(Vs, vbase, a.kv_ss, k0, GEN_TK, a.Skv, tid, GEN_ROWS);
+    if (tid < GEN_TK) {
+      int sk = 0;
+      if (mv.seg) {
+        int kj = min(k0 + tid, a.Skv - 1);
+        int ki = kj / mv.kc;
+        int idx = clamp_seg_index(((long long)mv.k_start + ki) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
+        sk = mv.seg[(int64_t)b * mv.seg_sb + idx];
+      }
+      seg_k[tid] = sk;
+    }
+    __syncthreads();
+    float s[GEN_TK];
+    float tile_max = RA_NEG_INF;
+#pragma unroll
+    for (int j = 0; j < GEN_TK; j++) {
+      float dot = 0.f;
+#pragma unroll
+      for (int d = 0; d < D; d++) dot = fmaf(q[d], Ks[j * D + d], dot);
+      s[j] = logit(mv, ri, dot, scale, k0 + j, seg_k[j]);
+      tile_max = fmaxf(tile_max, s[j]);
+    }
+    float m_new = fmaxf(m, tile_max);                             // :138
+    if (m_new == RA_NEG_INF) continue;                            // nothing ran for this row yet
+    float corr = (m == m_new) ? 1.f : expf(m - m_new);            // :142
+    float psum = 0.f;
+#pragma unroll
+    for (int j = 0; j < GEN_TK; j++) { s[j] = expf(s[j] - m_new); psum += s[j]; }   // :140
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+      float t = 0.f;
+#pragma unroll
+      for (int j = 0; j < GEN_TK; j++) t = fmaf(s[j], Vs[j * D + d], t);           // :141
+      acc[d] = acc[d] * corr + t;                                 // :143
+    }
+    l = l * corr + psum;                                          // :144
+    m = m_new;
+  }
+  if (valid) {
+#pragma unroll
+    for (int d = 0; d < D; d++) nump[d] = acc[d];
+    a.mx[st] = m; a.den[st] = l;
+  }
+}
+
+// ------------------------------------------------------------------ backward, dq (one query row per lane)
+template <typename T, int D>
+__global__ __launch_bounds__(GEN_ROWS) void attn_bwd_dq_generic_kernel(GenericArgs a) {
+  __shared__ float Ks[GEN_TK * D];
+  __shared__ float Vs[GEN_TK * D];
+  __shared__ int seg_k[GEN_TK];
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, b = blockIdx.z, h = blockIdx.y;
+  const int row = blockIdx.x * GEN_ROWS + tid;
+  const bool valid = row < a.Sq;
+  const int rrow = valid ? row : a.Sq - 1;
+  const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)rrow * a.q_ss + (int64_t)h * D;
+  const T* qp = (const T*)a.q + qoff;
+  const T* gp = (const T*)a.g + qoff;
+  const T* kbase = (const T*)a.k + (int64_t)b * a.kv_sb + (int64_t)h * D;
+  const T* vbase = (const T*)a.v + (int64_t)b * a.kv_sb + (int64_t)h * D;
+  float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)rrow * a.dq_ss + (int64_t)h * D;
+  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rrow;
+  const float scale = sqrtf((float)D);
+
+  float q[D], g[D], dq[D];
+#pragma unroll
+  for (int d = 0; d < D; d++) { q[d] = load_f32<T>(qp + d); g[d] = load_f32<T>(gp + d); dq[d] = 0.f; }
+  const float m = a.mx[st], den = a.den[st], delta = a.delta[st];
+  RowInfo ri = row_info(mv, b, h, rrow, a.Skv);
+  if (!valid) ri.kend = 0;
+  int kend_wg = ri.kend;
+  for (int off = 32; off > 0; off >>= 1) kend_wg = max(kend_wg, __shfl_xor(kend_wg, off));
+
+  for (int k0 = 0; k0 < kend_wg; k0 += GEN_TK) {
+    __syncthreads();
+    stage_rows<T, D>(Ks, kbase, a.kv_ss, k0, GEN_TK, a.Skv, tid, GEN_ROWS);
+    stage_rows<T, D>(Vs, vbase, a.kv_ss, k0, GEN_TK, a.Skv, tid, GEN_ROWS);
+    if (tid < GEN_TK) {
+      int sk = 0;
+      if (mv.seg) {
+        int kj = min(k0 + tid, a.Skv - 1);
+        int ki = kj / mv.kc;
+        int idx = clamp_seg_index(((long long)mv.k_start + ki) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
+        sk = mv.seg[(int64_t)b * mv.seg_sb + idx];
+      }
+      seg_k[tid] = sk;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int j = 0; j < GEN_TK; j++) {
+      if (k0 + j >= ri.kend) continue;                            // tile does not run: zero contribution (:246-257)
+      float dot = 0.f, dp = 0.f;
+#pragma unroll
+      for (int d = 0; d < D; d++) { dot = fmaf(q[d], Ks[j * D + d], dot); dp = fmaf(g[d], Vs[j * D + d], dp); }
+      float s = logit(mv, ri, dot, scale, k0 + j, seg_k[j]);
+      float p = expf(s - m) / den;                                // :226
+      float ds = (dp - delta) * p;                                // :229
+#pragma unroll
+      for (int d = 0; d < D; d++) dq[d] = fmaf(ds, Ks[j * D + d], dq[d]);   // :230
+    }
+  }
+  if (valid) {
+#pragma unroll
+    for (int d = 0; d < D; d++) dqp[d] += dq[d] / scale;
+  }
+}
+
+// ------------------------------------------------------------------ backward, dk or dv (one key row per lane)
+template <typename T, int D, bool WANT_DK>
+__global__ __launch_bounds__(GEN_ROWS) void attn_bwd_dkv_generic_kernel(GenericArgs a) {
+  __shared__ float Qs[GEN_TK * D];
+  __shared__ float Gs[GEN_TK * D];
+  __shared__ float r_m[GEN_TK], r_den[GEN_TK], r_delta[GEN_TK];
+  __shared__ RowInfo r_info[GEN_TK];
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, b = blockIdx.z, h = blockIdx.y;
+  const int kj = blockIdx.x * GEN_ROWS + tid;
+  const bool valid = kj < a.Skv;
+  const int rk = valid ? kj : a.Skv - 1;
+  const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)rk * a.kv_ss + (int64_t)h * D;
+  const T* kp = (const T*)a.k + koff;
+  const T* vp = (const T*)a.v + koff;
+  const T* qbase = (const T*)a.q + (int64_t)b * a.q_sb + (int64_t)h * D;
+  const T* gbase = (const T*)a.g + (int64_t)b * a.q_sb + (int64_t)h * D;
+  float* outp = (WANT_DK ? a.dk : a.dv) + (int64_t)b * a.dkv_sb + (int64_t)rk * a.dkv_ss + (int64_t)h * D;
+  const float scale = sqrtf((float)D);
+
+  float k[D], v[WANT_DK ? D : 1], acc[D];
+#pragma unroll
+  for (int d = 0; d < D; d++) { k[d] = load_f32<T>(kp + d); acc[d] = 0.f; }
+  if (WANT_DK) {
+#pragma unroll
+    for (int d = 0; d < D; d++) v[d] = load_f32<T>(vp + d);
+  }
+  int seg_k = 0;
+  if (mv.seg) {
+    int ki = rk / mv.kc;
+    int idx = clamp_seg_index(((long long)mv.k_start + ki) * mv.kc, mv.kc, mv.seg_len, rk % mv.kc);
+    seg_k = mv.seg[(int64_t)b * mv.seg_sb + idx];
+  }
+  const int first_key = blockIdx.x * GEN_ROWS;
+
+  for (int q0 = 0; q0 < a.Sq; q0 += GEN_TK) {
+    // the run prefix grows with the query chunk: skip query tiles that end before this block's first key runs
+    int last_row = min(q0 + GEN_TK, a.Sq) - 1;
+    if (mv.run_prefix_keys(last_row / mv.qc, a.Skv) <= first_key) continue;
+    __syncthreads();
+    stage_rows<T, D>(Qs, qbase, a.q_ss, q0, GEN_TK, a.Sq, tid, GEN_ROWS);
+    stage_rows<T, D>(Gs, gbase, a.q_ss, q0, GEN_TK, a.Sq, tid, GEN_ROWS);
+    if (tid < GEN_TK) {
+      int row = q0 + tid;
+      bool rv = row < a.Sq;
+      int rr = rv ? row : a.Sq - 1;
+      const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rr;
+      r_m[tid] = a.mx[st]; r_den[tid] = a.den[st]; r_delta[tid] = a.delta[st];
+      RowInfo ri = row_info(mv, b, h, rr, a.Skv);
+      if (!rv) ri.kend = 0;
+      r_info[tid] = ri;
+    }
+    __syncthreads();
+#pragma unroll 2
+    for (int i = 0; i < GEN_TK; i++) {
+      const RowInfo ri = r_info[i];
+      if (!valid || kj >= ri.kend) continue;
+      float dot = 0.f, dp = 0.f;
+#pragma unroll
+      for (int d = 0; d < D; d++) {
+        dot = fmaf(Qs[i * D + d], k[d], dot);
+        if (WANT_DK) dp = fmaf(Gs[i * D + d], v[d], dp);
+      }
+      float s = logit(mv, ri, dot, scale, kj, seg_k);
+      float p = expf(s - r_m[i]) / r_den[i];                      // :226
+      if (WANT_DK) {
+        float ds = (dp - r_delta[i]) * p;                         // :229
+#pragma unroll
+        for (int d = 0; d < D; d++) acc[d] = fmaf(ds, Qs[i * D + d], acc[d]);   // :231
+      } else {
+#pragma unroll
+        for (int d = 0; d < D; d++) acc[d] = fmaf(p, Gs[i * D + d], acc[d]);    // :232
+      }
+    }
+  }
+  if (valid) {
+#pragma unroll
+    for (int d = 0; d < D; d++) outp[d] += WANT_DK ? acc[d] / scale : acc[d];
+  }
+}
+
+// ------------------------------------------------------------------ small elementwise kernels
+__global__ void carry_init_kernel(float* num, int64_t num_sb, int64_t num_ss, float* den, float* mx,
+                                  int64_t st_sb, int64_t st_sh, int Sq, int H, int D) {
+  const int b = blockIdx.z, row = blockIdx.x;
+  const int hd = H * D;
+  float* np = num + (int64_t)b * num_sb + (int64_t)row * num_ss;
+  for (int i = threadIdx.x; i < hd; i += blockDim.x) np[i] = 0.f;
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
+    int64_t st = (int64_t)b * st_sb + (int64_t)h * st_sh + row;
+    den[st] = 0.f; mx[st] = RA_NEG_INF;
+  }
+}
+
+template <typename TO>
+__global__ void finalize_kernel(const float* num, int64_t num_sb, int64_t num_ss, const float* den,
+                                int64_t st_sb, int64_t st_sh, TO* out, int64_t out_sb, int64_t out_ss,
+                                int Sq, int H, int D) {
+  const int b = blockIdx.z, row = blockIdx.x;
+  const int hd = H * D;
+  const float* np = num + (int64_t)b * num_sb + (int64_t)row * num_ss;
+  TO* op = out + (int64_t)b * out_sb + (int64_t)row * out_ss;
+  for (int i = threadIdx.x; i < hd; i += blockDim.x) {
+    int h = i / D;
+    float dn = den[(int64_t)b * st_sb + (int64_t)h * st_sh + row];
+    store_from_f32<TO>(op + i, np[i] / dn);                       // :52
+  }
+}
+
+template <typename T>
+__global__ void delta_kernel(const T* g, const T* o, int64_t sb, int64_t ss, float* delta, int64_t st_sb,
+                             int64_t st_sh, int Sq, int H, int D) {
+  // one wavefront per (b, row, h)
+  const int b = blockIdx.z, row = blockIdx.x;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, nw = blockDim.x / 64;
+  for (int h = wave; h < H; h += nw) {
+    const int64_t off = (int64_t)b * sb + (int64_t)row * ss + (int64_t)h * D;
+    float s = 0.f;
+    for (int d = lane; d < D; d += 64) s = fmaf(load_f32<T>(g + off + d), load_f32<T>(o + off + d), s);
+    for (int x = 32; x > 0; x >>= 1) s += __shfl_xor(s, x);
+    if (lane == 0) delta[(int64_t)b * st_sb + (int64_t)h * st_sh + row] = s;   // :218
+  }
+}
+
+// ------------------------------------------------------------------ host-side launchers
+static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
+  GenericArgs a{};
+  a.q = p->q; a.k = p->k; a.v = p->v; a.g = nullptr;
+  a.B = p->B; a.Sq = p->Sq; a.Skv = p->Skv; a.H = p->H; a.D = p->D;
+  a.q_sb = p->q_stride_b; a.q_ss = p->q_stride_s; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s;
+  a.num = p->numerator; a.num_sb = p->num_stride_b; a.num_ss = p->num_stride_s;
+  a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
+  a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
+  a.cache_idx = p->mask.cache_idx;
+  a.carry_is_initial = p->carry_is_initial;
+  return a;
+}
+
+template <typename T>
+static int launch_fwd_T(const GenericArgs& a, hipStream_t s) {
+  dim3 grid((a.Sq + GEN_ROWS - 1) / GEN_ROWS, a.H, a.B), block(GEN_ROWS);
+  switch (a.D) {
+    case 32: attn_fwd_generic_kernel<T, 32><<<grid, block, 0, s>>>(a); break;
+    case 64: attn_fwd_generic_kernel<T, 64><<<grid, block, 0, s>>>(a); break;
+    case 128: attn_fwd_generic_kernel<T, 128><<<grid, block, 0, s>>>(a); break;
+    default: set_error("generic attention: head size %d not in {32,64,128}", a.D); return RA_ERR_UNSUPPORTED;
+  }
+  RA_CHECK_LAUNCH("attn_fwd_generic");
+  return RA_OK;
+}
+
+int attn_fwd_generic(const ra_attn_fwd_params* p, hipStream_t s) {
+  GenericArgs a = make_args_fwd(p);
+  return p->dtype == RA_F32 ? launch_fwd_T<float>(a, s) : launch_fwd_T<uint16_t>(a, s);
+}
+
+template <typename T, int D>
+static void launch_bwd_TD(const GenericArgs& a, hipStream_t s) {
+  dim3 block(GEN_ROWS);
+  dim3 gq((a.Sq + GEN_ROWS - 1) / GEN_ROWS, a.H, a.B), gk((a.Skv + GEN_ROWS - 1) / GEN_ROWS, a.H, a.B);
+  attn_bwd_dq_generic_kernel<T, D><<<gq, block, 0, s>>>(a);
+  attn_bwd_dkv_generic_kernel<T, D, true><<<gk, block, 0, s>>>(a);
+  attn_bwd_dkv_generic_kernel<T, D, false><<<gk, block, 0, s>>>(a);
+}
+
+template <typename T>
+static int launch_bwd_T(const GenericArgs& a, hipStream_t s) {
+  switch (a.D) {
+    case 32: launch_bwd_TD<T, 32>(a, s); break;
+    case 64: launch_bwd_TD<T, 64>(a, s); break;
+    case 128: launch_bwd_TD<T, 128>(a, s); break;
+    default: set_error("generic attention: head size %d not in {32,64,128}", a.D); return RA_ERR_UNSUPPORTED;
+  }
+  RA_CHECK_LAUNCH("attn_bwd_generic");
+  return RA_OK;
+}
+
+int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s) {
+  GenericArgs a{};
+  a.q = p->q; a.k = p->k; a.v = p->v; a.g = p->g;
+  a.B = p->B; a.Sq = p->Sq; a.Skv = p->Skv; a.H = p->H; a.D = p->D;
+  a.q_sb = p->q_stride_b; a.q_ss = p->q_stride_s; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s;
+  a.den = const_cast<float*>(p->denominator); a.mx = const_cast<float*>(p->max_score); a.delta = p->delta;
+  a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
+  a.dq = p->dq; a.dq_sb = p->dq_stride_b; a.dq_ss = p->dq_stride_s;
+  a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
+  a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
+  a.cache_idx = p->mask.cache_idx;
+  return p->dtype == RA_F32 ? launch_bwd_T<float>(a, s) : launch_bwd_T<uint16_t>(a, s);
+}
+
+int carry_init(float* num, int64_t num_sb, int64_t num_ss, float* den, float* mx, int64_t st_sb, int64_t st_sh,
+               int B, int Sq, int H, int D, hipStream_t s) {
+  dim3 grid(Sq, 1, B);
+  carry_init_kernel<<<grid, 256, 0, s>>>(num, num_sb, num_ss, den, mx, st_sb, st_sh, Sq, H, D);
+  RA_CHECK_LAUNCH("carry_init");
+  return RA_OK;
+}
+
+int finalize(const float* num, int64_t num_sb, int64_t num_ss, const float* den, int64_t st_sb, int64_t st_sh,
+             void* out, int out_dtype, int64_t out_sb, int64_t out_ss, int B, int Sq, int H, int D,
+             hipStream_t s) {
+  dim3 grid(Sq, 1, B);
+  if (out_dtype == RA_F32)
+    finalize_kernel<float><<<grid, 256, 0, s>>>(num, num_sb, num_ss, den, st_sb, st_sh, (float*)out, out_sb,
+                                               out_ss, Sq, H, D);
+  else
+    finalize_kernel<uint16_t><<<grid, 256, 0, s>>>(num, num_sb, num_ss, den, st_sb, st_sh, (uint16_t*)out,
+                                                  out_sb, out_ss, Sq, H, D);
+  RA_CHECK_LAUNCH("finalize");
+  return RA_OK;
+}
+
+int bwd_delta(const void* g, const void* o, int dtype, int64_t sb, int64_t ss, float* delta, int64_t st_sb,
+              int64_t st_sh, int B, int Sq, int H, int D, hipStream_t s) {
+  dim3 grid(Sq, 1, B);
+  if (dtype == RA_F32)
+    delta_kernel<float><<<grid, 256, 0, s>>>((const float*)g, (const float*)o, sb, ss, delta, st_sb, st_sh, Sq,
+                                            H, D);
+  else
+    delta_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)o, sb, ss, delta, st_sb,
+                                               st_sh, Sq, H, D);
+  RA_CHECK_LAUNCH("bwd_delta");
+  return RA_OK;
+}
+
+}  // namespace ra

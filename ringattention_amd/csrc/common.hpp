@@ -1,0 +1,106 @@
+// Shared host/device helpers for the ring-attention HIP kernels (gfx950).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+#include "../../include/ringattn_hip.h"
+
+#define RA_NEG_INF (-__builtin_inff())
+
+namespace ra {
+
+void set_error(const char* fmt, ...);
+
+#define RA_REQUIRE(cond, code, ...)            \
+  do {                                         \
+    if (!(cond)) {                             \
+      ra::set_error(__VA_ARGS__);              \
+      return (code);                           \
+    }                                          \
+  } while (0)
+
+#define RA_CHECK_LAUNCH(name)                                              \
+  do {                                                                     \
+    hipError_t e_ = hipGetLastError();                                     \
+    if (e_ != hipSuccess) {                                                \
+      ra::set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return RA_ERR_LAUNCH;                                                \
+    }                                                                      \
+  } while (0)
+
+// ---------------------------------------------------------------- bf16 <-> fp32
+__device__ __forceinline__ float bf16_to_f32(uint16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even, NaN kept
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+template <typename T> __device__ __forceinline__ float load_f32(const T* p);
+template <> __device__ __forceinline__ float load_f32<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_f32<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
+template <typename T> __device__ __forceinline__ void store_from_f32(T* p, float v);
+template <> __device__ __forceinline__ void store_from_f32<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_from_f32<uint16_t>(uint16_t* p, float v) { *p = f32_to_bf16(v); }
+
+// ---------------------------------------------------------------- mask arithmetic
+// Device-side view of ra_mask with the chunk arithmetic of below_or_on_diag
+// (ringattention_jax.py:324-331) folded into "how many keys of this shard run
+// for a query chunk": the predicate is monotone in the key chunk index, so the
+// chunks that run are a prefix.
+struct MaskView {
+  const float* bias;
+  int64_t bias_sb, bias_sh, bias_sq, bias_sk;
+  const int32_t* seg;
+  int64_t seg_sb;
+  int seg_len;
+  int cbs, qc, kc;
+  int q_start, k_start;   // global chunk indices of local chunk 0
+  float mask_min;
+  int any_mask;
+  int skip_tiles;
+
+  __host__ __device__ static MaskView make(const ra_mask& m, int q_chunk_idx_start) {
+    MaskView v;
+    v.bias = m.bias; v.bias_sb = m.bias_stride_b; v.bias_sh = m.bias_stride_h;
+    v.bias_sq = m.bias_stride_q; v.bias_sk = m.bias_stride_k;
+    v.seg = m.segment_ids; v.seg_sb = m.seg_stride_b; v.seg_len = m.seg_len;
+    v.cbs = m.causal_block_size; v.qc = m.query_chunk_size; v.kc = m.key_chunk_size;
+    v.q_start = q_chunk_idx_start; v.k_start = m.k_chunk_idx_start;
+    v.mask_min = m.mask_min;
+    v.any_mask = (m.segment_ids != nullptr) || (m.causal_block_size > 0);
+    v.skip_tiles = m.skip_masked_tiles;
+    return v;
+  }
+
+  // Number of leading local keys (out of skv) whose chunk runs against local query chunk qi.
+  __host__ __device__ int run_prefix_keys(int qi, int skv) const {
+    if (cbs <= 0) return skv;
+    long long cq = cbs > qc ? cbs : qc;
+    long long ck = cbs > kc ? cbs : kc;
+    long long r = ((long long)q_start + qi) / (cq / qc);
+    long long x = (r + 1) * cq - 1;          // run iff x > c' * ck  with c' = c / (ck / kc)
+    if (x <= 0) return 0;
+    long long cmax = (x - 1) / ck;           // largest c' that runs
+    long long climit = (cmax + 1) * (ck / kc);   // global key chunks [0, climit) run
+    long long nloc = climit - k_start;
+    if (nloc <= 0) return 0;
+    long long keys = nloc * kc;
+    return keys > skv ? skv : (int)keys;
+  }
+  __host__ __device__ long long global_q(int local_row) const { return (long long)q_start * qc + local_row; }
+  __host__ __device__ long long global_k(int local_col) const { return (long long)k_start * kc + local_col; }
+};
+
+__device__ __forceinline__ int clamp_seg_index(long long chunk_offset, int chunk, int seg_len, int within) {
+  // lax.dynamic_slice clamps the slice start (ringattention_jax.py:286-295)
+  long long s = chunk_offset;
+  long long hi = (long long)seg_len - chunk;
+  if (s > hi) s = hi;
+  if (s < 0) s = 0;
+  long long i = s + within;
+  if (i >= seg_len) i = seg_len - 1;
+  return (int)i;
+}
+
+}  // namespace ra

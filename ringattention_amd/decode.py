@@ -1,0 +1,54 @@
+"""Decode through cache_idx (ringattention_jax.py:31-35 with one query token): host wrapper of the
+streaming kernel ra_decode_fwd."""
+import ctypes
+
+import torch
+
+from . import _lib as L
+from .ringattention_hip import _Config, _MaskInputs, _check_qkv, _ra_dtype, _rows, _stream
+
+_WORKSPACES = {}
+
+
+def _workspace(device, nbytes):
+    ws = _WORKSPACES.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _WORKSPACES[device] = ws
+    return ws
+
+
+def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs, out=None, num_splits=0):
+    """q (B,1,H,D) against the cache buffers k, v (B,L,H,D); cache_idx is a Python int or a device
+    int32 scalar (read by the kernel, so the call can sit in a captured graph or a tight loop).
+    blockwise_kwargs must carry query_chunk_size == 1, as q_len // query_chunk_size demands."""
+    cfg = _Config(blockwise_kwargs)
+    _check_qkv(q, k, v)
+    B, Sq, H, D = q.shape
+    if Sq != 1:
+        raise ValueError("decode_attention takes one query token per batch row")
+    if cfg.qc != 1:
+        raise ValueError("query_chunk_size must be 1 when q_len is 1")
+    L_buf = k.shape[1]
+    if L_buf % cfg.kc:
+        raise ValueError("cache length %d must divide by key_chunk_size %d" % (L_buf, cfg.kc))
+    mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, L_buf)
+    if out is None:
+        out = torch.empty_like(q)
+    lib = L.load()
+    p = L.RaDecodeParams()
+    p.q, p.k, p.v, p.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+    p.dtype = _ra_dtype(q)
+    p.B, p.L, p.H, p.D = B, L_buf, H, D
+    p.q_stride_b = _rows(q)[0]
+    p.kv_stride_b, p.kv_stride_s = _rows(k)
+    if _rows(v) != _rows(k):
+        raise ValueError("k and v caches must share strides")
+    p.out_stride_b = _rows(out)[0]
+    q_start = mi.cache_idx_host if mi.cache_idx_host is not None else 0
+    p.mask = mi.fill(cfg, q_start, 0, False)
+    nbytes = lib.ra_decode_workspace_bytes(B, L_buf, H, D, num_splits)
+    ws = _workspace(q.device, nbytes)
+    p.workspace, p.workspace_bytes, p.num_splits = ws.data_ptr(), ws.numel(), num_splits
+    L.check(lib.ra_decode_fwd(ctypes.byref(p), _stream()), "ra_decode_fwd")
+    return out

@@ -1,0 +1,115 @@
+"""blockwise_feedforward (ringattention_jax.py:333-352) and the SwiGLU MLP it is used with,
+over the bf16 MFMA GEMM kernels of libringattn_hip.so."""
+import ctypes
+
+import torch
+
+from . import _lib as L
+from .ringattention_hip import _stream
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+class _SwiGLUFn(torch.autograd.Function):
+    """y = (silu(x w1) * (x w3)) w2 on one chunk of tokens.  Nothing but x is kept for the backward
+    pass (the reference's default policy is nothing_saveable, ringattention_jax.py:334): the
+    pre-activations are recomputed."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, w3):
+        T, d = x.shape
+        f = w1.shape[1]
+        dev = x.device
+        a = torch.empty((T, f), dtype=torch.bfloat16, device=dev)
+        b = torch.empty_like(a)
+        h = torch.empty_like(a)
+        y = torch.empty((T, d), dtype=torch.bfloat16, device=dev)
+        p = L.RaSwigluParams()
+        p.T, p.d, p.f = T, d, f
+        p.x, p.w1, p.w2, p.w3 = x.data_ptr(), w1.data_ptr(), w2.data_ptr(), w3.data_ptr()
+        p.a, p.b, p.h, p.y = a.data_ptr(), b.data_ptr(), h.data_ptr(), y.data_ptr()
+        L.check(L.load().ra_swiglu_fwd(ctypes.byref(p), _stream()), "ra_swiglu_fwd")
+        ctx.save_for_backward(x, w1, w2, w3)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w1, w2, w3 = ctx.saved_tensors
+        T, d = x.shape
+        f = w1.shape[1]
+        dev = x.device
+        dy = dy.to(torch.bfloat16).contiguous()
+        bf = dict(dtype=torch.bfloat16, device=dev)
+        a, b, h, da, db = (torch.empty((T, f), **bf) for _ in range(5))
+        dx = torch.empty((T, d), **bf)
+        dw1 = torch.zeros((d, f), dtype=torch.float32, device=dev)
+        dw3 = torch.zeros((d, f), dtype=torch.float32, device=dev)
+        dw2 = torch.zeros((f, d), dtype=torch.float32, device=dev)
+        p = L.RaSwigluParams()
+        p.T, p.d, p.f = T, d, f
+        p.x, p.w1, p.w2, p.w3 = x.data_ptr(), w1.data_ptr(), w2.data_ptr(), w3.data_ptr()
+        p.a, p.b, p.h, p.y = a.data_ptr(), b.data_ptr(), h.data_ptr(), None
+        p.dy, p.dx = dy.data_ptr(), dx.data_ptr()
+        p.dw1, p.dw2, p.dw3 = dw1.data_ptr(), dw2.data_ptr(), dw3.data_ptr()
+        p.da, p.db = da.data_ptr(), db.data_ptr()
+        L.check(L.load().ra_swiglu_bwd(ctypes.byref(p), _stream()), "ra_swiglu_bwd")
+        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype)
+
+
+class SwiGLU(torch.nn.Module):
+    """The LLaMA-style MLP the reference's README pairs with blockwise_feedforward:
+    w2(silu(x w1) * (x w3)); weights stored (in, out), bf16."""
+
+    def __init__(self, hidden, intermediate, device=None, init_std=0.02):
+        super().__init__()
+        mk = lambda i, o: torch.nn.Parameter(
+            (torch.randn(i, o, device=device, dtype=torch.float32) * init_std).to(torch.bfloat16))
+        self.w1 = mk(hidden, intermediate)
+        self.w3 = mk(hidden, intermediate)
+        self.w2 = mk(intermediate, hidden)
+
+    def forward(self, hidden_states):
+        shp = hidden_states.shape
+        x = hidden_states.reshape(-1, shp[-1])
+        if x.dtype != torch.bfloat16:
+            raise NotImplementedError("SwiGLU kernels are bf16")
+        if not x.is_cuda:
+            raise RuntimeError("ringattention_amd runs on the GPU only")
+        y = _SwiGLUFn.apply(x.contiguous(), self.w1, self.w2, self.w3)
+        return y.reshape(*shp[:-1], y.shape[-1])
+
+
+def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), policy=None, pre_remat=True):
+    """ringattention_jax.py:333-352: apply ``feedforward`` to ``chunk_size`` tokens at a time.
+
+    The reference groups tokens with 'b (c n) d -> b c n d', c=chunk_size and scans over n, so step
+    j sees the strided token set {ci * n + j}.  A generic callable gets exactly those groups.  A
+    ``SwiGLU`` instance is token-wise, so it is fed contiguous slabs of chunk_size tokens instead:
+    the same number of steps and the same result, with dense memory access.  ``policy`` /
+    ``pre_remat`` / ``static_argnums`` steer XLA rematerialisation only; SwiGLU always recomputes."""
+    b, s, d = inputs.shape
+    if s % chunk_size:
+        raise ValueError("sequence length %d must divide by chunk_size %d" % (s, chunk_size))
+    n = s // chunk_size
+    if isinstance(feedforward, SwiGLU):
+        outs = [feedforward(inputs[:, j * chunk_size:(j + 1) * chunk_size]) for j in range(n)]
+        return torch.cat(outs, dim=1)
+    x = inputs.reshape(b, chunk_size, n, d)
+    outs = [feedforward(x[:, :, j, :]) for j in range(n)]
+    out = torch.stack(outs, dim=2)
+    return out.reshape(b, s, out.shape[-1])
+
+
+def gemm_bf16(A, B, trans_a=False, trans_b=False, out_dtype=torch.bfloat16, out=None, accumulate=False):
+    """C = op(A) op(B) with the library's bf16 MFMA GEMM (used by the SwiGLU kernels; exposed for tests)."""
+    M = A.shape[1] if trans_a else A.shape[0]
+    K = A.shape[0] if trans_a else A.shape[1]
+    N = B.shape[0] if trans_b else B.shape[1]
+    if out is None:
+        out = torch.zeros((M, N), dtype=out_dtype, device=A.device)
+    cd = L.RA_F32 if out.dtype == torch.float32 else L.RA_BF16
+    L.check(L.load().ra_gemm_bf16(A.data_ptr(), B.data_ptr(), out.data_ptr(), M, N, K, int(trans_a),
+                                  int(trans_b), cd, int(accumulate), _stream()), "ra_gemm_bf16")
+    return out

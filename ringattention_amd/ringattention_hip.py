@@ -1,0 +1,458 @@
+"""Host side of the MI355X ring-attention hot path: the interface of the reference's
+``ringattention/ringattention_jax.py`` over the HIP kernels of libringattn_hip.so.
+
+Same names, argument order and meaning as the reference:
+
+* ``ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits,
+  blockwise_kwargs)``  (ringattention_jax.py:92-97), differentiable in q, k, v;
+* ``_blockwise_attention_fwd`` / ``_blockwise_attention_bwd`` (:99-179, :181-270): one ring
+  step on one device, carry in / carry out;
+* ``below_or_on_diag`` (:324-331).
+
+Tensors are torch tensors in device memory (torch only owns memory and streams).  The ring over
+``axis_name`` is virtual: ``ring_axis(name, size)`` declares its size, q/k/v are then the global
+arrays a ``shard_map`` caller holds, and every device's program is run in turn on the one GPU
+with the K/V shard that the ring would have delivered at each step.  No bytes move.
+"""
+import contextlib
+import ctypes
+import math
+
+import torch
+
+from . import _lib as L
+
+# --------------------------------------------------------------------------- virtual ring axes
+_AXES = {}
+
+
+@contextlib.contextmanager
+def ring_axis(axis_name, size):
+    """Declare that ``axis_name`` is a ring of ``size`` virtual devices (the sp mesh axis)."""
+    if size < 1:
+        raise ValueError("ring size must be >= 1")
+    old = _AXES.get(axis_name)
+    _AXES[axis_name] = int(size)
+    try:
+        yield
+    finally:
+        if old is None:
+            _AXES.pop(axis_name, None)
+        else:
+            _AXES[axis_name] = old
+
+
+def axis_size(axis_name):
+    """Counterpart of lax.psum(1, axis_name) (ringattention_jax.py:24): 1 for an undeclared axis."""
+    if axis_name is None:
+        return 1
+    if isinstance(axis_name, int):
+        return axis_name
+    return _AXES.get(axis_name, 1)
+
+
+# --------------------------------------------------------------------------- helpers
+_DTYPES = {
+    "float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16,
+    "torch.float32": torch.float32, "torch.bfloat16": torch.bfloat16, "torch.float16": torch.float16,
+    "<class 'jax.numpy.float32'>": torch.float32, "<class 'jax.numpy.bfloat16'>": torch.bfloat16,
+}
+
+
+def _as_torch_dtype(dt):
+    if isinstance(dt, torch.dtype):
+        return dt
+    name = getattr(dt, "__name__", None) or getattr(dt, "name", None) or str(dt)
+    if name in _DTYPES:
+        return _DTYPES[name]
+    raise ValueError("blockwise_kwargs['dtype']=%r is not float32/bfloat16/float16" % (dt,))
+
+
+def _ra_dtype(t):
+    if t.dtype == torch.float32:
+        return L.RA_F32
+    if t.dtype == torch.bfloat16:
+        return L.RA_BF16
+    raise NotImplementedError("q/k/v dtype %s: only float32 and bfloat16 are supported" % t.dtype)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def below_or_on_diag(r, r_blk_size, c, c_blk_size, causal_block_size):
+    """ringattention_jax.py:324-331 on Python ints."""
+    cq = max(causal_block_size, r_blk_size)
+    ck = max(causal_block_size, c_blk_size)
+    r = r // (cq // r_blk_size)
+    c = c // (ck // c_blk_size)
+    return ((r + 1) * cq - 1) > (c * ck)
+
+
+def run_prefix_keys(q_chunk_global, qc, kc, cbs, k_chunk_idx_start, kv_len):
+    """How many leading keys of a K/V shard lie in chunks that run against one query chunk.
+
+    The skip predicate is monotone in the key chunk index, so the chunks that run are a prefix;
+    the kernels use the same closed form."""
+    if cbs is None or cbs <= 0:
+        return kv_len
+    cq, ck = max(cbs, qc), max(cbs, kc)
+    r = q_chunk_global // (cq // qc)
+    x = (r + 1) * cq - 1
+    if x <= 0:
+        return 0
+    cmax = (x - 1) // ck
+    climit = (cmax + 1) * (ck // kc)
+    nloc = climit - k_chunk_idx_start
+    if nloc <= 0:
+        return 0
+    return min(nloc * kc, kv_len)
+
+
+class _Config:
+    """blockwise_kwargs (ringattention_jax.py:99-100) reduced to what the kernels need."""
+
+    def __init__(self, blockwise_kwargs):
+        kw = dict(blockwise_kwargs)
+        self.qc = int(kw["query_chunk_size"])
+        self.kc = int(kw["key_chunk_size"])
+        cbs = kw.get("causal_block_size", None)
+        self.cbs = None if cbs is None else int(cbs)
+        if self.cbs is not None and self.cbs < 1:
+            raise ValueError("causal_block_size must be None or >= 1")
+        if (not kw.get("deterministic", True)) and float(kw.get("attn_pdrop", 0.0)) > 0.0:
+            raise NotImplementedError(
+                "attention dropout is not supported: its mask comes from the jax.random stream")
+        self.dtype = _as_torch_dtype(kw.get("dtype", torch.float32))
+        self.mask_min = float(torch.finfo(self.dtype).min)
+        self.impl = {"auto": L.RA_IMPL_AUTO, "generic": L.RA_IMPL_GENERIC, "mfma": L.RA_IMPL_MFMA}[
+            kw.get("impl", "auto")]
+        self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
+        # policy / precision / prevent_cse / dropout_rng only steer XLA rematerialisation: the
+        # kernels always recompute the probabilities in the backward pass.
+
+
+class _MaskInputs:
+    """attn_bias / segment_ids / cache_idx in the form ra_mask wants (device memory kept alive here)."""
+
+    def __init__(self, cfg, attn_bias, segment_ids, cache_idx, batch, device, k_total):
+        self.bias = None
+        self.bias_strides = (0, 0, 0, 0)
+        if attn_bias is not None:
+            if attn_bias.dim() != 4:
+                raise ValueError("attn_bias must be 4-D (B, H, Q, K)")
+            bb, hb, qb, kb = attn_bias.shape
+            if qb != 1 and qb < cfg.qc:
+                raise ValueError("attn_bias query dim must be 1 or >= query_chunk_size")
+            if kb != 1 and kb < k_total:
+                raise ValueError("attn_bias key dim %d is smaller than the global key length %d" % (kb, k_total))
+            # chunk_bias.astype(dtype) (ringattention_jax.py:322): values rounded to the kwargs dtype
+            b = attn_bias.detach().to(device=device).to(cfg.dtype).to(torch.float32).contiguous()
+            self.bias = b
+            self.bias_strides = (0 if bb == 1 else b.stride(0), 0 if hb == 1 else b.stride(1),
+                                 0 if qb == 1 else b.stride(2), 0 if kb == 1 else b.stride(3))
+        self.seg = None
+        self.seg_stride_b = 0
+        self.seg_len = 0
+        if segment_ids is not None:
+            if segment_ids.dim() != 2:
+                raise ValueError("segment_ids must be 2-D (B, S)")
+            s = segment_ids.detach().to(device=device, dtype=torch.int32).contiguous()
+            self.seg = s
+            self.seg_stride_b = 0 if s.shape[0] == 1 else s.stride(0)
+            self.seg_len = s.shape[1]
+        self.cache_idx_host = None
+        self.cache_idx_dev = None
+        if cache_idx is not None:
+            if isinstance(cache_idx, torch.Tensor):
+                if cache_idx.is_cuda:
+                    self.cache_idx_dev = cache_idx.detach().to(torch.int32).reshape(1).contiguous()
+                else:
+                    self.cache_idx_host = int(cache_idx)
+            else:
+                self.cache_idx_host = int(cache_idx)
+
+    def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip):
+        m = L.RaMask()
+        m.bias = self.bias.data_ptr() if self.bias is not None else None
+        m.bias_stride_b, m.bias_stride_h, m.bias_stride_q, m.bias_stride_k = self.bias_strides
+        m.segment_ids = self.seg.data_ptr() if self.seg is not None else None
+        m.seg_stride_b = self.seg_stride_b
+        m.seg_len = self.seg_len
+        m.causal_block_size = 0 if cfg.cbs is None else cfg.cbs
+        m.query_chunk_size = cfg.qc
+        m.key_chunk_size = cfg.kc
+        m.q_chunk_idx_start = q_chunk_idx_start
+        m.k_chunk_idx_start = k_chunk_idx_start
+        m.cache_idx = self.cache_idx_dev.data_ptr() if self.cache_idx_dev is not None else None
+        m.mask_min = cfg.mask_min
+        m.skip_masked_tiles = 1 if skip else 0
+        return m
+
+
+def _check_qkv(q, k, v):
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("ringattention_amd runs on the GPU only: q, k, v must be device tensors")
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape:
+        raise ValueError("q, k, v must be (B, S, H, D) with k.shape == v.shape")
+    if q.shape[0] != k.shape[0] or q.shape[2:] != k.shape[2:]:
+        raise ValueError("q and k must agree in batch, heads and head size")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share a dtype")
+
+
+def _rows(t):
+    """(stride_b, stride_s) of a (B, S, H, D) tensor whose last two dims are dense."""
+    if t.stride(3) != 1 or t.stride(2) != t.shape[3]:
+        raise ValueError("tensor must be dense in its last two (H, D) dims")
+    return t.stride(0), t.stride(1)
+
+
+# --------------------------------------------------------------------------- one ring step
+def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_start, bias, segment_ids,
+                             causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
+                             dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
+                             precision=None, prevent_cse=True, cache_idx=None, _mask_inputs=None,
+                             _cfg=None, _carry_is_initial=False, **extra):
+    """ringattention_jax.py:99-179.  ``carry`` = (numerator (B,Sq,H,D), denominator (B,H,Sq),
+    max_score (B,H,Sq)), fp32, updated IN PLACE and returned."""
+    cfg = _cfg or _Config(dict(causal_block_size=causal_block_size, query_chunk_size=query_chunk_size,
+                               key_chunk_size=key_chunk_size, deterministic=deterministic,
+                               attn_pdrop=attn_pdrop, dtype=dtype, **extra))
+    _check_qkv(q, k, v)
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    mi = _mask_inputs or _MaskInputs(cfg, bias, segment_ids, cache_idx, B, q.device,
+                                     k_chunk_idx_start * cfg.kc + Skv)
+    num, den, mx = carry
+    p = L.RaAttnFwdParams()
+    p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    p.dtype = _ra_dtype(q)
+    p.B, p.Sq, p.Skv, p.H, p.D = B, Sq, Skv, H, D
+    p.q_stride_b, p.q_stride_s = _rows(q)
+    p.kv_stride_b, p.kv_stride_s = _rows(k)
+    if _rows(v) != _rows(k):
+        raise ValueError("k and v must share strides")
+    p.numerator = num.data_ptr()
+    p.num_stride_b, p.num_stride_s = _rows(num)
+    p.denominator, p.max_score = den.data_ptr(), mx.data_ptr()
+    if den.stride() != mx.stride() or den.stride(2) != 1:
+        raise ValueError("denominator / max_score must share strides and be dense in the last dim")
+    p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
+    if mi.cache_idx_host is not None:
+        q_chunk_idx_start = mi.cache_idx_host // cfg.qc                    # :35
+    skip = cfg.skip_masked_tiles
+    if skip is None:
+        skip = cfg.qc >= 2 and cache_idx is None
+    p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
+    p.impl = cfg.impl
+    p.carry_is_initial = 1 if _carry_is_initial else 0
+    L.check(L.load().ra_attn_fwd_block(ctypes.byref(p), _stream()), "ra_attn_fwd_block")
+    return num, den, mx
+
+
+def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_start, bias, segment_ids,
+                             causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
+                             dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
+                             precision=None, prevent_cse=True, cache_idx=None, _mask_inputs=None,
+                             _cfg=None, _delta=None, **extra):
+    """ringattention_jax.py:181-270.  ``carry`` = (dq, dk, dv, output, denominator, max_score); the
+    fp32 accumulators dq, dk, dv are added into IN PLACE and returned."""
+    cfg = _cfg or _Config(dict(causal_block_size=causal_block_size, query_chunk_size=query_chunk_size,
+                               key_chunk_size=key_chunk_size, deterministic=deterministic,
+                               attn_pdrop=attn_pdrop, dtype=dtype, **extra))
+    _check_qkv(q, k, v)
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    mi = _mask_inputs or _MaskInputs(cfg, bias, segment_ids, cache_idx, B, q.device,
+                                     k_chunk_idx_start * cfg.kc + Skv)
+    dq, dk, dv, output, den, mx = carry
+    if g.dtype != q.dtype:
+        g = g.to(q.dtype)
+    if _rows(g) != _rows(q):
+        g = g.contiguous()
+        if _rows(g) != _rows(q):
+            raise ValueError("g must share q's strides")
+    delta = _delta if _delta is not None else _bwd_delta(g, output)
+    p = L.RaAttnBwdParams()
+    p.q, p.k, p.v, p.g = q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr()
+    p.dtype = _ra_dtype(q)
+    p.B, p.Sq, p.Skv, p.H, p.D = B, Sq, Skv, H, D
+    p.q_stride_b, p.q_stride_s = _rows(q)
+    p.kv_stride_b, p.kv_stride_s = _rows(k)
+    p.delta, p.denominator, p.max_score = delta.data_ptr(), den.data_ptr(), mx.data_ptr()
+    if not (delta.stride() == den.stride() == mx.stride()):
+        raise ValueError("delta / denominator / max_score must share strides")
+    p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
+    p.dq = dq.data_ptr()
+    p.dq_stride_b, p.dq_stride_s = _rows(dq)
+    p.dk, p.dv = dk.data_ptr(), dv.data_ptr()
+    p.dkv_stride_b, p.dkv_stride_s = _rows(dk)
+    if _rows(dv) != _rows(dk):
+        raise ValueError("dk and dv must share strides")
+    if mi.cache_idx_host is not None:
+        q_chunk_idx_start = mi.cache_idx_host // cfg.qc
+    skip = cfg.skip_masked_tiles
+    if skip is None:
+        skip = cfg.qc >= 2 and cache_idx is None
+    p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
+    p.impl = cfg.impl
+    L.check(L.load().ra_attn_bwd_block(ctypes.byref(p), _stream()), "ra_attn_bwd_block")
+    return dq, dk, dv
+
+
+def _bwd_delta(g, output):
+    """dl_part of ringattention_jax.py:218: sum_d g * output, (B, H, Sq) fp32."""
+    B, Sq, H, D = g.shape
+    if output.dtype != g.dtype:
+        output = output.to(g.dtype)
+    if _rows(output) != _rows(g):
+        output = output.contiguous()
+        g = g.contiguous()
+    delta = torch.empty((B, H, Sq), dtype=torch.float32, device=g.device)
+    sb, ss = _rows(g)
+    L.check(L.load().ra_attn_bwd_delta(g.data_ptr(), output.data_ptr(), _ra_dtype(g), sb, ss, delta.data_ptr(),
+                                       delta.stride(0), delta.stride(1), B, Sq, H, D, _stream()),
+            "ra_attn_bwd_delta")
+    return delta
+
+
+def _finalize(num, den, out):
+    B, Sq, H, D = num.shape
+    nb, ns = _rows(num)
+    ob, os_ = _rows(out)
+    L.check(L.load().ra_attn_finalize(num.data_ptr(), nb, ns, den.data_ptr(), den.stride(0), den.stride(1),
+                                      out.data_ptr(), _ra_dtype(out), ob, os_, B, Sq, H, D, _stream()),
+            "ra_attn_finalize")
+
+
+def _carry_init(num, den, mx):
+    B, Sq, H, D = num.shape
+    nb, ns = _rows(num)
+    L.check(L.load().ra_attn_carry_init(num.data_ptr(), nb, ns, den.data_ptr(), mx.data_ptr(), den.stride(0),
+                                        den.stride(1), B, Sq, H, D, _stream()), "ra_attn_carry_init")
+
+
+# --------------------------------------------------------------------------- the ring
+def _q_start(cfg, mi, dev, q_len):
+    if mi.cache_idx_host is not None:
+        return mi.cache_idx_host // cfg.qc                                   # :35
+    if mi.cache_idx_dev is not None:
+        return 0            # resolved on the device from the cache_idx scalar
+    return dev * (q_len // cfg.qc)                                           # :32-33
+
+
+def _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
+    """False when the skip predicate drops every tile of this ring step (whole future shards)."""
+    if cfg.cbs is None or mi.cache_idx_dev is not None:
+        return True
+    last_q_chunk = q_start + q_len // cfg.qc - 1
+    return run_prefix_keys(last_q_chunk, cfg.qc, cfg.kc, cfg.cbs, k_start, kv_len) > 0
+
+
+def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
+    """ringattention_jax.py:17-53 for every device of the virtual ring.
+
+    Logits, softmax statistics and the carry are always fp32 (what float32_logits=True asks for;
+    with False the reference computes them in the input dtype, which this path exceeds).
+    Returns (out, residuals)."""
+    cfg = _Config(blockwise_kwargs)
+    _check_qkv(q, k, v)
+    q, k, v = (t if (t.stride(3) == 1 and t.stride(2) == t.shape[3]) else t.contiguous() for t in (q, k, v))
+    n = axis_size(axis_name)
+    B, q_total, H, D = q.shape
+    kv_total = k.shape[1]
+    if q_total % n or kv_total % n:
+        raise ValueError("sequence lengths must divide by the ring size %d" % n)
+    q_len, kv_len = q_total // n, kv_total // n
+    if q_len % cfg.qc or kv_len % cfg.kc:
+        raise ValueError("per-device lengths (%d, %d) must divide by the chunk sizes (%d, %d)"
+                         % (q_len, kv_len, cfg.qc, cfg.kc))
+    mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, kv_total)
+    if cfg.skip_masked_tiles is None:
+        cfg.skip_masked_tiles = bool(cfg.qc >= 2 and cache_idx is None and q_total == kv_total)
+    num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)      # :22
+    den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)         # :23
+    mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)          # :49
+    for dev in range(n):
+        qs = slice(dev * q_len, (dev + 1) * q_len)
+        carry = (num[:, qs], den[:, :, qs], mx[:, :, qs])
+        started = False
+        for idx in range(n):                                                          # :50-51
+            k_blk = (dev - idx) % n                                                   # :36
+            k_start = k_blk * (kv_len // cfg.kc)                                      # :37
+            q_start = _q_start(cfg, mi, dev, q_len)
+            if not _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
+                continue
+            ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, q_start, k_start, None, None,
+                                     cfg.cbs, cfg.qc, cfg.kc, _mask_inputs=mi, _cfg=cfg,
+                                     _carry_is_initial=not started, cache_idx=cache_idx)
+            started = True
+        if not started:
+            _carry_init(*carry)
+    out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
+    _finalize(num, den, out)                                                          # :52
+    del num
+    return out, (out, q, k, v, mi, cfg, n, den, mx)
+
+
+def _ring_attention_bwd(res, g):
+    """ringattention_jax.py:55-90 for every device of the virtual ring; returns dq, dk, dv in the
+    primal dtype (accumulated in fp32)."""
+    out, q, k, v, mi, cfg, n, den, mx = res
+    B, q_total, H, D = q.shape
+    kv_total = k.shape[1]
+    q_len, kv_len = q_total // n, kv_total // n
+    g = g.to(q.dtype).contiguous()
+    delta = _bwd_delta(g, out)
+    dq = torch.zeros((B, q_total, H, D), dtype=torch.float32, device=q.device)        # :61
+    dk = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)       # :62
+    dv = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)       # :63
+    for dev in range(n):
+        qs = slice(dev * q_len, (dev + 1) * q_len)
+        for idx in range(n):                                                          # :88
+            k_blk = (dev - idx) % n
+            k_start = k_blk * (kv_len // cfg.kc)
+            q_start = _q_start(cfg, mi, dev, q_len)
+            if not _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
+                continue
+            ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            # the dk/dv partials ride with their K/V shard (:85-86): accumulate at the shard's home
+            _blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], g[:, qs],
+                                     (dq[:, qs], dk[:, ks], dv[:, ks], out[:, qs], den[:, :, qs], mx[:, :, qs]),
+                                     q_start, k_start, None, None, cfg.cbs, cfg.qc, cfg.kc,
+                                     _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs])
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
+
+
+class _RingAttentionFn(torch.autograd.Function):
+    """custom_vjp of ringattention_jax.py:92-97: cotangents for q, k, v only (:90)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
+        out, res = _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits,
+                                       blockwise_kwargs)
+        ctx.res = res
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        dq, dk, dv = _ring_attention_bwd(ctx.res, g)
+        ctx.res = None
+        return dq, dk, dv, None, None, None, None, None, None
+
+
+def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
+    """Drop-in for ringattention_jax.py:92-97 (exported as ``ringattention``).
+
+    q, k, v: (B, S, H, D) device tensors, bf16 or fp32; with a declared ring axis they are the global
+    arrays and the sequence axis is split over the virtual devices.  attn_bias (B|1, H|1, 1, K_total)
+    and segment_ids (B|1, S_total) are global / replicated, as in the reference's shard_map specs.
+    One query token with cache_idx set takes the streaming decode kernel."""
+    if cache_idx is not None and q.shape[1] == 1 and axis_size(axis_name) == 1 and not (
+            torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
+        from .decode import decode_attention
+        return decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs)
+    return _RingAttentionFn.apply(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits,
+                                  blockwise_kwargs)

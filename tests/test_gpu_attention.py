@@ -1,0 +1,153 @@
+"""Parity of the HIP attention path (through the C-ABI) with the CPU oracle.
+
+Bar: forward output and dq/dk/dv within max-abs 1e-4 (fp32 inputs) or 2e-2 (bf16 inputs) and
+relative L2 <= 1e-2; NaN rows (no tile runs) must coincide; masked keys must have bitwise no effect.
+"""
+import pytest
+import torch
+
+import ringattention_amd as ra
+from tests.util import (assert_close, errors, kwargs, make_qkv, oracle_fwd_bwd, packed_segment_ids)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def run_hip(q, k, v, do, bias, seg, cache_idx, n, kw, name="sp"):
+    qd, kd, vd = (t.to(DEV).requires_grad_(do is not None) for t in (q, k, v))
+    bd = bias.to(DEV) if bias is not None else None
+    sd = seg.to(DEV) if seg is not None else None
+    with ra.ring_axis(name, n):
+        out = ra.ringattention(qd, kd, vd, bd, sd, cache_idx, axis_name=name, float32_logits=True,
+                               blockwise_kwargs=kw)
+        grads = None
+        if do is not None:
+            out.backward(do.to(DEV))
+            grads = (qd.grad, kd.grad, vd.grad)
+    torch.cuda.synchronize()
+    return out, grads
+
+
+def check_case(B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, dtype, impl="auto", seed=0, bwd=True,
+               seg_mean=None, bias_heads=False):
+    print("case", dict(B=B, S=S, H=H, D=D, qc=qc, kc=kc, cbs=cbs, n=n, bias=use_bias, seg=use_seg,
+                       dtype=str(dtype), impl=impl), flush=True)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=seed, scale=1.0)
+    g = torch.Generator().manual_seed(seed + 100)
+    bias = torch.randn(B, H if bias_heads else 1, 1, S, generator=g) if use_bias else None
+    seg = packed_segment_ids(B, S, seg_mean or max(4, S // 6), seed=seed + 7) if use_seg else None
+    kw = kwargs(qc, kc, cbs, dtype=torch.float32, impl=impl)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do if bwd else None, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do if bwd else None, bias, seg, None, n, kw)
+    assert out.dtype == dtype and out.shape == q.shape
+    assert_close(out, ref_out, dtype, "out")
+    if bwd:
+        for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+            assert a.dtype == dtype
+            assert_close(a, b, dtype, name)
+
+
+# --- BASELINE config 1: the reference's own CPU-runnable case
+def test_config1_fp32_fwd_bwd():
+    B, S, H, D = 1, 2048, 8, 64
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=0)
+    bias = torch.zeros(1, 1, 1, S)
+    seg = torch.zeros(1, S, dtype=torch.int32)
+    kw = kwargs(512, 512, 1, dtype=torch.float32)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, 1, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, 1, kw)
+    assert_close(out, ref_out, torch.float32, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, torch.float32, name)
+
+
+GENERIC_CASES = [
+    # B, S, H, D, qc, kc, cbs, n, bias, seg, dtype
+    (2, 128, 2, 32, 32, 32, 1, 1, False, False, torch.float32),
+    (2, 128, 2, 32, 32, 32, 1, 2, True, True, torch.float32),
+    (1, 192, 3, 64, 16, 32, 1, 3, True, True, torch.float32),
+    (1, 256, 2, 64, 64, 16, 1, 4, True, False, torch.float32),
+    (1, 256, 2, 64, 32, 32, 8, 2, False, True, torch.float32),
+    (1, 256, 2, 64, 8, 8, 32, 2, True, True, torch.float32),
+    (1, 128, 2, 64, 32, 32, None, 2, True, True, torch.float32),
+    (1, 128, 2, 64, 32, 32, None, 1, False, False, torch.float32),
+    (1, 200, 1, 32, 20, 10, 1, 2, False, False, torch.float32),
+    (1, 256, 2, 128, 64, 64, 1, 2, True, True, torch.float32),
+    (2, 256, 4, 128, 64, 64, 1, 2, True, True, torch.bfloat16),
+    (1, 256, 2, 64, 32, 64, 1, 1, False, True, torch.bfloat16),
+    (1, 128, 2, 32, 2, 2, 1, 1, False, False, torch.float32),
+]
+
+
+@pytest.mark.parametrize("case", GENERIC_CASES)
+def test_generic_kernels_match_oracle(case):
+    B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, dtype = case
+    check_case(B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, dtype, impl="generic")
+
+
+def test_bias_per_head_and_batch():
+    check_case(2, 128, 3, 32, 32, 32, 1, 2, True, True, torch.float32, impl="generic", bias_heads=True)
+
+
+def test_ring_sizes_agree_with_single_device():
+    B, S, H, D = 1, 512, 2, 64
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=3)
+    seg = packed_segment_ids(B, S, 100, seed=4)
+    kw = kwargs(32, 32, 1, impl="generic")
+    base, gb = run_hip(q, k, v, do, None, seg, None, 1, kw)
+    for n in (2, 4, 8):
+        o, gg = run_hip(q, k, v, do, None, seg, None, n, kw)
+        assert errors(o, base)[0] < 2e-6
+        for a, b in zip(gg, gb):
+            assert errors(a, b)[0] < 2e-5
+
+
+def test_masked_keys_are_bitwise_isolated():
+    B, S, H, D = 1, 256, 2, 64
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=5)
+    kw = kwargs(32, 32, 1, impl="generic")
+    a, ga = run_hip(q, k, v, do, None, None, None, 2, kw)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, 150:] += 50.0
+    v2[:, 150:] -= 20.0
+    do2 = do.clone()
+    do2[:, 150:] = 0.0
+    b, gb = run_hip(q, k2, v2, do, None, None, None, 2, kw)
+    assert torch.equal(a[:, :150], b[:, :150])
+    # with no cotangent on rows >= 150, keys >= 150 get exactly zero gradient and dq rows < 150 do not move
+    c, gc = run_hip(q, k, v, do2, None, None, None, 2, kw)
+    d, gd = run_hip(q, k2, v2, do2, None, None, None, 2, kw)
+    assert torch.equal(gc[0][:, :150], gd[0][:, :150])
+    assert float(gd[1][:, 150:].abs().max()) == 0.0 and float(gd[2][:, 150:].abs().max()) == 0.0
+
+
+def test_blockwise_fwd_carry_roundtrip_matches_oracle():
+    """_blockwise_attention_fwd called step by step with an explicit carry, like the ring does."""
+    from oracle import ringattention_oracle as O
+    B, S, H, D = 1, 128, 2, 32
+    q, k, v, _ = make_qkv(B, S, H, D, seed=9)
+    kw = kwargs(16, 16, 1)
+    okw = {kk: vv for kk, vv in kw.items()}
+    num = torch.zeros(B, 64, H, D)
+    den = torch.zeros(B, H, 64)
+    mx = torch.full((B, H, 64), float("-inf"))
+    # device 1 of a ring of 2: its own shard (step 0), then shard 0 (step 1)
+    ref = (num, den, mx)
+    ref = O.blockwise_attention_fwd(q[:, 64:], k[:, 64:], v[:, 64:], ref, 4, 4, None, None, **okw)
+    ref = O.blockwise_attention_fwd(q[:, 64:], k[:, :64], v[:, :64], ref, 4, 0, None, None, **okw)
+    carry = tuple(t.to(DEV) for t in (num, den, mx))
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    ra._blockwise_attention_fwd(qd[:, 64:], kd[:, 64:], vd[:, 64:], carry, 4, 4, None, None, impl="generic", **kw)
+    ra._blockwise_attention_fwd(qd[:, 64:], kd[:, :64], vd[:, :64], carry, 4, 0, None, None, impl="generic", **kw)
+    torch.cuda.synchronize()
+    for a, b, name in zip(carry, ref, ("numerator", "denominator", "max_score")):
+        assert errors(a, b)[0] < 1e-4, name
+
+
+def test_invalid_shapes_raise():
+    q = torch.zeros(1, 100, 1, 64, device=DEV)
+    with pytest.raises(ValueError):
+        ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1))
+    q = torch.zeros(1, 64, 1, 48, device=DEV)
+    with pytest.raises(NotImplementedError):
+        ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1))

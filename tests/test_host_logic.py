@@ -1,0 +1,91 @@
+"""CPU tests of the host side: the C-ABI library loads and exports every declared symbol, the
+closed-form run prefix equals the reference predicate, argument checking raises like the reference."""
+import os
+import re
+
+import pytest
+import torch
+
+import ringattention_amd as ra
+from ringattention_amd import _lib
+from oracle import ringattention_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "ringattn_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ra_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations parsed"
+    assert declared == set(_lib.SYMBOLS), declared ^ set(_lib.SYMBOLS)
+    lib = _lib.load()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.ra_version() >= 1
+
+
+def test_struct_sizes_match_a_c_compiler(tmp_path):
+    import ctypes
+    import subprocess
+    src = tmp_path / "sz.c"
+    src.write_text('#include <stdio.h>\n#include "%s"\nint main(){printf("%%zu %%zu %%zu %%zu %%zu\\n",'
+                   'sizeof(ra_mask),sizeof(ra_attn_fwd_params),sizeof(ra_attn_bwd_params),'
+                   'sizeof(ra_decode_params),sizeof(ra_swiglu_params));return 0;}\n'
+                   % os.path.join(ROOT, "include", "ringattn_hip.h"))
+    exe = tmp_path / "sz"
+    subprocess.check_call(["gcc", str(src), "-o", str(exe)])
+    sizes = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    mine = [ctypes.sizeof(c) for c in (_lib.RaMask, _lib.RaAttnFwdParams, _lib.RaAttnBwdParams,
+                                       _lib.RaDecodeParams, _lib.RaSwigluParams)]
+    assert sizes == mine
+
+
+@pytest.mark.parametrize("qc,kc,cbs", [(1, 1, 1), (1, 8, 1), (2, 2, 1), (4, 8, 1), (8, 4, 1), (4, 4, 8),
+                                       (4, 4, 2), (2, 8, 4), (8, 2, 16), (3, 5, 1), (512, 512, 1)])
+def test_run_prefix_equals_predicate(qc, kc, cbs):
+    nkv = 12
+    for k_start in (0, 3, 7):
+        for r in range(0, 20):
+            runs = [bool(O.below_or_on_diag(r, qc, k_start + c, kc, cbs)) for c in range(nkv)]
+            # monotone: a prefix of the key chunks runs
+            n_run = sum(runs)
+            assert runs == [True] * n_run + [False] * (nkv - n_run)
+            assert ra.run_prefix_keys(r, qc, kc, cbs, k_start, nkv * kc) == n_run * kc
+            assert bool(ra.below_or_on_diag(r, qc, k_start, kc, cbs)) == runs[0]
+
+
+def test_ring_axis_registry():
+    assert ra.axis_size("sp") == 1
+    with ra.ring_axis("sp", 8):
+        assert ra.axis_size("sp") == 8
+        with ra.ring_axis("sp", 2):
+            assert ra.axis_size("sp") == 2
+        assert ra.axis_size("sp") == 8
+    assert ra.axis_size("sp") == 1
+    assert ra.axis_size(None) == 1
+
+
+def test_cpu_tensors_are_refused():
+    q = torch.zeros(1, 8, 1, 64)
+    kw = dict(causal_block_size=1, query_chunk_size=4, key_chunk_size=4, dtype=torch.float32)
+    with pytest.raises(RuntimeError):
+        ra.ringattention(q, q, q, None, None, None, "sp", True, kw)
+
+
+def test_dropout_is_refused():
+    from ringattention_amd.ringattention_hip import _Config
+    with pytest.raises(NotImplementedError):
+        _Config(dict(causal_block_size=1, query_chunk_size=4, key_chunk_size=4, deterministic=False,
+                     attn_pdrop=0.1, dtype=torch.float32))
+
+
+def test_invalid_arguments_return_codes_without_gpu():
+    import ctypes
+    lib = _lib.load()
+    assert lib.ra_attn_fwd_block(None, None) == _lib.RA_ERR_INVALID
+    assert b"null" in lib.ra_last_error()
+    p = _lib.RaAttnFwdParams()
+    assert lib.ra_attn_fwd_block(ctypes.byref(p), None) == _lib.RA_ERR_INVALID
+    assert lib.ra_decode_fwd(None, None) == _lib.RA_ERR_INVALID
+    assert lib.ra_decode_workspace_bytes(16, 1024, 32, 128, 4) == 16 * 32 * 4 * 130 * 4
