@@ -151,3 +151,47 @@ def test_invalid_shapes_raise():
     q = torch.zeros(1, 64, 1, 48, device=DEV)
     with pytest.raises(NotImplementedError):
         ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1))
+
+
+# --------------------------------------------------------------------------- MFMA kernels (bf16, D=128)
+MFMA_FWD_CASES = [
+    # B, S, H, qc, kc, cbs, n, bias, seg
+    (1, 256, 1, 128, 64, 1, 1, False, False),
+    (1, 512, 2, 128, 128, 1, 1, False, False),
+    (2, 512, 2, 256, 128, 1, 2, True, True),
+    (1, 1024, 2, 128, 64, 1, 4, False, True),
+    (1, 1024, 1, 256, 256, 1, 1, True, False),
+    (1, 512, 2, 128, 128, None, 2, True, True),
+    (1, 512, 2, 128, 128, None, 1, False, False),
+    (1, 1024, 1, 128, 128, 256, 2, False, False),
+    (1, 1024, 1, 128, 64, 32, 1, False, True),
+    (1, 2048, 2, 512, 512, 1, 2, False, True),
+]
+
+
+@pytest.mark.parametrize("case", MFMA_FWD_CASES)
+def test_mfma_forward_matches_oracle(case):
+    B, S, H, qc, kc, cbs, n, use_bias, use_seg = case
+    check_case(B, S, H, 128, qc, kc, cbs, n, use_bias, use_seg, torch.bfloat16, impl="mfma", bwd=False,
+               seg_mean=S // 5)
+
+
+def test_mfma_forward_matches_generic_kernels_at_4k():
+    """Beyond what the CPU oracle does quickly: the two kernel families against each other."""
+    B, S, H, D = 1, 4096, 4, 128
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=11, scale=D ** -0.25)
+    seg = packed_segment_ids(B, S, 700, seed=12)
+    g = torch.Generator().manual_seed(13)
+    bias = torch.randn(B, 1, 1, S, generator=g)
+    outs = {}
+    for impl in ("generic", "mfma"):
+        outs[impl], _ = run_hip(q, k, v, None, bias, seg, None, 4, kwargs(512, 512, 1, impl=impl))
+    assert_close(outs["mfma"], outs["generic"], torch.bfloat16, "mfma vs generic")
+
+
+def test_mfma_skip_masked_tiles_flag_is_exact_here():
+    B, S, H, D = 1, 1024, 2, 128
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=14)
+    a, _ = run_hip(q, k, v, None, None, None, None, 2, kwargs(256, 256, 1, impl="mfma", skip_masked_tiles=True))
+    b, _ = run_hip(q, k, v, None, None, None, None, 2, kwargs(256, 256, 1, impl="mfma", skip_masked_tiles=False))
+    assert torch.equal(a, b)
