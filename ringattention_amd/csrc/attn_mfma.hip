@@ -286,14 +286,424 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
   }
 }
 
+// ================================================================== backward
+// Two deterministic kernels (fp32 atomics reach ~1.3 TB/s at best on this part, far below what a
+// fused dQ accumulation would need):
+//   dQ   : query-stationary, same shape as the forward.  S^T = K Q^T and dP^T = V dO^T share the
+//          lane <-> query-column layout, so max / 1/denominator / delta are per-lane scalars;
+//          dQ^T += K^T dS^T takes K^T from the row-major K tile with LDS transpose reads.
+//   dK,dV: key-stationary.  S = Q K^T and dP = dO V^T with K / V fragments resident in registers;
+//          P and dS (accumulator layout, lane <-> key column) feed dV^T += dO^T P and
+//          dK^T += Q^T dS directly as B operands; Q^T / dO^T come from LDS transpose reads.
+// Probabilities are recomputed from the saved max_score / denominator (ringattention_jax.py:226).
+constexpr int BSTR = HD + 24;    // LDS row stride for tiles read both row-wise and transposed
+
+struct BwdArgs {
+  const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* g;
+  int B, Sq, Skv, H;
+  int64_t q_sb, q_ss, kv_sb, kv_ss;
+  const float* delta; const float* den; const float* mx;
+  int64_t st_sb, st_sh;
+  float* dq; int64_t dq_sb, dq_ss;
+  float* dk; float* dv; int64_t dkv_sb, dkv_ss;
+  MaskView mv;
+  const int32_t* cache_idx;
+};
+
+template <bool HAS_SEG, bool HAS_BIAS>
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][FBN * BSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][FBN * KSTR];
+  __shared__ int seg_ks[2][FBN];
+  __shared__ float bias_ks[2][FBN];
+
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int nqt = a.Sq / FBM;
+  int wg = blockIdx.x;
+  const int qt = nqt - 1 - (wg % nqt);
+  wg /= nqt;
+  const int h = wg % a.H, b = wg / a.H;
+  const int q0 = qt * FBM;
+  const int qrow = q0 + wave * 32 + lo;
+
+  const int qi = q0 / mv.qc;
+  int kend = mv.run_prefix_keys(qi, a.Skv);
+  const long long gq0 = mv.global_q(q0);
+  const long long gk0 = mv.global_k(0);
+  if (mv.cbs > 0 && mv.skip_tiles) {
+    long long lim = ((gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
+    long long n = lim - gk0;
+    if (n < kend) kend = n > 0 ? (int)n : 0;
+  }
+  const int ntiles = (kend + FBN - 1) / FBN;
+  if (ntiles == 0) return;     // nothing to add to dq
+
+  const long long gq = gq0 + wave * 32 + lo;
+  const long long klim = mv.cbs > 0 ? (gq / mv.cbs + 1) * mv.cbs : 0x7fffffffffffffffLL;
+  const long long klim_wave = mv.cbs > 0 ? ((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs : 0x7fffffffffffffffLL;
+  int seg_q = 0;
+  if (HAS_SEG) {
+    int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
+    seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
+  }
+  const float c = kLog2e / sqrtf((float)HD);
+  const float kMask2 = mv.mask_min;
+
+  const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
+  bf16x8 qf[8], gf[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) {
+    qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
+    gf[t] = *(const bf16x8*)(a.g + qoff + t * 16);
+  }
+  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+  const float m2 = max_to_log2(a.mx[st], kMask2);
+  const float rden = 1.f / a.den[st];
+  const float delta = a.delta[st];
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+
+  const int srow = tid >> 4, schunk = tid & 15;
+  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8;
+  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8;
+  uint4 kr[4], vr[4];
+  int seg_r = 0;
+  float bias_r = 0.f;
+  auto load_tile = [&](int j) {
+    const int k0 = j * FBN;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const int64_t off = (int64_t)(k0 + p * 16 + srow) * a.kv_ss;
+      kr[p] = *(const uint4*)(kg + off);
+      vr[p] = *(const uint4*)(vg + off);
+    }
+    if (tid < FBN) {
+      const int kj = k0 + tid;
+      if (HAS_SEG) {
+        int idx = clamp_seg_index(((long long)mv.k_start + kj / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
+        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx];
+      }
+      if (HAS_BIAS) {
+        float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (gk0 + kj) * mv.bias_sk];
+        if (mv.any_mask) bv = fminf(bv, 0.f);
+        bias_r = bv * kLog2e;
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      *(uint4*)(&Ks[buf][(p * 16 + srow) * BSTR + schunk * 8]) = kr[p];
+      *(uint4*)(&Vs[buf][(p * 16 + srow) * KSTR + schunk * 8]) = vr[p];
+    }
+    if (tid < FBN) {
+      if (HAS_SEG) seg_ks[buf][tid] = seg_r;
+      if (HAS_BIAS) bias_ks[buf][tid] = bias_r;
+    }
+  };
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+
+  const int ktr_lane_off = ((lane & 15) >> 2) * BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * BSTR;
+  const int k_lane_off = lo * BSTR + hi * 8;
+  const int v_lane_off = lo * KSTR + hi * 8;
+
+  for (int j = 0; j < ntiles; j++) {
+    const int cur = j & 1;
+    const bool more = j + 1 < ntiles;
+    if (more) load_tile(j + 1);
+    const long long gk_tile = gk0 + (long long)j * FBN;
+    const bool need_mask = HAS_SEG || HAS_BIAS || (gk_tile + FBN - 1 >= klim_wave);
+
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+      f32x16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+      const uint16_t* kp = &Ks[cur][blk * 32 * BSTR + k_lane_off];
+      const uint16_t* vp = &Vs[cur][blk * 32 * KSTR + v_lane_off];
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        bf16x8 kf = *(const bf16x8*)(kp + t * 16);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s, 0, 0, 0);          // S^T = K Q^T
+      }
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        bf16x8 vf = *(const bf16x8*)(vp + t * 16);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, gf[t], dp, 0, 0, 0);        // dP^T = V dO^T
+      }
+      bf16x8 dsf[2];
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float p;
+        if (!need_mask) {
+          p = fast_exp2(fmaf(s[r], c, -m2)) * rden;
+        } else {
+          const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+          float x = s[r] * c;
+          if (HAS_BIAS) x += bias_ks[cur][kr_];
+          bool masked = (gk_tile + kr_ >= klim);
+          if (HAS_SEG) masked = masked || (seg_ks[cur][kr_] != seg_q);
+          x = masked ? kMask2 : x;
+          p = fast_exp2(x - m2) * rden;                                              // :226
+        }
+        dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - delta));                          // :229
+      }
+      // dQ^T += K^T dS^T over these 32 keys
+      const uint16_t* ktp = &Ks[cur][blk * 32 * BSTR + ktr_lane_off];
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+          s16x4 k0v = lds_read_tr(ktp + t * 16 * BSTR + db * 32);
+          s16x4 k1v = lds_read_tr(ktp + (t * 16 + 8) * BSTR + db * 32);
+          s16x8 kk = __builtin_shufflevector(k0v, k1v, 0, 1, 2, 3, 4, 5, 6, 7);
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), dsf[t], acc[db], 0, 0, 0);
+        }
+    }
+    if (more) store_tile(cur ^ 1);
+    __syncthreads();
+  }
+
+  // dq += acc / sqrt(D)   (:230)
+  const float rscale = 1.f / sqrtf((float)HD);
+  float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      f32x4 t = *(const f32x4*)(dqp + db * 32 + g * 8);
+      t[0] += acc[db][g * 4 + 0] * rscale; t[1] += acc[db][g * 4 + 1] * rscale;
+      t[2] += acc[db][g * 4 + 2] * rscale; t[3] += acc[db][g * 4 + 3] * rscale;
+      *(f32x4*)(dqp + db * 32 + g * 8) = t;
+    }
+}
+
+constexpr int KBN = 128;   // keys per workgroup in the dK/dV kernel (32 per wavefront)
+constexpr int KBM = 64;    // query rows per step
+
+template <bool HAS_SEG, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][KBM * BSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t Gs[2][KBM * BSTR];
+  __shared__ __attribute__((aligned(16))) float st_m2[2][KBM];
+  __shared__ __attribute__((aligned(16))) float st_rden[2][KBM];
+  __shared__ __attribute__((aligned(16))) float st_delta[2][KBM];
+  __shared__ __attribute__((aligned(16))) int st_seg[2][KBM];
+
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int nkt = a.Skv / KBN;
+  int wg = blockIdx.x;
+  const int kt = wg % nkt;                 // earliest key blocks (most query tiles under causal) first
+  wg /= nkt;
+  const int h = wg % a.H, b = wg / a.H;
+  const int k0 = kt * KBN;
+  const int krow = k0 + wave * 32 + lo;    // this lane's key row (local)
+
+  const long long gk0 = mv.global_k(k0);
+  const long long gk = gk0 + wave * 32 + lo;
+  const long long gq_base = mv.global_q(0);
+  // first query tile that has work for this key block: run prefix (chunk level), then sub-tile clip
+  const int nqt = a.Sq / KBM;
+  int qt_first = nqt;
+  {
+    // the run prefix is non-decreasing in the query chunk index: binary search the first chunk that reaches k0
+    int nqc = a.Sq / mv.qc, lo_c = 0, hi_c = nqc;
+    while (lo_c < hi_c) {
+      int mid = (lo_c + hi_c) >> 1;
+      if (mv.run_prefix_keys(mid, a.Skv) > k0) hi_c = mid; else lo_c = mid + 1;
+    }
+    if (lo_c < nqc) qt_first = lo_c * (mv.qc / KBM);
+    if (mv.cbs > 0 && mv.skip_tiles && qt_first < nqt) {
+      // query tiles whose every row is masked against every key of the block: (gq_max / cbs) < (gk_min / cbs)
+      long long need = (gk0 / mv.cbs) * mv.cbs - gq_base;     // first local query row that can see key gk0
+      if (need > 0) {
+        int t = (int)(need / KBM);
+        if (t > qt_first) qt_first = t < nqt ? t : nqt;
+      }
+    }
+  }
+  if (qt_first >= nqt) return;            // no query sees this key block: dk, dv unchanged
+
+  // masked iff gq / cbs < gk / cbs  <=>  gq < qlim
+  const long long qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffffffffffffLL;
+  const long long qlim_wave = mv.cbs > 0 ? ((gk0 + wave * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffffffffffffLL;
+  int seg_k = 0;
+  float bias2 = 0.f;
+  if (HAS_SEG) {
+    int idx = clamp_seg_index(((long long)mv.k_start + krow / mv.kc) * mv.kc, mv.kc, mv.seg_len, krow % mv.kc);
+    seg_k = mv.seg[(int64_t)b * mv.seg_sb + idx];
+  }
+  if (HAS_BIAS) {
+    float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + gk * mv.bias_sk];
+    if (mv.any_mask) bv = fminf(bv, 0.f);
+    bias2 = bv * kLog2e;
+  }
+  const float c = kLog2e / sqrtf((float)HD);
+  const float kMask2 = mv.mask_min;
+
+  // K and V fragments of this lane's key column (B operands), resident for the whole loop
+  const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
+  bf16x8 kf[8], vf[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) {
+    kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
+    vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
+  }
+  f32x16 dkacc[4], dvacc[4];
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+
+  const int srow = tid >> 4, schunk = tid & 15;
+  const uint16_t* qg = a.q + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8;
+  const uint16_t* gg = a.g + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8;
+  uint4 qr[4], gr[4];
+  float r_m2 = 0.f, r_rden = 0.f, r_delta = 0.f;
+  int r_seg = 0;
+  auto load_tile = [&](int qt) {
+    const int q0 = qt * KBM;
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const int64_t off = (int64_t)(q0 + p * 16 + srow) * a.q_ss;
+      qr[p] = *(const uint4*)(qg + off);
+      gr[p] = *(const uint4*)(gg + off);
+    }
+    if (tid < KBM) {
+      const int row = q0 + tid;
+      const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row;
+      r_m2 = max_to_log2(a.mx[st], kMask2);
+      r_rden = 1.f / a.den[st];
+      r_delta = a.delta[st];
+      if (HAS_SEG) {
+        int idx = clamp_seg_index(((long long)mv.q_start + row / mv.qc) * mv.qc, mv.qc, mv.seg_len, row % mv.qc);
+        r_seg = mv.seg[(int64_t)b * mv.seg_sb + idx];
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      *(uint4*)(&Qs[buf][(p * 16 + srow) * BSTR + schunk * 8]) = qr[p];
+      *(uint4*)(&Gs[buf][(p * 16 + srow) * BSTR + schunk * 8]) = gr[p];
+    }
+    if (tid < KBM) {
+      st_m2[buf][tid] = r_m2; st_rden[buf][tid] = r_rden; st_delta[buf][tid] = r_delta;
+      if (HAS_SEG) st_seg[buf][tid] = r_seg;
+    }
+  };
+  load_tile(qt_first);
+  store_tile(0);
+  __syncthreads();
+
+  const int tr_lane_off = ((lane & 15) >> 2) * BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * BSTR;
+  const int nat_lane_off = lo * BSTR + hi * 8;
+
+  for (int qt = qt_first; qt < nqt; qt++) {
+    const int cur = (qt - qt_first) & 1;
+    const bool more = qt + 1 < nqt;
+    if (more) load_tile(qt + 1);
+    const long long gq_tile = gq_base + (long long)qt * KBM;
+    const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave);
+
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+      f32x16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+      const uint16_t* qp = &Qs[cur][qb * 32 * BSTR + nat_lane_off];
+      const uint16_t* gp = &Gs[cur][qb * 32 * BSTR + nat_lane_off];
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        bf16x8 qa = *(const bf16x8*)(qp + t * 16);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[t], s, 0, 0, 0);          // S = Q K^T
+      }
+#pragma unroll
+      for (int t = 0; t < 8; t++) {
+        bf16x8 ga = *(const bf16x8*)(gp + t * 16);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[t], dp, 0, 0, 0);        // dP = dO V^T
+      }
+      bf16x8 pf[2], dsf[2];
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int qrow0 = qb * 32 + g * 8 + hi * 4;          // rows qrow0 .. +3 of the tile
+        const f32x4 vm2 = *(const f32x4*)&st_m2[cur][qrow0];
+        const f32x4 vrd = *(const f32x4*)&st_rden[cur][qrow0];
+        const f32x4 vdl = *(const f32x4*)&st_delta[cur][qrow0];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int r = g * 4 + e;
+          float p;
+          if (!need_mask) {
+            p = fast_exp2(fmaf(s[r], c, -vm2[e])) * vrd[e];
+          } else {
+            float x = s[r] * c;
+            if (HAS_BIAS) x += bias2;
+            bool masked = (gq_tile + qrow0 + e < qlim);
+            if (HAS_SEG) masked = masked || (st_seg[cur][qrow0 + e] != seg_k);
+            x = masked ? kMask2 : x;
+            p = fast_exp2(x - vm2[e]) * vrd[e];
+          }
+          pf[r >> 3][r & 7] = (__bf16)p;
+          dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - vdl[e]));
+        }
+      }
+      // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over these 32 query rows)
+      const uint16_t* gtp = &Gs[cur][qb * 32 * BSTR + tr_lane_off];
+      const uint16_t* qtp = &Qs[cur][qb * 32 * BSTR + tr_lane_off];
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+          s16x4 g0 = lds_read_tr(gtp + t * 16 * BSTR + db * 32);
+          s16x4 g1 = lds_read_tr(gtp + (t * 16 + 8) * BSTR + db * 32);
+          s16x8 gv = __builtin_shufflevector(g0, g1, 0, 1, 2, 3, 4, 5, 6, 7);
+          dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, gv), pf[t], dvacc[db], 0, 0, 0);
+          s16x4 q0v = lds_read_tr(qtp + t * 16 * BSTR + db * 32);
+          s16x4 q1v = lds_read_tr(qtp + (t * 16 + 8) * BSTR + db * 32);
+          s16x8 qv = __builtin_shufflevector(q0v, q1v, 0, 1, 2, 3, 4, 5, 6, 7);
+          dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), dsf[t], dkacc[db], 0, 0, 0);
+        }
+    }
+    if (more) store_tile(cur ^ 1);
+    __syncthreads();
+  }
+
+  // dk += acc / sqrt(D) (:231), dv += acc (:232); this workgroup owns its key rows
+  const float rscale = 1.f / sqrtf((float)HD);
+  const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      float* pk = a.dk + ooff + db * 32 + g * 8;
+      float* pv = a.dv + ooff + db * 32 + g * 8;
+      f32x4 tk = *(const f32x4*)pk, tv = *(const f32x4*)pv;
+#pragma unroll
+      for (int e = 0; e < 4; e++) { tk[e] += dkacc[db][g * 4 + e] * rscale; tv[e] += dvacc[db][g * 4 + e]; }
+      *(f32x4*)pk = tk; *(f32x4*)pv = tv;
+    }
+}
+
 // ------------------------------------------------------------------ host side
+static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
+
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
   const ra_mask& m = p->mask;
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
          (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
-         ((uintptr_t)p->q % 16 == 0) && ((uintptr_t)p->k % 16 == 0) && ((uintptr_t)p->v % 16 == 0) &&
-         ((uintptr_t)p->numerator % 16 == 0);
+         aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator);
 }
 
 int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
@@ -318,10 +728,45 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   return RA_OK;
 }
 
-bool attn_bwd_mfma_supported(const ra_attn_bwd_params*) { return false; }
-int attn_bwd_mfma(const ra_attn_bwd_params*, hipStream_t) {
-  set_error("mfma bwd: not built");
-  return RA_ERR_UNSUPPORTED;
+bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
+  const ra_mask& m = p->mask;
+  return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % KBN == 0 &&
+         (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
+         p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0 &&
+         p->dkv_stride_s % 4 == 0 && p->dkv_stride_b % 4 == 0 && aligned16(p->q) && aligned16(p->k) &&
+         aligned16(p->v) && aligned16(p->g) && aligned16(p->dq) && aligned16(p->dk) && aligned16(p->dv);
+}
+
+int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
+  BwdArgs a{};
+  a.q = (const uint16_t*)p->q; a.k = (const uint16_t*)p->k; a.v = (const uint16_t*)p->v; a.g = (const uint16_t*)p->g;
+  a.B = p->B; a.Sq = p->Sq; a.Skv = p->Skv; a.H = p->H;
+  a.q_sb = p->q_stride_b; a.q_ss = p->q_stride_s; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s;
+  a.delta = p->delta; a.den = p->denominator; a.mx = p->max_score;
+  a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
+  a.dq = p->dq; a.dq_sb = p->dq_stride_b; a.dq_ss = p->dq_stride_s;
+  a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
+  a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
+  a.cache_idx = p->mask.cache_idx;
+  const long long nq = (long long)(p->Sq / FBM) * p->H * p->B, nk = (long long)(p->Skv / KBN) * p->H * p->B;
+  RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_mfma: grid too large");
+  dim3 gq((unsigned)nq), gk((unsigned)nk), block(256);
+  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
+  if (seg && bias) {
+    attn_bwd_dkv_mfma_kernel<true, true><<<gk, block, 0, s>>>(a);
+    attn_bwd_dq_mfma_kernel<true, true><<<gq, block, 0, s>>>(a);
+  } else if (seg) {
+    attn_bwd_dkv_mfma_kernel<true, false><<<gk, block, 0, s>>>(a);
+    attn_bwd_dq_mfma_kernel<true, false><<<gq, block, 0, s>>>(a);
+  } else if (bias) {
+    attn_bwd_dkv_mfma_kernel<false, true><<<gk, block, 0, s>>>(a);
+    attn_bwd_dq_mfma_kernel<false, true><<<gq, block, 0, s>>>(a);
+  } else {
+    attn_bwd_dkv_mfma_kernel<false, false><<<gk, block, 0, s>>>(a);
+    attn_bwd_dq_mfma_kernel<false, false><<<gq, block, 0, s>>>(a);
+  }
+  RA_CHECK_LAUNCH("attn_bwd_mfma");
+  return RA_OK;
 }
 
 }  // namespace ra

@@ -195,3 +195,37 @@ def test_mfma_skip_masked_tiles_flag_is_exact_here():
     a, _ = run_hip(q, k, v, None, None, None, None, 2, kwargs(256, 256, 1, impl="mfma", skip_masked_tiles=True))
     b, _ = run_hip(q, k, v, None, None, None, None, 2, kwargs(256, 256, 1, impl="mfma", skip_masked_tiles=False))
     assert torch.equal(a, b)
+
+
+MFMA_BWD_CASES = [
+    # B, S, H, qc, kc, cbs, n, bias, seg
+    (1, 256, 1, 128, 128, 1, 1, False, False),
+    (1, 512, 2, 128, 128, 1, 1, False, False),
+    (2, 512, 2, 256, 128, 1, 2, True, True),
+    (1, 1024, 2, 128, 128, 1, 4, False, True),
+    (1, 1024, 1, 256, 256, 1, 1, True, False),
+    (1, 512, 2, 128, 128, None, 2, True, True),
+    (1, 512, 2, 128, 128, None, 1, False, False),
+    (1, 1024, 1, 128, 128, 256, 2, False, False),
+    (1, 1024, 1, 128, 128, 32, 1, False, True),
+    (1, 2048, 2, 512, 512, 1, 2, False, True),
+]
+
+
+@pytest.mark.parametrize("case", MFMA_BWD_CASES)
+def test_mfma_backward_matches_oracle(case):
+    B, S, H, qc, kc, cbs, n, use_bias, use_seg = case
+    check_case(B, S, H, 128, qc, kc, cbs, n, use_bias, use_seg, torch.bfloat16, impl="mfma", bwd=True,
+               seg_mean=S // 5)
+
+
+def test_mfma_backward_matches_generic_kernels_at_4k():
+    B, S, H, D = 1, 4096, 2, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=D ** -0.25)
+    seg = packed_segment_ids(B, S, 700, seed=22)
+    res = {}
+    for impl in ("generic", "mfma"):
+        res[impl] = run_hip(q, k, v, do, None, seg, None, 2, kwargs(512, 512, 1, impl=impl))
+    assert_close(res["mfma"][0], res["generic"][0], torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), res["mfma"][1], res["generic"][1]):
+        assert_close(a, b, torch.bfloat16, name)
