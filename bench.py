@@ -1,0 +1,313 @@
+#!/usr/bin/env python3
+"""Benchmark of the ring-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode]
+
+One step = one pass of the hot path over one batch of synthetic input already resident in HBM.
+Default workload ``attn32k`` is the configuration the headline metric is quoted on: blockwise
+causal attention forward+backward, bf16, B=1 H=32 S=32768 D=128, chunks 512/512.  Prints ONE JSON
+line with the throughput, the roofline figures of the dominant kernel (timed live with events on
+the launch stream) and a CPU baseline (the CPU oracle timed on a bounded slice of the workload).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+
+
+def _kwargs(qc, kc, cbs=1, **extra):
+    import torch
+    kw = dict(causal_block_size=cbs, deterministic=True, dropout_rng=None, attn_pdrop=0.0,
+              query_chunk_size=qc, key_chunk_size=kc, dtype=torch.float32, policy=None, precision=None,
+              prevent_cse=True)
+    kw.update(extra)
+    return kw
+
+
+def _time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _event_ms(fn, reps):
+    """Average duration of ``fn`` (which launches on torch's current stream) from events on that stream."""
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    total = 0.0
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn()
+        e1.record()
+        e1.synchronize()
+        total += e0.elapsed_time(e1)
+    return total / reps
+
+
+def _packed_segments(S, mean_len, seed, device):
+    import numpy as np
+    import torch
+    rng = np.random.default_rng(seed)
+    lens = []
+    tot = 0
+    while tot < S:
+        ln = int(rng.geometric(1.0 / mean_len))
+        lens.append(ln)
+        tot += ln
+    ids = np.repeat(np.arange(len(lens)), lens)[:S].astype(np.int32)
+    lens[-1] -= tot - S
+    return torch.from_numpy(ids).reshape(1, S).to(device), lens
+
+
+# --------------------------------------------------------------------------- attention workloads
+def bench_attention(args, ring):
+    import torch
+    import ringattention_amd as ra
+    from ringattention_amd import ringattention_hip as rh
+    dev = "cuda:0"
+    D, H, B = 128, 32, 1
+    if ring:
+        S, n, name = 131072, 8, "ring131k"
+    else:
+        S, n, name = 32768, 1, "attn32k"
+    if args.seq_len:
+        S = args.seq_len
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda: (torch.randn(B, S, H, D, device=dev, generator=g) * D ** -0.5).to(torch.bfloat16)
+    q, k, v = mk().requires_grad_(True), mk().requires_grad_(True), mk().requires_grad_(True)
+    do = torch.randn(B, S, H, D, device=dev, generator=g).to(torch.bfloat16)
+    bias = seg = None
+    pairs = S * (S + 1) / 2
+    if ring:
+        bias = torch.randn(1, 1, 1, S, device=dev, generator=g)
+        seg, lens = _packed_segments(S, 4096, 0, dev)
+        pairs = float(sum(l * (l + 1) / 2 for l in lens))
+    kw = _kwargs(512, 512, 1)
+    flops_fwd = 4.0 * D * pairs * B * H
+    flops_bwd = 10.0 * D * pairs * B * H
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        with ra.ring_axis("sp", n):
+            out = ra.ringattention(q, k, v, bias, seg, None, axis_name="sp", float32_logits=True, blockwise_kwargs=kw)
+            out.backward(do)
+
+    ms = _time_steps(step, args.steps, args.warmup)
+    value = (flops_fwd + flops_bwd) / (ms * 1e-3) / 1e12
+
+    # --- per-kernel durations (events on the launch stream), N=1 shape of one ring step
+    roof = None
+    kern = {}
+    if not ring:
+        with torch.no_grad():
+            cfg = rh._Config(kw)
+            mi = rh._MaskInputs(cfg, None, None, None, B, q.device, S)
+            num = torch.empty(B, S, H, D, dtype=torch.float32, device=dev)
+            den = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+            mx = torch.empty(B, H, S, dtype=torch.float32, device=dev)
+            qd, kd, vd = q.detach(), k.detach(), v.detach()
+            fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (num, den, mx), 0, 0, None, None, 1, 512, 512,
+                                                      _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True)
+            kern["attn_fwd_mfma_kernel"] = (_event_ms(fwd, 5), flops_fwd)
+            out = torch.empty_like(qd)
+            rh._finalize(num, den, out)
+            delta = rh._bwd_delta(do, out)
+            dq = torch.zeros(B, S, H, D, dtype=torch.float32, device=dev)
+            dk, dv = torch.zeros_like(dq), torch.zeros_like(dq)
+            for which, share in (("dkv", 8.0), ("dq", 2.0)):
+                cfg1 = rh._Config(dict(kw, bwd_only=which))
+                bw = lambda: rh._blockwise_attention_bwd(qd, kd, vd, do, (dq, dk, dv, out, den, mx), 0, 0, None, None,
+                                                         1, 512, 512, _mask_inputs=mi, _cfg=cfg1, _delta=delta)
+                kern["attn_bwd_%s_mfma_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
+        dom = max(kern, key=lambda n_: kern[n_][0])
+        dms, dfl = kern[dom]
+        ach = dfl / (dms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
+                "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
+    cpu = cpu_baseline_attention() if not args.no_cpu else None
+    return {
+        "metric": "attn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
+        "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+        "config": {"workload": name, "B": B, "H": H, "S": S, "D": D, "causal_block_size": 1,
+                   "query_chunk_size": 512, "key_chunk_size": 512, "virtual_ring": n,
+                   "segment_ids": bool(ring), "bias": bool(ring),
+                   "flop_convention": "4*D fwd + 10*D bwd per unmasked (q,k) pair per head"},
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+
+
+def cpu_baseline_attention():
+    """The CPU oracle (torch-CPU fp32, the reference's loop structure) on 4 of the 32 heads of the
+    attn32k workload at full S=32768: forward + backward, fp32 logits, chunks 512/512."""
+    import torch
+    from oracle import ringattention_oracle as O
+    S, D, Hc = 32768, 128, 4
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    q, k, v, do = (torch.randn(1, S, Hc, D, generator=g) * (D ** -0.5 if i < 2 else 1.0) for i in range(4))
+    kw = _kwargs(512, 512, 1)
+    t0 = time.perf_counter()
+    out, res = O.ring_attention_fwd(q, k, v, None, None, None, 1, True, kw)
+    O.ring_attention_bwd(1, True, kw, res, do)
+    dt = time.perf_counter() - t0
+    flops = 14.0 * D * (S * (S + 1) / 2) * Hc
+    return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "4 heads (of 32) at full S=32768, fwd+bwd, %.1f s" % dt}
+
+
+# --------------------------------------------------------------------------- decode workload
+def bench_decode(args):
+    import torch
+    import ringattention_amd as ra
+    dev = "cuda:0"
+    B, H, D, kc = 16, 32, 128, 512
+    Lf = args.seq_len or 262144
+    L = Lf + kc
+    k = torch.empty(B, L, H, D, dtype=torch.bfloat16, device=dev)
+    v = torch.empty(B, L, H, D, dtype=torch.bfloat16, device=dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    for b in range(B):      # filled batch row by batch row to bound the fp32 temporaries
+        k[b].copy_(torch.randn(L, H, D, device=dev, generator=g))
+        v[b].copy_(torch.randn(L, H, D, device=dev, generator=g))
+    q = torch.randn(B, 1, H, D, device=dev, generator=g).to(torch.bfloat16)
+    out = torch.empty_like(q)
+    kw = _kwargs(1, kc, 1)
+    ci = torch.zeros(1, dtype=torch.int32, device=dev)
+    state = {"t": 0}
+
+    def step():
+        ci.fill_(Lf + state["t"] % 64)      # one new token per step, read by the kernel from device memory
+        state["t"] += 1
+        ra.decode_attention(q, k, v, None, None, ci, kw, out=out)
+
+    ms = _time_steps(step, args.steps, args.warmup)
+    bytes_step = 2.0 * B * (Lf + 1) * H * D * 2
+    value = bytes_step / (ms * 1e-3) / 1e9
+    kms = _event_ms(step, 5)
+    ach = bytes_step / (kms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        from oracle import ringattention_oracle as O
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        Bc, Lc = 1, 65536
+        gq = torch.Generator().manual_seed(0)
+        qc_, kc_, vc_ = (torch.randn(Bc, n_, H, D, generator=gq).to(torch.bfloat16) for n_ in (1, Lc + kc, Lc + kc))
+        t0 = time.perf_counter()
+        O.ring_attention(qc_, kc_, vc_, None, None, Lc + 1, 1, True, _kwargs(1, kc, 1))
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(2.0 * Bc * (Lc + 2) * H * D * 2 / dt / 1e9, 3), "unit": "GB/s", "cores": cores,
+               "kind": "port", "sample": "B=1 (of 16), cache 65536 (of 262144), one step, %.1f s" % dt}
+    return {
+        "metric": "decode_hbm_gbs", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms, 3),
+        "dtype": "bf16", "pct_hbm_peak": round(100 * value / PEAK_HBM_GBS, 2),
+        "config": {"workload": "decode", "B": B, "H": H, "D": D, "cache_len": Lf, "key_chunk_size": kc,
+                   "query_chunk_size": 1, "bytes_per_step": bytes_step},
+        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+
+
+# --------------------------------------------------------------------------- feed-forward workload
+def bench_ffn(args):
+    import torch
+    import ringattention_amd as ra
+    dev = "cuda:0"
+    T, d, f, chunk = args.seq_len or 65536, 4096, 11008, 2048
+    g = torch.Generator(device=dev).manual_seed(0)
+    ff = ra.SwiGLU(d, f, device=dev)
+    x = torch.randn(1, T, d, device=dev, generator=g).to(torch.bfloat16).requires_grad_(True)
+    dy = torch.randn(1, T, d, device=dev, generator=g).to(torch.bfloat16)
+
+    def step():
+        x.grad = None
+        for p in ff.parameters():
+            p.grad = None
+        y = ra.blockwise_feedforward(ff, x, chunk)
+        y.backward(dy)
+
+    ms = _time_steps(step, args.steps, args.warmup)
+    flops = 18.0 * T * d * f
+    value = flops / (ms * 1e-3) / 1e12
+    cpu = None
+    if not args.no_cpu:
+        from oracle import ringattention_oracle as O
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        Tc = 2048
+        gc = torch.Generator().manual_seed(0)
+        xc = torch.randn(1, Tc, d, generator=gc, requires_grad=True)
+        w1, w3 = (torch.randn(d, f, generator=gc) * 0.02).requires_grad_(True), (torch.randn(d, f, generator=gc) * 0.02).requires_grad_(True)
+        w2 = (torch.randn(f, d, generator=gc) * 0.02).requires_grad_(True)
+        t0 = time.perf_counter()
+        y = O.blockwise_feedforward(lambda h_: O.swiglu(h_, w1, w2, w3), xc, Tc)
+        y.backward(torch.ones_like(y))
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(18.0 * Tc * d * f / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": "one chunk of 2048 tokens (of 65536), fwd+bwd fp32, %.1f s" % dt}
+    return {
+        "metric": "swiglu_ffn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
+        "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+        "config": {"workload": "ffn", "tokens": T, "hidden": d, "intermediate": f, "chunk_size": chunk,
+                   "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
+        "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel", "achieved": round(value, 1), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode"])
+    ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the ring is virtual); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    if args.workload in ("attn32k", "ring131k"):
+        r = bench_attention(args, ring=(args.workload == "ring131k"))
+    elif args.workload == "decode":
+        r = bench_decode(args)
+    else:
+        r = bench_ffn(args)
+    line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"],
+            "roofline": r["roofline"], "cpu_baseline": r["cpu_baseline"]}
+    for extra in ("pct_bf16_mfma_peak", "pct_hbm_peak"):
+        if extra in r:
+            line[extra] = r[extra]
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

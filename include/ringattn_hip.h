@@ -32,7 +32,11 @@ enum { RA_F32 = 0, RA_BF16 = 1 };
 enum {
   RA_IMPL_AUTO = 0,    /* MFMA kernels when the shape allows, else the generic ones */
   RA_IMPL_GENERIC = 1, /* fp32 vector-ALU kernels: any chunk sizes, fp32 or bf16 inputs */
-  RA_IMPL_MFMA = 2     /* bf16 MFMA kernels only; RA_ERR_UNSUPPORTED if the shape does not fit */
+  RA_IMPL_MFMA = 2,    /* bf16 MFMA kernels only; RA_ERR_UNSUPPORTED if the shape does not fit */
+  /* ra_attn_bwd_params.impl may OR in one of these to launch a single backward kernel (for timing
+     one kernel in isolation; a full backward needs both) */
+  RA_BWD_ONLY_DQ = 0x10,
+  RA_BWD_ONLY_DKV = 0x20
 };
 
 /*

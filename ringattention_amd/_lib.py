@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libringattn_hip.so")
 RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
 RA_F32, RA_BF16 = 0, 1
 RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
+RA_BWD_ONLY_DQ, RA_BWD_ONLY_DKV = 0x10, 0x20
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 

@@ -115,9 +115,10 @@ int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_bwd_block: B and H must be <= 65535");
   if (int rc = check_mask(p->mask, p->Sq, p->Skv, "attn_bwd_block")) return rc;
   hipStream_t s = (hipStream_t)stream;
-  if (p->impl == RA_IMPL_GENERIC) return attn_bwd_generic(p, s);
+  const int impl = p->impl & 0xf;
+  if (impl == RA_IMPL_GENERIC) return attn_bwd_generic(p, s);
   if (attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, s);
-  RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
+  RA_REQUIRE(impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
              "attn_bwd_block: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128");
   return attn_bwd_generic(p, s);
 }

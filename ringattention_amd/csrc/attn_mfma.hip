@@ -752,19 +752,17 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
   RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_mfma: grid too large");
   dim3 gq((unsigned)nq), gk((unsigned)nk), block(256);
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
-  if (seg && bias) {
-    attn_bwd_dkv_mfma_kernel<true, true><<<gk, block, 0, s>>>(a);
-    attn_bwd_dq_mfma_kernel<true, true><<<gq, block, 0, s>>>(a);
-  } else if (seg) {
-    attn_bwd_dkv_mfma_kernel<true, false><<<gk, block, 0, s>>>(a);
-    attn_bwd_dq_mfma_kernel<true, false><<<gq, block, 0, s>>>(a);
-  } else if (bias) {
-    attn_bwd_dkv_mfma_kernel<false, true><<<gk, block, 0, s>>>(a);
-    attn_bwd_dq_mfma_kernel<false, true><<<gq, block, 0, s>>>(a);
-  } else {
-    attn_bwd_dkv_mfma_kernel<false, false><<<gk, block, 0, s>>>(a);
-    attn_bwd_dq_mfma_kernel<false, false><<<gq, block, 0, s>>>(a);
-  }
+  const bool do_dkv = !(p->impl & RA_BWD_ONLY_DQ), do_dq = !(p->impl & RA_BWD_ONLY_DKV);
+#define RA_LAUNCH_BWD(SEG, BIAS)                                                         \
+  do {                                                                                   \
+    if (do_dkv) attn_bwd_dkv_mfma_kernel<SEG, BIAS><<<gk, block, 0, s>>>(a);             \
+    if (do_dq) attn_bwd_dq_mfma_kernel<SEG, BIAS><<<gq, block, 0, s>>>(a);               \
+  } while (0)
+  if (seg && bias) RA_LAUNCH_BWD(true, true);
+  else if (seg) RA_LAUNCH_BWD(true, false);
+  else if (bias) RA_LAUNCH_BWD(false, true);
+  else RA_LAUNCH_BWD(false, false);
+#undef RA_LAUNCH_BWD
   RA_CHECK_LAUNCH("attn_bwd_mfma");
   return RA_OK;
 }

@@ -127,6 +127,7 @@ class _Config:
         self.mask_min = float(torch.finfo(self.dtype).min)
         self.impl = {"auto": L.RA_IMPL_AUTO, "generic": L.RA_IMPL_GENERIC, "mfma": L.RA_IMPL_MFMA}[
             kw.get("impl", "auto")]
+        self.bwd_only = {None: 0, "dq": L.RA_BWD_ONLY_DQ, "dkv": L.RA_BWD_ONLY_DKV}[kw.get("bwd_only", None)]
         self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
         # policy / precision / prevent_cse / dropout_rng only steer XLA rematerialisation: the
         # kernels always recompute the probabilities in the backward pass.
@@ -296,7 +297,7 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
     if skip is None:
         skip = cfg.qc >= 2 and cache_idx is None
     p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
-    p.impl = cfg.impl
+    p.impl = cfg.impl | cfg.bwd_only
     L.check(L.load().ra_attn_bwd_block(ctypes.byref(p), _stream()), "ra_attn_bwd_block")
     return dq, dk, dv
 
