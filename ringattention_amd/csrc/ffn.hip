@@ -1,6 +1,262 @@
+// bf16 MFMA GEMM for gfx950 and the SwiGLU feed-forward built on it: the body that
+// blockwise_feedforward (ringattention_jax.py:333-352) scans over chunks of tokens.
+//
+// GEMM: C (M,N) = op(A) op(B) [+ op(A2) op(B2)], fp32 accumulation in v_mfma_f32_32x32x16_bf16.
+//   workgroup = 4 wavefronts (2 x 2), tile BM x BN, K step 64, LDS double buffered.
+//   An operand whose contraction index is contiguous in memory is staged row-major and read with
+//   16-byte LDS reads; one whose contraction index is the slow axis is staged as it lies in memory
+//   and read with ds_read_b64_tr_b16, so no layout ever needs a transposing copy.
 #include "common.hpp"
+
 namespace ra {
-int swiglu_fwd(const ra_swiglu_params*, hipStream_t) { set_error("swiglu: not built"); return RA_ERR_UNSUPPORTED; }
-int swiglu_bwd(const ra_swiglu_params*, hipStream_t) { set_error("swiglu: not built"); return RA_ERR_UNSUPPORTED; }
-int gemm_bf16(const void*, const void*, void*, int, int, int, int, int, int, int, hipStream_t) { set_error("gemm: not built"); return RA_ERR_UNSUPPORTED; }
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int GBK = 64;
+constexpr int NAT_STR = GBK + 8;      // row stride (elements) of a tile read row-wise
+
+struct GemmArgs {
+  const uint16_t* A; const uint16_t* B; const uint16_t* A2; const uint16_t* B2;
+  void* C;
+  int M, N, K;
+  int c_f32, beta_one;
+};
+
+__device__ __forceinline__ s16x4 lds_tr(const uint16_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
 }
+
+// TA: A is stored (K,M).  TB: B is stored (N,K).
+template <bool TA, bool TB, int BM, int BN>
+__global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
+  constexpr int WM = BM / 2, WN = BN / 2, MB = WM / 32, NB = WN / 32;
+  constexpr int A_STR = TA ? BM + 32 : NAT_STR;     // elements
+  constexpr int B_STR = TB ? NAT_STR : BN + 32;
+  constexpr int A_ROWS = TA ? GBK : BM, B_ROWS = TB ? BN : GBK;
+  constexpr int A_CPR = (TA ? BM : GBK) / 8, B_CPR = (TB ? GBK : BN) / 8;   // 16-byte chunks per staged row
+  constexpr int A_CH = A_ROWS * A_CPR / 256, B_CH = B_ROWS * B_CPR / 256;   // chunks per thread
+  __shared__ __attribute__((aligned(16))) uint16_t As[2][A_ROWS * A_STR];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs[2][B_ROWS * B_STR];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  // neighbouring workgroups share the A row panel (and, 8 apart, the same XCD's L2)
+  const int ntn = g.N / BN;
+  const int tm = blockIdx.x / ntn, tn = blockIdx.x % ntn;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x16 acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  uint4 ar[A_CH], br[B_CH];
+  const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
+  const uint16_t* Ap = g.A; const uint16_t* Bp = g.B;
+  auto load_stage = [&](int k0) {
+#pragma unroll
+    for (int c = 0; c < A_CH; c++) {
+      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;
+      const int64_t off = TA ? (int64_t)(k0 + row) * lda + m0 + ch * 8 : (int64_t)(m0 + row) * lda + k0 + ch * 8;
+      ar[c] = *(const uint4*)(Ap + off);
+    }
+#pragma unroll
+    for (int c = 0; c < B_CH; c++) {
+      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;
+      const int64_t off = TB ? (int64_t)(n0 + row) * ldb + k0 + ch * 8 : (int64_t)(k0 + row) * ldb + n0 + ch * 8;
+      br[c] = *(const uint4*)(Bp + off);
+    }
+  };
+  auto store_stage = [&](int buf) {
+#pragma unroll
+    for (int c = 0; c < A_CH; c++) {
+      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;
+      *(uint4*)(&As[buf][row * A_STR + ch * 8]) = ar[c];
+    }
+#pragma unroll
+    for (int c = 0; c < B_CH; c++) {
+      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;
+      *(uint4*)(&Bs[buf][row * B_STR + ch * 8]) = br[c];
+    }
+  };
+
+  // transpose-read lane offset: 16-lane group reads 4 contraction rows x 16 columns
+  const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  const int nk = g.K / GBK;
+  const int npairs = g.A2 ? 2 : 1;
+  const int total = nk * npairs;
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+  for (int it = 0; it < total; it++) {
+    const int cur = it & 1;
+    const bool more = it + 1 < total;
+    if (more) {
+      const int nx = it + 1;
+      if (nx == nk) { Ap = g.A2; Bp = g.B2; }
+      load_stage((nx % nk) * GBK);
+    }
+#pragma unroll
+    for (int kk = 0; kk < GBK / 16; kk++) {
+      bf16x8 af[MB], bfr[NB];
+#pragma unroll
+      for (int i = 0; i < MB; i++) {
+        if (!TA) {
+          af[i] = *(const bf16x8*)(&As[cur][(wm * WM + i * 32 + lo) * A_STR + kk * 16 + hi * 8]);
+        } else {
+          const uint16_t* p = &As[cur][kk * 16 * A_STR + trA + wm * WM + i * 32];
+          s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);
+          af[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < NB; j++) {
+        if (TB) {
+          bfr[j] = *(const bf16x8*)(&Bs[cur][(wn * WN + j * 32 + lo) * B_STR + kk * 16 + hi * 8]);
+        } else {
+          const uint16_t* p = &Bs[cur][kk * 16 * B_STR + trB + wn * WN + j * 32];
+          s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);
+          bfr[j] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int j = 0; j < NB; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) store_stage(cur ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: lane holds column n = lo of each 32x32 block, rows 8*(r/4) + 4*hi + r%4
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+      const int n = n0 + wn * WN + j * 32 + lo;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int m = m0 + wm * WM + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+        const int64_t o = (int64_t)m * g.N + n;
+        if (g.c_f32) {
+          float* c = (float*)g.C + o;
+          *c = g.beta_one ? *c + acc[i][j][r] : acc[i][j][r];
+        } else {
+          ((uint16_t*)g.C)[o] = f32_to_bf16(acc[i][j][r]);
+        }
+      }
+    }
+}
+
+template <bool TA, bool TB>
+static int launch_gemm(const GemmArgs& g, hipStream_t s) {
+  constexpr int BM = 128, BN = 128;
+  if (g.M % BM || g.N % BN || g.K % GBK) {
+    set_error("gemm_bf16: M, N must be multiples of 128 and K of 64 (got %d, %d, %d)", g.M, g.N, g.K);
+    return RA_ERR_UNSUPPORTED;
+  }
+  const long long nwg = (long long)(g.M / BM) * (g.N / BN);
+  gemm_bf16_kernel<TA, TB, BM, BN><<<dim3((unsigned)nwg), 256, 0, s>>>(g);
+  RA_CHECK_LAUNCH("gemm_bf16");
+  return RA_OK;
+}
+
+static int gemm_dispatch(const GemmArgs& g, int ta, int tb, hipStream_t s) {
+  if (ta && tb) return launch_gemm<true, true>(g, s);
+  if (ta) return launch_gemm<true, false>(g, s);
+  if (tb) return launch_gemm<false, true>(g, s);
+  return launch_gemm<false, false>(g, s);
+}
+
+int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype, int beta_one,
+              hipStream_t s) {
+  GemmArgs g{(const uint16_t*)A, (const uint16_t*)B, nullptr, nullptr, C, M, N, K, c_dtype == RA_F32, beta_one};
+  return gemm_dispatch(g, ta, tb, s);
+}
+
+// ------------------------------------------------------------------ SwiGLU elementwise parts
+__device__ __forceinline__ float silu(float x) { return x / (1.f + __expf(-x)); }
+
+__global__ void swiglu_act_kernel(const uint16_t* a, const uint16_t* b, uint16_t* h, int64_t n8) {
+  // 8 elements (16 bytes) per thread
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+    uint4 ua = ((const uint4*)a)[i], ub = ((const uint4*)b)[i], uh;
+    const uint16_t* pa = (const uint16_t*)&ua; const uint16_t* pb = (const uint16_t*)&ub; uint16_t* ph = (uint16_t*)&uh;
+#pragma unroll
+    for (int e = 0; e < 8; e++) ph[e] = f32_to_bf16(silu(bf16_to_f32(pa[e])) * bf16_to_f32(pb[e]));
+    ((uint4*)h)[i] = uh;
+  }
+}
+
+__global__ void swiglu_act_bwd_kernel(const uint16_t* a, const uint16_t* b, const uint16_t* dh, uint16_t* h,
+                                      uint16_t* da, uint16_t* db, int64_t n8) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8; i += (int64_t)gridDim.x * blockDim.x) {
+    uint4 ua = ((const uint4*)a)[i], ub = ((const uint4*)b)[i], ud = ((const uint4*)dh)[i], uh, uda, udb;
+    const uint16_t* pa = (const uint16_t*)&ua; const uint16_t* pb = (const uint16_t*)&ub;
+    const uint16_t* pd = (const uint16_t*)&ud;
+    uint16_t* ph = (uint16_t*)&uh; uint16_t* pda = (uint16_t*)&uda; uint16_t* pdb = (uint16_t*)&udb;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float av = bf16_to_f32(pa[e]), bv = bf16_to_f32(pb[e]), dv = bf16_to_f32(pd[e]);
+      const float sg = 1.f / (1.f + __expf(-av));
+      const float sl = av * sg;
+      ph[e] = f32_to_bf16(sl * bv);
+      pdb[e] = f32_to_bf16(dv * sl);
+      pda[e] = f32_to_bf16(dv * bv * (sg * (1.f + av * (1.f - sg))));   // d silu / da
+    }
+    ((uint4*)h)[i] = uh; ((uint4*)da)[i] = uda; ((uint4*)db)[i] = udb;
+  }
+}
+
+static int check_ffn_shape(const ra_swiglu_params* p, const char* who) {
+  if (p->T % 128 || p->d % 128 || p->f % 128) {
+    set_error("%s: tokens, hidden and intermediate sizes must be multiples of 128 (got %d, %d, %d)", who, p->T,
+              p->d, p->f);
+    return RA_ERR_UNSUPPORTED;
+  }
+  return RA_OK;
+}
+
+int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s) {
+  if (int rc = check_ffn_shape(p, "swiglu_fwd")) return rc;
+  const int T = p->T, d = p->d, f = p->f;
+  if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;     // a = x w1
+  if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;     // b = x w3
+  const int64_t n8 = (int64_t)T * f / 8;
+  swiglu_act_kernel<<<2048, 256, 0, s>>>((const uint16_t*)p->a, (const uint16_t*)p->b, (uint16_t*)p->h, n8);
+  RA_CHECK_LAUNCH("swiglu_act");
+  return gemm_bf16(p->h, p->w2, p->y, T, d, f, 0, 0, RA_BF16, 0, s);                       // y = h w2
+}
+
+int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s) {
+  if (int rc = check_ffn_shape(p, "swiglu_bwd")) return rc;
+  const int T = p->T, d = p->d, f = p->f;
+  // recompute the pre-activations (nothing_saveable), then
+  //   dh = dy w2^T ; da, db from the activation ; dx = da w1^T + db w3^T
+  //   dw1 += x^T da ; dw3 += x^T db ; dw2 += h^T dy
+  if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
+  if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
+  // dh goes into the da buffer first, the activation backward then rewrites it in place
+  if (int rc = gemm_bf16(p->dy, p->w2, p->da, T, f, d, 0, 1, RA_BF16, 0, s)) return rc;
+  const int64_t n8 = (int64_t)T * f / 8;
+  swiglu_act_bwd_kernel<<<2048, 256, 0, s>>>((const uint16_t*)p->a, (const uint16_t*)p->b, (const uint16_t*)p->da,
+                                             (uint16_t*)p->h, (uint16_t*)p->da, (uint16_t*)p->db, n8);
+  RA_CHECK_LAUNCH("swiglu_act_bwd");
+  GemmArgs g{(const uint16_t*)p->da, (const uint16_t*)p->w1, (const uint16_t*)p->db, (const uint16_t*)p->w3,
+             p->dx, T, d, f, 0, 0};
+  if (int rc = gemm_dispatch(g, 0, 1, s)) return rc;                                        // dx
+  if (int rc = gemm_bf16(p->x, p->da, p->dw1, d, f, T, 1, 0, RA_F32, 1, s)) return rc;
+  if (int rc = gemm_bf16(p->x, p->db, p->dw3, d, f, T, 1, 0, RA_F32, 1, s)) return rc;
+  return gemm_bf16(p->h, p->dy, p->dw2, f, d, T, 1, 0, RA_F32, 1, s);
+}
+
+}  // namespace ra
