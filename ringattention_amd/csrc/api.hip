@@ -48,6 +48,9 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
   }
   RA_REQUIRE(m.q_chunk_idx_start >= 0 && m.k_chunk_idx_start >= 0, RA_ERR_INVALID, "%s: negative chunk start", who);
   if (m.segment_ids) RA_REQUIRE(m.seg_len > 0, RA_ERR_INVALID, "%s: segment_ids given with seg_len 0", who);
+  RA_REQUIRE((long long)m.q_chunk_idx_start * m.query_chunk_size + Sq < (1LL << 31) - 4096 &&
+                 (long long)m.k_chunk_idx_start * m.key_chunk_size + Skv < (1LL << 31) - 4096,
+             RA_ERR_UNSUPPORTED, "%s: global positions must stay below 2^31", who);
   return RA_OK;
 }
 

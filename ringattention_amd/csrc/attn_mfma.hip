@@ -71,19 +71,20 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
   // ---- tile range: chunks that run (reference predicate), clipped to tiles with an unmasked pair
   const int qi = q0 / mv.qc;
   int kend = mv.run_prefix_keys(qi, a.Skv);
-  const long long gq0 = mv.global_q(q0);
-  const long long gk0 = mv.global_k(0);
+  // global positions fit 31 bits (checked on the host)
+  const int gq0 = (int)mv.global_q(q0);
+  const int gk0 = (int)mv.global_k(0);
   if (mv.cbs > 0 && mv.skip_tiles) {
-    long long lim = ((gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;   // first key position masked for every row
+    long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;   // first key position masked for every row
     long long n = lim - gk0;
     if (n < kend) kend = n > 0 ? (int)n : 0;
   }
   const int ntiles = (kend + FBN - 1) / FBN;
 
-  // per-lane mask constants
-  const long long gq = gq0 + wave * 32 + lo;
-  const long long klim = mv.cbs > 0 ? (gq / mv.cbs + 1) * mv.cbs : 0x7fffffffffffffffLL;   // keys >= klim are masked
-  const long long klim_wave = mv.cbs > 0 ? ((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs : 0x7fffffffffffffffLL;
+  // per-lane mask constants: keys at global position >= klim are masked
+  const int gq = gq0 + wave * 32 + lo;
+  const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
+  const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
   int seg_q = 0;
   if (HAS_SEG) {
     int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
@@ -127,42 +128,43 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
   uint4 kr[4], vr[4];
   int seg_r = 0;
   float bias_r = 0.f;
-  auto load_tile = [&](int j) {
-    const int k0 = j * FBN;
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-      const int64_t off = (int64_t)(k0 + p * 16 + srow) * a.kv_ss;
-      kr[p] = *(const uint4*)(kg + off);
-      vr[p] = *(const uint4*)(vg + off);
-    }
-    if (tid < FBN) {
-      const int kj = k0 + tid;
-      if (HAS_SEG) {
-        int idx = clamp_seg_index(((long long)mv.k_start + kj / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
-        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx];
-      }
-      if (HAS_BIAS) {
-        float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (gk0 + kj) * mv.bias_sk];
-        if (mv.any_mask) bv = fminf(bv, 0.f);
-        bias_r = bv * kLog2e;
-      }
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-      *(uint4*)(&Ks[buf][(p * 16 + srow) * KSTR + schunk * 8]) = kr[p];
-      *(uint4*)(&Vs[buf][(p * 16 + srow) * VSTR + schunk * 8]) = vr[p];
-    }
-    if (tid < FBN) {
-      if (HAS_SEG) seg_ks[buf][tid] = seg_r;
-      if (HAS_BIAS) bias_ks[buf][tid] = bias_r;
-    }
-  };
+  // Straight-line staging (no lambdas, no conditionals) so the prefetch registers stay registers.
+#define RA_LOAD_KV_TILE(J)                                                                              \
+  {                                                                                                     \
+    const int k0_ = (J) * FBN;                                                                          \
+    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
+      const int64_t off_ = (int64_t)(k0_ + p * 16 + srow) * a.kv_ss;                                    \
+      kr[p] = *(const uint4*)(kg + off_);                                                               \
+      vr[p] = *(const uint4*)(vg + off_);                                                               \
+    }                                                                                                   \
+    if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                           \
+      const int kj_ = k0_ + tid;                                                                        \
+      if (HAS_SEG) {                                                                                    \
+        int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
+      }                                                                                                 \
+      if (HAS_BIAS) {                                                                                   \
+        float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0 + kj_) * mv.bias_sk]; \
+        if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
+        bias_r = bv_ * kLog2e;                                                                          \
+      }                                                                                                 \
+    }                                                                                                   \
+  }
+#define RA_STORE_KV_TILE(BUF, KSTRIDE, VSTRIDE)                                                         \
+  {                                                                                                     \
+    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
+      *(uint4*)(&Ks[BUF][(p * 16 + srow) * (KSTRIDE) + schunk * 8]) = kr[p];                            \
+      *(uint4*)(&Vs[BUF][(p * 16 + srow) * (VSTRIDE) + schunk * 8]) = vr[p];                            \
+    }                                                                                                   \
+    if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                           \
+      if (HAS_SEG) seg_ks[BUF][tid] = seg_r;                                                            \
+      if (HAS_BIAS) bias_ks[BUF][tid] = bias_r;                                                         \
+    }                                                                                                   \
+  }
 
   if (ntiles > 0) {
-    load_tile(0);
-    store_tile(0);
+    RA_LOAD_KV_TILE(0);
+    RA_STORE_KV_TILE(0, KSTR, VSTR);
   }
   __syncthreads();
 
@@ -174,8 +176,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
 
   for (int j = 0; j < ntiles; j++) {
     const int cur = j & 1;
-    const bool more = j + 1 < ntiles;
-    if (more) load_tile(j + 1);
+    // prefetch the next tile (the last iteration re-reads its own tile into the idle buffer)
+    RA_LOAD_KV_TILE(min(j + 1, ntiles - 1));
 
     // ---- S^T = K Q^T : two 32(key) x 32(query) blocks
     f32x16 s[2];
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
     }
 
     // ---- online softmax in the log2 domain
-    const long long gk_tile = gk0 + (long long)j * FBN;
+    const int gk_tile = gk0 + j * FBN;
     bool need_mask = HAS_SEG || HAS_BIAS || (gk_tile + FBN - 1 >= klim_wave);
     float alpha;
     bf16x8 pf[2][2];
@@ -246,10 +248,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
         }
       l = l * alpha + ps;
     }
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {     // no row of this wavefront raised its max: skip
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+      for (int db = 0; db < 4; db++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[db][r] *= alpha;
+        for (int r = 0; r < 16; r++) acc[db][r] *= alpha;
+    }
 
     // ---- O^T += V^T P^T : four 32(d) x 32(query) blocks, contraction over the 64 keys
     const uint16_t* vp = &Vs[cur][v_lane_off];
@@ -267,7 +271,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
         }
       }
 
-    if (more) store_tile(cur ^ 1);
+    RA_STORE_KV_TILE(cur ^ 1, KSTR, VSTR);
     __syncthreads();
   }
 
@@ -330,19 +334,19 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
 
   const int qi = q0 / mv.qc;
   int kend = mv.run_prefix_keys(qi, a.Skv);
-  const long long gq0 = mv.global_q(q0);
-  const long long gk0 = mv.global_k(0);
+  const int gq0 = (int)mv.global_q(q0);
+  const int gk0 = (int)mv.global_k(0);
   if (mv.cbs > 0 && mv.skip_tiles) {
-    long long lim = ((gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
+    long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
     long long n = lim - gk0;
     if (n < kend) kend = n > 0 ? (int)n : 0;
   }
   const int ntiles = (kend + FBN - 1) / FBN;
   if (ntiles == 0) return;     // nothing to add to dq
 
-  const long long gq = gq0 + wave * 32 + lo;
-  const long long klim = mv.cbs > 0 ? (gq / mv.cbs + 1) * mv.cbs : 0x7fffffffffffffffLL;
-  const long long klim_wave = mv.cbs > 0 ? ((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs : 0x7fffffffffffffffLL;
+  const int gq = gq0 + wave * 32 + lo;
+  const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
+  const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
   int seg_q = 0;
   if (HAS_SEG) {
     int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
@@ -375,40 +379,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
   uint4 kr[4], vr[4];
   int seg_r = 0;
   float bias_r = 0.f;
-  auto load_tile = [&](int j) {
-    const int k0 = j * FBN;
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-      const int64_t off = (int64_t)(k0 + p * 16 + srow) * a.kv_ss;
-      kr[p] = *(const uint4*)(kg + off);
-      vr[p] = *(const uint4*)(vg + off);
-    }
-    if (tid < FBN) {
-      const int kj = k0 + tid;
-      if (HAS_SEG) {
-        int idx = clamp_seg_index(((long long)mv.k_start + kj / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
-        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx];
-      }
-      if (HAS_BIAS) {
-        float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (gk0 + kj) * mv.bias_sk];
-        if (mv.any_mask) bv = fminf(bv, 0.f);
-        bias_r = bv * kLog2e;
-      }
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-      *(uint4*)(&Ks[buf][(p * 16 + srow) * BSTR + schunk * 8]) = kr[p];
-      *(uint4*)(&Vs[buf][(p * 16 + srow) * KSTR + schunk * 8]) = vr[p];
-    }
-    if (tid < FBN) {
-      if (HAS_SEG) seg_ks[buf][tid] = seg_r;
-      if (HAS_BIAS) bias_ks[buf][tid] = bias_r;
-    }
-  };
-  load_tile(0);
-  store_tile(0);
+  RA_LOAD_KV_TILE(0);
+  RA_STORE_KV_TILE(0, BSTR, KSTR);
   __syncthreads();
 
   const int ktr_lane_off = ((lane & 15) >> 2) * BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * BSTR;
@@ -417,9 +389,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
 
   for (int j = 0; j < ntiles; j++) {
     const int cur = j & 1;
-    const bool more = j + 1 < ntiles;
-    if (more) load_tile(j + 1);
-    const long long gk_tile = gk0 + (long long)j * FBN;
+    RA_LOAD_KV_TILE(min(j + 1, ntiles - 1));
+    const int gk_tile = gk0 + j * FBN;
     const bool need_mask = HAS_SEG || HAS_BIAS || (gk_tile + FBN - 1 >= klim_wave);
 
 #pragma unroll
@@ -468,9 +439,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
           acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), dsf[t], acc[db], 0, 0, 0);
         }
     }
-    if (more) store_tile(cur ^ 1);
+    RA_STORE_KV_TILE(cur ^ 1, BSTR, KSTR);
     __syncthreads();
   }
+#undef RA_LOAD_KV_TILE
+#undef RA_STORE_KV_TILE
 
   // dq += acc / sqrt(D)   (:230)
   const float rscale = 1.f / sqrtf((float)HD);
@@ -509,9 +482,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   const int k0 = kt * KBN;
   const int krow = k0 + wave * 32 + lo;    // this lane's key row (local)
 
-  const long long gk0 = mv.global_k(k0);
-  const long long gk = gk0 + wave * 32 + lo;
-  const long long gq_base = mv.global_q(0);
+  const int gk0 = (int)mv.global_k(k0);
+  const int gk = gk0 + wave * 32 + lo;
+  const int gq_base = (int)mv.global_q(0);
   // first query tile that has work for this key block: run prefix (chunk level), then sub-tile clip
   const int nqt = a.Sq / KBM;
   int qt_first = nqt;
@@ -525,7 +498,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
     if (lo_c < nqc) qt_first = lo_c * (mv.qc / KBM);
     if (mv.cbs > 0 && mv.skip_tiles && qt_first < nqt) {
       // query tiles whose every row is masked against every key of the block: (gq_max / cbs) < (gk_min / cbs)
-      long long need = (gk0 / mv.cbs) * mv.cbs - gq_base;     // first local query row that can see key gk0
+      long long need = (long long)(gk0 / mv.cbs) * mv.cbs - gq_base;     // first local query row that can see key gk0
       if (need > 0) {
         int t = (int)(need / KBM);
         if (t > qt_first) qt_first = t < nqt ? t : nqt;
@@ -535,8 +508,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   if (qt_first >= nqt) return;            // no query sees this key block: dk, dv unchanged
 
   // masked iff gq / cbs < gk / cbs  <=>  gq < qlim
-  const long long qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffffffffffffLL;
-  const long long qlim_wave = mv.cbs > 0 ? ((gk0 + wave * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffffffffffffLL;
+  const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;
+  const int qlim_wave = mv.cbs > 0 ? ((gk0 + wave * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffff;
   int seg_k = 0;
   float bias2 = 0.f;
   if (HAS_SEG) {
@@ -544,7 +517,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
     seg_k = mv.seg[(int64_t)b * mv.seg_sb + idx];
   }
   if (HAS_BIAS) {
-    float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + gk * mv.bias_sk];
+    float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)gk * mv.bias_sk];
     if (mv.any_mask) bv = fminf(bv, 0.f);
     bias2 = bv * kLog2e;
   }
@@ -571,39 +544,39 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   uint4 qr[4], gr[4];
   float r_m2 = 0.f, r_rden = 0.f, r_delta = 0.f;
   int r_seg = 0;
-  auto load_tile = [&](int qt) {
-    const int q0 = qt * KBM;
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-      const int64_t off = (int64_t)(q0 + p * 16 + srow) * a.q_ss;
-      qr[p] = *(const uint4*)(qg + off);
-      gr[p] = *(const uint4*)(gg + off);
-    }
-    if (tid < KBM) {
-      const int row = q0 + tid;
-      const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row;
-      r_m2 = max_to_log2(a.mx[st], kMask2);
-      r_rden = 1.f / a.den[st];
-      r_delta = a.delta[st];
-      if (HAS_SEG) {
-        int idx = clamp_seg_index(((long long)mv.q_start + row / mv.qc) * mv.qc, mv.qc, mv.seg_len, row % mv.qc);
-        r_seg = mv.seg[(int64_t)b * mv.seg_sb + idx];
-      }
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-      *(uint4*)(&Qs[buf][(p * 16 + srow) * BSTR + schunk * 8]) = qr[p];
-      *(uint4*)(&Gs[buf][(p * 16 + srow) * BSTR + schunk * 8]) = gr[p];
-    }
-    if (tid < KBM) {
-      st_m2[buf][tid] = r_m2; st_rden[buf][tid] = r_rden; st_delta[buf][tid] = r_delta;
-      if (HAS_SEG) st_seg[buf][tid] = r_seg;
-    }
-  };
-  load_tile(qt_first);
-  store_tile(0);
+#define RA_LOAD_Q_TILE(QT)                                                                              \
+  {                                                                                                     \
+    const int q0_ = (QT) * KBM;                                                                         \
+    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
+      const int64_t off_ = (int64_t)(q0_ + p * 16 + srow) * a.q_ss;                                     \
+      qr[p] = *(const uint4*)(qg + off_);                                                               \
+      gr[p] = *(const uint4*)(gg + off_);                                                               \
+    }                                                                                                   \
+    if (tid < KBM) {                                                                                    \
+      const int row_ = q0_ + tid;                                                                       \
+      const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
+      r_m2 = max_to_log2(a.mx[st_], kMask2);                                                            \
+      r_rden = 1.f / a.den[st_];                                                                        \
+      r_delta = a.delta[st_];                                                                           \
+      if (HAS_SEG) {                                                                                    \
+        int idx_ = clamp_seg_index(((long long)mv.q_start + row_ / mv.qc) * mv.qc, mv.qc, mv.seg_len, row_ % mv.qc); \
+        r_seg = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
+      }                                                                                                 \
+    }                                                                                                   \
+  }
+#define RA_STORE_Q_TILE(BUF)                                                                            \
+  {                                                                                                     \
+    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
+      *(uint4*)(&Qs[BUF][(p * 16 + srow) * BSTR + schunk * 8]) = qr[p];                                 \
+      *(uint4*)(&Gs[BUF][(p * 16 + srow) * BSTR + schunk * 8]) = gr[p];                                 \
+    }                                                                                                   \
+    if (tid < KBM) {                                                                                    \
+      st_m2[BUF][tid] = r_m2; st_rden[BUF][tid] = r_rden; st_delta[BUF][tid] = r_delta;                 \
+      if (HAS_SEG) st_seg[BUF][tid] = r_seg;                                                            \
+    }                                                                                                   \
+  }
+  RA_LOAD_Q_TILE(qt_first);
+  RA_STORE_Q_TILE(0);
   __syncthreads();
 
   const int tr_lane_off = ((lane & 15) >> 2) * BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * BSTR;
@@ -611,9 +584,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
 
   for (int qt = qt_first; qt < nqt; qt++) {
     const int cur = (qt - qt_first) & 1;
-    const bool more = qt + 1 < nqt;
-    if (more) load_tile(qt + 1);
-    const long long gq_tile = gq_base + (long long)qt * KBM;
+    RA_LOAD_Q_TILE(min(qt + 1, nqt - 1));
+    const int gq_tile = gq_base + qt * KBM;
     const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave);
 
 #pragma unroll
@@ -675,9 +647,11 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
           dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), dsf[t], dkacc[db], 0, 0, 0);
         }
     }
-    if (more) store_tile(cur ^ 1);
+    RA_STORE_Q_TILE(cur ^ 1);
     __syncthreads();
   }
+#undef RA_LOAD_Q_TILE
+#undef RA_STORE_Q_TILE
 
   // dk += acc / sqrt(D) (:231), dv += acc (:232); this workgroup owns its key rows
   const float rscale = 1.f / sqrtf((float)HD);

@@ -59,32 +59,31 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
   uint4 ar[A_CH], br[B_CH];
   const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
   const uint16_t* Ap = g.A; const uint16_t* Bp = g.B;
-  auto load_stage = [&](int k0) {
-#pragma unroll
-    for (int c = 0; c < A_CH; c++) {
-      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;
-      const int64_t off = TA ? (int64_t)(k0 + row) * lda + m0 + ch * 8 : (int64_t)(m0 + row) * lda + k0 + ch * 8;
-      ar[c] = *(const uint4*)(Ap + off);
-    }
-#pragma unroll
-    for (int c = 0; c < B_CH; c++) {
-      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;
-      const int64_t off = TB ? (int64_t)(n0 + row) * ldb + k0 + ch * 8 : (int64_t)(k0 + row) * ldb + n0 + ch * 8;
-      br[c] = *(const uint4*)(Bp + off);
-    }
-  };
-  auto store_stage = [&](int buf) {
-#pragma unroll
-    for (int c = 0; c < A_CH; c++) {
-      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;
-      *(uint4*)(&As[buf][row * A_STR + ch * 8]) = ar[c];
-    }
-#pragma unroll
-    for (int c = 0; c < B_CH; c++) {
-      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;
-      *(uint4*)(&Bs[buf][row * B_STR + ch * 8]) = br[c];
-    }
-  };
+#define RA_LOAD_STAGE(K0)                                                                               \
+  {                                                                                                     \
+    const int k0_ = (K0);                                                                               \
+    _Pragma("unroll") for (int c = 0; c < A_CH; c++) {                                                  \
+      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;                               \
+      const int64_t off = TA ? (int64_t)(k0_ + row) * lda + m0 + ch * 8 : (int64_t)(m0 + row) * lda + k0_ + ch * 8; \
+      ar[c] = *(const uint4*)(Ap + off);                                                                \
+    }                                                                                                   \
+    _Pragma("unroll") for (int c = 0; c < B_CH; c++) {                                                  \
+      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;                               \
+      const int64_t off = TB ? (int64_t)(n0 + row) * ldb + k0_ + ch * 8 : (int64_t)(k0_ + row) * ldb + n0 + ch * 8; \
+      br[c] = *(const uint4*)(Bp + off);                                                                \
+    }                                                                                                   \
+  }
+#define RA_STORE_STAGE(BUF)                                                                             \
+  {                                                                                                     \
+    _Pragma("unroll") for (int c = 0; c < A_CH; c++) {                                                  \
+      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;                               \
+      *(uint4*)(&As[BUF][row * A_STR + ch * 8]) = ar[c];                                                \
+    }                                                                                                   \
+    _Pragma("unroll") for (int c = 0; c < B_CH; c++) {                                                  \
+      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;                               \
+      *(uint4*)(&Bs[BUF][row * B_STR + ch * 8]) = br[c];                                                \
+    }                                                                                                   \
+  }
 
   // transpose-read lane offset: 16-lane group reads 4 contraction rows x 16 columns
   const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
@@ -93,16 +92,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
   const int nk = g.K / GBK;
   const int npairs = g.A2 ? 2 : 1;
   const int total = nk * npairs;
-  load_stage(0);
-  store_stage(0);
+  RA_LOAD_STAGE(0);
+  RA_STORE_STAGE(0);
   __syncthreads();
   for (int it = 0; it < total; it++) {
     const int cur = it & 1;
-    const bool more = it + 1 < total;
-    if (more) {
-      const int nx = it + 1;
-      if (nx == nk) { Ap = g.A2; Bp = g.B2; }
-      load_stage((nx % nk) * GBK);
+    {
+      // prefetch the next K slab (the last iteration re-reads its own slab into the idle buffer)
+      const int nx = min(it + 1, total - 1);
+      if (nx >= nk) { Ap = g.A2; Bp = g.B2; }
+      RA_LOAD_STAGE((nx % nk) * GBK);
     }
 #pragma unroll
     for (int kk = 0; kk < GBK / 16; kk++) {
@@ -133,9 +132,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
         for (int j = 0; j < NB; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
     }
-    if (more) store_stage(cur ^ 1);
+    RA_STORE_STAGE(cur ^ 1);
     __syncthreads();
   }
+#undef RA_LOAD_STAGE
+#undef RA_STORE_STAGE
 
   // epilogue: lane holds column n = lo of each 32x32 block, rows 8*(r/4) + 4*hi + r%4
 #pragma unroll
