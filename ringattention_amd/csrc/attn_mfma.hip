@@ -9,6 +9,7 @@
 //       layout of the second product O^T = V^T P^T - P never goes through LDS.
 //   V^T fragments come from the row-major V tile with ds_read_b64_tr_b16 (LDS transpose read).
 //   Softmax runs in the log2 domain: p = exp2(s * log2(e)/sqrt(D) - m2).
+#include <stdlib.h>
 #include "common.hpp"
 
 namespace ra {
@@ -18,6 +19,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int HD = 128;          // head size
 constexpr int FBM = 128;         // query rows per workgroup
@@ -41,6 +43,16 @@ struct FwdArgs {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32); }
+// max / sum of a value with its partner lane (lane ^ 32) through v_permlane32_swap: no LDS round trip
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float max_xor32(float x) {
+  u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_xor32(float x) {
+  u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 __device__ __forceinline__ s16x4 lds_read_tr(const uint16_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
@@ -50,10 +62,77 @@ __device__ __forceinline__ s16x4 lds_read_tr(const uint16_t* p) {
 __device__ __forceinline__ float max_to_log2(float m, float mask_min) { return m == mask_min ? m : m * kLog2e; }
 __device__ __forceinline__ float max_from_log2(float m2, float mask_min) { return m2 == mask_min ? m2 : m2 * kLn2; }
 
+// LDS tiles hold rows of 128 bf16 (256 bytes = all 64 banks) with no padding.  The 16-byte slot c
+// of row r is stored at slot c ^ swz(r): sixteen consecutive rows then put a given logical slot in
+// sixteen different bank groups (conflict-free 16-byte row reads), and four consecutive rows put four
+// adjacent slots in sixteen different bank groups (conflict-free 4-row transpose reads).
+__device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+constexpr int TROW = HD;          // elements per LDS tile row
+constexpr int KV_TILE = FBN * TROW;
+
+// Staging helpers shared by the kernels below.  They expect in scope: tid, s_off (this thread's
+// swizzled element offset inside a 16-row slab), row16 (global element stride of 16 rows).
+#define RA_LOAD_TILE(REGS, BASE, STRIDE, J, ROWS)                                                       \
+  {                                                                                                     \
+    const uint16_t* p_ = (BASE) + (int64_t)(J) * (ROWS) * (STRIDE);                                     \
+    _Pragma("unroll") for (int p = 0; p < 4; p++) REGS[p] = *(const uint4*)(p_ + p * row16);            \
+  }
+#define RA_STORE_TILE(REGS, LDS)                                                                        \
+  {                                                                                                     \
+    _Pragma("unroll") for (int p = 0; p < 4; p++) *(uint4*)(&(LDS)[p * 16 * TROW + s_off]) = REGS[p];   \
+  }
+// Direct global -> LDS staging of a 64-row tile (no registers): wavefront w issues four
+// global_load_lds of 16 bytes per lane; instruction i fills tile rows 16 w + 4 i .. +3, lane l the
+// physical slot (l & 15) of row 16 w + 4 i + (l >> 4), i.e. logical slot (l & 15) ^ swz(row).
+// Expects in scope: wave_u (wavefront index, uniform), dchunk0 = (lane & 15) ^ ((lane >> 4) << 2).
+// GROW0 points at element 0 of this lane's row for i = 0 in tile 0; STRIDE = global row stride.
+#define RA_DMA_TILE(LDS, GROW0, STRIDE, J, ROWS)                                                        \
+  {                                                                                                     \
+    const uint16_t* g_ = (GROW0) + (int64_t)(J) * (ROWS) * (STRIDE);                                    \
+    _Pragma("unroll") for (int i = 0; i < 4; i++)                                                       \
+      __builtin_amdgcn_global_load_lds(                                                                 \
+          (const __attribute__((address_space(1))) void*)(g_ + (int64_t)(4 * i) * (STRIDE) + ((dchunk0 ^ i) << 3)), \
+          (__attribute__((address_space(3))) void*)(&(LDS)[(16 * wave_u + 4 * i) * TROW]), 16, 0, 0);   \
+  }
+#define RA_DMA_WAIT() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+// per-key segment id / bias of key tile J (threads 0..63), for kernels that stream key tiles
+#define RA_LOAD_KEYINFO(J)                                                                              \
+  if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                             \
+    const int kj_ = (J) * FBN + tid;                                                                    \
+    if (HAS_SEG) {                                                                                      \
+      int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+      seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                    \
+    }                                                                                                   \
+    if (HAS_BIAS) {                                                                                     \
+      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0 + kj_) * mv.bias_sk]; \
+      if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
+      bias_r = bv_ * kLog2e;                                                                            \
+    }                                                                                                   \
+  }
+#define RA_STORE_KEYINFO(BUF)                                                                           \
+  if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                             \
+    if (HAS_SEG) seg_ks[BUF][tid] = seg_r;                                                              \
+    if (HAS_BIAS) bias_ks[BUF][tid] = bias_r;                                                           \
+  }
+// Per-lane LDS read offsets (elements) into a swizzled tile.
+//  NAT[t]: 16-byte read of row lo, d = 16 t + 8 hi .. +8 (MFMA operand whose contraction index is d).
+//  TR[db][x]: ds_read_b64_tr_b16 address; lane i of a 16-lane group addresses tile row
+//  (i >> 2) + 4 hi + 8 x and the 8-byte unit (i & 3) of columns 32 db + 16 g .. +16, g = (lane >> 4) & 1.
+#define RA_LANE_OFFSETS(NAT, TR)                                                                        \
+  {                                                                                                     \
+    _Pragma("unroll") for (int t = 0; t < 8; t++) NAT[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);  \
+    const int i_ = lane & 15, rr_ = (i_ >> 2) + 4 * hi, c0_ = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), \
+              half_ = lane & 1;                                                                         \
+    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+      TR[db][0] = rr_ * TROW + (((4 * db + c0_) ^ swz(rr_)) << 3) + half_ * 4;                          \
+      TR[db][1] = (rr_ + 8) * TROW + (((4 * db + c0_) ^ swz(rr_ + 8)) << 3) + half_ * 4;                \
+    }                                                                                                   \
+  }
+
 template <bool HAS_SEG, bool HAS_BIAS>
 __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][FBN * KSTR];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][FBN * VSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
   __shared__ int seg_ks[2][FBN];
   __shared__ float bias_ks[2][FBN];
 
@@ -120,162 +199,559 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
     m2 = max_to_log2(a.mx[st], kMask2);
     l = hi == 0 ? a.den[st] : 0.f;     // the two half-wave partial sums are added at the end
   }
+  if (ntiles == 0) {
+    if (a.carry_is_initial) {         // nothing runs for these rows: the carry stays (0, 0, -inf)
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) *(f32x4*)(nump + db * 32 + g * 8) = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (hi == 0) { a.den[st] = 0.f; a.mx[st] = RA_NEG_INF; }
+    }
+    return;
+  }
 
-  // ---- staging: thread -> (row, 16-byte chunk) of the 64 x 128 tile, 4 passes of 16 rows
-  const int srow = tid >> 4, schunk = tid & 15;
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8;
-  uint4 kr[4], vr[4];
+  // ---- staging: direct global -> LDS loads, see RA_DMA_TILE
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int dchunk0 = (lane & 15) ^ ((lane >> 4) << 2);
+  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * wave + (lane >> 4)) * a.kv_ss;
+  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * wave + (lane >> 4)) * a.kv_ss;
   int seg_r = 0;
   float bias_r = 0.f;
-  // Straight-line staging (no lambdas, no conditionals) so the prefetch registers stay registers.
-#define RA_LOAD_KV_TILE(J)                                                                              \
+  int k_off[8], v_off[4][2];
+  RA_LANE_OFFSETS(k_off, v_off);
+
+#define RA_QK(S, KBUF)                                                                                  \
   {                                                                                                     \
-    const int k0_ = (J) * FBN;                                                                          \
-    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
-      const int64_t off_ = (int64_t)(k0_ + p * 16 + srow) * a.kv_ss;                                    \
-      kr[p] = *(const uint4*)(kg + off_);                                                               \
-      vr[p] = *(const uint4*)(vg + off_);                                                               \
-    }                                                                                                   \
-    if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                           \
-      const int kj_ = k0_ + tid;                                                                        \
-      if (HAS_SEG) {                                                                                    \
-        int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
-        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
-      }                                                                                                 \
-      if (HAS_BIAS) {                                                                                   \
-        float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0 + kj_) * mv.bias_sk]; \
-        if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
-        bias_r = bv_ * kLog2e;                                                                          \
+    _Pragma("unroll") for (int blk = 0; blk < 2; blk++) {                                               \
+      _Pragma("unroll") for (int r = 0; r < 16; r++) S[blk][r] = 0.f;                                   \
+      _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                   \
+        bf16x8 kf_ = *(const bf16x8*)(&(KBUF)[blk * 32 * TROW + k_off[t]]);                             \
+        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_, qf[t], S[blk], 0, 0, 0);                  \
       }                                                                                                 \
     }                                                                                                   \
   }
-#define RA_STORE_KV_TILE(BUF, KSTRIDE, VSTRIDE)                                                         \
+// one MFMA step of S(j+1): key block BLK, d step T
+#define RA_QK_STEP(S, KBUF, BLK, T)                                                                     \
   {                                                                                                     \
-    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
-      *(uint4*)(&Ks[BUF][(p * 16 + srow) * (KSTRIDE) + schunk * 8]) = kr[p];                            \
-      *(uint4*)(&Vs[BUF][(p * 16 + srow) * (VSTRIDE) + schunk * 8]) = vr[p];                            \
+    bf16x8 kf_ = *(const bf16x8*)(&(KBUF)[(BLK) * 32 * TROW + k_off[T]]);                               \
+    S[BLK] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_, qf[T], S[BLK], 0, 0, 0);                      \
+  }
+// eight probabilities of key block BLK, half HALF: p = exp2(s c - m), summed and rounded to bf16
+#define RA_EXP_GROUP(BLK, HALF)                                                                         \
+  {                                                                                                     \
+    _Pragma("unroll") for (int e = 0; e < 8; e++) {                                                     \
+      float p_ = fast_exp2(fmaf(s[BLK][(HALF) * 8 + e], c, -m2));                                       \
+      ps += p_;                                                                                         \
+      pf[BLK][HALF][e] = (__bf16)p_;                                                                    \
     }                                                                                                   \
-    if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                           \
-      if (HAS_SEG) seg_ks[BUF][tid] = seg_r;                                                            \
-      if (HAS_BIAS) bias_ks[BUF][tid] = bias_r;                                                         \
+    /* pin the results here: without it the optimiser sinks the exponentials below the next branch */   \
+    i32x4 pin_ = __builtin_bit_cast(i32x4, pf[BLK][HALF]);                                              \
+    asm volatile("" : "+v"(pin_), "+v"(ps));                                                            \
+    pf[BLK][HALF] = __builtin_bit_cast(bf16x8, pin_);                                                   \
+  }
+// four MFMA steps of O^T += V^T P^T: keys 32 BLK + 16 T .. +16, all four d blocks
+#define RA_PV_GROUP(VBUF, BLK, T)                                                                       \
+  {                                                                                                     \
+    const uint16_t* vt_ = &(VBUF)[((BLK) * 32 + (T) * 16) * TROW];                                      \
+    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+      s16x4 v0_ = lds_read_tr(vt_ + v_off[db][0]);                                                      \
+      s16x4 v1_ = lds_read_tr(vt_ + v_off[db][1]);                                                      \
+      s16x8 vv_ = __builtin_shufflevector(v0_, v1_, 0, 1, 2, 3, 4, 5, 6, 7);                            \
+      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vv_), pf[BLK][T], acc[db], 0, 0, 0); \
     }                                                                                                   \
+  }
+// ask the scheduler for N repetitions of (1 MFMA, V vector-ALU ops), then fence the group
+#define RA_INTERLEAVE(N, V)                                                                             \
+  {                                                                                                     \
+    _Pragma("unroll") for (int i_ = 0; i_ < (N); i_++) {                                                \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                \
+      __builtin_amdgcn_sched_group_barrier(0x002, (V), 0);                                              \
+    }                                                                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
 
-  if (ntiles > 0) {
-    RA_LOAD_KV_TILE(0);
-    RA_STORE_KV_TILE(0, KSTR, VSTR);
-  }
+  // ---- prologue: K(0), V(0), K(1) into LDS, S(0)
+  RA_DMA_TILE(Ks[0], kg, a.kv_ss, 0, FBN);
+  RA_DMA_TILE(Vs[0], vg, a.kv_ss, 0, FBN);
+  RA_DMA_TILE(Ks[1], kg, a.kv_ss, min(1, ntiles - 1), FBN);
+  RA_LOAD_KEYINFO(0);
+  RA_STORE_KEYINFO(0);
+  RA_DMA_WAIT();
   __syncthreads();
+  f32x16 s[2];
+  RA_QK(s, Ks[0]);
 
-  // V^T fragment addressing for ds_read_b64_tr_b16: within each 16-lane group, lane i supplies the
-  // address of 4 consecutive d of key row (i / 4); lane j of the group receives, for d column j,
-  // the 4 key rows.  Group g covers d columns 16 * (g & 1) .. +16 and key rows 4 * hi .. +4.
-  const int v_lane_off = ((lane & 15) >> 2) * VSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * VSTR;
-  const int k_lane_off = lo * KSTR + hi * 8;
+  // Tiles [0, n_plain) need no mask for any wavefront of the workgroup: they run the interleaved
+  // loop; the rest (diagonal tiles, or every tile when segment ids / bias are present) run the
+  // plain loop with the element-wise mask.
+  int n_plain = 0;
+  if (!HAS_SEG && !HAS_BIAS) {
+    const long long klim_wg = mv.cbs > 0 ? (long long)(gq0 / mv.cbs + 1) * mv.cbs : 0x7fffffffLL;   // smallest klim in the workgroup
+    long long n = (klim_wg - gk0) / FBN;       // tiles whose last key is < klim_wg
+    n_plain = n < 0 ? 0 : (n > ntiles ? ntiles : (int)n);
+  }
 
-  for (int j = 0; j < ntiles; j++) {
+  // m2 is the reference max the exponentials are taken against.  In the interleaved loop it is only
+  // raised when some row's true max has outgrown it by more than kLazy (log2 units): the accumulator
+  // rescale then runs once in a long while; m_true tracks the exact running max and the carry is
+  // brought to it at the end.
+  constexpr float kLazy = 16.f;
+  float m_true = m2;
+
+  int j = 0;
+  for (; j < n_plain; j++) {
     const int cur = j & 1;
-    // prefetch the next tile (the last iteration re-reads its own tile into the idle buffer)
-    RA_LOAD_KV_TILE(min(j + 1, ntiles - 1));
+    // K(j+2) replaces K(j) (consumed last iteration), V(j+1) replaces V(j-1); clamped at the tail
+    RA_DMA_TILE(Ks[cur], kg, a.kv_ss, min(j + 2, ntiles - 1), FBN);
+    RA_DMA_TILE(Vs[cur ^ 1], vg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
+    __builtin_amdgcn_sched_barrier(0);
 
-    // ---- S^T = K Q^T : two 32(key) x 32(query) blocks
-    f32x16 s[2];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) s[blk][r] = 0.f;
-      const uint16_t* kp = &Ks[cur][blk * 32 * KSTR + k_lane_off];
-#pragma unroll
-      for (int t = 0; t < 8; t++) {
-        bf16x8 kf = *(const bf16x8*)(kp + t * 16);
-        s[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s[blk], 0, 0, 0);
-      }
-    }
-
-    // ---- online softmax in the log2 domain
-    const int gk_tile = gk0 + j * FBN;
-    bool need_mask = HAS_SEG || HAS_BIAS || (gk_tile + FBN - 1 >= klim_wave);
-    float alpha;
+    f32x16 sn[2];
     bf16x8 pf[2][2];
-    if (!need_mask) {
-      float mxv = s[0][0];
+    float ps = 0.f;
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+    for (int r = 0; r < 16; r++) { sn[0][r] = 0.f; sn[1][r] = 0.f; }
+    // group 1: first S(j+1) steps under the row max of S(j)
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 0); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 0);
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 1); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 1);
+    float mxv = s[0][0];
 #pragma unroll
-        for (int r = 0; r < 16; r++) mxv = fmaxf(mxv, s[blk][r]);
-      mxv = fmaxf(mxv, xor32(mxv));
-      const float m_new = fmaxf(m2, mxv * c);
-      alpha = fast_exp2(m2 - m_new);
-      m2 = m_new;
-      float ps = 0.f;
+    for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float p = fast_exp2(fmaf(s[blk][r], c, -m_new));
-          ps += p;
-          pf[blk][r >> 3][r & 7] = (__bf16)p;
-        }
-      l = l * alpha + ps;
-    } else {
-      float mxv = RA_NEG_INF;
-#pragma unroll
-      for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);     // key row inside the tile
-          float x = s[blk][r] * c;
-          if (HAS_BIAS) x += bias_ks[cur][kr_];
-          bool masked = (gk_tile + kr_ >= klim);
-          if (HAS_SEG) masked = masked || (seg_ks[cur][kr_] != seg_q);
-          x = masked ? kMask2 : x;
-          s[blk][r] = x;
-          mxv = fmaxf(mxv, x);
-        }
-      mxv = fmaxf(mxv, xor32(mxv));
-      const float m_new = fmaxf(m2, mxv);
-      alpha = fast_exp2(m2 - m_new);
-      m2 = m_new;
-      float ps = 0.f;
-#pragma unroll
-      for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float p = fast_exp2(s[blk][r] - m_new);
-          ps += p;
-          pf[blk][r >> 3][r & 7] = (__bf16)p;
-        }
-      l = l * alpha + ps;
-    }
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {     // no row of this wavefront raised its max: skip
+      for (int r = 0; r < 16; r++) mxv = fmaxf(mxv, s[blk][r]);
+    mxv = fmaxf(mxv, xor32(mxv));
+    m_true = fmaxf(m_true, mxv * c);
+    const bool raise = __builtin_amdgcn_ballot_w64(m_true - m2 > kLazy) != 0;
+    RA_INTERLEAVE(4, 5);
+    if (raise) {
+      const float alpha = fast_exp2(m2 - m_true);
+      m2 = m_true;
+      l *= alpha;
 #pragma unroll
       for (int db = 0; db < 4; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[db][r] *= alpha;
     }
-
-    // ---- O^T += V^T P^T : four 32(d) x 32(query) blocks, contraction over the 64 keys
-    const uint16_t* vp = &Vs[cur][v_lane_off];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int t = 0; t < 2; t++) {
-        const uint16_t* vrow = vp + (blk * 32 + t * 16) * VSTR;
-#pragma unroll
-        for (int db = 0; db < 4; db++) {
-          s16x4 v0 = lds_read_tr(vrow + db * 32);
-          s16x4 v1 = lds_read_tr(vrow + 8 * VSTR + db * 32);
-          s16x8 vv = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vv), pf[blk][t], acc[db], 0, 0, 0);
-        }
-      }
-
-    RA_STORE_KV_TILE(cur ^ 1, KSTR, VSTR);
+    // groups 2-4: remaining S(j+1) steps under the exponentials of S(j)
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 2); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 2);
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 3); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 3);
+    RA_EXP_GROUP(0, 0);
+    RA_INTERLEAVE(4, 7);
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 4); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 4);
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 5); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 5);
+    RA_EXP_GROUP(0, 1);
+    RA_INTERLEAVE(4, 7);
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 6); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 6);
+    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 7); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 7);
+    RA_EXP_GROUP(1, 0);
+    RA_INTERLEAVE(4, 7);
+    // groups 5-8: O^T += V(j)^T P^T, the first of them under the last exponentials
+    RA_PV_GROUP(Vs[cur], 0, 0);
+    RA_EXP_GROUP(1, 1);
+    RA_INTERLEAVE(4, 7);
+    RA_PV_GROUP(Vs[cur], 0, 1);
+    RA_PV_GROUP(Vs[cur], 1, 0);
+    RA_PV_GROUP(Vs[cur], 1, 1);
+    l += ps;
+    s[0] = sn[0]; s[1] = sn[1];
+    RA_DMA_WAIT();
     __syncthreads();
   }
 
+  for (; j < ntiles; j++) {
+    const int cur = j & 1;
+    RA_DMA_TILE(Ks[cur], kg, a.kv_ss, min(j + 2, ntiles - 1), FBN);
+    RA_DMA_TILE(Vs[cur ^ 1], vg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
+    RA_LOAD_KEYINFO(min(j + 1, ntiles - 1));
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- S(j+1)^T = K(j+1) Q^T
+    f32x16 sn[2];
+    RA_QK(sn, Ks[cur ^ 1]);
+
+    // ---- online softmax of S(j) in the log2 domain, element-wise mask
+    const int gk_tile = gk0 + j * FBN;
+    float mxv = RA_NEG_INF;
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);     // key row inside the tile
+        float x = s[blk][r] * c;
+        if (HAS_BIAS) x += bias_ks[cur][kr_];
+        bool masked = (gk_tile + kr_ >= klim);
+        if (HAS_SEG) masked = masked || (seg_ks[cur][kr_] != seg_q);
+        x = masked ? kMask2 : x;
+        s[blk][r] = x;
+        mxv = fmaxf(mxv, x);
+      }
+    mxv = fmaxf(mxv, xor32(mxv));
+    m_true = fmaxf(m_true, mxv);
+    const float m_new = fmaxf(m2, mxv);
+    const float alpha = fast_exp2(m2 - m_new);
+    m2 = m_new;
+    float ps = 0.f;
+    bf16x8 pf[2][2];
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float p = fast_exp2(s[blk][r] - m_new);
+        ps += p;
+        pf[blk][r >> 3][r & 7] = (__bf16)p;
+      }
+    l = l * alpha + ps;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] *= alpha;
+    }
+    RA_PV_GROUP(Vs[cur], 0, 0);
+    RA_PV_GROUP(Vs[cur], 0, 1);
+    RA_PV_GROUP(Vs[cur], 1, 0);
+    RA_PV_GROUP(Vs[cur], 1, 1);
+    RA_STORE_KEYINFO(cur ^ 1);
+    s[0] = sn[0]; s[1] = sn[1];
+    RA_DMA_WAIT();
+    __syncthreads();
+  }
+  if (__builtin_amdgcn_ballot_w64(m_true != m2) != 0) {     // bring the carry to the exact running max
+    const float fix = (m_true == m2) ? 1.f : fast_exp2(m2 - m_true);
+    m2 = m_true;
+    l *= fix;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[db][r] *= fix;
+  }
+#undef RA_QK
+#undef RA_QK_STEP
+#undef RA_EXP_GROUP
+#undef RA_PV_GROUP
+
   // ---- write the carry back: numerator (fp32), denominator, max_score (natural log domain)
+#pragma unroll
+  for (int db = 0; db < 4; db++)
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      f32x4 t = {acc[db][g * 4 + 0], acc[db][g * 4 + 1], acc[db][g * 4 + 2], acc[db][g * 4 + 3]};
+      *(f32x4*)(nump + db * 32 + g * 8) = t;
+    }
+  l += xor32(l);
+  if (hi == 0) {
+    a.den[st] = l;
+    a.mx[st] = max_from_log2(m2, kMask2);
+  }
+}
+
+// ------------------------------------------------------------------ forward, ping-pong variant
+// 8 wavefronts per workgroup, 256 query rows: group A (waves 0-3) owns rows 0..127, group B (waves
+// 4-7) rows 128..255; wave i of each group shares SIMD i.  Time is cut into phases separated by
+// workgroup barriers.  In every phase one group runs its matrix work for a key tile j - S(j+1)^T =
+// K(j+1) Q^T and O^T += V(j)^T P(j)^T, 32 MFMAs - while the other group runs its vector work - the
+// softmax of its S - so each SIMD always has one wave feeding the matrix pipe and one feeding the
+// vector ALU.  Both groups read the same K / V tiles from LDS, one phase apart.
+//   group A: M(0) V(1) M(1) V(2) ...        group B: V(0) M(0) V(1) M(1) ...
+// K(j+2), V(j+1) are brought in by direct global->LDS loads issued at the start of phase 2j and
+// awaited before the barrier that ends phase 2j+1.
+constexpr int PBM = 256;
+#ifdef RA_TRACE
+__device__ long long g_trace[8][4096];
+#define RA_TRACE_MARK() { if (trace_on && lane == 0 && trace_n < 4096) g_trace[wave][trace_n++] = __builtin_readcyclecounter(); }
+#else
+#define RA_TRACE_MARK() {}
+#endif
+constexpr int PP_DEPTH = 1;       // LDS fragment prefetch distance of the matrix phase, in steps of 4 MFMAs
+constexpr bool PP_PRIO = false;  // raise the wave priority during the matrix phase
+
+template <bool HAS_SEG, bool HAS_BIAS>
+__global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
+  __shared__ int seg_ks[4][FBN];
+  __shared__ float bias_ks[4][FBN];
+
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int grp = __builtin_amdgcn_readfirstlane(wave >> 2), w4 = wave & 3;
+  const int nqt = a.Sq / PBM;
+  int wg = blockIdx.x;
+  const int qt = nqt - 1 - (wg % nqt);       // heaviest (latest) query tiles first
+  wg /= nqt;
+  const int h = wg % a.H, b = wg / a.H;
+  const int q0 = qt * PBM;
+  const int qg0 = q0 + grp * 128;            // first row of this group
+  const int qrow = qg0 + w4 * 32 + lo;       // this lane's query row (local)
+
+  // ---- tile ranges.  The workgroup iterates over the tiles its last rows need; a group whose rows
+  // end earlier sees its extra tiles fully masked and contributes nothing there.
+  const int qi = q0 / mv.qc;                 // 256 | query_chunk_size: one chunk per workgroup
+  const int kend_chunk = mv.run_prefix_keys(qi, a.Skv);
+  const int gk0 = (int)mv.global_k(0);
+  const int gq_wg = (int)mv.global_q(q0);
+  int kend_wg = kend_chunk, kend_grp = kend_chunk;
+  if (mv.cbs > 0 && mv.skip_tiles) {
+    long long lim_wg = ((long long)(gq_wg + PBM - 1) / mv.cbs + 1) * mv.cbs - gk0;
+    long long lim_grp = ((long long)(gq_wg + grp * 128 + 127) / mv.cbs + 1) * mv.cbs - gk0;
+    if (lim_wg < kend_wg) kend_wg = lim_wg > 0 ? (int)lim_wg : 0;
+    if (lim_grp < kend_grp) kend_grp = lim_grp > 0 ? (int)lim_grp : 0;
+  }
+  const int ntiles = (kend_wg + FBN - 1) / FBN;        // workgroup-uniform
+  const int ntiles_grp = (kend_grp + FBN - 1) / FBN;   // tiles >= this are fully masked for the group
+
+  const int gq = gq_wg + grp * 128 + w4 * 32 + lo;
+  const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
+  const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq_wg + grp * 128 + w4 * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
+  int seg_q = 0;
+  if (HAS_SEG) {
+    int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
+    seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
+  }
+  const float c = kLog2e / sqrtf((float)HD);
+  const float kMask2 = mv.mask_min;
+
+  const uint16_t* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
+  bf16x8 qf[8];
+#pragma unroll
+  for (int t = 0; t < 8; t++) qf[t] = *(const bf16x8*)(qp + t * 16);
+
+  f32x16 acc[4];
+  float m2 = RA_NEG_INF, l = 0.f;
+  float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
+  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+  if (a.carry_is_initial) {
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+  } else {
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4 t = *(const f32x4*)(nump + db * 32 + g * 8);
+        acc[db][g * 4 + 0] = t[0]; acc[db][g * 4 + 1] = t[1]; acc[db][g * 4 + 2] = t[2]; acc[db][g * 4 + 3] = t[3];
+      }
+    m2 = max_to_log2(a.mx[st], kMask2);
+    l = hi == 0 ? a.den[st] : 0.f;
+  }
+  if (ntiles == 0) {                  // workgroup-uniform
+    if (a.carry_is_initial) {
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) *(f32x4*)(nump + db * 32 + g * 8) = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (hi == 0) { a.den[st] = 0.f; a.mx[st] = RA_NEG_INF; }
+    }
+    return;
+  }
+
+  // ---- staging: direct global -> LDS loads (RA_DMA_TILE), issued by the four wavefronts of group B
+  // at the start of their softmax phase (the compiler makes every LDS read of a wavefront wait for
+  // all of its outstanding direct loads, so they must not be issued right before a matrix phase).
+  const int wave_u = __builtin_amdgcn_readfirstlane(w4);
+  const int dchunk0 = (lane & 15) ^ ((lane >> 4) << 2);
+  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * w4 + (lane >> 4)) * a.kv_ss;
+  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * w4 + (lane >> 4)) * a.kv_ss;
+#define RA_PP_DMA(LDS, GROW0, J) RA_DMA_TILE(LDS, GROW0, a.kv_ss, J, FBN)
+#define RA_PP_KEYINFO(J)                                                                                \
+  if ((HAS_SEG || HAS_BIAS) && tid >= 256 && tid < 256 + FBN) {                                         \
+    const int kj_ = (J) * FBN + tid - 256;                                                              \
+    if (HAS_SEG) {                                                                                      \
+      int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+      seg_ks[(J) & 3][tid - 256] = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                     \
+    }                                                                                                   \
+    if (HAS_BIAS) {                                                                                     \
+      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0 + kj_) * mv.bias_sk]; \
+      if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
+      bias_ks[(J) & 3][tid - 256] = bv_ * kLog2e;                                                             \
+    }                                                                                                   \
+  }
+
+  int k_off[8], v_off[4][2];
+  RA_LANE_OFFSETS(k_off, v_off);
+
+  f32x16 s[2];
+  bf16x8 pf[2][2];
+  float m_true = m2;
+  constexpr float kLazy = 16.f;
+
+// matrix phase for key tile J: S(J+1) and O += P(J) V(J).  Eight steps of four MFMAs on six
+// independent accumulator chains; the LDS fragments of step t+1 are requested before the MFMAs of
+// step t are issued, and nothing may move across a step boundary (bounded register pressure).
+#define RA_PP_FRAGS(T, KF, VF)                                                                          \
+  {                                                                                                     \
+    KF[0] = *(const bf16x8*)(&kb_[k_off[T]]);                                                           \
+    KF[1] = *(const bf16x8*)(&kb_[32 * TROW + k_off[T]]);                                               \
+    const uint16_t* vt_ = &vb_[((((T) >> 2) * 32) + (((T) >> 1) & 1) * 16) * TROW];                     \
+    _Pragma("unroll") for (int x = 0; x < 2; x++) {                                                     \
+      const int db_ = ((T) & 1) * 2 + x;                                                                \
+      s16x4 v0_ = lds_read_tr(vt_ + v_off[db_][0]);                                                     \
+      s16x4 v1_ = lds_read_tr(vt_ + v_off[db_][1]);                                                     \
+      VF[x] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(v0_, v1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
+    }                                                                                                   \
+  }
+#define RA_PP_MATRIX(J)                                                                                 \
+  {                                                                                                     \
+    const uint16_t* kb_ = Ks[((J) + 1) & 1];                                                            \
+    const uint16_t* vb_ = Vs[(J) & 1];                                                                  \
+    _Pragma("unroll") for (int r = 0; r < 16; r++) { s[0][r] = 0.f; s[1][r] = 0.f; }                    \
+    bf16x8 kf_[PP_DEPTH + 1][2], vf_[PP_DEPTH + 1][2];                                                  \
+    _Pragma("unroll") for (int t = 0; t < PP_DEPTH; t++) RA_PP_FRAGS(t, kf_[t], vf_[t]);                \
+    _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                     \
+      if (t + PP_DEPTH < 8)                                                                             \
+        RA_PP_FRAGS(t + PP_DEPTH, kf_[(t + PP_DEPTH) % (PP_DEPTH + 1)], vf_[(t + PP_DEPTH) % (PP_DEPTH + 1)]); \
+      const int blk_ = t >> 2, tt_ = (t >> 1) & 1, db_ = (t & 1) * 2, c_ = t % (PP_DEPTH + 1);          \
+      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_[c_][0], qf[t], s[0], 0, 0, 0);                 \
+      acc[db_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf_[c_][0], pf[blk_][tt_], acc[db_], 0, 0, 0); \
+      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_[c_][1], qf[t], s[1], 0, 0, 0);                 \
+      acc[db_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf_[c_][1], pf[blk_][tt_], acc[db_ + 1], 0, 0, 0); \
+      __builtin_amdgcn_sched_barrier(0);                                                                \
+    }                                                                                                   \
+  }
+
+// vector phase: softmax of s = S(T) -> pf = P(T); updates m2, m_true, l, rescales acc when needed
+#define RA_PP_SOFTMAX(T)                                                                                \
+  {                                                                                                     \
+    const int t_ = (T);                                                                                 \
+    const int gk_tile_ = gk0 + t_ * FBN;                                                                \
+    if (t_ >= ntiles_grp) {                                                                             \
+      _Pragma("unroll") for (int x = 0; x < 8; x++) {                                                   \
+        pf[0][0][x] = (__bf16)0.f; pf[0][1][x] = (__bf16)0.f; pf[1][0][x] = (__bf16)0.f; pf[1][1][x] = (__bf16)0.f; \
+      }                                                                                                 \
+    } else if (!(HAS_SEG || HAS_BIAS) && (gk_tile_ + FBN - 1 < klim_wave)) {                            \
+      float mxv_ = s[0][0];                                                                             \
+      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
+        _Pragma("unroll") for (int r = 0; r < 16; r++) mxv_ = fmaxf(mxv_, s[blk][r]);                   \
+      mxv_ = max_xor32(mxv_);                                                                  \
+      m_true = fmaxf(m_true, mxv_ * c);                                                                 \
+      if (__builtin_amdgcn_ballot_w64(m_true - m2 > kLazy) != 0) {                                      \
+        const float alpha_ = fast_exp2(m2 - m_true);                                                    \
+        m2 = m_true;                                                                                    \
+        l *= alpha_;                                                                                    \
+        _Pragma("unroll") for (int db = 0; db < 4; db++)                                                \
+          _Pragma("unroll") for (int r = 0; r < 16; r++) acc[db][r] *= alpha_;                          \
+      }                                                                                                 \
+      float ps_ = 0.f;                                                                                  \
+      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
+        _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
+          float p_ = fast_exp2(fmaf(s[blk][r], c, -m2));                                                \
+          ps_ += p_;                                                                                    \
+          pf[blk][r >> 3][r & 7] = (__bf16)p_;                                                          \
+        }                                                                                               \
+      l += ps_;                                                                                         \
+    } else {                                                                                            \
+      float mxv_ = RA_NEG_INF;                                                                          \
+      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
+        _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
+          const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);                                   \
+          float x_ = s[blk][r] * c;                                                                     \
+          if (HAS_BIAS) x_ += bias_ks[t_ & 3][kr_];                                                     \
+          bool masked_ = (gk_tile_ + kr_ >= klim);                                                      \
+          if (HAS_SEG) masked_ = masked_ || (seg_ks[t_ & 3][kr_] != seg_q);                             \
+          x_ = masked_ ? kMask2 : x_;                                                                   \
+          s[blk][r] = x_;                                                                               \
+          mxv_ = fmaxf(mxv_, x_);                                                                       \
+        }                                                                                               \
+      mxv_ = max_xor32(mxv_);                                                                  \
+      m_true = fmaxf(m_true, mxv_);                                                                     \
+      const float m_new_ = fmaxf(m2, mxv_);                                                             \
+      const float alpha_ = fast_exp2(m2 - m_new_);                                                      \
+      m2 = m_new_;                                                                                      \
+      float ps_ = 0.f;                                                                                  \
+      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
+        _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
+          float p_ = fast_exp2(s[blk][r] - m_new_);                                                     \
+          ps_ += p_;                                                                                    \
+          pf[blk][r >> 3][r & 7] = (__bf16)p_;                                                          \
+        }                                                                                               \
+      l = l * alpha_ + ps_;                                                                             \
+      if (__builtin_amdgcn_ballot_w64(alpha_ != 1.f) != 0) {                                            \
+        _Pragma("unroll") for (int db = 0; db < 4; db++)                                                \
+          _Pragma("unroll") for (int r = 0; r < 16; r++) acc[db][r] *= alpha_;                          \
+      }                                                                                                 \
+    }                                                                                                   \
+  }
+
+  // ---- prologue
+  if (grp == 1) {
+    RA_PP_DMA(Ks[0], kg, 0);
+    RA_PP_DMA(Vs[0], vg, 0);
+    RA_PP_DMA(Ks[1], kg, min(1, ntiles - 1));
+  }
+  RA_PP_KEYINFO(0);
+  RA_PP_KEYINFO(min(1, ntiles - 1));
+  RA_DMA_WAIT();
+  __syncthreads();
+  {
+    f32x16 sn0, sn1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) { sn0[r] = 0.f; sn1[r] = 0.f; }
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      bf16x8 kf0 = *(const bf16x8*)(&Ks[0][k_off[t]]);
+      sn0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf0, qf[t], sn0, 0, 0, 0);
+      bf16x8 kf1 = *(const bf16x8*)(&Ks[0][32 * TROW + k_off[t]]);
+      sn1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf1, qf[t], sn1, 0, 0, 0);
+    }
+    s[0] = sn0; s[1] = sn1;
+  }
+  // One loop body for every wavefront: matrix(j), barrier, softmax(j+1), barrier.  Group B enters the
+  // loop one phase (one barrier) later than group A, which puts its matrix phases against group A's
+  // softmax phases; group A pays the missing barrier at the end.
+#ifdef RA_TRACE
+  const bool trace_on = blockIdx.x == 0;
+  int trace_n = 0;
+#endif
+  if (grp == 0) RA_PP_SOFTMAX(0);
+  __syncthreads();                    // every wave is done with K(0) before phase 0 overwrites it
+  // K(j+2) -> Ks[j&1] and V(j+1) -> Vs[(j+1)&1] are requested at the start of phase 2j (both buffers
+  // were last read in phase 2j-1) and awaited before the barrier that ends phase 2j+1.
+#define RA_PP_STAGE(J)                                                                                  \
+  {                                                                                                     \
+    RA_PP_DMA(Ks[(J) & 1], kg, min((J) + 2, ntiles - 1));                                               \
+    RA_PP_DMA(Vs[((J) + 1) & 1], vg, min((J) + 1, ntiles - 1));                                         \
+    RA_PP_KEYINFO(min((J) + 2, ntiles - 1));                                                            \
+  }
+  if (grp == 1) {
+    RA_PP_STAGE(0);
+    RA_PP_SOFTMAX(0);                 // phase 0 of group B
+    __syncthreads();
+  }
+  for (int j = 0; j < ntiles; j++) {
+    RA_TRACE_MARK();
+    if (PP_PRIO) __builtin_amdgcn_s_setprio(1);
+    RA_PP_MATRIX(j);                  // phase 2j (A) / 2j+1 (B)
+    if (PP_PRIO) __builtin_amdgcn_s_setprio(0);
+    RA_TRACE_MARK();
+    if (grp == 1) RA_DMA_WAIT();      // end of phase 2j+1: K(j+2), V(j+1) have landed
+    __syncthreads();
+    RA_TRACE_MARK();
+    if (grp == 1 && j + 1 < ntiles) RA_PP_STAGE(j + 1);     // start of phase 2(j+1)
+    RA_TRACE_MARK();
+    RA_PP_SOFTMAX(j + 1);             // for j + 1 == ntiles the tile is past the range: P = 0
+    RA_TRACE_MARK();
+    __syncthreads();
+  }
+#undef RA_PP_STAGE
+#undef RA_PP_DMA
+  if (grp == 0) __syncthreads();
+#undef RA_PP_KEYINFO
+#undef RA_PP_MATRIX
+#undef RA_PP_FRAGS
+#undef RA_PP_SOFTMAX
+
+  if (__builtin_amdgcn_ballot_w64(m_true != m2) != 0) {     // bring the carry to the exact running max
+    const float fix = (m_true == m2) ? 1.f : fast_exp2(m2 - m_true);
+    m2 = m_true;
+    l *= fix;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[db][r] *= fix;
+  }
 #pragma unroll
   for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -300,7 +776,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
 //          P and dS (accumulator layout, lane <-> key column) feed dV^T += dO^T P and
 //          dK^T += Q^T dS directly as B operands; Q^T / dO^T come from LDS transpose reads.
 // Probabilities are recomputed from the saved max_score / denominator (ringattention_jax.py:226).
-constexpr int BSTR = HD + 24;    // LDS row stride for tiles read both row-wise and transposed
 
 struct BwdArgs {
   const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* g;
@@ -316,8 +791,8 @@ struct BwdArgs {
 
 template <bool HAS_SEG, bool HAS_BIAS>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][FBN * BSTR];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][FBN * KSTR];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
   __shared__ int seg_ks[2][FBN];
   __shared__ float bias_ks[2][FBN];
 
@@ -374,22 +849,29 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
     for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
 
   const int srow = tid >> 4, schunk = tid & 15;
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8;
+  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.kv_ss;
+  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.kv_ss;
+  const int64_t row16 = 16 * a.kv_ss;
   uint4 kr[4], vr[4];
   int seg_r = 0;
   float bias_r = 0.f;
-  RA_LOAD_KV_TILE(0);
-  RA_STORE_KV_TILE(0, BSTR, KSTR);
+  RA_LOAD_TILE(kr, kg, a.kv_ss, 0, FBN);
+  RA_LOAD_TILE(vr, vg, a.kv_ss, 0, FBN);
+  RA_LOAD_KEYINFO(0);
+  RA_STORE_TILE(kr, Ks[0]);
+  RA_STORE_TILE(vr, Vs[0]);
+  RA_STORE_KEYINFO(0);
   __syncthreads();
 
-  const int ktr_lane_off = ((lane & 15) >> 2) * BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * BSTR;
-  const int k_lane_off = lo * BSTR + hi * 8;
-  const int v_lane_off = lo * KSTR + hi * 8;
+  int n_off[8], t_off[4][2];
+  RA_LANE_OFFSETS(n_off, t_off);
 
   for (int j = 0; j < ntiles; j++) {
     const int cur = j & 1;
-    RA_LOAD_KV_TILE(min(j + 1, ntiles - 1));
+    RA_LOAD_TILE(kr, kg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
+    RA_LOAD_TILE(vr, vg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
+    RA_LOAD_KEYINFO(min(j + 1, ntiles - 1));
     const int gk_tile = gk0 + j * FBN;
     const bool need_mask = HAS_SEG || HAS_BIAS || (gk_tile + FBN - 1 >= klim_wave);
 
@@ -398,16 +880,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
       f32x16 s, dp;
 #pragma unroll
       for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
-      const uint16_t* kp = &Ks[cur][blk * 32 * BSTR + k_lane_off];
-      const uint16_t* vp = &Vs[cur][blk * 32 * KSTR + v_lane_off];
+      const uint16_t* kp = &Ks[cur][blk * 32 * TROW];
+      const uint16_t* vp = &Vs[cur][blk * 32 * TROW];
 #pragma unroll
       for (int t = 0; t < 8; t++) {
-        bf16x8 kf = *(const bf16x8*)(kp + t * 16);
+        bf16x8 kf = *(const bf16x8*)(kp + n_off[t]);
         s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s, 0, 0, 0);          // S^T = K Q^T
       }
 #pragma unroll
       for (int t = 0; t < 8; t++) {
-        bf16x8 vf = *(const bf16x8*)(vp + t * 16);
+        bf16x8 vf = *(const bf16x8*)(vp + n_off[t]);
         dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, gf[t], dp, 0, 0, 0);        // dP^T = V dO^T
       }
       bf16x8 dsf[2];
@@ -428,22 +910,22 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
         dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - delta));                          // :229
       }
       // dQ^T += K^T dS^T over these 32 keys
-      const uint16_t* ktp = &Ks[cur][blk * 32 * BSTR + ktr_lane_off];
 #pragma unroll
       for (int t = 0; t < 2; t++)
 #pragma unroll
         for (int db = 0; db < 4; db++) {
-          s16x4 k0v = lds_read_tr(ktp + t * 16 * BSTR + db * 32);
-          s16x4 k1v = lds_read_tr(ktp + (t * 16 + 8) * BSTR + db * 32);
+          const uint16_t* ktp = &Ks[cur][(blk * 32 + t * 16) * TROW];
+          s16x4 k0v = lds_read_tr(ktp + t_off[db][0]);
+          s16x4 k1v = lds_read_tr(ktp + t_off[db][1]);
           s16x8 kk = __builtin_shufflevector(k0v, k1v, 0, 1, 2, 3, 4, 5, 6, 7);
           acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), dsf[t], acc[db], 0, 0, 0);
         }
     }
-    RA_STORE_KV_TILE(cur ^ 1, BSTR, KSTR);
+    RA_STORE_TILE(kr, Ks[cur ^ 1]);
+    RA_STORE_TILE(vr, Vs[cur ^ 1]);
+    RA_STORE_KEYINFO(cur ^ 1);
     __syncthreads();
   }
-#undef RA_LOAD_KV_TILE
-#undef RA_STORE_KV_TILE
 
   // dq += acc / sqrt(D)   (:230)
   const float rscale = 1.f / sqrtf((float)HD);
@@ -462,10 +944,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
 constexpr int KBN = 128;   // keys per workgroup in the dK/dV kernel (32 per wavefront)
 constexpr int KBM = 64;    // query rows per step
 
-template <bool HAS_SEG, bool HAS_BIAS>
-__global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][KBM * BSTR];
-  __shared__ __attribute__((aligned(16))) uint16_t Gs[2][KBM * BSTR];
+template <bool HAS_SEG, bool HAS_BIAS, bool WANT_DK, bool WANT_DV>
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][KBM * TROW];
+  __shared__ __attribute__((aligned(16))) uint16_t Gs[2][KBM * TROW];
   __shared__ __attribute__((aligned(16))) float st_m2[2][KBM];
   __shared__ __attribute__((aligned(16))) float st_rden[2][KBM];
   __shared__ __attribute__((aligned(16))) float st_delta[2][KBM];
@@ -526,34 +1008,35 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
 
   // K and V fragments of this lane's key column (B operands), resident for the whole loop
   const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
-  bf16x8 kf[8], vf[8];
+  bf16x8 kf[8], vf[WANT_DK ? 8 : 1];
 #pragma unroll
   for (int t = 0; t < 8; t++) {
     kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
-    vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
+    if (WANT_DK) vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
   }
-  f32x16 dkacc[4], dvacc[4];
+  f32x16 dkacc[WANT_DK ? 4 : 1], dvacc[WANT_DV ? 4 : 1];
 #pragma unroll
   for (int db = 0; db < 4; db++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+    for (int r = 0; r < 16; r++) {
+      if (WANT_DK) dkacc[db][r] = 0.f;
+      if (WANT_DV) dvacc[db][r] = 0.f;
+    }
 
   const int srow = tid >> 4, schunk = tid & 15;
-  const uint16_t* qg = a.q + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8;
-  const uint16_t* gg = a.g + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8;
+  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const uint16_t* qg = a.q + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.q_ss;
+  const uint16_t* gg = a.g + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.q_ss;
+  const int64_t row16 = 16 * a.q_ss;
   uint4 qr[4], gr[4];
   float r_m2 = 0.f, r_rden = 0.f, r_delta = 0.f;
   int r_seg = 0;
 #define RA_LOAD_Q_TILE(QT)                                                                              \
   {                                                                                                     \
-    const int q0_ = (QT) * KBM;                                                                         \
-    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
-      const int64_t off_ = (int64_t)(q0_ + p * 16 + srow) * a.q_ss;                                     \
-      qr[p] = *(const uint4*)(qg + off_);                                                               \
-      gr[p] = *(const uint4*)(gg + off_);                                                               \
-    }                                                                                                   \
+    RA_LOAD_TILE(qr, qg, a.q_ss, (QT), KBM);                                                            \
+    RA_LOAD_TILE(gr, gg, a.q_ss, (QT), KBM);                                                            \
     if (tid < KBM) {                                                                                    \
-      const int row_ = q0_ + tid;                                                                       \
+      const int row_ = (QT) * KBM + tid;                                                                \
       const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
       r_m2 = max_to_log2(a.mx[st_], kMask2);                                                            \
       r_rden = 1.f / a.den[st_];                                                                        \
@@ -566,10 +1049,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   }
 #define RA_STORE_Q_TILE(BUF)                                                                            \
   {                                                                                                     \
-    _Pragma("unroll") for (int p = 0; p < 4; p++) {                                                     \
-      *(uint4*)(&Qs[BUF][(p * 16 + srow) * BSTR + schunk * 8]) = qr[p];                                 \
-      *(uint4*)(&Gs[BUF][(p * 16 + srow) * BSTR + schunk * 8]) = gr[p];                                 \
-    }                                                                                                   \
+    RA_STORE_TILE(qr, Qs[BUF]);                                                                         \
+    RA_STORE_TILE(gr, Gs[BUF]);                                                                         \
     if (tid < KBM) {                                                                                    \
       st_m2[BUF][tid] = r_m2; st_rden[BUF][tid] = r_rden; st_delta[BUF][tid] = r_delta;                 \
       if (HAS_SEG) st_seg[BUF][tid] = r_seg;                                                            \
@@ -579,8 +1060,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   RA_STORE_Q_TILE(0);
   __syncthreads();
 
-  const int tr_lane_off = ((lane & 15) >> 2) * BSTR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + 4 * hi * BSTR;
-  const int nat_lane_off = lo * BSTR + hi * 8;
+  int n_off[8], t_off[4][2];
+  RA_LANE_OFFSETS(n_off, t_off);
 
   for (int qt = qt_first; qt < nqt; qt++) {
     const int cur = (qt - qt_first) & 1;
@@ -593,17 +1074,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
       f32x16 s, dp;
 #pragma unroll
       for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
-      const uint16_t* qp = &Qs[cur][qb * 32 * BSTR + nat_lane_off];
-      const uint16_t* gp = &Gs[cur][qb * 32 * BSTR + nat_lane_off];
+      const uint16_t* qp = &Qs[cur][qb * 32 * TROW];
+      const uint16_t* gp = &Gs[cur][qb * 32 * TROW];
 #pragma unroll
       for (int t = 0; t < 8; t++) {
-        bf16x8 qa = *(const bf16x8*)(qp + t * 16);
+        bf16x8 qa = *(const bf16x8*)(qp + n_off[t]);
         s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[t], s, 0, 0, 0);          // S = Q K^T
       }
+      if (WANT_DK) {
 #pragma unroll
-      for (int t = 0; t < 8; t++) {
-        bf16x8 ga = *(const bf16x8*)(gp + t * 16);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[t], dp, 0, 0, 0);        // dP = dO V^T
+        for (int t = 0; t < 8; t++) {
+          bf16x8 ga = *(const bf16x8*)(gp + n_off[t]);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[t], dp, 0, 0, 0);      // dP = dO V^T
+        }
       }
       bf16x8 pf[2], dsf[2];
 #pragma unroll
@@ -626,25 +1109,29 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
             x = masked ? kMask2 : x;
             p = fast_exp2(x - vm2[e]) * vrd[e];
           }
-          pf[r >> 3][r & 7] = (__bf16)p;
-          dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - vdl[e]));
+          if (WANT_DV) pf[r >> 3][r & 7] = (__bf16)p;
+          if (WANT_DK) dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - vdl[e]));
         }
       }
       // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over these 32 query rows)
-      const uint16_t* gtp = &Gs[cur][qb * 32 * BSTR + tr_lane_off];
-      const uint16_t* qtp = &Qs[cur][qb * 32 * BSTR + tr_lane_off];
 #pragma unroll
       for (int t = 0; t < 2; t++)
 #pragma unroll
         for (int db = 0; db < 4; db++) {
-          s16x4 g0 = lds_read_tr(gtp + t * 16 * BSTR + db * 32);
-          s16x4 g1 = lds_read_tr(gtp + (t * 16 + 8) * BSTR + db * 32);
-          s16x8 gv = __builtin_shufflevector(g0, g1, 0, 1, 2, 3, 4, 5, 6, 7);
-          dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, gv), pf[t], dvacc[db], 0, 0, 0);
-          s16x4 q0v = lds_read_tr(qtp + t * 16 * BSTR + db * 32);
-          s16x4 q1v = lds_read_tr(qtp + (t * 16 + 8) * BSTR + db * 32);
-          s16x8 qv = __builtin_shufflevector(q0v, q1v, 0, 1, 2, 3, 4, 5, 6, 7);
-          dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), dsf[t], dkacc[db], 0, 0, 0);
+          if (WANT_DV) {
+            const uint16_t* gtp = &Gs[cur][(qb * 32 + t * 16) * TROW];
+            s16x4 g0 = lds_read_tr(gtp + t_off[db][0]);
+            s16x4 g1 = lds_read_tr(gtp + t_off[db][1]);
+            s16x8 gv = __builtin_shufflevector(g0, g1, 0, 1, 2, 3, 4, 5, 6, 7);
+            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, gv), pf[t], dvacc[db], 0, 0, 0);
+          }
+          if (WANT_DK) {
+            const uint16_t* qtp = &Qs[cur][(qb * 32 + t * 16) * TROW];
+            s16x4 q0v = lds_read_tr(qtp + t_off[db][0]);
+            s16x4 q1v = lds_read_tr(qtp + t_off[db][1]);
+            s16x8 qv = __builtin_shufflevector(q0v, q1v, 0, 1, 2, 3, 4, 5, 6, 7);
+            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), dsf[t], dkacc[db], 0, 0, 0);
+          }
         }
     }
     RA_STORE_Q_TILE(cur ^ 1);
@@ -660,12 +1147,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   for (int db = 0; db < 4; db++)
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      float* pk = a.dk + ooff + db * 32 + g * 8;
-      float* pv = a.dv + ooff + db * 32 + g * 8;
-      f32x4 tk = *(const f32x4*)pk, tv = *(const f32x4*)pv;
+      if (WANT_DK) {
+        float* pk = a.dk + ooff + db * 32 + g * 8;
+        f32x4 tk = *(const f32x4*)pk;
 #pragma unroll
-      for (int e = 0; e < 4; e++) { tk[e] += dkacc[db][g * 4 + e] * rscale; tv[e] += dvacc[db][g * 4 + e]; }
-      *(f32x4*)pk = tk; *(f32x4*)pv = tv;
+        for (int e = 0; e < 4; e++) tk[e] += dkacc[db][g * 4 + e] * rscale;
+        *(f32x4*)pk = tk;
+      }
+      if (WANT_DV) {
+        float* pv = a.dv + ooff + db * 32 + g * 8;
+        f32x4 tv = *(const f32x4*)pv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) tv[e] += dvacc[db][g * 4 + e];
+        *(f32x4*)pv = tv;
+      }
     }
 }
 
@@ -690,10 +1185,21 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
+  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
+  if (p->mask.query_chunk_size % PBM == 0 && !getenv("RA_FWD_NO_PINGPONG")) {
+    const long long nwg2 = (long long)(p->Sq / PBM) * p->H * p->B;
+    RA_REQUIRE(nwg2 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
+    dim3 grid2((unsigned)nwg2), block2(512);
+    if (seg && bias) attn_fwd_pp_kernel<true, true><<<grid2, block2, 0, s>>>(a);
+    else if (seg) attn_fwd_pp_kernel<true, false><<<grid2, block2, 0, s>>>(a);
+    else if (bias) attn_fwd_pp_kernel<false, true><<<grid2, block2, 0, s>>>(a);
+    else attn_fwd_pp_kernel<false, false><<<grid2, block2, 0, s>>>(a);
+    RA_CHECK_LAUNCH("attn_fwd_pp");
+    return RA_OK;
+  }
   const long long nwg = (long long)(p->Sq / FBM) * p->H * p->B;
   RA_REQUIRE(nwg < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
   dim3 grid((unsigned)nwg), block(256);
-  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   if (seg && bias) attn_fwd_mfma_kernel<true, true><<<grid, block, 0, s>>>(a);
   else if (seg) attn_fwd_mfma_kernel<true, false><<<grid, block, 0, s>>>(a);
   else if (bias) attn_fwd_mfma_kernel<false, true><<<grid, block, 0, s>>>(a);
@@ -729,7 +1235,10 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
   const bool do_dkv = !(p->impl & RA_BWD_ONLY_DQ), do_dq = !(p->impl & RA_BWD_ONLY_DKV);
 #define RA_LAUNCH_BWD(SEG, BIAS)                                                         \
   do {                                                                                   \
-    if (do_dkv) attn_bwd_dkv_mfma_kernel<SEG, BIAS><<<gk, block, 0, s>>>(a);             \
+    if (do_dkv) {                                                                        \
+      attn_bwd_dkv_mfma_kernel<SEG, BIAS, true, false><<<gk, block, 0, s>>>(a);          \
+      attn_bwd_dkv_mfma_kernel<SEG, BIAS, false, true><<<gk, block, 0, s>>>(a);          \
+    }                                                                                    \
     if (do_dq) attn_bwd_dq_mfma_kernel<SEG, BIAS><<<gq, block, 0, s>>>(a);               \
   } while (0)
   if (seg && bias) RA_LAUNCH_BWD(true, true);
