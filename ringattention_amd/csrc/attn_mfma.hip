@@ -548,14 +548,27 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
     return;
   }
 
-  // ---- staging: direct global -> LDS loads (RA_DMA_TILE), issued by the four wavefronts of group B
-  // at the start of their softmax phase (the compiler makes every LDS read of a wavefront wait for
-  // all of its outstanding direct loads, so they must not be issued right before a matrix phase).
-  const int wave_u = __builtin_amdgcn_readfirstlane(w4);
-  const int dchunk0 = (lane & 15) ^ ((lane >> 4) << 2);
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * w4 + (lane >> 4)) * a.kv_ss;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * w4 + (lane >> 4)) * a.kv_ss;
-#define RA_PP_DMA(LDS, GROW0, J) RA_DMA_TILE(LDS, GROW0, a.kv_ss, J, FBN)
+  // ---- staging through registers, two phases ahead.  (Direct global->LDS loads allow very few
+  // requests in flight per CU on this part and block the issuing wavefront; plain loads do not.)
+  // Group B brings in the K tiles, group A the V tiles: at the start of each of its softmax phases a
+  // group stores the tile it requested in its previous softmax phase - the loads have had a whole
+  // matrix phase to land - and requests the next one.
+  const int srow = (tid & 255) >> 4, schunk = tid & 15;
+  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const uint16_t* sg = (grp == 1 ? a.k : a.v) + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.kv_ss;
+  const int64_t row16 = 16 * a.kv_ss;
+  uint4 sr0, sr1, sr2, sr3;       // scalars, not an array: an array here ends up in scratch memory
+#define RA_PP_LOAD4(J)                                                                                  \
+  {                                                                                                     \
+    const uint16_t* p_ = sg + (int64_t)(J) * FBN * a.kv_ss;                                             \
+    sr0 = *(const uint4*)(p_); sr1 = *(const uint4*)(p_ + row16);                                       \
+    sr2 = *(const uint4*)(p_ + 2 * row16); sr3 = *(const uint4*)(p_ + 3 * row16);                       \
+  }
+#define RA_PP_STORE4(LDS)                                                                               \
+  {                                                                                                     \
+    *(uint4*)(&(LDS)[s_off]) = sr0; *(uint4*)(&(LDS)[16 * TROW + s_off]) = sr1;                         \
+    *(uint4*)(&(LDS)[32 * TROW + s_off]) = sr2; *(uint4*)(&(LDS)[48 * TROW + s_off]) = sr3;             \
+  }
 #define RA_PP_KEYINFO(J)                                                                                \
   if ((HAS_SEG || HAS_BIAS) && tid >= 256 && tid < 256 + FBN) {                                         \
     const int kj_ = (J) * FBN + tid - 256;                                                              \
@@ -675,15 +688,21 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
     }                                                                                                   \
   }
 
-  // ---- prologue
+  // ---- prologue: K(0), K(1) into LDS and K(2) into registers by group B; V(0) into LDS and V(1)
+  // into registers by group A
   if (grp == 1) {
-    RA_PP_DMA(Ks[0], kg, 0);
-    RA_PP_DMA(Vs[0], vg, 0);
-    RA_PP_DMA(Ks[1], kg, min(1, ntiles - 1));
+    RA_PP_LOAD4(0);
+    RA_PP_STORE4(Ks[0]);
+    RA_PP_LOAD4(min(1, ntiles - 1));
+    RA_PP_STORE4(Ks[1]);
+    RA_PP_LOAD4(min(2, ntiles - 1));
+  } else {
+    RA_PP_LOAD4(0);
+    RA_PP_STORE4(Vs[0]);
+    RA_PP_LOAD4(min(1, ntiles - 1));
   }
   RA_PP_KEYINFO(0);
   RA_PP_KEYINFO(min(1, ntiles - 1));
-  RA_DMA_WAIT();
   __syncthreads();
   {
     f32x16 sn0, sn1;
@@ -707,38 +726,41 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
 #endif
   if (grp == 0) RA_PP_SOFTMAX(0);
   __syncthreads();                    // every wave is done with K(0) before phase 0 overwrites it
-  // K(j+2) -> Ks[j&1] and V(j+1) -> Vs[(j+1)&1] are requested at the start of phase 2j (both buffers
-  // were last read in phase 2j-1) and awaited before the barrier that ends phase 2j+1.
-#define RA_PP_STAGE(J)                                                                                  \
-  {                                                                                                     \
-    RA_PP_DMA(Ks[(J) & 1], kg, min((J) + 2, ntiles - 1));                                               \
-    RA_PP_DMA(Vs[((J) + 1) & 1], vg, min((J) + 1, ntiles - 1));                                         \
-    RA_PP_KEYINFO(min((J) + 2, ntiles - 1));                                                            \
-  }
   if (grp == 1) {
-    RA_PP_STAGE(0);
+    RA_PP_STORE4(Ks[0]);                                     // K(2); K(0) was consumed by the prologue
+    RA_PP_LOAD4(min(3, ntiles - 1));       // K(3)
+    RA_PP_KEYINFO(min(2, ntiles - 1));
     RA_PP_SOFTMAX(0);                 // phase 0 of group B
     __syncthreads();
   }
   for (int j = 0; j < ntiles; j++) {
     RA_TRACE_MARK();
     if (PP_PRIO) __builtin_amdgcn_s_setprio(1);
+#ifndef RA_ABL_NOMATRIX
     RA_PP_MATRIX(j);                  // phase 2j (A) / 2j+1 (B)
+#endif
     if (PP_PRIO) __builtin_amdgcn_s_setprio(0);
     RA_TRACE_MARK();
-    if (grp == 1) RA_DMA_WAIT();      // end of phase 2j+1: K(j+2), V(j+1) have landed
     __syncthreads();
     RA_TRACE_MARK();
-    if (grp == 1 && j + 1 < ntiles) RA_PP_STAGE(j + 1);     // start of phase 2(j+1)
+#ifndef RA_ABL_NOSTAGE
+    // group A, phase 2j+1: V(j+1) -> Vs[(j+1)&1] (V(j-1) was last read in phase 2j-1), request V(j+2);
+    // group B, phase 2j+2: K(j+3) -> Ks[(j+1)&1] (K(j+1) was last read in phase 2j+1), request K(j+4)
+    if (grp == 0) { RA_PP_STORE4(Vs[(j + 1) & 1]); } else { RA_PP_STORE4(Ks[(j + 1) & 1]); }
+    RA_PP_LOAD4(min(j + 2 + 2 * grp, ntiles - 1));
+    if (grp == 1) RA_PP_KEYINFO(min(j + 3, ntiles - 1));
+#endif
     RA_TRACE_MARK();
+#ifndef RA_ABL_NOSOFTMAX
     RA_PP_SOFTMAX(j + 1);             // for j + 1 == ntiles the tile is past the range: P = 0
+#endif
     RA_TRACE_MARK();
     __syncthreads();
   }
-#undef RA_PP_STAGE
-#undef RA_PP_DMA
   if (grp == 0) __syncthreads();
 #undef RA_PP_KEYINFO
+#undef RA_PP_LOAD4
+#undef RA_PP_STORE4
 #undef RA_PP_MATRIX
 #undef RA_PP_FRAGS
 #undef RA_PP_SOFTMAX
