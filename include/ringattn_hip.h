@@ -62,6 +62,11 @@ typedef struct ra_mask {
   float mask_min;             /* finfo(blockwise_kwargs["dtype"]).min (:298,:308) */
   int32_t skip_masked_tiles;  /* 1: kernels may also skip sub-tiles whose every pair is masked; exact
                                  unless a query row has no unmasked key at all in the whole ring */
+  const int32_t* seg_tile_minmax; /* nullable; from ra_segment_tile_ranges: (B or 1, seg_tiles, 2) = min and max
+                                     segment id of every run of RA_SEG_TILE global positions.  With
+                                     skip_masked_tiles it lets kernels skip key (query) tiles whose id range
+                                     cannot meet the ids of the query (key) rows at hand */
+  int32_t seg_tiles;
 } ra_mask;
 
 /* _blockwise_attention_fwd (ringattention_jax.py:99-179): one ring step on one device.
@@ -96,6 +101,13 @@ typedef struct ra_attn_bwd_params {
   ra_mask mask;
   int32_t impl;
 } ra_attn_bwd_params;
+
+enum { RA_SEG_TILE = 64 };
+/* min / max segment id per run of RA_SEG_TILE positions: out (Bseg, ceil(seg_len / RA_SEG_TILE), 2).
+ * No counterpart in the reference (it evaluates the segment mask element by element, :285-299); this
+ * only feeds the tile-skipping of the kernels. */
+int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int32_t Bseg, int32_t seg_len,
+                           int32_t* out, ra_stream_t stream);
 
 /* Carry initialisation (ringattention_jax.py:22-23,:49): numerator = 0, denominator = 0, max = -inf. */
 int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s,

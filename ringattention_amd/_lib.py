@@ -13,6 +13,7 @@ RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
 RA_F32, RA_BF16 = 0, 1
 RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
 RA_BWD_ONLY_DQ, RA_BWD_ONLY_DKV = 0x10, 0x20
+RA_SEG_TILE = 64
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
@@ -23,7 +24,7 @@ class RaMask(C.Structure):
         ("bias_stride_k", i64), ("segment_ids", vp), ("seg_stride_b", i64), ("seg_len", i32),
         ("causal_block_size", i32), ("query_chunk_size", i32), ("key_chunk_size", i32),
         ("q_chunk_idx_start", i32), ("k_chunk_idx_start", i32), ("cache_idx", vp), ("mask_min", f32),
-        ("skip_masked_tiles", i32),
+        ("skip_masked_tiles", i32), ("seg_tile_minmax", vp), ("seg_tiles", i32),
     ]
 
 
@@ -70,6 +71,7 @@ class RaSwigluParams(C.Structure):
 
 # every symbol include/ringattn_hip.h declares: (name, restype, argtypes)
 SYMBOLS = {
+    "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
     "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),

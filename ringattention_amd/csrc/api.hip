@@ -26,6 +26,7 @@ int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, voi
              int, int, int, hipStream_t);
 int bwd_delta(const void*, const void*, int, int64_t, int64_t, float*, int64_t, int64_t, int, int, int, int,
               hipStream_t);
+int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
@@ -48,6 +49,9 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
   }
   RA_REQUIRE(m.q_chunk_idx_start >= 0 && m.k_chunk_idx_start >= 0, RA_ERR_INVALID, "%s: negative chunk start", who);
   if (m.segment_ids) RA_REQUIRE(m.seg_len > 0, RA_ERR_INVALID, "%s: segment_ids given with seg_len 0", who);
+  if (m.seg_tile_minmax)
+    RA_REQUIRE(m.segment_ids && m.seg_tiles == (m.seg_len + RA_SEG_TILE - 1) / RA_SEG_TILE, RA_ERR_INVALID,
+               "%s: seg_tile_minmax needs segment_ids and seg_tiles == ceil(seg_len / %d)", who, (int)RA_SEG_TILE);
   RA_REQUIRE((long long)m.q_chunk_idx_start * m.query_chunk_size + Sq < (1LL << 31) - 4096 &&
                  (long long)m.k_chunk_idx_start * m.key_chunk_size + Skv < (1LL << 31) - 4096,
              RA_ERR_UNSUPPORTED, "%s: global positions must stay below 2^31", who);
@@ -70,6 +74,13 @@ int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_strid
   RA_REQUIRE(B > 0 && Sq > 0 && H > 0 && D > 0, RA_ERR_INVALID, "carry_init: empty shape");
   return carry_init(numerator, num_stride_b, num_stride_s, denominator, max_score, stat_stride_b, stat_stride_h, B,
                     Sq, H, D, (hipStream_t)stream);
+}
+
+int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int32_t Bseg, int32_t seg_len,
+                           int32_t* out, ra_stream_t stream) {
+  RA_REQUIRE(segment_ids && out, RA_ERR_INVALID, "segment_tile_ranges: null pointer");
+  RA_REQUIRE(Bseg > 0 && Bseg <= 65535 && seg_len > 0, RA_ERR_INVALID, "segment_tile_ranges: bad shape");
+  return seg_tile_ranges(segment_ids, seg_stride_b, Bseg, seg_len, out, (hipStream_t)stream);
 }
 
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {

@@ -352,6 +352,26 @@ __global__ void delta_kernel(const T* g, const T* o, int64_t sb, int64_t ss, flo
   }
 }
 
+// min / max segment id of every run of RA_SEG_TILE positions: one wavefront per run
+__global__ void seg_tile_ranges_kernel(const int32_t* seg, int64_t seg_sb, int seg_len, int ntile, int32_t* out) {
+  const int b = blockIdx.y;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / 64, lane = threadIdx.x % 64;
+  if (wave >= ntile) return;
+  const int pos = wave * RA_SEG_TILE + lane;
+  const int v = seg[(int64_t)b * seg_sb + min(pos, seg_len - 1)];
+  int mn = v, mx = v;
+  for (int o = 32; o > 0; o >>= 1) { mn = min(mn, __shfl_xor(mn, o)); mx = max(mx, __shfl_xor(mx, o)); }
+  if (lane == 0) { out[((int64_t)b * ntile + wave) * 2] = mn; out[((int64_t)b * ntile + wave) * 2 + 1] = mx; }
+}
+
+int seg_tile_ranges(const int32_t* seg, int64_t seg_sb, int Bseg, int seg_len, int32_t* out, hipStream_t s) {
+  const int ntile = (seg_len + RA_SEG_TILE - 1) / RA_SEG_TILE;
+  dim3 grid((ntile + 3) / 4, Bseg);
+  seg_tile_ranges_kernel<<<grid, 256, 0, s>>>(seg, seg_sb, seg_len, ntile, out);
+  RA_CHECK_LAUNCH("seg_tile_ranges");
+  return RA_OK;
+}
+
 // ------------------------------------------------------------------ host-side launchers
 static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
   GenericArgs a{};

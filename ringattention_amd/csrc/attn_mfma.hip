@@ -70,6 +70,34 @@ __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 
 constexpr int TROW = HD;          // elements per LDS tile row
 constexpr int KV_TILE = FBN * TROW;
 
+// Hull [first, last+1) of the 64-position tiles, among the n tiles starting at global tile gt0, whose
+// segment-id range meets [lo, hi] (ids from ra_segment_tile_ranges).  Conservative: a tile outside the
+// hull holds no key (query) of a segment present in the rows at hand; tiles inside may still be fully
+// masked.  Every thread of the workgroup must call it; hull2 points at two ints of LDS.
+__device__ __forceinline__ void seg_tile_hull(const MaskView& mv, int b, int gt0, int n, int lo, int hi, int* hull2,
+                                              int tid, int nthreads, int& first, int& last) {
+  if (tid == 0) { hull2[0] = n; hull2[1] = 0; }
+  __syncthreads();
+  const int32_t* mm = mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2;
+  for (int t = tid; t < n; t += nthreads) {
+    const int g = min(gt0 + t, mv.seg_tiles - 1);
+    const int mn = mm[2 * g], mx = mm[2 * g + 1];
+    if (mx >= lo && mn <= hi) { atomicMin(&hull2[0], t); atomicMax(&hull2[1], t + 1); }
+  }
+  __syncthreads();
+  first = hull2[0]; last = hull2[1];
+  if (last < first) { first = 0; last = 0; }
+}
+// segment-id range of the rows [g0, g0 + rows) (global positions, multiples of 64)
+__device__ __forceinline__ void seg_rows_range(const MaskView& mv, int b, int g0, int rows, int& lo, int& hi) {
+  const int32_t* mm = mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2;
+  lo = 0x7fffffff; hi = -0x7fffffff - 1;
+  for (int t = g0 / RA_SEG_TILE; t < (g0 + rows) / RA_SEG_TILE; t++) {
+    const int g = min(t, mv.seg_tiles - 1);
+    lo = min(lo, mm[2 * g]); hi = max(hi, mm[2 * g + 1]);
+  }
+}
+
 // Staging helpers shared by the kernels below.  They expect in scope: tid, s_off (this thread's
 // swizzled element offset inside a 16-row slab), row16 (global element stride of 16 rows).
 #define RA_LOAD_TILE(REGS, BASE, STRIDE, J, ROWS)                                                       \
@@ -98,13 +126,13 @@ constexpr int KV_TILE = FBN * TROW;
 // per-key segment id / bias of key tile J (threads 0..63), for kernels that stream key tiles
 #define RA_LOAD_KEYINFO(J)                                                                              \
   if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                             \
-    const int kj_ = (J) * FBN + tid;                                                                    \
+    const int kj_ = k_base + (J) * FBN + tid;                                                           \
     if (HAS_SEG) {                                                                                      \
       int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
       seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                    \
     }                                                                                                   \
     if (HAS_BIAS) {                                                                                     \
-      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0 + kj_) * mv.bias_sk]; \
+      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
       if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
       bias_r = bv_ * kLog2e;                                                                            \
     }                                                                                                   \
@@ -152,13 +180,24 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
   int kend = mv.run_prefix_keys(qi, a.Skv);
   // global positions fit 31 bits (checked on the host)
   const int gq0 = (int)mv.global_q(q0);
-  const int gk0 = (int)mv.global_k(0);
+  const int gk0_shard = (int)mv.global_k(0);
   if (mv.cbs > 0 && mv.skip_tiles) {
     long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;   // first key position masked for every row
-    long long n = lim - gk0;
+    long long n = lim - gk0_shard;
     if (n < kend) kend = n > 0 ? (int)n : 0;
   }
-  const int ntiles = (kend + FBN - 1) / FBN;
+  int ntiles = (kend + FBN - 1) / FBN;
+  // key tiles outside the hull of those sharing a segment with these 128 rows are skipped
+  int k_base = 0;                           // local key index of the first tile processed
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gq0, FBM, slo, shi);
+    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 256, t_first, t_last);
+    k_base = t_first * FBN;
+    ntiles = t_last - t_first;
+  }
+  const int gk0 = gk0_shard + k_base;       // global position of the first key processed
 
   // per-lane mask constants: keys at global position >= klim are masked
   const int gq = gq0 + wave * 32 + lo;
@@ -213,8 +252,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
   // ---- staging: direct global -> LDS loads, see RA_DMA_TILE
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int dchunk0 = (lane & 15) ^ ((lane >> 4) << 2);
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * wave + (lane >> 4)) * a.kv_ss;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(16 * wave + (lane >> 4)) * a.kv_ss;
+  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(k_base + 16 * wave + (lane >> 4)) * a.kv_ss;
+  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(k_base + 16 * wave + (lane >> 4)) * a.kv_ss;
   int seg_r = 0;
   float bias_r = 0.f;
   int k_off[8], v_off[4][2];
@@ -489,17 +528,29 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   // end earlier sees its extra tiles fully masked and contributes nothing there.
   const int qi = q0 / mv.qc;                 // 256 | query_chunk_size: one chunk per workgroup
   const int kend_chunk = mv.run_prefix_keys(qi, a.Skv);
-  const int gk0 = (int)mv.global_k(0);
+  const int gk0_shard = (int)mv.global_k(0);
   const int gq_wg = (int)mv.global_q(q0);
   int kend_wg = kend_chunk, kend_grp = kend_chunk;
   if (mv.cbs > 0 && mv.skip_tiles) {
-    long long lim_wg = ((long long)(gq_wg + PBM - 1) / mv.cbs + 1) * mv.cbs - gk0;
-    long long lim_grp = ((long long)(gq_wg + grp * 128 + 127) / mv.cbs + 1) * mv.cbs - gk0;
+    long long lim_wg = ((long long)(gq_wg + PBM - 1) / mv.cbs + 1) * mv.cbs - gk0_shard;
+    long long lim_grp = ((long long)(gq_wg + grp * 128 + 127) / mv.cbs + 1) * mv.cbs - gk0_shard;
     if (lim_wg < kend_wg) kend_wg = lim_wg > 0 ? (int)lim_wg : 0;
     if (lim_grp < kend_grp) kend_grp = lim_grp > 0 ? (int)lim_grp : 0;
   }
-  const int ntiles = (kend_wg + FBN - 1) / FBN;        // workgroup-uniform
-  const int ntiles_grp = (kend_grp + FBN - 1) / FBN;   // tiles >= this are fully masked for the group
+  int ntiles = (kend_wg + FBN - 1) / FBN;              // workgroup-uniform
+  int ntiles_grp = (kend_grp + FBN - 1) / FBN;         // tiles >= this are fully masked for the group
+  // key tiles outside the hull of those sharing a segment with these 256 rows are skipped
+  int k_base = 0;                                      // local key index of the first tile processed
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gq_wg, PBM, slo, shi);
+    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
+    k_base = t_first * FBN;
+    ntiles = t_last - t_first;
+    ntiles_grp = min(max(ntiles_grp - t_first, 0), ntiles);
+  }
+  const int gk0 = gk0_shard + k_base;                  // global position of the first key processed
 
   const int gq = gq_wg + grp * 128 + w4 * 32 + lo;
   const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
@@ -555,7 +606,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   // matrix phase to land - and requests the next one.
   const int srow = (tid & 255) >> 4, schunk = tid & 15;
   const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const uint16_t* sg = (grp == 1 ? a.k : a.v) + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.kv_ss;
+  const uint16_t* sg = (grp == 1 ? a.k : a.v) + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
   const int64_t row16 = 16 * a.kv_ss;
   uint4 sr0, sr1, sr2, sr3;       // scalars, not an array: an array here ends up in scratch memory
 #define RA_PP_LOAD4(J)                                                                                  \
@@ -571,13 +622,13 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   }
 #define RA_PP_KEYINFO(J)                                                                                \
   if ((HAS_SEG || HAS_BIAS) && tid >= 256 && tid < 256 + FBN) {                                         \
-    const int kj_ = (J) * FBN + tid - 256;                                                              \
+    const int kj_ = k_base + (J) * FBN + tid - 256;                                                              \
     if (HAS_SEG) {                                                                                      \
       int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
       seg_ks[(J) & 3][tid - 256] = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                     \
     }                                                                                                   \
     if (HAS_BIAS) {                                                                                     \
-      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0 + kj_) * mv.bias_sk]; \
+      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
       if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
       bias_ks[(J) & 3][tid - 256] = bv_ * kLog2e;                                                             \
     }                                                                                                   \
@@ -832,14 +883,24 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
   const int qi = q0 / mv.qc;
   int kend = mv.run_prefix_keys(qi, a.Skv);
   const int gq0 = (int)mv.global_q(q0);
-  const int gk0 = (int)mv.global_k(0);
+  const int gk0_shard = (int)mv.global_k(0);
   if (mv.cbs > 0 && mv.skip_tiles) {
     long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
-    long long n = lim - gk0;
+    long long n = lim - gk0_shard;
     if (n < kend) kend = n > 0 ? (int)n : 0;
   }
-  const int ntiles = (kend + FBN - 1) / FBN;
+  int ntiles = (kend + FBN - 1) / FBN;
+  int k_base = 0;
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gq0, FBM, slo, shi);
+    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 256, t_first, t_last);
+    k_base = t_first * FBN;
+    ntiles = t_last - t_first;
+  }
   if (ntiles == 0) return;     // nothing to add to dq
+  const int gk0 = gk0_shard + k_base;
 
   const int gq = gq0 + wave * 32 + lo;
   const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
@@ -872,8 +933,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
 
   const int srow = tid >> 4, schunk = tid & 15;
   const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.kv_ss;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.kv_ss;
+  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
+  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
   const int64_t row16 = 16 * a.kv_ss;
   uint4 kr[4], vr[4];
   int seg_r = 0;
@@ -1009,7 +1070,17 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
       }
     }
   }
-  if (qt_first >= nqt) return;            // no query sees this key block: dk, dv unchanged
+  int qt_end = nqt;
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && qt_first < nqt) {
+    // query tiles outside the hull of those sharing a segment with these 128 keys are skipped
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gk0, KBN, slo, shi);
+    seg_tile_hull(mv, b, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, slo, shi, hull2, tid, 256, t_first, t_last);
+    qt_end = qt_first + t_last;
+    qt_first += t_first;
+  }
+  if (qt_first >= qt_end) return;         // no query sees this key block: dk, dv unchanged
 
   // masked iff gq / cbs < gk / cbs  <=>  gq < qlim
   const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;
@@ -1085,9 +1156,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
   int n_off[8], t_off[4][2];
   RA_LANE_OFFSETS(n_off, t_off);
 
-  for (int qt = qt_first; qt < nqt; qt++) {
+  for (int qt = qt_first; qt < qt_end; qt++) {
     const int cur = (qt - qt_first) & 1;
-    RA_LOAD_Q_TILE(min(qt + 1, nqt - 1));
+    RA_LOAD_Q_TILE(min(qt + 1, qt_end - 1));
     const int gq_tile = gq_base + qt * KBM;
     const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave);
 

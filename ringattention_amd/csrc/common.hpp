@@ -59,6 +59,8 @@ struct MaskView {
   float mask_min;
   int any_mask;
   int skip_tiles;
+  const int32_t* seg_mm;   // per-64-position (min, max) segment ids, or null
+  int seg_tiles;
 
   __host__ __device__ static MaskView make(const ra_mask& m, int q_chunk_idx_start) {
     MaskView v;
@@ -70,6 +72,7 @@ struct MaskView {
     v.mask_min = m.mask_min;
     v.any_mask = (m.segment_ids != nullptr) || (m.causal_block_size > 0);
     v.skip_tiles = m.skip_masked_tiles;
+    v.seg_mm = m.seg_tile_minmax; v.seg_tiles = m.seg_tiles;
     return v;
   }
 

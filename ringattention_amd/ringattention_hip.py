@@ -155,6 +155,8 @@ class _MaskInputs:
         self.seg = None
         self.seg_stride_b = 0
         self.seg_len = 0
+        self.seg_mm = None
+        self.seg_tiles = 0
         if segment_ids is not None:
             if segment_ids.dim() != 2:
                 raise ValueError("segment_ids must be 2-D (B, S)")
@@ -162,6 +164,12 @@ class _MaskInputs:
             self.seg = s
             self.seg_stride_b = 0 if s.shape[0] == 1 else s.stride(0)
             self.seg_len = s.shape[1]
+            # per-64-position (min, max) ids: lets the MFMA kernels skip tiles of foreign segments
+            self.seg_tiles = (self.seg_len + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
+            self.seg_mm = torch.empty((s.shape[0], self.seg_tiles, 2), dtype=torch.int32, device=device)
+            L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], self.seg_len,
+                                                    self.seg_mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
+            self._seg_mm_host = None
         self.cache_idx_host = None
         self.cache_idx_dev = None
         if cache_idx is not None:
@@ -188,7 +196,25 @@ class _MaskInputs:
         m.cache_idx = self.cache_idx_dev.data_ptr() if self.cache_idx_dev is not None else None
         m.mask_min = cfg.mask_min
         m.skip_masked_tiles = 1 if skip else 0
+        m.seg_tile_minmax = self.seg_mm.data_ptr() if self.seg_mm is not None else None
+        m.seg_tiles = self.seg_tiles
         return m
+
+    def segments_meet(self, q_lo, q_hi, k_lo, k_hi):
+        """False when no batch row has a segment id present both in global query positions
+        [q_lo, q_hi) and in global key positions [k_lo, k_hi) (conservative: id ranges are compared).
+        Costs one device->host copy of the per-tile ranges per call of ring_attention."""
+        if self.seg_mm is None:
+            return True
+        if self._seg_mm_host is None:
+            self._seg_mm_host = self.seg_mm.cpu().numpy()
+        mm = self._seg_mm_host
+        t = L.RA_SEG_TILE
+        qs = mm[:, q_lo // t:max(q_lo // t + 1, -(-q_hi // t))]
+        ks = mm[:, k_lo // t:max(k_lo // t + 1, -(-k_hi // t))]
+        q_min, q_max = qs[..., 0].min(axis=1), qs[..., 1].max(axis=1)
+        k_min, k_max = ks[..., 0].min(axis=1), ks[..., 1].max(axis=1)
+        return bool(((k_max >= q_min) & (k_min <= q_max)).any())
 
 
 def _check_qkv(q, k, v):
@@ -344,11 +370,18 @@ def _q_start(cfg, mi, dev, q_len):
 
 
 def _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
-    """False when the skip predicate drops every tile of this ring step (whole future shards)."""
-    if cfg.cbs is None or mi.cache_idx_dev is not None:
+    """False when the skip predicate drops every tile of this ring step (whole future shards), or -
+    with skip_masked_tiles - when no segment id is shared between the query and the key shard."""
+    if mi.cache_idx_dev is not None:
         return True
-    last_q_chunk = q_start + q_len // cfg.qc - 1
-    return run_prefix_keys(last_q_chunk, cfg.qc, cfg.kc, cfg.cbs, k_start, kv_len) > 0
+    if cfg.cbs is not None:
+        last_q_chunk = q_start + q_len // cfg.qc - 1
+        if run_prefix_keys(last_q_chunk, cfg.qc, cfg.kc, cfg.cbs, k_start, kv_len) <= 0:
+            return False
+    if cfg.skip_masked_tiles and mi.seg_mm is not None:
+        return mi.segments_meet(q_start * cfg.qc, q_start * cfg.qc + q_len, k_start * cfg.kc,
+                                k_start * cfg.kc + kv_len)
+    return True
 
 
 def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
