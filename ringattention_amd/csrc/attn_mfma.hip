@@ -1257,6 +1257,311 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
     }
 }
 
+// ------------------------------------------------------------------ dK / dV, wave-specialised
+// 8 wavefronts per workgroup, 128 keys: pair i = (wave i, wave i + 4) shares a SIMD and owns keys
+// 32 i .. 32 i + 31.  The producer (wave i) runs S = Q K^T and dP - delta = dO V^T - delta with its
+// K / V fragments in registers, turns them into P and dS (all of the vector work) and leaves both,
+// rounded to bf16, in LDS.  The consumer (wave i + 4) reads them back as B operands and runs
+// dV^T += dO^T P and dK^T += Q^T dS, with the 128 accumulator registers but no K / V fragments and no
+// vector work.  Unlike the separate dK and dV kernels, S, dP and the exponentials are computed once.
+//
+// Steps are blocks of 32 query rows, one barrier per step.  In step n the producer issues the matrix
+// products of block n + 1 between the vector work of block n, and the consumer accumulates block
+// n - 1.  Query tiles (64 rows of Q and dO plus row statistics) cycle through three LDS buffers:
+// tile t is read by the producer's products in steps 2t-1, 2t, by its vector work in 2t, 2t+1 and by
+// the consumer in 2t+1, 2t+2; tile t+2 is stored in step 2t+1 (its buffer held tile t-1) from
+// registers loaded two steps earlier.
+constexpr int WS_PSTR = 40;                 // P / dS row stride in elements (conflict-free 16-byte reads)
+constexpr int WS_PD = 32 * WS_PSTR;         // one 32 x 32 block
+constexpr int WS_TILE = KBM * TROW;
+
+template <bool HAS_SEG, bool HAS_BIAS>
+__global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[3 * WS_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Gs[3 * WS_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Ps[4][2][2][WS_PD];     // [pair][buffer][P | dS]
+  __shared__ __attribute__((aligned(16))) float st_m2[3][KBM];
+  __shared__ __attribute__((aligned(16))) float st_rden[3][KBM];
+  __shared__ __attribute__((aligned(16))) float st_lse2[3][KBM];
+  __shared__ __attribute__((aligned(16))) float st_delta[3][KBM];
+  __shared__ __attribute__((aligned(16))) int st_seg[3][KBM];
+
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
+  const int nkt = a.Skv / KBN;
+  int wg = blockIdx.x;
+  const int kt = wg % nkt;
+  wg /= nkt;
+  const int h = wg % a.H, b = wg / a.H;
+  const int k0 = kt * KBN;
+  const int krow = k0 + pair * 32 + lo;    // this lane's key row (local)
+
+  const int gk0 = (int)mv.global_k(k0);
+  const int gk = gk0 + pair * 32 + lo;
+  const int gq_base = (int)mv.global_q(0);
+  const int nqt = a.Sq / KBM;
+  int qt_first = nqt;
+  {
+    int nqc = a.Sq / mv.qc, lo_c = 0, hi_c = nqc;
+    while (lo_c < hi_c) {
+      int mid = (lo_c + hi_c) >> 1;
+      if (mv.run_prefix_keys(mid, a.Skv) > k0) hi_c = mid; else lo_c = mid + 1;
+    }
+    if (lo_c < nqc) qt_first = lo_c * (mv.qc / KBM);
+    if (mv.cbs > 0 && mv.skip_tiles && qt_first < nqt) {
+      long long need = (long long)(gk0 / mv.cbs) * mv.cbs - gq_base;
+      if (need > 0) {
+        int t = (int)(need / KBM);
+        if (t > qt_first) qt_first = t < nqt ? t : nqt;
+      }
+    }
+  }
+  int qt_end = nqt;
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && qt_first < nqt) {
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gk0, KBN, slo, shi);
+    seg_tile_hull(mv, b, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, slo, shi, hull2, tid, 512, t_first, t_last);
+    qt_end = qt_first + t_last;
+    qt_first += t_first;
+  }
+  if (qt_first >= qt_end) return;
+  const int ntq = qt_end - qt_first;       // query tiles of 64 rows
+  const int nblk = 2 * ntq;                // blocks of 32 rows
+
+  const float c = kLog2e / sqrtf((float)HD);
+  const float kMask2 = mv.mask_min;
+
+  // ---- staging of the Q / dO tiles through registers: producers bring Q, consumers dO and the statistics
+  const int srow = (tid & 255) >> 4, schunk = tid & 15;
+  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const uint16_t* sg = (role == 0 ? a.q : a.g) + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8 +
+                       (int64_t)(qt_first * KBM + srow) * a.q_ss;
+  uint16_t* sl = (role == 0 ? Qs : Gs) + s_off;
+  const int64_t row16 = 16 * a.q_ss;
+  uint4 sr0, sr1, sr2, sr3;
+  float r_m = 0.f, r_den = 1.f, r_delta = 0.f;
+  int r_seg = 0;
+#define RA_WS_LOAD(T)                                                                                   \
+  {                                                                                                     \
+    const int t_ = min((T), ntq - 1);                                                                   \
+    const uint16_t* p_ = sg + (int64_t)t_ * KBM * a.q_ss;                                               \
+    sr0 = *(const uint4*)(p_); sr1 = *(const uint4*)(p_ + row16);                                       \
+    sr2 = *(const uint4*)(p_ + 2 * row16); sr3 = *(const uint4*)(p_ + 3 * row16);                       \
+    if (tid >= 256 && tid < 256 + KBM) {                                                                \
+      const int row_ = (qt_first + t_) * KBM + tid - 256;                                               \
+      const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
+      r_m = a.mx[st_]; r_den = a.den[st_]; r_delta = a.delta[st_];                                      \
+      if (HAS_SEG) {                                                                                    \
+        int idx_ = clamp_seg_index(((long long)mv.q_start + row_ / mv.qc) * mv.qc, mv.qc, mv.seg_len, row_ % mv.qc); \
+        r_seg = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
+      }                                                                                                 \
+    }                                                                                                   \
+  }
+#define RA_WS_STORE(BUF)                                                                                \
+  {                                                                                                     \
+    uint16_t* d_ = sl + (BUF) * WS_TILE;                                                                \
+    *(uint4*)(d_) = sr0; *(uint4*)(d_ + 16 * TROW) = sr1;                                               \
+    *(uint4*)(d_ + 32 * TROW) = sr2; *(uint4*)(d_ + 48 * TROW) = sr3;                                   \
+    if (tid >= 256 && tid < 256 + KBM) {                                                                \
+      const float m2_ = max_to_log2(r_m, kMask2);                                                       \
+      st_m2[BUF][tid - 256] = m2_; st_rden[BUF][tid - 256] = 1.f / r_den;                               \
+      st_lse2[BUF][tid - 256] = m2_ + __log2f(r_den); st_delta[BUF][tid - 256] = r_delta;               \
+      if (HAS_SEG) st_seg[BUF][tid - 256] = r_seg;                                                      \
+    }                                                                                                   \
+  }
+  RA_WS_LOAD(0);
+  RA_WS_STORE(0);
+  RA_WS_LOAD(1);
+  RA_WS_STORE(1);
+  RA_WS_LOAD(2);
+  __syncthreads();
+
+  if (role == 0) {
+    // =========================== producer: S, dP -> P, dS
+    const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;       // masked iff gq < qlim
+    const int qlim_wave = mv.cbs > 0 ? ((gk0 + pair * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffff;
+    int seg_k = 0;
+    float bias2 = 0.f;
+    if (HAS_SEG) {
+      int idx = clamp_seg_index(((long long)mv.k_start + krow / mv.kc) * mv.kc, mv.kc, mv.seg_len, krow % mv.kc);
+      seg_k = mv.seg[(int64_t)b * mv.seg_sb + idx];
+    }
+    if (HAS_BIAS) {
+      float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)gk * mv.bias_sk];
+      if (mv.any_mask) bv = fminf(bv, 0.f);
+      bias2 = bv * kLog2e;
+    }
+    const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
+    bf16x8 kf[8], vf[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
+      vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
+    }
+    int n_off[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);
+    uint16_t* const pw = &Ps[pair][0][0][lo * WS_PSTR + hi * 4];
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+    // accumulators start at S = 0 and dP = -delta[row] (rows 8g + 4hi + e of block BLK of buffer BUF)
+#define RA_WS_INIT(SN, DPN, BUF, BLK)                                                                   \
+  _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                       \
+    const f32x4 d_ = *(const f32x4*)&st_delta[BUF][(BLK) * 32 + g * 8 + hi * 4];                        \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = 0.f; DPN[g * 4 + e] = -d_[e]; }     \
+  }
+    // two contraction steps (32 of the 128 head dimensions) of S and dP for block BLK of buffer BUF
+#define RA_WS_MATRIX(G, SN, DPN, BUF, BLK)                                                              \
+  _Pragma("unroll") for (int tt = 2 * (G); tt < 2 * (G) + 2; tt++) {                                    \
+    const bf16x8 qa_ = *(const bf16x8*)(Qs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[tt]);          \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa_, kf[tt], SN, 0, 0, 0);                             \
+    const bf16x8 ga_ = *(const bf16x8*)(Gs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[tt]);          \
+    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga_, vf[tt], DPN, 0, 0, 0);                           \
+  }
+    // eight rows (registers 4G .. 4G+3 of both halves) of P and dS for block BLK of buffer BUF
+#define RA_WS_VECTOR(G, SC, DPC, BUF, BLK, PB)                                                          \
+  {                                                                                                     \
+    const int qrow0 = (BLK) * 32 + (G) * 8 + hi * 4;                                                    \
+    bf16x4 p4, d4;                                                                                      \
+    if (!need_mask) {                                                                                   \
+      const f32x4 vl = *(const f32x4*)&st_lse2[BUF][qrow0];                                             \
+      _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                   \
+        const float p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -vl[e]));                                    \
+        p4[e] = (__bf16)p;                                                                              \
+        d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                                         \
+      }                                                                                                 \
+    } else {                                                                                            \
+      const f32x4 vm2 = *(const f32x4*)&st_m2[BUF][qrow0];                                              \
+      const f32x4 vrd = *(const f32x4*)&st_rden[BUF][qrow0];                                            \
+      _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                   \
+        float x = SC[(G) * 4 + e] * c;                                                                  \
+        if (HAS_BIAS) x += bias2;                                                                       \
+        bool masked = (gq_tile + qrow0 + e < qlim);                                                     \
+        if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                              \
+        x = masked ? kMask2 : x;                                                                        \
+        const float p = fast_exp2(x - vm2[e]) * vrd[e];                                  /* :226 */     \
+        p4[e] = (__bf16)p;                                                                              \
+        d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                          /* :229 */     \
+      }                                                                                                 \
+    }                                                                                                   \
+    *(bf16x4*)(pw + (PB) * 2 * WS_PD + (G) * 8) = p4;                                                   \
+    *(bf16x4*)(pw + (PB) * 2 * WS_PD + WS_PD + (G) * 8) = d4;                                           \
+  }
+#define RA_WS_PRODUCE(SC, DPC, SN, DPN, BUF, BLK, NBUF, NBLK, PB)                                       \
+  {                                                                                                     \
+    RA_WS_INIT(SN, DPN, NBUF, NBLK);                                                                    \
+    _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                     \
+      RA_WS_MATRIX(g, SN, DPN, NBUF, NBLK);                                                             \
+      RA_WS_VECTOR(g, SC, DPC, BUF, BLK, PB);                                                           \
+    }                                                                                                   \
+  }
+
+    f32x16 s_a, dp_a, s_b, dp_b;
+    RA_WS_INIT(s_a, dp_a, 0, 0);
+#pragma unroll
+    for (int g = 0; g < 4; g++) RA_WS_MATRIX(g, s_a, dp_a, 0, 0);
+
+    int cur = 0;
+    for (int t = 0; t < ntq; t++) {
+      const int nxt = cur == 2 ? 0 : cur + 1, prv = cur == 0 ? 2 : cur - 1;
+      const int gq_tile = gq_base + (qt_first + t) * KBM;
+      // step 2t: vector work of block 0 of tile t, products of block 1
+      {
+        const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave);
+        RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0);
+      }
+      __syncthreads();
+      // step 2t + 1: tile t + 2 goes to LDS, tile t + 3 is requested; vector work of block 1, products of
+      // block 0 of tile t + 1 (the last tile computes a block that is never used)
+      RA_WS_STORE(prv);
+      RA_WS_LOAD(t + 3);
+      {
+        const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile + 32 < qlim_wave);
+        RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1);
+      }
+      __syncthreads();
+      cur = nxt;
+    }
+    __syncthreads();      // step 2 ntq: the consumer's last block
+  } else {
+    // =========================== consumer: dV^T += dO^T P, dK^T += Q^T dS
+    f32x16 dkacc[4], dvacc[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+    // transpose reads with the natural contraction order: rows 8 hi + (i >> 2) (+4 for the second read)
+    int t_off[4][2];
+    {
+      const int i = lane & 15, rr = (i >> 2) + 8 * hi, c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
+#pragma unroll
+      for (int db = 0; db < 4; db++) {
+        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz(rr)) << 3) + half * 4;
+        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz(rr + 4)) << 3) + half * 4;
+      }
+    }
+    const uint16_t* const pr = &Ps[pair][0][0][lo * WS_PSTR + hi * 8];   // B operand: key column lo, 8 query rows
+
+    // block BLK of buffer BUF with the P / dS pair PB
+#define RA_WS_CONSUME(BUF, BLK, PB)                                                                     \
+  _Pragma("unroll") for (int tt = 0; tt < 2; tt++) {                                                    \
+    const bf16x8 pb_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + tt * 16);                               \
+    const bf16x8 db_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + WS_PD + tt * 16);                       \
+    const uint16_t* gtp = Gs + (BUF) * WS_TILE + ((BLK) * 32 + tt * 16) * TROW;                         \
+    const uint16_t* qtp = Qs + (BUF) * WS_TILE + ((BLK) * 32 + tt * 16) * TROW;                         \
+    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+      s16x4 g0 = lds_read_tr(gtp + t_off[db][0]);                                                       \
+      s16x4 g1 = lds_read_tr(gtp + t_off[db][1]);                                                       \
+      s16x8 gv = __builtin_shufflevector(g0, g1, 0, 1, 2, 3, 4, 5, 6, 7);                               \
+      dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, gv), pb_, dvacc[db], 0, 0, 0); \
+      s16x4 q0v = lds_read_tr(qtp + t_off[db][0]);                                                      \
+      s16x4 q1v = lds_read_tr(qtp + t_off[db][1]);                                                      \
+      s16x8 qv = __builtin_shufflevector(q0v, q1v, 0, 1, 2, 3, 4, 5, 6, 7);                             \
+      dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), db_, dkacc[db], 0, 0, 0); \
+    }                                                                                                   \
+  }
+    int cur = 0;
+    __syncthreads();      // step 0
+    for (int t = 0; t < ntq; t++) {
+      const int prv = cur == 0 ? 2 : cur - 1;
+      // step 2t + 1
+      RA_WS_STORE(prv);
+      RA_WS_LOAD(t + 3);
+      RA_WS_CONSUME(cur, 0, 0);
+      __syncthreads();
+      // step 2t + 2
+      RA_WS_CONSUME(cur, 1, 1);
+      __syncthreads();
+      cur = cur == 2 ? 0 : cur + 1;
+    }
+
+    // dk += acc / sqrt(D) (:231), dv += acc (:232); this pair owns its 32 key rows
+    const float rscale = 1.f / sqrtf((float)HD);
+    const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        float* pk = a.dk + ooff + db * 32 + g * 8;
+        float* pv = a.dv + ooff + db * 32 + g * 8;
+        f32x4 tk = *(const f32x4*)pk, tv = *(const f32x4*)pv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { tk[e] += dkacc[db][g * 4 + e] * rscale; tv[e] += dvacc[db][g * 4 + e]; }
+        *(f32x4*)pk = tk; *(f32x4*)pv = tv;
+      }
+  }
+#undef RA_WS_LOAD
+#undef RA_WS_STORE
+#undef RA_WS_INIT
+#undef RA_WS_MATRIX
+#undef RA_WS_VECTOR
+#undef RA_WS_PRODUCE
+#undef RA_WS_CONSUME
+}
+
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
@@ -1326,9 +1631,12 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
   dim3 gq((unsigned)nq), gk((unsigned)nk), block(256);
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool do_dkv = !(p->impl & RA_BWD_ONLY_DQ), do_dq = !(p->impl & RA_BWD_ONLY_DKV);
+  const bool use_ws = !getenv("RA_BWD_NO_WAVE_SPEC");
 #define RA_LAUNCH_BWD(SEG, BIAS)                                                         \
   do {                                                                                   \
-    if (do_dkv) {                                                                        \
+    if (do_dkv && use_ws) {                                                              \
+      attn_bwd_dkv_ws_kernel<SEG, BIAS><<<gk, dim3(512), 0, s>>>(a);                     \
+    } else if (do_dkv) {                                                                 \
       attn_bwd_dkv_mfma_kernel<SEG, BIAS, true, false><<<gk, block, 0, s>>>(a);          \
       attn_bwd_dkv_mfma_kernel<SEG, BIAS, false, true><<<gk, block, 0, s>>>(a);          \
     }                                                                                    \
