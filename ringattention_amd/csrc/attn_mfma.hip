@@ -1271,6 +1271,16 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
 // tile t is read by the producer's products in steps 2t-1, 2t, by its vector work in 2t, 2t+1 and by
 // the consumer in 2t+1, 2t+2; tile t+2 is stored in step 2t+1 (its buffer held tile t-1) from
 // registers loaded two steps earlier.
+// timing experiments only: each switch removes one part of the work (results are then wrong)
+#ifndef RA_ABL_WS_NOVEC
+#define RA_ABL_WS_NOVEC 0
+#endif
+#ifndef RA_ABL_WS_NOPMFMA
+#define RA_ABL_WS_NOPMFMA 0
+#endif
+#ifndef RA_ABL_WS_NOCONS
+#define RA_ABL_WS_NOCONS 0
+#endif
 constexpr int WS_PSTR = 40;                 // P / dS row stride in elements (conflict-free 16-byte reads)
 constexpr int WS_PD = 32 * WS_PSTR;         // one 32 x 32 block
 constexpr int WS_TILE = KBM * TROW;
@@ -1291,7 +1301,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
   const int nkt = a.Skv / KBN;
-  int wg = blockIdx.x;
+  // Workgroups go to the 8 XCDs round-robin, and each XCD has its own L2.  Give XCD x the contiguous
+  // range x of (batch, head, key block) triples: the workgroups resident on one XCD are then
+  // neighbouring key blocks of one head, which sweep nearly the same query rows at the same time, so a
+  // Q / dO tile is fetched into that L2 once instead of once per workgroup.
+  const int per_xcd = (a.B * a.H * nkt + 7) >> 3;
+  int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (wg >= a.B * a.H * nkt) return;
   const int kt = wg % nkt;
   wg /= nkt;
   const int h = wg % a.H, b = wg / a.H;
@@ -1413,36 +1429,28 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     const f32x4 d_ = *(const f32x4*)&st_delta[BUF][(BLK) * 32 + g * 8 + hi * 4];                        \
     _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = 0.f; DPN[g * 4 + e] = -d_[e]; }     \
   }
-    // two contraction steps (32 of the 128 head dimensions) of S and dP for block BLK of buffer BUF
-#define RA_WS_MATRIX(G, SN, DPN, BUF, BLK)                                                              \
-  _Pragma("unroll") for (int tt = 2 * (G); tt < 2 * (G) + 2; tt++) {                                    \
-    const bf16x8 qa_ = *(const bf16x8*)(Qs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[tt]);          \
-    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa_, kf[tt], SN, 0, 0, 0);                             \
-    const bf16x8 ga_ = *(const bf16x8*)(Gs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[tt]);          \
-    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga_, vf[tt], DPN, 0, 0, 0);                           \
+    // A operands of two contraction steps (32 of the 128 head dimensions) of block BLK of buffer BUF
+#define RA_WS_AREAD(G, QA, GA, BUF, BLK)                                                                \
+  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
+    QA[i] = *(const bf16x8*)(Qs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
+    GA[i] = *(const bf16x8*)(Gs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
   }
-    // eight rows (registers 4G .. 4G+3 of both halves) of P and dS for block BLK of buffer BUF
-#define RA_WS_VECTOR(G, SC, DPC, BUF, BLK, PB)                                                          \
+#define RA_WS_AMFMA(G, QA, GA, SN, DPN)                                                                 \
+  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
+    if (RA_ABL_WS_NOPMFMA) break;                                                                       \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(QA[i], kf[2 * (G) + i], SN, 0, 0, 0);                  \
+    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(GA[i], vf[2 * (G) + i], DPN, 0, 0, 0);                \
+  }
+    // eight rows (registers 4G .. 4G+3 of both halves) of P and dS, no masking: VL = lse2 of the rows
+#define RA_WS_VECTOR_PLAIN(G, SC, DPC, VL, PB)                                                          \
   {                                                                                                     \
-    const int qrow0 = (BLK) * 32 + (G) * 8 + hi * 4;                                                    \
     bf16x4 p4, d4;                                                                                      \
-    if (!need_mask) {                                                                                   \
-      const f32x4 vl = *(const f32x4*)&st_lse2[BUF][qrow0];                                             \
-      _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                   \
-        const float p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -vl[e]));                                    \
-        p4[e] = (__bf16)p;                                                                              \
-        d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                                         \
-      }                                                                                                 \
-    } else {                                                                                            \
-      const f32x4 vm2 = *(const f32x4*)&st_m2[BUF][qrow0];                                              \
-      const f32x4 vrd = *(const f32x4*)&st_rden[BUF][qrow0];                                            \
-      _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                   \
-        float x = SC[(G) * 4 + e] * c;                                                                  \
-        if (HAS_BIAS) x += bias2;                                                                       \
-        bool masked = (gq_tile + qrow0 + e < qlim);                                                     \
-        if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                              \
-        x = masked ? kMask2 : x;                                                                        \
-        const float p = fast_exp2(x - vm2[e]) * vrd[e];                                  /* :226 */     \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
+      if (RA_ABL_WS_NOVEC) {                                                                            \
+        p4[e] = __builtin_bit_cast(__bf16, (uint16_t)(__float_as_uint(SC[(G) * 4 + e]) >> 16));         \
+        d4[e] = __builtin_bit_cast(__bf16, (uint16_t)(__float_as_uint(DPC[(G) * 4 + e]) >> 16));        \
+      } else {                                                                                          \
+        const float p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -VL[e]));                     /* :226 */     \
         p4[e] = (__bf16)p;                                                                              \
         d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                          /* :229 */     \
       }                                                                                                 \
@@ -1450,37 +1458,76 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     *(bf16x4*)(pw + (PB) * 2 * WS_PD + (G) * 8) = p4;                                                   \
     *(bf16x4*)(pw + (PB) * 2 * WS_PD + WS_PD + (G) * 8) = d4;                                           \
   }
-#define RA_WS_PRODUCE(SC, DPC, SN, DPN, BUF, BLK, NBUF, NBLK, PB)                                       \
+#define RA_WS_VECTOR_MASKED(G, SC, DPC, BUF, BLK, PB)                                                   \
   {                                                                                                     \
+    const int qrow0 = (BLK) * 32 + (G) * 8 + hi * 4;                                                    \
+    bf16x4 p4, d4;                                                                                      \
+    const f32x4 vm2 = *(const f32x4*)&st_m2[BUF][qrow0];                                                \
+    const f32x4 vrd = *(const f32x4*)&st_rden[BUF][qrow0];                                              \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
+      float x = SC[(G) * 4 + e] * c;                                                                    \
+      if (HAS_BIAS) x += bias2;                                                                         \
+      bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
+      if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
+      x = masked ? kMask2 : x;                                                                          \
+      const float p = fast_exp2(x - vm2[e]) * vrd[e];                                    /* :226 */     \
+      p4[e] = (__bf16)p;                                                                                \
+      d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                            /* :229 */     \
+    }                                                                                                   \
+    *(bf16x4*)(pw + (PB) * 2 * WS_PD + (G) * 8) = p4;                                                   \
+    *(bf16x4*)(pw + (PB) * 2 * WS_PD + WS_PD + (G) * 8) = d4;                                           \
+  }
+    // one step: vector work of block BLK of buffer BUF (accumulators SC, DPC) in four groups of eight
+    // rows, each preceded by a quarter of the products of block NBLK of buffer NBUF (into SN, DPN);
+    // the operands of a group are requested from LDS one group ahead
+#define RA_WS_PRODUCE(SC, DPC, SN, DPN, BUF, BLK, NBUF, NBLK, PB, MASKED)                               \
+  {                                                                                                     \
+    bf16x8 qa_[2][2], ga_[2][2];                                                                        \
+    f32x4 vl_[2];                                                                                       \
+    RA_WS_AREAD(0, qa_[0], ga_[0], NBUF, NBLK);                                                         \
+    if (!(MASKED)) vl_[0] = *(const f32x4*)&st_lse2[BUF][(BLK) * 32 + hi * 4];                          \
     RA_WS_INIT(SN, DPN, NBUF, NBLK);                                                                    \
     _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                     \
-      RA_WS_MATRIX(g, SN, DPN, NBUF, NBLK);                                                             \
-      RA_WS_VECTOR(g, SC, DPC, BUF, BLK, PB);                                                           \
+      if (g < 3) {                                                                                      \
+        RA_WS_AREAD(g + 1, qa_[(g + 1) & 1], ga_[(g + 1) & 1], NBUF, NBLK);                             \
+        if (!(MASKED)) vl_[(g + 1) & 1] = *(const f32x4*)&st_lse2[BUF][(BLK) * 32 + (g + 1) * 8 + hi * 4]; \
+      }                                                                                                 \
+      __builtin_amdgcn_sched_barrier(0);                                                                \
+      RA_WS_AMFMA(g, qa_[g & 1], ga_[g & 1], SN, DPN);                                                  \
+      if (MASKED) RA_WS_VECTOR_MASKED(g, SC, DPC, BUF, BLK, PB)                                         \
+      else RA_WS_VECTOR_PLAIN(g, SC, DPC, vl_[g & 1], PB)                                               \
+      __builtin_amdgcn_sched_barrier(0);                                                                \
     }                                                                                                   \
   }
 
     f32x16 s_a, dp_a, s_b, dp_b;
     RA_WS_INIT(s_a, dp_a, 0, 0);
 #pragma unroll
-    for (int g = 0; g < 4; g++) RA_WS_MATRIX(g, s_a, dp_a, 0, 0);
+    for (int g = 0; g < 4; g++) {
+      bf16x8 qa_[2], ga_[2];
+      RA_WS_AREAD(g, qa_, ga_, 0, 0);
+      RA_WS_AMFMA(g, qa_, ga_, s_a, dp_a);
+    }
 
     int cur = 0;
     for (int t = 0; t < ntq; t++) {
       const int nxt = cur == 2 ? 0 : cur + 1, prv = cur == 0 ? 2 : cur - 1;
       const int gq_tile = gq_base + (qt_first + t) * KBM;
       // step 2t: vector work of block 0 of tile t, products of block 1
-      {
-        const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave);
-        RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0);
+      if (HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave)) {
+        RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, true);
+      } else {
+        RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, false);
       }
       __syncthreads();
       // step 2t + 1: tile t + 2 goes to LDS, tile t + 3 is requested; vector work of block 1, products of
       // block 0 of tile t + 1 (the last tile computes a block that is never used)
       RA_WS_STORE(prv);
       RA_WS_LOAD(t + 3);
-      {
-        const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile + 32 < qlim_wave);
-        RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1);
+      if (HAS_SEG || HAS_BIAS || (gq_tile + 32 < qlim_wave)) {
+        RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, true);
+      } else {
+        RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, false);
       }
       __syncthreads();
       cur = nxt;
@@ -1505,37 +1552,60 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     }
     const uint16_t* const pr = &Ps[pair][0][0][lo * WS_PSTR + hi * 8];   // B operand: key column lo, 8 query rows
 
-    // block BLK of buffer BUF with the P / dS pair PB
-#define RA_WS_CONSUME(BUF, BLK, PB)                                                                     \
-  _Pragma("unroll") for (int tt = 0; tt < 2; tt++) {                                                    \
-    const bf16x8 pb_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + tt * 16);                               \
-    const bf16x8 db_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + WS_PD + tt * 16);                       \
-    const uint16_t* gtp = Gs + (BUF) * WS_TILE + ((BLK) * 32 + tt * 16) * TROW;                         \
-    const uint16_t* qtp = Qs + (BUF) * WS_TILE + ((BLK) * 32 + tt * 16) * TROW;                         \
+    // The 16 products of a block run as four groups of four: dV with query rows 0..15 of the block, dK
+    // with the same rows, then both with rows 16..31.  The transposed A operands of a group are read
+    // one group ahead, those of the first group before the barrier that publishes the block's P / dS.
+#define RA_WS_CREAD(K, F, BUF, BLK)                                                                     \
+  {                                                                                                     \
+    const uint16_t* tp_ = (((K) & 1) ? Qs : Gs) + (BUF) * WS_TILE + ((BLK) * 32 + ((K) >> 1) * 16) * TROW; \
     _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
-      s16x4 g0 = lds_read_tr(gtp + t_off[db][0]);                                                       \
-      s16x4 g1 = lds_read_tr(gtp + t_off[db][1]);                                                       \
-      s16x8 gv = __builtin_shufflevector(g0, g1, 0, 1, 2, 3, 4, 5, 6, 7);                               \
-      dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, gv), pb_, dvacc[db], 0, 0, 0); \
-      s16x4 q0v = lds_read_tr(qtp + t_off[db][0]);                                                      \
-      s16x4 q1v = lds_read_tr(qtp + t_off[db][1]);                                                      \
-      s16x8 qv = __builtin_shufflevector(q0v, q1v, 0, 1, 2, 3, 4, 5, 6, 7);                             \
-      dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), db_, dkacc[db], 0, 0, 0); \
+      const s16x4 x0_ = lds_read_tr(tp_ + t_off[db][0]);                                                \
+      const s16x4 x1_ = lds_read_tr(tp_ + t_off[db][1]);                                                \
+      F[db] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0_, x1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
   }
+#define RA_WS_CMFMA(K, F, BOP)                                                                          \
+  _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                    \
+    if (RA_ABL_WS_NOCONS) break;                                                                        \
+    if ((K) & 1) dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, dkacc[db], 0, 0, 0);   \
+    else dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, dvacc[db], 0, 0, 0);           \
+  }
+    // block BLK of buffer BUF with the P / dS pair PB; fa holds group 0 on entry and, on exit, group 0
+    // of block NBLK of buffer NBUF
+#define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
+  {                                                                                                     \
+    const bf16x8 p0_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD);                                         \
+    const bf16x8 p1_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + 16);                                    \
+    const bf16x8 d0_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + WS_PD);                                 \
+    const bf16x8 d1_ = *(const bf16x8*)(pr + (PB) * 2 * WS_PD + WS_PD + 16);                            \
+    RA_WS_CREAD(1, fb, BUF, BLK);                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(0, fa, p0_);                                                                            \
+    RA_WS_CREAD(2, fa, BUF, BLK);                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(1, fb, d0_);                                                                            \
+    RA_WS_CREAD(3, fb, BUF, BLK);                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(2, fa, p1_);                                                                            \
+    RA_WS_CREAD(0, fa, NBUF, NBLK);                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(3, fb, d1_);                                                                            \
+  }
+    bf16x8 fa[4], fb[4];
     int cur = 0;
+    RA_WS_CREAD(0, fa, 0, 0);
     __syncthreads();      // step 0
     for (int t = 0; t < ntq; t++) {
-      const int prv = cur == 0 ? 2 : cur - 1;
+      const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;
       // step 2t + 1
       RA_WS_STORE(prv);
       RA_WS_LOAD(t + 3);
-      RA_WS_CONSUME(cur, 0, 0);
+      RA_WS_CONSUME(cur, 0, 0, cur, 1);
       __syncthreads();
       // step 2t + 2
-      RA_WS_CONSUME(cur, 1, 1);
+      RA_WS_CONSUME(cur, 1, 1, nxt, 0);
       __syncthreads();
-      cur = cur == 2 ? 0 : cur + 1;
+      cur = nxt;
     }
 
     // dk += acc / sqrt(D) (:231), dv += acc (:232); this pair owns its 32 key rows
@@ -1556,8 +1626,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #undef RA_WS_LOAD
 #undef RA_WS_STORE
 #undef RA_WS_INIT
-#undef RA_WS_MATRIX
-#undef RA_WS_VECTOR
+#undef RA_WS_AREAD
+#undef RA_WS_AMFMA
+#undef RA_WS_VECTOR_PLAIN
+#undef RA_WS_VECTOR_MASKED
+#undef RA_WS_CREAD
+#undef RA_WS_CMFMA
 #undef RA_WS_PRODUCE
 #undef RA_WS_CONSUME
 }
@@ -1635,7 +1709,7 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
 #define RA_LAUNCH_BWD(SEG, BIAS)                                                         \
   do {                                                                                   \
     if (do_dkv && use_ws) {                                                              \
-      attn_bwd_dkv_ws_kernel<SEG, BIAS><<<gk, dim3(512), 0, s>>>(a);                     \
+      attn_bwd_dkv_ws_kernel<SEG, BIAS><<<dim3((gk.x + 7) / 8 * 8), dim3(512), 0, s>>>(a); \
     } else if (do_dkv) {                                                                 \
       attn_bwd_dkv_mfma_kernel<SEG, BIAS, true, false><<<gk, block, 0, s>>>(a);          \
       attn_bwd_dkv_mfma_kernel<SEG, BIAS, false, true><<<gk, block, 0, s>>>(a);          \
