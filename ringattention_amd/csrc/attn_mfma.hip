@@ -498,8 +498,14 @@ constexpr int PBM = 256;
 #ifdef RA_TRACE
 __device__ long long g_trace[8][4096];
 #define RA_TRACE_MARK() { if (trace_on && lane == 0 && trace_n < 4096) g_trace[wave][trace_n++] = __builtin_readcyclecounter(); }
+#ifdef RA_TRACE2
+#define RA_TRACE_MARK2() { __builtin_amdgcn_sched_barrier(0); RA_TRACE_MARK(); __builtin_amdgcn_sched_barrier(0); }
+#else
+#define RA_TRACE_MARK2() {}
+#endif
 #else
 #define RA_TRACE_MARK() {}
+#define RA_TRACE_MARK2() {}
 #endif
 constexpr int PP_DEPTH = 1;       // LDS fragment prefetch distance of the matrix phase, in steps of 4 MFMAs
 constexpr bool PP_PRIO = false;  // raise the wave priority during the matrix phase
@@ -1398,7 +1404,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   if (role == 0) {
     // =========================== producer: S, dP -> P, dS
     const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;       // masked iff gq < qlim
-    const int qlim_wave = mv.cbs > 0 ? ((gk0 + pair * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffff;
+    const int qlim_wave = __builtin_amdgcn_readfirstlane(mv.cbs > 0 ? ((gk0 + pair * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffff);
     int seg_k = 0;
     float bias2 = 0.f;
     if (HAS_SEG) {
@@ -1636,6 +1642,357 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #undef RA_WS_CONSUME
 }
 
+// ------------------------------------------------------------------ dQ, wave-specialised
+// The mirror image of the dK / dV kernel above: 128 query rows per workgroup, pair i owns rows
+// 32 i .. 32 i + 31 and keeps their Q and dO fragments in the producer's registers; K / V tiles of 64
+// keys stream through three LDS buffers.  Per block of 32 keys the producer runs S^T = K Q^T and
+// dP^T - delta = V dO^T - delta, forms dS^T and leaves it in LDS; the consumer accumulates
+// dQ^T += K^T dS^T one block behind.  The row statistics belong to the lane's query column and stay in
+// registers.
+#ifndef WS_DQ_VALU_PER_MFMA
+#define WS_DQ_VALU_PER_MFMA 5
+#endif
+template <bool HAS_SEG, bool HAS_BIAS>
+__global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[3 * WS_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[3 * WS_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Ds[4][2][WS_PD];        // [pair][buffer] dS^T as [q][key]
+  __shared__ int seg_ks[3][FBN];
+  __shared__ float bias_ks[3][FBN];
+
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
+  const int nqt = a.Sq / FBM;
+  // XCD x takes the contiguous range x of (batch, head, query tile) triples: the workgroups resident on
+  // one XCD then stream the same K / V tiles of one head through that XCD's L2 at the same time
+  const int per_xcd = (a.B * a.H * nqt + 7) >> 3;
+  int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (wg >= a.B * a.H * nqt) return;
+  const int qt = nqt - 1 - (wg % nqt);     // latest query tiles (most keys under causal) first
+  wg /= nqt;
+  const int h = wg % a.H, b = wg / a.H;
+  const int q0 = qt * FBM;
+  const int qrow = q0 + pair * 32 + lo;
+
+  const int qi = q0 / mv.qc;
+  int kend = mv.run_prefix_keys(qi, a.Skv);
+  const int gq0 = (int)mv.global_q(q0);
+  const int gk0_shard = (int)mv.global_k(0);
+  if (mv.cbs > 0 && mv.skip_tiles) {
+    long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
+    long long n = lim - gk0_shard;
+    if (n < kend) kend = n > 0 ? (int)n : 0;
+  }
+  int ntiles = (kend + FBN - 1) / FBN;
+  int k_base = 0;
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gq0, FBM, slo, shi);
+    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
+    k_base = t_first * FBN;
+    ntiles = t_last - t_first;
+  }
+  if (ntiles == 0) return;     // nothing to add to dq
+  const int gk0 = gk0_shard + k_base;
+  const float c = kLog2e / sqrtf((float)HD);
+  const float kMask2 = mv.mask_min;
+
+  // ---- staging of the K / V tiles through registers, by the consumer waves (which have registers and
+  // issue slots to spare): tile t + 2 is stored in step 2t + 1, two steps after it was requested
+  const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
+  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const int64_t sg_off = (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
+  const uint16_t* sgk = a.k + sg_off;
+  const uint16_t* sgv = a.v + sg_off;
+  const int64_t row16 = 16 * a.kv_ss;
+  uint4 sk0, sk1, sk2, sk3, sv0, sv1, sv2, sv3;
+  int seg_r = 0;
+  float bias_r = 0.f;
+  // K half (with the key info) and V half of a tile are staged separately so that the requests and the
+  // LDS writes of a tile spread over two steps
+#define RA_WS_LOAD_K(T)                                                                                 \
+  {                                                                                                     \
+    const int t_ = min((T), ntiles - 1);                                                                \
+    const uint16_t* pk_ = sgk + (int64_t)t_ * FBN * a.kv_ss;                                            \
+    sk0 = *(const uint4*)(pk_); sk1 = *(const uint4*)(pk_ + row16);                                     \
+    sk2 = *(const uint4*)(pk_ + 2 * row16); sk3 = *(const uint4*)(pk_ + 3 * row16);                     \
+    if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
+      const int kj_ = k_base + t_ * FBN + stid;                                                         \
+      if (HAS_SEG) {                                                                                    \
+        int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
+      }                                                                                                 \
+      if (HAS_BIAS) {                                                                                   \
+        float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
+        if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
+        bias_r = bv_ * kLog2e;                                                                          \
+      }                                                                                                 \
+    }                                                                                                   \
+  }
+#define RA_WS_LOAD_V(T)                                                                                 \
+  {                                                                                                     \
+    const int t_ = min((T), ntiles - 1);                                                                \
+    const uint16_t* pv_ = sgv + (int64_t)t_ * FBN * a.kv_ss;                                            \
+    sv0 = *(const uint4*)(pv_); sv1 = *(const uint4*)(pv_ + row16);                                     \
+    sv2 = *(const uint4*)(pv_ + 2 * row16); sv3 = *(const uint4*)(pv_ + 3 * row16);                     \
+  }
+#define RA_WS_STORE_K(BUF)                                                                              \
+  {                                                                                                     \
+    uint16_t* dk_ = Ks + (BUF) * WS_TILE + s_off;                                                       \
+    *(uint4*)(dk_) = sk0; *(uint4*)(dk_ + 16 * TROW) = sk1;                                             \
+    *(uint4*)(dk_ + 32 * TROW) = sk2; *(uint4*)(dk_ + 48 * TROW) = sk3;                                 \
+    if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
+      if (HAS_SEG) seg_ks[BUF][stid] = seg_r;                                                           \
+      if (HAS_BIAS) bias_ks[BUF][stid] = bias_r;                                                        \
+    }                                                                                                   \
+  }
+#define RA_WS_STORE_V(BUF)                                                                              \
+  {                                                                                                     \
+    uint16_t* dv_ = Vs + (BUF) * WS_TILE + s_off;                                                       \
+    *(uint4*)(dv_) = sv0; *(uint4*)(dv_ + 16 * TROW) = sv1;                                             \
+    *(uint4*)(dv_ + 32 * TROW) = sv2; *(uint4*)(dv_ + 48 * TROW) = sv3;                                 \
+  }
+#ifdef RA_TRACE
+  const bool trace_on = blockIdx.x == 0;
+  int trace_n = 0;
+#endif
+  if (role == 1) {
+    RA_WS_LOAD_K(0); RA_WS_LOAD_V(0);
+    RA_WS_STORE_K(0); RA_WS_STORE_V(0);
+    RA_WS_LOAD_K(1); RA_WS_LOAD_V(1);
+    RA_WS_STORE_K(1); RA_WS_STORE_V(1);
+    RA_WS_LOAD_K(2); RA_WS_LOAD_V(2);
+  }
+  __syncthreads();
+
+  if (role == 0) {
+    // =========================== producer: S^T, dP^T -> dS^T
+    const int gq = gq0 + pair * 32 + lo;
+    const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
+    const int klim_wave = __builtin_amdgcn_readfirstlane(
+        mv.cbs > 0 ? (int)min((long long)((gq0 + pair * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff);
+    int seg_q = 0;
+    if (HAS_SEG) {
+      int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
+      seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
+    }
+    const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
+    bf16x8 qf[8], gf[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+      qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
+      gf[t] = *(const bf16x8*)(a.g + qoff + t * 16);
+    }
+    const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+    const float den = a.den[st];
+    const float m2 = max_to_log2(a.mx[st], kMask2);
+    const float rden = 1.f / den;
+    const float lse2 = m2 + __log2f(den);
+    const float ndelta = -a.delta[st];
+    int n_off[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);
+    uint16_t* const dw = &Ds[pair][0][lo * WS_PSTR + hi * 4];
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+#define RA_WS_INIT(SN, DPN)                                                                             \
+  _Pragma("unroll") for (int r = 0; r < 16; r++) { SN[r] = 0.f; DPN[r] = ndelta; }
+#define RA_WS_AREAD(G, KA, VA, BUF, BLK)                                                                \
+  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
+    KA[i] = *(const bf16x8*)(Ks + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
+    VA[i] = *(const bf16x8*)(Vs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
+  }
+#define RA_WS_AMFMA(G, KA, VA, SN, DPN)                                                                 \
+  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
+    if (RA_ABL_WS_NOPMFMA) break;                                                                       \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[2 * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T */ \
+    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(VA[i], gf[2 * (G) + i], DPN, 0, 0, 0); /* dP^T = V dO^T */ \
+  }
+    // eight keys (registers 4G .. 4G+3 of both halves) of dS^T
+#define RA_WS_VECTOR(G, SC, DPC, BUF, BLK, PB, MASKED)                                                  \
+  {                                                                                                     \
+    bf16x4 d4;                                                                                          \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
+      float p;                                                                                          \
+      if (RA_ABL_WS_NOVEC) {                                                                            \
+        d4[e] = __builtin_bit_cast(__bf16, (uint16_t)(__float_as_uint(SC[(G) * 4 + e] + DPC[(G) * 4 + e]) >> 16)); \
+        continue;                                                                                       \
+      }                                                                                                 \
+      if (!(MASKED)) {                                                                                  \
+        p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -lse2));                                                 \
+      } else {                                                                                          \
+        const int kr_ = (BLK) * 32 + (G) * 8 + hi * 4 + e;                                              \
+        float x = SC[(G) * 4 + e] * c;                                                                  \
+        if (HAS_BIAS) x += bias_ks[BUF][kr_];                                                           \
+        bool masked = (gk_tile + kr_ >= klim);                                                          \
+        if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
+        x = masked ? kMask2 : x;                                                                        \
+        p = fast_exp2(x - m2) * rden;                                                    /* :226 */     \
+      }                                                                                                 \
+      d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                            /* :229 */     \
+    }                                                                                                   \
+    *(bf16x4*)(dw + (PB) * WS_PD + (G) * 8) = d4;                                                       \
+  }
+    // one step: vector work of block BLK of buffer BUF (accumulators SC, DPC) in four groups of eight
+    // keys, each next to a quarter of the products of block NBLK of buffer NBUF (into SN, DPN).  The
+    // K / V operands of a quarter are requested from LDS three quarters ahead - the last three of a step
+    // request the first three quarters of the following step's block NNBLK of buffer NNBUF - which
+    // covers the LDS latency under load.
+#define RA_WS_PRODUCE(SC, DPC, SN, DPN, BUF, BLK, NBUF, NBLK, NNBUF, NNBLK, PB, MASKED)                 \
+  {                                                                                                     \
+    RA_WS_INIT(SN, DPN);                                                                                \
+    _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                     \
+      if (g == 0) { RA_WS_AREAD(3, ka[3], va[3], NBUF, NBLK); }                                         \
+      else { RA_WS_AREAD(g - 1, ka[g - 1], va[g - 1], NNBUF, NNBLK); }                                  \
+      RA_WS_AMFMA(g, ka[g], va[g], SN, DPN);                                                            \
+      RA_WS_VECTOR(g, SC, DPC, BUF, BLK, PB, MASKED);                                                   \
+      /* issue order: the LDS reads, then each product followed by a share of the vector work */        \
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);                                                \
+      _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                                \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                              \
+        __builtin_amdgcn_sched_group_barrier(0x002, WS_DQ_VALU_PER_MFMA, 0);                            \
+      }                                                                                                 \
+      __builtin_amdgcn_sched_barrier(0);                                                                \
+    }                                                                                                   \
+  }
+
+    f32x16 s_a, dp_a, s_b, dp_b;
+    bf16x8 ka[4][2], va[4][2];
+    RA_WS_INIT(s_a, dp_a);
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      RA_WS_AREAD(g, ka[0], va[0], 0, 0);
+      RA_WS_AMFMA(g, ka[0], va[0], s_a, dp_a);
+    }
+#pragma unroll
+    for (int g = 0; g < 3; g++) RA_WS_AREAD(g, ka[g], va[g], 0, 1);
+
+    // Under a causal mask the tiles that need no masking come first: one loop for them, one for the rest
+    // (which also takes every tile when segment ids or a bias are present).
+    int t_plain = 0;
+    if (!(HAS_SEG || HAS_BIAS)) t_plain = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
+    int cur = 0;
+#define RA_WS_TILE(MASKED)                                                                              \
+  {                                                                                                     \
+    const int nxt = cur == 2 ? 0 : cur + 1;                                                             \
+    const int gk_tile = gk0 + t * FBN;                                                                  \
+    (void)gk_tile;                                                                                      \
+    /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
+    RA_TRACE_MARK();                                                                                    \
+    RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, nxt, 0, 0, MASKED);                             \
+    RA_TRACE_MARK();                                                                                    \
+    __syncthreads();                                                                                    \
+    /* step 2t + 1: vector work of block 1, products of block 0 of tile t + 1 (the last tile computes  \
+       a block that is never used) */                                                                   \
+    RA_TRACE_MARK();                                                                                    \
+    RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, nxt, 1, 1, MASKED);                             \
+    RA_TRACE_MARK();                                                                                    \
+    __syncthreads();                                                                                    \
+    cur = nxt;                                                                                          \
+  }
+    int t = 0;
+    for (; t < t_plain; t++) RA_WS_TILE(false);
+    for (; t < ntiles; t++) RA_WS_TILE(true);
+#undef RA_WS_TILE
+    __syncthreads();      // step 2 ntiles: the consumer's last block
+#undef RA_WS_INIT
+#undef RA_WS_AREAD
+#undef RA_WS_AMFMA
+#undef RA_WS_VECTOR
+#undef RA_WS_PRODUCE
+  } else {
+    // =========================== consumer: dQ^T += K^T dS^T
+    f32x16 acc[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+    int t_off[4][2];
+    {
+      const int i = lane & 15, rr = (i >> 2) + 8 * hi, c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
+#pragma unroll
+      for (int db = 0; db < 4; db++) {
+        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz(rr)) << 3) + half * 4;
+        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz(rr + 4)) << 3) + half * 4;
+      }
+    }
+    const uint16_t* const dr = &Ds[pair][0][lo * WS_PSTR + hi * 8];   // B operand: query column lo, 8 keys
+
+    // keys 16 K .. 16 K + 15 of block BLK of buffer BUF, transposed
+#define RA_WS_CREAD(K, F, BUF, BLK)                                                                     \
+  {                                                                                                     \
+    const uint16_t* tp_ = Ks + (BUF) * WS_TILE + ((BLK) * 32 + (K) * 16) * TROW;                        \
+    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+      const s16x4 x0_ = lds_read_tr(tp_ + t_off[db][0]);                                                \
+      const s16x4 x1_ = lds_read_tr(tp_ + t_off[db][1]);                                                \
+      F[db] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0_, x1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
+    }                                                                                                   \
+  }
+#define RA_WS_CMFMA(F, BOP)                                                                             \
+  _Pragma("unroll") for (int db = 0; db < 4; db++)                                                      \
+    if (!RA_ABL_WS_NOCONS) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
+    // fa holds the first 16 keys of the block on entry and, on exit, those of block NBLK of buffer NBUF
+#define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
+  {                                                                                                     \
+    const bf16x8 d0_ = *(const bf16x8*)(dr + (PB) * WS_PD);                                             \
+    const bf16x8 d1_ = *(const bf16x8*)(dr + (PB) * WS_PD + 16);                                        \
+    RA_WS_CREAD(1, fb, BUF, BLK);                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(fa, d0_);                                                                               \
+    RA_WS_CREAD(0, fa, NBUF, NBLK);                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(fb, d1_);                                                                               \
+  }
+    bf16x8 fa[4], fb[4];
+    int cur = 0;
+    RA_WS_CREAD(0, fa, 0, 0);
+    __syncthreads();      // step 0
+    for (int t = 0; t < ntiles; t++) {
+      const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;
+      // tile t + 2 goes to the buffer that held tile t - 1 (K in step 2t + 1, V in step 2t + 2) and
+      // tile t + 3 is requested
+      RA_TRACE_MARK();
+      RA_WS_STORE_K(prv);
+      RA_TRACE_MARK2();
+      RA_WS_LOAD_K(t + 3);
+      RA_TRACE_MARK2();
+      RA_WS_CONSUME(cur, 0, 0, cur, 1);
+      RA_TRACE_MARK();
+      __syncthreads();
+      RA_TRACE_MARK();
+      RA_WS_STORE_V(prv);
+      RA_WS_LOAD_V(t + 3);
+      RA_WS_CONSUME(cur, 1, 1, nxt, 0);
+      RA_TRACE_MARK();
+      __syncthreads();
+      cur = nxt;
+    }
+#undef RA_WS_CREAD
+#undef RA_WS_CMFMA
+#undef RA_WS_CONSUME
+
+    // dq += acc / sqrt(D)   (:230)
+    const float rscale = 1.f / sqrtf((float)HD);
+    float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4 t = *(const f32x4*)(dqp + db * 32 + g * 8);
+#pragma unroll
+        for (int e = 0; e < 4; e++) t[e] += acc[db][g * 4 + e] * rscale;
+        *(f32x4*)(dqp + db * 32 + g * 8) = t;
+      }
+  }
+#undef RA_WS_LOAD_K
+#undef RA_WS_LOAD_V
+#undef RA_WS_STORE_K
+#undef RA_WS_STORE_V
+}
+
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
@@ -1714,7 +2071,11 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
       attn_bwd_dkv_mfma_kernel<SEG, BIAS, true, false><<<gk, block, 0, s>>>(a);          \
       attn_bwd_dkv_mfma_kernel<SEG, BIAS, false, true><<<gk, block, 0, s>>>(a);          \
     }                                                                                    \
-    if (do_dq) attn_bwd_dq_mfma_kernel<SEG, BIAS><<<gq, block, 0, s>>>(a);               \
+    if (do_dq && use_ws) {                                                               \
+      attn_bwd_dq_ws_kernel<SEG, BIAS><<<dim3((gq.x + 7) / 8 * 8), dim3(512), 0, s>>>(a); \
+    } else if (do_dq) {                                                                  \
+      attn_bwd_dq_mfma_kernel<SEG, BIAS><<<gq, block, 0, s>>>(a);                        \
+    }                                                                                    \
   } while (0)
   if (seg && bias) RA_LAUNCH_BWD(true, true);
   else if (seg) RA_LAUNCH_BWD(true, false);
