@@ -124,7 +124,7 @@ def bench_attention(args, ring):
             qd, kd, vd = q.detach(), k.detach(), v.detach()
             fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (num, den, mx), 0, 0, None, None, 1, 512, 512,
                                                       _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True)
-            kern["attn_fwd_mfma_kernel"] = (_event_ms(fwd, 5), flops_fwd)
+            kern["attn_fwd_pp_kernel"] = (_event_ms(fwd, 5), flops_fwd)
             out = torch.empty_like(qd)
             rh._finalize(num, den, out)
             delta = rh._bwd_delta(do, out)
@@ -134,7 +134,7 @@ def bench_attention(args, ring):
                 cfg1 = rh._Config(dict(kw, bwd_only=which))
                 bw = lambda: rh._blockwise_attention_bwd(qd, kd, vd, do, (dq, dk, dv, out, den, mx), 0, 0, None, None,
                                                          1, 512, 512, _mask_inputs=mi, _cfg=cfg1, _delta=delta)
-                kern["attn_bwd_%s_mfma_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
+                kern["attn_bwd_%s_ws_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
         dom = max(kern, key=lambda n_: kern[n_][0])
         dms, dfl = kern[dom]
         ach = dfl / (dms * 1e-3) / 1e12
