@@ -58,6 +58,57 @@ class _SwiGLUFn(torch.autograd.Function):
         return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype)
 
 
+class _BlockwiseSwiGLUFn(torch.autograd.Function):
+    """The whole scan of blockwise_feedforward over a SwiGLU MLP as one autograd node: chunk after chunk
+    through the same scratch buffers; in the backward pass the weight gradients of all chunks
+    accumulate in fp32 inside the GEMM epilogue and are rounded to the weights' dtype once."""
+
+    @staticmethod
+    def forward(ctx, x, w1, w2, w3, chunk_tokens):
+        T, d = x.shape
+        f = w1.shape[1]
+        bf = dict(dtype=torch.bfloat16, device=x.device)
+        a, b, h = (torch.empty((chunk_tokens, f), **bf) for _ in range(3))
+        y = torch.empty((T, d), **bf)
+        lib, stream = L.load(), _stream()
+        p = L.RaSwigluParams()
+        p.T, p.d, p.f = chunk_tokens, d, f
+        p.w1, p.w2, p.w3 = w1.data_ptr(), w2.data_ptr(), w3.data_ptr()
+        p.a, p.b, p.h = a.data_ptr(), b.data_ptr(), h.data_ptr()
+        for t0 in range(0, T, chunk_tokens):
+            p.x, p.y = x[t0:].data_ptr(), y[t0:].data_ptr()
+            L.check(lib.ra_swiglu_fwd(ctypes.byref(p), stream), "ra_swiglu_fwd")
+        ctx.save_for_backward(x, w1, w2, w3)
+        ctx.chunk_tokens = chunk_tokens
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w1, w2, w3 = ctx.saved_tensors
+        ct = ctx.chunk_tokens
+        T, d = x.shape
+        f = w1.shape[1]
+        dev = x.device
+        dy = dy.to(torch.bfloat16).contiguous()
+        bf = dict(dtype=torch.bfloat16, device=dev)
+        a, b, h, da, db = (torch.empty((ct, f), **bf) for _ in range(5))
+        dx = torch.empty((T, d), **bf)
+        dw1 = torch.zeros((d, f), dtype=torch.float32, device=dev)
+        dw3 = torch.zeros((d, f), dtype=torch.float32, device=dev)
+        dw2 = torch.zeros((f, d), dtype=torch.float32, device=dev)
+        lib, stream = L.load(), _stream()
+        p = L.RaSwigluParams()
+        p.T, p.d, p.f = ct, d, f
+        p.w1, p.w2, p.w3 = w1.data_ptr(), w2.data_ptr(), w3.data_ptr()
+        p.a, p.b, p.h, p.y = a.data_ptr(), b.data_ptr(), h.data_ptr(), None
+        p.dw1, p.dw2, p.dw3 = dw1.data_ptr(), dw2.data_ptr(), dw3.data_ptr()
+        p.da, p.db = da.data_ptr(), db.data_ptr()
+        for t0 in range(0, T, ct):
+            p.x, p.dy, p.dx = x[t0:].data_ptr(), dy[t0:].data_ptr(), dx[t0:].data_ptr()
+            L.check(lib.ra_swiglu_bwd(ctypes.byref(p), stream), "ra_swiglu_bwd")
+        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None
+
+
 class SwiGLU(torch.nn.Module):
     """The LLaMA-style MLP the reference's README pairs with blockwise_feedforward:
     w2(silu(x w1) * (x w3)); weights stored (in, out), bf16."""
@@ -94,6 +145,15 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
         raise ValueError("sequence length %d must divide by chunk_size %d" % (s, chunk_size))
     n = s // chunk_size
     if isinstance(feedforward, SwiGLU):
+        if inputs.dtype != torch.bfloat16:
+            raise NotImplementedError("SwiGLU kernels are bf16")
+        if not inputs.is_cuda:
+            raise RuntimeError("ringattention_amd runs on the GPU only")
+        if b == 1:
+            # contiguous slabs of chunk_size tokens, one autograd node for the whole scan
+            y = _BlockwiseSwiGLUFn.apply(inputs.reshape(s, d).contiguous(), feedforward.w1, feedforward.w2,
+                                         feedforward.w3, chunk_size)
+            return y.reshape(1, s, y.shape[-1])
         outs = [feedforward(inputs[:, j * chunk_size:(j + 1) * chunk_size]) for j in range(n)]
         return torch.cat(outs, dim=1)
     x = inputs.reshape(b, chunk_size, n, d)

@@ -83,3 +83,24 @@ def test_blockwise_feedforward_matches_oracle_and_unchunked():
     y2 = ra.blockwise_feedforward(probe, x.to(DEV), chunk)
     assert seen == [(B, chunk, d)] * (S // chunk)
     assert torch.equal(y2, whole)
+
+
+def test_blockwise_feedforward_single_batch_scan_gradients():
+    """B = 1 takes the one-node scan (weight gradients of all chunks accumulate in fp32 in the GEMM
+    epilogue): forward equals the unchunked MLP bit for bit, gradients match fp32 autograd."""
+    S, d, f, chunk = 1024, 128, 256, 256
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(1, S, d, generator=g).bfloat16()
+    dy = torch.randn(1, S, d, generator=g).bfloat16()
+    ff = ra.SwiGLU(d, f, device=DEV, init_std=0.05)
+    xd = x.to(DEV).requires_grad_(True)
+    y = ra.blockwise_feedforward(ff, xd, chunk)
+    assert torch.equal(y, ff(x.to(DEV)))
+    y.backward(dy.to(DEV))
+    w1, w2, w3 = (w.detach().float().cpu().requires_grad_(True) for w in (ff.w1, ff.w2, ff.w3))
+    xr = x.float().requires_grad_(True)
+    O.swiglu(xr, w1, w2, w3).backward(dy.float())
+    rel_ok(xd.grad, xr.grad, "dx")
+    rel_ok(ff.w1.grad, w1.grad, "dw1")
+    rel_ok(ff.w2.grad, w2.grad, "dw2")
+    rel_ok(ff.w3.grad, w3.grad, "dw3")
