@@ -2,11 +2,15 @@
 // blockwise_feedforward (ringattention_jax.py:333-352) scans over chunks of tokens.
 //
 // GEMM: C (M,N) = op(A) op(B) [+ op(A2) op(B2)], fp32 accumulation in v_mfma_f32_32x32x16_bf16.
-//   workgroup = 4 wavefronts (2 x 2), tile BM x BN, K step 64, LDS double buffered.
+//   workgroup = WGM x WGN wavefronts, tile BM x BN, K step 64, LDS double buffered.  The tile is
+//   chosen per problem: 256 x 256 over 8 wavefronts (each 128 x 64: six operand fragments from LDS
+//   per eight MFMAs, and half the global bytes per flop of a 128 x 128 tile) when that still gives
+//   every CU work, smaller tiles otherwise.
 //   An operand whose contraction index is contiguous in memory is staged row-major and read with
 //   16-byte LDS reads; one whose contraction index is the slow axis is staged as it lies in memory
 //   and read with ds_read_b64_tr_b16, so no layout ever needs a transposing copy.
 #include "common.hpp"
+#include <stdlib.h>
 
 namespace ra {
 
@@ -30,19 +34,21 @@ __device__ __forceinline__ s16x4 lds_tr(const uint16_t* p) {
 }
 
 // TA: A is stored (K,M).  TB: B is stored (N,K).
-template <bool TA, bool TB, int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
-  constexpr int WM = BM / 2, WN = BN / 2, MB = WM / 32, NB = WN / 32;
+template <bool TA, bool TB, int BM, int BN, int WGM, int WGN, bool DEEP>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
+  constexpr int NT = 64 * WGM * WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN, MB = WM / 32, NB = WN / 32;
   constexpr int A_STR = TA ? BM + 32 : NAT_STR;     // elements
   constexpr int B_STR = TB ? NAT_STR : BN + 32;
   constexpr int A_ROWS = TA ? GBK : BM, B_ROWS = TB ? BN : GBK;
   constexpr int A_CPR = (TA ? BM : GBK) / 8, B_CPR = (TB ? GBK : BN) / 8;   // 16-byte chunks per staged row
-  constexpr int A_CH = A_ROWS * A_CPR / 256, B_CH = B_ROWS * B_CPR / 256;   // chunks per thread
+  constexpr int A_CH = A_ROWS * A_CPR / NT, B_CH = B_ROWS * B_CPR / NT;     // chunks per thread
+  static_assert(A_CH * NT == A_ROWS * A_CPR && B_CH * NT == B_ROWS * B_CPR, "tile does not divide over the threads");
   __shared__ __attribute__((aligned(16))) uint16_t As[2][A_ROWS * A_STR];
   __shared__ __attribute__((aligned(16))) uint16_t Bs[2][B_ROWS * B_STR];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   // neighbouring workgroups share the A row panel (and, 8 apart, the same XCD's L2)
   const int ntn = g.N / BN;
   const int tm = blockIdx.x / ntn, tn = blockIdx.x % ntn;
@@ -56,87 +62,124 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  uint4 ar[A_CH], br[B_CH];
+  // staging registers: two sets (P, Q) of named scalars and straight-line code (arrays that stay live
+  // across the MFMA section end up in scratch memory).  A K slab is requested two iterations before it
+  // is stored to LDS, which covers the global latency under load.
+  static_assert(A_CH <= 4 && B_CH <= 4, "at most four 16-byte chunks per thread and operand");
+  uint4 Pa0, Pa1, Pa2, Pa3, Pb0, Pb1, Pb2, Pb3, Qa0, Qa1, Qa2, Qa3, Qb0, Qb1, Qb2, Qb3;
   const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
-  const uint16_t* Ap = g.A; const uint16_t* Bp = g.B;
-#define RA_LOAD_STAGE(K0)                                                                               \
+  const int nk = g.K / GBK;
+  const int total = nk * (g.A2 ? 2 : 1);
+  // chunk c of this thread: staged row and 16-byte column, fixed for the whole kernel
+#define RA_A_OFF(C, K0) (TA ? (int64_t)((K0) + ((C) * NT + tid) / A_CPR) * lda + m0 + (((C) * NT + tid) % A_CPR) * 8 \
+                            : (int64_t)(m0 + ((C) * NT + tid) / A_CPR) * lda + (K0) + (((C) * NT + tid) % A_CPR) * 8)
+#define RA_B_OFF(C, K0) (TB ? (int64_t)(n0 + ((C) * NT + tid) / B_CPR) * ldb + (K0) + (((C) * NT + tid) % B_CPR) * 8 \
+                            : (int64_t)((K0) + ((C) * NT + tid) / B_CPR) * ldb + n0 + (((C) * NT + tid) % B_CPR) * 8)
+#define RA_A_LDS(C) ((((C) * NT + tid) / A_CPR) * A_STR + (((C) * NT + tid) % A_CPR) * 8)
+#define RA_B_LDS(C) ((((C) * NT + tid) / B_CPR) * B_STR + (((C) * NT + tid) % B_CPR) * 8)
+  // slab T (clamped to the last one; slabs nk .. 2 nk - 1 belong to the second operand pair)
+#define RA_LOAD_STAGE(S, T)                                                                             \
   {                                                                                                     \
-    const int k0_ = (K0);                                                                               \
-    _Pragma("unroll") for (int c = 0; c < A_CH; c++) {                                                  \
-      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;                               \
-      const int64_t off = TA ? (int64_t)(k0_ + row) * lda + m0 + ch * 8 : (int64_t)(m0 + row) * lda + k0_ + ch * 8; \
-      ar[c] = *(const uint4*)(Ap + off);                                                                \
-    }                                                                                                   \
-    _Pragma("unroll") for (int c = 0; c < B_CH; c++) {                                                  \
-      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;                               \
-      const int64_t off = TB ? (int64_t)(n0 + row) * ldb + k0_ + ch * 8 : (int64_t)(k0_ + row) * ldb + n0 + ch * 8; \
-      br[c] = *(const uint4*)(Bp + off);                                                                \
-    }                                                                                                   \
+    const int t_ = min((T), total - 1);                                                                 \
+    const uint16_t* Ap = t_ >= nk ? g.A2 : g.A;                                                         \
+    const uint16_t* Bp = t_ >= nk ? g.B2 : g.B;                                                         \
+    const int k0_ = (t_ >= nk ? t_ - nk : t_) * GBK;                                                    \
+    if (A_CH > 0) S##a0 = *(const uint4*)(Ap + RA_A_OFF(0, k0_));                                       \
+    if (A_CH > 1) S##a1 = *(const uint4*)(Ap + RA_A_OFF(1, k0_));                                       \
+    if (A_CH > 2) S##a2 = *(const uint4*)(Ap + RA_A_OFF(2, k0_));                                       \
+    if (A_CH > 3) S##a3 = *(const uint4*)(Ap + RA_A_OFF(3, k0_));                                       \
+    if (B_CH > 0) S##b0 = *(const uint4*)(Bp + RA_B_OFF(0, k0_));                                       \
+    if (B_CH > 1) S##b1 = *(const uint4*)(Bp + RA_B_OFF(1, k0_));                                       \
+    if (B_CH > 2) S##b2 = *(const uint4*)(Bp + RA_B_OFF(2, k0_));                                       \
+    if (B_CH > 3) S##b3 = *(const uint4*)(Bp + RA_B_OFF(3, k0_));                                       \
   }
-#define RA_STORE_STAGE(BUF)                                                                             \
+#define RA_STORE_STAGE(S, BUF)                                                                          \
   {                                                                                                     \
-    _Pragma("unroll") for (int c = 0; c < A_CH; c++) {                                                  \
-      const int idx = c * 256 + tid, row = idx / A_CPR, ch = idx % A_CPR;                               \
-      *(uint4*)(&As[BUF][row * A_STR + ch * 8]) = ar[c];                                                \
-    }                                                                                                   \
-    _Pragma("unroll") for (int c = 0; c < B_CH; c++) {                                                  \
-      const int idx = c * 256 + tid, row = idx / B_CPR, ch = idx % B_CPR;                               \
-      *(uint4*)(&Bs[BUF][row * B_STR + ch * 8]) = br[c];                                                \
-    }                                                                                                   \
+    if (A_CH > 0) *(uint4*)(&As[BUF][RA_A_LDS(0)]) = S##a0;                                             \
+    if (A_CH > 1) *(uint4*)(&As[BUF][RA_A_LDS(1)]) = S##a1;                                             \
+    if (A_CH > 2) *(uint4*)(&As[BUF][RA_A_LDS(2)]) = S##a2;                                             \
+    if (A_CH > 3) *(uint4*)(&As[BUF][RA_A_LDS(3)]) = S##a3;                                             \
+    if (B_CH > 0) *(uint4*)(&Bs[BUF][RA_B_LDS(0)]) = S##b0;                                             \
+    if (B_CH > 1) *(uint4*)(&Bs[BUF][RA_B_LDS(1)]) = S##b1;                                             \
+    if (B_CH > 2) *(uint4*)(&Bs[BUF][RA_B_LDS(2)]) = S##b2;                                             \
+    if (B_CH > 3) *(uint4*)(&Bs[BUF][RA_B_LDS(3)]) = S##b3;                                             \
   }
 
   // transpose-read lane offset: 16-lane group reads 4 contraction rows x 16 columns
   const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
   const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  const int nk = g.K / GBK;
-  const int npairs = g.A2 ? 2 : 1;
-  const int total = nk * npairs;
-  RA_LOAD_STAGE(0);
-  RA_STORE_STAGE(0);
-  __syncthreads();
-  for (int it = 0; it < total; it++) {
-    const int cur = it & 1;
-    {
-      // prefetch the next K slab (the last iteration re-reads its own slab into the idle buffer)
-      const int nx = min(it + 1, total - 1);
-      if (nx >= nk) { Ap = g.A2; Bp = g.B2; }
-      RA_LOAD_STAGE((nx % nk) * GBK);
-    }
-#pragma unroll
-    for (int kk = 0; kk < GBK / 16; kk++) {
-      bf16x8 af[MB], bfr[NB];
-#pragma unroll
-      for (int i = 0; i < MB; i++) {
-        if (!TA) {
-          af[i] = *(const bf16x8*)(&As[cur][(wm * WM + i * 32 + lo) * A_STR + kk * 16 + hi * 8]);
-        } else {
-          const uint16_t* p = &As[cur][kk * 16 * A_STR + trA + wm * WM + i * 32];
-          s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);
-          af[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < NB; j++) {
-        if (TB) {
-          bfr[j] = *(const bf16x8*)(&Bs[cur][(wn * WN + j * 32 + lo) * B_STR + kk * 16 + hi * 8]);
-        } else {
-          const uint16_t* p = &Bs[cur][kk * 16 * B_STR + trB + wn * WN + j * 32];
-          s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);
-          bfr[j] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < MB; i++)
-#pragma unroll
-        for (int j = 0; j < NB; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-    }
-    RA_STORE_STAGE(cur ^ 1);
-    __syncthreads();
+#define RA_COMPUTE(CUR_)                                                                                \
+  {                                                                                                     \
+    _Pragma("unroll")                                                                                  \
+    for (int kk = 0; kk < GBK / 16; kk++) {                                                             \
+      bf16x8 af[MB], bfr[NB];                                                                           \
+    _Pragma("unroll")                                                                                  \
+      for (int i = 0; i < MB; i++) {                                                                    \
+        if (!TA) {                                                                                      \
+          af[i] = *(const bf16x8*)(&As[CUR_][(wm * WM + i * 32 + lo) * A_STR + kk * 16 + hi * 8]);      \
+        } else {                                                                                        \
+          const uint16_t* p = &As[CUR_][kk * 16 * A_STR + trA + wm * WM + i * 32];                      \
+          s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);                                             \
+          af[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));  \
+        }                                                                                               \
+      }                                                                                                 \
+    _Pragma("unroll")                                                                                  \
+      for (int j = 0; j < NB; j++) {                                                                    \
+        if (TB) {                                                                                       \
+          bfr[j] = *(const bf16x8*)(&Bs[CUR_][(wn * WN + j * 32 + lo) * B_STR + kk * 16 + hi * 8]);     \
+        } else {                                                                                        \
+          const uint16_t* p = &Bs[CUR_][kk * 16 * B_STR + trB + wn * WN + j * 32];                      \
+          s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);                                             \
+          bfr[j] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7)); \
+        }                                                                                               \
+      }                                                                                                 \
+    _Pragma("unroll")                                                                                  \
+      for (int i = 0; i < MB; i++)                                                                      \
+    _Pragma("unroll")                                                                                  \
+        for (int j = 0; j < NB; j++)                                                                    \
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);       \
+    }                                                                                                   \
   }
+  RA_LOAD_STAGE(P, 0);
+  RA_STORE_STAGE(P, 0);
+  if (DEEP) {
+    RA_LOAD_STAGE(Q, 1);
+    RA_LOAD_STAGE(P, 2);
+    __syncthreads();
+    for (int it = 0; it < total; it += 2) {
+      // slab it is in buffer 0; slab it + 1 goes to buffer 1, slab it + 3 is requested
+      RA_STORE_STAGE(Q, 1);
+      RA_LOAD_STAGE(Q, it + 3);
+      __builtin_amdgcn_sched_barrier(0);
+      RA_COMPUTE(0);
+      __syncthreads();
+      if (it + 1 >= total) break;
+      RA_STORE_STAGE(P, 0);
+      RA_LOAD_STAGE(P, it + 4);
+      __builtin_amdgcn_sched_barrier(0);
+      RA_COMPUTE(1);
+      __syncthreads();
+    }
+  } else {
+    // one register set (the tile's accumulators leave no room for two): a slab is in flight for one iteration
+    __syncthreads();
+    for (int it = 0; it < total; it++) {
+      const int cur = it & 1;
+      RA_LOAD_STAGE(P, it + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      RA_COMPUTE(cur);
+      RA_STORE_STAGE(P, cur ^ 1);
+      __syncthreads();
+    }
+  }
+#undef RA_COMPUTE
 #undef RA_LOAD_STAGE
 #undef RA_STORE_STAGE
+#undef RA_A_OFF
+#undef RA_B_OFF
+#undef RA_A_LDS
+#undef RA_B_LDS
 
   // epilogue: lane holds column n = lo of each 32x32 block, rows 8*(r/4) + 4*hi + r%4
 #pragma unroll
@@ -158,17 +201,51 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
     }
 }
 
+template <bool TA, bool TB, int BM, int BN, int WGM, int WGN, bool DEEP>
+static int launch_tile(const GemmArgs& g, hipStream_t s) {
+  const long long nwg = (long long)(g.M / BM) * (g.N / BN);
+  gemm_bf16_kernel<TA, TB, BM, BN, WGM, WGN, DEEP><<<dim3((unsigned)nwg), 64 * WGM * WGN, 0, s>>>(g);
+  RA_CHECK_LAUNCH("gemm_bf16");
+  return RA_OK;
+}
+
+// Tile choice.  One workgroup of the large tiles fills a CU's LDS, so the grid runs in rounds of (number of CUs)
+// workgroups: take the largest tile whose last round is not mostly idle.
+static int pick_tile(int M, int N) {
+  if (const char* e = getenv("RA_GEMM_TILE")) return atoi(e);
+  static int ncu = 0;
+  if (!ncu) {
+    int dev = 0;
+    hipDeviceProp_t pr;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) ncu = pr.multiProcessorCount;
+    if (ncu <= 0) ncu = 256;
+  }
+  auto eff = [&](int bm, int bn) {
+    if (M % bm || N % bn) return 0.0;
+    const double n = (double)(M / bm) * (N / bn);
+    return n / (ceil(n / ncu) * ncu);
+  };
+  if (eff(256, 256) >= 0.8) return 0;
+  if (eff(256, 128) >= 0.8) return 1;
+  if (eff(256, 256) >= 0.66) return 0;
+  if (eff(256, 128) >= 0.66) return 1;
+  return 2;
+}
+
 template <bool TA, bool TB>
 static int launch_gemm(const GemmArgs& g, hipStream_t s) {
-  constexpr int BM = 128, BN = 128;
-  if (g.M % BM || g.N % BN || g.K % GBK) {
+  if (g.M % 128 || g.N % 128 || g.K % GBK) {
     set_error("gemm_bf16: M, N must be multiples of 128 and K of 64 (got %d, %d, %d)", g.M, g.N, g.K);
     return RA_ERR_UNSUPPORTED;
   }
-  const long long nwg = (long long)(g.M / BM) * (g.N / BN);
-  gemm_bf16_kernel<TA, TB, BM, BN><<<dim3((unsigned)nwg), 256, 0, s>>>(g);
-  RA_CHECK_LAUNCH("gemm_bf16");
-  return RA_OK;
+  int t = pick_tile(g.M, g.N);
+  if (t == 0 && (g.M % 256 || g.N % 256)) t = 1;
+  if (t == 1 && g.M % 256) t = 2;
+  switch (t) {
+    case 0: return launch_tile<TA, TB, 256, 256, 2, 4, false>(g, s);
+    case 1: return launch_tile<TA, TB, 256, 128, 4, 2, true>(g, s);
+    default: return launch_tile<TA, TB, 128, 128, 2, 2, false>(g, s);
+  }
 }
 
 static int gemm_dispatch(const GemmArgs& g, int ta, int tb, hipStream_t s) {
