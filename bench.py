@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ring-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|copy]
 
 One step = one pass of the hot path over one batch of synthetic input already resident in HBM.
 Default workload ``attn32k`` is the configuration the headline metric is quoted on: blockwise
@@ -21,6 +21,10 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters'
+# reading for the 1 GiB copy of --workload copy) at the default sizes of each workload
+MEASURED_TRAFFIC = {"attn_fwd_pp_kernel": 7.30e9, "attn_bwd_dkv_ws_kernel": 6.28e9, "attn_bwd_dq_ws_kernel": 4.56e9,
+                    "decode_split_kernel": 68.88e9}
 
 
 def _kwargs(qc, kc, cbs=1, **extra):
@@ -139,7 +143,8 @@ def bench_attention(args, ring):
         dms, dfl = kern[dom]
         ach = dfl / (dms * 1e-3) / 1e12
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
+                "traffic": MEASURED_TRAFFIC.get(dom) if S == 32768 else None,
                 "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
                 "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
     cpu = cpu_baseline_attention() if not args.no_cpu else None
@@ -228,7 +233,8 @@ def bench_decode(args):
         "config": {"workload": "decode", "B": B, "H": H, "D": D, "cache_len": Lf, "key_chunk_size": kc,
                    "query_chunk_size": 1, "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "kernel": "decode_split_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC["decode_split_kernel"] if (B, Lf) == (16, 262144) else None},
         "cpu_baseline": cpu,
     }
 
@@ -281,12 +287,29 @@ def bench_ffn(args):
     }
 
 
+# --------------------------------------------------------------------------- calibration copy
+def bench_copy(args):
+    """A plain 1 GiB device-to-device copy: the kernel of known size that the FETCH_SIZE / WRITE_SIZE
+    counters of a ``rocprofv3 --pmc`` run are scaled by (it reads and writes exactly 2**30 bytes)."""
+    import torch
+    n = 1 << 28
+    src = torch.empty(n, dtype=torch.float32, device="cuda:0").normal_()
+    dst = torch.empty_like(src)
+    ms = _time_steps(lambda: dst.copy_(src), args.steps, args.warmup)
+    gbs = 2.0 * n * 4 / (ms * 1e-3) / 1e9
+    return {"metric": "device_copy_gbs", "value": round(gbs, 1), "unit": "GB/s", "ms_per_step": round(ms, 3),
+            "dtype": "u8", "config": {"workload": "copy", "bytes_read": n * 4, "bytes_written": n * 4},
+            "roofline": {"bound": "hbm", "kernel": "copyBuffer", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": 2.0 * n * 4},
+            "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode"])
+    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "copy"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -301,6 +324,8 @@ def main():
         r = bench_attention(args, ring=(args.workload == "ring131k"))
     elif args.workload == "decode":
         r = bench_decode(args)
+    elif args.workload == "copy":
+        r = bench_copy(args)
     else:
         r = bench_ffn(args)
     line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
