@@ -67,6 +67,14 @@ typedef struct ra_mask {
                                      skip_masked_tiles it lets kernels skip key (query) tiles whose id range
                                      cannot meet the ids of the query (key) rows at hand */
   int32_t seg_tiles;
+  const uint8_t* keep;        /* nullable; the boolean attn_mask of ring_attention_inference
+                                 (ringattention_inference.py:19-22): nonzero = attend, zero = the logit becomes
+                                 mask_min.  Indexed by the LOCAL query row of the call and the GLOBAL key position;
+                                 only the generic kernels take it */
+  int64_t keep_stride_b;      /* element (byte) strides; 0 broadcasts that axis */
+  int64_t keep_stride_h;
+  int64_t keep_stride_q;
+  int64_t keep_stride_k;
 } ra_mask;
 
 /* _blockwise_attention_fwd (ringattention_jax.py:99-179): one ring step on one device.

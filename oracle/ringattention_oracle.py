@@ -21,6 +21,9 @@ vectors, and JAX/flax are not importable where this was written):
   the ``min(bias, 0)`` clamp and the two ``finfo.min`` constants.
 * ``blockwise_feedforward``: equals the un-chunked feed-forward; SwiGLU
   backward is torch autograd.
+* ``ring_attention_inference_fwd`` / ``_bwd`` (ringattention_inference.py): checked in float64
+  against ``dense_attention_inference`` (an un-chunked masked softmax) and its torch autograd, over
+  ring sizes, broadcast mask shapes and rows with no attended key.
 
 Parity unpinned (would need the reference's own runtime): the dropout mask
 bits (``jax.random`` stream) - dropout is refused - and XLA-CPU's exact
@@ -332,6 +335,102 @@ def dense_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, block
         logits = torch.where(run[None, None], logits, torch.full((), -math.inf, dtype=wd))
     p = torch.softmax(logits, dim=-1)      # all -inf rows -> NaN, as 0/0 in the reference (:52)
     return torch.einsum('bhqk,bkhd->bqhd', p, v.to(wd))
+
+
+# --------------------------------------------------------------------------- mask-based inference ring
+def _mask_rows(attn_mask, dev, q_len, q_total):
+    """The device's view of the global boolean mask (B|1, H|1, Q_total|1, K_total): its own query rows
+    when the mask has a query axis (the mask is sharded like q), the broadcast row otherwise."""
+    if attn_mask.shape[2] == 1:
+        return attn_mask
+    assert attn_mask.shape[2] == q_total
+    return attn_mask[:, :, dev * q_len:(dev + 1) * q_len]
+
+
+def ring_attention_inference_fwd(q, k, v, attn_mask, axis_size, float32_logits=True, compute_dtype=None):
+    """ringattention_inference.py:8-36 for every device of a ring of ``axis_size`` (global arrays, as in
+    ring_attention_fwd above): un-chunked online softmax per ring step, boolean mask sliced along its key
+    axis at the block that would have arrived at that step (:19-20), masked logits set to finfo.min of the
+    logits' dtype (:22)."""
+    wd = compute_dtype or (torch.float32 if (float32_logits or q.dtype == torch.float32) else q.dtype)
+    n = axis_size
+    qw, kw = q.to(wd), k.to(wd)                                            # :9-10
+    batch, q_total, num_heads, dim = q.shape
+    kv_total = k.shape[1]
+    q_len, kv_len = q_total // n, kv_total // n
+    scale = math.sqrt(dim)                                                  # :16
+    neg = finfo_min(wd)
+    outs, nums, dens, maxs = [], [], [], []
+    for dev in range(n):
+        q_d = qw[:, dev * q_len:(dev + 1) * q_len]
+        m_d = _mask_rows(attn_mask, dev, q_len, q_total)
+        num = torch.zeros((batch, q_len, num_heads, dim), dtype=wd)         # :13
+        den = torch.zeros((batch, num_heads, q_len), dtype=wd)              # :14
+        prev = torch.full((batch, num_heads, q_len), -math.inf, dtype=wd)   # :31
+        for idx in range(n):                                                # :32-33
+            k_blk = (dev - idx) % n                                         # :20
+            ksl = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            mask = m_d[..., ksl]                                            # :19-20
+            w = torch.einsum("bqhd,bkhd->bhqk", q_d, kw[:, ksl]) / scale    # :21
+            w = torch.where(mask, w, torch.full_like(w, neg))               # :22
+            mx = torch.maximum(prev, w.max(dim=-1).values)                  # :23
+            e = torch.exp(w - mx[..., None])                                # :24
+            corr = torch.exp(prev - mx)                                     # :25
+            num = num * corr.permute(0, 2, 1)[..., None] + torch.einsum("bhqk,bkhd->bqhd", e, v[:, ksl].to(wd))   # :26
+            den = den * corr + e.sum(dim=-1)                                # :27
+            prev = mx
+        outs.append(num / den.permute(0, 2, 1)[..., None])                  # :34
+        nums.append(num); dens.append(den); maxs.append(prev)
+    output = torch.cat(outs, dim=1)
+    res = (output, qw, kw, v, attn_mask, torch.cat(nums, dim=1), torch.cat(dens, dim=2), torch.cat(maxs, dim=2))
+    return output.to(v.dtype), res                                          # :35
+
+
+def ring_attention_inference_bwd(axis_size, res, g):
+    """ringattention_inference.py:38-64 for every device of the ring; returns global fp32 dq, dk, dv cast to
+    the residual dtypes (:62)."""
+    output, q, k, v, attn_mask, _num, denominator, max_score = res
+    n = axis_size
+    batch, q_total, num_heads, dim = q.shape
+    kv_total = k.shape[1]
+    q_len, kv_len = q_total // n, kv_total // n
+    scale = math.sqrt(dim)                                                  # :46
+    neg = finfo_min(q.dtype)
+    acc = torch.float64 if q.dtype == torch.float64 else torch.float32   # fp32 in the reference
+    dq = torch.zeros(q.shape, dtype=acc)                                    # :42
+    dk = torch.zeros(k.shape, dtype=acc)                                    # :43
+    dv = torch.zeros(v.shape, dtype=acc)                                    # :44
+    gf = g.to(acc)
+    for dev in range(n):
+        qsl = slice(dev * q_len, (dev + 1) * q_len)
+        m_d = _mask_rows(attn_mask, dev, q_len, q_total)
+        for idx in range(n):
+            k_blk = (dev - idx) % n                                         # :50
+            ksl = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            mask = m_d[..., ksl]
+            w = torch.einsum("bqhd,bkhd->bhqk", q[:, qsl], k[:, ksl]) / scale              # :51
+            w = torch.where(mask, w, torch.full_like(w, neg))                              # :52
+            p = torch.exp(w - max_score[:, :, qsl, None]) / denominator[:, :, qsl, None]   # :53
+            ds = torch.einsum("bqhd,bkhd->bhqk", gf[:, qsl], v[:, ksl].to(acc))  # :54
+            dl = (ds - torch.einsum("bqhd,bqhd->bhq", gf[:, qsl], output[:, qsl].to(acc))[..., None]) * p   # :55
+            dq[:, qsl] += torch.einsum("bhqk,bkhd->bqhd", dl, k[:, ksl].to(acc)) / scale   # :56
+            dk[:, ksl] += torch.einsum("bqhd,bhqk->bkhd", q[:, qsl].to(acc), dl) / scale   # :57
+            dv[:, ksl] += torch.einsum("bhqk,bqhd->bkhd", p.to(acc), gf[:, qsl])           # :58
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)                   # :62
+
+
+def dense_attention_inference(q, k, v, attn_mask, dtype=torch.float64):
+    """Independent closed form for ring_attention_inference: softmax over all keys of
+    where(mask, Q K^T / sqrt(D), -inf) times V.  A row with no attended key is the mean of V over all keys:
+    the reference's finfo.min logits are all equal there and softmax of a constant is uniform."""
+    qd, kd, vd = q.to(dtype), k.to(dtype), v.to(dtype)
+    w = torch.einsum("bqhd,bkhd->bhqk", qd, kd) / math.sqrt(q.shape[-1])
+    mask = attn_mask.expand(w.shape[0], w.shape[1], w.shape[2], w.shape[3])
+    none = ~mask.any(dim=-1, keepdim=True)
+    w = torch.where(mask | none, w, torch.full_like(w, -math.inf))
+    w = torch.where(none, torch.zeros_like(w), w)
+    p = torch.softmax(w, dim=-1)
+    return torch.einsum("bhqk,bkhd->bqhd", p, vd)
 
 
 def swiglu(x, w1, w2, w3):

@@ -3,7 +3,7 @@
 Exports the names of the reference package (ringattention/__init__.py:26-27 binds ``ringattention``
 per backend; here there is one backend, the gfx950 HIP kernels):
 
-    ringattention, ringattention_jax, blockwise_feedforward
+    ringattention, ringattention_jax, ringattention_inference, blockwise_feedforward
 
 plus ``ring_axis`` to declare the size of the (virtual) sequence-parallel ring, ``SwiGLU`` and
 ``decode_attention``.
@@ -12,9 +12,12 @@ from .ringattention_hip import (ring_attention, ring_axis, axis_size, below_or_o
                                 _blockwise_attention_fwd, _blockwise_attention_bwd)
 from .feedforward import blockwise_feedforward, SwiGLU, gemm_bf16
 from .decode import decode_attention
+from .inference import ring_attention_inference
 
 ringattention = ring_attention
 ringattention_jax = ring_attention
+ringattention_inference = ring_attention_inference
 
-__all__ = ["ringattention", "ringattention_jax", "ring_attention", "blockwise_feedforward", "ring_axis",
+__all__ = ["ringattention", "ringattention_jax", "ringattention_inference", "ring_attention",
+           "ring_attention_inference", "blockwise_feedforward", "ring_axis",
            "axis_size", "SwiGLU", "decode_attention", "below_or_on_diag"]

@@ -25,6 +25,8 @@ class RaMask(C.Structure):
         ("causal_block_size", i32), ("query_chunk_size", i32), ("key_chunk_size", i32),
         ("q_chunk_idx_start", i32), ("k_chunk_idx_start", i32), ("cache_idx", vp), ("mask_min", f32),
         ("skip_masked_tiles", i32), ("seg_tile_minmax", vp), ("seg_tiles", i32),
+        ("keep", vp), ("keep_stride_b", i64), ("keep_stride_h", i64), ("keep_stride_q", i64),
+        ("keep_stride_k", i64),
     ]
 
 

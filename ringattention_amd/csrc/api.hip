@@ -151,6 +151,7 @@ int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->mask.query_chunk_size == 1, RA_ERR_INVALID,
              "decode_fwd: one query token needs query_chunk_size == 1 (q_len // query_chunk_size chunks)");
   if (int rc = check_mask(p->mask, 1, p->L, "decode_fwd")) return rc;
+  RA_REQUIRE(p->mask.keep == nullptr, RA_ERR_UNSUPPORTED, "decode_fwd: the boolean keep mask is taken by the generic attention kernels only");
   int ns = p->num_splits > 0 ? p->num_splits : decode_pick_splits(p->B, p->L, p->H, p->D, p->dtype);
   RA_REQUIRE(ns <= 256, RA_ERR_INVALID, "decode_fwd: num_splits %d > 256", ns);
   size_t need = (size_t)p->B * p->H * ns * (p->D + 2) * sizeof(float);

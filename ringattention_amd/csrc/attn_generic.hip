@@ -36,6 +36,7 @@ struct RowInfo {
   long long gq_blk;
   int seg;
   int64_t bias_off;
+  int64_t keep_off;
 };
 
 __device__ __forceinline__ RowInfo row_info(const MaskView& mv, int b, int h, int row, int skv) {
@@ -50,6 +51,7 @@ __device__ __forceinline__ RowInfo row_info(const MaskView& mv, int b, int h, in
     r.seg = mv.seg[(int64_t)b * mv.seg_sb + idx];
   }
   r.bias_off = (int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(row % mv.qc) * mv.bias_sq;
+  r.keep_off = (int64_t)b * mv.keep_sb + (int64_t)h * mv.keep_sh + (int64_t)row * mv.keep_sq;
   return r;
 }
 
@@ -64,6 +66,7 @@ __device__ __forceinline__ float logit(const MaskView& mv, const RowInfo& r, flo
     if (mv.any_mask) add = fminf(add, 0.f);                       // minimum(), :299,:309
   }
   bool masked = (mv.cbs > 0 && r.gq_blk < gk / mv.cbs) || (mv.seg && r.seg != seg_k);
+  if (mv.keep && !mv.keep[r.keep_off + gk * mv.keep_sk]) masked = true;   // where(mask, w, finfo.min), ringattention_inference.py:24
   if (masked) add = mv.mask_min;
   return dot / scale + add;                                       // :134-136
 }

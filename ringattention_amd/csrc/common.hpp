@@ -61,6 +61,8 @@ struct MaskView {
   int skip_tiles;
   const int32_t* seg_mm;   // per-64-position (min, max) segment ids, or null
   int seg_tiles;
+  const uint8_t* keep;     // boolean mask (local query row, global key), or null
+  int64_t keep_sb, keep_sh, keep_sq, keep_sk;
 
   __host__ __device__ static MaskView make(const ra_mask& m, int q_chunk_idx_start) {
     MaskView v;
@@ -73,6 +75,8 @@ struct MaskView {
     v.any_mask = (m.segment_ids != nullptr) || (m.causal_block_size > 0);
     v.skip_tiles = m.skip_masked_tiles;
     v.seg_mm = m.seg_tile_minmax; v.seg_tiles = m.seg_tiles;
+    v.keep = m.keep; v.keep_sb = m.keep_stride_b; v.keep_sh = m.keep_stride_h;
+    v.keep_sq = m.keep_stride_q; v.keep_sk = m.keep_stride_k;
     return v;
   }
 

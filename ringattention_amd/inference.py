@@ -1,0 +1,91 @@
+"""ring_attention_inference (ringattention/ringattention_inference.py:8-73): the ring with a boolean
+attention mask and no chunking inside a ring step, over the fp32 vector-ALU kernels of
+libringattn_hip.so (the MFMA kernels take no per-pair mask operand)."""
+import torch
+
+from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, _blockwise_attention_fwd,
+                                _bwd_delta, _check_qkv, _finalize, axis_size)
+
+
+def _inference_cfg(q, q_len, kv_len, float32_logits):
+    # one "chunk" per ring step (:21 is a single einsum over the shard); finfo.min of the logits' dtype (:22)
+    logits_dtype = torch.float32 if (float32_logits or q.dtype == torch.float32) else q.dtype
+    return _Config(dict(causal_block_size=None, query_chunk_size=q_len, key_chunk_size=kv_len, deterministic=True,
+                        attn_pdrop=0.0, dtype=logits_dtype, impl="generic", skip_masked_tiles=False))
+
+
+def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
+    _check_qkv(q, k, v)
+    q, k, v = (t if (t.stride(3) == 1 and t.stride(2) == t.shape[3]) else t.contiguous() for t in (q, k, v))
+    n = axis_size(axis_name)                                                     # :15
+    B, q_total, H, D = q.shape
+    kv_total = k.shape[1]
+    if q_total % n or kv_total % n:
+        raise ValueError("sequence lengths must divide by the ring size %d" % n)
+    q_len, kv_len = q_total // n, kv_total // n
+    if attn_mask.dim() != 4 or attn_mask.shape[3] != kv_total or attn_mask.shape[2] not in (1, q_total) or \
+            attn_mask.shape[0] not in (1, B) or attn_mask.shape[1] not in (1, H):
+        raise ValueError("attn_mask must be (B|1, H|1, Q|1, K) with Q = %d and K = %d" % (q_total, kv_total))
+    cfg = _inference_cfg(q, q_len, kv_len, float32_logits)
+    mi = _MaskInputs(cfg, None, None, None, B, q.device, kv_total)
+    mi.set_keep(attn_mask, q.device)
+    num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)   # :13
+    den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)      # :14
+    mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)       # :31
+    for dev in range(n):
+        qs = slice(dev * q_len, (dev + 1) * q_len)
+        mi.keep_row0 = dev * q_len                  # the device's rows of a mask that is sharded like q
+        carry = (num[:, qs], den[:, :, qs], mx[:, :, qs])
+        for idx in range(n):                                                      # :32-33
+            k_blk = (dev - idx) % n                                               # :20
+            ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, dev, k_blk, None, None,
+                                     None, q_len, kv_len, _mask_inputs=mi, _cfg=cfg, _carry_is_initial=(idx == 0))
+    out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
+    _finalize(num, den, out)                                                      # :34
+    return out, (out, q, k, v, mi, cfg, n, den, mx)
+
+
+def _bwd(res, g):
+    out, q, k, v, mi, cfg, n, den, mx = res
+    B, q_total, H, D = q.shape
+    kv_total = k.shape[1]
+    q_len, kv_len = q_total // n, kv_total // n
+    g = g.to(q.dtype).contiguous()
+    delta = _bwd_delta(g, out)                                                    # :55
+    dq = torch.zeros((B, q_total, H, D), dtype=torch.float32, device=q.device)    # :42
+    dk = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)   # :43
+    dv = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)   # :44
+    for dev in range(n):
+        qs = slice(dev * q_len, (dev + 1) * q_len)
+        mi.keep_row0 = dev * q_len
+        for idx in range(n):
+            k_blk = (dev - idx) % n                                               # :50
+            ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            _blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], g[:, qs],
+                                     (dq[:, qs], dk[:, ks], dv[:, ks], out[:, qs], den[:, :, qs], mx[:, :, qs]),
+                                     dev, k_blk, None, None, None, q_len, kv_len,
+                                     _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs])
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)                         # :62
+
+
+class _RingAttentionInferenceFn(torch.autograd.Function):
+    """custom_vjp of ringattention_inference.py:67-73: cotangents for q, k, v; None for the mask (:64)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, attn_mask, axis_name, float32_logits):
+        out, res = _fwd(q, k, v, attn_mask, axis_name, float32_logits)
+        ctx.res = res
+        return out
+
+    @staticmethod
+    def backward(ctx, g):
+        dq, dk, dv = _bwd(ctx.res, g)
+        ctx.res = None
+        return dq, dk, dv, None, None, None
+
+
+def ring_attention_inference(q, k, v, attn_mask, axis_name, float32_logits=True):
+    """ringattention_inference.py:67-70.  q, k, v are the global (B, S, H, D) arrays of the virtual ring
+    declared with ``ring_axis``; attn_mask is the global boolean mask (B|1, H|1, Q|1, K), True = attend."""
+    return _RingAttentionInferenceFn.apply(q, k, v, attn_mask, axis_name, float32_logits)

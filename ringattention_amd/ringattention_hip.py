@@ -170,6 +170,9 @@ class _MaskInputs:
             L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], self.seg_len,
                                                     self.seg_mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
             self._seg_mm_host = None
+        self.keep = None                   # boolean mask of ring_attention_inference, set by set_keep()
+        self.keep_strides = (0, 0, 0, 0)
+        self.keep_row0 = 0
         self.cache_idx_host = None
         self.cache_idx_dev = None
         if cache_idx is not None:
@@ -180,6 +183,14 @@ class _MaskInputs:
                     self.cache_idx_host = int(cache_idx)
             else:
                 self.cache_idx_host = int(cache_idx)
+
+    def set_keep(self, attn_mask, device):
+        """attn_mask (B|1, H|1, Q|1, K_total), nonzero = attend (ringattention_inference.py:19-22)."""
+        if attn_mask.dim() != 4:
+            raise ValueError("attn_mask must be 4-D (B, H, Q, K)")
+        m = (attn_mask.detach().to(device=device) != 0).to(torch.uint8).contiguous()
+        self.keep = m
+        self.keep_strides = tuple(0 if m.shape[i] == 1 else m.stride(i) for i in range(4))
 
     def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip):
         m = L.RaMask()
@@ -198,6 +209,9 @@ class _MaskInputs:
         m.skip_masked_tiles = 1 if skip else 0
         m.seg_tile_minmax = self.seg_mm.data_ptr() if self.seg_mm is not None else None
         m.seg_tiles = self.seg_tiles
+        if self.keep is not None:
+            m.keep = self.keep.data_ptr() + self.keep_row0 * self.keep_strides[2]
+            m.keep_stride_b, m.keep_stride_h, m.keep_stride_q, m.keep_stride_k = self.keep_strides
         return m
 
     def segments_meet(self, q_lo, q_hi, k_lo, k_hi):

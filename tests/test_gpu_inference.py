@@ -1,0 +1,96 @@
+"""Parity of ring_attention_inference (boolean-mask ring, ringattention_inference.py) on the HIP path
+with the CPU oracle.  Tolerances: fp32 max-abs 1e-4, bf16 2e-2, rel-L2 1e-2 (tests/util.assert_close)."""
+import pytest
+import torch
+
+import ringattention_amd as ra
+from oracle import ringattention_oracle as O
+from tests.util import assert_close, make_qkv
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _mask(shape, seed, p_keep=0.6, causal=False):
+    g = torch.Generator().manual_seed(seed)
+    m = torch.rand(shape, generator=g) < p_keep
+    if causal:
+        S = shape[-1]
+        m = m & torch.tril(torch.ones(S, S, dtype=torch.bool))
+    m[..., 0] = True
+    return m
+
+
+def _run(q, k, v, do, mask, n, f32_logits=True):
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention_inference(qd, kd, vd, mask.to(DEV), "sp", f32_logits)
+    out.backward(do.to(DEV))
+    return out.detach().cpu(), tuple(t.grad.cpu() for t in (qd, kd, vd))
+
+
+CASES = [
+    # B, S, H, D, n, mask shape kind, dtype
+    (2, 128, 2, 64, 1, "full", torch.float32),
+    (2, 128, 2, 64, 4, "full", torch.float32),
+    (1, 192, 3, 32, 2, "bcast_bh", torch.float32),
+    (2, 256, 2, 128, 2, "key_only", torch.float32),
+    (1, 256, 2, 128, 4, "per_head", torch.bfloat16),
+    (2, 512, 2, 128, 2, "full", torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_inference_matches_oracle(case):
+    B, S, H, D, n, kind, dtype = case
+    shape = {"full": (B, H, S, S), "bcast_bh": (1, 1, S, S), "key_only": (B, 1, 1, S), "per_head": (1, H, S, S)}[kind]
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=3, scale=D ** -0.25)
+    mask = _mask(shape, 11, causal=(kind == "bcast_bh"))
+    out, grads = _run(q, k, v, do, mask, n)
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+    ref_grads = O.ring_attention_inference_bwd(n, res, do)
+    assert_close(out, ref_out, dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, dtype, name)
+
+
+def test_inference_fully_masked_row_and_ring_invariance():
+    """A query row that attends to nothing gets the mean of V (equal finfo.min logits) and, as in the
+    reference's backward formula, uniform weights in the gradients; the ring size changes nothing."""
+    B, S, H, D = 1, 128, 2, 64
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=5)
+    mask = _mask((1, 1, S, S), 13)
+    mask[:, :, 7, :] = False
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, 4, True)
+    ref_grads = O.ring_attention_inference_bwd(4, res, do)
+    outs = {}
+    for n in (1, 4):
+        out, grads = _run(q, k, v, do, mask, n)
+        assert torch.allclose(out[:, 7], v.mean(dim=1), atol=1e-5)
+        assert_close(out, ref_out, torch.float32, "out")
+        for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+            assert_close(a, b, torch.float32, name)
+        outs[n] = out
+    assert (outs[1] - outs[4]).abs().max() < 1e-5
+
+
+def test_inference_causal_mask_equals_blockwise_ring_attention():
+    """The same causal problem through both entry points of the library."""
+    from tests.util import kwargs
+    B, S, H, D = 1, 512, 2, 128
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=6, scale=D ** -0.25)
+    mask = torch.tril(torch.ones(S, S, dtype=torch.bool)).reshape(1, 1, S, S)
+    with ra.ring_axis("sp", 2):
+        a = ra.ringattention_inference(q.to(DEV), k.to(DEV), v.to(DEV), mask.to(DEV), "sp", True)
+        b = ra.ringattention(q.to(DEV), k.to(DEV), v.to(DEV), None, None, None, axis_name="sp",
+                             float32_logits=True, blockwise_kwargs=kwargs(128, 128, 1))
+    assert_close(a.cpu(), b.cpu(), torch.bfloat16, "out")
+
+
+def test_inference_rejects_bad_mask_shapes():
+    q = torch.zeros(1, 128, 2, 64, device=DEV)
+    with ra.ring_axis("sp", 1):
+        with pytest.raises(ValueError):
+            ra.ringattention_inference(q, q, q, torch.ones(1, 1, 64, 128, dtype=torch.bool, device=DEV), "sp", True)
+        with pytest.raises(ValueError):
+            ra.ringattention_inference(q, q, q, torch.ones(128, 128, dtype=torch.bool, device=DEV), "sp", True)

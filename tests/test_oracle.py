@@ -335,3 +335,59 @@ def test_dropout_is_refused():
     kw.update(deterministic=False, attn_pdrop=0.1)
     with pytest.raises(NotImplementedError):
         O.ring_attention(q, k, v, None, None, None, 1, True, kw)
+
+
+# --------------------------------------------------------------------------- ring_attention_inference
+INFER_MASK_SHAPES = [("full", lambda B, H, S: (B, H, S, S)), ("bcast_bh", lambda B, H, S: (1, 1, S, S)),
+                     ("key_only", lambda B, H, S: (B, 1, 1, S)), ("per_head", lambda B, H, S: (1, H, S, S))]
+
+
+@pytest.mark.parametrize("name,shape_fn", INFER_MASK_SHAPES)
+@pytest.mark.parametrize("n", [1, 2, 4])
+def test_inference_ring_matches_dense_masked_softmax(name, shape_fn, n):
+    """ringattention_inference.py restated vs an un-chunked masked softmax and its autograd, float64."""
+    B, S, H, D = 2, 48, 3, 16
+    g0 = torch.Generator().manual_seed(7)
+    q, k, v, g = (torch.randn(B, S, H, D, dtype=torch.float64, generator=g0) for _ in range(4))
+    mask = torch.rand(shape_fn(B, H, S), generator=g0) > 0.4
+    mask[..., 0] = True                      # every row attends to something: the closed form has a gradient
+    out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True, compute_dtype=torch.float64)
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = O.dense_attention_inference(qq, kk, vv, mask)
+    assert (out - ref.detach()).abs().max() < 1e-12
+    ref.backward(g)
+    dq, dk, dv = O.ring_attention_inference_bwd(n, res, g)
+    for a, b in ((dq, qq.grad), (dk, kk.grad), (dv, vv.grad)):
+        assert (a - b).abs().max() < 1e-11
+
+
+def test_inference_row_without_attended_key_is_uniform():
+    """where(mask, w, finfo.min) leaves equal logits on a fully masked row: its output is the mean of V
+    over every key of the ring, whatever the ring size, and dv matches the uniform weights."""
+    B, S, H, D = 1, 32, 2, 8
+    g0 = torch.Generator().manual_seed(8)
+    q, k, v, g = (torch.randn(B, S, H, D, generator=g0) for _ in range(4))
+    mask = torch.rand(1, 1, S, S, generator=g0) > 0.5
+    mask[..., 0] = True
+    mask[:, :, 5, :] = False
+    for n in (1, 4):
+        out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+        assert torch.allclose(out[:, 5], v.mean(dim=1), atol=1e-6)
+        ref = O.dense_attention_inference(q, k, v, mask).float()
+        assert (out - ref).abs().max() < 1e-5
+        _dq, _dk, dv = O.ring_attention_inference_bwd(n, res, g)
+        vv = v.clone().double().requires_grad_(True)
+        O.dense_attention_inference(q, k, vv, mask).backward(g.double())
+        assert (dv - vv.grad.float()).abs().max() < 1e-5
+
+
+def test_inference_equals_ring_attention_with_causal_mask():
+    """A causal boolean mask reproduces the blockwise path (chunk sizes >= 2, so no diagonal tile is
+    dropped): two independently restated reference functions agree."""
+    B, S, H, D = 1, 64, 2, 16
+    g0 = torch.Generator().manual_seed(9)
+    q, k, v = (torch.randn(B, S, H, D, generator=g0) for _ in range(3))
+    mask = torch.tril(torch.ones(S, S, dtype=torch.bool)).reshape(1, 1, S, S)
+    a, _ = O.ring_attention_inference_fwd(q, k, v, mask, 2, True)
+    b = O.ring_attention(q, k, v, None, None, None, 2, True, kwargs(16, 16, 1))
+    assert (a - b).abs().max() < 1e-5
