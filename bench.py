@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ring-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|inference|copy]
 
 One step = one pass of the hot path over one batch of synthetic input already resident in HBM.
 Default workload ``attn32k`` is the configuration the headline metric is quoted on: blockwise
@@ -304,12 +304,52 @@ def bench_copy(args):
             "cpu_baseline": None}
 
 
+# --------------------------------------------------------------------------- boolean-mask ring (inference twin)
+def bench_inference(args):
+    """ring_attention_inference on a causal + key-padding boolean mask, forward + backward, bf16 inputs,
+    2 virtual shards: the MFMA kernels with the mask in packed form (ra_keep_pack, inside the timed step)."""
+    import torch
+    import ringattention_amd as ra
+    dev = "cuda:0"
+    B, H, D, n = 1, 32, 128, 2
+    S = args.seq_len or 32768
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda: (torch.randn(B, S, H, D, device=dev, generator=g) * D ** -0.5).to(torch.bfloat16)
+    q, k, v = mk().requires_grad_(True), mk().requires_grad_(True), mk().requires_grad_(True)
+    do = torch.randn(B, S, H, D, device=dev, generator=g).to(torch.bfloat16)
+    mask = torch.tril(torch.ones(S, S, dtype=torch.bool, device=dev))
+    mask[:, S - S // 16:] = False                      # the last sixteenth of the keys is padding
+    mask[:, 0] = True
+    mask = mask.reshape(1, 1, S, S)
+    pairs = float(mask.sum().item())
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        with ra.ring_axis("sp", n):
+            out = ra.ringattention_inference(q, k, v, mask, "sp", True)
+            out.backward(do)
+
+    ms = _time_steps(step, args.steps, args.warmup)
+    flops = 14.0 * D * pairs * B * H
+    value = flops / (ms * 1e-3) / 1e12
+    return {"metric": "inference_attn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s",
+            "ms_per_step": round(ms, 3), "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+            "config": {"workload": "inference", "B": B, "H": H, "S": S, "D": D, "virtual_ring": n,
+                       "mask": "causal and 1/16 key padding, boolean (1,1,S,S)",
+                       "flop_convention": "4*D fwd + 10*D bwd per attended (q,k) pair per head"},
+            "roofline": {"bound": "mfma", "kernel": "attn_fwd_pp_kernel + attn_bwd_dkv_ws_kernel + attn_bwd_dq_ws_kernel "
+                                                    "(packed boolean mask), whole step",
+                         "achieved": round(value, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None},
+            "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "copy"])
+    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -326,6 +366,8 @@ def main():
         r = bench_decode(args)
     elif args.workload == "copy":
         r = bench_copy(args)
+    elif args.workload == "inference":
+        r = bench_inference(args)
     else:
         r = bench_ffn(args)
     line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,

@@ -75,6 +75,17 @@ typedef struct ra_mask {
   int64_t keep_stride_h;
   int64_t keep_stride_q;
   int64_t keep_stride_k;
+  /* Packed forms of the same mask from ra_keep_pack, which let the MFMA kernels take it (all three null:
+     generic kernels only).  They cover the GLOBAL mask (keep_q_total x keep_k_total, both multiples of 64);
+     keep_q0 is the global row of the call's local query row 0 (a multiple of 64). */
+  const uint64_t* keep_bits_k;   /* [b][h][k_total/64][q_total]: bit i = keep[q][64 kt + i] */
+  const uint64_t* keep_bits_q;   /* [b][h][q_total/64][k_total]: bit i = keep[64 qt + i][k] */
+  const uint8_t* keep_summary;   /* [b][h][q_total/64][k_total/64]: 0 none kept, 1 mixed, 2 all kept */
+  int64_t keep_pack_stride_b;    /* of both bit arrays, in 64-bit words; 0 broadcasts */
+  int64_t keep_pack_stride_h;
+  int64_t keep_sum_stride_b;     /* of keep_summary, in bytes; 0 broadcasts */
+  int64_t keep_sum_stride_h;
+  int32_t keep_q_total, keep_k_total, keep_q0;
 } ra_mask;
 
 /* _blockwise_attention_fwd (ringattention_jax.py:99-179): one ring step on one device.
@@ -116,6 +127,14 @@ enum { RA_SEG_TILE = 64 };
  * only feeds the tile-skipping of the kernels. */
 int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int32_t Bseg, int32_t seg_len,
                            int32_t* out, ra_stream_t stream);
+
+/* Packs a boolean mask (nonzero = attend; byte strides, 0 broadcasts an axis) of Q x K positions, both
+ * multiples of 64, into the three arrays ra_mask.keep_bits_k / keep_bits_q / keep_summary describe, for Bm x Hm
+ * (batch, head) planes.  No counterpart in the reference (ringattention_inference.py:22 applies the mask
+ * element by element); this only lets the MFMA kernels read 64 mask bits per load and skip uniform tiles. */
+int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_t stride_q, int64_t stride_k,
+                 int32_t Bm, int32_t Hm, int32_t Q, int32_t K, uint64_t* bits_k, uint64_t* bits_q,
+                 uint8_t* summary, ra_stream_t stream);
 
 /* Carry initialisation (ringattention_jax.py:22-23,:49): numerator = 0, denominator = 0, max = -inf. */
 int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s,

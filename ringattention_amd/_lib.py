@@ -27,6 +27,9 @@ class RaMask(C.Structure):
         ("skip_masked_tiles", i32), ("seg_tile_minmax", vp), ("seg_tiles", i32),
         ("keep", vp), ("keep_stride_b", i64), ("keep_stride_h", i64), ("keep_stride_q", i64),
         ("keep_stride_k", i64),
+        ("keep_bits_k", vp), ("keep_bits_q", vp), ("keep_summary", vp),
+        ("keep_pack_stride_b", i64), ("keep_pack_stride_h", i64), ("keep_sum_stride_b", i64),
+        ("keep_sum_stride_h", i64), ("keep_q_total", i32), ("keep_k_total", i32), ("keep_q0", i32),
     ]
 
 
@@ -74,6 +77,7 @@ class RaSwigluParams(C.Structure):
 # every symbol include/ringattn_hip.h declares: (name, restype, argtypes)
 SYMBOLS = {
     "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
+    "ra_keep_pack": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]),
     "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),

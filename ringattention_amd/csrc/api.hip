@@ -27,6 +27,7 @@ int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, voi
 int bwd_delta(const void*, const void*, int, int64_t, int64_t, float*, int64_t, int64_t, int, int, int, int,
               hipStream_t);
 int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
+int keep_pack(const uint8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, uint64_t*, uint64_t*, uint8_t*, hipStream_t);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
@@ -52,6 +53,14 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
   if (m.seg_tile_minmax)
     RA_REQUIRE(m.segment_ids && m.seg_tiles == (m.seg_len + RA_SEG_TILE - 1) / RA_SEG_TILE, RA_ERR_INVALID,
                "%s: seg_tile_minmax needs segment_ids and seg_tiles == ceil(seg_len / %d)", who, (int)RA_SEG_TILE);
+  if (m.keep_bits_k || m.keep_bits_q || m.keep_summary) {
+    RA_REQUIRE(m.keep && m.keep_bits_k && m.keep_bits_q && m.keep_summary, RA_ERR_INVALID,
+               "%s: the packed keep mask needs keep, keep_bits_k, keep_bits_q and keep_summary together", who);
+    RA_REQUIRE(m.keep_q_total > 0 && m.keep_k_total > 0 && m.keep_q_total % 64 == 0 && m.keep_k_total % 64 == 0 &&
+                   m.keep_q0 >= 0 && m.keep_q0 % 64 == 0 && m.keep_q0 + Sq <= m.keep_q_total &&
+                   (long long)m.k_chunk_idx_start * m.key_chunk_size + Skv <= m.keep_k_total,
+               RA_ERR_INVALID, "%s: packed keep mask does not cover the rows / keys of the call", who);
+  }
   RA_REQUIRE((long long)m.q_chunk_idx_start * m.query_chunk_size + Sq < (1LL << 31) - 4096 &&
                  (long long)m.k_chunk_idx_start * m.key_chunk_size + Skv < (1LL << 31) - 4096,
              RA_ERR_UNSUPPORTED, "%s: global positions must stay below 2^31", who);
@@ -81,6 +90,17 @@ int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int
   RA_REQUIRE(segment_ids && out, RA_ERR_INVALID, "segment_tile_ranges: null pointer");
   RA_REQUIRE(Bseg > 0 && Bseg <= 65535 && seg_len > 0, RA_ERR_INVALID, "segment_tile_ranges: bad shape");
   return seg_tile_ranges(segment_ids, seg_stride_b, Bseg, seg_len, out, (hipStream_t)stream);
+}
+
+int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_t stride_q, int64_t stride_k,
+                 int32_t Bm, int32_t Hm, int32_t Q, int32_t K, uint64_t* bits_k, uint64_t* bits_q,
+                 uint8_t* summary, ra_stream_t stream) {
+  RA_REQUIRE(keep && bits_k && bits_q && summary, RA_ERR_INVALID, "keep_pack: null pointer");
+  RA_REQUIRE(Bm > 0 && Hm > 0 && (long long)Bm * Hm <= 65535, RA_ERR_INVALID, "keep_pack: bad plane count");
+  RA_REQUIRE(Q > 0 && K > 0 && Q % 64 == 0 && K % 64 == 0 && Q / 64 <= 65535, RA_ERR_UNSUPPORTED,
+             "keep_pack: Q and K must be positive multiples of 64 (got %d, %d)", Q, K);
+  return keep_pack(keep, stride_b, stride_h, stride_q, stride_k, Bm, Hm, Q, K, bits_k, bits_q, summary,
+                   (hipStream_t)stream);
 }
 
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {

@@ -375,6 +375,42 @@ int seg_tile_ranges(const int32_t* seg, int64_t seg_sb, int Bseg, int seg_len, i
   return RA_OK;
 }
 
+// One 64 x 64 tile of the boolean mask per workgroup of 64 threads: thread i writes the word of query row i
+// (bits over the tile's keys) and the word of key column i (bits over the tile's query rows).
+__global__ __launch_bounds__(64) void keep_pack_kernel(const uint8_t* keep, int64_t sb, int64_t sh, int64_t sq,
+                                                       int64_t sk, int Hm, int Q, int K, uint64_t* bits_k,
+                                                       uint64_t* bits_q, uint8_t* summary) {
+  __shared__ uint8_t tile[64][65];
+  __shared__ int cnt;
+  const int kt = blockIdx.x, qt = blockIdx.y, plane = blockIdx.z;
+  const int b = plane / Hm, h = plane % Hm;
+  const int i = threadIdx.x;
+  if (i == 0) cnt = 0;
+  const uint8_t* base = keep + sb * b + sh * h;
+  for (int r = 0; r < 64; r++) tile[r][i] = base[(int64_t)(qt * 64 + r) * sq + (int64_t)(kt * 64 + i) * sk] != 0;
+  __syncthreads();
+  uint64_t wrow = 0, wcol = 0;
+  for (int j = 0; j < 64; j++) {
+    wrow |= (uint64_t)tile[i][j] << j;
+    wcol |= (uint64_t)tile[j][i] << j;
+  }
+  atomicAdd(&cnt, __popcll(wrow));
+  __syncthreads();
+  const int64_t words = (int64_t)Q * K / 64;
+  bits_k[plane * words + (int64_t)kt * Q + qt * 64 + i] = wrow;
+  bits_q[plane * words + (int64_t)qt * K + kt * 64 + i] = wcol;
+  if (i == 0)
+    summary[(int64_t)plane * (Q / 64) * (K / 64) + (int64_t)qt * (K / 64) + kt] = cnt == 0 ? 0 : (cnt == 4096 ? 2 : 1);
+}
+
+int keep_pack(const uint8_t* keep, int64_t sb, int64_t sh, int64_t sq, int64_t sk, int Bm, int Hm, int Q, int K,
+              uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, hipStream_t s) {
+  dim3 grid(K / 64, Q / 64, Bm * Hm);
+  keep_pack_kernel<<<grid, 64, 0, s>>>(keep, sb, sh, sq, sk, Hm, Q, K, bits_k, bits_q, summary);
+  RA_CHECK_LAUNCH("keep_pack");
+  return RA_OK;
+}
+
 // ------------------------------------------------------------------ host-side launchers
 static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
   GenericArgs a{};

@@ -98,6 +98,51 @@ __device__ __forceinline__ void seg_rows_range(const MaskView& mv, int b, int g0
   }
 }
 
+// ---- boolean keep mask in packed form (ra_keep_pack): 64-bit words and a per-64x64-tile summary
+// (0 none kept, 1 mixed, 2 all kept).  Hull of the key tiles [gkt0, gkt0 + n) that hold a kept pair for
+// any of the nrows summary rows starting at qt64 (every thread of the workgroup must call it).
+__device__ __forceinline__ void keep_ktile_hull(const MaskView& mv, int b, int h, int qt64, int nrows, int gkt0, int n,
+                                                int* hull2, int tid, int nthreads, int& first, int& last) {
+  if (tid == 0) { hull2[0] = n; hull2[1] = 0; }
+  __syncthreads();
+  const int KT = mv.keep_K / 64;
+  const uint8_t* sm = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh + (int64_t)qt64 * KT + gkt0;
+  for (int t = tid; t < n; t += nthreads) {
+    int any = 0;
+    for (int r = 0; r < nrows; r++) any |= sm[(int64_t)r * KT + t];
+    if (any) { atomicMin(&hull2[0], t); atomicMax(&hull2[1], t + 1); }
+  }
+  __syncthreads();
+  first = hull2[0]; last = hull2[1];
+  if (last < first) { first = 0; last = 0; }
+}
+// the same over the query tiles [gqt0, gqt0 + n) for the ncols summary columns starting at kt64
+__device__ __forceinline__ void keep_qtile_hull(const MaskView& mv, int b, int h, int kt64, int ncols, int gqt0, int n,
+                                                int* hull2, int tid, int nthreads, int& first, int& last) {
+  if (tid == 0) { hull2[0] = n; hull2[1] = 0; }
+  __syncthreads();
+  const int KT = mv.keep_K / 64;
+  const uint8_t* sm = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh + (int64_t)gqt0 * KT + kt64;
+  for (int t = tid; t < n; t += nthreads) {
+    int any = 0;
+    for (int cidx = 0; cidx < ncols; cidx++) any |= sm[(int64_t)t * KT + cidx];
+    if (any) { atomicMin(&hull2[0], t); atomicMax(&hull2[1], t + 1); }
+  }
+  __syncthreads();
+  first = hull2[0]; last = hull2[1];
+  if (last < first) { first = 0; last = 0; }
+}
+// number of leading tiles of a summary row (or column, with the given stride) that are "all kept"
+__device__ __forceinline__ int keep_leading_full(const uint8_t* sm, int64_t stride, int n, int lane) {
+  for (int base = 0; base < n; base += 64) {
+    const int t = base + lane;
+    const bool bad = t < n && sm[(int64_t)t * stride] != 2;
+    const unsigned long long m = __builtin_amdgcn_ballot_w64(bad);
+    if (m) return base + __builtin_ctzll(m);
+  }
+  return n;
+}
+
 // Staging helpers shared by the kernels below.  They expect in scope: tid, s_off (this thread's
 // swizzled element offset inside a 16-row slab), row16 (global element stride of 16 rows).
 #define RA_LOAD_TILE(REGS, BASE, STRIDE, J, ROWS)                                                       \
@@ -510,7 +555,7 @@ __device__ long long g_trace[8][4096];
 constexpr int PP_DEPTH = 1;       // LDS fragment prefetch distance of the matrix phase, in steps of 4 MFMAs
 constexpr bool PP_PRIO = false;  // raise the wave priority during the matrix phase
 
-template <bool HAS_SEG, bool HAS_BIAS>
+template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
   __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
@@ -556,7 +601,29 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
     ntiles = t_last - t_first;
     ntiles_grp = min(max(ntiles_grp - t_first, 0), ntiles);
   }
+  // key tiles outside the hull of those with a kept pair for these 256 rows are skipped
+  if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {
+    __shared__ int khull2[2];
+    int t_first, t_last;
+    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, PBM / 64, (gk0_shard + k_base) / 64, ntiles, khull2, tid, 512,
+                    t_first, t_last);
+    k_base += t_first * FBN;
+    ntiles = t_last - t_first;
+    ntiles_grp = min(max(ntiles_grp - t_first, 0), ntiles);
+  }
   const int gk0 = gk0_shard + k_base;                  // global position of the first key processed
+  // packed keep mask: this lane's word per key tile, this wavefront's summary byte per key tile
+  const uint64_t* kw_ptr = nullptr;
+  const uint8_t* ks_ptr = nullptr;
+  uint64_t kw_cur = 0, kw_nxt = 0;
+  int ks_cur = 2, ks_nxt = 2;
+  if (HAS_KEEP) {
+    kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
+             mv.keep_q0 + qrow;
+    ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
+             (int64_t)((mv.keep_q0 + qg0 + w4 * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
+    if (ntiles > 0) { kw_nxt = kw_ptr[0]; ks_nxt = ks_ptr[0]; }
+  }
 
   const int gq = gq_wg + grp * 128 + w4 * 32 + lo;
   const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
@@ -687,11 +754,16 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   {                                                                                                     \
     const int t_ = (T);                                                                                 \
     const int gk_tile_ = gk0 + t_ * FBN;                                                                \
-    if (t_ >= ntiles_grp) {                                                                             \
+    if (HAS_KEEP) {                       /* this tile's word and summary; request the next tile's */   \
+      kw_cur = kw_nxt >> (4 * hi); ks_cur = ks_nxt;                                                     \
+      const int tn_ = min(t_ + 1, ntiles - 1);                                                          \
+      kw_nxt = kw_ptr[(int64_t)tn_ * mv.keep_Q]; ks_nxt = ks_ptr[tn_];                                  \
+    }                                                                                                   \
+    if (t_ >= ntiles_grp || (HAS_KEEP && ks_cur == 0 && mv.skip_tiles)) {                               \
       _Pragma("unroll") for (int x = 0; x < 8; x++) {                                                   \
         pf[0][0][x] = (__bf16)0.f; pf[0][1][x] = (__bf16)0.f; pf[1][0][x] = (__bf16)0.f; pf[1][1][x] = (__bf16)0.f; \
       }                                                                                                 \
-    } else if (!(HAS_SEG || HAS_BIAS) && (gk_tile_ + FBN - 1 < klim_wave)) {                            \
+    } else if (!(HAS_SEG || HAS_BIAS) && (gk_tile_ + FBN - 1 < klim_wave) && (!HAS_KEEP || ks_cur == 2)) { \
       float mxv_ = s[0][0];                                                                             \
       _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
         _Pragma("unroll") for (int r = 0; r < 16; r++) mxv_ = fmaxf(mxv_, s[blk][r]);                   \
@@ -721,6 +793,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
           if (HAS_BIAS) x_ += bias_ks[t_ & 3][kr_];                                                     \
           bool masked_ = (gk_tile_ + kr_ >= klim);                                                      \
           if (HAS_SEG) masked_ = masked_ || (seg_ks[t_ & 3][kr_] != seg_q);                             \
+          if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> (blk * 32 + (r >> 2) * 8 + (r & 3))) & 1);    \
           x_ = masked_ ? kMask2 : x_;                                                                   \
           s[blk][r] = x_;                                                                               \
           mxv_ = fmaxf(mxv_, x_);                                                                       \
@@ -1291,7 +1364,7 @@ constexpr int WS_PSTR = 40;                 // P / dS row stride in elements (co
 constexpr int WS_PD = 32 * WS_PSTR;         // one 32 x 32 block
 constexpr int WS_TILE = KBM * TROW;
 
-template <bool HAS_SEG, bool HAS_BIAS>
+template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t Qs[3 * WS_TILE];
   __shared__ __attribute__((aligned(16))) uint16_t Gs[3 * WS_TILE];
@@ -1346,6 +1419,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     int slo, shi, t_first, t_last;
     seg_rows_range(mv, b, gk0, KBN, slo, shi);
     seg_tile_hull(mv, b, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, slo, shi, hull2, tid, 512, t_first, t_last);
+    qt_end = qt_first + t_last;
+    qt_first += t_first;
+  }
+  if (HAS_KEEP && mv.skip_tiles && qt_first < qt_end) {
+    __shared__ int khull2[2];
+    int t_first, t_last;
+    keep_qtile_hull(mv, b, h, gk0 / 64, KBN / 64, mv.keep_q0 / 64 + qt_first, qt_end - qt_first, khull2, tid, 512,
+                    t_first, t_last);
     qt_end = qt_first + t_last;
     qt_first += t_first;
   }
@@ -1475,6 +1556,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       if (HAS_BIAS) x += bias2;                                                                         \
       bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
       if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
+      if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                   \
       x = masked ? kMask2 : x;                                                                          \
       const float p = fast_exp2(x - vm2[e]) * vrd[e];                                    /* :226 */     \
       p4[e] = (__bf16)p;                                                                                \
@@ -1515,12 +1597,29 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       RA_WS_AMFMA(g, qa_, ga_, s_a, dp_a);
     }
 
+    // packed keep mask: this lane's word (bits over the 64 rows of a query tile) and this pair's summary byte
+    const uint64_t* kw_ptr = nullptr;
+    const uint8_t* ks_ptr = nullptr;
+    uint64_t kw_cur = 0, kw_nxt = 0;
+    int ks_cur = 2, ks_nxt = 2;
+    if (HAS_KEEP) {
+      kw_ptr = mv.kbits_q + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
+               (int64_t)(mv.keep_q0 / 64 + qt_first) * mv.keep_K + gk;
+      ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
+               (int64_t)(mv.keep_q0 / 64 + qt_first) * (mv.keep_K / 64) + (gk0 + pair * 32) / 64;
+      kw_nxt = kw_ptr[0]; ks_nxt = ks_ptr[0];
+    }
     int cur = 0;
     for (int t = 0; t < ntq; t++) {
       const int nxt = cur == 2 ? 0 : cur + 1, prv = cur == 0 ? 2 : cur - 1;
       const int gq_tile = gq_base + (qt_first + t) * KBM;
+      if (HAS_KEEP) {                      // this tile's word and summary; request the next tile's
+        kw_cur = kw_nxt >> (4 * hi); ks_cur = ks_nxt;
+        const int tn = min(t + 1, ntq - 1);
+        kw_nxt = kw_ptr[(int64_t)tn * mv.keep_K]; ks_nxt = ks_ptr[(int64_t)tn * (mv.keep_K / 64)];
+      }
       // step 2t: vector work of block 0 of tile t, products of block 1
-      if (HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave)) {
+      if (HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
         RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, true);
       } else {
         RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, false);
@@ -1530,7 +1629,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       // block 0 of tile t + 1 (the last tile computes a block that is never used)
       RA_WS_STORE(prv);
       RA_WS_LOAD(t + 3);
-      if (HAS_SEG || HAS_BIAS || (gq_tile + 32 < qlim_wave)) {
+      if (HAS_SEG || HAS_BIAS || (gq_tile + 32 < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
         RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, true);
       } else {
         RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, false);
@@ -1652,7 +1751,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #ifndef WS_DQ_VALU_PER_MFMA
 #define WS_DQ_VALU_PER_MFMA 5
 #endif
-template <bool HAS_SEG, bool HAS_BIAS>
+template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t Ks[3 * WS_TILE];
   __shared__ __attribute__((aligned(16))) uint16_t Vs[3 * WS_TILE];
@@ -1693,6 +1792,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     seg_rows_range(mv, b, gq0, FBM, slo, shi);
     seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
     k_base = t_first * FBN;
+    ntiles = t_last - t_first;
+  }
+  if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {
+    __shared__ int khull2[2];
+    int t_first, t_last;
+    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, FBM / 64, (gk0_shard + k_base) / 64, ntiles, khull2, tid, 512,
+                    t_first, t_last);
+    k_base += t_first * FBN;
     ntiles = t_last - t_first;
   }
   if (ntiles == 0) return;     // nothing to add to dq
@@ -1829,6 +1936,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
         if (HAS_BIAS) x += bias_ks[BUF][kr_];                                                           \
         bool masked = (gk_tile + kr_ >= klim);                                                          \
         if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
+        if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                 \
         x = masked ? kMask2 : x;                                                                        \
         p = fast_exp2(x - m2) * rden;                                                    /* :226 */     \
       }                                                                                                 \
@@ -1874,12 +1982,27 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     // (which also takes every tile when segment ids or a bias are present).
     int t_plain = 0;
     if (!(HAS_SEG || HAS_BIAS)) t_plain = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
+    // packed keep mask: the tiles whose 64 x 64 summary says "all kept" for these rows need no masking either
+    const uint64_t* kw_ptr = nullptr;
+    uint64_t kw_cur = 0, kw_nxt = 0;
+    if (HAS_KEEP) {
+      const uint8_t* ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
+                              (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
+      t_plain = __builtin_amdgcn_readfirstlane(min(t_plain, keep_leading_full(ks_ptr, 1, ntiles, lane)));
+      kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
+               mv.keep_q0 + qrow;
+      kw_nxt = kw_ptr[(int64_t)min(t_plain, ntiles - 1) * mv.keep_Q];
+    }
     int cur = 0;
 #define RA_WS_TILE(MASKED)                                                                              \
   {                                                                                                     \
     const int nxt = cur == 2 ? 0 : cur + 1;                                                             \
     const int gk_tile = gk0 + t * FBN;                                                                  \
     (void)gk_tile;                                                                                      \
+    if (HAS_KEEP && (MASKED)) {        /* this tile's word; request the next tile's */                  \
+      kw_cur = kw_nxt >> (4 * hi);                                                                      \
+      kw_nxt = kw_ptr[(int64_t)min(t + 1, ntiles - 1) * mv.keep_Q];                                     \
+    }                                                                                                   \
     /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
     RA_TRACE_MARK();                                                                                    \
     RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, nxt, 0, 0, MASKED);                             \
@@ -1996,10 +2119,16 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
+// a boolean keep mask is taken in packed form only, alone (no bias, no segment ids), by the 8-wave kernels
+static bool keep_ok(const ra_mask& m, bool shape_ok) {
+  if (!m.keep) return true;
+  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids && shape_ok;
+}
+
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
   const ra_mask& m = p->mask;
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
-         m.keep == nullptr && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
+         keep_ok(m, m.query_chunk_size % PBM == 0) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
          aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator);
 }
@@ -2015,11 +2144,13 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
-  if (p->mask.query_chunk_size % PBM == 0 && !getenv("RA_FWD_NO_PINGPONG")) {
+  const bool keep = p->mask.keep != nullptr;      // packed form checked by attn_fwd_mfma_supported
+  if (p->mask.query_chunk_size % PBM == 0 && (keep || !getenv("RA_FWD_NO_PINGPONG"))) {
     const long long nwg2 = (long long)(p->Sq / PBM) * p->H * p->B;
     RA_REQUIRE(nwg2 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
     dim3 grid2((unsigned)nwg2), block2(512);
-    if (seg && bias) attn_fwd_pp_kernel<true, true><<<grid2, block2, 0, s>>>(a);
+    if (keep) attn_fwd_pp_kernel<false, false, true><<<grid2, block2, 0, s>>>(a);
+    else if (seg && bias) attn_fwd_pp_kernel<true, true><<<grid2, block2, 0, s>>>(a);
     else if (seg) attn_fwd_pp_kernel<true, false><<<grid2, block2, 0, s>>>(a);
     else if (bias) attn_fwd_pp_kernel<false, true><<<grid2, block2, 0, s>>>(a);
     else attn_fwd_pp_kernel<false, false><<<grid2, block2, 0, s>>>(a);
@@ -2040,7 +2171,7 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
   const ra_mask& m = p->mask;
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % KBN == 0 &&
-         m.keep == nullptr && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
+         keep_ok(m, true) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0 &&
          p->dkv_stride_s % 4 == 0 && p->dkv_stride_b % 4 == 0 && aligned16(p->q) && aligned16(p->k) &&
          aligned16(p->v) && aligned16(p->g) && aligned16(p->dq) && aligned16(p->dk) && aligned16(p->dv);
@@ -2077,7 +2208,10 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
       attn_bwd_dq_mfma_kernel<SEG, BIAS><<<gq, block, 0, s>>>(a);                        \
     }                                                                                    \
   } while (0)
-  if (seg && bias) RA_LAUNCH_BWD(true, true);
+  if (p->mask.keep) {        // packed boolean mask: the wave-specialised kernels only
+    if (do_dkv) attn_bwd_dkv_ws_kernel<false, false, true><<<dim3((gk.x + 7) / 8 * 8), dim3(512), 0, s>>>(a);
+    if (do_dq) attn_bwd_dq_ws_kernel<false, false, true><<<dim3((gq.x + 7) / 8 * 8), dim3(512), 0, s>>>(a);
+  } else if (seg && bias) RA_LAUNCH_BWD(true, true);
   else if (seg) RA_LAUNCH_BWD(true, false);
   else if (bias) RA_LAUNCH_BWD(false, true);
   else RA_LAUNCH_BWD(false, false);

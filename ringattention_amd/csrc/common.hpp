@@ -63,6 +63,11 @@ struct MaskView {
   int seg_tiles;
   const uint8_t* keep;     // boolean mask (local query row, global key), or null
   int64_t keep_sb, keep_sh, keep_sq, keep_sk;
+  const uint64_t* kbits_k;   // packed mask, see ra_keep_pack; all null unless the MFMA kernels take the mask
+  const uint64_t* kbits_q;
+  const uint8_t* ksum;
+  int64_t kpack_sb, kpack_sh, ksum_sb, ksum_sh;
+  int keep_Q, keep_K, keep_q0;
 
   __host__ __device__ static MaskView make(const ra_mask& m, int q_chunk_idx_start) {
     MaskView v;
@@ -77,6 +82,10 @@ struct MaskView {
     v.seg_mm = m.seg_tile_minmax; v.seg_tiles = m.seg_tiles;
     v.keep = m.keep; v.keep_sb = m.keep_stride_b; v.keep_sh = m.keep_stride_h;
     v.keep_sq = m.keep_stride_q; v.keep_sk = m.keep_stride_k;
+    v.kbits_k = m.keep_bits_k; v.kbits_q = m.keep_bits_q; v.ksum = m.keep_summary;
+    v.kpack_sb = m.keep_pack_stride_b; v.kpack_sh = m.keep_pack_stride_h;
+    v.ksum_sb = m.keep_sum_stride_b; v.ksum_sh = m.keep_sum_stride_h;
+    v.keep_Q = m.keep_q_total; v.keep_K = m.keep_k_total; v.keep_q0 = m.keep_q0;
     return v;
   }
 

@@ -1,6 +1,7 @@
 """ring_attention_inference (ringattention/ringattention_inference.py:8-73): the ring with a boolean
-attention mask and no chunking inside a ring step, over the fp32 vector-ALU kernels of
-libringattn_hip.so (the MFMA kernels take no per-pair mask operand)."""
+attention mask and no chunking inside a ring step.  bf16 inputs with head size 128 and shard lengths that
+are multiples of 256 run on the MFMA kernels, which read the mask in a packed form (ra_keep_pack);
+anything else runs on the fp32 vector-ALU kernels."""
 import torch
 
 from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, _blockwise_attention_fwd,
@@ -11,7 +12,7 @@ def _inference_cfg(q, q_len, kv_len, float32_logits):
     # one "chunk" per ring step (:21 is a single einsum over the shard); finfo.min of the logits' dtype (:22)
     logits_dtype = torch.float32 if (float32_logits or q.dtype == torch.float32) else q.dtype
     return _Config(dict(causal_block_size=None, query_chunk_size=q_len, key_chunk_size=kv_len, deterministic=True,
-                        attn_pdrop=0.0, dtype=logits_dtype, impl="generic", skip_masked_tiles=False))
+                        attn_pdrop=0.0, dtype=logits_dtype, impl="auto", skip_masked_tiles=False))
 
 
 def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
@@ -28,7 +29,12 @@ def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
         raise ValueError("attn_mask must be (B|1, H|1, Q|1, K) with Q = %d and K = %d" % (q_total, kv_total))
     cfg = _inference_cfg(q, q_len, kv_len, float32_logits)
     mi = _MaskInputs(cfg, None, None, None, B, q.device, kv_total)
-    mi.set_keep(attn_mask, q.device)
+    mi.set_keep(attn_mask, q.device, q_total, kv_total)
+    if q_len % 64 or kv_len % 64:
+        mi.keep_packed = None                        # shards not aligned to the 64 x 64 packing: generic kernels
+    # tiles without a kept pair may be skipped unless some row attends to nothing at all (its logits stay
+    # equal at finfo.min and its weights uniform, ringattention_inference.py:22-24)
+    cfg.skip_masked_tiles = not mi.keep_has_empty_row
     num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)   # :13
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)      # :14
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)       # :31

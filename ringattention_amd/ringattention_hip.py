@@ -184,13 +184,29 @@ class _MaskInputs:
             else:
                 self.cache_idx_host = int(cache_idx)
 
-    def set_keep(self, attn_mask, device):
-        """attn_mask (B|1, H|1, Q|1, K_total), nonzero = attend (ringattention_inference.py:19-22)."""
+    def set_keep(self, attn_mask, device, q_total, k_total):
+        """attn_mask (B|1, H|1, Q|1, K_total), nonzero = attend (ringattention_inference.py:19-22).
+        When both global lengths divide by 64 the mask is also packed into 64-bit words and a per-tile
+        summary (ra_keep_pack), the form the MFMA kernels read."""
         if attn_mask.dim() != 4:
             raise ValueError("attn_mask must be 4-D (B, H, Q, K)")
         m = (attn_mask.detach().to(device=device) != 0).to(torch.uint8).contiguous()
         self.keep = m
         self.keep_strides = tuple(0 if m.shape[i] == 1 else m.stride(i) for i in range(4))
+        # a query row with no attended key keeps equal finfo.min logits (uniform weights): kernels must not
+        # skip its fully masked tiles
+        self.keep_has_empty_row = bool((m.amax(dim=3) == 0).any().item())
+        self.keep_packed = None
+        if q_total % 64 == 0 and k_total % 64 == 0:
+            bm, hm = m.shape[0], m.shape[1]
+            words = q_total * k_total // 64
+            bits_k = torch.empty((bm, hm, words), dtype=torch.int64, device=device)
+            bits_q = torch.empty((bm, hm, words), dtype=torch.int64, device=device)
+            summ = torch.empty((bm, hm, (q_total // 64) * (k_total // 64)), dtype=torch.uint8, device=device)
+            L.check(L.load().ra_keep_pack(m.data_ptr(), m.stride(0), m.stride(1), self.keep_strides[2], m.stride(3),
+                                          bm, hm, q_total, k_total, bits_k.data_ptr(), bits_q.data_ptr(),
+                                          summ.data_ptr(), _stream()), "ra_keep_pack")
+            self.keep_packed = (bits_k, bits_q, summ, q_total, k_total)
 
     def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip):
         m = L.RaMask()
@@ -212,6 +228,14 @@ class _MaskInputs:
         if self.keep is not None:
             m.keep = self.keep.data_ptr() + self.keep_row0 * self.keep_strides[2]
             m.keep_stride_b, m.keep_stride_h, m.keep_stride_q, m.keep_stride_k = self.keep_strides
+            if self.keep_packed is not None:
+                bits_k, bits_q, summ, q_total, k_total = self.keep_packed
+                m.keep_bits_k, m.keep_bits_q, m.keep_summary = bits_k.data_ptr(), bits_q.data_ptr(), summ.data_ptr()
+                m.keep_pack_stride_b = 0 if bits_k.shape[0] == 1 else bits_k.stride(0)
+                m.keep_pack_stride_h = 0 if bits_k.shape[1] == 1 else bits_k.stride(1)
+                m.keep_sum_stride_b = 0 if summ.shape[0] == 1 else summ.stride(0)
+                m.keep_sum_stride_h = 0 if summ.shape[1] == 1 else summ.stride(1)
+                m.keep_q_total, m.keep_k_total, m.keep_q0 = q_total, k_total, self.keep_row0
         return m
 
     def segments_meet(self, q_lo, q_hi, k_lo, k_hi):

@@ -94,3 +94,88 @@ def test_inference_rejects_bad_mask_shapes():
             ra.ringattention_inference(q, q, q, torch.ones(1, 1, 64, 128, dtype=torch.bool, device=DEV), "sp", True)
         with pytest.raises(ValueError):
             ra.ringattention_inference(q, q, q, torch.ones(128, 128, dtype=torch.bool, device=DEV), "sp", True)
+
+
+def _structured_mask(B, H, S, kind, seed):
+    """Masks with whole tiles kept / dropped (what the packed summary shortcuts) plus ragged edges."""
+    g = torch.Generator().manual_seed(seed)
+    causal = torch.tril(torch.ones(S, S, dtype=torch.bool))
+    if kind == "causal":
+        return causal.reshape(1, 1, S, S).clone()
+    if kind == "causal_padding":
+        m = causal.reshape(1, 1, S, S).repeat(B, 1, 1, 1)
+        for b in range(B):
+            m[b, :, :, S - 37 * (b + 1):] = False
+        m[..., 0] = True
+        return m
+    if kind == "band_per_head":
+        idx = torch.arange(S)
+        m = torch.stack([(idx[:, None] - idx[None, :]).abs() <= 100 * (h + 1) for h in range(H)]).reshape(1, H, S, S)
+        return m & (torch.rand(1, H, S, S, generator=g) < 0.97) | torch.eye(S, dtype=torch.bool)
+    if kind == "key_only":
+        m = torch.rand(B, 1, 1, S, generator=g) < 0.7
+        m[..., 0] = True
+        return m
+    raise ValueError(kind)
+
+
+MFMA_CASES = [
+    # B, S, H, n, mask kind   (bf16, D = 128, shards of a multiple of 256 rows: the MFMA kernels run)
+    (1, 512, 2, 1, "causal"),
+    (1, 1024, 2, 2, "causal"),
+    (2, 1024, 2, 2, "causal_padding"),
+    (1, 1024, 3, 4, "band_per_head"),
+    (2, 512, 2, 2, "key_only"),
+]
+
+
+@pytest.mark.parametrize("case", MFMA_CASES)
+def test_inference_mfma_path_matches_oracle(case):
+    B, S, H, n, kind = case
+    D = 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=D ** -0.25)
+    mask = _structured_mask(B, H, S, kind, 22)
+    out, grads = _run(q, k, v, do, mask, n)
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+    ref_grads = O.ring_attention_inference_bwd(n, res, do)
+    assert_close(out, ref_out, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, torch.bfloat16, name)
+
+
+def test_inference_mfma_path_with_a_row_that_attends_to_nothing():
+    """Tile skipping is switched off by the host when a row has no attended key: that row must come out
+    as the mean of V on the MFMA kernels too."""
+    B, S, H, D, n = 1, 512, 2, 128, 2
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=23, scale=D ** -0.25)
+    mask = _structured_mask(B, H, S, "causal", 24)
+    mask[:, :, 300, :] = False
+    out, grads = _run(q, k, v, do, mask, n)
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+    ref_grads = O.ring_attention_inference_bwd(n, res, do)
+    assert torch.allclose(out[:, 300].float(), v.float().mean(dim=1), atol=2e-2)
+    assert_close(out, ref_out, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, torch.bfloat16, name)
+
+
+def test_inference_mfma_and_generic_kernels_agree():
+    """Same call with and without the packed mask (the latter forces the generic kernels)."""
+    from ringattention_amd import inference as inf, ringattention_hip as rh
+    B, S, H, D, n = 1, 1024, 2, 128, 2
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=25, scale=D ** -0.25)
+    mask = _structured_mask(B, H, S, "causal_padding", 26)
+    out, grads = _run(q, k, v, do, mask, n)
+    orig = rh._MaskInputs.set_keep
+
+    def unpacked(self, attn_mask, device, q_total, k_total):
+        orig(self, attn_mask, device, q_total, k_total)
+        self.keep_packed = None
+    rh._MaskInputs.set_keep = unpacked
+    try:
+        out_g, grads_g = _run(q, k, v, do, mask, n)
+    finally:
+        rh._MaskInputs.set_keep = orig
+    assert_close(out, out_g, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, grads_g):
+        assert_close(a, b, torch.bfloat16, name)
