@@ -625,6 +625,21 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
     if (ntiles > 0) { kw_nxt = kw_ptr[0]; ks_nxt = ks_ptr[0]; }
   }
 
+  // segment ids: a tile whose keys all carry the one id of this wave's rows needs no segment compare
+  const int2* smm_ptr = nullptr;
+  bool sq_uniform = false, sp_cur = false, sp_nxt = false;
+  int sq_id = 0;
+  if (HAS_SEG && mv.seg_mm) {
+    smm_ptr = (const int2*)(mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2);
+    const int2 qmm = smm_ptr[min((gq_wg + grp * 128 + w4 * 32) / RA_SEG_TILE, mv.seg_tiles - 1)];
+    sq_uniform = qmm.x == qmm.y;
+    sq_id = qmm.x;
+    if (sq_uniform && ntiles > 0) {
+      const int2 kmm = smm_ptr[min(gk0 / RA_SEG_TILE, mv.seg_tiles - 1)];
+      sp_nxt = kmm.x == sq_id && kmm.y == sq_id;
+    }
+  }
+
   const int gq = gq_wg + grp * 128 + w4 * 32 + lo;
   const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
   const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq_wg + grp * 128 + w4 * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
@@ -703,7 +718,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
     if (HAS_BIAS) {                                                                                     \
       float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
       if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
-      bias_ks[(J) & 3][tid - 256] = bv_ * kLog2e;                                                             \
+      bias_ks[(J) & 3][tid - 256] = bv_ * kLog2e / c;    /* the S accumulators start from it */             \
     }                                                                                                   \
   }
 
@@ -734,7 +749,15 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   {                                                                                                     \
     const uint16_t* kb_ = Ks[((J) + 1) & 1];                                                            \
     const uint16_t* vb_ = Vs[(J) & 1];                                                                  \
-    _Pragma("unroll") for (int r = 0; r < 16; r++) { s[0][r] = 0.f; s[1][r] = 0.f; }                    \
+    if (HAS_BIAS) {          /* bias (per key = per accumulator row) enters as the initial value of S */ \
+      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
+        _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                 \
+          const f32x4 b4_ = *(const f32x4*)&bias_ks[((J) + 1) & 3][blk * 32 + g * 8 + hi * 4];          \
+          _Pragma("unroll") for (int e = 0; e < 4; e++) s[blk][g * 4 + e] = b4_[e];                     \
+        }                                                                                               \
+    } else {                                                                                            \
+      _Pragma("unroll") for (int r = 0; r < 16; r++) { s[0][r] = 0.f; s[1][r] = 0.f; }                  \
+    }                                                                                                   \
     bf16x8 kf_[PP_DEPTH + 1][2], vf_[PP_DEPTH + 1][2];                                                  \
     _Pragma("unroll") for (int t = 0; t < PP_DEPTH; t++) RA_PP_FRAGS(t, kf_[t], vf_[t]);                \
     _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                     \
@@ -754,6 +777,13 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   {                                                                                                     \
     const int t_ = (T);                                                                                 \
     const int gk_tile_ = gk0 + t_ * FBN;                                                                \
+    if (HAS_SEG) {                        /* are this tile's keys all of this wave's (single) segment? */ \
+      sp_cur = sp_nxt;                                                                                  \
+      if (sq_uniform) {                                                                                 \
+        const int2 kmm_ = smm_ptr[min(gk0 / RA_SEG_TILE + min(t_ + 1, ntiles - 1), mv.seg_tiles - 1)];  \
+        sp_nxt = kmm_.x == sq_id && kmm_.y == sq_id;                                                    \
+      }                                                                                                 \
+    }                                                                                                   \
     if (HAS_KEEP) {                       /* this tile's word and summary; request the next tile's */   \
       kw_cur = kw_nxt >> (4 * hi); ks_cur = ks_nxt;                                                     \
       const int tn_ = min(t_ + 1, ntiles - 1);                                                          \
@@ -763,7 +793,7 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
       _Pragma("unroll") for (int x = 0; x < 8; x++) {                                                   \
         pf[0][0][x] = (__bf16)0.f; pf[0][1][x] = (__bf16)0.f; pf[1][0][x] = (__bf16)0.f; pf[1][1][x] = (__bf16)0.f; \
       }                                                                                                 \
-    } else if (!(HAS_SEG || HAS_BIAS) && (gk_tile_ + FBN - 1 < klim_wave) && (!HAS_KEEP || ks_cur == 2)) { \
+    } else if ((!HAS_SEG || sp_cur) && (gk_tile_ + FBN - 1 < klim_wave) && (!HAS_KEEP || ks_cur == 2)) {   \
       float mxv_ = s[0][0];                                                                             \
       _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
         _Pragma("unroll") for (int r = 0; r < 16; r++) mxv_ = fmaxf(mxv_, s[blk][r]);                   \
@@ -790,7 +820,6 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
         _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
           const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);                                   \
           float x_ = s[blk][r] * c;                                                                     \
-          if (HAS_BIAS) x_ += bias_ks[t_ & 3][kr_];                                                     \
           bool masked_ = (gk_tile_ + kr_ >= klim);                                                      \
           if (HAS_SEG) masked_ = masked_ || (seg_ks[t_ & 3][kr_] != seg_q);                             \
           if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> (blk * 32 + (r >> 2) * 8 + (r & 3))) & 1);    \
@@ -837,7 +866,11 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
   {
     f32x16 sn0, sn1;
 #pragma unroll
-    for (int r = 0; r < 16; r++) { sn0[r] = 0.f; sn1[r] = 0.f; }
+    for (int r = 0; r < 16; r++) {
+      const int kr = (r >> 2) * 8 + hi * 4 + (r & 3);
+      sn0[r] = HAS_BIAS ? bias_ks[0][kr] : 0.f;
+      sn1[r] = HAS_BIAS ? bias_ks[0][32 + kr] : 0.f;
+    }
 #pragma unroll
     for (int t = 0; t < 8; t++) {
       bf16x8 kf0 = *(const bf16x8*)(&Ks[0][k_off[t]]);
@@ -1495,7 +1528,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     if (HAS_BIAS) {
       float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)gk * mv.bias_sk];
       if (mv.any_mask) bv = fminf(bv, 0.f);
-      bias2 = bv * kLog2e;
+      bias2 = bv * kLog2e / c;          // the S accumulators start from it
     }
     const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
     bf16x8 kf[8], vf[8];
@@ -1514,7 +1547,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #define RA_WS_INIT(SN, DPN, BUF, BLK)                                                                   \
   _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                       \
     const f32x4 d_ = *(const f32x4*)&st_delta[BUF][(BLK) * 32 + g * 8 + hi * 4];                        \
-    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = 0.f; DPN[g * 4 + e] = -d_[e]; }     \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = HAS_BIAS ? bias2 : 0.f; DPN[g * 4 + e] = -d_[e]; } \
   }
     // A operands of two contraction steps (32 of the 128 head dimensions) of block BLK of buffer BUF
 #define RA_WS_AREAD(G, QA, GA, BUF, BLK)                                                                \
@@ -1553,7 +1586,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     const f32x4 vrd = *(const f32x4*)&st_rden[BUF][qrow0];                                              \
     _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
       float x = SC[(G) * 4 + e] * c;                                                                    \
-      if (HAS_BIAS) x += bias2;                                                                         \
       bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
       if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
       if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                   \
@@ -1609,17 +1641,38 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
                (int64_t)(mv.keep_q0 / 64 + qt_first) * (mv.keep_K / 64) + (gk0 + pair * 32) / 64;
       kw_nxt = kw_ptr[0]; ks_nxt = ks_ptr[0];
     }
+    // segment ids: a query tile whose 64 rows all carry the one id of this pair's keys needs no compare
+    const int2* smm_ptr = nullptr;
+    bool sk_uniform = false, sp_cur = false, sp_nxt = false;
+    int sk_id = 0;
+    if (HAS_SEG && mv.seg_mm) {
+      smm_ptr = (const int2*)(mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2);
+      const int2 kmm = smm_ptr[min((gk0 + pair * 32) / RA_SEG_TILE, mv.seg_tiles - 1)];
+      sk_uniform = kmm.x == kmm.y;
+      sk_id = kmm.x;
+      if (sk_uniform) {
+        const int2 qmm = smm_ptr[min(gq_base / RA_SEG_TILE + qt_first, mv.seg_tiles - 1)];
+        sp_nxt = qmm.x == sk_id && qmm.y == sk_id;
+      }
+    }
     int cur = 0;
     for (int t = 0; t < ntq; t++) {
       const int nxt = cur == 2 ? 0 : cur + 1, prv = cur == 0 ? 2 : cur - 1;
       const int gq_tile = gq_base + (qt_first + t) * KBM;
+      if (HAS_SEG) {
+        sp_cur = sp_nxt;
+        if (sk_uniform) {
+          const int2 qmm = smm_ptr[min(gq_base / RA_SEG_TILE + qt_first + min(t + 1, ntq - 1), mv.seg_tiles - 1)];
+          sp_nxt = qmm.x == sk_id && qmm.y == sk_id;
+        }
+      }
       if (HAS_KEEP) {                      // this tile's word and summary; request the next tile's
         kw_cur = kw_nxt >> (4 * hi); ks_cur = ks_nxt;
         const int tn = min(t + 1, ntq - 1);
         kw_nxt = kw_ptr[(int64_t)tn * mv.keep_K]; ks_nxt = ks_ptr[(int64_t)tn * (mv.keep_K / 64)];
       }
       // step 2t: vector work of block 0 of tile t, products of block 1
-      if (HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
+      if ((HAS_SEG && !sp_cur) || (gq_tile < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
         RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, true);
       } else {
         RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, false);
@@ -1629,7 +1682,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       // block 0 of tile t + 1 (the last tile computes a block that is never used)
       RA_WS_STORE(prv);
       RA_WS_LOAD(t + 3);
-      if (HAS_SEG || HAS_BIAS || (gq_tile + 32 < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
+      if ((HAS_SEG && !sp_cur) || (gq_tile + 32 < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
         RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, true);
       } else {
         RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, false);
@@ -1835,7 +1888,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       if (HAS_BIAS) {                                                                                   \
         float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
         if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
-        bias_r = bv_ * kLog2e;                                                                          \
+        bias_r = bv_ * kLog2e / c;   /* the S accumulators start from it */                             \
       }                                                                                                 \
     }                                                                                                   \
   }
@@ -1905,8 +1958,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     uint16_t* const dw = &Ds[pair][0][lo * WS_PSTR + hi * 4];
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-#define RA_WS_INIT(SN, DPN)                                                                             \
-  _Pragma("unroll") for (int r = 0; r < 16; r++) { SN[r] = 0.f; DPN[r] = ndelta; }
+#define RA_WS_INIT(SN, DPN, BUF, BLK)                                                                   \
+  _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                       \
+    f32x4 b4_ = {0.f, 0.f, 0.f, 0.f};                                                                   \
+    if (HAS_BIAS) b4_ = *(const f32x4*)&bias_ks[BUF][(BLK) * 32 + g * 8 + hi * 4];                      \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = b4_[e]; DPN[g * 4 + e] = ndelta; }  \
+  }
 #define RA_WS_AREAD(G, KA, VA, BUF, BLK)                                                                \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
     KA[i] = *(const bf16x8*)(Ks + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
@@ -1933,7 +1990,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       } else {                                                                                          \
         const int kr_ = (BLK) * 32 + (G) * 8 + hi * 4 + e;                                              \
         float x = SC[(G) * 4 + e] * c;                                                                  \
-        if (HAS_BIAS) x += bias_ks[BUF][kr_];                                                           \
         bool masked = (gk_tile + kr_ >= klim);                                                          \
         if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
         if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                 \
@@ -1951,7 +2007,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     // covers the LDS latency under load.
 #define RA_WS_PRODUCE(SC, DPC, SN, DPN, BUF, BLK, NBUF, NBLK, NNBUF, NNBLK, PB, MASKED)                 \
   {                                                                                                     \
-    RA_WS_INIT(SN, DPN);                                                                                \
+    RA_WS_INIT(SN, DPN, NBUF, NBLK);                                                                    \
     _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                     \
       if (g == 0) { RA_WS_AREAD(3, ka[3], va[3], NBUF, NBLK); }                                         \
       else { RA_WS_AREAD(g - 1, ka[g - 1], va[g - 1], NNBUF, NNBLK); }                                  \
@@ -1969,7 +2025,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 
     f32x16 s_a, dp_a, s_b, dp_b;
     bf16x8 ka[4][2], va[4][2];
-    RA_WS_INIT(s_a, dp_a);
+    RA_WS_INIT(s_a, dp_a, 0, 0);
 #pragma unroll
     for (int g = 0; g < 4; g++) {
       RA_WS_AREAD(g, ka[0], va[0], 0, 0);
@@ -1980,19 +2036,56 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 
     // Under a causal mask the tiles that need no masking come first: one loop for them, one for the rest
     // (which also takes every tile when segment ids or a bias are present).
-    int t_plain = 0;
-    if (!(HAS_SEG || HAS_BIAS)) t_plain = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
-    // packed keep mask: the tiles whose 64 x 64 summary says "all kept" for these rows need no masking either
+    // Which key tiles need no masking at all: below the causal limit of every row, keys all of this wave's
+    // single segment id, packed keep summary "all kept".  They form (at most) one run [t_a, t_b) in the
+    // cases that matter - document interiors, the part of a causal row left of the diagonal - and get a
+    // loop of their own; the tiles before and after take the masked loop.
+    const int t_causal = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
     const uint64_t* kw_ptr = nullptr;
+    const uint8_t* ks_ptr = nullptr;
     uint64_t kw_cur = 0, kw_nxt = 0;
     if (HAS_KEEP) {
-      const uint8_t* ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
-                              (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
-      t_plain = __builtin_amdgcn_readfirstlane(min(t_plain, keep_leading_full(ks_ptr, 1, ntiles, lane)));
+      ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
+               (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
       kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
                mv.keep_q0 + qrow;
-      kw_nxt = kw_ptr[(int64_t)min(t_plain, ntiles - 1) * mv.keep_Q];
     }
+    const int2* smm_ptr = nullptr;
+    bool sq_uniform = false;
+    int sq_id = 0;
+    if (HAS_SEG && mv.seg_mm) {
+      smm_ptr = (const int2*)(mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2);
+      const int2 qmm = smm_ptr[min((gq0 + pair * 32) / RA_SEG_TILE, mv.seg_tiles - 1)];
+      sq_uniform = qmm.x == qmm.y;
+      sq_id = qmm.x;
+    }
+    int t_a = ntiles, t_b = ntiles;
+    for (int base = 0; base < ntiles; base += 64) {
+      const int tt = base + lane;
+      bool ok = tt < t_causal;
+      if (HAS_SEG && ok) {
+        ok = sq_uniform;
+        if (ok) {
+          const int2 kmm = smm_ptr[min(gk0 / RA_SEG_TILE + tt, mv.seg_tiles - 1)];
+          ok = kmm.x == sq_id && kmm.y == sq_id;
+        }
+      }
+      if (HAS_KEEP && ok) ok = ks_ptr[tt] == 2;
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(ok);
+      unsigned long long stop;      // tiles of this group of 64 that end the run
+      if (t_a == ntiles) {
+        if (!m) continue;
+        const int f = __builtin_ctzll(m);
+        t_a = base + f;
+        stop = ~m & (~0ULL << f);
+      } else {
+        stop = ~m;
+      }
+      if (stop) { t_b = min(ntiles, base + (int)__builtin_ctzll(stop)); break; }
+    }
+    t_a = __builtin_amdgcn_readfirstlane(t_a);
+    t_b = __builtin_amdgcn_readfirstlane(t_a == ntiles ? ntiles : t_b);
+    if (HAS_KEEP) kw_nxt = kw_ptr[(int64_t)min(t_a == 0 ? t_b : 0, ntiles - 1) * mv.keep_Q];
     int cur = 0;
 #define RA_WS_TILE(MASKED)                                                                              \
   {                                                                                                     \
@@ -2001,7 +2094,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     (void)gk_tile;                                                                                      \
     if (HAS_KEEP && (MASKED)) {        /* this tile's word; request the next tile's */                  \
       kw_cur = kw_nxt >> (4 * hi);                                                                      \
-      kw_nxt = kw_ptr[(int64_t)min(t + 1, ntiles - 1) * mv.keep_Q];                                     \
+      kw_nxt = kw_ptr[(int64_t)min(t + 1 == t_a ? t_b : t + 1, ntiles - 1) * mv.keep_Q];                \
     }                                                                                                   \
     /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
     RA_TRACE_MARK();                                                                                    \
@@ -2017,7 +2110,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     cur = nxt;                                                                                          \
   }
     int t = 0;
-    for (; t < t_plain; t++) RA_WS_TILE(false);
+    for (; t < t_a; t++) RA_WS_TILE(true);
+    for (; t < t_b; t++) RA_WS_TILE(false);
     for (; t < ntiles; t++) RA_WS_TILE(true);
 #undef RA_WS_TILE
     __syncthreads();      // step 2 ntiles: the consumer's last block
