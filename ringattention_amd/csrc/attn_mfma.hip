@@ -143,50 +143,6 @@ __device__ __forceinline__ int keep_leading_full(const uint8_t* sm, int64_t stri
   return n;
 }
 
-// Staging helpers shared by the kernels below.  They expect in scope: tid, s_off (this thread's
-// swizzled element offset inside a 16-row slab), row16 (global element stride of 16 rows).
-#define RA_LOAD_TILE(REGS, BASE, STRIDE, J, ROWS)                                                       \
-  {                                                                                                     \
-    const uint16_t* p_ = (BASE) + (int64_t)(J) * (ROWS) * (STRIDE);                                     \
-    _Pragma("unroll") for (int p = 0; p < 4; p++) REGS[p] = *(const uint4*)(p_ + p * row16);            \
-  }
-#define RA_STORE_TILE(REGS, LDS)                                                                        \
-  {                                                                                                     \
-    _Pragma("unroll") for (int p = 0; p < 4; p++) *(uint4*)(&(LDS)[p * 16 * TROW + s_off]) = REGS[p];   \
-  }
-// Direct global -> LDS staging of a 64-row tile (no registers): wavefront w issues four
-// global_load_lds of 16 bytes per lane; instruction i fills tile rows 16 w + 4 i .. +3, lane l the
-// physical slot (l & 15) of row 16 w + 4 i + (l >> 4), i.e. logical slot (l & 15) ^ swz(row).
-// Expects in scope: wave_u (wavefront index, uniform), dchunk0 = (lane & 15) ^ ((lane >> 4) << 2).
-// GROW0 points at element 0 of this lane's row for i = 0 in tile 0; STRIDE = global row stride.
-#define RA_DMA_TILE(LDS, GROW0, STRIDE, J, ROWS)                                                        \
-  {                                                                                                     \
-    const uint16_t* g_ = (GROW0) + (int64_t)(J) * (ROWS) * (STRIDE);                                    \
-    _Pragma("unroll") for (int i = 0; i < 4; i++)                                                       \
-      __builtin_amdgcn_global_load_lds(                                                                 \
-          (const __attribute__((address_space(1))) void*)(g_ + (int64_t)(4 * i) * (STRIDE) + ((dchunk0 ^ i) << 3)), \
-          (__attribute__((address_space(3))) void*)(&(LDS)[(16 * wave_u + 4 * i) * TROW]), 16, 0, 0);   \
-  }
-#define RA_DMA_WAIT() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
-// per-key segment id / bias of key tile J (threads 0..63), for kernels that stream key tiles
-#define RA_LOAD_KEYINFO(J)                                                                              \
-  if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                             \
-    const int kj_ = k_base + (J) * FBN + tid;                                                           \
-    if (HAS_SEG) {                                                                                      \
-      int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
-      seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                    \
-    }                                                                                                   \
-    if (HAS_BIAS) {                                                                                     \
-      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
-      if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
-      bias_r = bv_ * kLog2e;                                                                            \
-    }                                                                                                   \
-  }
-#define RA_STORE_KEYINFO(BUF)                                                                           \
-  if ((HAS_SEG || HAS_BIAS) && tid < FBN) {                                                             \
-    if (HAS_SEG) seg_ks[BUF][tid] = seg_r;                                                              \
-    if (HAS_BIAS) bias_ks[BUF][tid] = bias_r;                                                           \
-  }
 // Per-lane LDS read offsets (elements) into a swizzled tile.
 //  NAT[t]: 16-byte read of row lo, d = 16 t + 8 hi .. +8 (MFMA operand whose contraction index is d).
 //  TR[db][x]: ds_read_b64_tr_b16 address; lane i of a 16-lane group addresses tile row
@@ -201,333 +157,6 @@ __device__ __forceinline__ int keep_leading_full(const uint8_t* sm, int64_t stri
       TR[db][1] = (rr_ + 8) * TROW + (((4 * db + c0_) ^ swz(rr_ + 8)) << 3) + half_ * 4;                \
     }                                                                                                   \
   }
-
-template <bool HAS_SEG, bool HAS_BIAS>
-__global__ __launch_bounds__(256, 2) void attn_fwd_mfma_kernel(FwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
-  __shared__ int seg_ks[2][FBN];
-  __shared__ float bias_ks[2][FBN];
-
-  MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
-  const int nqt = a.Sq / FBM;
-  int wg = blockIdx.x;
-  const int qt = nqt - 1 - (wg % nqt);       // heaviest (latest) query tiles first
-  wg /= nqt;
-  const int h = wg % a.H, b = wg / a.H;
-  const int q0 = qt * FBM;
-  const int qrow = q0 + wave * 32 + lo;      // this lane's query row (local)
-
-  // ---- tile range: chunks that run (reference predicate), clipped to tiles with an unmasked pair
-  const int qi = q0 / mv.qc;
-  int kend = mv.run_prefix_keys(qi, a.Skv);
-  // global positions fit 31 bits (checked on the host)
-  const int gq0 = (int)mv.global_q(q0);
-  const int gk0_shard = (int)mv.global_k(0);
-  if (mv.cbs > 0 && mv.skip_tiles) {
-    long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;   // first key position masked for every row
-    long long n = lim - gk0_shard;
-    if (n < kend) kend = n > 0 ? (int)n : 0;
-  }
-  int ntiles = (kend + FBN - 1) / FBN;
-  // key tiles outside the hull of those sharing a segment with these 128 rows are skipped
-  int k_base = 0;                           // local key index of the first tile processed
-  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
-    __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gq0, FBM, slo, shi);
-    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 256, t_first, t_last);
-    k_base = t_first * FBN;
-    ntiles = t_last - t_first;
-  }
-  const int gk0 = gk0_shard + k_base;       // global position of the first key processed
-
-  // per-lane mask constants: keys at global position >= klim are masked
-  const int gq = gq0 + wave * 32 + lo;
-  const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
-  const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
-  int seg_q = 0;
-  if (HAS_SEG) {
-    int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
-    seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
-  }
-  const float c = kLog2e / sqrtf((float)HD);
-  const float kMask2 = mv.mask_min;
-
-  // ---- Q fragments (B operand of S^T = K Q^T): column = query row, 8 consecutive d per MFMA step
-  const uint16_t* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-  bf16x8 qf[8];
-#pragma unroll
-  for (int t = 0; t < 8; t++) qf[t] = *(const bf16x8*)(qp + t * 16);
-
-  // ---- carry
-  f32x16 acc[4];
-  float m2 = RA_NEG_INF, l = 0.f;
-  float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
-  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
-  if (a.carry_is_initial) {
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
-  } else {
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        f32x4 t = *(const f32x4*)(nump + db * 32 + g * 8);
-        acc[db][g * 4 + 0] = t[0]; acc[db][g * 4 + 1] = t[1]; acc[db][g * 4 + 2] = t[2]; acc[db][g * 4 + 3] = t[3];
-      }
-    m2 = max_to_log2(a.mx[st], kMask2);
-    l = hi == 0 ? a.den[st] : 0.f;     // the two half-wave partial sums are added at the end
-  }
-  if (ntiles == 0) {
-    if (a.carry_is_initial) {         // nothing runs for these rows: the carry stays (0, 0, -inf)
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) *(f32x4*)(nump + db * 32 + g * 8) = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (hi == 0) { a.den[st] = 0.f; a.mx[st] = RA_NEG_INF; }
-    }
-    return;
-  }
-
-  // ---- staging: direct global -> LDS loads, see RA_DMA_TILE
-  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-  const int dchunk0 = (lane & 15) ^ ((lane >> 4) << 2);
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(k_base + 16 * wave + (lane >> 4)) * a.kv_ss;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)(k_base + 16 * wave + (lane >> 4)) * a.kv_ss;
-  int seg_r = 0;
-  float bias_r = 0.f;
-  int k_off[8], v_off[4][2];
-  RA_LANE_OFFSETS(k_off, v_off);
-
-#define RA_QK(S, KBUF)                                                                                  \
-  {                                                                                                     \
-    _Pragma("unroll") for (int blk = 0; blk < 2; blk++) {                                               \
-      _Pragma("unroll") for (int r = 0; r < 16; r++) S[blk][r] = 0.f;                                   \
-      _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                   \
-        bf16x8 kf_ = *(const bf16x8*)(&(KBUF)[blk * 32 * TROW + k_off[t]]);                             \
-        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_, qf[t], S[blk], 0, 0, 0);                  \
-      }                                                                                                 \
-    }                                                                                                   \
-  }
-// one MFMA step of S(j+1): key block BLK, d step T
-#define RA_QK_STEP(S, KBUF, BLK, T)                                                                     \
-  {                                                                                                     \
-    bf16x8 kf_ = *(const bf16x8*)(&(KBUF)[(BLK) * 32 * TROW + k_off[T]]);                               \
-    S[BLK] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_, qf[T], S[BLK], 0, 0, 0);                      \
-  }
-// eight probabilities of key block BLK, half HALF: p = exp2(s c - m), summed and rounded to bf16
-#define RA_EXP_GROUP(BLK, HALF)                                                                         \
-  {                                                                                                     \
-    _Pragma("unroll") for (int e = 0; e < 8; e++) {                                                     \
-      float p_ = fast_exp2(fmaf(s[BLK][(HALF) * 8 + e], c, -m2));                                       \
-      ps += p_;                                                                                         \
-      pf[BLK][HALF][e] = (__bf16)p_;                                                                    \
-    }                                                                                                   \
-    /* pin the results here: without it the optimiser sinks the exponentials below the next branch */   \
-    i32x4 pin_ = __builtin_bit_cast(i32x4, pf[BLK][HALF]);                                              \
-    asm volatile("" : "+v"(pin_), "+v"(ps));                                                            \
-    pf[BLK][HALF] = __builtin_bit_cast(bf16x8, pin_);                                                   \
-  }
-// four MFMA steps of O^T += V^T P^T: keys 32 BLK + 16 T .. +16, all four d blocks
-#define RA_PV_GROUP(VBUF, BLK, T)                                                                       \
-  {                                                                                                     \
-    const uint16_t* vt_ = &(VBUF)[((BLK) * 32 + (T) * 16) * TROW];                                      \
-    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
-      s16x4 v0_ = lds_read_tr(vt_ + v_off[db][0]);                                                      \
-      s16x4 v1_ = lds_read_tr(vt_ + v_off[db][1]);                                                      \
-      s16x8 vv_ = __builtin_shufflevector(v0_, v1_, 0, 1, 2, 3, 4, 5, 6, 7);                            \
-      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vv_), pf[BLK][T], acc[db], 0, 0, 0); \
-    }                                                                                                   \
-  }
-// ask the scheduler for N repetitions of (1 MFMA, V vector-ALU ops), then fence the group
-#define RA_INTERLEAVE(N, V)                                                                             \
-  {                                                                                                     \
-    _Pragma("unroll") for (int i_ = 0; i_ < (N); i_++) {                                                \
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                \
-      __builtin_amdgcn_sched_group_barrier(0x002, (V), 0);                                              \
-    }                                                                                                   \
-    __builtin_amdgcn_sched_barrier(0);                                                                  \
-  }
-
-  // ---- prologue: K(0), V(0), K(1) into LDS, S(0)
-  RA_DMA_TILE(Ks[0], kg, a.kv_ss, 0, FBN);
-  RA_DMA_TILE(Vs[0], vg, a.kv_ss, 0, FBN);
-  RA_DMA_TILE(Ks[1], kg, a.kv_ss, min(1, ntiles - 1), FBN);
-  RA_LOAD_KEYINFO(0);
-  RA_STORE_KEYINFO(0);
-  RA_DMA_WAIT();
-  __syncthreads();
-  f32x16 s[2];
-  RA_QK(s, Ks[0]);
-
-  // Tiles [0, n_plain) need no mask for any wavefront of the workgroup: they run the interleaved
-  // loop; the rest (diagonal tiles, or every tile when segment ids / bias are present) run the
-  // plain loop with the element-wise mask.
-  int n_plain = 0;
-  if (!HAS_SEG && !HAS_BIAS) {
-    const long long klim_wg = mv.cbs > 0 ? (long long)(gq0 / mv.cbs + 1) * mv.cbs : 0x7fffffffLL;   // smallest klim in the workgroup
-    long long n = (klim_wg - gk0) / FBN;       // tiles whose last key is < klim_wg
-    n_plain = n < 0 ? 0 : (n > ntiles ? ntiles : (int)n);
-  }
-
-  // m2 is the reference max the exponentials are taken against.  In the interleaved loop it is only
-  // raised when some row's true max has outgrown it by more than kLazy (log2 units): the accumulator
-  // rescale then runs once in a long while; m_true tracks the exact running max and the carry is
-  // brought to it at the end.
-  constexpr float kLazy = 16.f;
-  float m_true = m2;
-
-  int j = 0;
-  for (; j < n_plain; j++) {
-    const int cur = j & 1;
-    // K(j+2) replaces K(j) (consumed last iteration), V(j+1) replaces V(j-1); clamped at the tail
-    RA_DMA_TILE(Ks[cur], kg, a.kv_ss, min(j + 2, ntiles - 1), FBN);
-    RA_DMA_TILE(Vs[cur ^ 1], vg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
-    __builtin_amdgcn_sched_barrier(0);
-
-    f32x16 sn[2];
-    bf16x8 pf[2][2];
-    float ps = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; r++) { sn[0][r] = 0.f; sn[1][r] = 0.f; }
-    // group 1: first S(j+1) steps under the row max of S(j)
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 0); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 0);
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 1); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 1);
-    float mxv = s[0][0];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) mxv = fmaxf(mxv, s[blk][r]);
-    mxv = fmaxf(mxv, xor32(mxv));
-    m_true = fmaxf(m_true, mxv * c);
-    const bool raise = __builtin_amdgcn_ballot_w64(m_true - m2 > kLazy) != 0;
-    RA_INTERLEAVE(4, 5);
-    if (raise) {
-      const float alpha = fast_exp2(m2 - m_true);
-      m2 = m_true;
-      l *= alpha;
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[db][r] *= alpha;
-    }
-    // groups 2-4: remaining S(j+1) steps under the exponentials of S(j)
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 2); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 2);
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 3); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 3);
-    RA_EXP_GROUP(0, 0);
-    RA_INTERLEAVE(4, 7);
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 4); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 4);
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 5); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 5);
-    RA_EXP_GROUP(0, 1);
-    RA_INTERLEAVE(4, 7);
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 6); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 6);
-    RA_QK_STEP(sn, Ks[cur ^ 1], 0, 7); RA_QK_STEP(sn, Ks[cur ^ 1], 1, 7);
-    RA_EXP_GROUP(1, 0);
-    RA_INTERLEAVE(4, 7);
-    // groups 5-8: O^T += V(j)^T P^T, the first of them under the last exponentials
-    RA_PV_GROUP(Vs[cur], 0, 0);
-    RA_EXP_GROUP(1, 1);
-    RA_INTERLEAVE(4, 7);
-    RA_PV_GROUP(Vs[cur], 0, 1);
-    RA_PV_GROUP(Vs[cur], 1, 0);
-    RA_PV_GROUP(Vs[cur], 1, 1);
-    l += ps;
-    s[0] = sn[0]; s[1] = sn[1];
-    RA_DMA_WAIT();
-    __syncthreads();
-  }
-
-  for (; j < ntiles; j++) {
-    const int cur = j & 1;
-    RA_DMA_TILE(Ks[cur], kg, a.kv_ss, min(j + 2, ntiles - 1), FBN);
-    RA_DMA_TILE(Vs[cur ^ 1], vg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
-    RA_LOAD_KEYINFO(min(j + 1, ntiles - 1));
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- S(j+1)^T = K(j+1) Q^T
-    f32x16 sn[2];
-    RA_QK(sn, Ks[cur ^ 1]);
-
-    // ---- online softmax of S(j) in the log2 domain, element-wise mask
-    const int gk_tile = gk0 + j * FBN;
-    float mxv = RA_NEG_INF;
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);     // key row inside the tile
-        float x = s[blk][r] * c;
-        if (HAS_BIAS) x += bias_ks[cur][kr_];
-        bool masked = (gk_tile + kr_ >= klim);
-        if (HAS_SEG) masked = masked || (seg_ks[cur][kr_] != seg_q);
-        x = masked ? kMask2 : x;
-        s[blk][r] = x;
-        mxv = fmaxf(mxv, x);
-      }
-    mxv = fmaxf(mxv, xor32(mxv));
-    m_true = fmaxf(m_true, mxv);
-    const float m_new = fmaxf(m2, mxv);
-    const float alpha = fast_exp2(m2 - m_new);
-    m2 = m_new;
-    float ps = 0.f;
-    bf16x8 pf[2][2];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float p = fast_exp2(s[blk][r] - m_new);
-        ps += p;
-        pf[blk][r >> 3][r & 7] = (__bf16)p;
-      }
-    l = l * alpha + ps;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[db][r] *= alpha;
-    }
-    RA_PV_GROUP(Vs[cur], 0, 0);
-    RA_PV_GROUP(Vs[cur], 0, 1);
-    RA_PV_GROUP(Vs[cur], 1, 0);
-    RA_PV_GROUP(Vs[cur], 1, 1);
-    RA_STORE_KEYINFO(cur ^ 1);
-    s[0] = sn[0]; s[1] = sn[1];
-    RA_DMA_WAIT();
-    __syncthreads();
-  }
-  if (__builtin_amdgcn_ballot_w64(m_true != m2) != 0) {     // bring the carry to the exact running max
-    const float fix = (m_true == m2) ? 1.f : fast_exp2(m2 - m_true);
-    m2 = m_true;
-    l *= fix;
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[db][r] *= fix;
-  }
-#undef RA_QK
-#undef RA_QK_STEP
-#undef RA_EXP_GROUP
-#undef RA_PV_GROUP
-
-  // ---- write the carry back: numerator (fp32), denominator, max_score (natural log domain)
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      f32x4 t = {acc[db][g * 4 + 0], acc[db][g * 4 + 1], acc[db][g * 4 + 2], acc[db][g * 4 + 3]};
-      *(f32x4*)(nump + db * 32 + g * 8) = t;
-    }
-  l += xor32(l);
-  if (hi == 0) {
-    a.den[st] = l;
-    a.mx[st] = max_from_log2(m2, kMask2);
-  }
-}
 
 // ------------------------------------------------------------------ forward, ping-pong variant
 // 8 wavefronts per workgroup, 256 query rows: group A (waves 0-3) owns rows 0..127, group B (waves
@@ -953,14 +582,15 @@ __global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
 
 // ================================================================== backward
 // Two deterministic kernels (fp32 atomics reach ~1.3 TB/s at best on this part, far below what a
-// fused dQ accumulation would need):
-//   dQ   : query-stationary, same shape as the forward.  S^T = K Q^T and dP^T = V dO^T share the
-//          lane <-> query-column layout, so max / 1/denominator / delta are per-lane scalars;
-//          dQ^T += K^T dS^T takes K^T from the row-major K tile with LDS transpose reads.
+// fused dQ accumulation would need), both wave-specialised (see below):
 //   dK,dV: key-stationary.  S = Q K^T and dP = dO V^T with K / V fragments resident in registers;
-//          P and dS (accumulator layout, lane <-> key column) feed dV^T += dO^T P and
-//          dK^T += Q^T dS directly as B operands; Q^T / dO^T come from LDS transpose reads.
+//          P and dS feed dV^T += dO^T P and dK^T += Q^T dS; Q^T / dO^T come from LDS transpose reads.
+//   dQ   : query-stationary.  S^T = K Q^T and dP^T = V dO^T share the lane <-> query-column layout, so
+//          max / denominator / delta are per-lane scalars; dQ^T += K^T dS^T takes K^T from the row-major
+//          K tile with LDS transpose reads.
 // Probabilities are recomputed from the saved max_score / denominator (ringattention_jax.py:226).
+constexpr int KBN = 128;   // keys per workgroup in the dK/dV kernel (32 per wavefront pair)
+constexpr int KBM = 64;    // query rows per tile
 
 struct BwdArgs {
   const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* g;
@@ -973,401 +603,6 @@ struct BwdArgs {
   MaskView mv;
   const int32_t* cache_idx;
 };
-
-template <bool HAS_SEG, bool HAS_BIAS>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dq_mfma_kernel(BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
-  __shared__ int seg_ks[2][FBN];
-  __shared__ float bias_ks[2][FBN];
-
-  MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
-  const int nqt = a.Sq / FBM;
-  int wg = blockIdx.x;
-  const int qt = nqt - 1 - (wg % nqt);
-  wg /= nqt;
-  const int h = wg % a.H, b = wg / a.H;
-  const int q0 = qt * FBM;
-  const int qrow = q0 + wave * 32 + lo;
-
-  const int qi = q0 / mv.qc;
-  int kend = mv.run_prefix_keys(qi, a.Skv);
-  const int gq0 = (int)mv.global_q(q0);
-  const int gk0_shard = (int)mv.global_k(0);
-  if (mv.cbs > 0 && mv.skip_tiles) {
-    long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
-    long long n = lim - gk0_shard;
-    if (n < kend) kend = n > 0 ? (int)n : 0;
-  }
-  int ntiles = (kend + FBN - 1) / FBN;
-  int k_base = 0;
-  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
-    __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gq0, FBM, slo, shi);
-    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 256, t_first, t_last);
-    k_base = t_first * FBN;
-    ntiles = t_last - t_first;
-  }
-  if (ntiles == 0) return;     // nothing to add to dq
-  const int gk0 = gk0_shard + k_base;
-
-  const int gq = gq0 + wave * 32 + lo;
-  const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
-  const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq0 + wave * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
-  int seg_q = 0;
-  if (HAS_SEG) {
-    int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
-    seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
-  }
-  const float c = kLog2e / sqrtf((float)HD);
-  const float kMask2 = mv.mask_min;
-
-  const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-  bf16x8 qf[8], gf[8];
-#pragma unroll
-  for (int t = 0; t < 8; t++) {
-    qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
-    gf[t] = *(const bf16x8*)(a.g + qoff + t * 16);
-  }
-  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
-  const float m2 = max_to_log2(a.mx[st], kMask2);
-  const float rden = 1.f / a.den[st];
-  const float delta = a.delta[st];
-
-  f32x16 acc[4];
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
-
-  const int srow = tid >> 4, schunk = tid & 15;
-  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const uint16_t* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
-  const uint16_t* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
-  const int64_t row16 = 16 * a.kv_ss;
-  uint4 kr[4], vr[4];
-  int seg_r = 0;
-  float bias_r = 0.f;
-  RA_LOAD_TILE(kr, kg, a.kv_ss, 0, FBN);
-  RA_LOAD_TILE(vr, vg, a.kv_ss, 0, FBN);
-  RA_LOAD_KEYINFO(0);
-  RA_STORE_TILE(kr, Ks[0]);
-  RA_STORE_TILE(vr, Vs[0]);
-  RA_STORE_KEYINFO(0);
-  __syncthreads();
-
-  int n_off[8], t_off[4][2];
-  RA_LANE_OFFSETS(n_off, t_off);
-
-  for (int j = 0; j < ntiles; j++) {
-    const int cur = j & 1;
-    RA_LOAD_TILE(kr, kg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
-    RA_LOAD_TILE(vr, vg, a.kv_ss, min(j + 1, ntiles - 1), FBN);
-    RA_LOAD_KEYINFO(min(j + 1, ntiles - 1));
-    const int gk_tile = gk0 + j * FBN;
-    const bool need_mask = HAS_SEG || HAS_BIAS || (gk_tile + FBN - 1 >= klim_wave);
-
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
-      f32x16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
-      const uint16_t* kp = &Ks[cur][blk * 32 * TROW];
-      const uint16_t* vp = &Vs[cur][blk * 32 * TROW];
-#pragma unroll
-      for (int t = 0; t < 8; t++) {
-        bf16x8 kf = *(const bf16x8*)(kp + n_off[t]);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[t], s, 0, 0, 0);          // S^T = K Q^T
-      }
-#pragma unroll
-      for (int t = 0; t < 8; t++) {
-        bf16x8 vf = *(const bf16x8*)(vp + n_off[t]);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, gf[t], dp, 0, 0, 0);        // dP^T = V dO^T
-      }
-      bf16x8 dsf[2];
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float p;
-        if (!need_mask) {
-          p = fast_exp2(fmaf(s[r], c, -m2)) * rden;
-        } else {
-          const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-          float x = s[r] * c;
-          if (HAS_BIAS) x += bias_ks[cur][kr_];
-          bool masked = (gk_tile + kr_ >= klim);
-          if (HAS_SEG) masked = masked || (seg_ks[cur][kr_] != seg_q);
-          x = masked ? kMask2 : x;
-          p = fast_exp2(x - m2) * rden;                                              // :226
-        }
-        dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - delta));                          // :229
-      }
-      // dQ^T += K^T dS^T over these 32 keys
-#pragma unroll
-      for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int db = 0; db < 4; db++) {
-          const uint16_t* ktp = &Ks[cur][(blk * 32 + t * 16) * TROW];
-          s16x4 k0v = lds_read_tr(ktp + t_off[db][0]);
-          s16x4 k1v = lds_read_tr(ktp + t_off[db][1]);
-          s16x8 kk = __builtin_shufflevector(k0v, k1v, 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kk), dsf[t], acc[db], 0, 0, 0);
-        }
-    }
-    RA_STORE_TILE(kr, Ks[cur ^ 1]);
-    RA_STORE_TILE(vr, Vs[cur ^ 1]);
-    RA_STORE_KEYINFO(cur ^ 1);
-    __syncthreads();
-  }
-
-  // dq += acc / sqrt(D)   (:230)
-  const float rscale = 1.f / sqrtf((float)HD);
-  float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      f32x4 t = *(const f32x4*)(dqp + db * 32 + g * 8);
-      t[0] += acc[db][g * 4 + 0] * rscale; t[1] += acc[db][g * 4 + 1] * rscale;
-      t[2] += acc[db][g * 4 + 2] * rscale; t[3] += acc[db][g * 4 + 3] * rscale;
-      *(f32x4*)(dqp + db * 32 + g * 8) = t;
-    }
-}
-
-constexpr int KBN = 128;   // keys per workgroup in the dK/dV kernel (32 per wavefront)
-constexpr int KBM = 64;    // query rows per step
-
-template <bool HAS_SEG, bool HAS_BIAS, bool WANT_DK, bool WANT_DV>
-__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_mfma_kernel(BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][KBM * TROW];
-  __shared__ __attribute__((aligned(16))) uint16_t Gs[2][KBM * TROW];
-  __shared__ __attribute__((aligned(16))) float st_m2[2][KBM];
-  __shared__ __attribute__((aligned(16))) float st_rden[2][KBM];
-  __shared__ __attribute__((aligned(16))) float st_delta[2][KBM];
-  __shared__ __attribute__((aligned(16))) int st_seg[2][KBM];
-
-  MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
-  const int nkt = a.Skv / KBN;
-  int wg = blockIdx.x;
-  const int kt = wg % nkt;                 // earliest key blocks (most query tiles under causal) first
-  wg /= nkt;
-  const int h = wg % a.H, b = wg / a.H;
-  const int k0 = kt * KBN;
-  const int krow = k0 + wave * 32 + lo;    // this lane's key row (local)
-
-  const int gk0 = (int)mv.global_k(k0);
-  const int gk = gk0 + wave * 32 + lo;
-  const int gq_base = (int)mv.global_q(0);
-  // first query tile that has work for this key block: run prefix (chunk level), then sub-tile clip
-  const int nqt = a.Sq / KBM;
-  int qt_first = nqt;
-  {
-    // the run prefix is non-decreasing in the query chunk index: binary search the first chunk that reaches k0
-    int nqc = a.Sq / mv.qc, lo_c = 0, hi_c = nqc;
-    while (lo_c < hi_c) {
-      int mid = (lo_c + hi_c) >> 1;
-      if (mv.run_prefix_keys(mid, a.Skv) > k0) hi_c = mid; else lo_c = mid + 1;
-    }
-    if (lo_c < nqc) qt_first = lo_c * (mv.qc / KBM);
-    if (mv.cbs > 0 && mv.skip_tiles && qt_first < nqt) {
-      // query tiles whose every row is masked against every key of the block: (gq_max / cbs) < (gk_min / cbs)
-      long long need = (long long)(gk0 / mv.cbs) * mv.cbs - gq_base;     // first local query row that can see key gk0
-      if (need > 0) {
-        int t = (int)(need / KBM);
-        if (t > qt_first) qt_first = t < nqt ? t : nqt;
-      }
-    }
-  }
-  int qt_end = nqt;
-  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && qt_first < nqt) {
-    // query tiles outside the hull of those sharing a segment with these 128 keys are skipped
-    __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gk0, KBN, slo, shi);
-    seg_tile_hull(mv, b, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, slo, shi, hull2, tid, 256, t_first, t_last);
-    qt_end = qt_first + t_last;
-    qt_first += t_first;
-  }
-  if (qt_first >= qt_end) return;         // no query sees this key block: dk, dv unchanged
-
-  // masked iff gq / cbs < gk / cbs  <=>  gq < qlim
-  const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;
-  const int qlim_wave = mv.cbs > 0 ? ((gk0 + wave * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffff;
-  int seg_k = 0;
-  float bias2 = 0.f;
-  if (HAS_SEG) {
-    int idx = clamp_seg_index(((long long)mv.k_start + krow / mv.kc) * mv.kc, mv.kc, mv.seg_len, krow % mv.kc);
-    seg_k = mv.seg[(int64_t)b * mv.seg_sb + idx];
-  }
-  if (HAS_BIAS) {
-    float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)gk * mv.bias_sk];
-    if (mv.any_mask) bv = fminf(bv, 0.f);
-    bias2 = bv * kLog2e;
-  }
-  const float c = kLog2e / sqrtf((float)HD);
-  const float kMask2 = mv.mask_min;
-
-  // K and V fragments of this lane's key column (B operands), resident for the whole loop
-  const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
-  bf16x8 kf[8], vf[WANT_DK ? 8 : 1];
-#pragma unroll
-  for (int t = 0; t < 8; t++) {
-    kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
-    if (WANT_DK) vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
-  }
-  f32x16 dkacc[WANT_DK ? 4 : 1], dvacc[WANT_DV ? 4 : 1];
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      if (WANT_DK) dkacc[db][r] = 0.f;
-      if (WANT_DV) dvacc[db][r] = 0.f;
-    }
-
-  const int srow = tid >> 4, schunk = tid & 15;
-  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const uint16_t* qg = a.q + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.q_ss;
-  const uint16_t* gg = a.g + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8 + (int64_t)srow * a.q_ss;
-  const int64_t row16 = 16 * a.q_ss;
-  uint4 qr[4], gr[4];
-  float r_m2 = 0.f, r_rden = 0.f, r_delta = 0.f;
-  int r_seg = 0;
-#define RA_LOAD_Q_TILE(QT)                                                                              \
-  {                                                                                                     \
-    RA_LOAD_TILE(qr, qg, a.q_ss, (QT), KBM);                                                            \
-    RA_LOAD_TILE(gr, gg, a.q_ss, (QT), KBM);                                                            \
-    if (tid < KBM) {                                                                                    \
-      const int row_ = (QT) * KBM + tid;                                                                \
-      const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
-      r_m2 = max_to_log2(a.mx[st_], kMask2);                                                            \
-      r_rden = 1.f / a.den[st_];                                                                        \
-      r_delta = a.delta[st_];                                                                           \
-      if (HAS_SEG) {                                                                                    \
-        int idx_ = clamp_seg_index(((long long)mv.q_start + row_ / mv.qc) * mv.qc, mv.qc, mv.seg_len, row_ % mv.qc); \
-        r_seg = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
-      }                                                                                                 \
-    }                                                                                                   \
-  }
-#define RA_STORE_Q_TILE(BUF)                                                                            \
-  {                                                                                                     \
-    RA_STORE_TILE(qr, Qs[BUF]);                                                                         \
-    RA_STORE_TILE(gr, Gs[BUF]);                                                                         \
-    if (tid < KBM) {                                                                                    \
-      st_m2[BUF][tid] = r_m2; st_rden[BUF][tid] = r_rden; st_delta[BUF][tid] = r_delta;                 \
-      if (HAS_SEG) st_seg[BUF][tid] = r_seg;                                                            \
-    }                                                                                                   \
-  }
-  RA_LOAD_Q_TILE(qt_first);
-  RA_STORE_Q_TILE(0);
-  __syncthreads();
-
-  int n_off[8], t_off[4][2];
-  RA_LANE_OFFSETS(n_off, t_off);
-
-  for (int qt = qt_first; qt < qt_end; qt++) {
-    const int cur = (qt - qt_first) & 1;
-    RA_LOAD_Q_TILE(min(qt + 1, qt_end - 1));
-    const int gq_tile = gq_base + qt * KBM;
-    const bool need_mask = HAS_SEG || HAS_BIAS || (gq_tile < qlim_wave);
-
-#pragma unroll
-    for (int qb = 0; qb < 2; qb++) {
-      f32x16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
-      const uint16_t* qp = &Qs[cur][qb * 32 * TROW];
-      const uint16_t* gp = &Gs[cur][qb * 32 * TROW];
-#pragma unroll
-      for (int t = 0; t < 8; t++) {
-        bf16x8 qa = *(const bf16x8*)(qp + n_off[t]);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[t], s, 0, 0, 0);          // S = Q K^T
-      }
-      if (WANT_DK) {
-#pragma unroll
-        for (int t = 0; t < 8; t++) {
-          bf16x8 ga = *(const bf16x8*)(gp + n_off[t]);
-          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ga, vf[t], dp, 0, 0, 0);      // dP = dO V^T
-        }
-      }
-      bf16x8 pf[2], dsf[2];
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        const int qrow0 = qb * 32 + g * 8 + hi * 4;          // rows qrow0 .. +3 of the tile
-        const f32x4 vm2 = *(const f32x4*)&st_m2[cur][qrow0];
-        const f32x4 vrd = *(const f32x4*)&st_rden[cur][qrow0];
-        const f32x4 vdl = *(const f32x4*)&st_delta[cur][qrow0];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int r = g * 4 + e;
-          float p;
-          if (!need_mask) {
-            p = fast_exp2(fmaf(s[r], c, -vm2[e])) * vrd[e];
-          } else {
-            float x = s[r] * c;
-            if (HAS_BIAS) x += bias2;
-            bool masked = (gq_tile + qrow0 + e < qlim);
-            if (HAS_SEG) masked = masked || (st_seg[cur][qrow0 + e] != seg_k);
-            x = masked ? kMask2 : x;
-            p = fast_exp2(x - vm2[e]) * vrd[e];
-          }
-          if (WANT_DV) pf[r >> 3][r & 7] = (__bf16)p;
-          if (WANT_DK) dsf[r >> 3][r & 7] = (__bf16)(p * (dp[r] - vdl[e]));
-        }
-      }
-      // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over these 32 query rows)
-#pragma unroll
-      for (int t = 0; t < 2; t++)
-#pragma unroll
-        for (int db = 0; db < 4; db++) {
-          if (WANT_DV) {
-            const uint16_t* gtp = &Gs[cur][(qb * 32 + t * 16) * TROW];
-            s16x4 g0 = lds_read_tr(gtp + t_off[db][0]);
-            s16x4 g1 = lds_read_tr(gtp + t_off[db][1]);
-            s16x8 gv = __builtin_shufflevector(g0, g1, 0, 1, 2, 3, 4, 5, 6, 7);
-            dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, gv), pf[t], dvacc[db], 0, 0, 0);
-          }
-          if (WANT_DK) {
-            const uint16_t* qtp = &Qs[cur][(qb * 32 + t * 16) * TROW];
-            s16x4 q0v = lds_read_tr(qtp + t_off[db][0]);
-            s16x4 q1v = lds_read_tr(qtp + t_off[db][1]);
-            s16x8 qv = __builtin_shufflevector(q0v, q1v, 0, 1, 2, 3, 4, 5, 6, 7);
-            dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qv), dsf[t], dkacc[db], 0, 0, 0);
-          }
-        }
-    }
-    RA_STORE_Q_TILE(cur ^ 1);
-    __syncthreads();
-  }
-#undef RA_LOAD_Q_TILE
-#undef RA_STORE_Q_TILE
-
-  // dk += acc / sqrt(D) (:231), dv += acc (:232); this workgroup owns its key rows
-  const float rscale = 1.f / sqrtf((float)HD);
-  const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      if (WANT_DK) {
-        float* pk = a.dk + ooff + db * 32 + g * 8;
-        f32x4 tk = *(const f32x4*)pk;
-#pragma unroll
-        for (int e = 0; e < 4; e++) tk[e] += dkacc[db][g * 4 + e] * rscale;
-        *(f32x4*)pk = tk;
-      }
-      if (WANT_DV) {
-        float* pv = a.dv + ooff + db * 32 + g * 8;
-        f32x4 tv = *(const f32x4*)pv;
-#pragma unroll
-        for (int e = 0; e < 4; e++) tv[e] += dvacc[db][g * 4 + e];
-        *(f32x4*)pv = tv;
-      }
-    }
-}
 
 // ------------------------------------------------------------------ dK / dV, wave-specialised
 // 8 wavefronts per workgroup, 128 keys: pair i = (wave i, wave i + 4) shares a SIMD and owns keys
@@ -2210,6 +1445,475 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #undef RA_WS_STORE_V
 }
 
+// ------------------------------------------------------------------ forward, wave-specialised
+// Same structure as the dQ kernel above: 128 query rows per workgroup, pair i = (wave i, wave i + 4) owns
+// rows 32 i .. 32 i + 31.  The producer runs S^T = K Q^T and the online softmax (running max and sum are
+// per-lane scalars: a lane owns a query column) and leaves P^T, rounded to bf16, in LDS together with the
+// factor by which the output accumulator has to shrink when the reference max moved; the consumer runs
+// O^T += V^T P^T one block of 32 keys behind.
+template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
+__global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[3 * WS_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[3 * WS_TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t Ds[4][2][WS_PD];        // [pair][buffer] P^T as [q][key]
+  __shared__ float al[4][2][32];     // [pair][buffer][query]: factor the consumer applies to O before adding the block
+  __shared__ float fixs[4][32];      // [pair][query]: final factor (lazy reference max -> exact max)
+  __shared__ int seg_ks[3][FBN];
+  __shared__ float bias_ks[3][FBN];
+
+  MaskView mv = a.mv;
+  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
+  const int nqt = a.Sq / FBM;
+  // XCD x takes the contiguous range x of (batch, head, query tile) triples: the workgroups resident on
+  // one XCD then stream the same K / V tiles of one head through that XCD's L2 at the same time
+  const int per_xcd = (a.B * a.H * nqt + 7) >> 3;
+  int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (wg >= a.B * a.H * nqt) return;
+  const int qt = nqt - 1 - (wg % nqt);     // latest query tiles (most keys under causal) first
+  wg /= nqt;
+  const int h = wg % a.H, b = wg / a.H;
+  const int q0 = qt * FBM;
+  const int qrow = q0 + pair * 32 + lo;
+
+  const int qi = q0 / mv.qc;
+  int kend = mv.run_prefix_keys(qi, a.Skv);
+  const int gq0 = (int)mv.global_q(q0);
+  const int gk0_shard = (int)mv.global_k(0);
+  if (mv.cbs > 0 && mv.skip_tiles) {
+    long long lim = ((long long)(gq0 + FBM - 1) / mv.cbs + 1) * mv.cbs;
+    long long n = lim - gk0_shard;
+    if (n < kend) kend = n > 0 ? (int)n : 0;
+  }
+  int ntiles = (kend + FBN - 1) / FBN;
+  int k_base = 0;
+  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
+    __shared__ int hull2[2];
+    int slo, shi, t_first, t_last;
+    seg_rows_range(mv, b, gq0, FBM, slo, shi);
+    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
+    k_base = t_first * FBN;
+    ntiles = t_last - t_first;
+  }
+  if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {
+    __shared__ int khull2[2];
+    int t_first, t_last;
+    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, FBM / 64, (gk0_shard + k_base) / 64, ntiles, khull2, tid, 512,
+                    t_first, t_last);
+    k_base += t_first * FBN;
+    ntiles = t_last - t_first;
+  }
+  if (ntiles == 0) {           // no key tile runs for these rows: the carry stays as it is
+    if (a.carry_is_initial) {
+      const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+      float* np0 = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
+      if (role == 1) {
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) *(f32x4*)(np0 + db * 32 + g * 8) = f32x4{0.f, 0.f, 0.f, 0.f};
+      } else if (hi == 0) {
+        a.den[st0] = 0.f; a.mx[st0] = RA_NEG_INF;
+      }
+    }
+    return;
+  }
+  const int gk0 = gk0_shard + k_base;
+  const float c = kLog2e / sqrtf((float)HD);
+  const float kMask2 = mv.mask_min;
+
+  // ---- staging of the K / V tiles through registers, by the consumer waves (which have registers and
+  // issue slots to spare): tile t + 2 is stored in step 2t + 1, two steps after it was requested
+  const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
+  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const int64_t sg_off = (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
+  const uint16_t* sgk = a.k + sg_off;
+  const uint16_t* sgv = a.v + sg_off;
+  const int64_t row16 = 16 * a.kv_ss;
+  uint4 sk0, sk1, sk2, sk3, sv0, sv1, sv2, sv3;
+  int seg_r = 0;
+  float bias_r = 0.f;
+  // K half (with the key info) and V half of a tile are staged separately so that the requests and the
+  // LDS writes of a tile spread over two steps
+#define RA_WS_LOAD_K(T)                                                                                 \
+  {                                                                                                     \
+    const int t_ = min((T), ntiles - 1);                                                                \
+    const uint16_t* pk_ = sgk + (int64_t)t_ * FBN * a.kv_ss;                                            \
+    sk0 = *(const uint4*)(pk_); sk1 = *(const uint4*)(pk_ + row16);                                     \
+    sk2 = *(const uint4*)(pk_ + 2 * row16); sk3 = *(const uint4*)(pk_ + 3 * row16);                     \
+    if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
+      const int kj_ = k_base + t_ * FBN + stid;                                                         \
+      if (HAS_SEG) {                                                                                    \
+        int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
+      }                                                                                                 \
+      if (HAS_BIAS) {                                                                                   \
+        float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
+        if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
+        bias_r = bv_ * kLog2e / c;   /* the S accumulators start from it */                             \
+      }                                                                                                 \
+    }                                                                                                   \
+  }
+#define RA_WS_LOAD_V(T)                                                                                 \
+  {                                                                                                     \
+    const int t_ = min((T), ntiles - 1);                                                                \
+    const uint16_t* pv_ = sgv + (int64_t)t_ * FBN * a.kv_ss;                                            \
+    sv0 = *(const uint4*)(pv_); sv1 = *(const uint4*)(pv_ + row16);                                     \
+    sv2 = *(const uint4*)(pv_ + 2 * row16); sv3 = *(const uint4*)(pv_ + 3 * row16);                     \
+  }
+#define RA_WS_STORE_K(BUF)                                                                              \
+  {                                                                                                     \
+    uint16_t* dk_ = Ks + (BUF) * WS_TILE + s_off;                                                       \
+    *(uint4*)(dk_) = sk0; *(uint4*)(dk_ + 16 * TROW) = sk1;                                             \
+    *(uint4*)(dk_ + 32 * TROW) = sk2; *(uint4*)(dk_ + 48 * TROW) = sk3;                                 \
+    if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
+      if (HAS_SEG) seg_ks[BUF][stid] = seg_r;                                                           \
+      if (HAS_BIAS) bias_ks[BUF][stid] = bias_r;                                                        \
+    }                                                                                                   \
+  }
+#define RA_WS_STORE_V(BUF)                                                                              \
+  {                                                                                                     \
+    uint16_t* dv_ = Vs + (BUF) * WS_TILE + s_off;                                                       \
+    *(uint4*)(dv_) = sv0; *(uint4*)(dv_ + 16 * TROW) = sv1;                                             \
+    *(uint4*)(dv_ + 32 * TROW) = sv2; *(uint4*)(dv_ + 48 * TROW) = sv3;                                 \
+  }
+#ifdef RA_TRACE
+  const bool trace_on = blockIdx.x == 0;
+  int trace_n = 0;
+#endif
+  if (role == 1) {
+    RA_WS_LOAD_K(0); RA_WS_LOAD_V(0);
+    RA_WS_STORE_K(0); RA_WS_STORE_V(0);
+    RA_WS_LOAD_K(1); RA_WS_LOAD_V(1);
+    RA_WS_STORE_K(1); RA_WS_STORE_V(1);
+    RA_WS_LOAD_K(2); RA_WS_LOAD_V(2);
+  }
+  __syncthreads();
+
+  if (role == 0) {
+    // =========================== producer: S^T -> online softmax -> P^T
+    const int gq = gq0 + pair * 32 + lo;
+    const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
+    const int klim_wave = __builtin_amdgcn_readfirstlane(
+        mv.cbs > 0 ? (int)min((long long)((gq0 + pair * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff);
+    int seg_q = 0;
+    if (HAS_SEG) {
+      int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
+      seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
+    }
+    const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
+    bf16x8 qf[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
+    const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+    // running max (log2 domain; m2 is the lazy reference the probabilities are taken against, m_true the
+    // exact one) and this half-row's share of the running sum
+    float m2 = RA_NEG_INF, l = 0.f;
+    if (!a.carry_is_initial) {
+      m2 = max_to_log2(a.mx[st], kMask2);
+      l = hi == 0 ? a.den[st] : 0.f;
+    }
+    float m_true = m2, ps = 0.f;
+    constexpr float kLazy = 16.f;
+    int n_off[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);
+    uint16_t* const dw = &Ds[pair][0][lo * WS_PSTR + hi * 4];
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+#define RA_WS_INIT(SN, BUF, BLK)                                                                        \
+  _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                       \
+    f32x4 b4_ = {0.f, 0.f, 0.f, 0.f};                                                                   \
+    if (HAS_BIAS) b4_ = *(const f32x4*)&bias_ks[BUF][(BLK) * 32 + g * 8 + hi * 4];                      \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) SN[g * 4 + e] = b4_[e];                               \
+  }
+#define RA_WS_AREAD(G, KA, BUF, BLK)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < 2; i++)                                                         \
+    KA[i] = *(const bf16x8*)(Ks + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);
+#define RA_WS_AMFMA(G, KA, SN)                                                                          \
+  _Pragma("unroll") for (int i = 0; i < 2; i++)                                                         \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[2 * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T (:134) */
+    // The block's 32 keys x this lane's query: the running max first (group 0), then eight keys
+    // (registers 4G .. 4G+3 of both halves) of P^T per group.  (:138-144)
+#define RA_WS_ROWMAX(SC, BUF, BLK, PB, MASKED)                                                          \
+  {                                                                                                     \
+    float alpha_ = 1.f;                                                                                 \
+    if (!(MASKED)) {                                                                                    \
+      float mxv_ = SC[0];                                                                               \
+      _Pragma("unroll") for (int r = 1; r < 16; r++) mxv_ = fmaxf(mxv_, SC[r]);                         \
+      mxv_ = max_xor32(mxv_);                                                                           \
+      m_true = fmaxf(m_true, mxv_ * c);                                                                 \
+      if (__builtin_amdgcn_ballot_w64(m_true - m2 > kLazy) != 0) {   /* rescale only on a large jump */ \
+        alpha_ = fast_exp2(m2 - m_true);                                                                \
+        m2 = m_true;                                                                                    \
+        l *= alpha_;                                                                                    \
+      }                                                                                                 \
+    } else {                                                                                            \
+      float mxv_ = RA_NEG_INF;                                                                          \
+      _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                  \
+        const int kr_ = (BLK) * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);                                   \
+        float x_ = SC[r] * c;                                                                           \
+        bool masked_ = (gk_tile + kr_ >= klim);                                                         \
+        if (HAS_SEG) masked_ = masked_ || (seg_ks[BUF][kr_] != seg_q);                                  \
+        if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1);    \
+        x_ = masked_ ? kMask2 : x_;                                                                     \
+        SC[r] = x_;                                                                                     \
+        mxv_ = fmaxf(mxv_, x_);                                                                         \
+      }                                                                                                 \
+      mxv_ = max_xor32(mxv_);                                                                           \
+      m_true = fmaxf(m_true, mxv_);                                                                     \
+      const float m_new_ = fmaxf(m2, mxv_);                                                             \
+      alpha_ = fast_exp2(m2 - m_new_);                                                                  \
+      m2 = m_new_;                                                                                      \
+      l *= alpha_;                                                                                      \
+    }                                                                                                   \
+    if (hi == 0) al[pair][PB][lo] = alpha_;                                                             \
+  }
+#define RA_WS_VECTOR(G, SC, BUF, BLK, PB, MASKED)                                                       \
+  {                                                                                                     \
+    if ((G) == 0) RA_WS_ROWMAX(SC, BUF, BLK, PB, MASKED);                                               \
+    bf16x4 d4;                                                                                          \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
+      const float p = (MASKED) ? fast_exp2(SC[(G) * 4 + e] - m2) : fast_exp2(fmaf(SC[(G) * 4 + e], c, -m2)); \
+      ps += p;                                                                                          \
+      d4[e] = (__bf16)p;                                                                                \
+    }                                                                                                   \
+    *(bf16x4*)(dw + (PB) * WS_PD + (G) * 8) = d4;                                                       \
+    if ((G) == 3) { l += ps; ps = 0.f; }                                                                \
+  }
+    // one step: vector work of block BLK of buffer BUF (accumulators SC, DPC) in four groups of eight
+    // keys, each next to a quarter of the products of block NBLK of buffer NBUF (into SN, DPN).  The
+    // K / V operands of a quarter are requested from LDS three quarters ahead - the last three of a step
+    // request the first three quarters of the following step's block NNBLK of buffer NNBUF - which
+    // covers the LDS latency under load.
+#define RA_WS_PRODUCE(SC, SN, BUF, BLK, NBUF, NBLK, NNBUF, NNBLK, PB, MASKED)                           \
+  {                                                                                                     \
+    RA_WS_INIT(SN, NBUF, NBLK);                                                                         \
+    _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                     \
+      if (g == 0) { RA_WS_AREAD(3, ka[3], NBUF, NBLK); }                                                \
+      else { RA_WS_AREAD(g - 1, ka[g - 1], NNBUF, NNBLK); }                                             \
+      RA_WS_AMFMA(g, ka[g], SN);                                                                        \
+      RA_WS_VECTOR(g, SC, BUF, BLK, PB, MASKED);                                                        \
+      __builtin_amdgcn_sched_barrier(0);                                                                \
+    }                                                                                                   \
+  }
+
+    f32x16 s_a, s_b;
+    bf16x8 ka[4][2];
+    RA_WS_INIT(s_a, 0, 0);
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      RA_WS_AREAD(g, ka[0], 0, 0);
+      RA_WS_AMFMA(g, ka[0], s_a);
+    }
+#pragma unroll
+    for (int g = 0; g < 3; g++) RA_WS_AREAD(g, ka[g], 0, 1);
+
+    // Under a causal mask the tiles that need no masking come first: one loop for them, one for the rest
+    // (which also takes every tile when segment ids or a bias are present).
+    // Which key tiles need no masking at all: below the causal limit of every row, keys all of this wave's
+    // single segment id, packed keep summary "all kept".  They form (at most) one run [t_a, t_b) in the
+    // cases that matter - document interiors, the part of a causal row left of the diagonal - and get a
+    // loop of their own; the tiles before and after take the masked loop.
+    const int t_causal = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
+    const uint64_t* kw_ptr = nullptr;
+    const uint8_t* ks_ptr = nullptr;
+    uint64_t kw_cur = 0, kw_nxt = 0;
+    if (HAS_KEEP) {
+      ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
+               (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
+      kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
+               mv.keep_q0 + qrow;
+    }
+    const int2* smm_ptr = nullptr;
+    bool sq_uniform = false;
+    int sq_id = 0;
+    if (HAS_SEG && mv.seg_mm) {
+      smm_ptr = (const int2*)(mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2);
+      const int2 qmm = smm_ptr[min((gq0 + pair * 32) / RA_SEG_TILE, mv.seg_tiles - 1)];
+      sq_uniform = qmm.x == qmm.y;
+      sq_id = qmm.x;
+    }
+    int t_a = ntiles, t_b = ntiles;
+    for (int base = 0; base < ntiles; base += 64) {
+      const int tt = base + lane;
+      bool ok = tt < t_causal;
+      if (HAS_SEG && ok) {
+        ok = sq_uniform;
+        if (ok) {
+          const int2 kmm = smm_ptr[min(gk0 / RA_SEG_TILE + tt, mv.seg_tiles - 1)];
+          ok = kmm.x == sq_id && kmm.y == sq_id;
+        }
+      }
+      if (HAS_KEEP && ok) ok = ks_ptr[tt] == 2;
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(ok);
+      unsigned long long stop;      // tiles of this group of 64 that end the run
+      if (t_a == ntiles) {
+        if (!m) continue;
+        const int f = __builtin_ctzll(m);
+        t_a = base + f;
+        stop = ~m & (~0ULL << f);
+      } else {
+        stop = ~m;
+      }
+      if (stop) { t_b = min(ntiles, base + (int)__builtin_ctzll(stop)); break; }
+    }
+    t_a = __builtin_amdgcn_readfirstlane(t_a);
+    t_b = __builtin_amdgcn_readfirstlane(t_a == ntiles ? ntiles : t_b);
+    if (HAS_KEEP) kw_nxt = kw_ptr[(int64_t)min(t_a == 0 ? t_b : 0, ntiles - 1) * mv.keep_Q];
+    int cur = 0;
+#define RA_WS_TILE(MASKED)                                                                              \
+  {                                                                                                     \
+    const int nxt = cur == 2 ? 0 : cur + 1;                                                             \
+    const int gk_tile = gk0 + t * FBN;                                                                  \
+    (void)gk_tile;                                                                                      \
+    if (HAS_KEEP && (MASKED)) {        /* this tile's word; request the next tile's */                  \
+      kw_cur = kw_nxt >> (4 * hi);                                                                      \
+      kw_nxt = kw_ptr[(int64_t)min(t + 1 == t_a ? t_b : t + 1, ntiles - 1) * mv.keep_Q];                \
+    }                                                                                                   \
+    /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
+    RA_TRACE_MARK();                                                                                    \
+    RA_WS_PRODUCE(s_a, s_b, cur, 0, cur, 1, nxt, 0, 0, MASKED);                                         \
+    RA_TRACE_MARK();                                                                                    \
+    __syncthreads();                                                                                    \
+    /* step 2t + 1: vector work of block 1, products of block 0 of tile t + 1 (the last tile computes  \
+       a block that is never used) */                                                                   \
+    RA_TRACE_MARK();                                                                                    \
+    RA_WS_PRODUCE(s_b, s_a, cur, 1, nxt, 0, nxt, 1, 1, MASKED);                                         \
+    RA_TRACE_MARK();                                                                                    \
+    __syncthreads();                                                                                    \
+    cur = nxt;                                                                                          \
+  }
+    int t = 0;
+    for (; t < t_a; t++) RA_WS_TILE(true);
+    for (; t < t_b; t++) RA_WS_TILE(false);
+    for (; t < ntiles; t++) RA_WS_TILE(true);
+#undef RA_WS_TILE
+    __syncthreads();      // step 2 ntiles: the consumer's last block
+    // bring the carry to the exact running max (:138) and hand the factor to the consumer
+    const float fix = (m_true == m2) ? 1.f : fast_exp2(m2 - m_true);
+    m2 = m_true;
+    l *= fix;
+    if (hi == 0) fixs[pair][lo] = fix;
+    __syncthreads();
+    l += xor32(l);
+    if (hi == 0) {
+      a.den[st] = l;
+      a.mx[st] = max_from_log2(m2, kMask2);
+    }
+#undef RA_WS_ROWMAX
+#undef RA_WS_INIT
+#undef RA_WS_AREAD
+#undef RA_WS_AMFMA
+#undef RA_WS_VECTOR
+#undef RA_WS_PRODUCE
+  } else {
+    // =========================== consumer: O^T += V^T P^T   (:141-143)
+    f32x16 acc[4];
+    float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
+    if (a.carry_is_initial) {
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+    } else {
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const f32x4 t4 = *(const f32x4*)(nump + db * 32 + g * 8);
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[db][g * 4 + e] = t4[e];
+        }
+    }
+    int t_off[4][2];
+    {
+      const int i = lane & 15, rr = (i >> 2) + 8 * hi, c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
+#pragma unroll
+      for (int db = 0; db < 4; db++) {
+        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz(rr)) << 3) + half * 4;
+        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz(rr + 4)) << 3) + half * 4;
+      }
+    }
+    const uint16_t* const dr = &Ds[pair][0][lo * WS_PSTR + hi * 8];   // B operand: query column lo, 8 keys
+
+    // keys 16 K .. 16 K + 15 of block BLK of buffer BUF, transposed
+#define RA_WS_CREAD(K, F, BUF, BLK)                                                                     \
+  {                                                                                                     \
+    const uint16_t* tp_ = Vs + (BUF) * WS_TILE + ((BLK) * 32 + (K) * 16) * TROW;                        \
+    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+      const s16x4 x0_ = lds_read_tr(tp_ + t_off[db][0]);                                                \
+      const s16x4 x1_ = lds_read_tr(tp_ + t_off[db][1]);                                                \
+      F[db] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0_, x1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
+    }                                                                                                   \
+  }
+#define RA_WS_CMFMA(F, BOP)                                                                             \
+  _Pragma("unroll") for (int db = 0; db < 4; db++)                                                      \
+    if (!RA_ABL_WS_NOCONS) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
+    // fa holds the first 16 keys of the block on entry and, on exit, those of block NBLK of buffer NBUF
+#define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
+  {                                                                                                     \
+    const bf16x8 d0_ = *(const bf16x8*)(dr + (PB) * WS_PD);                                             \
+    const bf16x8 d1_ = *(const bf16x8*)(dr + (PB) * WS_PD + 16);                                        \
+    const float alpha_ = al[pair][PB][lo];                                                              \
+    if (__builtin_amdgcn_ballot_w64(alpha_ != 1.f) != 0) {                                              \
+      _Pragma("unroll") for (int db = 0; db < 4; db++)                                                  \
+        _Pragma("unroll") for (int r = 0; r < 16; r++) acc[db][r] *= alpha_;                            \
+    }                                                                                                   \
+    RA_WS_CREAD(1, fb, BUF, BLK);                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(fa, d0_);                                                                               \
+    RA_WS_CREAD(0, fa, NBUF, NBLK);                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_WS_CMFMA(fb, d1_);                                                                               \
+  }
+    bf16x8 fa[4], fb[4];
+    int cur = 0;
+    RA_WS_CREAD(0, fa, 0, 0);
+    __syncthreads();      // step 0
+    for (int t = 0; t < ntiles; t++) {
+      const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;
+      // tile t + 2 goes to the buffer that held tile t - 1 (K in step 2t + 1, V in step 2t + 2) and
+      // tile t + 3 is requested
+      RA_TRACE_MARK();
+      RA_WS_STORE_K(prv);
+      RA_TRACE_MARK2();
+      RA_WS_LOAD_K(t + 3);
+      RA_TRACE_MARK2();
+      RA_WS_CONSUME(cur, 0, 0, cur, 1);
+      RA_TRACE_MARK();
+      __syncthreads();
+      RA_TRACE_MARK();
+      RA_WS_STORE_V(prv);
+      RA_WS_LOAD_V(t + 3);
+      RA_WS_CONSUME(cur, 1, 1, nxt, 0);
+      RA_TRACE_MARK();
+      __syncthreads();
+      cur = nxt;
+    }
+#undef RA_WS_CREAD
+#undef RA_WS_CMFMA
+#undef RA_WS_CONSUME
+
+    __syncthreads();      // the producer's final factor
+    const float fix = fixs[pair][lo];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4 t4;
+#pragma unroll
+        for (int e = 0; e < 4; e++) t4[e] = acc[db][g * 4 + e] * fix;
+        *(f32x4*)(nump + db * 32 + g * 8) = t4;
+      }
+  }
+#undef RA_WS_LOAD_K
+#undef RA_WS_LOAD_V
+#undef RA_WS_STORE_K
+#undef RA_WS_STORE_V
+}
+
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
@@ -2222,7 +1926,7 @@ static bool keep_ok(const ra_mask& m, bool shape_ok) {
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
   const ra_mask& m = p->mask;
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
-         keep_ok(m, m.query_chunk_size % PBM == 0) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
+         keep_ok(m, true) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
          aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator);
 }
@@ -2239,7 +1943,9 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   a.carry_is_initial = p->carry_is_initial;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool keep = p->mask.keep != nullptr;      // packed form checked by attn_fwd_mfma_supported
-  if (p->mask.query_chunk_size % PBM == 0 && (keep || !getenv("RA_FWD_NO_PINGPONG"))) {
+  // chunks of a multiple of 256 rows: the ping-pong kernel (256 rows per workgroup, half the K / V traffic per
+  // row); other multiples of 128: the wave-specialised kernel
+  if (p->mask.query_chunk_size % PBM == 0 && !getenv("RA_FWD_WAVE_SPEC")) {
     const long long nwg2 = (long long)(p->Sq / PBM) * p->H * p->B;
     RA_REQUIRE(nwg2 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
     dim3 grid2((unsigned)nwg2), block2(512);
@@ -2251,14 +1957,15 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
     RA_CHECK_LAUNCH("attn_fwd_pp");
     return RA_OK;
   }
-  const long long nwg = (long long)(p->Sq / FBM) * p->H * p->B;
-  RA_REQUIRE(nwg < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
-  dim3 grid((unsigned)nwg), block(256);
-  if (seg && bias) attn_fwd_mfma_kernel<true, true><<<grid, block, 0, s>>>(a);
-  else if (seg) attn_fwd_mfma_kernel<true, false><<<grid, block, 0, s>>>(a);
-  else if (bias) attn_fwd_mfma_kernel<false, true><<<grid, block, 0, s>>>(a);
-  else attn_fwd_mfma_kernel<false, false><<<grid, block, 0, s>>>(a);
-  RA_CHECK_LAUNCH("attn_fwd_mfma");
+  const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
+  RA_REQUIRE(nwg3 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
+  dim3 grid3((unsigned)((nwg3 + 7) / 8 * 8)), block3(512);
+  if (keep) attn_fwd_ws_kernel<false, false, true><<<grid3, block3, 0, s>>>(a);
+  else if (seg && bias) attn_fwd_ws_kernel<true, true><<<grid3, block3, 0, s>>>(a);
+  else if (seg) attn_fwd_ws_kernel<true, false><<<grid3, block3, 0, s>>>(a);
+  else if (bias) attn_fwd_ws_kernel<false, true><<<grid3, block3, 0, s>>>(a);
+  else attn_fwd_ws_kernel<false, false><<<grid3, block3, 0, s>>>(a);
+  RA_CHECK_LAUNCH("attn_fwd_ws");
   return RA_OK;
 }
 
@@ -2284,28 +1991,16 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
   a.cache_idx = p->mask.cache_idx;
   const long long nq = (long long)(p->Sq / FBM) * p->H * p->B, nk = (long long)(p->Skv / KBN) * p->H * p->B;
   RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_mfma: grid too large");
-  dim3 gq((unsigned)nq), gk((unsigned)nk), block(256);
+  const dim3 gq((unsigned)((nq + 7) / 8 * 8)), gk((unsigned)((nk + 7) / 8 * 8)), block(512);
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool do_dkv = !(p->impl & RA_BWD_ONLY_DQ), do_dq = !(p->impl & RA_BWD_ONLY_DKV);
-  const bool use_ws = !getenv("RA_BWD_NO_WAVE_SPEC");
-#define RA_LAUNCH_BWD(SEG, BIAS)                                                         \
+#define RA_LAUNCH_BWD(...)                                                               \
   do {                                                                                   \
-    if (do_dkv && use_ws) {                                                              \
-      attn_bwd_dkv_ws_kernel<SEG, BIAS><<<dim3((gk.x + 7) / 8 * 8), dim3(512), 0, s>>>(a); \
-    } else if (do_dkv) {                                                                 \
-      attn_bwd_dkv_mfma_kernel<SEG, BIAS, true, false><<<gk, block, 0, s>>>(a);          \
-      attn_bwd_dkv_mfma_kernel<SEG, BIAS, false, true><<<gk, block, 0, s>>>(a);          \
-    }                                                                                    \
-    if (do_dq && use_ws) {                                                               \
-      attn_bwd_dq_ws_kernel<SEG, BIAS><<<dim3((gq.x + 7) / 8 * 8), dim3(512), 0, s>>>(a); \
-    } else if (do_dq) {                                                                  \
-      attn_bwd_dq_mfma_kernel<SEG, BIAS><<<gq, block, 0, s>>>(a);                        \
-    }                                                                                    \
+    if (do_dkv) attn_bwd_dkv_ws_kernel<__VA_ARGS__><<<gk, block, 0, s>>>(a);             \
+    if (do_dq) attn_bwd_dq_ws_kernel<__VA_ARGS__><<<gq, block, 0, s>>>(a);               \
   } while (0)
-  if (p->mask.keep) {        // packed boolean mask: the wave-specialised kernels only
-    if (do_dkv) attn_bwd_dkv_ws_kernel<false, false, true><<<dim3((gk.x + 7) / 8 * 8), dim3(512), 0, s>>>(a);
-    if (do_dq) attn_bwd_dq_ws_kernel<false, false, true><<<dim3((gq.x + 7) / 8 * 8), dim3(512), 0, s>>>(a);
-  } else if (seg && bias) RA_LAUNCH_BWD(true, true);
+  if (p->mask.keep) RA_LAUNCH_BWD(false, false, true);      // packed boolean mask
+  else if (seg && bias) RA_LAUNCH_BWD(true, true);
   else if (seg) RA_LAUNCH_BWD(true, false);
   else if (bias) RA_LAUNCH_BWD(false, true);
   else RA_LAUNCH_BWD(false, false);
