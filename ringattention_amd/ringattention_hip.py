@@ -190,12 +190,13 @@ class _MaskInputs:
         summary (ra_keep_pack), the form the MFMA kernels read."""
         if attn_mask.dim() != 4:
             raise ValueError("attn_mask must be 4-D (B, H, Q, K)")
-        m = (attn_mask.detach().to(device=device) != 0).to(torch.uint8).contiguous()
+        m = attn_mask.detach().to(device=device)
+        if m.dtype == torch.bool:
+            m = m.contiguous().view(torch.uint8)          # same bytes, no copy for a contiguous bool mask
+        else:
+            m = (m != 0).to(torch.uint8).contiguous()
         self.keep = m
         self.keep_strides = tuple(0 if m.shape[i] == 1 else m.stride(i) for i in range(4))
-        # a query row with no attended key keeps equal finfo.min logits (uniform weights): kernels must not
-        # skip its fully masked tiles
-        self.keep_has_empty_row = bool((m.amax(dim=3) == 0).any().item())
         self.keep_packed = None
         if q_total % 64 == 0 and k_total % 64 == 0:
             bm, hm = m.shape[0], m.shape[1]
@@ -206,7 +207,13 @@ class _MaskInputs:
             L.check(L.load().ra_keep_pack(m.data_ptr(), m.stride(0), m.stride(1), self.keep_strides[2], m.stride(3),
                                           bm, hm, q_total, k_total, bits_k.data_ptr(), bits_q.data_ptr(),
                                           summ.data_ptr(), _stream()), "ra_keep_pack")
+            # a query row with no attended key keeps equal finfo.min logits (uniform weights): kernels must
+            # not skip its fully masked tiles.  Read off the packed words (an eighth of the mask's bytes).
+            row_has_key = (bits_k.view(bm, hm, k_total // 64, q_total) != 0).any(dim=2)
+            self.keep_has_empty_row = not bool(row_has_key.all().item())
             self.keep_packed = (bits_k, bits_q, summ, q_total, k_total)
+        else:
+            self.keep_has_empty_row = bool((m.amax(dim=3) == 0).any().item())
 
     def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip):
         m = L.RaMask()
