@@ -181,21 +181,35 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
 #undef RA_A_LDS
 #undef RA_B_LDS
 
-  // epilogue: lane holds column n = lo of each 32x32 block, rows 8*(r/4) + 4*hi + r%4
+  // epilogue.  A lane holds column n = lo of each 32x32 block, rows 8*(r/4) + 4*hi + r%4: written straight to
+  // memory that is one 4-byte access per lane and register.  Each block goes through a private 32 x 36 float
+  // patch of LDS instead (the operand tiles are dead by now) and leaves as 16 bytes per lane: rows of 128
+  // bytes, a quarter of the memory instructions.
+  __syncthreads();
+  static_assert(sizeof(As) >= (size_t)NT / 64 * 32 * 36 * sizeof(float), "operand tile too small for the epilogue patches");
+  float* patch = (float*)&As[0][0] + wave * (32 * 36);
+  const int er = lane >> 3, ec = (lane & 7) * 4;          // this lane's row (of 8 per pass) and first column
 #pragma unroll
   for (int i = 0; i < MB; i++)
 #pragma unroll
     for (int j = 0; j < NB; j++) {
-      const int n = n0 + wn * WN + j * 32 + lo;
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int m = m0 + wm * WM + i * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-        const int64_t o = (int64_t)m * g.N + n;
+      for (int r = 0; r < 16; r++) patch[((r >> 2) * 8 + hi * 4 + (r & 3)) * 36 + lo] = acc[i][j][r];
+#pragma unroll
+      for (int pass = 0; pass < 4; pass++) {
+        const int row = pass * 8 + er;
+        const float4 v = *(const float4*)&patch[row * 36 + ec];
+        const int64_t o = (int64_t)(m0 + wm * WM + i * 32 + row) * g.N + n0 + wn * WN + j * 32 + ec;
         if (g.c_f32) {
-          float* c = (float*)g.C + o;
-          *c = g.beta_one ? *c + acc[i][j][r] : acc[i][j][r];
+          float4* c = (float4*)((float*)g.C + o);
+          float4 w = v;
+          if (g.beta_one) { const float4 old = *c; w.x += old.x; w.y += old.y; w.z += old.z; w.w += old.w; }
+          *c = w;
         } else {
-          ((uint16_t*)g.C)[o] = f32_to_bf16(acc[i][j][r]);
+          uint2 w;
+          w.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+          w.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+          *(uint2*)((uint16_t*)g.C + o) = w;
         }
       }
     }
