@@ -160,11 +160,11 @@ def bench_attention(args, ring):
 
 
 def cpu_baseline_attention():
-    """The CPU oracle (torch-CPU fp32, the reference's loop structure) on 4 of the 32 heads of the
+    """The CPU oracle (torch-CPU fp32, the reference's loop structure) on 8 of the 32 heads of the
     attn32k workload at full S=32768: forward + backward, fp32 logits, chunks 512/512."""
     import torch
     from oracle import ringattention_oracle as O
-    S, D, Hc = 32768, 128, 4
+    S, D, Hc = 32768, 128, 8
     cores = os.cpu_count() or 1
     cores = min(cores, 16)
     torch.set_num_threads(cores)
@@ -177,7 +177,7 @@ def cpu_baseline_attention():
     dt = time.perf_counter() - t0
     flops = 14.0 * D * (S * (S + 1) / 2) * Hc
     return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": "4 heads (of 32) at full S=32768, fwd+bwd, %.1f s" % dt}
+            "sample": "8 heads (of 32) at full S=32768, fwd+bwd, %.1f s" % dt}
 
 
 # --------------------------------------------------------------------------- decode workload
