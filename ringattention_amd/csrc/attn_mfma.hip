@@ -1917,10 +1917,12 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
-// a boolean keep mask is taken in packed form only, alone (no bias, no segment ids), by the 8-wave kernels
+// a boolean keep mask is taken in packed form only and alone (no bias, segment ids or causal block size next to it:
+// ring_attention_inference has none of them, and the generic kernels serve any combination)
 static bool keep_ok(const ra_mask& m, bool shape_ok) {
   if (!m.keep) return true;
-  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids && shape_ok;
+  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids && m.causal_block_size == 0 &&
+         shape_ok;
 }
 
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {

@@ -89,3 +89,8 @@ def test_invalid_arguments_return_codes_without_gpu():
     assert lib.ra_attn_fwd_block(ctypes.byref(p), None) == _lib.RA_ERR_INVALID
     assert lib.ra_decode_fwd(None, None) == _lib.RA_ERR_INVALID
     assert lib.ra_decode_workspace_bytes(16, 1024, 32, 128, 4) == 16 * 32 * 4 * 130 * 4
+    # ra_keep_pack validates before touching the device
+    assert lib.ra_keep_pack(None, 0, 0, 0, 1, 1, 1, 64, 64, None, None, None, None) == _lib.RA_ERR_INVALID
+    one = ctypes.c_void_p(16)      # any non-null address: the shape check comes before any use
+    assert lib.ra_keep_pack(one, 0, 0, 100, 1, 1, 1, 100, 64, one, one, one, None) == _lib.RA_ERR_UNSUPPORTED
+    assert b"multiples of 64" in lib.ra_last_error()
