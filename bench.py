@@ -23,7 +23,7 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters'
 # reading for the 1 GiB copy of --workload copy) at the default sizes of each workload
-MEASURED_TRAFFIC = {"attn_fwd_pp_kernel": 7.30e9, "attn_bwd_dkv_ws_kernel": 6.28e9, "attn_bwd_dq_ws_kernel": 4.56e9,
+MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.48e9, "attn_bwd_dkv_ws_kernel": 6.29e9, "attn_bwd_dq_ws_kernel": 4.28e9,
                     "decode_split_kernel": 68.88e9}
 
 
@@ -128,7 +128,7 @@ def bench_attention(args, ring):
             qd, kd, vd = q.detach(), k.detach(), v.detach()
             fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (num, den, mx), 0, 0, None, None, 1, 512, 512,
                                                       _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True)
-            kern["attn_fwd_pp_kernel"] = (_event_ms(fwd, 5), flops_fwd)
+            kern["attn_fwd_ws_kernel"] = (_event_ms(fwd, 5), flops_fwd)
             out = torch.empty_like(qd)
             rh._finalize(num, den, out)
             delta = rh._bwd_delta(do, out)
@@ -337,7 +337,7 @@ def bench_inference(args):
             "config": {"workload": "inference", "B": B, "H": H, "S": S, "D": D, "virtual_ring": n,
                        "mask": "causal and 1/16 key padding, boolean (1,1,S,S)",
                        "flop_convention": "4*D fwd + 10*D bwd per attended (q,k) pair per head"},
-            "roofline": {"bound": "mfma", "kernel": "attn_fwd_pp_kernel + attn_bwd_dkv_ws_kernel + attn_bwd_dq_ws_kernel "
+            "roofline": {"bound": "mfma", "kernel": "attn_fwd_ws_kernel + attn_bwd_dkv_ws_kernel + attn_bwd_dq_ws_kernel "
                                                     "(packed boolean mask), whole step",
                          "achieved": round(value, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                          "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None},

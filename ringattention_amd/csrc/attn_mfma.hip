@@ -1,14 +1,16 @@
-// bf16 MFMA blockwise attention for gfx950, head size 128.
+// bf16 MFMA blockwise attention for gfx950, head size 128: forward, dK/dV and dQ of one ring step
+// (carry in / carry out; ringattention_jax.py:130-145 forward, :147-209 backward).
 //
-// Forward (one ring step, carry in / carry out; ringattention_jax.py:130-145):
-//   workgroup = 4 wavefronts = 128 query rows of one (batch, head); each wavefront owns 32 rows.
-//   K/V tiles of 64 keys are staged global -> registers -> LDS, double buffered.
-//   The logits are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16, so that
-//   (a) a lane owns one query column: the running max / sum need one cross-lane step, and
-//   (b) the fp32 accumulator layout of S^T is, after rounding to bf16, exactly the B-operand
-//       layout of the second product O^T = V^T P^T - P never goes through LDS.
-//   V^T fragments come from the row-major V tile with ds_read_b64_tr_b16 (LDS transpose read).
-//   Softmax runs in the log2 domain: p = exp2(s * log2(e)/sqrt(D) - m2).
+// All three kernels share one structure.  A workgroup of 8 wavefronts owns 128 rows of one
+// (batch, head) and walks 64-position tiles of the other operand, staged global -> registers -> LDS
+// through three tile buffers.  The 8 wavefronts are 4 pairs; wave i and wave i+4 sit on the same SIMD.
+// The producer wave of a pair computes the logits product (and dP in the backward) with
+// v_mfma_f32_32x32x16_bf16 and does all the vector work (mask, online softmax, dS), then writes the bf16
+// P / dS block to LDS; the consumer wave runs one 32-row block behind and does only the accumulation
+// products, reading P / dS and the transposed operand with ds_read_b64_tr_b16.
+// The logits are computed TRANSPOSED (S^T = K Q^T in the forward) so that a lane owns one query
+// column: the running max / sum need one cross-lane step.
+// Softmax runs in the log2 domain: p = exp2(s * log2(e)/sqrt(D) - m2).
 #include <stdlib.h>
 #include "common.hpp"
 
@@ -16,16 +18,12 @@ namespace ra {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int HD = 128;          // head size
 constexpr int FBM = 128;         // query rows per workgroup
 constexpr int FBN = 64;          // keys per tile
-constexpr int KSTR = HD + 8;     // LDS row stride of the K tile, elements: conflict-free 16-byte row reads
-constexpr int VSTR = HD + 32;    // LDS row stride of the V tile: conflict-free 4-row transpose reads
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -49,10 +47,6 @@ __device__ __forceinline__ float max_xor32(float x) {
   u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
-__device__ __forceinline__ float sum_xor32(float x) {
-  u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
 
 __device__ __forceinline__ s16x4 lds_read_tr(const uint16_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
@@ -68,7 +62,6 @@ __device__ __forceinline__ float max_from_log2(float m2, float mask_min) { retur
 // adjacent slots in sixteen different bank groups (conflict-free 4-row transpose reads).
 __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 constexpr int TROW = HD;          // elements per LDS tile row
-constexpr int KV_TILE = FBN * TROW;
 
 // Hull [first, last+1) of the 64-position tiles, among the n tiles starting at global tile gt0, whose
 // segment-id range meets [lo, hi] (ids from ra_segment_tile_ranges).  Conservative: a tile outside the
@@ -143,32 +136,7 @@ __device__ __forceinline__ int keep_leading_full(const uint8_t* sm, int64_t stri
   return n;
 }
 
-// Per-lane LDS read offsets (elements) into a swizzled tile.
-//  NAT[t]: 16-byte read of row lo, d = 16 t + 8 hi .. +8 (MFMA operand whose contraction index is d).
-//  TR[db][x]: ds_read_b64_tr_b16 address; lane i of a 16-lane group addresses tile row
-//  (i >> 2) + 4 hi + 8 x and the 8-byte unit (i & 3) of columns 32 db + 16 g .. +16, g = (lane >> 4) & 1.
-#define RA_LANE_OFFSETS(NAT, TR)                                                                        \
-  {                                                                                                     \
-    _Pragma("unroll") for (int t = 0; t < 8; t++) NAT[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);  \
-    const int i_ = lane & 15, rr_ = (i_ >> 2) + 4 * hi, c0_ = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), \
-              half_ = lane & 1;                                                                         \
-    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
-      TR[db][0] = rr_ * TROW + (((4 * db + c0_) ^ swz(rr_)) << 3) + half_ * 4;                          \
-      TR[db][1] = (rr_ + 8) * TROW + (((4 * db + c0_) ^ swz(rr_ + 8)) << 3) + half_ * 4;                \
-    }                                                                                                   \
-  }
-
-// ------------------------------------------------------------------ forward, ping-pong variant
-// 8 wavefronts per workgroup, 256 query rows: group A (waves 0-3) owns rows 0..127, group B (waves
-// 4-7) rows 128..255; wave i of each group shares SIMD i.  Time is cut into phases separated by
-// workgroup barriers.  In every phase one group runs its matrix work for a key tile j - S(j+1)^T =
-// K(j+1) Q^T and O^T += V(j)^T P(j)^T, 32 MFMAs - while the other group runs its vector work - the
-// softmax of its S - so each SIMD always has one wave feeding the matrix pipe and one feeding the
-// vector ALU.  Both groups read the same K / V tiles from LDS, one phase apart.
-//   group A: M(0) V(1) M(1) V(2) ...        group B: V(0) M(0) V(1) M(1) ...
-// K(j+2), V(j+1) are brought in by direct global->LDS loads issued at the start of phase 2j and
-// awaited before the barrier that ends phase 2j+1.
-constexpr int PBM = 256;
+// optional cycle-counter marks for timing experiments (compiled out unless RA_TRACE is defined)
 #ifdef RA_TRACE
 __device__ long long g_trace[8][4096];
 #define RA_TRACE_MARK() { if (trace_on && lane == 0 && trace_n < 4096) g_trace[wave][trace_n++] = __builtin_readcyclecounter(); }
@@ -181,404 +149,6 @@ __device__ long long g_trace[8][4096];
 #define RA_TRACE_MARK() {}
 #define RA_TRACE_MARK2() {}
 #endif
-constexpr int PP_DEPTH = 1;       // LDS fragment prefetch distance of the matrix phase, in steps of 4 MFMAs
-constexpr bool PP_PRIO = false;  // raise the wave priority during the matrix phase
-
-template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
-__global__ __launch_bounds__(512) void attn_fwd_pp_kernel(FwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][KV_TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][KV_TILE];
-  __shared__ int seg_ks[4][FBN];
-  __shared__ float bias_ks[4][FBN];
-
-  MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
-  const int grp = __builtin_amdgcn_readfirstlane(wave >> 2), w4 = wave & 3;
-  const int nqt = a.Sq / PBM;
-  int wg = blockIdx.x;
-  const int qt = nqt - 1 - (wg % nqt);       // heaviest (latest) query tiles first
-  wg /= nqt;
-  const int h = wg % a.H, b = wg / a.H;
-  const int q0 = qt * PBM;
-  const int qg0 = q0 + grp * 128;            // first row of this group
-  const int qrow = qg0 + w4 * 32 + lo;       // this lane's query row (local)
-
-  // ---- tile ranges.  The workgroup iterates over the tiles its last rows need; a group whose rows
-  // end earlier sees its extra tiles fully masked and contributes nothing there.
-  const int qi = q0 / mv.qc;                 // 256 | query_chunk_size: one chunk per workgroup
-  const int kend_chunk = mv.run_prefix_keys(qi, a.Skv);
-  const int gk0_shard = (int)mv.global_k(0);
-  const int gq_wg = (int)mv.global_q(q0);
-  int kend_wg = kend_chunk, kend_grp = kend_chunk;
-  if (mv.cbs > 0 && mv.skip_tiles) {
-    long long lim_wg = ((long long)(gq_wg + PBM - 1) / mv.cbs + 1) * mv.cbs - gk0_shard;
-    long long lim_grp = ((long long)(gq_wg + grp * 128 + 127) / mv.cbs + 1) * mv.cbs - gk0_shard;
-    if (lim_wg < kend_wg) kend_wg = lim_wg > 0 ? (int)lim_wg : 0;
-    if (lim_grp < kend_grp) kend_grp = lim_grp > 0 ? (int)lim_grp : 0;
-  }
-  int ntiles = (kend_wg + FBN - 1) / FBN;              // workgroup-uniform
-  int ntiles_grp = (kend_grp + FBN - 1) / FBN;         // tiles >= this are fully masked for the group
-  // key tiles outside the hull of those sharing a segment with these 256 rows are skipped
-  int k_base = 0;                                      // local key index of the first tile processed
-  if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
-    __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gq_wg, PBM, slo, shi);
-    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
-    k_base = t_first * FBN;
-    ntiles = t_last - t_first;
-    ntiles_grp = min(max(ntiles_grp - t_first, 0), ntiles);
-  }
-  // key tiles outside the hull of those with a kept pair for these 256 rows are skipped
-  if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {
-    __shared__ int khull2[2];
-    int t_first, t_last;
-    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, PBM / 64, (gk0_shard + k_base) / 64, ntiles, khull2, tid, 512,
-                    t_first, t_last);
-    k_base += t_first * FBN;
-    ntiles = t_last - t_first;
-    ntiles_grp = min(max(ntiles_grp - t_first, 0), ntiles);
-  }
-  const int gk0 = gk0_shard + k_base;                  // global position of the first key processed
-  // packed keep mask: this lane's word per key tile, this wavefront's summary byte per key tile
-  const uint64_t* kw_ptr = nullptr;
-  const uint8_t* ks_ptr = nullptr;
-  uint64_t kw_cur = 0, kw_nxt = 0;
-  int ks_cur = 2, ks_nxt = 2;
-  if (HAS_KEEP) {
-    kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
-             mv.keep_q0 + qrow;
-    ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
-             (int64_t)((mv.keep_q0 + qg0 + w4 * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
-    if (ntiles > 0) { kw_nxt = kw_ptr[0]; ks_nxt = ks_ptr[0]; }
-  }
-
-  // segment ids: a tile whose keys all carry the one id of this wave's rows needs no segment compare
-  const int2* smm_ptr = nullptr;
-  bool sq_uniform = false, sp_cur = false, sp_nxt = false;
-  int sq_id = 0;
-  if (HAS_SEG && mv.seg_mm) {
-    smm_ptr = (const int2*)(mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2);
-    const int2 qmm = smm_ptr[min((gq_wg + grp * 128 + w4 * 32) / RA_SEG_TILE, mv.seg_tiles - 1)];
-    sq_uniform = qmm.x == qmm.y;
-    sq_id = qmm.x;
-    if (sq_uniform && ntiles > 0) {
-      const int2 kmm = smm_ptr[min(gk0 / RA_SEG_TILE, mv.seg_tiles - 1)];
-      sp_nxt = kmm.x == sq_id && kmm.y == sq_id;
-    }
-  }
-
-  const int gq = gq_wg + grp * 128 + w4 * 32 + lo;
-  const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
-  const int klim_wave = mv.cbs > 0 ? (int)min((long long)((gq_wg + grp * 128 + w4 * 32) / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
-  int seg_q = 0;
-  if (HAS_SEG) {
-    int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
-    seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
-  }
-  const float c = kLog2e / sqrtf((float)HD);
-  const float kMask2 = mv.mask_min;
-
-  const uint16_t* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-  bf16x8 qf[8];
-#pragma unroll
-  for (int t = 0; t < 8; t++) qf[t] = *(const bf16x8*)(qp + t * 16);
-
-  f32x16 acc[4];
-  float m2 = RA_NEG_INF, l = 0.f;
-  float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
-  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
-  if (a.carry_is_initial) {
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
-  } else {
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-      for (int g = 0; g < 4; g++) {
-        f32x4 t = *(const f32x4*)(nump + db * 32 + g * 8);
-        acc[db][g * 4 + 0] = t[0]; acc[db][g * 4 + 1] = t[1]; acc[db][g * 4 + 2] = t[2]; acc[db][g * 4 + 3] = t[3];
-      }
-    m2 = max_to_log2(a.mx[st], kMask2);
-    l = hi == 0 ? a.den[st] : 0.f;
-  }
-  if (ntiles == 0) {                  // workgroup-uniform
-    if (a.carry_is_initial) {
-#pragma unroll
-      for (int db = 0; db < 4; db++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) *(f32x4*)(nump + db * 32 + g * 8) = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (hi == 0) { a.den[st] = 0.f; a.mx[st] = RA_NEG_INF; }
-    }
-    return;
-  }
-
-  // ---- staging through registers, two phases ahead.  (Direct global->LDS loads allow very few
-  // requests in flight per CU on this part and block the issuing wavefront; plain loads do not.)
-  // Group B brings in the K tiles, group A the V tiles: at the start of each of its softmax phases a
-  // group stores the tile it requested in its previous softmax phase - the loads have had a whole
-  // matrix phase to land - and requests the next one.
-  const int srow = (tid & 255) >> 4, schunk = tid & 15;
-  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const uint16_t* sg = (grp == 1 ? a.k : a.v) + (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
-  const int64_t row16 = 16 * a.kv_ss;
-  uint4 sr0, sr1, sr2, sr3;       // scalars, not an array: an array here ends up in scratch memory
-#define RA_PP_LOAD4(J)                                                                                  \
-  {                                                                                                     \
-    const uint16_t* p_ = sg + (int64_t)(J) * FBN * a.kv_ss;                                             \
-    sr0 = *(const uint4*)(p_); sr1 = *(const uint4*)(p_ + row16);                                       \
-    sr2 = *(const uint4*)(p_ + 2 * row16); sr3 = *(const uint4*)(p_ + 3 * row16);                       \
-  }
-#define RA_PP_STORE4(LDS)                                                                               \
-  {                                                                                                     \
-    *(uint4*)(&(LDS)[s_off]) = sr0; *(uint4*)(&(LDS)[16 * TROW + s_off]) = sr1;                         \
-    *(uint4*)(&(LDS)[32 * TROW + s_off]) = sr2; *(uint4*)(&(LDS)[48 * TROW + s_off]) = sr3;             \
-  }
-#define RA_PP_KEYINFO(J)                                                                                \
-  if ((HAS_SEG || HAS_BIAS) && tid >= 256 && tid < 256 + FBN) {                                         \
-    const int kj_ = k_base + (J) * FBN + tid - 256;                                                              \
-    if (HAS_SEG) {                                                                                      \
-      int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
-      seg_ks[(J) & 3][tid - 256] = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                     \
-    }                                                                                                   \
-    if (HAS_BIAS) {                                                                                     \
-      float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
-      if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                           \
-      bias_ks[(J) & 3][tid - 256] = bv_ * kLog2e / c;    /* the S accumulators start from it */             \
-    }                                                                                                   \
-  }
-
-  int k_off[8], v_off[4][2];
-  RA_LANE_OFFSETS(k_off, v_off);
-
-  f32x16 s[2];
-  bf16x8 pf[2][2];
-  float m_true = m2;
-  constexpr float kLazy = 16.f;
-
-// matrix phase for key tile J: S(J+1) and O += P(J) V(J).  Eight steps of four MFMAs on six
-// independent accumulator chains; the LDS fragments of step t+1 are requested before the MFMAs of
-// step t are issued, and nothing may move across a step boundary (bounded register pressure).
-#define RA_PP_FRAGS(T, KF, VF)                                                                          \
-  {                                                                                                     \
-    KF[0] = *(const bf16x8*)(&kb_[k_off[T]]);                                                           \
-    KF[1] = *(const bf16x8*)(&kb_[32 * TROW + k_off[T]]);                                               \
-    const uint16_t* vt_ = &vb_[((((T) >> 2) * 32) + (((T) >> 1) & 1) * 16) * TROW];                     \
-    _Pragma("unroll") for (int x = 0; x < 2; x++) {                                                     \
-      const int db_ = ((T) & 1) * 2 + x;                                                                \
-      s16x4 v0_ = lds_read_tr(vt_ + v_off[db_][0]);                                                     \
-      s16x4 v1_ = lds_read_tr(vt_ + v_off[db_][1]);                                                     \
-      VF[x] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(v0_, v1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
-    }                                                                                                   \
-  }
-#define RA_PP_MATRIX(J)                                                                                 \
-  {                                                                                                     \
-    const uint16_t* kb_ = Ks[((J) + 1) & 1];                                                            \
-    const uint16_t* vb_ = Vs[(J) & 1];                                                                  \
-    if (HAS_BIAS) {          /* bias (per key = per accumulator row) enters as the initial value of S */ \
-      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
-        _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                 \
-          const f32x4 b4_ = *(const f32x4*)&bias_ks[((J) + 1) & 3][blk * 32 + g * 8 + hi * 4];          \
-          _Pragma("unroll") for (int e = 0; e < 4; e++) s[blk][g * 4 + e] = b4_[e];                     \
-        }                                                                                               \
-    } else {                                                                                            \
-      _Pragma("unroll") for (int r = 0; r < 16; r++) { s[0][r] = 0.f; s[1][r] = 0.f; }                  \
-    }                                                                                                   \
-    bf16x8 kf_[PP_DEPTH + 1][2], vf_[PP_DEPTH + 1][2];                                                  \
-    _Pragma("unroll") for (int t = 0; t < PP_DEPTH; t++) RA_PP_FRAGS(t, kf_[t], vf_[t]);                \
-    _Pragma("unroll") for (int t = 0; t < 8; t++) {                                                     \
-      if (t + PP_DEPTH < 8)                                                                             \
-        RA_PP_FRAGS(t + PP_DEPTH, kf_[(t + PP_DEPTH) % (PP_DEPTH + 1)], vf_[(t + PP_DEPTH) % (PP_DEPTH + 1)]); \
-      const int blk_ = t >> 2, tt_ = (t >> 1) & 1, db_ = (t & 1) * 2, c_ = t % (PP_DEPTH + 1);          \
-      s[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_[c_][0], qf[t], s[0], 0, 0, 0);                 \
-      acc[db_] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf_[c_][0], pf[blk_][tt_], acc[db_], 0, 0, 0); \
-      s[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf_[c_][1], qf[t], s[1], 0, 0, 0);                 \
-      acc[db_ + 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf_[c_][1], pf[blk_][tt_], acc[db_ + 1], 0, 0, 0); \
-      __builtin_amdgcn_sched_barrier(0);                                                                \
-    }                                                                                                   \
-  }
-
-// vector phase: softmax of s = S(T) -> pf = P(T); updates m2, m_true, l, rescales acc when needed
-#define RA_PP_SOFTMAX(T)                                                                                \
-  {                                                                                                     \
-    const int t_ = (T);                                                                                 \
-    const int gk_tile_ = gk0 + t_ * FBN;                                                                \
-    if (HAS_SEG) {                        /* are this tile's keys all of this wave's (single) segment? */ \
-      sp_cur = sp_nxt;                                                                                  \
-      if (sq_uniform) {                                                                                 \
-        const int2 kmm_ = smm_ptr[min(gk0 / RA_SEG_TILE + min(t_ + 1, ntiles - 1), mv.seg_tiles - 1)];  \
-        sp_nxt = kmm_.x == sq_id && kmm_.y == sq_id;                                                    \
-      }                                                                                                 \
-    }                                                                                                   \
-    if (HAS_KEEP) {                       /* this tile's word and summary; request the next tile's */   \
-      kw_cur = kw_nxt >> (4 * hi); ks_cur = ks_nxt;                                                     \
-      const int tn_ = min(t_ + 1, ntiles - 1);                                                          \
-      kw_nxt = kw_ptr[(int64_t)tn_ * mv.keep_Q]; ks_nxt = ks_ptr[tn_];                                  \
-    }                                                                                                   \
-    if (t_ >= ntiles_grp || (HAS_KEEP && ks_cur == 0 && mv.skip_tiles)) {                               \
-      _Pragma("unroll") for (int x = 0; x < 8; x++) {                                                   \
-        pf[0][0][x] = (__bf16)0.f; pf[0][1][x] = (__bf16)0.f; pf[1][0][x] = (__bf16)0.f; pf[1][1][x] = (__bf16)0.f; \
-      }                                                                                                 \
-    } else if ((!HAS_SEG || sp_cur) && (gk_tile_ + FBN - 1 < klim_wave) && (!HAS_KEEP || ks_cur == 2)) {   \
-      float mxv_ = s[0][0];                                                                             \
-      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
-        _Pragma("unroll") for (int r = 0; r < 16; r++) mxv_ = fmaxf(mxv_, s[blk][r]);                   \
-      mxv_ = max_xor32(mxv_);                                                                  \
-      m_true = fmaxf(m_true, mxv_ * c);                                                                 \
-      if (__builtin_amdgcn_ballot_w64(m_true - m2 > kLazy) != 0) {                                      \
-        const float alpha_ = fast_exp2(m2 - m_true);                                                    \
-        m2 = m_true;                                                                                    \
-        l *= alpha_;                                                                                    \
-        _Pragma("unroll") for (int db = 0; db < 4; db++)                                                \
-          _Pragma("unroll") for (int r = 0; r < 16; r++) acc[db][r] *= alpha_;                          \
-      }                                                                                                 \
-      float ps_ = 0.f;                                                                                  \
-      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
-        _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
-          float p_ = fast_exp2(fmaf(s[blk][r], c, -m2));                                                \
-          ps_ += p_;                                                                                    \
-          pf[blk][r >> 3][r & 7] = (__bf16)p_;                                                          \
-        }                                                                                               \
-      l += ps_;                                                                                         \
-    } else {                                                                                            \
-      float mxv_ = RA_NEG_INF;                                                                          \
-      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
-        _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
-          const int kr_ = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);                                   \
-          float x_ = s[blk][r] * c;                                                                     \
-          bool masked_ = (gk_tile_ + kr_ >= klim);                                                      \
-          if (HAS_SEG) masked_ = masked_ || (seg_ks[t_ & 3][kr_] != seg_q);                             \
-          if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> (blk * 32 + (r >> 2) * 8 + (r & 3))) & 1);    \
-          x_ = masked_ ? kMask2 : x_;                                                                   \
-          s[blk][r] = x_;                                                                               \
-          mxv_ = fmaxf(mxv_, x_);                                                                       \
-        }                                                                                               \
-      mxv_ = max_xor32(mxv_);                                                                  \
-      m_true = fmaxf(m_true, mxv_);                                                                     \
-      const float m_new_ = fmaxf(m2, mxv_);                                                             \
-      const float alpha_ = fast_exp2(m2 - m_new_);                                                      \
-      m2 = m_new_;                                                                                      \
-      float ps_ = 0.f;                                                                                  \
-      _Pragma("unroll") for (int blk = 0; blk < 2; blk++)                                               \
-        _Pragma("unroll") for (int r = 0; r < 16; r++) {                                                \
-          float p_ = fast_exp2(s[blk][r] - m_new_);                                                     \
-          ps_ += p_;                                                                                    \
-          pf[blk][r >> 3][r & 7] = (__bf16)p_;                                                          \
-        }                                                                                               \
-      l = l * alpha_ + ps_;                                                                             \
-      if (__builtin_amdgcn_ballot_w64(alpha_ != 1.f) != 0) {                                            \
-        _Pragma("unroll") for (int db = 0; db < 4; db++)                                                \
-          _Pragma("unroll") for (int r = 0; r < 16; r++) acc[db][r] *= alpha_;                          \
-      }                                                                                                 \
-    }                                                                                                   \
-  }
-
-  // ---- prologue: K(0), K(1) into LDS and K(2) into registers by group B; V(0) into LDS and V(1)
-  // into registers by group A
-  if (grp == 1) {
-    RA_PP_LOAD4(0);
-    RA_PP_STORE4(Ks[0]);
-    RA_PP_LOAD4(min(1, ntiles - 1));
-    RA_PP_STORE4(Ks[1]);
-    RA_PP_LOAD4(min(2, ntiles - 1));
-  } else {
-    RA_PP_LOAD4(0);
-    RA_PP_STORE4(Vs[0]);
-    RA_PP_LOAD4(min(1, ntiles - 1));
-  }
-  RA_PP_KEYINFO(0);
-  RA_PP_KEYINFO(min(1, ntiles - 1));
-  __syncthreads();
-  {
-    f32x16 sn0, sn1;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int kr = (r >> 2) * 8 + hi * 4 + (r & 3);
-      sn0[r] = HAS_BIAS ? bias_ks[0][kr] : 0.f;
-      sn1[r] = HAS_BIAS ? bias_ks[0][32 + kr] : 0.f;
-    }
-#pragma unroll
-    for (int t = 0; t < 8; t++) {
-      bf16x8 kf0 = *(const bf16x8*)(&Ks[0][k_off[t]]);
-      sn0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf0, qf[t], sn0, 0, 0, 0);
-      bf16x8 kf1 = *(const bf16x8*)(&Ks[0][32 * TROW + k_off[t]]);
-      sn1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf1, qf[t], sn1, 0, 0, 0);
-    }
-    s[0] = sn0; s[1] = sn1;
-  }
-  // One loop body for every wavefront: matrix(j), barrier, softmax(j+1), barrier.  Group B enters the
-  // loop one phase (one barrier) later than group A, which puts its matrix phases against group A's
-  // softmax phases; group A pays the missing barrier at the end.
-#ifdef RA_TRACE
-  const bool trace_on = blockIdx.x == 0;
-  int trace_n = 0;
-#endif
-  if (grp == 0) RA_PP_SOFTMAX(0);
-  __syncthreads();                    // every wave is done with K(0) before phase 0 overwrites it
-  if (grp == 1) {
-    RA_PP_STORE4(Ks[0]);                                     // K(2); K(0) was consumed by the prologue
-    RA_PP_LOAD4(min(3, ntiles - 1));       // K(3)
-    RA_PP_KEYINFO(min(2, ntiles - 1));
-    RA_PP_SOFTMAX(0);                 // phase 0 of group B
-    __syncthreads();
-  }
-  for (int j = 0; j < ntiles; j++) {
-    RA_TRACE_MARK();
-    if (PP_PRIO) __builtin_amdgcn_s_setprio(1);
-#ifndef RA_ABL_NOMATRIX
-    RA_PP_MATRIX(j);                  // phase 2j (A) / 2j+1 (B)
-#endif
-    if (PP_PRIO) __builtin_amdgcn_s_setprio(0);
-    RA_TRACE_MARK();
-    __syncthreads();
-    RA_TRACE_MARK();
-#ifndef RA_ABL_NOSTAGE
-    // group A, phase 2j+1: V(j+1) -> Vs[(j+1)&1] (V(j-1) was last read in phase 2j-1), request V(j+2);
-    // group B, phase 2j+2: K(j+3) -> Ks[(j+1)&1] (K(j+1) was last read in phase 2j+1), request K(j+4)
-    if (grp == 0) { RA_PP_STORE4(Vs[(j + 1) & 1]); } else { RA_PP_STORE4(Ks[(j + 1) & 1]); }
-    RA_PP_LOAD4(min(j + 2 + 2 * grp, ntiles - 1));
-    if (grp == 1) RA_PP_KEYINFO(min(j + 3, ntiles - 1));
-#endif
-    RA_TRACE_MARK();
-#ifndef RA_ABL_NOSOFTMAX
-    RA_PP_SOFTMAX(j + 1);             // for j + 1 == ntiles the tile is past the range: P = 0
-#endif
-    RA_TRACE_MARK();
-    __syncthreads();
-  }
-  if (grp == 0) __syncthreads();
-#undef RA_PP_KEYINFO
-#undef RA_PP_LOAD4
-#undef RA_PP_STORE4
-#undef RA_PP_MATRIX
-#undef RA_PP_FRAGS
-#undef RA_PP_SOFTMAX
-
-  if (__builtin_amdgcn_ballot_w64(m_true != m2) != 0) {     // bring the carry to the exact running max
-    const float fix = (m_true == m2) ? 1.f : fast_exp2(m2 - m_true);
-    m2 = m_true;
-    l *= fix;
-#pragma unroll
-    for (int db = 0; db < 4; db++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[db][r] *= fix;
-  }
-#pragma unroll
-  for (int db = 0; db < 4; db++)
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      f32x4 t = {acc[db][g * 4 + 0], acc[db][g * 4 + 1], acc[db][g * 4 + 2], acc[db][g * 4 + 3]};
-      *(f32x4*)(nump + db * 32 + g * 8) = t;
-    }
-  l += xor32(l);
-  if (hi == 0) {
-    a.den[st] = l;
-    a.mx[st] = max_from_log2(m2, kMask2);
-  }
-}
 
 // ================================================================== backward
 // Two deterministic kernels (fp32 atomics reach ~1.3 TB/s at best on this part, far below what a
@@ -1919,16 +1489,15 @@ static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
 // a boolean keep mask is taken in packed form only and alone (no bias, segment ids or causal block size next to it:
 // ring_attention_inference has none of them, and the generic kernels serve any combination)
-static bool keep_ok(const ra_mask& m, bool shape_ok) {
+static bool keep_ok(const ra_mask& m) {
   if (!m.keep) return true;
-  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids && m.causal_block_size == 0 &&
-         shape_ok;
+  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids && m.causal_block_size == 0;
 }
 
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
   const ra_mask& m = p->mask;
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
-         keep_ok(m, true) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
+         keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
          aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator);
 }
@@ -1945,20 +1514,6 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   a.carry_is_initial = p->carry_is_initial;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool keep = p->mask.keep != nullptr;      // packed form checked by attn_fwd_mfma_supported
-  // chunks of a multiple of 256 rows: the ping-pong kernel (256 rows per workgroup, half the K / V traffic per
-  // row); other multiples of 128: the wave-specialised kernel
-  if (p->mask.query_chunk_size % PBM == 0 && !getenv("RA_FWD_WAVE_SPEC")) {
-    const long long nwg2 = (long long)(p->Sq / PBM) * p->H * p->B;
-    RA_REQUIRE(nwg2 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
-    dim3 grid2((unsigned)nwg2), block2(512);
-    if (keep) attn_fwd_pp_kernel<false, false, true><<<grid2, block2, 0, s>>>(a);
-    else if (seg && bias) attn_fwd_pp_kernel<true, true><<<grid2, block2, 0, s>>>(a);
-    else if (seg) attn_fwd_pp_kernel<true, false><<<grid2, block2, 0, s>>>(a);
-    else if (bias) attn_fwd_pp_kernel<false, true><<<grid2, block2, 0, s>>>(a);
-    else attn_fwd_pp_kernel<false, false><<<grid2, block2, 0, s>>>(a);
-    RA_CHECK_LAUNCH("attn_fwd_pp");
-    return RA_OK;
-  }
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
   RA_REQUIRE(nwg3 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
   dim3 grid3((unsigned)((nwg3 + 7) / 8 * 8)), block3(512);
@@ -1974,7 +1529,7 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
   const ra_mask& m = p->mask;
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % KBN == 0 &&
-         keep_ok(m, true) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
+         keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0 &&
          p->dkv_stride_s % 4 == 0 && p->dkv_stride_b % 4 == 0 && aligned16(p->q) && aligned16(p->k) &&
          aligned16(p->v) && aligned16(p->g) && aligned16(p->dq) && aligned16(p->dk) && aligned16(p->dv);
