@@ -204,13 +204,15 @@ constexpr int WS_TILE = KBM * TROW;
 
 template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Qs[3 * WS_TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t Gs[3 * WS_TILE];
+  // Q tiles then dO tiles in one array: a dO address is the Q address plus a constant (an immediate offset)
+  __shared__ __attribute__((aligned(16))) uint16_t QGs[6 * WS_TILE];
+  uint16_t* const Qs = QGs;
+  uint16_t* const Gs = QGs + 3 * WS_TILE;
   __shared__ __attribute__((aligned(16))) uint16_t Ps[4][2][2][WS_PD];     // [pair][buffer][P | dS]
   __shared__ __attribute__((aligned(16))) float st_m2[3][KBM];
   __shared__ __attribute__((aligned(16))) float st_rden[3][KBM];
   __shared__ __attribute__((aligned(16))) float st_lse2[3][KBM];
-  __shared__ __attribute__((aligned(16))) float st_delta[3][KBM];
+  __shared__ __attribute__((aligned(16))) float st_delta[3][KBM];   // holds -delta
   __shared__ __attribute__((aligned(16))) int st_seg[3][KBM];
 
   MaskView mv = a.mv;
@@ -309,7 +311,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     if (tid >= 256 && tid < 256 + KBM) {                                                                \
       const float m2_ = max_to_log2(r_m, kMask2);                                                       \
       st_m2[BUF][tid - 256] = m2_; st_rden[BUF][tid - 256] = 1.f / r_den;                               \
-      st_lse2[BUF][tid - 256] = m2_ + __log2f(r_den); st_delta[BUF][tid - 256] = r_delta;               \
+      st_lse2[BUF][tid - 256] = m2_ + __log2f(r_den); st_delta[BUF][tid - 256] = -r_delta;              \
       if (HAS_SEG) st_seg[BUF][tid - 256] = r_seg;                                                      \
     }                                                                                                   \
   }
@@ -352,13 +354,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #define RA_WS_INIT(SN, DPN, BUF, BLK)                                                                   \
   _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                       \
     const f32x4 d_ = *(const f32x4*)&st_delta[BUF][(BLK) * 32 + g * 8 + hi * 4];                        \
-    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = HAS_BIAS ? bias2 : 0.f; DPN[g * 4 + e] = -d_[e]; } \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = HAS_BIAS ? bias2 : 0.f; DPN[g * 4 + e] = d_[e]; } \
   }
     // A operands of two contraction steps (32 of the 128 head dimensions) of block BLK of buffer BUF
 #define RA_WS_AREAD(G, QA, GA, BUF, BLK)                                                                \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    QA[i] = *(const bf16x8*)(Qs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
-    GA[i] = *(const bf16x8*)(Gs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
+    const uint16_t* p_ = Qs + (BUF) * WS_TILE + n_off[2 * (G) + i];                                     \
+    QA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW);                                                   \
+    GA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW + 3 * WS_TILE);                                     \
   }
 #define RA_WS_AMFMA(G, QA, GA, SN, DPN)                                                                 \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
@@ -611,8 +614,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #endif
 template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[3 * WS_TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[3 * WS_TILE];
+  // K tiles then V tiles in one array: a V address is the K address plus a constant (an immediate offset)
+  __shared__ __attribute__((aligned(16))) uint16_t KVs[6 * WS_TILE];
+  uint16_t* const Ks = KVs;
+  uint16_t* const Vs = KVs + 3 * WS_TILE;
   __shared__ __attribute__((aligned(16))) uint16_t Ds[4][2][WS_PD];        // [pair][buffer] dS^T as [q][key]
   __shared__ int seg_ks[3][FBN];
   __shared__ float bias_ks[3][FBN];
@@ -771,8 +776,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   }
 #define RA_WS_AREAD(G, KA, VA, BUF, BLK)                                                                \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    KA[i] = *(const bf16x8*)(Ks + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
-    VA[i] = *(const bf16x8*)(Vs + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);            \
+    const uint16_t* p_ = Ks + (BUF) * WS_TILE + n_off[2 * (G) + i];                                     \
+    KA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW);                                                   \
+    VA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW + 3 * WS_TILE);                                     \
   }
 #define RA_WS_AMFMA(G, KA, VA, SN, DPN)                                                                 \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
@@ -1023,8 +1029,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 // O^T += V^T P^T one block of 32 keys behind.
 template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[3 * WS_TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[3 * WS_TILE];
+  // K tiles then V tiles in one array: a V address is the K address plus a constant (an immediate offset)
+  __shared__ __attribute__((aligned(16))) uint16_t KVs[6 * WS_TILE];
+  uint16_t* const Ks = KVs;
+  uint16_t* const Vs = KVs + 3 * WS_TILE;
   __shared__ __attribute__((aligned(16))) uint16_t Ds[4][2][WS_PD];        // [pair][buffer] P^T as [q][key]
   __shared__ float al[4][2][32];     // [pair][buffer][query]: factor the consumer applies to O before adding the block
   __shared__ float fixs[4][32];      // [pair][query]: final factor (lazy reference max -> exact max)
