@@ -2,10 +2,10 @@
 // blockwise_feedforward (ringattention_jax.py:333-352) scans over chunks of tokens.
 //
 // GEMM: C (M,N) = op(A) op(B) [+ op(A2) op(B2)], fp32 accumulation in v_mfma_f32_32x32x16_bf16.
-//   workgroup = WGM x WGN wavefronts, tile BM x BN, K step 64, LDS double buffered.  The tile is
-//   chosen per problem: 256 x 256 over 8 wavefronts (each 128 x 64: six operand fragments from LDS
-//   per eight MFMAs, and half the global bytes per flop of a 128 x 128 tile) when that still gives
-//   every CU work, smaller tiles otherwise.
+//   The tile is chosen per problem: 256 x 256 over 4 wavefronts (gemm_bf16_w4_kernel: each wavefront
+//   128 x 128, eight operand fragments from LDS per sixteen MFMAs) when that still gives every CU work;
+//   otherwise gemm_bf16_kernel with WGM x WGN wavefronts on a BM x BN tile (256 x 128 over 8, 128 x 128
+//   over 4), K step 64, LDS double buffered.
 //   An operand whose contraction index is contiguous in memory is staged row-major and read with
 //   16-byte LDS reads; one whose contraction index is the slow axis is staged as it lies in memory
 //   and read with ds_read_b64_tr_b16, so no layout ever needs a transposing copy.
@@ -19,8 +19,10 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int GBK = 64;
-constexpr int NAT_STR = GBK + 8;      // row stride (elements) of a tile read row-wise
+#ifndef RA_W4_ABL
+#define RA_W4_ABL 0     // timing experiments only: 1 = no global loads, 2 = no LDS stores, 4 = no LDS reads in the K loop, 8 = no barrier, 16 = no epilogue
+#endif
+constexpr int GBK = 64;               // K step of the 8-wavefront tiles (and the granularity required of K)
 
 struct GemmArgs {
   const uint16_t* A; const uint16_t* B; const uint16_t* A2; const uint16_t* B2;
@@ -33,15 +35,34 @@ __device__ __forceinline__ s16x4 lds_tr(const uint16_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p));
 }
 
+// Workgroup -> tile.  Workgroups go to the 8 XCDs round-robin and each XCD has its own L2, so XCD x takes the
+// contiguous range x of a tile order in which consecutive tiles form groups of GROUP_M tile rows walked column by
+// column: the 32 workgroups resident on an XCD then cover about 4 x 8 tiles, an A panel is fetched into that L2
+// once per 8 tiles and a B panel once per 4, instead of once per tile.
+constexpr int GROUP_M = 4;
+__device__ __forceinline__ bool tile_of_block(int ntm, int ntn, int& tm, int& tn) {
+  const int ntiles = ntm * ntn;
+  const int per_xcd = (ntiles + 7) >> 3;
+  const int pid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (pid >= ntiles) return false;
+  const int group = pid / (GROUP_M * ntn), first_m = group * GROUP_M;
+  const int rows = min(GROUP_M, ntm - first_m);
+  const int in_group = pid - group * GROUP_M * ntn;
+  tm = first_m + in_group % rows;
+  tn = in_group / rows;
+  return true;
+}
+
 // TA: A is stored (K,M).  TB: B is stored (N,K).
 template <bool TA, bool TB, int BM, int BN, int WGM, int WGN, bool DEEP>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
-  constexpr int NT = 64 * WGM * WGN;
+  constexpr int NT = 64 * WGM * WGN, BK = GBK;
+  constexpr int NAT_STR = BK + 8;      // row stride (elements) of a tile read row-wise
   constexpr int WM = BM / WGM, WN = BN / WGN, MB = WM / 32, NB = WN / 32;
   constexpr int A_STR = TA ? BM + 32 : NAT_STR;     // elements
   constexpr int B_STR = TB ? NAT_STR : BN + 32;
-  constexpr int A_ROWS = TA ? GBK : BM, B_ROWS = TB ? BN : GBK;
-  constexpr int A_CPR = (TA ? BM : GBK) / 8, B_CPR = (TB ? GBK : BN) / 8;   // 16-byte chunks per staged row
+  constexpr int A_ROWS = TA ? BK : BM, B_ROWS = TB ? BN : BK;
+  constexpr int A_CPR = (TA ? BM : BK) / 8, B_CPR = (TB ? BK : BN) / 8;   // 16-byte chunks per staged row
   constexpr int A_CH = A_ROWS * A_CPR / NT, B_CH = B_ROWS * B_CPR / NT;     // chunks per thread
   static_assert(A_CH * NT == A_ROWS * A_CPR && B_CH * NT == B_ROWS * B_CPR, "tile does not divide over the threads");
   __shared__ __attribute__((aligned(16))) uint16_t As[2][A_ROWS * A_STR];
@@ -49,9 +70,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int wm = wave / WGN, wn = wave % WGN;
-  // neighbouring workgroups share the A row panel (and, 8 apart, the same XCD's L2)
-  const int ntn = g.N / BN;
-  const int tm = blockIdx.x / ntn, tn = blockIdx.x % ntn;
+  int tm, tn;
+  if (!tile_of_block(g.M / BM, g.N / BN, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
 
   f32x16 acc[MB][NB];
@@ -68,7 +88,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
   static_assert(A_CH <= 4 && B_CH <= 4, "at most four 16-byte chunks per thread and operand");
   uint4 Pa0, Pa1, Pa2, Pa3, Pb0, Pb1, Pb2, Pb3, Qa0, Qa1, Qa2, Qa3, Qb0, Qb1, Qb2, Qb3;
   const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
-  const int nk = g.K / GBK;
+  const int nk = g.K / BK;
   const int total = nk * (g.A2 ? 2 : 1);
   // chunk c of this thread: staged row and 16-byte column, fixed for the whole kernel
 #define RA_A_OFF(C, K0) (TA ? (int64_t)((K0) + ((C) * NT + tid) / A_CPR) * lda + m0 + (((C) * NT + tid) % A_CPR) * 8 \
@@ -83,7 +103,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
     const int t_ = min((T), total - 1);                                                                 \
     const uint16_t* Ap = t_ >= nk ? g.A2 : g.A;                                                         \
     const uint16_t* Bp = t_ >= nk ? g.B2 : g.B;                                                         \
-    const int k0_ = (t_ >= nk ? t_ - nk : t_) * GBK;                                                    \
+    const int k0_ = (t_ >= nk ? t_ - nk : t_) * BK;                                                    \
     if (A_CH > 0) S##a0 = *(const uint4*)(Ap + RA_A_OFF(0, k0_));                                       \
     if (A_CH > 1) S##a1 = *(const uint4*)(Ap + RA_A_OFF(1, k0_));                                       \
     if (A_CH > 2) S##a2 = *(const uint4*)(Ap + RA_A_OFF(2, k0_));                                       \
@@ -112,7 +132,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
 #define RA_COMPUTE(CUR_)                                                                                \
   {                                                                                                     \
     _Pragma("unroll")                                                                                  \
-    for (int kk = 0; kk < GBK / 16; kk++) {                                                             \
+    for (int kk = 0; kk < BK / 16; kk++) {                                                             \
       bf16x8 af[MB], bfr[NB];                                                                           \
     _Pragma("unroll")                                                                                  \
       for (int i = 0; i < MB; i++) {                                                                    \
@@ -215,9 +235,199 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
     }
 }
 
+// 256 x 256 tile over FOUR wavefronts (2 x 2), one per SIMD with all 512 registers: each wavefront owns 128 x 128
+// of C (256 accumulator registers), so a K slice of 16 takes eight operand fragments from LDS for sixteen MFMAs -
+// half the LDS bytes per MFMA of the eight-wavefront tile, which is LDS-bound.  With a single wavefront per SIMD
+// nothing hides latency but the wavefront's own pipelining: K step 32 = two slices; the fragments of a slice are
+// requested from LDS one slice (sixteen MFMAs) before their use, across the barrier of the K step; a K slab stays
+// in flight from global memory for two K steps in one of two register sets.
+template <bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
+  constexpr int BM = 256, BN = 256, BK = 32, NT = 256, WM = 128, WN = 128;
+  constexpr int NAT_STR = BK + 8;
+  constexpr int A_STR = TA ? BM + 32 : NAT_STR, B_STR = TB ? NAT_STR : BN + 32;
+  constexpr int A_ROWS = TA ? BK : BM, B_ROWS = TB ? BN : BK;
+  constexpr int A_CPR = (TA ? BM : BK) / 8, B_CPR = (TB ? BK : BN) / 8;
+  static_assert(A_ROWS * A_CPR == 4 * NT && B_ROWS * B_CPR == 4 * NT, "four 16-byte chunks per thread and operand");
+  // one array per buffer and operand: reads of one buffer and writes of the other can then be reordered freely
+  __shared__ __attribute__((aligned(16))) uint16_t As0[A_ROWS * A_STR];
+  __shared__ __attribute__((aligned(16))) uint16_t As1[A_ROWS * A_STR];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs0[B_ROWS * B_STR];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs1[B_ROWS * B_STR];
+#define RA_W4_AS(BUF) ((BUF) ? As1 : As0)
+#define RA_W4_BS(BUF) ((BUF) ? Bs1 : Bs0)
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  if (!tile_of_block(g.M / BM, g.N / BN, tm, tn)) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  uint4 Pa0, Pa1, Pa2, Pa3, Pb0, Pb1, Pb2, Pb3, Qa0, Qa1, Qa2, Qa3, Qb0, Qb1, Qb2, Qb3;
+  const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
+  const int nk = g.K / BK;
+  const int total = nk * (g.A2 ? 2 : 1);
+  // this thread's four chunks of a slab: global offsets (without the K position) and LDS offsets
+  int64_t ga[4], gb[4];
+  int la[4], lb[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) {
+    const int ia = c * NT + tid, ib = c * NT + tid;
+    ga[c] = TA ? (int64_t)(ia / A_CPR) * lda + m0 + (ia % A_CPR) * 8 : (int64_t)(m0 + ia / A_CPR) * lda + (ia % A_CPR) * 8;
+    gb[c] = TB ? (int64_t)(n0 + ib / B_CPR) * ldb + (ib % B_CPR) * 8 : (int64_t)(ib / B_CPR) * ldb + n0 + (ib % B_CPR) * 8;
+    la[c] = (ia / A_CPR) * A_STR + (ia % A_CPR) * 8;
+    lb[c] = (ib / B_CPR) * B_STR + (ib % B_CPR) * 8;
+  }
+  const int64_t ka = TA ? (int64_t)lda : 1, kb = TB ? 1 : (int64_t)ldb;    // stride of the K position
+#define RA_W4_LOAD_A(S, T)                                                                              \
+  {                                                                                                     \
+    const int t_ = min((T), total - 1);                                                                 \
+    const uint16_t* Ap = (t_ >= nk ? g.A2 : g.A) + (int64_t)((t_ >= nk ? t_ - nk : t_) * BK) * ka;      \
+    S##a0 = *(const uint4*)(Ap + ga[0]); S##a1 = *(const uint4*)(Ap + ga[1]);                           \
+    S##a2 = *(const uint4*)(Ap + ga[2]); S##a3 = *(const uint4*)(Ap + ga[3]);                           \
+  }
+#define RA_W4_LOAD_B(S, T)                                                                              \
+  {                                                                                                     \
+    const int t_ = min((T), total - 1);                                                                 \
+    const uint16_t* Bp = (t_ >= nk ? g.B2 : g.B) + (int64_t)((t_ >= nk ? t_ - nk : t_) * BK) * kb;      \
+    S##b0 = *(const uint4*)(Bp + gb[0]); S##b1 = *(const uint4*)(Bp + gb[1]);                           \
+    S##b2 = *(const uint4*)(Bp + gb[2]); S##b3 = *(const uint4*)(Bp + gb[3]);                           \
+  }
+#define RA_W4_LOAD(S, T) { RA_W4_LOAD_A(S, T); RA_W4_LOAD_B(S, T); }
+#define RA_W4_STORE(S, BUF)                                                                             \
+  {                                                                                                     \
+    *(uint4*)(&RA_W4_AS(BUF)[la[0]]) = S##a0; *(uint4*)(&RA_W4_AS(BUF)[la[1]]) = S##a1;                             \
+    *(uint4*)(&RA_W4_AS(BUF)[la[2]]) = S##a2; *(uint4*)(&RA_W4_AS(BUF)[la[3]]) = S##a3;                             \
+    *(uint4*)(&RA_W4_BS(BUF)[lb[0]]) = S##b0; *(uint4*)(&RA_W4_BS(BUF)[lb[1]]) = S##b1;                             \
+    *(uint4*)(&RA_W4_BS(BUF)[lb[2]]) = S##b2; *(uint4*)(&RA_W4_BS(BUF)[lb[3]]) = S##b3;                             \
+  }
+  const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wm * WM;
+  const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wn * WN;
+  const int natA = (wm * WM + lo) * A_STR + hi * 8, natB = (wn * WN + lo) * B_STR + hi * 8;
+  // the eight fragments of K slice KK of buffer BUF into set F (F##a[0..3], F##b[0..3])
+#define RA_W4_FRAGS(F, BUF, KK)                                                                         \
+  _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                       \
+    if (!TA) {                                                                                          \
+      F##a[i] = *(const bf16x8*)(&RA_W4_AS(BUF)[natA + i * 32 * A_STR + (KK) * 16]);                          \
+    } else {                                                                                            \
+      const uint16_t* p = &RA_W4_AS(BUF)[(KK) * 16 * A_STR + trA + i * 32];                                   \
+      s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);                                                 \
+      F##a[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
+    }                                                                                                   \
+    if (TB) {                                                                                           \
+      F##b[i] = *(const bf16x8*)(&RA_W4_BS(BUF)[natB + i * 32 * B_STR + (KK) * 16]);                          \
+    } else {                                                                                            \
+      const uint16_t* p = &RA_W4_BS(BUF)[(KK) * 16 * B_STR + trB + i * 32];                                   \
+      s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);                                                 \
+      F##b[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
+    }                                                                                                   \
+  }
+#define RA_W4_MFMA(F)                                                                                   \
+  _Pragma("unroll") for (int i = 0; i < 4; i++)                                                         \
+    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                       \
+      acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F##a[i], F##b[j], acc[i][j], 0, 0, 0);
+  // one K step: slab in buffer CUR (its slice 0 already in set F); set S of staging registers holds the next slab,
+  // which goes to the other buffer, and is then reloaded with slab NEXT_T
+  // A single wavefront per SIMD issues in order: the MFMA pipe only stays busy if every MFMA is followed by at most
+  // a few other instructions.  Sixteen groups of one MFMA, one LDS read and one LDS write or global load.
+#define RA_W4_SCHED(WRITES, LOADS)                                                                      \
+  _Pragma("unroll") for (int m_ = 0; m_ < 16; m_++) {                                                   \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                  \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                  \
+    if (m_ < (WRITES)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                               \
+    else if (m_ < (WRITES) + (LOADS)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                \
+  }
+  // one K step: slab in buffer CUR (its slice 0 already in set F); set S of staging registers holds the next slab,
+  // which goes to the other buffer, and is then reloaded with slab NEXT_T
+#define RA_W4_STEP(CUR, S, NEXT_T)                                                                      \
+  {                                                                                                     \
+    if (!(RA_W4_ABL & 4)) { RA_W4_FRAGS(G, CUR, 1); }                                                   \
+    if (!(RA_W4_ABL & 2)) { RA_W4_STORE(S, (CUR) ^ 1); }                                                \
+    if (!(RA_W4_ABL & 1)) { RA_W4_LOAD_A(S, NEXT_T); }                                                  \
+    RA_W4_MFMA(F);                                                                                      \
+    RA_W4_SCHED(8, 4);                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    if (!(RA_W4_ABL & 8)) __syncthreads();                                                              \
+    if (!(RA_W4_ABL & 4)) { RA_W4_FRAGS(F, (CUR) ^ 1, 0); }                                             \
+    if (!(RA_W4_ABL & 1)) { RA_W4_LOAD_B(S, NEXT_T); }                                                  \
+    RA_W4_MFMA(G);                                                                                      \
+    RA_W4_SCHED(0, 4);                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+  }
+  bf16x8 Fa[4], Fb[4], Ga[4], Gb[4];
+  RA_W4_LOAD(P, 0);
+  RA_W4_LOAD(Q, 1);
+  RA_W4_STORE(P, 0);
+  RA_W4_LOAD(P, 2);
+  __syncthreads();
+  RA_W4_FRAGS(F, 0, 0);
+  // K is a multiple of 64: an even number of slabs
+  for (int it = 0; it < total; it += 2) {
+    RA_W4_STEP(0, Q, it + 3);
+    RA_W4_STEP(1, P, it + 4);
+  }
+#undef RA_W4_STEP
+#undef RA_W4_AS
+#undef RA_W4_BS
+#undef RA_W4_MFMA
+#undef RA_W4_FRAGS
+#undef RA_W4_STORE
+#undef RA_W4_LOAD
+#undef RA_W4_LOAD_A
+#undef RA_W4_LOAD_B
+#undef RA_W4_SCHED
+
+  // epilogue through per-wavefront LDS patches, as in gemm_bf16_kernel
+  if (RA_W4_ABL & 16) { if (acc[0][0][0] == 123.f) *(float*)g.C = acc[1][1][1] + acc[2][2][2] + acc[3][3][3]; return; }
+  __syncthreads();
+  static_assert(sizeof(As0) >= (size_t)4 * 32 * 36 * sizeof(float), "operand tile too small for the epilogue patches");
+  float* patch = (float*)&As0[0] + wave * (32 * 36);
+  const int er = lane >> 3, ec = (lane & 7) * 4;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) patch[((r >> 2) * 8 + hi * 4 + (r & 3)) * 36 + lo] = acc[i][j][r];
+#pragma unroll
+      for (int pass = 0; pass < 4; pass++) {
+        const int row = pass * 8 + er;
+        const float4 v = *(const float4*)&patch[row * 36 + ec];
+        const int64_t o = (int64_t)(m0 + wm * WM + i * 32 + row) * g.N + n0 + wn * WN + j * 32 + ec;
+        if (g.c_f32) {
+          float4* c = (float4*)((float*)g.C + o);
+          float4 w = v;
+          if (g.beta_one) { const float4 old = *c; w.x += old.x; w.y += old.y; w.z += old.z; w.w += old.w; }
+          *c = w;
+        } else {
+          uint2 w;
+          w.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+          w.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+          *(uint2*)((uint16_t*)g.C + o) = w;
+        }
+      }
+    }
+}
+
+template <bool TA, bool TB>
+static int launch_w4(const GemmArgs& g, hipStream_t s) {
+  const long long nwg = ((long long)(g.M / 256) * (g.N / 256) + 7) / 8 * 8;
+  gemm_bf16_w4_kernel<TA, TB><<<dim3((unsigned)nwg), 256, 0, s>>>(g);
+  RA_CHECK_LAUNCH("gemm_bf16_w4");
+  return RA_OK;
+}
+
 template <bool TA, bool TB, int BM, int BN, int WGM, int WGN, bool DEEP>
 static int launch_tile(const GemmArgs& g, hipStream_t s) {
-  const long long nwg = (long long)(g.M / BM) * (g.N / BN);
+  const long long nwg = ((long long)(g.M / BM) * (g.N / BN) + 7) / 8 * 8;    // whole rounds over the 8 XCDs
   gemm_bf16_kernel<TA, TB, BM, BN, WGM, WGN, DEEP><<<dim3((unsigned)nwg), 64 * WGM * WGN, 0, s>>>(g);
   RA_CHECK_LAUNCH("gemm_bf16");
   return RA_OK;
@@ -256,7 +466,7 @@ static int launch_gemm(const GemmArgs& g, hipStream_t s) {
   if (t == 0 && (g.M % 256 || g.N % 256)) t = 1;
   if (t == 1 && g.M % 256) t = 2;
   switch (t) {
-    case 0: return launch_tile<TA, TB, 256, 256, 2, 4, false>(g, s);
+    case 0: return launch_w4<TA, TB>(g, s);
     case 1: return launch_tile<TA, TB, 256, 128, 4, 2, true>(g, s);
     default: return launch_tile<TA, TB, 128, 128, 2, 2, false>(g, s);
   }

@@ -109,6 +109,22 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
         return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None
 
 
+# Tokens are independent in a token-wise MLP, so several consecutive chunks may share one launch: the
+# result is the same, the GEMMs fill the 256 CUs in whole rounds, and the fp32 weight-gradient
+# accumulators are read and written once per slab instead of once per chunk.  The scratch of a slab
+# (five (tokens, intermediate) bf16 buffers) is what bounds it: 16384 tokens x 11008 is 1.8 GB.
+MAX_SLAB_TOKENS = 16384
+
+
+def _slab_tokens(chunk_size, n_chunks):
+    import os
+    cap = int(os.environ.get("RA_FFN_SLAB_TOKENS", MAX_SLAB_TOKENS))
+    g = max(1, min(n_chunks, cap // chunk_size))
+    while n_chunks % g:
+        g -= 1
+    return chunk_size * g
+
+
 class SwiGLU(torch.nn.Module):
     """The LLaMA-style MLP the reference's README pairs with blockwise_feedforward:
     w2(silu(x w1) * (x w3)); weights stored (in, out), bf16."""
@@ -152,7 +168,7 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
         if b == 1:
             # contiguous slabs of chunk_size tokens, one autograd node for the whole scan
             y = _BlockwiseSwiGLUFn.apply(inputs.reshape(s, d).contiguous(), feedforward.w1, feedforward.w2,
-                                         feedforward.w3, chunk_size)
+                                         feedforward.w3, _slab_tokens(chunk_size, n))
             return y.reshape(1, s, y.shape[-1])
         outs = [feedforward(inputs[:, j * chunk_size:(j + 1) * chunk_size]) for j in range(n)]
         return torch.cat(outs, dim=1)

@@ -35,6 +35,27 @@ def test_gemm_layouts(ta, tb, shape):
     assert errors(acc, ref + 1.0)[1] < 1e-5
 
 
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("shape", [(768, 512, 320), (1280, 256, 128)])
+def test_gemm_every_tile_kernel(monkeypatch, ta, tb, tile, shape):
+    """Each tile kernel (0: 256 x 256 over four wavefronts, 1: 256 x 128, 2: 128 x 128) on shapes whose tile
+    counts are no multiple of the 8 XCDs or of the tile-row group, so the workgroup -> tile order and its
+    surplus workgroups are exercised; the library picks the tile itself unless RA_GEMM_TILE names one."""
+    M, N, K = shape
+    print("gemm tile", tile, ta, tb, shape, flush=True)
+    monkeypatch.setenv("RA_GEMM_TILE", str(tile))
+    g = torch.Generator().manual_seed(M + N + K + tile)
+    A = torch.randn((K, M) if ta else (M, K), generator=g).bfloat16()
+    B = torch.randn((N, K) if tb else (K, N), generator=g).bfloat16()
+    ref = (A.float().t() if ta else A.float()) @ (B.float().t() if tb else B.float())
+    out = ra.gemm_bf16(A.to(DEV), B.to(DEV), trans_a=ta, trans_b=tb)
+    rel_ok(out, ref, "bf16 out")
+    acc = torch.ones(M, N, dtype=torch.float32, device=DEV)
+    ra.gemm_bf16(A.to(DEV), B.to(DEV), trans_a=ta, trans_b=tb, out=acc, accumulate=True)
+    assert errors(acc, ref + 1.0)[1] < 1e-5
+
+
 def test_gemm_rejects_ragged_shapes():
     A = torch.zeros(100, 64, dtype=torch.bfloat16, device=DEV)
     B = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
