@@ -30,11 +30,13 @@ void set_error(const char* fmt, ...);
 
 // ---------------------------------------------------------------- bf16 <-> fp32
 __device__ __forceinline__ float bf16_to_f32(uint16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even, NaN kept
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even, NaN kept: v_cvt_pk_bf16_f32
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {  // lo in bits 0..15
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
 }
 template <typename T> __device__ __forceinline__ float load_f32(const T* p);
 template <> __device__ __forceinline__ float load_f32<float>(const float* p) { return *p; }

@@ -20,7 +20,8 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #ifndef RA_W4_ABL
-#define RA_W4_ABL 0     // timing experiments only: 1 = no global loads, 2 = no LDS stores, 4 = no LDS reads in the K loop, 8 = no barrier, 16 = no epilogue
+// timing experiments only (results are wrong): 1 = no global loads, 2 = no LDS stores, 4 = no LDS reads, 8 = no barrier
+#define RA_W4_ABL 0
 #endif
 constexpr int GBK = 64;               // K step of the 8-wavefront tiles (and the granularity required of K)
 
@@ -51,6 +52,43 @@ __device__ __forceinline__ bool tile_of_block(int ntm, int ntn, int& tm, int& tn
   tm = first_m + in_group % rows;
   tn = in_group / rows;
   return true;
+}
+
+// One wavefront's accumulators -> C.  A lane holds column lo of each 32 x 32 block, rows 8 (r / 4) + 4 hi + r % 4:
+// written straight to memory that is one 4-byte access per lane and register.  Each block goes through a
+// 32 x 36 float patch of LDS private to the wavefront instead and leaves as 16 bytes per lane (rows of 128
+// bytes).  MODE 0: bf16 C, 1: fp32 C, 2: fp32 C +=.  Blocks alternate between patch0 and patch1 (which may be the
+// same): with two patches the LDS writes of a block overlap the reads and stores of the block before.
+template <int MODE, int MB, int NB>
+__device__ __forceinline__ void store_tile(f32x16 (&acc)[MB][NB], float* patch0, float* patch1, void* C, int ldc,
+                                           int row0, int col0, int lane) {
+  const int lo = lane & 31, hi = lane >> 5;
+  const int er = lane >> 3, ec = (lane & 7) * 4;          // this lane's row (of 8 per pass) and first column
+#pragma unroll
+  for (int i = 0; i < MB; i++)
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+      float* patch = ((i * NB + j) & 1) ? patch1 : patch0;
+#pragma unroll
+      for (int r = 0; r < 16; r++) patch[((r >> 2) * 8 + hi * 4 + (r & 3)) * 36 + lo] = acc[i][j][r];
+#pragma unroll
+      for (int pass = 0; pass < 4; pass++) {
+        const int row = pass * 8 + er;
+        const float4 v = *(const float4*)&patch[row * 36 + ec];
+        const int64_t o = (int64_t)(row0 + i * 32 + row) * ldc + col0 + j * 32 + ec;
+        if (MODE == 0) {
+          uint2 w;
+          w.x = f32x2_to_bf16x2(v.x, v.y);
+          w.y = f32x2_to_bf16x2(v.z, v.w);
+          *(uint2*)((uint16_t*)C + o) = w;
+        } else {
+          float4* c = (float4*)((float*)C + o);
+          float4 w = v;
+          if (MODE == 2) { const float4 old = *c; w.x += old.x; w.y += old.y; w.z += old.z; w.w += old.w; }
+          *c = w;
+        }
+      }
+    }
 }
 
 // TA: A is stored (K,M).  TB: B is stored (N,K).
@@ -201,38 +239,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
 #undef RA_A_LDS
 #undef RA_B_LDS
 
-  // epilogue.  A lane holds column n = lo of each 32x32 block, rows 8*(r/4) + 4*hi + r%4: written straight to
-  // memory that is one 4-byte access per lane and register.  Each block goes through a private 32 x 36 float
-  // patch of LDS instead (the operand tiles are dead by now) and leaves as 16 bytes per lane: rows of 128
-  // bytes, a quarter of the memory instructions.
+  // epilogue through one LDS patch per wavefront (the operand tiles are dead by now)
   __syncthreads();
   static_assert(sizeof(As) >= (size_t)NT / 64 * 32 * 36 * sizeof(float), "operand tile too small for the epilogue patches");
   float* patch = (float*)&As[0][0] + wave * (32 * 36);
-  const int er = lane >> 3, ec = (lane & 7) * 4;          // this lane's row (of 8 per pass) and first column
-#pragma unroll
-  for (int i = 0; i < MB; i++)
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) patch[((r >> 2) * 8 + hi * 4 + (r & 3)) * 36 + lo] = acc[i][j][r];
-#pragma unroll
-      for (int pass = 0; pass < 4; pass++) {
-        const int row = pass * 8 + er;
-        const float4 v = *(const float4*)&patch[row * 36 + ec];
-        const int64_t o = (int64_t)(m0 + wm * WM + i * 32 + row) * g.N + n0 + wn * WN + j * 32 + ec;
-        if (g.c_f32) {
-          float4* c = (float4*)((float*)g.C + o);
-          float4 w = v;
-          if (g.beta_one) { const float4 old = *c; w.x += old.x; w.y += old.y; w.z += old.z; w.w += old.w; }
-          *c = w;
-        } else {
-          uint2 w;
-          w.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
-          w.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
-          *(uint2*)((uint16_t*)g.C + o) = w;
-        }
-      }
-    }
+  if (!g.c_f32) store_tile<0>(acc, patch, patch, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
+  else if (!g.beta_one) store_tile<1>(acc, patch, patch, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
+  else store_tile<2>(acc, patch, patch, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
 // 256 x 256 tile over FOUR wavefronts (2 x 2), one per SIMD with all 512 registers: each wavefront owns 128 x 128
@@ -244,7 +257,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
 template <bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   constexpr int BM = 256, BN = 256, BK = 32, NT = 256, WM = 128, WN = 128;
-  constexpr int NAT_STR = BK + 8;
+  // A row-wise read tile has rows of 32 elements = four 16-byte chunks and no padding; chunk c of row r sits at
+  // chunk c ^ ((r >> 2) & 3): sixteen consecutive rows then put a given chunk in sixteen different bank groups
+  // (conflict-free fragment reads), and a row stays one contiguous 64 bytes (conflict-free staging writes).
+  constexpr int NAT_STR = BK;
   constexpr int A_STR = TA ? BM + 32 : NAT_STR, B_STR = TB ? NAT_STR : BN + 32;
   constexpr int A_ROWS = TA ? BK : BM, B_ROWS = TB ? BN : BK;
   constexpr int A_CPR = (TA ? BM : BK) / 8, B_CPR = (TB ? BK : BN) / 8;
@@ -283,8 +299,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
     const int ia = c * NT + tid, ib = c * NT + tid;
     ga[c] = TA ? (int64_t)(ia / A_CPR) * lda + m0 + (ia % A_CPR) * 8 : (int64_t)(m0 + ia / A_CPR) * lda + (ia % A_CPR) * 8;
     gb[c] = TB ? (int64_t)(n0 + ib / B_CPR) * ldb + (ib % B_CPR) * 8 : (int64_t)(ib / B_CPR) * ldb + n0 + (ib % B_CPR) * 8;
-    la[c] = (ia / A_CPR) * A_STR + (ia % A_CPR) * 8;
-    lb[c] = (ib / B_CPR) * B_STR + (ib % B_CPR) * 8;
+    la[c] = (ia / A_CPR) * A_STR + (TA ? ia % A_CPR : (ia % A_CPR) ^ ((ia / A_CPR >> 2) & 3)) * 8;
+    lb[c] = (ib / B_CPR) * B_STR + (TB ? (ib % B_CPR) ^ ((ib / B_CPR >> 2) & 3) : ib % B_CPR) * 8;
   }
   const int64_t ka = TA ? (int64_t)lda : 1, kb = TB ? 1 : (int64_t)ldb;    // stride of the K position
 #define RA_W4_LOAD_A(S, T)                                                                              \
@@ -311,19 +327,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   }
   const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wm * WM;
   const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wn * WN;
-  const int natA = (wm * WM + lo) * A_STR + hi * 8, natB = (wn * WN + lo) * B_STR + hi * 8;
+  // row-wise fragment of K slice kk: row lo, chunk (2 kk + hi) ^ ((lo >> 2) & 3)
+  const int nsw = hi ^ ((lo >> 2) & 3);
+  const int natA0 = (wm * WM + lo) * A_STR + nsw * 8, natA1 = (wm * WM + lo) * A_STR + (nsw ^ 2) * 8;
+  const int natB0 = (wn * WN + lo) * B_STR + nsw * 8, natB1 = (wn * WN + lo) * B_STR + (nsw ^ 2) * 8;
   // the eight fragments of K slice KK of buffer BUF into set F (F##a[0..3], F##b[0..3])
 #define RA_W4_FRAGS(F, BUF, KK)                                                                         \
   _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                       \
     if (!TA) {                                                                                          \
-      F##a[i] = *(const bf16x8*)(&RA_W4_AS(BUF)[natA + i * 32 * A_STR + (KK) * 16]);                          \
+      F##a[i] = *(const bf16x8*)(&RA_W4_AS(BUF)[((KK) ? natA1 : natA0) + i * 32 * A_STR]);                          \
     } else {                                                                                            \
       const uint16_t* p = &RA_W4_AS(BUF)[(KK) * 16 * A_STR + trA + i * 32];                                   \
       s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);                                                 \
       F##a[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
     if (TB) {                                                                                           \
-      F##b[i] = *(const bf16x8*)(&RA_W4_BS(BUF)[natB + i * 32 * B_STR + (KK) * 16]);                          \
+      F##b[i] = *(const bf16x8*)(&RA_W4_BS(BUF)[((KK) ? natB1 : natB0) + i * 32 * B_STR]);                          \
     } else {                                                                                            \
       const uint16_t* p = &RA_W4_BS(BUF)[(KK) * 16 * B_STR + trB + i * 32];                                   \
       s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);                                                 \
@@ -385,38 +404,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
 #undef RA_W4_LOAD_B
 #undef RA_W4_SCHED
 
-  // epilogue through per-wavefront LDS patches, as in gemm_bf16_kernel
-  if (RA_W4_ABL & 16) { if (acc[0][0][0] == 123.f) *(float*)g.C = acc[1][1][1] + acc[2][2][2] + acc[3][3][3]; return; }
+  // epilogue through two LDS patches per wavefront, one operand array each (the operand tiles are dead by now)
   __syncthreads();
-  static_assert(sizeof(As0) >= (size_t)4 * 32 * 36 * sizeof(float), "operand tile too small for the epilogue patches");
-  float* patch = (float*)&As0[0] + wave * (32 * 36);
-  const int er = lane >> 3, ec = (lane & 7) * 4;
-#pragma unroll
-  for (int i = 0; i < 4; i++)
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) patch[((r >> 2) * 8 + hi * 4 + (r & 3)) * 36 + lo] = acc[i][j][r];
-#pragma unroll
-      for (int pass = 0; pass < 4; pass++) {
-        const int row = pass * 8 + er;
-        const float4 v = *(const float4*)&patch[row * 36 + ec];
-        const int64_t o = (int64_t)(m0 + wm * WM + i * 32 + row) * g.N + n0 + wn * WN + j * 32 + ec;
-        if (g.c_f32) {
-          float4* c = (float4*)((float*)g.C + o);
-          float4 w = v;
-          if (g.beta_one) { const float4 old = *c; w.x += old.x; w.y += old.y; w.z += old.z; w.w += old.w; }
-          *c = w;
-        } else {
-          uint2 w;
-          w.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
-          w.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
-          *(uint2*)((uint16_t*)g.C + o) = w;
-        }
-      }
-    }
+  static_assert(sizeof(As0) >= (size_t)2 * 32 * 36 * sizeof(float) && sizeof(Bs0) >= (size_t)2 * 32 * 36 * sizeof(float),
+                "operand tile too small for two epilogue patches");
+  float* patch = (float*)(wave == 0 ? &As0[0] : wave == 1 ? &As1[0] : wave == 2 ? &Bs0[0] : &Bs1[0]);
+  if (!g.c_f32) store_tile<0>(acc, patch, patch + 32 * 36, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
+  else if (!g.beta_one) store_tile<1>(acc, patch, patch + 32 * 36, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
+  else store_tile<2>(acc, patch, patch + 32 * 36, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
 }
-
 template <bool TA, bool TB>
 static int launch_w4(const GemmArgs& g, hipStream_t s) {
   const long long nwg = ((long long)(g.M / 256) * (g.N / 256) + 7) / 8 * 8;
