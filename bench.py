@@ -260,6 +260,12 @@ def bench_ffn(args):
     ms = _time_steps(step, args.steps, args.warmup)
     flops = 18.0 * T * d * f
     value = flops / (ms * 1e-3) / 1e12
+    # dominant kernel: the GEMM a = x w1 of one launch (tokens_per_launch x hidden x intermediate), timed alone
+    slab = ra.feedforward._slab_tokens(chunk, T // chunk)
+    xs = x.detach()[0, :slab]
+    a_out = torch.empty(slab, f, dtype=torch.bfloat16, device=dev)
+    gemm_ms = _event_ms(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out), 5)
+    gemm_tf = 2.0 * slab * d * f / (gemm_ms * 1e-3) / 1e12
     cpu = None
     if not args.no_cpu:
         from oracle import ringattention_oracle as O
@@ -280,9 +286,12 @@ def bench_ffn(args):
         "metric": "swiglu_ffn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
         "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "config": {"workload": "ffn", "tokens": T, "hidden": d, "intermediate": f, "chunk_size": chunk,
+                   "tokens_per_launch": ra.feedforward._slab_tokens(chunk, T // chunk),
                    "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
-        "roofline": {"bound": "mfma", "kernel": "gemm_bf16_kernel", "achieved": round(value, 1), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None},
+        "roofline": {"bound": "mfma", "kernel": "gemm_bf16_w4_kernel<false, false> (a = x w1 of one launch)",
+                     "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel_ms": {"gemm_bf16_w4_kernel<false, false>": round(gemm_ms, 3)}},
         "cpu_baseline": cpu,
     }
 

@@ -433,13 +433,12 @@ static int launch_tile(const GemmArgs& g, hipStream_t s) {
 // workgroups: take the largest tile whose last round is not mostly idle.
 static int pick_tile(int M, int N) {
   if (const char* e = getenv("RA_GEMM_TILE")) return atoi(e);
-  static int ncu = 0;
-  if (!ncu) {
-    int dev = 0;
+  static const int ncu = [] {     // initialised once, thread-safe
+    int dev = 0, n = 0;
     hipDeviceProp_t pr;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) ncu = pr.multiProcessorCount;
-    if (ncu <= 0) ncu = 256;
-  }
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) n = pr.multiProcessorCount;
+    return n > 0 ? n : 256;
+  }();
   auto eff = [&](int bm, int bn) {
     if (M % bm || N % bn) return 0.0;
     const double n = (double)(M / bm) * (N / bn);

@@ -117,9 +117,8 @@ MAX_SLAB_TOKENS = 16384
 
 
 def _slab_tokens(chunk_size, n_chunks):
-    import os
-    cap = int(os.environ.get("RA_FFN_SLAB_TOKENS", MAX_SLAB_TOKENS))
-    g = max(1, min(n_chunks, cap // chunk_size))
+    """Tokens per launch: the largest whole number of chunks within MAX_SLAB_TOKENS that divides the scan."""
+    g = max(1, min(n_chunks, MAX_SLAB_TOKENS // chunk_size))
     while n_chunks % g:
         g -= 1
     return chunk_size * g

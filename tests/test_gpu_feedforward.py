@@ -63,8 +63,13 @@ def test_gemm_rejects_ragged_shapes():
         ra.gemm_bf16(A, B)
 
 
-def test_swiglu_forward_backward_match_autograd():
-    T, d, f = 256, 256, 384
+@pytest.mark.parametrize("tile,shape", [(None, (256, 256, 384)), (0, (512, 256, 768)), (1, (512, 256, 768))])
+def test_swiglu_forward_backward_match_autograd(monkeypatch, tile, shape):
+    """SwiGLU forward and backward (including the two-operand-pair GEMM of dx and the fp32 accumulation of the
+    weight gradients) with the library's own tile choice and with each of the large tile kernels forced."""
+    T, d, f = shape
+    if tile is not None:
+        monkeypatch.setenv("RA_GEMM_TILE", str(tile))
     g = torch.Generator().manual_seed(0)
     x = torch.randn(1, T, d, generator=g).bfloat16()
     dy = torch.randn(1, T, d, generator=g).bfloat16()
