@@ -253,7 +253,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
 // half the LDS bytes per MFMA of the eight-wavefront tile, which is LDS-bound.  With a single wavefront per SIMD
 // nothing hides latency but the wavefront's own pipelining: K step 32 = two slices; the fragments of a slice are
 // requested from LDS one slice (sixteen MFMAs) before their use, across the barrier of the K step; a K slab stays
-// in flight from global memory for two K steps in one of two register sets.
+// in flight from global memory for four K steps in one of four register sets.
 template <bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   constexpr int BM = 256, BN = 256, BK = 32, NT = 256, WM = 128, WN = 128;
@@ -287,7 +287,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
+  // four sets of staging registers: slab j lives in set j % 4 from its request until it is stored to LDS four K
+  // steps later (about 2 us: an L2 miss served from HBM under load takes that long)
   uint4 Pa0, Pa1, Pa2, Pa3, Pb0, Pb1, Pb2, Pb3, Qa0, Qa1, Qa2, Qa3, Qb0, Qb1, Qb2, Qb3;
+  uint4 Ra0, Ra1, Ra2, Ra3, Rb0, Rb1, Rb2, Rb3, Ta0, Ta1, Ta2, Ta3, Tb0, Tb1, Tb2, Tb3;
   const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
   const int nk = g.K / BK;
   const int total = nk * (g.A2 ? 2 : 1);
@@ -384,14 +387,23 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   bf16x8 Fa[4], Fb[4], Ga[4], Gb[4];
   RA_W4_LOAD(P, 0);
   RA_W4_LOAD(Q, 1);
+  RA_W4_LOAD(R, 2);
+  RA_W4_LOAD(T, 3);
   RA_W4_STORE(P, 0);
-  RA_W4_LOAD(P, 2);
+  RA_W4_LOAD(P, 4);
   __syncthreads();
   RA_W4_FRAGS(F, 0, 0);
-  // K is a multiple of 64: an even number of slabs
-  for (int it = 0; it < total; it += 2) {
-    RA_W4_STEP(0, Q, it + 3);
-    RA_W4_STEP(1, P, it + 4);
+  // K is a multiple of 64: an even number of slabs; four steps per trip, two more when that leaves a remainder
+  int it = 0;
+  for (; it + 4 <= total; it += 4) {
+    RA_W4_STEP(0, Q, it + 5);
+    RA_W4_STEP(1, R, it + 6);
+    RA_W4_STEP(0, T, it + 7);
+    RA_W4_STEP(1, P, it + 8);
+  }
+  if (it < total) {
+    RA_W4_STEP(0, Q, it + 5);
+    RA_W4_STEP(1, R, it + 6);
   }
 #undef RA_W4_STEP
 #undef RA_W4_AS
