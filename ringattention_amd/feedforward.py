@@ -164,13 +164,11 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
             raise NotImplementedError("SwiGLU kernels are bf16")
         if not inputs.is_cuda:
             raise RuntimeError("ringattention_amd runs on the GPU only")
-        if b == 1:
-            # contiguous slabs of chunk_size tokens, one autograd node for the whole scan
-            y = _BlockwiseSwiGLUFn.apply(inputs.reshape(s, d).contiguous(), feedforward.w1, feedforward.w2,
-                                         feedforward.w3, _slab_tokens(chunk_size, n))
-            return y.reshape(1, s, y.shape[-1])
-        outs = [feedforward(inputs[:, j * chunk_size:(j + 1) * chunk_size]) for j in range(n)]
-        return torch.cat(outs, dim=1)
+        # contiguous slabs of chunk_size tokens (batch rows one after the other: a token-wise MLP does not see the
+        # difference), one autograd node for the whole scan
+        y = _BlockwiseSwiGLUFn.apply(inputs.reshape(b * s, d).contiguous(), feedforward.w1, feedforward.w2,
+                                     feedforward.w3, _slab_tokens(chunk_size, b * n))
+        return y.reshape(b, s, y.shape[-1])
     x = inputs.reshape(b, chunk_size, n, d)
     outs = [feedforward(x[:, :, j, :]) for j in range(n)]
     out = torch.stack(outs, dim=2)
