@@ -258,3 +258,23 @@ def test_mfma_packed_documents_with_bias_ring8():
     assert_close(out, ref_out, torch.bfloat16, "out")
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
         assert_close(a, b, torch.bfloat16, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_frozen_vectors(dtype):
+    """The HIP path against tests/golden/oracle_vectors.npz (outputs of the CPU oracle, frozen; inputs are
+    bf16-representable, so both dtypes see the same numbers)."""
+    from tests.golden_vectors import load
+    cases = load()
+    for name in ("ring2_causal_bias_segments", "one_device_causal_block4", "decode_cache_idx_70"):
+        c = cases[name]
+        i, cfg = c["in"], c["cfg"]
+        print("frozen", name, dtype, flush=True)
+        kw = kwargs(cfg["qc"], cfg["kc"], cfg["cbs"])
+        do = i["do"].to(dtype) if "do" in i else None
+        out, grads = run_hip(i["q"].to(dtype), i["k"].to(dtype), i["v"].to(dtype), do, i.get("bias"), i.get("seg"),
+                             cfg.get("cache_idx"), cfg["n"], kw)
+        assert_close(out, c["out"]["out"], dtype, name + " out")
+        if grads is not None:
+            for nm, gr in zip(("dq", "dk", "dv"), grads):
+                assert_close(gr, c["out"][nm], dtype, name + " " + nm)

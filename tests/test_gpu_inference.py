@@ -179,3 +179,15 @@ def test_inference_mfma_and_generic_kernels_agree():
     assert_close(out, out_g, torch.bfloat16, "out")
     for name, a, b in zip(("dq", "dk", "dv"), grads, grads_g):
         assert_close(a, b, torch.bfloat16, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_inference_frozen_vectors(dtype):
+    """The HIP path against tests/golden/oracle_vectors.npz (outputs of the CPU oracle, frozen)."""
+    from tests.golden_vectors import load
+    c = load()["inference_ring2"]
+    i = c["in"]
+    out, grads = _run(i["q"].to(dtype), i["k"].to(dtype), i["v"].to(dtype), i["do"].to(dtype), i["mask"], 2)
+    assert_close(out, c["out"]["out"], dtype, "out")
+    for name, a in zip(("dq", "dk", "dv"), grads):
+        assert_close(a, c["out"][name], dtype, name)

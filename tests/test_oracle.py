@@ -391,3 +391,33 @@ def test_inference_equals_ring_attention_with_causal_mask():
     a, _ = O.ring_attention_inference_fwd(q, k, v, mask, 2, True)
     b = O.ring_attention(q, k, v, None, None, None, 2, True, kwargs(16, 16, 1))
     assert (a - b).abs().max() < 1e-5
+
+
+# ----------------------------------------------------------------------------- frozen vectors
+
+def test_oracle_reproduces_its_frozen_vectors():
+    """tests/golden/oracle_vectors.npz holds outputs of this oracle frozen after it passed the checks above (the
+    reference has no vectors): a change that moves them is caught here before it reaches the GPU comparisons."""
+    from tests.golden_vectors import load
+    cases = load()
+    for name in ("ring2_causal_bias_segments", "one_device_causal_block4", "decode_cache_idx_70"):
+        c = cases[name]
+        i, cfg = c["in"], c["cfg"]
+        out, res = O.ring_attention_fwd(i["q"], i["k"], i["v"], i.get("bias"), i.get("seg"), cfg.get("cache_idx"),
+                                        cfg["n"], True, kwargs(cfg["qc"], cfg["kc"], cfg["cbs"]))
+        assert torch.allclose(out, c["out"]["out"], rtol=1e-5, atol=1e-6), name
+        if "do" in i:
+            grads = O.ring_attention_bwd(cfg["n"], True, kwargs(cfg["qc"], cfg["kc"], cfg["cbs"]), res, i["do"])
+            for nm, gr in zip(("dq", "dk", "dv"), grads):
+                assert torch.allclose(gr, c["out"][nm], rtol=1e-5, atol=1e-6), (name, nm)
+    c = cases["inference_ring2"]
+    out, res = O.ring_attention_inference_fwd(c["in"]["q"], c["in"]["k"], c["in"]["v"], c["in"]["mask"], 2)
+    assert torch.allclose(out, c["out"]["out"], rtol=1e-5, atol=1e-6)
+    for nm, gr in zip(("dq", "dk", "dv"), O.ring_attention_inference_bwd(2, res, c["in"]["do"])):
+        assert torch.allclose(gr.float(), c["out"][nm], rtol=1e-5, atol=1e-6), nm
+    c = cases["ffn_chunk8"]
+    x, w1, w2, w3 = (c["in"][n_].clone().requires_grad_(True) for n_ in ("x", "w1", "w2", "w3"))
+    y = O.blockwise_feedforward(lambda h: O.swiglu(h, w1, w2, w3), x, 8)
+    y.backward(c["in"]["dy"])
+    for nm, t in dict(y=y, dx=x.grad, dw1=w1.grad, dw2=w2.grad, dw3=w3.grad).items():
+        assert torch.allclose(t, c["out"][nm], rtol=1e-5, atol=1e-6), nm
