@@ -296,6 +296,123 @@ def bench_ffn(args):
     }
 
 
+# --------------------------------------------------------------------------- steps either side of the path
+def bench_decode_step(args):
+    """A decode step as a model runs it: rotate + append the new token at cache_idx, then attend over the cache."""
+    import torch
+    import ringattention_amd as ra
+    dev = "cuda:0"
+    B, H, D, kc = 16, 32, 128, 512
+    Lf = args.seq_len or 262144
+    L = Lf + kc
+    k = torch.empty(B, L, H, D, dtype=torch.bfloat16, device=dev)
+    v = torch.empty(B, L, H, D, dtype=torch.bfloat16, device=dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    for b in range(B):
+        k[b].copy_(torch.randn(L, H, D, device=dev, generator=g))
+        v[b].copy_(torch.randn(L, H, D, device=dev, generator=g))
+    q, kn, vn = (torch.randn(B, 1, H, D, device=dev, generator=g).to(torch.bfloat16) for _ in range(3))
+    qr, out = torch.empty_like(q), torch.empty_like(q)
+    kw = _kwargs(1, kc, 1)
+    ci = torch.zeros(1, dtype=torch.int32, device=dev)
+    state = {"t": 0}
+
+    def prologue():
+        ra.rope_kv_append(q, kn, vn, k, v, ci, q_out=qr)
+
+    def step():
+        ci.fill_(Lf + state["t"] % 64)
+        state["t"] += 1
+        prologue()
+        ra.decode_attention(qr, k, v, None, None, ci, kw, out=out)
+
+    ms = _time_steps(step, args.steps, args.warmup)
+    bytes_step = 2.0 * B * (Lf + 1) * H * D * 2
+    value = bytes_step / (ms * 1e-3) / 1e9
+    pro_ms = _event_ms(prologue, 20)
+    pro_bytes = 7.0 * B * H * D * 2          # q, k_new, v_new in; q_out, cache K and V rows out
+    cpu = None
+    if not args.no_cpu:
+        from oracle import ringattention_oracle as O
+        gq = torch.Generator().manual_seed(0)
+        qc_, knc, vnc = (torch.randn(B, 1, H, D, generator=gq) for _ in range(3))
+        kcc, vcc = torch.zeros(B, 64, H, D), torch.zeros(B, 64, H, D)
+        t0 = time.perf_counter()
+        reps = 200
+        for _ in range(reps):
+            O.rope_kv_append(qc_, knc, vnc, kcc, vcc, 37)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(reps / dt, 1), "unit": "prologues/s", "cores": 1, "kind": "port",
+               "sample": "rotate + append of B=16 H=32 D=128 into a 64-position buffer, %d calls, %.2f s" % (reps, dt)}
+    return {
+        "metric": "decode_step_hbm_gbs", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms, 3),
+        "dtype": "bf16", "pct_hbm_peak": round(100 * value / PEAK_HBM_GBS, 2),
+        "config": {"workload": "decode_step", "B": B, "H": H, "D": D, "cache_len": Lf, "key_chunk_size": kc,
+                   "rope_theta": 10000.0, "bytes_per_step": bytes_step},
+        "roofline": {"bound": "hbm", "kernel": "rope_kv_append_kernel", "achieved": round(pro_bytes / (pro_ms * 1e-3) / 1e9, 2),
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(pro_bytes / (pro_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 6),
+                     "traffic": None, "kernel_ms": {"rope_kv_append_kernel": round(pro_ms, 4)},
+                     "note": "917 KB per call: the launch, not the memory system, bounds this kernel"},
+        "cpu_baseline": cpu,
+    }
+
+
+def bench_rmsnorm(args):
+    """residual add + RMSNorm, forward and backward, over the FFN workload's activations (65536 x 4096, bf16)."""
+    import torch
+    import ringattention_amd as ra
+    dev = "cuda:0"
+    T, d = args.seq_len or 65536, 4096
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(1, T, d, device=dev, generator=g).to(torch.bfloat16).requires_grad_(True)
+    r = torch.randn(1, T, d, device=dev, generator=g).to(torch.bfloat16).requires_grad_(True)
+    w = torch.ones(d, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+    dn = torch.randn(1, T, d, device=dev, generator=g).to(torch.bfloat16)
+    dres = torch.randn(1, T, d, device=dev, generator=g).to(torch.bfloat16)
+
+    def fwd():
+        return ra.rmsnorm_residual(x, r, w)
+
+    def step():
+        x.grad = r.grad = w.grad = None
+        y, n = fwd()
+        torch.autograd.backward((y, n), (dres, dn))
+
+    ms = _time_steps(step, args.steps, args.warmup)
+    bytes_step = 8.0 * T * d * 2            # forward: x, r in, y, n out; backward: dn, y, dres in, dy out
+    value = bytes_step / (ms * 1e-3) / 1e9
+    with torch.no_grad():
+        f_ms = _event_ms(fwd, 5)
+    ach = 4.0 * T * d * 2 / (f_ms * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu:
+        from oracle import ringattention_oracle as O
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        Tc = 8192
+        gc = torch.Generator().manual_seed(0)
+        xc = torch.randn(Tc, d, generator=gc, requires_grad=True)
+        rc = torch.randn(Tc, d, generator=gc, requires_grad=True)
+        wc = torch.ones(d, requires_grad=True)
+        t0 = time.perf_counter()
+        reps = 5
+        for _ in range(reps):
+            yc, nc = O.rmsnorm_residual(xc, rc, wc)
+            (yc.sum() + nc.sum()).backward()
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(reps * 8.0 * Tc * d * 2 / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": "8192 rows (of 65536), fwd+bwd fp32, %d repeats, %.1f s; bytes counted as for bf16" % (reps, dt)}
+    return {
+        "metric": "rmsnorm_residual_fwd_bwd_gbs", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms, 3),
+        "dtype": "bf16", "pct_hbm_peak": round(100 * value / PEAK_HBM_GBS, 2),
+        "config": {"workload": "rmsnorm", "tokens": T, "hidden": d, "bytes_per_step": bytes_step},
+        "roofline": {"bound": "hbm", "kernel": "rmsnorm_fwd_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                     "kernel_ms": {"rmsnorm_fwd_kernel": round(f_ms, 4)}},
+        "cpu_baseline": cpu,
+    }
+
+
 # --------------------------------------------------------------------------- calibration copy
 def bench_copy(args):
     """A plain 1 GiB device-to-device copy: the kernel of known size that the FETCH_SIZE / WRITE_SIZE
@@ -358,7 +475,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy"])
+    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -375,6 +492,10 @@ def main():
         r = bench_decode(args)
     elif args.workload == "copy":
         r = bench_copy(args)
+    elif args.workload == "decode_step":
+        r = bench_decode_step(args)
+    elif args.workload == "rmsnorm":
+        r = bench_rmsnorm(args)
     elif args.workload == "inference":
         r = bench_inference(args)
     else:

@@ -205,6 +205,52 @@ int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream);
 int ra_gemm_bf16(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K,
                  int32_t trans_a, int32_t trans_b, int32_t c_dtype, int32_t beta_one, ra_stream_t stream);
 
+/*
+ * Steps either side of the hot path (the reference repository has no counterpart: its README points at the LWM
+ * model code for them; the formulas are the LLaMA ones).
+ *
+ * ra_rope_kv_append: before a decode step.  Rotates the new token's query and key by position pos = *cache_idx
+ * (or cache_idx_host when cache_idx is null): pair (x0, x1) -> (x0 cos a - x1 sin a, x0 sin a + x1 cos a),
+ * a = pos * rope_theta^(-2j/D), j = 0 .. D/2-1, pairs (2j, 2j+1) [RA_ROPE_ADJACENT] or (j, j+D/2) [RA_ROPE_HALF];
+ * writes the rotated key and the value into the cache buffers at position pos of every batch row - the buffers
+ * that ra_decode_fwd / ringattention(..., cache_idx) then read whole (ringattention_jax.py:31-35).  rope_theta <= 0
+ * appends without rotating.  A position outside [0, L) writes nothing.
+ */
+enum { RA_ROPE_ADJACENT = 0, RA_ROPE_HALF = 1 };
+typedef struct ra_rope_append_params {
+  const void* q; void* q_out;             /* (B,1,H,D); q_out may alias q */
+  const void* k_new; const void* v_new;   /* (B,1,H,D) */
+  void* k_cache; void* v_cache;           /* (B,L,H,D) */
+  const int32_t* cache_idx;               /* device int32 scalar, nullable */
+  int32_t cache_idx_host;
+  int32_t dtype;
+  int32_t B, L, H, D;
+  int64_t q_stride_b, q_out_stride_b, new_stride_b, cache_stride_b, cache_stride_s;   /* elements; head stride D */
+  float rope_theta;
+  int32_t rope_style;
+} ra_rope_append_params;
+int ra_rope_kv_append(const ra_rope_append_params* p, ra_stream_t stream);
+
+/*
+ * ra_rmsnorm_fwd / _bwd: around blockwise_feedforward (ringattention_jax.py:333-352).  bf16 rows of d elements
+ * (d a multiple of 8, at most 8192), fp32 arithmetic:
+ *   forward   y = x + residual (residual nullable: then y is not written and y = x), rstd = rsqrt(mean(y^2) + eps),
+ *             normed = y * rstd * weight
+ *   backward  d_y = rstd * (d_normed * weight) - y * rstd^3 / d * sum(d_normed * weight * y) (+ d_residual, nullable),
+ *             d_weight += sum over rows of d_normed * y * rstd      (fp32, added into)
+ * dw_workspace: ra_rmsnorm_workspace_bytes(T, d) bytes, backward only.
+ */
+typedef struct ra_rmsnorm_params {
+  int64_t T; int32_t d; float eps;
+  const void* x; const void* residual; const void* weight;
+  void* y; void* normed; float* rstd;                 /* rstd (T) fp32: written by the forward, read by the backward */
+  const void* d_normed; const void* d_residual;       /* backward */
+  void* d_y; float* d_weight; float* dw_workspace; size_t dw_workspace_bytes;
+} ra_rmsnorm_params;
+size_t ra_rmsnorm_workspace_bytes(int64_t T, int32_t d);
+int ra_rmsnorm_fwd(const ra_rmsnorm_params* p, ra_stream_t stream);
+int ra_rmsnorm_bwd(const ra_rmsnorm_params* p, ra_stream_t stream);
+
 const char* ra_last_error(void);
 int ra_version(void);
 

@@ -25,6 +25,12 @@ vectors, and JAX/flax are not importable where this was written):
   against ``dense_attention_inference`` (an un-chunked masked softmax) and its torch autograd, over
   ring sizes, broadcast mask shapes and rows with no attended key.
 
+* ``rope_rotate`` / ``rope_kv_append`` / ``rmsnorm_residual`` (steps either side of the path; the reference
+  repository has no code for them, the formulas are the LLaMA ones): rotation checked against complex
+  multiplication, norm preservation, additivity in the position and the relative-position property of the
+  rotated dot product; RMSNorm against its definition in float64, unit RMS of the result, scale invariance and
+  torch autograd / finite differences for the backward formula.
+
 Parity unpinned (would need the reference's own runtime): the dropout mask
 bits (``jax.random`` stream) - dropout is refused - and XLA-CPU's exact
 summation order / its bf16 rounding of intermediate einsum results, both far
@@ -450,3 +456,43 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
     outs = [feedforward(x[:, :, j, :]) for j in range(n)]                   # :340-350
     out = torch.stack(outs, dim=2)
     return out.reshape(b, s, out.shape[-1])                                 # :351
+
+
+# ----------------------------------------------------------------------------- steps either side of the path
+
+def rope_rotate(x, pos, theta=10000.0, style="adjacent"):
+    """Rotary position embedding of x (..., D) at integer position ``pos``: the pair (x0, x1) of frequency index
+    j = 0 .. D/2-1 turns by the angle pos * theta^(-2j/D).  ``style`` "adjacent" pairs elements (2j, 2j+1),
+    "half" pairs (j, j + D/2).  Angles in float64; the result has x's dtype."""
+    D = x.shape[-1]
+    j = torch.arange(D // 2, dtype=torch.float64)
+    ang = float(pos) * torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * j / D)
+    cs, sn = torch.cos(ang).to(x.dtype), torch.sin(ang).to(x.dtype)
+    if style == "adjacent":
+        x0, x1 = x[..., 0::2], x[..., 1::2]
+    else:
+        x0, x1 = x[..., : D // 2], x[..., D // 2:]
+    y0, y1 = x0 * cs - x1 * sn, x0 * sn + x1 * cs
+    if style == "adjacent":
+        return torch.stack((y0, y1), dim=-1).reshape(x.shape)
+    return torch.cat((y0, y1), dim=-1)
+
+
+def rope_kv_append(q, k_new, v_new, k_cache, v_cache, cache_idx, theta=10000.0, style="adjacent"):
+    """The decode step's prologue: returns (q rotated, k_cache, v_cache) with the rotated new key and the new value
+    written at position cache_idx of copies of the caches.  theta None or 0: no rotation."""
+    rot = (lambda t: rope_rotate(t, cache_idx, theta, style)) if theta else (lambda t: t)
+    kc, vc = k_cache.clone(), v_cache.clone()
+    kc[:, cache_idx] = rot(k_new)[:, 0]
+    vc[:, cache_idx] = v_new[:, 0]
+    return rot(q), kc, vc
+
+
+def rmsnorm_residual(x, residual, weight, eps=1e-6, stream_dtype=None):
+    """y = x + residual (residual may be None); normed = y / sqrt(mean(y^2) + eps) * weight.  ``stream_dtype`` rounds
+    y to the dtype the residual stream is stored in before the norm is taken of it (what a bf16 model does)."""
+    y = x if residual is None else x + residual
+    if stream_dtype is not None:
+        y = y.to(stream_dtype).to(x.dtype)
+    rstd = torch.rsqrt((y * y).mean(dim=-1, keepdim=True) + eps)
+    return y, y * rstd * weight

@@ -74,6 +74,26 @@ class RaSwigluParams(C.Structure):
     ]
 
 
+class RaRopeAppendParams(C.Structure):
+    _fields_ = [
+        ("q", vp), ("q_out", vp), ("k_new", vp), ("v_new", vp), ("k_cache", vp), ("v_cache", vp),
+        ("cache_idx", vp), ("cache_idx_host", i32), ("dtype", i32),
+        ("B", i32), ("L", i32), ("H", i32), ("D", i32),
+        ("q_stride_b", i64), ("q_out_stride_b", i64), ("new_stride_b", i64), ("cache_stride_b", i64),
+        ("cache_stride_s", i64), ("rope_theta", f32), ("rope_style", i32),
+    ]
+
+
+class RaRmsnormParams(C.Structure):
+    _fields_ = [
+        ("T", i64), ("d", i32), ("eps", f32),
+        ("x", vp), ("residual", vp), ("weight", vp),
+        ("y", vp), ("normed", vp), ("rstd", vp),
+        ("d_normed", vp), ("d_residual", vp),
+        ("d_y", vp), ("d_weight", vp), ("dw_workspace", vp), ("dw_workspace_bytes", C.c_size_t),
+    ]
+
+
 # every symbol include/ringattn_hip.h declares: (name, restype, argtypes)
 SYMBOLS = {
     "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
@@ -88,6 +108,10 @@ SYMBOLS = {
     "ra_swiglu_fwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
     "ra_swiglu_bwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
     "ra_gemm_bf16": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp]),
+    "ra_rope_kv_append": (C.c_int, [C.POINTER(RaRopeAppendParams), vp]),
+    "ra_rmsnorm_workspace_bytes": (C.c_size_t, [i64, i32]),
+    "ra_rmsnorm_fwd": (C.c_int, [C.POINTER(RaRmsnormParams), vp]),
+    "ra_rmsnorm_bwd": (C.c_int, [C.POINTER(RaRmsnormParams), vp]),
     "ra_last_error": (C.c_char_p, []),
     "ra_version": (C.c_int, []),
 }

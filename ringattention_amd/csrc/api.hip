@@ -35,6 +35,12 @@ int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s);
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
               int beta_one, hipStream_t s);
 
+int rope_kv_append(const ra_rope_append_params* p, hipStream_t s);
+int rmsnorm_fwd(const ra_rmsnorm_params* p, hipStream_t s);
+int rmsnorm_bwd(const ra_rmsnorm_params* p, hipStream_t s);
+int rmsnorm_bwd_parts(int64_t T);
+int rmsnorm_max_d();
+
 static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
   RA_REQUIRE(m.query_chunk_size > 0 && m.key_chunk_size > 0, RA_ERR_INVALID, "%s: chunk sizes must be positive", who);
   RA_REQUIRE(Sq % m.query_chunk_size == 0, RA_ERR_INVALID, "%s: q_len %d is not a multiple of query_chunk_size %d",
@@ -72,6 +78,51 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
 using namespace ra;
 
 extern "C" {
+
+int ra_rope_kv_append(const ra_rope_append_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "rope_kv_append: null params");
+  RA_REQUIRE(p->q && p->q_out && p->k_new && p->v_new && p->k_cache && p->v_cache, RA_ERR_INVALID,
+             "rope_kv_append: null tensor");
+  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "rope_kv_append: dtype %d", p->dtype);
+  RA_REQUIRE(p->B > 0 && p->L > 0 && p->H > 0 && p->D > 0 && p->D % 2 == 0, RA_ERR_INVALID,
+             "rope_kv_append: bad shape (B %d, L %d, H %d, D %d; D must be even)", p->B, p->L, p->H, p->D);
+  RA_REQUIRE(p->rope_style == RA_ROPE_ADJACENT || p->rope_style == RA_ROPE_HALF, RA_ERR_INVALID,
+             "rope_kv_append: rope_style %d", p->rope_style);
+  if (!p->cache_idx)
+    RA_REQUIRE(p->cache_idx_host >= 0 && p->cache_idx_host < p->L, RA_ERR_INVALID,
+               "rope_kv_append: position %d outside the cache buffer of %d positions", p->cache_idx_host, p->L);
+  return rope_kv_append(p, (hipStream_t)stream);
+}
+
+size_t ra_rmsnorm_workspace_bytes(int64_t T, int32_t d) {
+  if (T <= 0 || d <= 0) return 0;
+  return (size_t)rmsnorm_bwd_parts(T) * (size_t)d * sizeof(float);
+}
+
+static int check_rmsnorm(const ra_rmsnorm_params* p, const char* who) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
+  RA_REQUIRE(p->T > 0 && p->T <= 0x7fffffff && p->d > 0, RA_ERR_INVALID, "%s: empty or oversized shape", who);
+  RA_REQUIRE(p->d % 8 == 0 && p->d <= rmsnorm_max_d(), RA_ERR_UNSUPPORTED,
+             "%s: row length %d must be a multiple of 8 and at most %d", who, p->d, rmsnorm_max_d());
+  return RA_OK;
+}
+
+int ra_rmsnorm_fwd(const ra_rmsnorm_params* p, ra_stream_t stream) {
+  if (int rc = check_rmsnorm(p, "rmsnorm_fwd")) return rc;
+  RA_REQUIRE(p->x && p->weight && p->normed && p->rstd && (p->residual == nullptr || p->y), RA_ERR_INVALID,
+             "rmsnorm_fwd: null tensor (y is needed when a residual is given)");
+  return rmsnorm_fwd(p, (hipStream_t)stream);
+}
+
+int ra_rmsnorm_bwd(const ra_rmsnorm_params* p, ra_stream_t stream) {
+  if (int rc = check_rmsnorm(p, "rmsnorm_bwd")) return rc;
+  RA_REQUIRE(p->d_normed && p->y && p->weight && p->rstd && p->d_y && p->d_weight && p->dw_workspace, RA_ERR_INVALID,
+             "rmsnorm_bwd: null tensor");
+  RA_REQUIRE(p->dw_workspace_bytes >= ra_rmsnorm_workspace_bytes(p->T, p->d), RA_ERR_INVALID,
+             "rmsnorm_bwd: workspace %zu bytes < %zu needed", p->dw_workspace_bytes,
+             ra_rmsnorm_workspace_bytes(p->T, p->d));
+  return rmsnorm_bwd(p, (hipStream_t)stream);
+}
 
 const char* ra_last_error(void) { return g_err; }
 int ra_version(void) { return 1; }

@@ -29,15 +29,17 @@ def test_struct_sizes_match_a_c_compiler(tmp_path):
     import ctypes
     import subprocess
     src = tmp_path / "sz.c"
-    src.write_text('#include <stdio.h>\n#include "%s"\nint main(){printf("%%zu %%zu %%zu %%zu %%zu\\n",'
+    src.write_text('#include <stdio.h>\n#include "%s"\nint main(){printf("%%zu %%zu %%zu %%zu %%zu %%zu %%zu\\n",'
                    'sizeof(ra_mask),sizeof(ra_attn_fwd_params),sizeof(ra_attn_bwd_params),'
-                   'sizeof(ra_decode_params),sizeof(ra_swiglu_params));return 0;}\n'
+                   'sizeof(ra_decode_params),sizeof(ra_swiglu_params),sizeof(ra_rope_append_params),'
+                   'sizeof(ra_rmsnorm_params));return 0;}\n'
                    % os.path.join(ROOT, "include", "ringattn_hip.h"))
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", str(src), "-o", str(exe)])
     sizes = [int(x) for x in subprocess.check_output([str(exe)]).split()]
     mine = [ctypes.sizeof(c) for c in (_lib.RaMask, _lib.RaAttnFwdParams, _lib.RaAttnBwdParams,
-                                       _lib.RaDecodeParams, _lib.RaSwigluParams)]
+                                       _lib.RaDecodeParams, _lib.RaSwigluParams, _lib.RaRopeAppendParams,
+                                       _lib.RaRmsnormParams)]
     assert sizes == mine
 
 
@@ -94,3 +96,15 @@ def test_invalid_arguments_return_codes_without_gpu():
     one = ctypes.c_void_p(16)      # any non-null address: the shape check comes before any use
     assert lib.ra_keep_pack(one, 0, 0, 100, 1, 1, 1, 100, 64, one, one, one, None) == _lib.RA_ERR_UNSUPPORTED
     assert b"multiples of 64" in lib.ra_last_error()
+    # the steps either side of the path validate before launching too
+    assert lib.ra_rope_kv_append(None, None) == _lib.RA_ERR_INVALID
+    r = _lib.RaRopeAppendParams()
+    r.q = r.q_out = r.k_new = r.v_new = r.k_cache = r.v_cache = 16
+    r.dtype, r.B, r.L, r.H, r.D, r.cache_idx_host = _lib.RA_BF16, 1, 8, 2, 15, 0
+    assert lib.ra_rope_kv_append(ctypes.byref(r), None) == _lib.RA_ERR_INVALID and b"even" in lib.ra_last_error()
+    r.D, r.cache_idx_host = 16, 8
+    assert lib.ra_rope_kv_append(ctypes.byref(r), None) == _lib.RA_ERR_INVALID and b"outside" in lib.ra_last_error()
+    n = _lib.RaRmsnormParams()
+    n.T, n.d = 4, 100
+    assert lib.ra_rmsnorm_fwd(ctypes.byref(n), None) == _lib.RA_ERR_UNSUPPORTED
+    assert lib.ra_rmsnorm_workspace_bytes(65536, 4096) == 4096 * 4096 * 4

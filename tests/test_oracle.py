@@ -421,3 +421,71 @@ def test_oracle_reproduces_its_frozen_vectors():
     y.backward(c["in"]["dy"])
     for nm, t in dict(y=y, dx=x.grad, dw1=w1.grad, dw2=w2.grad, dw3=w3.grad).items():
         assert torch.allclose(t, c["out"][nm], rtol=1e-5, atol=1e-6), nm
+
+
+# ----------------------------------------------------------------------------- steps either side of the path
+
+@pytest.mark.parametrize("style", ["adjacent", "half"])
+def test_rope_is_a_rotation_with_the_relative_position_property(style):
+    g = torch.Generator().manual_seed(5)
+    D = 32
+    x, y = torch.randn(3, 1, 2, D, generator=g, dtype=F64), torch.randn(3, 1, 2, D, generator=g, dtype=F64)
+    assert torch.equal(O.rope_rotate(x, 0, 10000.0, style), x)                                   # position 0: identity
+    r = O.rope_rotate(x, 1234, 10000.0, style)
+    assert torch.allclose(r.norm(dim=-1), x.norm(dim=-1), rtol=1e-12)                            # norms are kept
+    twice = O.rope_rotate(O.rope_rotate(x, 100, 10000.0, style), 23, 10000.0, style)
+    assert torch.allclose(twice, O.rope_rotate(x, 123, 10000.0, style), atol=1e-12)              # angles add
+    d1 = (O.rope_rotate(x, 700, 10000.0, style) * O.rope_rotate(y, 650, 10000.0, style)).sum(-1)
+    d2 = (O.rope_rotate(x, 50, 10000.0, style) * y).sum(-1)
+    assert torch.allclose(d1, d2, atol=1e-10)                                                    # only p - p' matters
+    # against complex multiplication by exp(i pos theta^(-2j/D)), an independent formulation
+    j = torch.arange(D // 2, dtype=F64)
+    w = torch.polar(torch.ones(D // 2, dtype=F64), 77.0 * 10000.0 ** (-2.0 * j / D))
+    if style == "adjacent":
+        z = torch.view_as_complex(x.reshape(*x.shape[:-1], D // 2, 2).contiguous()) * w
+        ref = torch.view_as_real(z).reshape(x.shape)
+    else:
+        z = torch.complex(x[..., : D // 2], x[..., D // 2:]) * w
+        ref = torch.cat((z.real, z.imag), dim=-1)
+    assert torch.allclose(O.rope_rotate(x, 77, 10000.0, style), ref, atol=1e-12)
+
+
+def test_rope_kv_append_writes_one_position():
+    g = torch.Generator().manual_seed(6)
+    B, L, H, D = 2, 9, 2, 8
+    q, kn, vn = (torch.randn(B, 1, H, D, generator=g, dtype=F64) for _ in range(3))
+    kc, vc = torch.randn(B, L, H, D, generator=g, dtype=F64), torch.randn(B, L, H, D, generator=g, dtype=F64)
+    qr, kc2, vc2 = O.rope_kv_append(q, kn, vn, kc, vc, 4)
+    keep = [i for i in range(L) if i != 4]
+    assert torch.equal(kc2[:, keep], kc[:, keep]) and torch.equal(vc2[:, keep], vc[:, keep])
+    assert torch.equal(vc2[:, 4], vn[:, 0]) and torch.equal(kc2[:, 4], O.rope_rotate(kn, 4)[:, 0])
+    assert torch.equal(qr, O.rope_rotate(q, 4))
+    q0, kc3, _ = O.rope_kv_append(q, kn, vn, kc, vc, 4, theta=None)
+    assert torch.equal(q0, q) and torch.equal(kc3[:, 4], kn[:, 0])
+
+
+def test_rmsnorm_residual_definition_invariances_and_gradient():
+    g = torch.Generator().manual_seed(7)
+    T, d = 5, 16
+    x, r = torch.randn(T, d, generator=g, dtype=F64), torch.randn(T, d, generator=g, dtype=F64)
+    w = torch.randn(d, generator=g, dtype=F64)
+    y, n = O.rmsnorm_residual(x, r, w, eps=0.0)
+    assert torch.equal(y, x + r)
+    ones = torch.ones(d, dtype=F64)
+    _, n1 = O.rmsnorm_residual(x, r, ones, eps=0.0)
+    assert torch.allclose((n1 * n1).mean(-1), torch.ones(T, dtype=F64), rtol=1e-12)              # unit RMS
+    assert torch.allclose(O.rmsnorm_residual(3.0 * x, 3.0 * r, w, eps=0.0)[1], n, rtol=1e-12)    # scale invariant
+    for t in range(T):                                                                          # the definition, row by row
+        row = (x + r)[t]
+        assert torch.allclose(n[t], row / math.sqrt(float((row * row).sum()) / d) * w, rtol=1e-12)
+    # the backward formula the kernels use, against autograd
+    xx, ww = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+    yy, nn_ = O.rmsnorm_residual(xx, r, ww, eps=1e-6)
+    dn, dres = torch.randn(T, d, generator=g, dtype=F64), torch.randn(T, d, generator=g, dtype=F64)
+    (nn_ * dn).sum().add((yy * dres).sum()).backward()
+    rstd = torch.rsqrt((yy * yy).mean(-1, keepdim=True) + 1e-6).detach()
+    yd = yy.detach()
+    gw = dn * w
+    dy = rstd * gw - yd * rstd ** 3 / d * (gw * yd).sum(-1, keepdim=True) + dres
+    assert torch.allclose(xx.grad, dy, rtol=1e-10, atol=1e-12)
+    assert torch.allclose(ww.grad, (dn * yd * rstd).sum(0), rtol=1e-10, atol=1e-12)
