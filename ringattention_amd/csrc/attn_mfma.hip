@@ -980,19 +980,20 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     __syncthreads();      // step 0
     for (int t = 0; t < ntiles; t++) {
       const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;
-      // tile t + 2 goes to the buffer that held tile t - 1 (K in step 2t + 1, V in step 2t + 2) and
-      // tile t + 3 is requested
+      // tile t + 2 goes to the buffer that held tile t - 1, K and V both in step 2t + 1: in step 2t + 2 the
+      // producer already requests K and V fragments of block 0 of tile t + 2 from that buffer, so nothing may
+      // still be written to it then.  Tile t + 3 is requested.
       RA_TRACE_MARK();
       RA_WS_STORE_K(prv);
+      RA_WS_STORE_V(prv);
       RA_TRACE_MARK2();
       RA_WS_LOAD_K(t + 3);
+      RA_WS_LOAD_V(t + 3);
       RA_TRACE_MARK2();
       RA_WS_CONSUME(cur, 0, 0, cur, 1);
       RA_TRACE_MARK();
       __syncthreads();
       RA_TRACE_MARK();
-      RA_WS_STORE_V(prv);
-      RA_WS_LOAD_V(t + 3);
       RA_WS_CONSUME(cur, 1, 1, nxt, 0);
       RA_TRACE_MARK();
       __syncthreads();

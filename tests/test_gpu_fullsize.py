@@ -142,3 +142,24 @@ def test_ffn_65k_tokens_chunked_equals_unchunked():
     # tokens are independent: the first chunk alone gives the same rows
     y_c = ff(x[:, :chunk])
     assert _rel(y_c, y_b[:, :chunk]) <= 1e-3
+
+
+def test_forward_and_backward_are_bitwise_reproducible():
+    """Same inputs, same bits: no kernel adds in an order that depends on timing (no atomics), so a difference
+    between two runs can only come from a wavefront reading a tile another one is still writing."""
+    B, S, H, D = 1, 32768, 8, 128
+    g = torch.Generator(device=DEV).manual_seed(5)
+    mk = lambda: (torch.randn(B, S, H, D, device=DEV, generator=g) * D ** -0.25).bfloat16()
+    q, k, v = mk(), mk(), torch.randn(B, S, H, D, device=DEV, generator=g).bfloat16()
+    do = torch.randn(B, S, H, D, device=DEV, generator=g).bfloat16()
+    seg = packed_segment_ids(1, S, 3000, seed=6).to(DEV)
+    bias = torch.randn(1, 1, 1, S, device=DEV, generator=g)
+    for name, b_, s_, n in (("causal", None, None, 1), ("causal ring 4", None, None, 4), ("documents + bias", bias, seg, 2)):
+        print("reproducible", name, flush=True)
+        kw = kwargs(512, 512, 1)
+        first = _attn(q, k, v, b_, s_, n, kw, do)
+        for _ in range(2):
+            again = _attn(q, k, v, b_, s_, n, kw, do)
+            assert torch.equal(torch.nan_to_num(first[0]), torch.nan_to_num(again[0])), name + " out"
+            for nm, a, b2 in zip(("dq", "dk", "dv"), again[1], first[1]):
+                assert torch.equal(a, b2), name + " " + nm
