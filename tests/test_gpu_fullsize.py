@@ -134,6 +134,10 @@ def test_ffn_65k_tokens_chunked_equals_unchunked():
         return y.detach(), xx.grad, [p.grad.clone() for p in ff.parameters()]
 
     y_b, dx_b, dw_b = run(lambda t: ra.blockwise_feedforward(ff, t, chunk))
+    y_2, dx_2, dw_2 = run(lambda t: ra.blockwise_feedforward(ff, t, chunk))
+    assert torch.equal(y_b, y_2) and torch.equal(dx_b, dx_2)          # same inputs, same bits
+    for a, b in zip(dw_b, dw_2):
+        assert torch.equal(a, b)
     y_u, dx_u, dw_u = run(lambda t: ff(t))
     assert not torch.isnan(y_b).any()
     assert _rel(y_b, y_u) <= 1e-3 and _rel(dx_b, dx_u) <= 1e-3

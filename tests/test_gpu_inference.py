@@ -191,3 +191,16 @@ def test_inference_frozen_vectors(dtype):
     assert_close(out, c["out"]["out"], dtype, "out")
     for name, a in zip(("dq", "dk", "dv"), grads):
         assert_close(a, c["out"][name], dtype, name)
+
+
+def test_inference_mfma_path_is_bitwise_reproducible():
+    B, S, H, D, n = 1, 8192, 8, 128, 2
+    g = torch.Generator().manual_seed(21)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=D ** -0.25)
+    mask = (torch.rand(1, 1, S, S, generator=g) < 0.7) & torch.tril(torch.ones(S, S, dtype=torch.bool))
+    mask[..., 0] = True
+    first = _run(q, k, v, do, mask, n)
+    again = _run(q, k, v, do, mask, n)
+    assert torch.equal(first[0], again[0])
+    for a, b in zip(first[1], again[1]):
+        assert torch.equal(a, b)
