@@ -681,8 +681,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   uint4 sk0, sk1, sk2, sk3, sv0, sv1, sv2, sv3;
   int seg_r = 0;
   float bias_r = 0.f;
-  // K half (with the key info) and V half of a tile are staged separately so that the requests and the
-  // LDS writes of a tile spread over two steps
+  // K half (with the key info) and V half of a tile have their own macros (the forward kernel, which shares this
+  // code shape, stores them in different steps); here both are stored in step 2t + 1, see the consumer loop
 #define RA_WS_LOAD_K(T)                                                                                 \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
