@@ -23,8 +23,9 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters'
 # reading for the 1 GiB copy of --workload copy) at the default sizes of each workload
-MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.48e9, "attn_bwd_dkv_ws_kernel": 6.29e9, "attn_bwd_dq_ws_kernel": 4.28e9,
-                    "decode_split_kernel": 68.88e9}
+MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.47e9, "attn_bwd_dkv_ws_kernel": 5.79e9, "attn_bwd_dq_ws_kernel": 4.44e9,
+                    "decode_split_kernel": 68.88e9, "gemm_bf16_w4_kernel<false, false>": 2.55e9,
+                    "rmsnorm_fwd_kernel": 2.15e9}
 
 
 def _kwargs(qc, kc, cbs=1, **extra):
@@ -290,7 +291,8 @@ def bench_ffn(args):
                    "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
         "roofline": {"bound": "mfma", "kernel": "gemm_bf16_w4_kernel<false, false> (a = x w1 of one launch)",
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC["gemm_bf16_w4_kernel<false, false>"] if (T, chunk) == (65536, 2048) else None,
                      "kernel_ms": {"gemm_bf16_w4_kernel<false, false>": round(gemm_ms, 3)}},
         "cpu_baseline": cpu,
     }
@@ -407,7 +409,8 @@ def bench_rmsnorm(args):
         "dtype": "bf16", "pct_hbm_peak": round(100 * value / PEAK_HBM_GBS, 2),
         "config": {"workload": "rmsnorm", "tokens": T, "hidden": d, "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "kernel": "rmsnorm_fwd_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC["rmsnorm_fwd_kernel"] if T == 65536 else None,
                      "kernel_ms": {"rmsnorm_fwd_kernel": round(f_ms, 4)}},
         "cpu_baseline": cpu,
     }
