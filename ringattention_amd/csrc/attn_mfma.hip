@@ -287,6 +287,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   uint4 sr0, sr1, sr2, sr3;
   float r_m = 0.f, r_den = 1.f, r_delta = 0.f;
   int r_seg = 0;
+  // query chunk index and offset inside the chunk of the first row of the next tile to request (tiles are requested
+  // in order and never straddle a chunk: query_chunk_size is a multiple of 128): no division per tile
+  int ld_c = 0, ld_o = 0;
+  if (HAS_SEG) { ld_c = (qt_first * KBM) / mv.qc; ld_o = qt_first * KBM - ld_c * mv.qc; }
 #define RA_WS_LOAD(T)                                                                                   \
   {                                                                                                     \
     const int t_ = min((T), ntq - 1);                                                                   \
@@ -298,10 +302,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
       r_m = a.mx[st_]; r_den = a.den[st_]; r_delta = a.delta[st_];                                      \
       if (HAS_SEG) {                                                                                    \
-        int idx_ = clamp_seg_index(((long long)mv.q_start + row_ / mv.qc) * mv.qc, mv.qc, mv.seg_len, row_ % mv.qc); \
+        int idx_ = clamp_seg_index(((long long)mv.q_start + ld_c) * mv.qc, mv.qc, mv.seg_len, ld_o + tid - 256); \
         r_seg = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
       }                                                                                                 \
     }                                                                                                   \
+    if (HAS_SEG && (T) < ntq - 1) { ld_o += KBM; if (ld_o >= mv.qc) { ld_o -= mv.qc; ld_c++; } }         \
   }
 #define RA_WS_STORE(BUF)                                                                                \
   {                                                                                                     \
@@ -453,6 +458,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     const int2* smm_ptr = nullptr;
     bool sk_uniform = false, sp_cur = false, sp_nxt = false;
     int sk_id = 0;
+    int2 qmm_nxt = make_int2(0, 0);
     if (HAS_SEG && mv.seg_mm) {
       smm_ptr = (const int2*)(mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2);
       const int2 kmm = smm_ptr[min((gk0 + pair * 32) / RA_SEG_TILE, mv.seg_tiles - 1)];
@@ -461,6 +467,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       if (sk_uniform) {
         const int2 qmm = smm_ptr[min(gq_base / RA_SEG_TILE + qt_first, mv.seg_tiles - 1)];
         sp_nxt = qmm.x == sk_id && qmm.y == sk_id;
+        qmm_nxt = smm_ptr[min(gq_base / RA_SEG_TILE + qt_first + min(1, ntq - 1), mv.seg_tiles - 1)];
       }
     }
     int cur = 0;
@@ -470,8 +477,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       if (HAS_SEG) {
         sp_cur = sp_nxt;
         if (sk_uniform) {
-          const int2 qmm = smm_ptr[min(gq_base / RA_SEG_TILE + qt_first + min(t + 1, ntq - 1), mv.seg_tiles - 1)];
-          sp_nxt = qmm.x == sk_id && qmm.y == sk_id;
+          // the range of tile t + 1 was requested one tile ago (a use right after the load would stall the
+          // producer for a global load's latency in every tile); request that of tile t + 2
+          sp_nxt = qmm_nxt.x == sk_id && qmm_nxt.y == sk_id;
+          qmm_nxt = smm_ptr[min(gq_base / RA_SEG_TILE + qt_first + min(t + 2, ntq - 1), mv.seg_tiles - 1)];
         }
       }
       if (HAS_KEEP) {                      // this tile's word and summary; request the next tile's
@@ -668,6 +677,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   if (ntiles == 0) return;     // nothing to add to dq
   const int gk0 = gk0_shard + k_base;
   const float c = kLog2e / sqrtf((float)HD);
+  const float bias_scale = kLog2e / c;
   const float kMask2 = mv.mask_min;
 
   // ---- staging of the K / V tiles through registers, by the consumer waves (which have registers and
@@ -681,6 +691,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   uint4 sk0, sk1, sk2, sk3, sv0, sv1, sv2, sv3;
   int seg_r = 0;
   float bias_r = 0.f;
+  // key chunk index and offset inside the chunk of the first key of the next tile to request (tiles are requested
+  // in order and never straddle a chunk: key_chunk_size is a multiple of 64): no division per tile
+  int ld_c = 0, ld_o = 0;
+  if (HAS_SEG) { ld_c = k_base / mv.kc; ld_o = k_base - ld_c * mv.kc; }
   // K half (with the key info) and V half of a tile have their own macros (the forward kernel, which shares this
   // code shape, stores them in different steps); here both are stored in step 2t + 1, see the consumer loop
 #define RA_WS_LOAD_K(T)                                                                                 \
@@ -692,15 +706,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
-        int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+        int idx_ = clamp_seg_index(((long long)mv.k_start + ld_c) * mv.kc, mv.kc, mv.seg_len, ld_o + stid); \
         seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
       }                                                                                                 \
-      if (HAS_BIAS) {                                                                                   \
-        float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
-        if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
-        bias_r = bv_ * kLog2e / c;   /* the S accumulators start from it */                             \
-      }                                                                                                 \
+      /* only the request: using the value here would make this wavefront wait for it right away */     \
+      if (HAS_BIAS) bias_r = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
     }                                                                                                   \
+    if (HAS_SEG && (T) < ntiles - 1) { ld_o += FBN; if (ld_o >= mv.kc) { ld_o -= mv.kc; ld_c++; } }      \
   }
 #define RA_WS_LOAD_V(T)                                                                                 \
   {                                                                                                     \
@@ -716,7 +728,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     *(uint4*)(dk_ + 32 * TROW) = sk2; *(uint4*)(dk_ + 48 * TROW) = sk3;                                 \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       if (HAS_SEG) seg_ks[BUF][stid] = seg_r;                                                           \
-      if (HAS_BIAS) bias_ks[BUF][stid] = bias_r;                                                        \
+      /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
+      if (HAS_BIAS) bias_ks[BUF][stid] = (mv.any_mask ? fminf(bias_r, 0.f) : bias_r) * bias_scale;      \
     }                                                                                                   \
   }
 #define RA_WS_STORE_V(BUF)                                                                              \
@@ -1100,6 +1113,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   }
   const int gk0 = gk0_shard + k_base;
   const float c = kLog2e / sqrtf((float)HD);
+  const float bias_scale = kLog2e / c;
   const float kMask2 = mv.mask_min;
 
   // ---- staging of the K / V tiles through registers, by the consumer waves (which have registers and
@@ -1113,6 +1127,10 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   uint4 sk0, sk1, sk2, sk3, sv0, sv1, sv2, sv3;
   int seg_r = 0;
   float bias_r = 0.f;
+  // key chunk index and offset inside the chunk of the first key of the next tile to request (tiles are requested
+  // in order and never straddle a chunk: key_chunk_size is a multiple of 64): no division per tile
+  int ld_c = 0, ld_o = 0;
+  if (HAS_SEG) { ld_c = k_base / mv.kc; ld_o = k_base - ld_c * mv.kc; }
   // K half (with the key info) and V half of a tile are staged separately so that the requests and the
   // LDS writes of a tile spread over two steps
 #define RA_WS_LOAD_K(T)                                                                                 \
@@ -1124,15 +1142,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
-        int idx_ = clamp_seg_index(((long long)mv.k_start + kj_ / mv.kc) * mv.kc, mv.kc, mv.seg_len, kj_ % mv.kc); \
+        int idx_ = clamp_seg_index(((long long)mv.k_start + ld_c) * mv.kc, mv.kc, mv.seg_len, ld_o + stid); \
         seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
       }                                                                                                 \
-      if (HAS_BIAS) {                                                                                   \
-        float bv_ = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
-        if (mv.any_mask) bv_ = fminf(bv_, 0.f);                                                         \
-        bias_r = bv_ * kLog2e / c;   /* the S accumulators start from it */                             \
-      }                                                                                                 \
+      /* only the request: using the value here would make this wavefront wait for it right away */     \
+      if (HAS_BIAS) bias_r = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
     }                                                                                                   \
+    if (HAS_SEG && (T) < ntiles - 1) { ld_o += FBN; if (ld_o >= mv.kc) { ld_o -= mv.kc; ld_c++; } }      \
   }
 #define RA_WS_LOAD_V(T)                                                                                 \
   {                                                                                                     \
@@ -1148,7 +1164,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     *(uint4*)(dk_ + 32 * TROW) = sk2; *(uint4*)(dk_ + 48 * TROW) = sk3;                                 \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       if (HAS_SEG) seg_ks[BUF][stid] = seg_r;                                                           \
-      if (HAS_BIAS) bias_ks[BUF][stid] = bias_r;                                                        \
+      /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
+      if (HAS_BIAS) bias_ks[BUF][stid] = (mv.any_mask ? fminf(bias_r, 0.f) : bias_r) * bias_scale;      \
     }                                                                                                   \
   }
 #define RA_WS_STORE_V(BUF)                                                                              \
