@@ -115,3 +115,39 @@ def test_rmsnorm_rejects_unsupported_rows():
     x = torch.zeros(2, 16384, dtype=torch.bfloat16, device=DEV)        # longer than the kernels' 8192
     with pytest.raises(NotImplementedError):
         ra.rmsnorm_residual(x, None, torch.ones(16384, dtype=torch.bfloat16, device=DEV))
+
+
+def test_decode_step_replays_from_a_hip_graph():
+    """The decode step (rotate + append, then attend) captured once in a HIP graph and replayed for several
+    positions: cache_idx is read from device memory by both kernels, so one graph serves every step.  Each replay
+    is checked against the same step run eagerly on a copy of the caches."""
+    B, L, H, D, kc = 2, 1024, 4, 128, 128
+    g = torch.Generator(device=DEV).manual_seed(11)
+    rnd = lambda *s: torch.randn(*s, device=DEV, generator=g).bfloat16()
+    k_cache, v_cache = rnd(B, L, H, D), rnd(B, L, H, D)
+    q, kn, vn = rnd(B, 1, H, D), rnd(B, 1, H, D), rnd(B, 1, H, D)
+    qr, out = torch.empty_like(q), torch.empty_like(q)
+    ci = torch.zeros(1, dtype=torch.int32, device=DEV)
+    kw = kwargs(1, kc, 1)
+
+    def step(kc_, vc_, qr_, out_):
+        ra.rope_kv_append(q, kn, vn, kc_, vc_, ci, q_out=qr_)
+        ra.decode_attention(qr_, kc_, vc_, None, None, ci, kw, out=out_)
+
+    ci.fill_(500)
+    step(k_cache.clone(), v_cache.clone(), torch.empty_like(q), torch.empty_like(q))     # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(k_cache, v_cache, qr, out)
+    for pos in (500, 501, 777, 1023, 130):
+        print("graph replay at", pos, flush=True)
+        ci.fill_(pos)
+        q.copy_(rnd(B, 1, H, D)); kn.copy_(rnd(B, 1, H, D)); vn.copy_(rnd(B, 1, H, D))
+        k_ref, v_ref = k_cache.clone(), v_cache.clone()
+        qr_ref, out_ref = torch.empty_like(q), torch.empty_like(q)
+        step(k_ref, v_ref, qr_ref, out_ref)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(torch.nan_to_num(out), torch.nan_to_num(out_ref))
+        assert torch.equal(qr, qr_ref) and torch.equal(k_cache, k_ref) and torch.equal(v_cache, v_ref)
