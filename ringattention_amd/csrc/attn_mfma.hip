@@ -681,73 +681,75 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   const float kMask2 = mv.mask_min;
 
   // ---- staging of the K / V tiles through registers, by the consumer waves (which have registers and
-  // issue slots to spare): tile t + 2 is stored in step 2t + 1, two steps after it was requested
+  // issue slots to spare), in two register sets A and B: tile T lives in set T & 1 from its request until it is
+  // stored to LDS two tiles (four steps) later
   const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
   const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
   const int64_t sg_off = (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
   const uint16_t* sgk = a.k + sg_off;
   const uint16_t* sgv = a.v + sg_off;
   const int64_t row16 = 16 * a.kv_ss;
-  uint4 sk0, sk1, sk2, sk3, sv0, sv1, sv2, sv3;
-  int seg_r = 0;
-  float bias_r = 0.f;
+  uint4 Ak0, Ak1, Ak2, Ak3, Av0, Av1, Av2, Av3, Bk0, Bk1, Bk2, Bk3, Bv0, Bv1, Bv2, Bv3;
+  int Aseg = 0, Bseg = 0;
+  float Abias = 0.f, Bbias = 0.f;
   // key chunk index and offset inside the chunk of the first key of the next tile to request (tiles are requested
   // in order and never straddle a chunk: key_chunk_size is a multiple of 64): no division per tile
   int ld_c = 0, ld_o = 0;
   if (HAS_SEG) { ld_c = k_base / mv.kc; ld_o = k_base - ld_c * mv.kc; }
   // K half (with the key info) and V half of a tile have their own macros (the forward kernel, which shares this
   // code shape, stores them in different steps); here both are stored in step 2t + 1, see the consumer loop
-#define RA_WS_LOAD_K(T)                                                                                 \
+#define RA_WS_LOAD_K(S, T)                                                                               \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
     const uint16_t* pk_ = sgk + (int64_t)t_ * FBN * a.kv_ss;                                            \
-    sk0 = *(const uint4*)(pk_); sk1 = *(const uint4*)(pk_ + row16);                                     \
-    sk2 = *(const uint4*)(pk_ + 2 * row16); sk3 = *(const uint4*)(pk_ + 3 * row16);                     \
+    S##k0 = *(const uint4*)(pk_); S##k1 = *(const uint4*)(pk_ + row16);                                 \
+    S##k2 = *(const uint4*)(pk_ + 2 * row16); S##k3 = *(const uint4*)(pk_ + 3 * row16);                 \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
         int idx_ = clamp_seg_index(((long long)mv.k_start + ld_c) * mv.kc, mv.kc, mv.seg_len, ld_o + stid); \
-        seg_r = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                  \
+        S##seg = mv.seg[(int64_t)b * mv.seg_sb + idx_];                                                 \
       }                                                                                                 \
       /* only the request: using the value here would make this wavefront wait for it right away */     \
-      if (HAS_BIAS) bias_r = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
+      if (HAS_BIAS) S##bias = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(gk0_shard + kj_) * mv.bias_sk]; \
     }                                                                                                   \
     if (HAS_SEG && (T) < ntiles - 1) { ld_o += FBN; if (ld_o >= mv.kc) { ld_o -= mv.kc; ld_c++; } }      \
   }
-#define RA_WS_LOAD_V(T)                                                                                 \
+#define RA_WS_LOAD_V(S, T)                                                                               \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
     const uint16_t* pv_ = sgv + (int64_t)t_ * FBN * a.kv_ss;                                            \
-    sv0 = *(const uint4*)(pv_); sv1 = *(const uint4*)(pv_ + row16);                                     \
-    sv2 = *(const uint4*)(pv_ + 2 * row16); sv3 = *(const uint4*)(pv_ + 3 * row16);                     \
+    S##v0 = *(const uint4*)(pv_); S##v1 = *(const uint4*)(pv_ + row16);                                 \
+    S##v2 = *(const uint4*)(pv_ + 2 * row16); S##v3 = *(const uint4*)(pv_ + 3 * row16);                 \
   }
-#define RA_WS_STORE_K(BUF)                                                                              \
+#define RA_WS_STORE_K(S, BUF)                                                                            \
   {                                                                                                     \
     uint16_t* dk_ = Ks + (BUF) * WS_TILE + s_off;                                                       \
-    *(uint4*)(dk_) = sk0; *(uint4*)(dk_ + 16 * TROW) = sk1;                                             \
-    *(uint4*)(dk_ + 32 * TROW) = sk2; *(uint4*)(dk_ + 48 * TROW) = sk3;                                 \
+    *(uint4*)(dk_) = S##k0; *(uint4*)(dk_ + 16 * TROW) = S##k1;                                         \
+    *(uint4*)(dk_ + 32 * TROW) = S##k2; *(uint4*)(dk_ + 48 * TROW) = S##k3;                             \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
-      if (HAS_SEG) seg_ks[BUF][stid] = seg_r;                                                           \
+      if (HAS_SEG) seg_ks[BUF][stid] = S##seg;                                                          \
       /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
-      if (HAS_BIAS) bias_ks[BUF][stid] = (mv.any_mask ? fminf(bias_r, 0.f) : bias_r) * bias_scale;      \
+      if (HAS_BIAS) bias_ks[BUF][stid] = (mv.any_mask ? fminf(S##bias, 0.f) : S##bias) * bias_scale;    \
     }                                                                                                   \
   }
-#define RA_WS_STORE_V(BUF)                                                                              \
+#define RA_WS_STORE_V(S, BUF)                                                                            \
   {                                                                                                     \
     uint16_t* dv_ = Vs + (BUF) * WS_TILE + s_off;                                                       \
-    *(uint4*)(dv_) = sv0; *(uint4*)(dv_ + 16 * TROW) = sv1;                                             \
-    *(uint4*)(dv_ + 32 * TROW) = sv2; *(uint4*)(dv_ + 48 * TROW) = sv3;                                 \
+    *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + 16 * TROW) = S##v1;                                         \
+    *(uint4*)(dv_ + 32 * TROW) = S##v2; *(uint4*)(dv_ + 48 * TROW) = S##v3;                             \
   }
 #ifdef RA_TRACE
   const bool trace_on = blockIdx.x == 0;
   int trace_n = 0;
 #endif
   if (role == 1) {
-    RA_WS_LOAD_K(0); RA_WS_LOAD_V(0);
-    RA_WS_STORE_K(0); RA_WS_STORE_V(0);
-    RA_WS_LOAD_K(1); RA_WS_LOAD_V(1);
-    RA_WS_STORE_K(1); RA_WS_STORE_V(1);
-    RA_WS_LOAD_K(2); RA_WS_LOAD_V(2);
+    RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
+    RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
+    RA_WS_STORE_K(A, 0); RA_WS_STORE_V(A, 0);
+    RA_WS_LOAD_K(A, 2); RA_WS_LOAD_V(A, 2);
+    RA_WS_STORE_K(B, 1); RA_WS_STORE_V(B, 1);
+    RA_WS_LOAD_K(B, 3); RA_WS_LOAD_V(B, 3);
   }
   __syncthreads();
 
@@ -991,27 +993,35 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     int cur = 0;
     RA_WS_CREAD(0, fa, 0, 0);
     __syncthreads();      // step 0
-    for (int t = 0; t < ntiles; t++) {
-      const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;
-      // tile t + 2 goes to the buffer that held tile t - 1, K and V both in step 2t + 1: in step 2t + 2 the
-      // producer already requests K and V fragments of block 0 of tile t + 2 from that buffer, so nothing may
-      // still be written to it then.  Tile t + 3 is requested.
-      RA_TRACE_MARK();
-      RA_WS_STORE_K(prv);
-      RA_WS_STORE_V(prv);
-      RA_TRACE_MARK2();
-      RA_WS_LOAD_K(t + 3);
-      RA_WS_LOAD_V(t + 3);
-      RA_TRACE_MARK2();
-      RA_WS_CONSUME(cur, 0, 0, cur, 1);
-      RA_TRACE_MARK();
-      __syncthreads();
-      RA_TRACE_MARK();
-      RA_WS_CONSUME(cur, 1, 1, nxt, 0);
-      RA_TRACE_MARK();
-      __syncthreads();
-      cur = nxt;
+    // tile T + 2 (in register set T & 1) goes to the buffer that held tile T - 1, K and V both in step 2T + 1: in
+    // step 2T + 2 the producer already requests K and V fragments of block 0 of tile T + 2 from that buffer, so
+    // nothing may still be written to it then.  Tile T + 4 is requested into the same set.
+#define RA_WS_CTILE(S, T)                                                                               \
+  {                                                                                                     \
+    const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;                               \
+    RA_TRACE_MARK();                                                                                    \
+    RA_WS_STORE_K(S, prv);                                                                              \
+    RA_WS_STORE_V(S, prv);                                                                              \
+    RA_TRACE_MARK2();                                                                                   \
+    RA_WS_LOAD_K(S, (T) + 4);                                                                           \
+    RA_WS_LOAD_V(S, (T) + 4);                                                                           \
+    RA_TRACE_MARK2();                                                                                   \
+    RA_WS_CONSUME(cur, 0, 0, cur, 1);                                                                   \
+    RA_TRACE_MARK();                                                                                    \
+    __syncthreads();                                                                                    \
+    RA_TRACE_MARK();                                                                                    \
+    RA_WS_CONSUME(cur, 1, 1, nxt, 0);                                                                   \
+    RA_TRACE_MARK();                                                                                    \
+    __syncthreads();                                                                                    \
+    cur = nxt;                                                                                          \
+  }
+    int t = 0;
+    for (; t + 2 <= ntiles; t += 2) {
+      RA_WS_CTILE(A, t);
+      RA_WS_CTILE(B, t + 1);
     }
+    if (t < ntiles) RA_WS_CTILE(A, t);
+#undef RA_WS_CTILE
 #undef RA_WS_CREAD
 #undef RA_WS_CMFMA
 #undef RA_WS_CONSUME
