@@ -67,17 +67,22 @@ typedef struct ra_mask {
                                      skip_masked_tiles it lets kernels skip key (query) tiles whose id range
                                      cannot meet the ids of the query (key) rows at hand */
   int32_t seg_tiles;
-  const uint8_t* keep;        /* nullable; the boolean attn_mask of ring_attention_inference
-                                 (ringattention_inference.py:19-22): nonzero = attend, zero = the logit becomes
-                                 mask_min.  Indexed by the LOCAL query row of the call and the GLOBAL key position;
-                                 only the generic kernels take it */
+  const uint8_t* keep;        /* nullable; a boolean mask, nonzero = attend.  keep_mode says what a zero does:
+                                 RA_KEEP_WHERE, the attn_mask of ring_attention_inference
+                                 (ringattention_inference.py:19-22): the logit becomes mask_min;
+                                 RA_KEEP_DROPOUT, the attention dropout mask (ringattention_jax.py:311-321, zero =
+                                 dropped): mask_min is ADDED to the logit and its bias, so the logit becomes mask_min,
+                                 or -inf where segment ids or the causal mask had already set it to mask_min.
+                                 Indexed by the LOCAL query row of the call and by the GLOBAL key position minus
+                                 keep_k0; only the generic kernels take this byte form */
   int64_t keep_stride_b;      /* element (byte) strides; 0 broadcasts that axis */
   int64_t keep_stride_h;
   int64_t keep_stride_q;
   int64_t keep_stride_k;
   /* Packed forms of the same mask from ra_keep_pack, which let the MFMA kernels take it (all three null:
      generic kernels only).  They cover the GLOBAL mask (keep_q_total x keep_k_total, both multiples of 64);
-     keep_q0 is the global row of the call's local query row 0 (a multiple of 64). */
+     keep_q0 is the global row of the call's local query row 0 (a multiple of 64), keep_k0 the global key position
+     of the mask's column 0 (a multiple of 64; 0 when the mask spans the global key axis). */
   const uint64_t* keep_bits_k;   /* [b][h][k_total/64][q_total]: bit i = keep[q][64 kt + i] */
   const uint64_t* keep_bits_q;   /* [b][h][q_total/64][k_total]: bit i = keep[64 qt + i][k] */
   const uint8_t* keep_summary;   /* [b][h][q_total/64][k_total/64]: 0 none kept, 1 mixed, 2 all kept */
@@ -86,7 +91,11 @@ typedef struct ra_mask {
   int64_t keep_sum_stride_b;     /* of keep_summary, in bytes; 0 broadcasts */
   int64_t keep_sum_stride_h;
   int32_t keep_q_total, keep_k_total, keep_q0;
+  int32_t keep_k0;
+  int32_t keep_mode;             /* RA_KEEP_WHERE | RA_KEEP_DROPOUT */
 } ra_mask;
+
+enum { RA_KEEP_WHERE = 0, RA_KEEP_DROPOUT = 1 };
 
 /* _blockwise_attention_fwd (ringattention_jax.py:99-179): one ring step on one device.
  * Updates the carry (numerator, denominator, max_score) in place. */
@@ -135,6 +144,18 @@ int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int
 int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_t stride_q, int64_t stride_k,
                  int32_t Bm, int32_t Hm, int32_t Q, int32_t K, uint64_t* bits_k, uint64_t* bits_q,
                  uint8_t* summary, ra_stream_t stream);
+
+/* The attention dropout mask of ringattention_jax.py:119-121 / :206-208 (jax.random.bernoulli(rng, attn_pdrop,
+ * (batch, heads, q_len, kv_len)), true = dropped), written as the boolean KEEP mask ra_mask.keep takes with
+ * RA_KEEP_DROPOUT: keep (B, H, Q, K) dense bytes, 1 = attend, 0 = dropped.  The bits do not come from the
+ * jax.random stream (threefry, not restated) but from Philox4x32-10 (Salmon et al., SC'11), one block per four
+ * consecutive key positions:
+ *   e = ((b * H + h) * Q + q) * K + k          (position in the dense mask; K is a multiple of 4)
+ *   block = philox4x32_10(counter = (lo32(e / 4), hi32(e / 4), 0, 0), key = (lo32(seed), hi32(seed)))
+ *   dropped(e) = block[e % 4] < floor(attn_pdrop * 2^32)
+ * so the mask is a pure function of (seed, attn_pdrop, shape); forward and backward pass take the same array. */
+int ra_dropout_keep(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K, uint8_t* keep,
+                    ra_stream_t stream);
 
 /* Carry initialisation (ringattention_jax.py:22-23,:49): numerator = 0, denominator = 0, max = -inf. */
 int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s,

@@ -31,8 +31,15 @@ vectors, and JAX/flax are not importable where this was written):
   rotated dot product; RMSNorm against its definition in float64, unit RMS of the result, scale invariance and
   torch autograd / finite differences for the backward formula.
 
+* attention dropout (ringattention_jax.py:119-123, :206-208, :311-321): the arithmetic given a mask
+  (``finfo.min`` ADDED to the tile bias, slices taken with ``dynamic_slice`` at global offsets of a mask
+  of local shape) is restated and checked against ``dense_attention`` with the same mask, against the
+  exact-zero weight of dropped keys and against a hand-enumerated row whose every allowed key is dropped.
+  The mask BITS are not the reference's: ``jax.random`` (threefry) is not restated; ``dropout_mask``
+  draws from Philox4x32-10, pinned by the known-answer vectors of the Random123 distribution.
+
 Parity unpinned (would need the reference's own runtime): the dropout mask
-bits (``jax.random`` stream) - dropout is refused - and XLA-CPU's exact
+bits of the ``jax.random`` stream (replaced by the documented Philox stream above) and XLA-CPU's exact
 summation order / its bf16 rounding of intermediate einsum results, both far
 below the stated tolerances.
 
@@ -40,6 +47,7 @@ Layout: q/k/v/out/grads ``(B, S, H, D)``; softmax statistics ``(B, H, S)``.
 """
 import math
 
+import numpy as np
 import torch
 
 _FINFO_MIN = {
@@ -68,10 +76,42 @@ def _dynamic_slice_start(start, size, dim):
     return max(0, min(start, dim - size))
 
 
+def philox4x32_10(counter, key):
+    """Philox4x32-10 of Salmon, Moraes, Dror and Shaw (SC'11), vectorised: counter (..., 4) and key (..., 2)
+    uint32 arrays -> (..., 4) uint32.  Ten rounds; the key is bumped by the Weyl constants between rounds."""
+    c = [np.asarray(counter[..., i], dtype=np.uint64) for i in range(4)]
+    k0 = np.asarray(key[..., 0], dtype=np.uint64)
+    k1 = np.asarray(key[..., 1], dtype=np.uint64)
+    m32 = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0 = np.uint64(0xD2511F53) * c[0]
+        p1 = np.uint64(0xCD9E8D57) * c[2]
+        c = [(p1 >> np.uint64(32)) ^ c[1] ^ k0, p1 & m32, (p0 >> np.uint64(32)) ^ c[3] ^ k1, p0 & m32]
+        k0 = (k0 + np.uint64(0x9E3779B9)) & m32
+        k1 = (k1 + np.uint64(0xBB67AE85)) & m32
+    return np.stack(c, axis=-1).astype(np.uint32)
+
+
+def dropout_mask(seed, attn_pdrop, shape):
+    """The boolean mask of ringattention_jax.py:120-121 / :207-208 (True = dropped, probability attn_pdrop)
+    of shape (batch, heads, q_len, kv_len), from the documented Philox stream instead of jax.random:
+    position e of the dense mask takes word e % 4 of block e // 4, keyed by the 64-bit seed; dropped iff
+    the word is below floor(float32(attn_pdrop) * 2^32)."""
+    n = int(np.prod(shape))
+    assert shape[-1] % 4 == 0
+    blk = np.arange(n // 4, dtype=np.uint64)
+    counter = np.stack([blk & np.uint64(0xFFFFFFFF), blk >> np.uint64(32), np.zeros_like(blk), np.zeros_like(blk)],
+                       axis=-1)
+    key = np.array([seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF], dtype=np.uint64)
+    words = philox4x32_10(counter, np.broadcast_to(key, (n // 4, 2))).reshape(n)
+    threshold = int(float(np.float32(attn_pdrop)) * 4294967296.0)
+    return torch.from_numpy((words.astype(np.uint64) < np.uint64(threshold)).reshape(shape))
+
+
 def chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
                          causal_block_size, dtype, query_chunk_idx, key_chunk_idx,
-                         work_dtype=torch.float32):
-    """ringattention_jax.py:272-322 without the dropout branch (:311-321).
+                         work_dtype=torch.float32, attn_dropout=None):
+    """ringattention_jax.py:272-322; ``attn_dropout`` is the boolean mask of :120-121 (True = dropped) or None.
 
     Returns the additive tile, broadcastable to (B, H, qc, kc), holding values
     representable in ``dtype`` but stored in ``work_dtype``.
@@ -98,15 +138,26 @@ def chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
         k_idx = (torch.arange(key_chunk_size).reshape(1, -1) + key_offset) // causal_block_size
         causal = (q_idx < k_idx).to(work_dtype) * fmin
         chunk_bias = torch.minimum(chunk_bias, causal.reshape(1, 1, *causal.shape))
+    if attn_dropout is not None:                                           # :311-321
+        qs = min(attn_dropout.shape[-2], query_chunk_size)
+        ks = min(attn_dropout.shape[-1], key_chunk_size)
+        q0 = _dynamic_slice_start(query_offset, qs, attn_dropout.shape[-2])
+        k0 = _dynamic_slice_start(key_offset, ks, attn_dropout.shape[-1])
+        chunk_bias = chunk_bias + attn_dropout[:, :, q0:q0 + qs, k0:k0 + ks].to(work_dtype) * fmin
+        # twice finfo.min overflows to -inf in ``dtype``; once plus a finite bias rounds back to finfo.min
+        chunk_bias = chunk_bias.to(dtype).to(work_dtype)
     # :322  .astype(dtype): round to the kwargs dtype, then carry on in work_dtype
     if dtype in (torch.bfloat16, torch.float16):
         chunk_bias = chunk_bias.to(dtype).to(work_dtype)
     return chunk_bias
 
 
-def _check_no_dropout(deterministic, attn_pdrop):
-    if (not deterministic) and attn_pdrop > 0.0:
-        raise NotImplementedError("attention dropout draws from the jax.random stream; not restated")
+def _attn_dropout(deterministic, attn_pdrop, dropout_rng, shape):
+    """:119-123 / :206-210: one mask of the LOCAL shape (batch, heads, q_len, kv_len) per call, the same in
+    the forward and the backward pass; ``dropout_rng`` is the integer seed of ``dropout_mask``."""
+    if deterministic or not attn_pdrop > 0.0:
+        return None
+    return dropout_mask(int(dropout_rng), attn_pdrop, shape)
 
 
 def blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_start, bias, segment_ids,
@@ -114,12 +165,12 @@ def blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_start
                             dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
                             precision=None, prevent_cse=True, cache_idx=None):
     """ringattention_jax.py:99-179.  q/k/v already in the working dtype; returns the new carry."""
-    _check_no_dropout(deterministic, attn_pdrop)
     batch, q_len, num_heads, dim = q.shape
     kv_len = k.shape[1]
     num_q = q_len // query_chunk_size
     num_kv = kv_len // key_chunk_size
     wd = q.dtype
+    attn_dropout = _attn_dropout(deterministic, attn_pdrop, dropout_rng, (batch, num_heads, q_len, kv_len))
     numerator, denominator, max_score = (x.clone() for x in carry)
     scale = math.sqrt(dim)                                                  # :118
     for qi in range(num_q):                                                 # :171
@@ -138,7 +189,8 @@ def blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_start
             w = torch.einsum('bqhd,bkhd->bhqk', q_chunk, k_chunk) / scale   # :134
             w = w + chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
                                          causal_block_size, dtype, q_chunk_idx_start + qi,
-                                         k_chunk_idx_start + ki, work_dtype=wd)  # :135-136
+                                         k_chunk_idx_start + ki, work_dtype=wd,
+                                         attn_dropout=attn_dropout)         # :135-136
             new_max = torch.maximum(max_c, w.max(dim=-1).values)            # :138
             e = torch.exp(w - new_max[..., None])                           # :140
             ev = torch.einsum('bhqk,bkhd->bqhd', e, v_chunk)                # :141
@@ -157,12 +209,12 @@ def blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_st
                             dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
                             precision=None, prevent_cse=True, cache_idx=None):
     """ringattention_jax.py:181-270.  Adds this block's gradients into the incoming dq/dk/dv."""
-    _check_no_dropout(deterministic, attn_pdrop)
     batch, q_len, num_heads, dim = q.shape
     kv_len = k.shape[1]
     num_q = q_len // query_chunk_size
     num_kv = kv_len // key_chunk_size
     wd = q.dtype
+    attn_dropout = _attn_dropout(deterministic, attn_pdrop, dropout_rng, (batch, num_heads, q_len, kv_len))
     dq, dk, dv, output, denominator, max_score = carry
     dq, dk, dv = dq.clone(), dk.clone(), dv.clone()
     g = g.to(wd)
@@ -183,7 +235,8 @@ def blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_st
             w = torch.einsum('bqhd,bkhd->bhqk', q_chunk, k_chunk) / scale   # :223
             w = w + chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,
                                          causal_block_size, dtype, q_chunk_idx_start + qi,
-                                         k_chunk_idx_start + ki, work_dtype=wd)  # :224-225
+                                         k_chunk_idx_start + ki, work_dtype=wd,
+                                         attn_dropout=attn_dropout)         # :224-225
             p = torch.exp(w - max_c[..., None]) / den_c[..., None]          # :226
             ds = torch.einsum('bqhd,bkhd->bhqk', g_chunk, v_chunk)          # :228
             dl = (ds - dl_part) * p                                         # :229
@@ -333,6 +386,17 @@ def dense_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, block
         masked = masked | ((g_q // cbs)[:, None] < (g_k // cbs)[None, :])[None, None]
     logits = logits + add
     logits = torch.where(masked, torch.full((), fmin, dtype=wd), logits)
+    if (not blockwise_kwargs.get("deterministic", True)) and blockwise_kwargs.get("attn_pdrop", 0.0) > 0.0:
+        # the mask has the LOCAL shape and is sliced at GLOBAL chunk offsets, clamped (:312-320)
+        kv_len = kv_total // n
+        drop = dropout_mask(int(blockwise_kwargs["dropout_rng"]), blockwise_kwargs["attn_pdrop"],
+                            (batch, num_heads, q_len, kv_len))
+        row = torch.clamp(q_chunk * qc, max=q_len - qc) + loc_q % qc
+        col = torch.clamp(k_chunk * kc, max=kv_len - kc) + g_k % kc
+        dropped = drop[:, :, row][:, :, :, col]
+        # finfo.min is added: once -> finfo.min (logit and bias are absorbed), twice -> -inf
+        logits = torch.where(dropped, torch.where(masked, torch.full((), -math.inf, dtype=wd),
+                                                  torch.full((), fmin, dtype=wd)), logits)
     if cbs is not None:
         cq, ck = max(cbs, qc), max(cbs, kc)
         r = q_chunk // (cq // qc)

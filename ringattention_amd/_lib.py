@@ -14,6 +14,7 @@ RA_F32, RA_BF16 = 0, 1
 RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
 RA_BWD_ONLY_DQ, RA_BWD_ONLY_DKV = 0x10, 0x20
 RA_SEG_TILE = 64
+RA_KEEP_WHERE, RA_KEEP_DROPOUT = 0, 1
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
@@ -30,6 +31,7 @@ class RaMask(C.Structure):
         ("keep_bits_k", vp), ("keep_bits_q", vp), ("keep_summary", vp),
         ("keep_pack_stride_b", i64), ("keep_pack_stride_h", i64), ("keep_sum_stride_b", i64),
         ("keep_sum_stride_h", i64), ("keep_q_total", i32), ("keep_k_total", i32), ("keep_q0", i32),
+        ("keep_k0", i32), ("keep_mode", i32),
     ]
 
 
@@ -98,6 +100,7 @@ class RaRmsnormParams(C.Structure):
 SYMBOLS = {
     "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
     "ra_keep_pack": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]),
+    "ra_dropout_keep": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp]),
     "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),

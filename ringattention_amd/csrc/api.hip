@@ -28,6 +28,7 @@ int bwd_delta(const void*, const void*, int, int64_t, int64_t, float*, int64_t, 
               hipStream_t);
 int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
 int keep_pack(const uint8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, uint64_t*, uint64_t*, uint8_t*, hipStream_t);
+int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hipStream_t s);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
@@ -64,8 +65,16 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
                "%s: the packed keep mask needs keep, keep_bits_k, keep_bits_q and keep_summary together", who);
     RA_REQUIRE(m.keep_q_total > 0 && m.keep_k_total > 0 && m.keep_q_total % 64 == 0 && m.keep_k_total % 64 == 0 &&
                    m.keep_q0 >= 0 && m.keep_q0 % 64 == 0 && m.keep_q0 + Sq <= m.keep_q_total &&
-                   (long long)m.k_chunk_idx_start * m.key_chunk_size + Skv <= m.keep_k_total,
+                   m.keep_k0 >= 0 && m.keep_k0 % 64 == 0 &&
+                   (long long)m.k_chunk_idx_start * m.key_chunk_size >= m.keep_k0 &&
+                   (long long)m.k_chunk_idx_start * m.key_chunk_size - m.keep_k0 + Skv <= m.keep_k_total,
                RA_ERR_INVALID, "%s: packed keep mask does not cover the rows / keys of the call", who);
+  }
+  if (m.keep) {
+    RA_REQUIRE(m.keep_mode == RA_KEEP_WHERE || m.keep_mode == RA_KEEP_DROPOUT, RA_ERR_INVALID,
+               "%s: keep_mode must be RA_KEEP_WHERE or RA_KEEP_DROPOUT", who);
+    RA_REQUIRE(m.keep_k0 >= 0 && (long long)m.k_chunk_idx_start * m.key_chunk_size >= m.keep_k0, RA_ERR_INVALID,
+               "%s: keep_k0 lies after the first key of the call", who);
   }
   RA_REQUIRE((long long)m.q_chunk_idx_start * m.query_chunk_size + Sq < (1LL << 31) - 4096 &&
                  (long long)m.k_chunk_idx_start * m.key_chunk_size + Skv < (1LL << 31) - 4096,
@@ -152,6 +161,19 @@ int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_
              "keep_pack: Q and K must be positive multiples of 64 (got %d, %d)", Q, K);
   return keep_pack(keep, stride_b, stride_h, stride_q, stride_k, Bm, Hm, Q, K, bits_k, bits_q, summary,
                    (hipStream_t)stream);
+}
+
+int ra_dropout_keep(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K, uint8_t* keep,
+                    ra_stream_t stream) {
+  RA_REQUIRE(keep, RA_ERR_INVALID, "dropout_keep: null pointer");
+  RA_REQUIRE(((uintptr_t)keep % 16) == 0, RA_ERR_UNSUPPORTED, "dropout_keep: keep must be 16-byte aligned");
+  RA_REQUIRE(B > 0 && H > 0 && Q > 0 && K > 0, RA_ERR_INVALID, "dropout_keep: empty shape");
+  RA_REQUIRE(K % 4 == 0, RA_ERR_UNSUPPORTED, "dropout_keep: K must be a multiple of 4 (got %d)", K);
+  RA_REQUIRE(attn_pdrop > 0.f && attn_pdrop < 1.f, RA_ERR_INVALID, "dropout_keep: attn_pdrop must lie in (0, 1)");
+  const int64_t n = (int64_t)B * H * Q * K;
+  RA_REQUIRE(n / 16 / 256 < (1LL << 31), RA_ERR_UNSUPPORTED, "dropout_keep: mask too large");
+  const uint32_t threshold = (uint32_t)((double)attn_pdrop * 4294967296.0);     // floor; < 2^32 since p < 1
+  return dropout_keep(seed, threshold, n, keep, (hipStream_t)stream);
 }
 
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {

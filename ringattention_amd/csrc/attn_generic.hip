@@ -66,7 +66,12 @@ __device__ __forceinline__ float logit(const MaskView& mv, const RowInfo& r, flo
     if (mv.any_mask) add = fminf(add, 0.f);                       // minimum(), :299,:309
   }
   bool masked = (mv.cbs > 0 && r.gq_blk < gk / mv.cbs) || (mv.seg && r.seg != seg_k);
-  if (mv.keep && !mv.keep[r.keep_off + gk * mv.keep_sk]) masked = true;   // where(mask, w, finfo.min), ringattention_inference.py:24
+  const bool off = mv.keep && !mv.keep[r.keep_off + (gk - mv.keep_k0) * mv.keep_sk];
+  if (off && mv.keep_drop) {
+    // chunk_bias += dropped * finfo.min (:321): twice finfo.min overflows to -inf, once absorbs logit and bias
+    return masked ? RA_NEG_INF : mv.mask_min;
+  }
+  if (off) masked = true;                  // where(mask, w, finfo.min), ringattention_inference.py:24
   if (masked) add = mv.mask_min;
   return dot / scale + add;                                       // :134-136
 }
@@ -408,6 +413,51 @@ int keep_pack(const uint8_t* keep, int64_t sb, int64_t sh, int64_t sq, int64_t s
   dim3 grid(K / 64, Q / 64, Bm * Hm);
   keep_pack_kernel<<<grid, 64, 0, s>>>(keep, sb, sh, sq, sk, Hm, Q, K, bits_k, bits_q, summary);
   RA_CHECK_LAUNCH("keep_pack");
+  return RA_OK;
+}
+
+// ------------------------------------------------------------------ attention dropout mask
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11): ten rounds of
+// two 32 x 32 -> 64 bit multiplications, the key bumped by the Weyl constants between rounds.
+struct philox4 { uint32_t v[4]; };
+__host__ __device__ inline philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                                 uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1; c3 = (uint32_t)p0; c0 = n0; c2 = n2;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return philox4{{c0, c1, c2, c3}};
+}
+
+// keep[e] = philox(block e / 4)[e % 4] >= threshold, over the dense (B, H, Q, K) mask: one thread per 16 positions
+__global__ __launch_bounds__(256) void dropout_keep_kernel(uint32_t k0, uint32_t k1, uint32_t threshold,
+                                                           int64_t nblocks, uint32_t* keep4) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  uint32_t w[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int64_t blk = 4 * t + j;
+    const philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)((uint64_t)blk >> 32), 0u, 0u, k0, k1);
+    w[j] = (r.v[0] >= threshold ? 1u : 0u) | (r.v[1] >= threshold ? 1u << 8 : 0u) |
+           (r.v[2] >= threshold ? 1u << 16 : 0u) | (r.v[3] >= threshold ? 1u << 24 : 0u);
+  }
+  if (4 * t + 3 < nblocks) {
+    *(uint4*)(keep4 + 4 * t) = uint4{w[0], w[1], w[2], w[3]};
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (4 * t + j < nblocks) keep4[4 * t + j] = w[j];
+  }
+}
+
+int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hipStream_t s) {
+  const int64_t nblocks = n / 4, nthreads = (nblocks + 3) / 4;
+  dropout_keep_kernel<<<(unsigned)((nthreads + 255) / 256), 256, 0, s>>>((uint32_t)seed, (uint32_t)(seed >> 32),
+                                                                        threshold, nblocks, (uint32_t*)keep);
+  RA_CHECK_LAUNCH("dropout_keep");
   return RA_OK;
 }
 

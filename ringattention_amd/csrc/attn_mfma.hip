@@ -202,7 +202,7 @@ constexpr int WS_PSTR = 40;                 // P / dS row stride in elements (co
 constexpr int WS_PD = 32 * WS_PSTR;         // one 32 x 32 block
 constexpr int WS_TILE = KBM * TROW;
 
-template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
+template <bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
 __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   // Q tiles then dO tiles in one array: a dO address is the Q address plus a constant (an immediate offset)
   __shared__ __attribute__((aligned(16))) uint16_t QGs[6 * WS_TILE];
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   if (HAS_KEEP && mv.skip_tiles && qt_first < qt_end) {
     __shared__ int khull2[2];
     int t_first, t_last;
-    keep_qtile_hull(mv, b, h, gk0 / 64, KBN / 64, mv.keep_q0 / 64 + qt_first, qt_end - qt_first, khull2, tid, 512,
+    keep_qtile_hull(mv, b, h, (gk0 - mv.keep_k0) / 64, KBN / 64, mv.keep_q0 / 64 + qt_first, qt_end - qt_first, khull2, tid, 512,
                     t_first, t_last);
     qt_end = qt_first + t_last;
     qt_first += t_first;
@@ -401,8 +401,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       float x = SC[(G) * 4 + e] * c;                                                                    \
       bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
       if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
-      if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                   \
-      x = masked ? kMask2 : x;                                                                          \
+      if (HAS_KEEP == 2) {     /* dropout adds mask_min (:321): -inf where the pair was masked already */\
+        const bool off_ = !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                                \
+        x = (masked || off_) ? ((masked && off_) ? RA_NEG_INF : kMask2) : x;                            \
+      } else {                                                                                          \
+        if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                 \
+        x = masked ? kMask2 : x;                                                                        \
+      }                                                                                                 \
       const float p = fast_exp2(x - vm2[e]) * vrd[e];                                    /* :226 */     \
       p4[e] = (__bf16)p;                                                                                \
       d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                            /* :229 */     \
@@ -449,9 +454,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     int ks_cur = 2, ks_nxt = 2;
     if (HAS_KEEP) {
       kw_ptr = mv.kbits_q + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
-               (int64_t)(mv.keep_q0 / 64 + qt_first) * mv.keep_K + gk;
+               (int64_t)(mv.keep_q0 / 64 + qt_first) * mv.keep_K + gk - mv.keep_k0;
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
-               (int64_t)(mv.keep_q0 / 64 + qt_first) * (mv.keep_K / 64) + (gk0 + pair * 32) / 64;
+               (int64_t)(mv.keep_q0 / 64 + qt_first) * (mv.keep_K / 64) + (gk0 - mv.keep_k0 + pair * 32) / 64;
       kw_nxt = kw_ptr[0]; ks_nxt = ks_ptr[0];
     }
     // segment ids: a query tile whose 64 rows all carry the one id of this pair's keys needs no compare
@@ -621,7 +626,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #ifndef WS_DQ_VALU_PER_MFMA
 #define WS_DQ_VALU_PER_MFMA 5
 #endif
-template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
+template <bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
 __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   // K tiles then V tiles in one array: a V address is the K address plus a constant (an immediate offset)
   __shared__ __attribute__((aligned(16))) uint16_t KVs[6 * WS_TILE];
@@ -669,7 +674,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {
     __shared__ int khull2[2];
     int t_first, t_last;
-    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, FBM / 64, (gk0_shard + k_base) / 64, ntiles, khull2, tid, 512,
+    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, FBM / 64, (gk0_shard + k_base - mv.keep_k0) / 64, ntiles, khull2, tid, 512,
                     t_first, t_last);
     k_base += t_first * FBN;
     ntiles = t_last - t_first;
@@ -818,8 +823,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
         float x = SC[(G) * 4 + e] * c;                                                                  \
         bool masked = (gk_tile + kr_ >= klim);                                                          \
         if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
-        if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                 \
-        x = masked ? kMask2 : x;                                                                        \
+        if (HAS_KEEP == 2) {     /* dropout adds mask_min (:321): -inf where the pair was masked already */\
+          const bool off_ = !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                              \
+          x = (masked || off_) ? ((masked && off_) ? RA_NEG_INF : kMask2) : x;                          \
+        } else {                                                                                        \
+          if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);               \
+          x = masked ? kMask2 : x;                                                                      \
+        }                                                                                               \
         p = fast_exp2(x - m2) * rden;                                                    /* :226 */     \
       }                                                                                                 \
       d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                            /* :229 */     \
@@ -872,8 +882,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     uint64_t kw_cur = 0, kw_nxt = 0;
     if (HAS_KEEP) {
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
-               (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
-      kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
+               (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + (gk0 - mv.keep_k0) / 64;
+      kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
+               (int64_t)((gk0 - mv.keep_k0) / 64) * mv.keep_Q +
                mv.keep_q0 + qrow;
     }
     const int2* smm_ptr = nullptr;
@@ -1051,7 +1062,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 // per-lane scalars: a lane owns a query column) and leaves P^T, rounded to bf16, in LDS together with the
 // factor by which the output accumulator has to shrink when the reference max moved; the consumer runs
 // O^T += V^T P^T one block of 32 keys behind.
-template <bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
+template <bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
 __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   // K tiles then V tiles in one array: a V address is the K address plus a constant (an immediate offset)
   __shared__ __attribute__((aligned(16))) uint16_t KVs[6 * WS_TILE];
@@ -1101,7 +1112,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {
     __shared__ int khull2[2];
     int t_first, t_last;
-    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, FBM / 64, (gk0_shard + k_base) / 64, ntiles, khull2, tid, 512,
+    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, FBM / 64, (gk0_shard + k_base - mv.keep_k0) / 64, ntiles, khull2, tid, 512,
                     t_first, t_last);
     k_base += t_first * FBN;
     ntiles = t_last - t_first;
@@ -1265,15 +1276,21 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
         float x_ = SC[r] * c;                                                                           \
         bool masked_ = (gk_tile + kr_ >= klim);                                                         \
         if (HAS_SEG) masked_ = masked_ || (seg_ks[BUF][kr_] != seg_q);                                  \
-        if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1);    \
-        x_ = masked_ ? kMask2 : x_;                                                                     \
+        if (HAS_KEEP == 2) {     /* dropout adds mask_min (:321): -inf where the pair was masked already */\
+          const bool off_ = !((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1);                   \
+          x_ = (masked_ || off_) ? ((masked_ && off_) ? RA_NEG_INF : kMask2) : x_;                      \
+        } else {                                                                                        \
+          if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1);  \
+          x_ = masked_ ? kMask2 : x_;                                                                   \
+        }                                                                                               \
         SC[r] = x_;                                                                                     \
         mxv_ = fmaxf(mxv_, x_);                                                                         \
       }                                                                                                 \
       mxv_ = max_xor32(mxv_);                                                                           \
       m_true = fmaxf(m_true, mxv_);                                                                     \
       const float m_new_ = fmaxf(m2, mxv_);                                                             \
-      alpha_ = fast_exp2(m2 - m_new_);                                                                  \
+      /* under dropout every pair so far may be -inf: nothing accumulated yet, nothing to rescale */    \
+      alpha_ = (HAS_KEEP == 2 && m_new_ == RA_NEG_INF) ? 1.f : fast_exp2(m2 - m_new_);                       \
       m2 = m_new_;                                                                                      \
       l *= alpha_;                                                                                      \
     }                                                                                                   \
@@ -1283,8 +1300,9 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   {                                                                                                     \
     if ((G) == 0) RA_WS_ROWMAX(SC, BUF, BLK, PB, MASKED);                                               \
     bf16x4 d4;                                                                                          \
+    const float mref_ = (HAS_KEEP == 2 && (MASKED) && m2 == RA_NEG_INF) ? 0.f : m2;   /* exp2(-inf - 0) = 0 */ \
     _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
-      const float p = (MASKED) ? fast_exp2(SC[(G) * 4 + e] - m2) : fast_exp2(fmaf(SC[(G) * 4 + e], c, -m2)); \
+      const float p = (MASKED) ? fast_exp2(SC[(G) * 4 + e] - mref_) : fast_exp2(fmaf(SC[(G) * 4 + e], c, -m2)); \
       ps += p;                                                                                          \
       d4[e] = (__bf16)p;                                                                                \
     }                                                                                                   \
@@ -1331,8 +1349,9 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     uint64_t kw_cur = 0, kw_nxt = 0;
     if (HAS_KEEP) {
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
-               (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + gk0 / 64;
-      kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + (int64_t)(gk0 / 64) * mv.keep_Q +
+               (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + (gk0 - mv.keep_k0) / 64;
+      kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
+               (int64_t)((gk0 - mv.keep_k0) / 64) * mv.keep_Q +
                mv.keep_q0 + qrow;
     }
     const int2* smm_ptr = nullptr;
@@ -1534,11 +1553,11 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
-// a boolean keep mask is taken in packed form only and alone (no bias, segment ids or causal block size next to it:
-// ring_attention_inference has none of them, and the generic kernels serve any combination)
+// a boolean keep mask is taken in packed form only, next to a causal block size at most (no bias or segment ids:
+// ring_attention_inference has neither, and the generic kernels serve any combination)
 static bool keep_ok(const ra_mask& m) {
   if (!m.keep) return true;
-  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids && m.causal_block_size == 0;
+  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids;
 }
 
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
@@ -1564,7 +1583,8 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
   RA_REQUIRE(nwg3 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
   dim3 grid3((unsigned)((nwg3 + 7) / 8 * 8)), block3(512);
-  if (keep) attn_fwd_ws_kernel<false, false, true><<<grid3, block3, 0, s>>>(a);
+  if (keep && p->mask.keep_mode == RA_KEEP_DROPOUT) attn_fwd_ws_kernel<false, false, 2><<<grid3, block3, 0, s>>>(a);
+  else if (keep) attn_fwd_ws_kernel<false, false, 1><<<grid3, block3, 0, s>>>(a);
   else if (seg && bias) attn_fwd_ws_kernel<true, true><<<grid3, block3, 0, s>>>(a);
   else if (seg) attn_fwd_ws_kernel<true, false><<<grid3, block3, 0, s>>>(a);
   else if (bias) attn_fwd_ws_kernel<false, true><<<grid3, block3, 0, s>>>(a);
@@ -1603,7 +1623,8 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
     if (do_dkv) attn_bwd_dkv_ws_kernel<__VA_ARGS__><<<gk, block, 0, s>>>(a);             \
     if (do_dq) attn_bwd_dq_ws_kernel<__VA_ARGS__><<<gq, block, 0, s>>>(a);               \
   } while (0)
-  if (p->mask.keep) RA_LAUNCH_BWD(false, false, true);      // packed boolean mask
+  if (p->mask.keep && p->mask.keep_mode == RA_KEEP_DROPOUT) RA_LAUNCH_BWD(false, false, 2);
+  else if (p->mask.keep) RA_LAUNCH_BWD(false, false, 1);      // packed boolean mask
   else if (seg && bias) RA_LAUNCH_BWD(true, true);
   else if (seg) RA_LAUNCH_BWD(true, false);
   else if (bias) RA_LAUNCH_BWD(false, true);

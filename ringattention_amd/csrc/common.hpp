@@ -63,13 +63,14 @@ struct MaskView {
   int skip_tiles;
   const int32_t* seg_mm;   // per-64-position (min, max) segment ids, or null
   int seg_tiles;
-  const uint8_t* keep;     // boolean mask (local query row, global key), or null
+  const uint8_t* keep;     // boolean mask (local query row, global key - keep_k0), or null
   int64_t keep_sb, keep_sh, keep_sq, keep_sk;
   const uint64_t* kbits_k;   // packed mask, see ra_keep_pack; all null unless the MFMA kernels take the mask
   const uint64_t* kbits_q;
   const uint8_t* ksum;
   int64_t kpack_sb, kpack_sh, ksum_sb, ksum_sh;
-  int keep_Q, keep_K, keep_q0;
+  int keep_Q, keep_K, keep_q0, keep_k0;
+  int keep_drop;           // 1: dropout semantics (mask_min added: a pair masked twice becomes -inf)
 
   __host__ __device__ static MaskView make(const ra_mask& m, int q_chunk_idx_start) {
     MaskView v;
@@ -88,6 +89,7 @@ struct MaskView {
     v.kpack_sb = m.keep_pack_stride_b; v.kpack_sh = m.keep_pack_stride_h;
     v.ksum_sb = m.keep_sum_stride_b; v.ksum_sh = m.keep_sum_stride_h;
     v.keep_Q = m.keep_q_total; v.keep_K = m.keep_k_total; v.keep_q0 = m.keep_q0;
+    v.keep_k0 = m.keep_k0; v.keep_drop = m.keep_mode == RA_KEEP_DROPOUT;
     return v;
   }
 

@@ -23,6 +23,8 @@ def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwarg
     int32 scalar (read by the kernel, so the call can sit in a captured graph or a tight loop).
     blockwise_kwargs must carry query_chunk_size == 1, as q_len // query_chunk_size demands."""
     cfg = _Config(blockwise_kwargs)
+    if cfg.pdrop > 0.0:
+        raise NotImplementedError("attention dropout together with cache_idx is not supported")
     _check_qkv(q, k, v)
     B, Sq, H, D = q.shape
     if Sq != 1:

@@ -120,17 +120,26 @@ class _Config:
         self.cbs = None if cbs is None else int(cbs)
         if self.cbs is not None and self.cbs < 1:
             raise ValueError("causal_block_size must be None or >= 1")
+        # attention dropout (:119-123): ``dropout_rng`` is an integer seed of the Philox stream ra_dropout_keep
+        # documents, not a jax.random key; the mask is a pure function of (seed, attn_pdrop, local shape)
+        self.pdrop = 0.0
+        self.seed = 0
         if (not kw.get("deterministic", True)) and float(kw.get("attn_pdrop", 0.0)) > 0.0:
-            raise NotImplementedError(
-                "attention dropout is not supported: its mask comes from the jax.random stream")
+            self.pdrop = float(kw["attn_pdrop"])
+            if not self.pdrop < 1.0:
+                raise ValueError("attn_pdrop must lie in [0, 1)")
+            rng = kw.get("dropout_rng", None)
+            if rng is None:
+                raise ValueError("attention dropout needs blockwise_kwargs['dropout_rng'] (an integer seed)")
+            self.seed = int(rng) & 0xFFFFFFFFFFFFFFFF
         self.dtype = _as_torch_dtype(kw.get("dtype", torch.float32))
         self.mask_min = float(torch.finfo(self.dtype).min)
         self.impl = {"auto": L.RA_IMPL_AUTO, "generic": L.RA_IMPL_GENERIC, "mfma": L.RA_IMPL_MFMA}[
             kw.get("impl", "auto")]
         self.bwd_only = {None: 0, "dq": L.RA_BWD_ONLY_DQ, "dkv": L.RA_BWD_ONLY_DKV}[kw.get("bwd_only", None)]
         self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
-        # policy / precision / prevent_cse / dropout_rng only steer XLA rematerialisation: the
-        # kernels always recompute the probabilities in the backward pass.
+        # policy / precision / prevent_cse only steer XLA rematerialisation: the kernels always recompute
+        # the probabilities in the backward pass.
 
 
 class _MaskInputs:
@@ -170,9 +179,14 @@ class _MaskInputs:
             L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], self.seg_len,
                                                     self.seg_mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
             self._seg_mm_host = None
-        self.keep = None                   # boolean mask of ring_attention_inference, set by set_keep()
+        self.keep = None                   # boolean mask: ring_attention_inference (set_keep) or dropout
         self.keep_strides = (0, 0, 0, 0)
         self.keep_row0 = 0
+        self.keep_k0 = 0
+        self.keep_mode = L.RA_KEEP_WHERE
+        self.keep_packed = None
+        self._drop_base = None             # (B, H, q_len, kv_len) keep bytes of the dropout mask
+        self._drop_steps = {}
         self.cache_idx_host = None
         self.cache_idx_dev = None
         if cache_idx is not None:
@@ -199,14 +213,8 @@ class _MaskInputs:
         self.keep_strides = tuple(0 if m.shape[i] == 1 else m.stride(i) for i in range(4))
         self.keep_packed = None
         if q_total % 64 == 0 and k_total % 64 == 0:
+            bits_k, bits_q, summ = self._pack(m, self.keep_strides, q_total, k_total)
             bm, hm = m.shape[0], m.shape[1]
-            words = q_total * k_total // 64
-            bits_k = torch.empty((bm, hm, words), dtype=torch.int64, device=device)
-            bits_q = torch.empty((bm, hm, words), dtype=torch.int64, device=device)
-            summ = torch.empty((bm, hm, (q_total // 64) * (k_total // 64)), dtype=torch.uint8, device=device)
-            L.check(L.load().ra_keep_pack(m.data_ptr(), m.stride(0), m.stride(1), self.keep_strides[2], m.stride(3),
-                                          bm, hm, q_total, k_total, bits_k.data_ptr(), bits_q.data_ptr(),
-                                          summ.data_ptr(), _stream()), "ra_keep_pack")
             # a query row with no attended key keeps equal finfo.min logits (uniform weights): kernels must
             # not skip its fully masked tiles.  Read off the packed words (an eighth of the mask's bytes).
             row_has_key = (bits_k.view(bm, hm, k_total // 64, q_total) != 0).any(dim=2)
@@ -214,6 +222,60 @@ class _MaskInputs:
             self.keep_packed = (bits_k, bits_q, summ, q_total, k_total)
         else:
             self.keep_has_empty_row = bool((m.amax(dim=3) == 0).any().item())
+
+    @staticmethod
+    def _pack(m, strides, q_total, k_total):
+        """ra_keep_pack of a (Bm, Hm, Q|1, K) byte mask: the 64-bit words by key tile and by query tile, and the
+        per-tile summary."""
+        bm, hm = m.shape[0], m.shape[1]
+        words = q_total * k_total // 64
+        bits_k = torch.empty((bm, hm, words), dtype=torch.int64, device=m.device)
+        bits_q = torch.empty((bm, hm, words), dtype=torch.int64, device=m.device)
+        summ = torch.empty((bm, hm, (q_total // 64) * (k_total // 64)), dtype=torch.uint8, device=m.device)
+        L.check(L.load().ra_keep_pack(m.data_ptr(), m.stride(0), m.stride(1), strides[2], m.stride(3),
+                                      bm, hm, q_total, k_total, bits_k.data_ptr(), bits_q.data_ptr(),
+                                      summ.data_ptr(), _stream()), "ra_keep_pack")
+        return bits_k, bits_q, summ
+
+    def use_dropout(self, cfg, batch, heads, q_len, kv_len, q_chunk_idx_start, k_chunk_idx_start, device):
+        """Points the keep mask at the dropout mask of this step (ringattention_jax.py:119-123, :311-321).
+
+        The reference draws ONE mask of the local shape (batch, heads, q_len, kv_len) per call - the same in
+        every ring step, the key being a constant of blockwise_kwargs - and slices it with dynamic_slice at the
+        GLOBAL chunk offsets, which clamps: chunk j of a step whose chunk index starts at s reads the mask rows
+        min((s + j) * qc, q_len - qc) ..., and likewise along the keys.  Steps that start at 0 read the mask as
+        it is; every other start is served by a gathered copy, cached per (row start, key start)."""
+        if self.cache_idx_host is not None or self.cache_idx_dev is not None:
+            raise NotImplementedError("attention dropout together with cache_idx is not supported")
+        if kv_len % 4:
+            raise NotImplementedError("attention dropout needs a key length that is a multiple of 4")
+        shape = (batch, heads, q_len, kv_len)
+        if self._drop_base is None:
+            base = torch.empty(shape, dtype=torch.uint8, device=device)
+            L.check(L.load().ra_dropout_keep(cfg.seed, cfg.pdrop, batch, heads, q_len, kv_len, base.data_ptr(),
+                                             _stream()), "ra_dropout_keep")
+            self._drop_base = base
+        elif tuple(self._drop_base.shape) != shape:
+            raise ValueError("the dropout mask of this call was drawn for another shape")
+        nq, nk = q_len // cfg.qc, kv_len // cfg.kc
+        key = (min(q_chunk_idx_start, nq), min(k_chunk_idx_start, nk))
+        if key not in self._drop_steps:
+            m = self._drop_base
+            if key[0] != 0:
+                starts = torch.clamp((key[0] + torch.arange(nq, device=device)) * cfg.qc, max=q_len - cfg.qc)
+                m = m.index_select(2, (starts[:, None] + torch.arange(cfg.qc, device=device)).reshape(-1))
+            if key[1] != 0:
+                starts = torch.clamp((key[1] + torch.arange(nk, device=device)) * cfg.kc, max=kv_len - cfg.kc)
+                m = m.index_select(3, (starts[:, None] + torch.arange(cfg.kc, device=device)).reshape(-1))
+            packed = None
+            if q_len % 64 == 0 and kv_len % 64 == 0:
+                packed = self._pack(m, m.stride(), q_len, kv_len) + (q_len, kv_len)
+            self._drop_steps[key] = (m, packed)
+        self.keep, self.keep_packed = self._drop_steps[key]
+        self.keep_strides = self.keep.stride()
+        self.keep_row0 = 0
+        self.keep_k0 = k_chunk_idx_start * cfg.kc
+        self.keep_mode = L.RA_KEEP_DROPOUT
 
     def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip):
         m = L.RaMask()
@@ -243,6 +305,8 @@ class _MaskInputs:
                 m.keep_sum_stride_b = 0 if summ.shape[0] == 1 else summ.stride(0)
                 m.keep_sum_stride_h = 0 if summ.shape[1] == 1 else summ.stride(1)
                 m.keep_q_total, m.keep_k_total, m.keep_q0 = q_total, k_total, self.keep_row0
+            m.keep_k0 = self.keep_k0
+            m.keep_mode = self.keep_mode
         return m
 
     def segments_meet(self, q_lo, q_hi, k_lo, k_hi):
@@ -316,6 +380,9 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
     skip = cfg.skip_masked_tiles
     if skip is None:
         skip = cfg.qc >= 2 and cache_idx is None
+    if cfg.pdrop > 0.0:
+        mi.use_dropout(cfg, B, H, Sq, Skv, q_chunk_idx_start, k_chunk_idx_start, q.device)
+        skip = False        # a row may lose every allowed key: its masked tiles then carry its (uniform) weights
     p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
     p.impl = cfg.impl
     p.carry_is_initial = 1 if _carry_is_initial else 0
@@ -367,6 +434,9 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
     skip = cfg.skip_masked_tiles
     if skip is None:
         skip = cfg.qc >= 2 and cache_idx is None
+    if cfg.pdrop > 0.0:
+        mi.use_dropout(cfg, B, H, Sq, Skv, q_chunk_idx_start, k_chunk_idx_start, q.device)
+        skip = False
     p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
     p.impl = cfg.impl | cfg.bwd_only
     L.check(L.load().ra_attn_bwd_block(ctypes.byref(p), _stream()), "ra_attn_bwd_block")
@@ -450,6 +520,10 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, kv_total)
     if cfg.skip_masked_tiles is None:
         cfg.skip_masked_tiles = bool(cfg.qc >= 2 and cache_idx is None and q_total == kv_total)
+    if cfg.pdrop > 0.0:
+        if cache_idx is not None:
+            raise NotImplementedError("attention dropout together with cache_idx is not supported")
+        cfg.skip_masked_tiles = False      # dropout can leave a row without any allowed key
     num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)      # :22
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)         # :23
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)          # :49

@@ -1,0 +1,175 @@
+"""Attention dropout (ringattention_jax.py:119-123, :206-208, :311-321) on the GPU against the oracle.
+
+The mask bits come from the Philox stream both sides document (not from jax.random, which is not restated), so
+the comparison is exact in the mask and to the parity bar in the values: max-abs 1e-4 (fp32) / 2e-2 (bf16),
+relative L2 1e-2."""
+import pytest
+import torch
+
+import ringattention_amd as ra
+from ringattention_amd import _lib as L
+from oracle import ringattention_oracle as O
+from tests.util import assert_close, errors, kwargs, make_qkv, oracle_fwd_bwd, packed_segment_ids
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("shape,seed,p", [
+    ((1, 1, 4, 8), 0, 0.5),
+    ((2, 3, 64, 128), 1234, 0.1),
+    ((1, 2, 100, 36), (1 << 40) + 17, 0.25),       # not a multiple of 16 positions: the tail of the last thread
+    ((1, 1, 256, 4100), 0xFFFFFFFFFFFFFFFF, 0.9),
+])
+def test_dropout_mask_bits_are_the_documented_philox_stream(shape, seed, p):
+    keep = torch.empty(shape, dtype=torch.uint8, device=DEV)
+    L.check(L.load().ra_dropout_keep(seed, p, *shape, keep.data_ptr(), None), "ra_dropout_keep")
+    torch.cuda.synchronize()
+    dropped = O.dropout_mask(seed, p, shape)
+    assert torch.equal(keep.cpu() == 0, dropped)
+    if dropped.numel() >= 10000:
+        assert abs(float(dropped.float().mean()) - p) < 0.02
+
+
+def test_dropout_mask_rejects():
+    lib = L.load()
+    keep = torch.empty(64, dtype=torch.uint8, device=DEV)
+    assert lib.ra_dropout_keep(0, 0.5, 1, 1, 8, 6, keep.data_ptr(), None) == L.RA_ERR_UNSUPPORTED     # K % 4
+    assert lib.ra_dropout_keep(0, 0.0, 1, 1, 8, 8, keep.data_ptr(), None) == L.RA_ERR_INVALID
+    assert lib.ra_dropout_keep(0, 1.0, 1, 1, 8, 8, keep.data_ptr(), None) == L.RA_ERR_INVALID
+    assert lib.ra_dropout_keep(0, 0.5, 1, 1, 8, 8, None, None) == L.RA_ERR_INVALID
+
+
+def _run(q, k, v, do, bias, seg, n, kw):
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention(qd, kd, vd, None if bias is None else bias.to(DEV),
+                               None if seg is None else seg.to(DEV), None, axis_name="sp", float32_logits=True,
+                               blockwise_kwargs=kw)
+        out.backward(do.to(DEV))
+    torch.cuda.synchronize()
+    return out, (qd.grad, kd.grad, vd.grad)
+
+
+def _compare(q, k, v, do, bias, seg, n, kw, dtype, what):
+    print("dropout", what, flush=True)
+    ref_out, ref_g = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = _run(q, k, v, do, bias, seg, n, kw)
+    assert_close(out, ref_out, dtype, what + " out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_g):
+        assert_close(a, b, dtype, what + " " + name)
+    return out
+
+
+@pytest.mark.parametrize("n", [1, 2, 4])
+@pytest.mark.parametrize("qc,kc,cbs", [(16, 16, 1), (16, 8, 1), (8, 16, 4), (16, 16, None)])
+def test_dropout_generic_fp32_matches_oracle(n, qc, kc, cbs):
+    """fp32, small chunks: the generic kernels; rings of 2 and 4 read the mask through the clamped slices."""
+    B, S, H, D = 2, 64, 2, 32
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=11)
+    kw = kwargs(qc, kc, cbs, deterministic=False, dropout_rng=1234, attn_pdrop=0.3)
+    _compare(q, k, v, do, None, None, n, kw, torch.float32, "generic n%d %d/%d cbs %s" % (n, qc, kc, cbs))
+
+
+def test_dropout_with_segments_and_bias_matches_oracle():
+    B, S, H, D = 2, 128, 2, 32
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=12)
+    seg = packed_segment_ids(B, S, 40, seed=3)
+    bias = torch.randn(B, 1, 1, S, generator=torch.Generator().manual_seed(4))
+    kw = kwargs(32, 16, 1, deterministic=False, dropout_rng=99, attn_pdrop=0.2)
+    _compare(q, k, v, do, bias, seg, 2, kw, torch.float32, "segments + bias")
+
+
+@pytest.mark.parametrize("n,S,qc,kc,cbs,p", [
+    (1, 512, 256, 256, 1, 0.1),
+    (1, 1024, 512, 256, 1, 0.5),
+    (2, 1024, 256, 256, 1, 0.1),
+    (4, 2048, 256, 512, 1, 0.3),
+    (1, 512, 256, 256, None, 0.1),
+    (2, 1024, 512, 512, 256, 0.2),
+])
+def test_dropout_mfma_bf16_matches_oracle(n, S, qc, kc, cbs, p):
+    """bf16, D 128, chunk sizes the MFMA kernels take: the packed mask, next to the causal block size."""
+    B, H, D = 1, 2, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=13, scale=D ** -0.25)
+    kw = kwargs(qc, kc, cbs, deterministic=False, dropout_rng=7, attn_pdrop=p, impl="mfma")
+    _compare(q, k, v, do, None, None, n, kw, torch.bfloat16, "mfma n%d S%d %d/%d cbs %s p %.1f" % (n, S, qc, kc, cbs, p))
+
+
+def test_dropout_mfma_equals_generic():
+    """The same mask through both kernel families, including the rows that lose every allowed key."""
+    B, S, H, D = 1, 1024, 4, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=14, scale=D ** -0.25)
+    res = {}
+    for impl in ("mfma", "generic"):
+        kw = kwargs(256, 256, 1, deterministic=False, dropout_rng=5, attn_pdrop=0.5, impl=impl)
+        res[impl] = _run(q, k, v, do, None, None, 2, kw)
+    # with p = 0.5 row 0 of every head loses its one allowed key with probability 1/2: such rows exist here
+    dropped = O.dropout_mask(5, 0.5, (B, H, S // 2, S // 2))
+    assert bool(dropped[0, :, 0, 0].any())
+    assert_close(res["mfma"][0], res["generic"][0].float(), torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), res["mfma"][1], res["generic"][1]):
+        # both sides are rounded to bf16 (2^-8 relative each) and the rows with uniform weights make |dv| reach 4:
+        # the absolute bar scales with the magnitude, the relative one is the usual 1e-2
+        ma, rl = errors(a, b.float())
+        assert ma <= 2e-2 * max(1.0, float(b.abs().max())) and rl <= 1e-2, (name, ma, rl)
+
+
+def test_dropout_row_without_allowed_key_takes_uniform_weights():
+    """Causal row 0 whose key 0 is dropped: logits are finfo.min at key 0 (dropped once) and at the causally masked
+    keys that were not dropped, -inf at those masked AND dropped (:321 adds finfo.min twice): the output is the mean
+    of V over the first set, in the one key chunk that runs for the row."""
+    B, S, H, D, kc = 1, 256, 8, 128, 256
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=15, scale=D ** -0.25)
+    seed, p = 21, 0.5
+    dropped = O.dropout_mask(seed, p, (B, H, S, S))
+    heads = [h for h in range(H) if bool(dropped[0, h, 0, 0])]
+    assert heads, "no head drops key 0 of row 0 with this seed"
+    for impl in ("mfma", "generic"):
+        kw = kwargs(256, kc, 1, deterministic=False, dropout_rng=seed, attn_pdrop=p, impl=impl)
+        out, _ = _run(q, k, v, do, None, None, 1, kw)
+        for h in heads:
+            level1 = ~dropped[0, h, 0, :kc]
+            level1[0] = True
+            want = v[0, :kc, h].float()[level1].mean(dim=0)
+            got = out.detach()[0, 0, h].float().cpu()
+            assert float((got - want).abs().max()) <= 2e-2, (impl, h)
+
+
+def test_dropout_probabilities_still_sum_to_one_at_8k():
+    """V = 1: every row is a convex combination, whatever was dropped (rows without any allowed key included)."""
+    B, S, H, D = 1, 8192, 4, 128
+    g = torch.Generator(device=DEV).manual_seed(0)
+    q = (torch.randn(B, S, H, D, device=DEV, generator=g) * D ** -0.25).bfloat16()
+    k = (torch.randn(B, S, H, D, device=DEV, generator=g) * D ** -0.25).bfloat16()
+    v = torch.ones(B, S, H, D, device=DEV, dtype=torch.bfloat16)
+    kw = kwargs(512, 512, 1, deterministic=False, dropout_rng=3, attn_pdrop=0.1)
+    out = ra.ringattention(q, k, v, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    assert float((out.float() - 1.0).abs().max()) <= 1e-2
+    # and the mask is a function of the seed: same seed same bits, another seed another result
+    v2 = torch.randn(B, S, H, D, device=DEV, generator=g).bfloat16()
+    a = ra.ringattention(q, k, v2, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    b = ra.ringattention(q, k, v2, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    c = ra.ringattention(q, k, v2, None, None, None, axis_name=None, float32_logits=True,
+                         blockwise_kwargs=dict(kw, dropout_rng=4))
+    assert torch.equal(a, b) and not torch.equal(a, c)
+
+
+def test_dropout_rejects():
+    q, k, v, _ = make_qkv(1, 64, 2, 32, dtype=torch.float32, seed=1)
+    q, k, v = (t.to(DEV) for t in (q, k, v))
+    kw = kwargs(16, 16, 1, deterministic=False, attn_pdrop=0.1)          # no dropout_rng
+    with pytest.raises(ValueError):
+        ra.ringattention(q, k, v, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    kw = kwargs(1, 16, 1, deterministic=False, attn_pdrop=0.1, dropout_rng=1)
+    with pytest.raises(NotImplementedError):                                # decode
+        ra.ringattention(q[:, :1], k, v, None, None, 5, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    kw = kwargs(16, 16, 1, deterministic=False, attn_pdrop=1.0, dropout_rng=1)
+    with pytest.raises(ValueError):
+        ra.ringattention(q, k, v, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    # deterministic=True ignores attn_pdrop, as the reference does (:119)
+    kw = kwargs(16, 16, 1, deterministic=True, attn_pdrop=0.5)
+    a = ra.ringattention(q, k, v, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+    b = ra.ringattention(q, k, v, None, None, None, axis_name=None, float32_logits=True,
+                         blockwise_kwargs=kwargs(16, 16, 1))
+    assert torch.equal(a, b)

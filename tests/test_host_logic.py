@@ -75,11 +75,17 @@ def test_cpu_tensors_are_refused():
         ra.ringattention(q, q, q, None, None, None, "sp", True, kw)
 
 
-def test_dropout_is_refused():
+def test_dropout_configuration():
     from ringattention_amd.ringattention_hip import _Config
-    with pytest.raises(NotImplementedError):
-        _Config(dict(causal_block_size=1, query_chunk_size=4, key_chunk_size=4, deterministic=False,
-                     attn_pdrop=0.1, dtype=torch.float32))
+    base = dict(causal_block_size=1, query_chunk_size=4, key_chunk_size=4, dtype=torch.float32)
+    cfg = _Config(dict(base, deterministic=False, attn_pdrop=0.1, dropout_rng=(1 << 40) + 3))
+    assert cfg.pdrop == 0.1 and cfg.seed == (1 << 40) + 3
+    assert _Config(dict(base, deterministic=True, attn_pdrop=0.1)).pdrop == 0.0        # :119: both conditions
+    assert _Config(dict(base, deterministic=False, attn_pdrop=0.0)).pdrop == 0.0
+    with pytest.raises(ValueError):
+        _Config(dict(base, deterministic=False, attn_pdrop=0.1))                         # no dropout_rng
+    with pytest.raises(ValueError):
+        _Config(dict(base, deterministic=False, attn_pdrop=1.0, dropout_rng=0))
 
 
 def test_invalid_arguments_return_codes_without_gpu():

@@ -329,12 +329,93 @@ def test_blockwise_feedforward_equals_unchunked_and_uses_strided_groups():
     assert torch.equal(seen[1], x[:, 1::4])
 
 
-def test_dropout_is_refused():
-    q, k, v = make(1, 8, 1, 4)
-    kw = kwargs(4, 4, 1)
-    kw.update(deterministic=False, attn_pdrop=0.1)
-    with pytest.raises(NotImplementedError):
-        O.ring_attention(q, k, v, None, None, None, 1, True, kw)
+# --------------------------------------------------------------------------- attention dropout
+def test_philox_known_answers():
+    """Philox4x32-10 known-answer vectors of the Random123 distribution (kat_vectors): zero, all ones, digits of pi."""
+    import numpy as np
+    cases = [
+        ([0, 0, 0, 0], [0, 0], "6627e8d5 e169c58d bc57ac4c 9b00dbd8"),
+        ([0xffffffff] * 4, [0xffffffff] * 2, "408f276d 41c83b0e a20bc7c6 6d5451fd"),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+         "d16cfe09 94fdcceb 5001e420 24126ea1"),
+    ]
+    for counter, key, want in cases:
+        got = O.philox4x32_10(np.array([counter], dtype=np.uint32), np.array([key], dtype=np.uint32))[0]
+        assert " ".join("%08x" % int(x) for x in got) == want
+
+
+def test_dropout_mask_is_a_function_of_seed_and_rate():
+    a = O.dropout_mask(5, 0.25, (2, 3, 32, 64))
+    assert a.dtype == torch.bool and a.shape == (2, 3, 32, 64)
+    assert torch.equal(a, O.dropout_mask(5, 0.25, (2, 3, 32, 64)))
+    assert not torch.equal(a, O.dropout_mask(6, 0.25, (2, 3, 32, 64)))
+    assert abs(float(a.float().mean()) - 0.25) < 0.02
+    # position e takes word e % 4 of block e // 4: a longer mask with the same seed starts with the same bits
+    b = O.dropout_mask(5, 0.25, (1, 1, 1, 128))
+    assert torch.equal(b.reshape(-1), O.dropout_mask(5, 0.25, (1, 1, 2, 128)).reshape(-1)[:128])
+    # a lower rate drops a subset (same words, lower threshold)
+    assert bool((O.dropout_mask(5, 0.1, (2, 3, 32, 64)) <= a).all())
+
+
+def _dropout_kwargs(qc, kc, cbs, p=0.3, seed=1234):
+    kw = kwargs(qc, kc, cbs)
+    kw.update(deterministic=False, attn_pdrop=p, dropout_rng=seed)
+    return kw
+
+
+@pytest.mark.parametrize("n", [1, 2, 4])
+@pytest.mark.parametrize("qc,kc,cbs", [(16, 16, 1), (16, 8, 1), (8, 16, 4), (16, 16, None)])
+def test_dropout_blockwise_matches_dense(n, qc, kc, cbs):
+    """The chunk loops with the sliced mask (:311-321) against the un-chunked softmax whose mask is built from
+    global positions, float64, on the rows that keep an allowed key (the others are covered in fp32 below); rings
+    of 2 and 4 read the mask of local shape through the clamped global offsets."""
+    q, k, v = make(2, 64, 2, 16, seed=1)
+    kw = _dropout_kwargs(qc, kc, cbs)
+    out, res = O.ring_attention_fwd(q, k, v, None, None, None, n, True, kw, compute_dtype=F64)
+    ref = O.dense_attention(q, k, v, None, None, None, n, kw)
+    real = (res[-1] > -1e30).permute(0, 2, 1)
+    assert int(real.sum()) >= real.numel() - 8
+    assert float((out - ref)[real].abs().max()) < 1e-12
+    # backward against autograd of the dense form, on cotangents that vanish on the other rows
+    g = torch.randn(out.shape, dtype=F64, generator=torch.Generator().manual_seed(2)) * real[..., None]
+    dq, dk, dv = O.ring_attention_bwd(n, True, kw, res, g)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    dense = O.dense_attention(qa, ka, va, None, None, None, n, kw)
+    torch.where(real[..., None], dense, torch.zeros_like(dense)).mul(g).sum().backward()
+    for a, b in ((dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
+        assert float((a - b).abs().max()) < 1e-10
+
+
+def test_dropped_keys_get_exactly_zero_weight():
+    q, k, v = make(1, 64, 2, 16, seed=3)
+    kw = _dropout_kwargs(16, 16, None, p=0.4, seed=9)
+    dropped = O.dropout_mask(9, 0.4, (1, 2, 64, 64))
+    out = O.ring_attention(q, k, v, None, None, None, 1, True, kw, compute_dtype=F64)
+    # equals a softmax over the kept keys only
+    logits = torch.einsum("bqhd,bkhd->bhqk", q, k) / math.sqrt(16)
+    p = torch.softmax(logits.masked_fill(dropped, -math.inf), dim=-1)
+    ref = torch.einsum("bhqk,bkhd->bqhd", p, v)
+    assert float((out - ref).abs().max()) < 1e-12
+    # no rescale by 1 / (1 - p) (:321 only masks): rows still sum to one
+    ones = O.ring_attention(q, k, torch.ones_like(v), None, None, None, 1, True, kw, compute_dtype=F64)
+    assert float((ones - 1.0).abs().max()) < 1e-12
+
+
+def test_dropout_row_without_allowed_key_fp32():
+    """Causal row 0 with key 0 dropped, fp32 as the reference computes: key 0 holds finfo.min (dropped once), the
+    causally masked keys hold finfo.min if kept and -inf if dropped (finfo.min added twice, :321), so the row is the
+    mean of V over {key 0} and the kept masked keys of the chunks that run."""
+    seed = next(s for s in range(100) if bool(O.dropout_mask(s, 0.5, (1, 1, 16, 16))[0, 0, 0, 0]))
+    dropped = O.dropout_mask(seed, 0.5, (1, 1, 16, 16))
+    q, k, v = make(1, 16, 1, 8, seed=4, dtype=torch.float32)
+    for qc, kc in ((16, 16), (8, 8), (16, 4)):
+        kw = _dropout_kwargs(qc, kc, 1, p=0.5, seed=seed)
+        out = O.ring_attention(q, k, v, None, None, None, 1, True, kw)
+        ncols = kc if qc <= kc else 16     # key chunks that run for row 0: below_or_on_diag keeps c * kc < qc
+        level1 = ~dropped[0, 0, 0, :ncols]
+        level1[0] = True
+        want = v[0, :ncols, 0][level1].mean(dim=0)
+        assert float((out[0, 0, 0] - want).abs().max()) < 1e-6, (qc, kc)
 
 
 # --------------------------------------------------------------------------- ring_attention_inference
