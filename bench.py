@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ring-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|inference|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|inference|copy|decode_step|rmsnorm|dropout32k]
 
 One step = one pass of the hot path over one batch of synthetic input already resident in HBM.
 Default workload ``attn32k`` is the configuration the headline metric is quoted on: blockwise
@@ -81,7 +81,7 @@ def _packed_segments(S, mean_len, seed, device):
 
 
 # --------------------------------------------------------------------------- attention workloads
-def bench_attention(args, ring):
+def bench_attention(args, ring, dropout=False):
     import torch
     import ringattention_amd as ra
     from ringattention_amd import ringattention_hip as rh
@@ -91,6 +91,8 @@ def bench_attention(args, ring):
         S, n, name = 131072, 8, "ring131k"
     else:
         S, n, name = 32768, 1, "attn32k"
+    if dropout:
+        name = "dropout32k"
     if args.seq_len:
         S = args.seq_len
     g = torch.Generator(device=dev).manual_seed(0)
@@ -104,13 +106,22 @@ def bench_attention(args, ring):
         seg, lens = _packed_segments(S, 4096, 0, dev)
         pairs = float(sum(l * (l + 1) / 2 for l in lens))
     kw = _kwargs(512, 512, 1)
+    pdrop = 0.1
+    if dropout:
+        # attention dropout: a fresh seed every step, so drawing and packing the mask is part of the step; only the
+        # pairs that are kept count as work
+        kw.update(deterministic=False, attn_pdrop=pdrop, dropout_rng=0)
+        pairs *= 1.0 - pdrop
     flops_fwd = 4.0 * D * pairs * B * H
     flops_bwd = 10.0 * D * pairs * B * H
+    seed = [0]
 
     def step():
         q.grad = k.grad = v.grad = None
+        seed[0] += 1
+        kws = dict(kw, dropout_rng=seed[0]) if dropout else kw
         with ra.ring_axis("sp", n):
-            out = ra.ringattention(q, k, v, bias, seg, None, axis_name="sp", float32_logits=True, blockwise_kwargs=kw)
+            out = ra.ringattention(q, k, v, bias, seg, None, axis_name="sp", float32_logits=True, blockwise_kwargs=kws)
             out.backward(do)
 
     ms = _time_steps(step, args.steps, args.warmup)
@@ -129,6 +140,7 @@ def bench_attention(args, ring):
             qd, kd, vd = q.detach(), k.detach(), v.detach()
             fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (num, den, mx), 0, 0, None, None, 1, 512, 512,
                                                       _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True)
+            fwd()            # under dropout the first call draws and packs the mask, which stays with mi
             kern["attn_fwd_ws_kernel"] = (_event_ms(fwd, 5), flops_fwd)
             out = torch.empty_like(qd)
             rh._finalize(num, den, out)
@@ -140,6 +152,12 @@ def bench_attention(args, ring):
                 bw = lambda: rh._blockwise_attention_bwd(qd, kd, vd, do, (dq, dk, dv, out, den, mx), 0, 0, None, None,
                                                          1, 512, 512, _mask_inputs=mi, _cfg=cfg1, _delta=delta)
                 kern["attn_bwd_%s_ws_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
+            if dropout:
+                def draw():
+                    m2 = rh._MaskInputs(cfg, None, None, None, B, q.device, S)
+                    m2.use_dropout(cfg, B, H, S, S, 0, 0, q.device)
+                del mi
+                mask_ms = _event_ms(draw, 3)
         dom = max(kern, key=lambda n_: kern[n_][0])
         dms, dfl = kern[dom]
         ach = dfl / (dms * 1e-3) / 1e12
@@ -148,13 +166,16 @@ def bench_attention(args, ring):
                 "traffic": MEASURED_TRAFFIC.get(dom) if S == 32768 else None,
                 "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
                 "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
-    cpu = cpu_baseline_attention() if not args.no_cpu else None
+        if dropout:
+            roof["traffic"] = None
+            roof["mask_draw_and_pack_ms"] = round(mask_ms, 3)
+    cpu = cpu_baseline_attention() if not (args.no_cpu or dropout) else None
     return {
         "metric": "attn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
         "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "config": {"workload": name, "B": B, "H": H, "S": S, "D": D, "causal_block_size": 1,
                    "query_chunk_size": 512, "key_chunk_size": 512, "virtual_ring": n,
-                   "segment_ids": bool(ring), "bias": bool(ring),
+                   "segment_ids": bool(ring), "bias": bool(ring), "attn_pdrop": pdrop if dropout else 0.0,
                    "flop_convention": "4*D fwd + 10*D bwd per unmasked (q,k) pair per head"},
         "roofline": roof, "cpu_baseline": cpu,
     }
@@ -478,7 +499,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm"])
+    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
+                                                              "dropout32k"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
@@ -489,8 +511,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
-    if args.workload in ("attn32k", "ring131k"):
-        r = bench_attention(args, ring=(args.workload == "ring131k"))
+    if args.workload in ("attn32k", "ring131k", "dropout32k"):
+        r = bench_attention(args, ring=(args.workload == "ring131k"), dropout=(args.workload == "dropout32k"))
     elif args.workload == "decode":
         r = bench_decode(args)
     elif args.workload == "copy":

@@ -823,9 +823,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
         float x = SC[(G) * 4 + e] * c;                                                                  \
         bool masked = (gk_tile + kr_ >= klim);                                                          \
         if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
-        if (HAS_KEEP == 2) {     /* dropout adds mask_min (:321): -inf where the pair was masked already */\
-          const bool off_ = !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                              \
-          x = (masked || off_) ? ((masked && off_) ? RA_NEG_INF : kMask2) : x;                          \
+        if (HAS_KEEP == 2) {                                                                            \
+          /* dropout adds mask_min (:321).  kw_cur: pairs kept and causally allowed; kw_some: at least  \
+             one of the two, so a clear bit there is mask_min added twice = -inf */                     \
+          x = ((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) ? x : kMask2;                                \
+          x = ((kw_some >> ((BLK) * 32 + (G) * 8 + e)) & 1) ? x : RA_NEG_INF;                           \
         } else {                                                                                        \
           if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);               \
           x = masked ? kMask2 : x;                                                                      \
@@ -879,7 +881,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     const int t_causal = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
     const uint64_t* kw_ptr = nullptr;
     const uint8_t* ks_ptr = nullptr;
-    uint64_t kw_cur = 0, kw_nxt = 0;
+    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0;
+    (void)kw_some;
     if (HAS_KEEP) {
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
                (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + (gk0 - mv.keep_k0) / 64;
@@ -932,6 +935,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     if (HAS_KEEP && (MASKED)) {        /* this tile's word; request the next tile's */                  \
       kw_cur = kw_nxt >> (4 * hi);                                                                      \
       kw_nxt = kw_ptr[(int64_t)min(t + 1 == t_a ? t_b : t + 1, ntiles - 1) * mv.keep_Q];                \
+      if (HAS_KEEP == 2) {             /* fold this row's causal limit into the words */                \
+        const int nall_ = max(0, min(64, klim - gk_tile));                                              \
+        const uint64_t cw_ = (nall_ >= 64 ? ~0ULL : ((1ULL << nall_) - 1ULL)) >> (4 * hi);              \
+        kw_some = kw_cur | cw_;                                                                         \
+        kw_cur &= cw_;                                                                                  \
+      }                                                                                                 \
     }                                                                                                   \
     /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
     RA_TRACE_MARK();                                                                                    \
