@@ -74,7 +74,8 @@ typedef struct ra_mask {
                                  dropped): mask_min is ADDED to the logit and its bias, so the logit becomes mask_min,
                                  or -inf where segment ids or the causal mask had already set it to mask_min.
                                  Indexed by the LOCAL query row of the call and by the GLOBAL key position minus
-                                 keep_k0; only the generic kernels take this byte form */
+                                 keep_k0; only the generic kernels take this byte form (they read the packed
+                                 form below when keep is null) */
   int64_t keep_stride_b;      /* element (byte) strides; 0 broadcasts that axis */
   int64_t keep_stride_h;
   int64_t keep_stride_q;
@@ -148,14 +149,20 @@ int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_
 /* The attention dropout mask of ringattention_jax.py:119-121 / :206-208 (jax.random.bernoulli(rng, attn_pdrop,
  * (batch, heads, q_len, kv_len)), true = dropped), written as the boolean KEEP mask ra_mask.keep takes with
  * RA_KEEP_DROPOUT: keep (B, H, Q, K) dense bytes, 1 = attend, 0 = dropped.  The bits do not come from the
- * jax.random stream (threefry, not restated) but from Philox4x32-10 (Salmon et al., SC'11), one block per four
- * consecutive key positions:
- *   e = ((b * H + h) * Q + q) * K + k          (position in the dense mask; K is a multiple of 4)
- *   block = philox4x32_10(counter = (lo32(e / 4), hi32(e / 4), 0, 0), key = (lo32(seed), hi32(seed)))
- *   dropped(e) = block[e % 4] < floor(attn_pdrop * 2^32)
+ * jax.random stream (threefry, not restated) but from Philox4x32-10 (Salmon et al., SC'11), 16 bits a position,
+ * one block per eight consecutive key positions:
+ *   e = ((b * H + h) * Q + q) * K + k          (position in the dense mask; K is a multiple of 8)
+ *   block = philox4x32_10(counter = (lo32(e / 8), hi32(e / 8), 0, 0), key = (lo32(seed), hi32(seed)))
+ *   half  = e % 8;  r = 16 bits of block[half / 2]: the low half for even half, the high half for odd
+ *   dropped(e) = r < floor(attn_pdrop * 2^16)
  * so the mask is a pure function of (seed, attn_pdrop, shape); forward and backward pass take the same array. */
 int ra_dropout_keep(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K, uint8_t* keep,
                     ra_stream_t stream);
+/* The same mask written directly in the packed form of ra_keep_pack (Q and K multiples of 64), without the byte
+ * array: what ra_keep_pack would make of ra_dropout_keep's output.  The attention entry points take the packed
+ * form alone (ra_mask.keep null). */
+int ra_dropout_keep_packed(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K,
+                           uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, ra_stream_t stream);
 
 /* Carry initialisation (ringattention_jax.py:22-23,:49): numerator = 0, denominator = 0, max = -inf. */
 int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s,

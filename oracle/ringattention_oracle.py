@@ -36,7 +36,7 @@ vectors, and JAX/flax are not importable where this was written):
   of local shape) is restated and checked against ``dense_attention`` with the same mask, against the
   exact-zero weight of dropped keys and against a hand-enumerated row whose every allowed key is dropped.
   The mask BITS are not the reference's: ``jax.random`` (threefry) is not restated; ``dropout_mask``
-  draws from Philox4x32-10, pinned by the known-answer vectors of the Random123 distribution.
+  draws 16 bits a position from Philox4x32-10, pinned by the known-answer vectors of the Random123 distribution.
 
 Parity unpinned (would need the reference's own runtime): the dropout mask
 bits of the ``jax.random`` stream (replaced by the documented Philox stream above) and XLA-CPU's exact
@@ -95,17 +95,18 @@ def philox4x32_10(counter, key):
 def dropout_mask(seed, attn_pdrop, shape):
     """The boolean mask of ringattention_jax.py:120-121 / :207-208 (True = dropped, probability attn_pdrop)
     of shape (batch, heads, q_len, kv_len), from the documented Philox stream instead of jax.random:
-    position e of the dense mask takes word e % 4 of block e // 4, keyed by the 64-bit seed; dropped iff
-    the word is below floor(float32(attn_pdrop) * 2^32)."""
+    position e of the dense mask takes 16 bits, half-word e % 8 of block e // 8 (word (e % 8) // 2, low half
+    first), keyed by the 64-bit seed; dropped iff they are below floor(float32(attn_pdrop) * 2^16)."""
     n = int(np.prod(shape))
-    assert shape[-1] % 4 == 0
-    blk = np.arange(n // 4, dtype=np.uint64)
+    assert shape[-1] % 8 == 0
+    blk = np.arange(n // 8, dtype=np.uint64)
     counter = np.stack([blk & np.uint64(0xFFFFFFFF), blk >> np.uint64(32), np.zeros_like(blk), np.zeros_like(blk)],
                        axis=-1)
     key = np.array([seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF], dtype=np.uint64)
-    words = philox4x32_10(counter, np.broadcast_to(key, (n // 4, 2))).reshape(n)
-    threshold = int(float(np.float32(attn_pdrop)) * 4294967296.0)
-    return torch.from_numpy((words.astype(np.uint64) < np.uint64(threshold)).reshape(shape))
+    words = philox4x32_10(counter, np.broadcast_to(key, (n // 8, 2)))                 # (n / 8, 4)
+    halves = np.stack([words & np.uint32(0xFFFF), words >> np.uint32(16)], axis=-1).reshape(n)
+    threshold = int(float(np.float32(attn_pdrop)) * 65536.0)
+    return torch.from_numpy((halves < np.uint32(threshold)).reshape(shape))
 
 
 def chunk_attention_bias(query_chunk_size, key_chunk_size, bias, segment_ids,

@@ -29,6 +29,8 @@ int bwd_delta(const void*, const void*, int, int64_t, int64_t, float*, int64_t, 
 int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
 int keep_pack(const uint8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, uint64_t*, uint64_t*, uint8_t*, hipStream_t);
 int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hipStream_t s);
+int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, int K, uint64_t* bits_k,
+                        uint64_t* bits_q, uint8_t* summary, hipStream_t s);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
@@ -61,8 +63,8 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
     RA_REQUIRE(m.segment_ids && m.seg_tiles == (m.seg_len + RA_SEG_TILE - 1) / RA_SEG_TILE, RA_ERR_INVALID,
                "%s: seg_tile_minmax needs segment_ids and seg_tiles == ceil(seg_len / %d)", who, (int)RA_SEG_TILE);
   if (m.keep_bits_k || m.keep_bits_q || m.keep_summary) {
-    RA_REQUIRE(m.keep && m.keep_bits_k && m.keep_bits_q && m.keep_summary, RA_ERR_INVALID,
-               "%s: the packed keep mask needs keep, keep_bits_k, keep_bits_q and keep_summary together", who);
+    RA_REQUIRE(m.keep_bits_k && m.keep_bits_q && m.keep_summary, RA_ERR_INVALID,
+               "%s: the packed keep mask needs keep_bits_k, keep_bits_q and keep_summary together", who);
     RA_REQUIRE(m.keep_q_total > 0 && m.keep_k_total > 0 && m.keep_q_total % 64 == 0 && m.keep_k_total % 64 == 0 &&
                    m.keep_q0 >= 0 && m.keep_q0 % 64 == 0 && m.keep_q0 + Sq <= m.keep_q_total &&
                    m.keep_k0 >= 0 && m.keep_k0 % 64 == 0 &&
@@ -70,7 +72,7 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
                    (long long)m.k_chunk_idx_start * m.key_chunk_size - m.keep_k0 + Skv <= m.keep_k_total,
                RA_ERR_INVALID, "%s: packed keep mask does not cover the rows / keys of the call", who);
   }
-  if (m.keep) {
+  if (m.keep || m.keep_bits_k) {
     RA_REQUIRE(m.keep_mode == RA_KEEP_WHERE || m.keep_mode == RA_KEEP_DROPOUT, RA_ERR_INVALID,
                "%s: keep_mode must be RA_KEEP_WHERE or RA_KEEP_DROPOUT", who);
     RA_REQUIRE(m.keep_k0 >= 0 && (long long)m.k_chunk_idx_start * m.key_chunk_size >= m.keep_k0, RA_ERR_INVALID,
@@ -163,17 +165,30 @@ int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_
                    (hipStream_t)stream);
 }
 
+static uint32_t dropout_threshold(float attn_pdrop) { return (uint32_t)((double)attn_pdrop * 65536.0); }   // floor
+
 int ra_dropout_keep(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K, uint8_t* keep,
                     ra_stream_t stream) {
   RA_REQUIRE(keep, RA_ERR_INVALID, "dropout_keep: null pointer");
-  RA_REQUIRE(((uintptr_t)keep % 16) == 0, RA_ERR_UNSUPPORTED, "dropout_keep: keep must be 16-byte aligned");
+  RA_REQUIRE(((uintptr_t)keep % 8) == 0, RA_ERR_UNSUPPORTED, "dropout_keep: keep must be 8-byte aligned");
   RA_REQUIRE(B > 0 && H > 0 && Q > 0 && K > 0, RA_ERR_INVALID, "dropout_keep: empty shape");
-  RA_REQUIRE(K % 4 == 0, RA_ERR_UNSUPPORTED, "dropout_keep: K must be a multiple of 4 (got %d)", K);
+  RA_REQUIRE(K % 8 == 0, RA_ERR_UNSUPPORTED, "dropout_keep: K must be a multiple of 8 (got %d)", K);
   RA_REQUIRE(attn_pdrop > 0.f && attn_pdrop < 1.f, RA_ERR_INVALID, "dropout_keep: attn_pdrop must lie in (0, 1)");
   const int64_t n = (int64_t)B * H * Q * K;
   RA_REQUIRE(n / 16 / 256 < (1LL << 31), RA_ERR_UNSUPPORTED, "dropout_keep: mask too large");
-  const uint32_t threshold = (uint32_t)((double)attn_pdrop * 4294967296.0);     // floor; < 2^32 since p < 1
-  return dropout_keep(seed, threshold, n, keep, (hipStream_t)stream);
+  return dropout_keep(seed, dropout_threshold(attn_pdrop), n, keep, (hipStream_t)stream);
+}
+
+int ra_dropout_keep_packed(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K,
+                           uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, ra_stream_t stream) {
+  RA_REQUIRE(bits_k && bits_q && summary, RA_ERR_INVALID, "dropout_keep_packed: null pointer");
+  RA_REQUIRE(B > 0 && H > 0 && (long long)B * H <= 65535, RA_ERR_INVALID, "dropout_keep_packed: bad plane count");
+  RA_REQUIRE(Q > 0 && K > 0 && Q % 64 == 0 && K % 64 == 0 && Q / 64 <= 65535, RA_ERR_UNSUPPORTED,
+             "dropout_keep_packed: Q and K must be positive multiples of 64 (got %d, %d)", Q, K);
+  RA_REQUIRE(attn_pdrop > 0.f && attn_pdrop < 1.f, RA_ERR_INVALID,
+             "dropout_keep_packed: attn_pdrop must lie in (0, 1)");
+  return dropout_keep_packed(seed, dropout_threshold(attn_pdrop), B * H, Q, K, bits_k, bits_q, summary,
+                             (hipStream_t)stream);
 }
 
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
@@ -244,7 +259,7 @@ int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->mask.query_chunk_size == 1, RA_ERR_INVALID,
              "decode_fwd: one query token needs query_chunk_size == 1 (q_len // query_chunk_size chunks)");
   if (int rc = check_mask(p->mask, 1, p->L, "decode_fwd")) return rc;
-  RA_REQUIRE(p->mask.keep == nullptr, RA_ERR_UNSUPPORTED, "decode_fwd: the boolean keep mask is taken by the generic attention kernels only");
+  RA_REQUIRE(p->mask.keep == nullptr && p->mask.keep_bits_k == nullptr, RA_ERR_UNSUPPORTED, "decode_fwd: the boolean keep mask is taken by the generic attention kernels only");
   int ns = p->num_splits > 0 ? p->num_splits : decode_pick_splits(p->B, p->L, p->H, p->D, p->dtype);
   RA_REQUIRE(ns <= 256, RA_ERR_INVALID, "decode_fwd: num_splits %d > 256", ns);
   size_t need = (size_t)p->B * p->H * ns * (p->D + 2) * sizeof(float);

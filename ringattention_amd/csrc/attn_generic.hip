@@ -37,6 +37,7 @@ struct RowInfo {
   int seg;
   int64_t bias_off;
   int64_t keep_off;
+  int64_t kbit_off;
 };
 
 __device__ __forceinline__ RowInfo row_info(const MaskView& mv, int b, int h, int row, int skv) {
@@ -52,6 +53,7 @@ __device__ __forceinline__ RowInfo row_info(const MaskView& mv, int b, int h, in
   }
   r.bias_off = (int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)(row % mv.qc) * mv.bias_sq;
   r.keep_off = (int64_t)b * mv.keep_sb + (int64_t)h * mv.keep_sh + (int64_t)row * mv.keep_sq;
+  r.kbit_off = (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh + mv.keep_q0 + row;
   return r;
 }
 
@@ -66,7 +68,13 @@ __device__ __forceinline__ float logit(const MaskView& mv, const RowInfo& r, flo
     if (mv.any_mask) add = fminf(add, 0.f);                       // minimum(), :299,:309
   }
   bool masked = (mv.cbs > 0 && r.gq_blk < gk / mv.cbs) || (mv.seg && r.seg != seg_k);
-  const bool off = mv.keep && !mv.keep[r.keep_off + (gk - mv.keep_k0) * mv.keep_sk];
+  bool off = false;
+  if (mv.keep) {
+    off = !mv.keep[r.keep_off + (gk - mv.keep_k0) * mv.keep_sk];
+  } else if (mv.kbits_k) {            // packed form only: bit (gk - keep_k0) % 64 of the row's word of that key tile
+    const long long kk = gk - mv.keep_k0;
+    off = !((mv.kbits_k[r.kbit_off + (kk >> 6) * mv.keep_Q] >> (kk & 63)) & 1);
+  }
   if (off && mv.keep_drop) {
     // chunk_bias += dropped * finfo.min (:321): twice finfo.min overflows to -inf, once absorbs logit and bias
     return masked ? RA_NEG_INF : mv.mask_min;
@@ -432,32 +440,73 @@ __host__ __device__ inline philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
   return philox4{{c0, c1, c2, c3}};
 }
 
-// keep[e] = philox(block e / 4)[e % 4] >= threshold, over the dense (B, H, Q, K) mask: one thread per 16 positions
-__global__ __launch_bounds__(256) void dropout_keep_kernel(uint32_t k0, uint32_t k1, uint32_t threshold,
-                                                           int64_t nblocks, uint32_t* keep4) {
-  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  uint32_t w[4];
+// Position e of the dense (B, H, Q, K) mask takes 16 bits: half-word e % 8 of Philox block e / 8 (word (e % 8) / 2, low
+// half first); it is dropped iff that half-word is below threshold = floor(attn_pdrop * 2^16).
+__device__ __forceinline__ uint32_t philox_keep8(int64_t blk, uint32_t k0, uint32_t k1, uint32_t threshold) {
+  const philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)((uint64_t)blk >> 32), 0u, 0u, k0, k1);
+  uint32_t bits = 0;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
-    const int64_t blk = 4 * t + j;
-    const philox4 r = philox4x32_10((uint32_t)blk, (uint32_t)((uint64_t)blk >> 32), 0u, 0u, k0, k1);
-    w[j] = (r.v[0] >= threshold ? 1u : 0u) | (r.v[1] >= threshold ? 1u << 8 : 0u) |
-           (r.v[2] >= threshold ? 1u << 16 : 0u) | (r.v[3] >= threshold ? 1u << 24 : 0u);
+    bits |= ((r.v[j] & 0xFFFFu) >= threshold ? 1u : 0u) << (2 * j);
+    bits |= ((r.v[j] >> 16) >= threshold ? 1u : 0u) << (2 * j + 1);
   }
-  if (4 * t + 3 < nblocks) {
-    *(uint4*)(keep4 + 4 * t) = uint4{w[0], w[1], w[2], w[3]};
-  } else {
+  return bits;      // bit i: position 8 blk + i is kept
+}
+
+// byte form: one thread per 16 positions (two blocks)
+__global__ __launch_bounds__(256) void dropout_keep_kernel(uint32_t k0, uint32_t k1, uint32_t threshold,
+                                                           int64_t nblocks, uint2* keep8) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-      if (4 * t + j < nblocks) keep4[4 * t + j] = w[j];
+  for (int j = 0; j < 2; j++) {
+    const int64_t blk = 2 * t + j;
+    if (blk >= nblocks) return;
+    const uint32_t bits = philox_keep8(blk, k0, k1, threshold);
+    uint2 w;
+    w.x = (bits & 1u) | ((bits >> 1 & 1u) << 8) | ((bits >> 2 & 1u) << 16) | ((bits >> 3 & 1u) << 24);
+    w.y = (bits >> 4 & 1u) | ((bits >> 5 & 1u) << 8) | ((bits >> 6 & 1u) << 16) | ((bits >> 7 & 1u) << 24);
+    keep8[blk] = w;
   }
 }
 
 int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hipStream_t s) {
-  const int64_t nblocks = n / 4, nthreads = (nblocks + 3) / 4;
+  const int64_t nblocks = n / 8, nthreads = (nblocks + 1) / 2;
   dropout_keep_kernel<<<(unsigned)((nthreads + 255) / 256), 256, 0, s>>>((uint32_t)seed, (uint32_t)(seed >> 32),
-                                                                        threshold, nblocks, (uint32_t*)keep);
+                                                                        threshold, nblocks, (uint2*)keep);
   RA_CHECK_LAUNCH("dropout_keep");
+  return RA_OK;
+}
+
+// packed form, the same bits: one 64 x 64 tile per wavefront, lane i draws the 64 positions of query row i (eight
+// blocks) and the columns' words come from 64 ballots.  Writes what keep_pack_kernel would write for the byte form.
+__global__ __launch_bounds__(64) void dropout_keep_packed_kernel(uint32_t k0, uint32_t k1, uint32_t threshold, int Q,
+                                                                 int K, uint64_t* bits_k, uint64_t* bits_q,
+                                                                 uint8_t* summary) {
+  const int kt = blockIdx.x, qt = blockIdx.y, plane = blockIdx.z, i = threadIdx.x;
+  const int64_t e0 = ((int64_t)plane * Q + qt * 64 + i) * K + (int64_t)kt * 64;
+  uint64_t wrow = 0;
+#pragma unroll
+  for (int j = 0; j < 8; j++) wrow |= (uint64_t)philox_keep8(e0 / 8 + j, k0, k1, threshold) << (8 * j);
+  uint64_t wcol = 0;
+  for (int j = 0; j < 64; j++) {
+    const unsigned long long m = __builtin_amdgcn_ballot_w64((wrow >> j) & 1);
+    if (i == j) wcol = m;
+  }
+  int cnt = __popcll(wrow);
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+  const int64_t words = (int64_t)Q * K / 64;
+  bits_k[plane * words + (int64_t)kt * Q + qt * 64 + i] = wrow;
+  bits_q[plane * words + (int64_t)qt * K + kt * 64 + i] = wcol;
+  if (i == 0)
+    summary[(int64_t)plane * (Q / 64) * (K / 64) + (int64_t)qt * (K / 64) + kt] = cnt == 0 ? 0 : (cnt == 4096 ? 2 : 1);
+}
+
+int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, int K, uint64_t* bits_k,
+                        uint64_t* bits_q, uint8_t* summary, hipStream_t s) {
+  dim3 grid(K / 64, Q / 64, planes);
+  dropout_keep_packed_kernel<<<grid, 64, 0, s>>>((uint32_t)seed, (uint32_t)(seed >> 32), threshold, Q, K, bits_k,
+                                                 bits_q, summary);
+  RA_CHECK_LAUNCH("dropout_keep_packed");
   return RA_OK;
 }
 

@@ -401,9 +401,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       float x = SC[(G) * 4 + e] * c;                                                                    \
       bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
       if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
-      if (HAS_KEEP == 2) {     /* dropout adds mask_min (:321): -inf where the pair was masked already */\
-        const bool off_ = !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                                \
-        x = (masked || off_) ? ((masked && off_) ? RA_NEG_INF : kMask2) : x;                            \
+      if (HAS_KEEP == 2) {                                                                              \
+        /* dropout adds mask_min (:321).  kw_cur: pairs kept and causally allowed; kw_some: at least    \
+           one of the two, so a clear bit there is mask_min added twice = -inf */                       \
+        x = ((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) ? x : kMask2;                                  \
+        x = ((kw_some >> ((BLK) * 32 + (G) * 8 + e)) & 1) ? x : RA_NEG_INF;                             \
       } else {                                                                                          \
         if (HAS_KEEP) masked = masked || !((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1);                 \
         x = masked ? kMask2 : x;                                                                        \
@@ -450,7 +452,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     // packed keep mask: this lane's word (bits over the 64 rows of a query tile) and this pair's summary byte
     const uint64_t* kw_ptr = nullptr;
     const uint8_t* ks_ptr = nullptr;
-    uint64_t kw_cur = 0, kw_nxt = 0;
+    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0;
+    (void)kw_some;
     int ks_cur = 2, ks_nxt = 2;
     if (HAS_KEEP) {
       kw_ptr = mv.kbits_q + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
@@ -492,6 +495,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
         kw_cur = kw_nxt >> (4 * hi); ks_cur = ks_nxt;
         const int tn = min(t + 1, ntq - 1);
         kw_nxt = kw_ptr[(int64_t)tn * mv.keep_K]; ks_nxt = ks_ptr[(int64_t)tn * (mv.keep_K / 64)];
+        if (HAS_KEEP == 2) {               // fold this key's causal limit (rows before qlim are masked) into the words
+          const int nmask = (int)max(0LL, min(64LL, (long long)qlim - gq_tile));
+          const uint64_t cw = (nmask >= 64 ? 0ULL : (~0ULL << nmask)) >> (4 * hi);
+          kw_some = kw_cur | cw;
+          kw_cur &= cw;
+        }
       }
       // step 2t: vector work of block 0 of tile t, products of block 1
       if ((HAS_SEG && !sp_cur) || (gq_tile < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
@@ -1285,9 +1294,11 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
         float x_ = SC[r] * c;                                                                           \
         bool masked_ = (gk_tile + kr_ >= klim);                                                         \
         if (HAS_SEG) masked_ = masked_ || (seg_ks[BUF][kr_] != seg_q);                                  \
-        if (HAS_KEEP == 2) {     /* dropout adds mask_min (:321): -inf where the pair was masked already */\
-          const bool off_ = !((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1);                   \
-          x_ = (masked_ || off_) ? ((masked_ && off_) ? RA_NEG_INF : kMask2) : x_;                      \
+        if (HAS_KEEP == 2) {                                                                            \
+          /* dropout adds mask_min (:321).  kw_cur: pairs kept and causally allowed; kw_some: at least  \
+             one of the two, so a clear bit there is mask_min added twice = -inf */                     \
+          x_ = ((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) ? x_ : kMask2;                   \
+          x_ = ((kw_some >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) ? x_ : RA_NEG_INF;              \
         } else {                                                                                        \
           if (HAS_KEEP) masked_ = masked_ || !((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1);  \
           x_ = masked_ ? kMask2 : x_;                                                                   \
@@ -1355,7 +1366,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const int t_causal = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
     const uint64_t* kw_ptr = nullptr;
     const uint8_t* ks_ptr = nullptr;
-    uint64_t kw_cur = 0, kw_nxt = 0;
+    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0;
+    (void)kw_some;
     if (HAS_KEEP) {
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
                (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + (gk0 - mv.keep_k0) / 64;
@@ -1408,6 +1420,12 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     if (HAS_KEEP && (MASKED)) {        /* this tile's word; request the next tile's */                  \
       kw_cur = kw_nxt >> (4 * hi);                                                                      \
       kw_nxt = kw_ptr[(int64_t)min(t + 1 == t_a ? t_b : t + 1, ntiles - 1) * mv.keep_Q];                \
+      if (HAS_KEEP == 2) {             /* fold this row's causal limit into the words */                \
+        const int nall_ = max(0, min(64, klim - gk_tile));                                              \
+        const uint64_t cw_ = (nall_ >= 64 ? ~0ULL : ((1ULL << nall_) - 1ULL)) >> (4 * hi);              \
+        kw_some = kw_cur | cw_;                                                                         \
+        kw_cur &= cw_;                                                                                  \
+      }                                                                                                 \
     }                                                                                                   \
     /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
     RA_TRACE_MARK();                                                                                    \
@@ -1565,7 +1583,7 @@ static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 // a boolean keep mask is taken in packed form only, next to a causal block size at most (no bias or segment ids:
 // ring_attention_inference has neither, and the generic kernels serve any combination)
 static bool keep_ok(const ra_mask& m) {
-  if (!m.keep) return true;
+  if (!m.keep && !m.keep_bits_k) return true;
   return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids;
 }
 
@@ -1588,7 +1606,7 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
-  const bool keep = p->mask.keep != nullptr;      // packed form checked by attn_fwd_mfma_supported
+  const bool keep = p->mask.keep_bits_k != nullptr;      // packed form checked by attn_fwd_mfma_supported
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
   RA_REQUIRE(nwg3 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
   dim3 grid3((unsigned)((nwg3 + 7) / 8 * 8)), block3(512);
@@ -1632,8 +1650,8 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
     if (do_dkv) attn_bwd_dkv_ws_kernel<__VA_ARGS__><<<gk, block, 0, s>>>(a);             \
     if (do_dq) attn_bwd_dq_ws_kernel<__VA_ARGS__><<<gq, block, 0, s>>>(a);               \
   } while (0)
-  if (p->mask.keep && p->mask.keep_mode == RA_KEEP_DROPOUT) RA_LAUNCH_BWD(false, false, 2);
-  else if (p->mask.keep) RA_LAUNCH_BWD(false, false, 1);      // packed boolean mask
+  if (p->mask.keep_bits_k && p->mask.keep_mode == RA_KEEP_DROPOUT) RA_LAUNCH_BWD(false, false, 2);
+  else if (p->mask.keep_bits_k) RA_LAUNCH_BWD(false, false, 1);      // packed boolean mask
   else if (seg && bias) RA_LAUNCH_BWD(true, true);
   else if (seg) RA_LAUNCH_BWD(true, false);
   else if (bias) RA_LAUNCH_BWD(false, true);

@@ -185,7 +185,8 @@ class _MaskInputs:
         self.keep_k0 = 0
         self.keep_mode = L.RA_KEEP_WHERE
         self.keep_packed = None
-        self._drop_base = None             # (B, H, q_len, kv_len) keep bytes of the dropout mask
+        self._drop_base = None             # (B, H, q_len, kv_len) keep bytes of the dropout mask, if needed
+        self._drop_shape = None
         self._drop_steps = {}
         self.cache_idx_host = None
         self.cache_idx_dev = None
@@ -247,19 +248,32 @@ class _MaskInputs:
         it is; every other start is served by a gathered copy, cached per (row start, key start)."""
         if self.cache_idx_host is not None or self.cache_idx_dev is not None:
             raise NotImplementedError("attention dropout together with cache_idx is not supported")
-        if kv_len % 4:
-            raise NotImplementedError("attention dropout needs a key length that is a multiple of 4")
+        if kv_len % 8:
+            raise NotImplementedError("attention dropout needs a key length that is a multiple of 8")
         shape = (batch, heads, q_len, kv_len)
-        if self._drop_base is None:
-            base = torch.empty(shape, dtype=torch.uint8, device=device)
-            L.check(L.load().ra_dropout_keep(cfg.seed, cfg.pdrop, batch, heads, q_len, kv_len, base.data_ptr(),
-                                             _stream()), "ra_dropout_keep")
-            self._drop_base = base
-        elif tuple(self._drop_base.shape) != shape:
+        if self._drop_shape is None:
+            self._drop_shape = shape
+        elif self._drop_shape != shape:
             raise ValueError("the dropout mask of this call was drawn for another shape")
         nq, nk = q_len // cfg.qc, kv_len // cfg.kc
         key = (min(q_chunk_idx_start, nq), min(k_chunk_idx_start, nk))
+        aligned = q_len % 64 == 0 and kv_len % 64 == 0
+        if key not in self._drop_steps and key == (0, 0) and aligned:
+            # the mask as drawn, written in packed form at once (no byte array: the kernels read the words)
+            words = q_len * kv_len // 64
+            bits_k = torch.empty((batch, heads, words), dtype=torch.int64, device=device)
+            bits_q = torch.empty((batch, heads, words), dtype=torch.int64, device=device)
+            summ = torch.empty((batch, heads, words // 64), dtype=torch.uint8, device=device)
+            L.check(L.load().ra_dropout_keep_packed(cfg.seed, cfg.pdrop, batch, heads, q_len, kv_len,
+                                                    bits_k.data_ptr(), bits_q.data_ptr(), summ.data_ptr(),
+                                                    _stream()), "ra_dropout_keep_packed")
+            self._drop_steps[key] = (None, (bits_k, bits_q, summ, q_len, kv_len))
         if key not in self._drop_steps:
+            if self._drop_base is None:
+                base = torch.empty(shape, dtype=torch.uint8, device=device)
+                L.check(L.load().ra_dropout_keep(cfg.seed, cfg.pdrop, batch, heads, q_len, kv_len, base.data_ptr(),
+                                                 _stream()), "ra_dropout_keep")
+                self._drop_base = base
             m = self._drop_base
             if key[0] != 0:
                 starts = torch.clamp((key[0] + torch.arange(nq, device=device)) * cfg.qc, max=q_len - cfg.qc)
@@ -268,11 +282,12 @@ class _MaskInputs:
                 starts = torch.clamp((key[1] + torch.arange(nk, device=device)) * cfg.kc, max=kv_len - cfg.kc)
                 m = m.index_select(3, (starts[:, None] + torch.arange(cfg.kc, device=device)).reshape(-1))
             packed = None
-            if q_len % 64 == 0 and kv_len % 64 == 0:
+            if aligned:
                 packed = self._pack(m, m.stride(), q_len, kv_len) + (q_len, kv_len)
+                m = None if key != (0, 0) else m          # the gathered bytes are not needed once packed
             self._drop_steps[key] = (m, packed)
         self.keep, self.keep_packed = self._drop_steps[key]
-        self.keep_strides = self.keep.stride()
+        self.keep_strides = self.keep.stride() if self.keep is not None else (0, 0, 0, 0)
         self.keep_row0 = 0
         self.keep_k0 = k_chunk_idx_start * cfg.kc
         self.keep_mode = L.RA_KEEP_DROPOUT
@@ -294,9 +309,10 @@ class _MaskInputs:
         m.skip_masked_tiles = 1 if skip else 0
         m.seg_tile_minmax = self.seg_mm.data_ptr() if self.seg_mm is not None else None
         m.seg_tiles = self.seg_tiles
-        if self.keep is not None:
-            m.keep = self.keep.data_ptr() + self.keep_row0 * self.keep_strides[2]
-            m.keep_stride_b, m.keep_stride_h, m.keep_stride_q, m.keep_stride_k = self.keep_strides
+        if self.keep is not None or self.keep_packed is not None:
+            if self.keep is not None:
+                m.keep = self.keep.data_ptr() + self.keep_row0 * self.keep_strides[2]
+                m.keep_stride_b, m.keep_stride_h, m.keep_stride_q, m.keep_stride_k = self.keep_strides
             if self.keep_packed is not None:
                 bits_k, bits_q, summ, q_total, k_total = self.keep_packed
                 m.keep_bits_k, m.keep_bits_q, m.keep_summary = bits_k.data_ptr(), bits_q.data_ptr(), summ.data_ptr()

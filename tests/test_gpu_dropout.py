@@ -18,8 +18,8 @@ DEV = "cuda"
 @pytest.mark.parametrize("shape,seed,p", [
     ((1, 1, 4, 8), 0, 0.5),
     ((2, 3, 64, 128), 1234, 0.1),
-    ((1, 2, 100, 36), (1 << 40) + 17, 0.25),       # not a multiple of 16 positions: the tail of the last thread
-    ((1, 1, 256, 4100), 0xFFFFFFFFFFFFFFFF, 0.9),
+    ((1, 2, 100, 40), (1 << 40) + 17, 0.25),       # an odd number of blocks: the tail of the last thread
+    ((1, 1, 256, 4104), 0xFFFFFFFFFFFFFFFF, 0.9),
 ])
 def test_dropout_mask_bits_are_the_documented_philox_stream(shape, seed, p):
     keep = torch.empty(shape, dtype=torch.uint8, device=DEV)
@@ -31,10 +31,30 @@ def test_dropout_mask_bits_are_the_documented_philox_stream(shape, seed, p):
         assert abs(float(dropped.float().mean()) - p) < 0.02
 
 
+@pytest.mark.parametrize("shape,seed,p", [((2, 3, 128, 192), 77, 0.3), ((1, 1, 64, 64), 1, 0.999), ((1, 2, 64, 128), 2, 1e-5)])
+def test_packed_dropout_mask_equals_packing_the_byte_mask(shape, seed, p):
+    B, H, Q, K = shape
+    lib = L.load()
+    keep = torch.empty(shape, dtype=torch.uint8, device=DEV)
+    L.check(lib.ra_dropout_keep(seed, p, B, H, Q, K, keep.data_ptr(), None), "ra_dropout_keep")
+    words = Q * K // 64
+    mk = lambda: (torch.zeros((B, H, words), dtype=torch.int64, device=DEV),
+                  torch.zeros((B, H, words), dtype=torch.int64, device=DEV),
+                  torch.full((B, H, words // 64), 9, dtype=torch.uint8, device=DEV))
+    a, b = mk(), mk()
+    L.check(lib.ra_keep_pack(keep.data_ptr(), keep.stride(0), keep.stride(1), keep.stride(2), keep.stride(3), B, H, Q,
+                             K, a[0].data_ptr(), a[1].data_ptr(), a[2].data_ptr(), None), "ra_keep_pack")
+    L.check(lib.ra_dropout_keep_packed(seed, p, B, H, Q, K, b[0].data_ptr(), b[1].data_ptr(), b[2].data_ptr(), None),
+            "ra_dropout_keep_packed")
+    torch.cuda.synchronize()
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
 def test_dropout_mask_rejects():
     lib = L.load()
     keep = torch.empty(64, dtype=torch.uint8, device=DEV)
-    assert lib.ra_dropout_keep(0, 0.5, 1, 1, 8, 6, keep.data_ptr(), None) == L.RA_ERR_UNSUPPORTED     # K % 4
+    assert lib.ra_dropout_keep(0, 0.5, 1, 1, 8, 12, keep.data_ptr(), None) == L.RA_ERR_UNSUPPORTED    # K % 8
     assert lib.ra_dropout_keep(0, 0.0, 1, 1, 8, 8, keep.data_ptr(), None) == L.RA_ERR_INVALID
     assert lib.ra_dropout_keep(0, 1.0, 1, 1, 8, 8, keep.data_ptr(), None) == L.RA_ERR_INVALID
     assert lib.ra_dropout_keep(0, 0.5, 1, 1, 8, 8, None, None) == L.RA_ERR_INVALID
