@@ -18,8 +18,9 @@ from oracle import ringattention_oracle as O   # noqa: E402
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def kwargs(qc, kc, cbs):
-    return dict(causal_block_size=cbs, deterministic=True, dropout_rng=None, attn_pdrop=0.0, query_chunk_size=qc,
+def kwargs(qc, kc, cbs, drop_permille=0, seed=None):
+    return dict(causal_block_size=cbs, deterministic=drop_permille == 0, dropout_rng=seed,
+                attn_pdrop=drop_permille / 1000.0, query_chunk_size=qc,
                 key_chunk_size=kc, dtype=torch.float32, policy=None, precision=None, prevent_cse=True)
 
 
@@ -46,6 +47,10 @@ def cases():
     seg = torch.tensor([[0] * 20 + [1] * 25 + [2] * 19], dtype=torch.int32)
     out["ring2_causal_bias_segments"] = (dict(q=q, k=k, v=v, do=do, bias=bias, seg=seg), dict(qc=16, kc=16, cbs=1, n=2))
     out["one_device_causal_block4"] = (dict(q=q, k=k, v=v, do=do), dict(qc=8, kc=16, cbs=4, n=1))
+    # attention dropout (rate 0.3, the documented Philox stream seeded with 1234), two devices: the second one
+    # reads the mask through the clamped slices
+    out["ring2_causal_dropout"] = (dict(q=q, k=k, v=v, do=do), dict(qc=16, kc=16, cbs=1, n=2, drop_permille=300,
+                                                                    seed=1234))
     qd = bf16_exact(torch.randn(2, 1, H, D, generator=g))
     kd, vd = bf16_exact(torch.randn(2, 96, H, D, generator=g)), bf16_exact(torch.randn(2, 96, H, D, generator=g))
     out["decode_cache_idx_70"] = (dict(q=qd, k=kd, v=vd), dict(qc=1, kc=32, cbs=1, n=1, cache_idx=70))
@@ -53,7 +58,7 @@ def cases():
 
 
 def run_case(inp, cfg):
-    kw = kwargs(cfg["qc"], cfg["kc"], cfg["cbs"])
+    kw = kwargs(cfg["qc"], cfg["kc"], cfg["cbs"], cfg.get("drop_permille", 0), cfg.get("seed"))
     out, res = O.ring_attention_fwd(inp["q"], inp["k"], inp["v"], inp.get("bias"), inp.get("seg"), cfg.get("cache_idx"),
                                     cfg["n"], True, kw)
     r = {"out": out}

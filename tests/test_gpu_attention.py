@@ -266,11 +266,14 @@ def test_frozen_vectors(dtype):
     bf16-representable, so both dtypes see the same numbers)."""
     from tests.golden_vectors import load
     cases = load()
-    for name in ("ring2_causal_bias_segments", "one_device_causal_block4", "decode_cache_idx_70"):
+    for name in ("ring2_causal_bias_segments", "one_device_causal_block4", "decode_cache_idx_70",
+                 "ring2_causal_dropout"):
         c = cases[name]
         i, cfg = c["in"], c["cfg"]
         print("frozen", name, dtype, flush=True)
         kw = kwargs(cfg["qc"], cfg["kc"], cfg["cbs"])
+        if "drop_permille" in cfg:
+            kw.update(deterministic=False, attn_pdrop=cfg["drop_permille"] / 1000.0, dropout_rng=cfg["seed"])
         do = i["do"].to(dtype) if "do" in i else None
         out, grads = run_hip(i["q"].to(dtype), i["k"].to(dtype), i["v"].to(dtype), do, i.get("bias"), i.get("seg"),
                              cfg.get("cache_idx"), cfg["n"], kw)

@@ -481,14 +481,18 @@ def test_oracle_reproduces_its_frozen_vectors():
     reference has no vectors): a change that moves them is caught here before it reaches the GPU comparisons."""
     from tests.golden_vectors import load
     cases = load()
-    for name in ("ring2_causal_bias_segments", "one_device_causal_block4", "decode_cache_idx_70"):
+    for name in ("ring2_causal_bias_segments", "one_device_causal_block4", "decode_cache_idx_70",
+                 "ring2_causal_dropout"):
         c = cases[name]
         i, cfg = c["in"], c["cfg"]
+        kw = kwargs(cfg["qc"], cfg["kc"], cfg["cbs"])
+        if "drop_permille" in cfg:
+            kw.update(deterministic=False, attn_pdrop=cfg["drop_permille"] / 1000.0, dropout_rng=cfg["seed"])
         out, res = O.ring_attention_fwd(i["q"], i["k"], i["v"], i.get("bias"), i.get("seg"), cfg.get("cache_idx"),
-                                        cfg["n"], True, kwargs(cfg["qc"], cfg["kc"], cfg["cbs"]))
+                                        cfg["n"], True, kw)
         assert torch.allclose(out, c["out"]["out"], rtol=1e-5, atol=1e-6), name
         if "do" in i:
-            grads = O.ring_attention_bwd(cfg["n"], True, kwargs(cfg["qc"], cfg["kc"], cfg["cbs"]), res, i["do"])
+            grads = O.ring_attention_bwd(cfg["n"], True, kw, res, i["do"])
             for nm, gr in zip(("dq", "dk", "dv"), grads):
                 assert torch.allclose(gr, c["out"][nm], rtol=1e-5, atol=1e-6), (name, nm)
     c = cases["inference_ring2"]
