@@ -133,6 +133,9 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs 
   int kend_wg = ri.kend;
   for (int off = 32; off > 0; off >>= 1) kend_wg = max(kend_wg, __shfl_xor(kend_wg, off));
 
+  // Under dropout a pair can hold -inf inside a key chunk that runs.  A chunk whose pairs are all -inf while the
+  // running max is still -inf makes the reference compute exp(-inf - -inf) = NaN (:138-144) and the row stays NaN
+  bool seen_finite = m != RA_NEG_INF, chunk_neg = true, poison = false;
   for (int k0 = 0; k0 < kend_wg; k0 += GEN_TK) {
     __syncthreads();
     stage_rows<T, D>(Ks, kbase, a.kv_ss, k0, GEN_TK, a.Skv, tid, GEN_ROWS);
@@ -157,6 +160,15 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs 
       for (int d = 0; d < D; d++) dot = fmaf(q[d], Ks[j * D + d], dot);
       s[j] = logit(mv, ri, dot, scale, k0 + j, seg_k[j]);
       tile_max = fmaxf(tile_max, s[j]);
+      if (mv.keep_drop && k0 + j < ri.kend) {
+        const int in_chunk = (k0 + j) % mv.kc;
+        if (in_chunk == 0) chunk_neg = true;
+        chunk_neg = chunk_neg && s[j] == RA_NEG_INF;
+        if (in_chunk == mv.kc - 1) {
+          poison = poison || (chunk_neg && !seen_finite);
+          seen_finite = seen_finite || !chunk_neg;
+        }
+      }
     }
     float m_new = fmaxf(m, tile_max);                             // :138
     if (m_new == RA_NEG_INF) continue;                            // nothing ran for this row yet
@@ -175,9 +187,10 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs 
     m = m_new;
   }
   if (valid) {
+    const float nan = poison ? __builtin_nanf("") : 0.f;
 #pragma unroll
-    for (int d = 0; d < D; d++) nump[d] = acc[d];
-    a.mx[st] = m; a.den[st] = l;
+    for (int d = 0; d < D; d++) nump[d] = poison ? nan : acc[d];
+    a.mx[st] = m; a.den[st] = poison ? nan : l;
   }
 }
 

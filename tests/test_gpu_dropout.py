@@ -156,6 +156,24 @@ def test_dropout_row_without_allowed_key_takes_uniform_weights():
             assert float((got - want).abs().max()) <= 2e-2, (impl, h)
 
 
+def test_dropout_first_chunk_all_minus_inf_turns_the_row_nan_like_the_reference():
+    """Small key chunks, a high rate and foreign documents: a row can meet a first key chunk whose pairs are all
+    masked AND dropped (-inf) while its running max is still -inf; the reference then computes exp(-inf - -inf) = NaN
+    (:138-144) and the row stays NaN, with the gradients that follow from it.  NaN positions must coincide."""
+    B, S, H, D = 1, 128, 3, 32
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=16)
+    seg = packed_segment_ids(B, S, 10, seed=5)
+    for seed in range(50):
+        kw = kwargs(32, 8, 1, deterministic=False, dropout_rng=seed, attn_pdrop=0.6)
+        ref_out, _ = oracle_fwd_bwd(q, k, v, None, None, seg, None, 1, kw)
+        if bool(torch.isnan(ref_out).any()):
+            break
+    else:
+        pytest.fail("no seed below 50 produces the case")
+    assert not bool(torch.isnan(ref_out).all())
+    _compare(q, k, v, do, None, seg, 1, kw, torch.float32, "first chunk -inf, seed %d" % seed)
+
+
 def test_dropout_probabilities_still_sum_to_one_at_8k():
     """V = 1: every row is a convex combination, whatever was dropped (rows without any allowed key included)."""
     B, S, H, D = 1, 8192, 4, 128
