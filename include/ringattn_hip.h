@@ -112,6 +112,13 @@ typedef struct ra_attn_fwd_params {
   ra_mask mask;
   int32_t impl;
   int32_t carry_is_initial;   /* 1: the carry holds (0, 0, -inf) by definition; kernels need not read it */
+  void* out;                  /* nullable.  When given, this call is the LAST ring step of its device: out =
+                                 numerator / denominator (:52) is written here in `dtype`, (B,Sq,H,D) with the strides
+                                 below, and the numerator is not written back (it may then be null when
+                                 carry_is_initial); denominator and max_score are updated as always (they are
+                                 residuals, :53).  Saves the numerator's round trip through memory and
+                                 ra_attn_finalize */
+  int64_t out_stride_b, out_stride_s;
 } ra_attn_fwd_params;
 
 /* _blockwise_attention_bwd (ringattention_jax.py:181-270): adds this step's gradients into the
@@ -129,7 +136,17 @@ typedef struct ra_attn_bwd_params {
   float* dk; float* dv; int64_t dkv_stride_b, dkv_stride_s;
   ra_mask mask;
   int32_t impl;
+  int32_t grads_are_initial;  /* RA_GRAD_INIT_DQ | RA_GRAD_INIT_DKV: that accumulator holds zeros by definition
+                                 (:61-63): it is not read, and may be null when the matching *_out is given */
+  void* dq_out;               /* nullable.  When given, this call is the LAST one that adds into this dq: the sum is
+                                 written here in `dtype` (the cast of :89), (B,Sq,H,D), and the fp32 dq is left as it
+                                 was */
+  int64_t dq_out_stride_b, dq_out_stride_s;
+  void* dk_out; void* dv_out; /* the same for dk and dv (both or neither), (B,Skv,H,D) */
+  int64_t dkv_out_stride_b, dkv_out_stride_s;
 } ra_attn_bwd_params;
+
+enum { RA_GRAD_INIT_DQ = 1, RA_GRAD_INIT_DKV = 2 };
 
 enum { RA_SEG_TILE = 64 };
 /* min / max segment id per run of RA_SEG_TILE positions: out (Bseg, ceil(seg_len / RA_SEG_TILE), 2).

@@ -15,6 +15,7 @@ RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
 RA_BWD_ONLY_DQ, RA_BWD_ONLY_DKV = 0x10, 0x20
 RA_SEG_TILE = 64
 RA_KEEP_WHERE, RA_KEEP_DROPOUT = 0, 1
+RA_GRAD_INIT_DQ, RA_GRAD_INIT_DKV = 1, 2
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
@@ -43,6 +44,7 @@ class RaAttnFwdParams(C.Structure):
         ("numerator", vp), ("num_stride_b", i64), ("num_stride_s", i64),
         ("denominator", vp), ("max_score", vp), ("stat_stride_b", i64), ("stat_stride_h", i64),
         ("mask", RaMask), ("impl", i32), ("carry_is_initial", i32),
+        ("out", vp), ("out_stride_b", i64), ("out_stride_s", i64),
     ]
 
 
@@ -54,7 +56,9 @@ class RaAttnBwdParams(C.Structure):
         ("delta", vp), ("denominator", vp), ("max_score", vp), ("stat_stride_b", i64), ("stat_stride_h", i64),
         ("dq", vp), ("dq_stride_b", i64), ("dq_stride_s", i64),
         ("dk", vp), ("dv", vp), ("dkv_stride_b", i64), ("dkv_stride_s", i64),
-        ("mask", RaMask), ("impl", i32),
+        ("mask", RaMask), ("impl", i32), ("grads_are_initial", i32),
+        ("dq_out", vp), ("dq_out_stride_b", i64), ("dq_out_stride_s", i64),
+        ("dk_out", vp), ("dv_out", vp), ("dkv_out_stride_b", i64), ("dkv_out_stride_s", i64),
     ]
 
 

@@ -193,8 +193,9 @@ int ra_dropout_keep_packed(uint64_t seed, float attn_pdrop, int32_t B, int32_t H
 
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p, RA_ERR_INVALID, "attn_fwd_block: null params");
-  RA_REQUIRE(p->q && p->k && p->v && p->numerator && p->denominator && p->max_score, RA_ERR_INVALID,
-             "attn_fwd_block: null tensor");
+  RA_REQUIRE(p->q && p->k && p->v && p->denominator && p->max_score, RA_ERR_INVALID, "attn_fwd_block: null tensor");
+  RA_REQUIRE(p->numerator || (p->carry_is_initial && p->out), RA_ERR_INVALID,
+             "attn_fwd_block: the numerator may be null only when carry_is_initial is set and out is given");
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_fwd_block: dtype %d", p->dtype);
   RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_fwd_block: empty shape");
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_fwd_block: B and H must be <= 65535");
@@ -230,8 +231,16 @@ int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t str
 
 int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p, RA_ERR_INVALID, "attn_bwd_block: null params");
-  RA_REQUIRE(p->q && p->k && p->v && p->g && p->delta && p->denominator && p->max_score && p->dq && p->dk && p->dv,
-             RA_ERR_INVALID, "attn_bwd_block: null tensor");
+  RA_REQUIRE(p->q && p->k && p->v && p->g && p->delta && p->denominator && p->max_score, RA_ERR_INVALID,
+             "attn_bwd_block: null tensor");
+  RA_REQUIRE((p->dk_out == nullptr) == (p->dv_out == nullptr), RA_ERR_INVALID,
+             "attn_bwd_block: dk_out and dv_out go together");
+  RA_REQUIRE((p->grads_are_initial & ~(RA_GRAD_INIT_DQ | RA_GRAD_INIT_DKV)) == 0, RA_ERR_INVALID,
+             "attn_bwd_block: unknown bits in grads_are_initial");
+  RA_REQUIRE(p->dq || ((p->grads_are_initial & RA_GRAD_INIT_DQ) && p->dq_out), RA_ERR_INVALID,
+             "attn_bwd_block: dq may be null only when it is initial and dq_out is given");
+  RA_REQUIRE((p->dk && p->dv) || ((p->grads_are_initial & RA_GRAD_INIT_DKV) && p->dk_out), RA_ERR_INVALID,
+             "attn_bwd_block: dk / dv may be null only when they are initial and dk_out / dv_out are given");
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_bwd_block: dtype %d", p->dtype);
   RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_bwd_block: empty shape");
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_bwd_block: B and H must be <= 65535");

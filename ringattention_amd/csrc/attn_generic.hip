@@ -22,6 +22,10 @@ struct GenericArgs {
   MaskView mv;
   const int32_t* cache_idx;
   int carry_is_initial;
+  void* out; int64_t out_sb, out_ss;             // forward, nullable: out = num / den instead of the numerator
+  int dq_initial, dkv_initial;                   // backward: that accumulator holds zeros by definition
+  void* dq_out; int64_t dqo_sb, dqo_ss;          // backward, nullable: the sum goes here in the primal dtype
+  void* dk_out; void* dv_out; int64_t dkvo_sb, dkvo_ss;
 };
 
 __device__ __forceinline__ MaskView resolve_mask(const GenericArgs& a) {
@@ -188,8 +192,14 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs 
   }
   if (valid) {
     const float nan = poison ? __builtin_nanf("") : 0.f;
+    if (a.out) {                       // last step of the device: out = numerator / denominator (:52)
+      T* op = (T*)a.out + (int64_t)b * a.out_sb + (int64_t)rrow * a.out_ss + (int64_t)h * D;
 #pragma unroll
-    for (int d = 0; d < D; d++) nump[d] = poison ? nan : acc[d];
+      for (int d = 0; d < D; d++) store_from_f32<T>(op + d, poison ? nan : acc[d] / l);
+    } else {
+#pragma unroll
+      for (int d = 0; d < D; d++) nump[d] = poison ? nan : acc[d];
+    }
     a.mx[st] = m; a.den[st] = poison ? nan : l;
   }
 }
@@ -252,8 +262,13 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_bwd_dq_generic_kernel(GenericAr
     }
   }
   if (valid) {
+    T* op = (T*)a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)rrow * a.dqo_ss + (int64_t)h * D;
 #pragma unroll
-    for (int d = 0; d < D; d++) dqp[d] += dq[d] / scale;
+    for (int d = 0; d < D; d++) {
+      const float t = (a.dq_initial ? 0.f : dqp[d]) + dq[d] / scale;
+      if (a.dq_out) store_from_f32<T>(op + d, t);                  // last call for these rows (:89)
+      else dqp[d] = t;
+    }
   }
 }
 
@@ -333,8 +348,13 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_bwd_dkv_generic_kernel(GenericA
     }
   }
   if (valid) {
+    T* op = (T*)(WANT_DK ? a.dk_out : a.dv_out) + (int64_t)b * a.dkvo_sb + (int64_t)rk * a.dkvo_ss + (int64_t)h * D;
 #pragma unroll
-    for (int d = 0; d < D; d++) outp[d] += WANT_DK ? acc[d] / scale : acc[d];
+    for (int d = 0; d < D; d++) {
+      const float t = (a.dkv_initial ? 0.f : outp[d]) + (WANT_DK ? acc[d] / scale : acc[d]);
+      if (a.dk_out) store_from_f32<T>(op + d, t);                  // last call for these keys (:89)
+      else outp[d] = t;
+    }
   }
 }
 
@@ -534,6 +554,7 @@ static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
+  a.out = p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s;
   return a;
 }
 
@@ -585,6 +606,10 @@ int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s) {
   a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.dq = p->dq; a.dq_sb = p->dq_stride_b; a.dq_ss = p->dq_stride_s;
   a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
+  a.dq_initial = (p->grads_are_initial & RA_GRAD_INIT_DQ) != 0;
+  a.dkv_initial = (p->grads_are_initial & RA_GRAD_INIT_DKV) != 0;
+  a.dq_out = p->dq_out; a.dqo_sb = p->dq_out_stride_b; a.dqo_ss = p->dq_out_stride_s;
+  a.dk_out = p->dk_out; a.dv_out = p->dv_out; a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   return p->dtype == RA_F32 ? launch_bwd_T<float>(a, s) : launch_bwd_T<uint16_t>(a, s);

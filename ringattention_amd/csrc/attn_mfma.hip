@@ -37,6 +37,7 @@ struct FwdArgs {
   MaskView mv;
   const int32_t* cache_idx;
   int carry_is_initial;
+  uint16_t* out; int64_t out_sb, out_ss;      // nullable: last step of the device, out = num / den instead of num
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -172,7 +173,31 @@ struct BwdArgs {
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
   const int32_t* cache_idx;
+  int dq_initial, dkv_initial;                 // the fp32 accumulator holds zeros by definition: not read
+  uint16_t* dq_out; int64_t dqo_sb, dqo_ss;    // nullable: last call that adds into it, the sum goes here as bf16
+  uint16_t* dk_out; uint16_t* dv_out; int64_t dkvo_sb, dkvo_ss;
 };
+
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_bf16x4(uint16_t* p, const f32x4& t) {
+  bf16x4_t o;
+#pragma unroll
+  for (int e = 0; e < 4; e++) o[e] = (__bf16)t[e];
+  *(bf16x4_t*)p = o;
+}
+// The rows of a gradient that a workgroup owns but has nothing to add to (rows x HD floats from acc / out, which
+// point at row 0, head h): hand the accumulator on as bf16, or set it to the zeros it holds by definition.
+__device__ __forceinline__ void pass_rows(float* acc, int64_t acc_ss, uint16_t* out, int64_t out_ss, int rows,
+                                          int initial, int tid) {
+  if (!out && !initial) return;
+  for (int i = tid; i < rows * (HD / 4); i += 512) {
+    const int r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+    f32x4 t = {0.f, 0.f, 0.f, 0.f};
+    if (!initial) t = *(const f32x4*)(acc + (int64_t)r * acc_ss + c4);
+    if (out) store_bf16x4(out + (int64_t)r * out_ss + c4, t);
+    else *(f32x4*)(acc + (int64_t)r * acc_ss + c4) = t;
+  }
+}
 
 // ------------------------------------------------------------------ dK / dV, wave-specialised
 // 8 wavefronts per workgroup, 128 keys: pair i = (wave i, wave i + 4) shares a SIMD and owns keys
@@ -270,7 +295,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     qt_end = qt_first + t_last;
     qt_first += t_first;
   }
-  if (qt_first >= qt_end) return;
+  if (qt_first >= qt_end) {                // nothing to add for these keys
+    const int64_t o = (int64_t)b * a.dkv_sb + (int64_t)k0 * a.dkv_ss + (int64_t)h * HD;
+    const int64_t oo = (int64_t)b * a.dkvo_sb + (int64_t)k0 * a.dkvo_ss + (int64_t)h * HD;
+    pass_rows(a.dk ? a.dk + o : nullptr, a.dkv_ss, a.dk_out ? a.dk_out + oo : nullptr, a.dkvo_ss, KBN, a.dkv_initial, tid);
+    pass_rows(a.dv ? a.dv + o : nullptr, a.dkv_ss, a.dv_out ? a.dv_out + oo : nullptr, a.dkvo_ss, KBN, a.dkv_initial, tid);
+    return;
+  }
   const int ntq = qt_end - qt_first;       // query tiles of 64 rows
   const int nblk = 2 * ntq;                // blocks of 32 rows
 
@@ -600,16 +631,23 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     // dk += acc / sqrt(D) (:231), dv += acc (:232); this pair owns its 32 key rows
     const float rscale = 1.f / sqrtf((float)HD);
     const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
+    const int64_t oout = (int64_t)b * a.dkvo_sb + (int64_t)krow * a.dkvo_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
     for (int db = 0; db < 4; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         float* pk = a.dk + ooff + db * 32 + g * 8;
         float* pv = a.dv + ooff + db * 32 + g * 8;
-        f32x4 tk = *(const f32x4*)pk, tv = *(const f32x4*)pv;
+        f32x4 tk = {0.f, 0.f, 0.f, 0.f}, tv = {0.f, 0.f, 0.f, 0.f};
+        if (!a.dkv_initial) { tk = *(const f32x4*)pk; tv = *(const f32x4*)pv; }
 #pragma unroll
         for (int e = 0; e < 4; e++) { tk[e] += dkacc[db][g * 4 + e] * rscale; tv[e] += dvacc[db][g * 4 + e]; }
-        *(f32x4*)pk = tk; *(f32x4*)pv = tv;
+        if (a.dk_out) {                  // last call for these keys: the sum as bf16 (:89)
+          store_bf16x4(a.dk_out + oout + db * 32 + g * 8, tk);
+          store_bf16x4(a.dv_out + oout + db * 32 + g * 8, tv);
+        } else {
+          *(f32x4*)pk = tk; *(f32x4*)pv = tv;
+        }
       }
   }
 #undef RA_WS_LOAD
@@ -688,7 +726,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     k_base += t_first * FBN;
     ntiles = t_last - t_first;
   }
-  if (ntiles == 0) return;     // nothing to add to dq
+  if (ntiles == 0) {           // nothing to add to dq
+    pass_rows(a.dq ? a.dq + (int64_t)b * a.dq_sb + (int64_t)q0 * a.dq_ss + (int64_t)h * HD : nullptr, a.dq_ss,
+              a.dq_out ? a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)q0 * a.dqo_ss + (int64_t)h * HD : nullptr,
+              a.dqo_ss, FBM, a.dq_initial, tid);
+    return;
+  }
   const int gk0 = gk0_shard + k_base;
   const float c = kLog2e / sqrtf((float)HD);
   const float bias_scale = kLog2e / c;
@@ -1058,14 +1101,17 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     // dq += acc / sqrt(D)   (:230)
     const float rscale = 1.f / sqrtf((float)HD);
     float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
+    uint16_t* dqo = a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)qrow * a.dqo_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
     for (int db = 0; db < 4; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        f32x4 t = *(const f32x4*)(dqp + db * 32 + g * 8);
+        f32x4 t = {0.f, 0.f, 0.f, 0.f};
+        if (!a.dq_initial) t = *(const f32x4*)(dqp + db * 32 + g * 8);
 #pragma unroll
         for (int e = 0; e < 4; e++) t[e] += acc[db][g * 4 + e] * rscale;
-        *(f32x4*)(dqp + db * 32 + g * 8) = t;
+        if (a.dq_out) store_bf16x4(dqo + db * 32 + g * 8, t);      // last call for these rows: the sum as bf16 (:89)
+        else *(f32x4*)(dqp + db * 32 + g * 8) = t;
       }
   }
 #undef RA_WS_LOAD_K
@@ -1136,15 +1182,27 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     ntiles = t_last - t_first;
   }
   if (ntiles == 0) {           // no key tile runs for these rows: the carry stays as it is
-    if (a.carry_is_initial) {
+    if (a.carry_is_initial || a.out) {
       const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
       float* np0 = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
+      uint16_t* op0 = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
       if (role == 1) {
+        const float rd = 1.f / (a.carry_is_initial ? 0.f : a.den[st0]);      // 0 / 0 = NaN, as :52
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
-          for (int g = 0; g < 4; g++) *(f32x4*)(np0 + db * 32 + g * 8) = f32x4{0.f, 0.f, 0.f, 0.f};
-      } else if (hi == 0) {
+          for (int g = 0; g < 4; g++) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            if (!a.carry_is_initial) t = *(const f32x4*)(np0 + db * 32 + g * 8);
+            if (a.out) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) t[e] *= rd;
+              store_bf16x4(op0 + db * 32 + g * 8, t);
+            } else {
+              *(f32x4*)(np0 + db * 32 + g * 8) = t;
+            }
+          }
+      } else if (hi == 0 && a.carry_is_initial) {
         a.den[st0] = 0.f; a.mx[st0] = RA_NEG_INF;
       }
     }
@@ -1450,9 +1508,10 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const float fix = (m_true == m2) ? 1.f : fast_exp2(m2 - m_true);
     m2 = m_true;
     l *= fix;
-    if (hi == 0) fixs[pair][lo] = fix;
-    __syncthreads();
     l += xor32(l);
+    // the last step of the device hands over fix / denominator: the consumer then writes out = numerator / denominator
+    if (hi == 0) fixs[pair][lo] = a.out ? fix / l : fix;
+    __syncthreads();
     if (hi == 0) {
       a.den[st] = l;
       a.mx[st] = max_from_log2(m2, kMask2);
@@ -1561,6 +1620,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 
     __syncthreads();      // the producer's final factor
     const float fix = fixs[pair][lo];
+    uint16_t* outp = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
     for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -1568,7 +1628,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
         f32x4 t4;
 #pragma unroll
         for (int e = 0; e < 4; e++) t4[e] = acc[db][g * 4 + e] * fix;
-        *(f32x4*)(nump + db * 32 + g * 8) = t4;
+        if (a.out) store_bf16x4(outp + db * 32 + g * 8, t4);
+        else *(f32x4*)(nump + db * 32 + g * 8) = t4;
       }
   }
 #undef RA_WS_LOAD_K
@@ -1592,7 +1653,8 @@ bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
   return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
          keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
-         aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator);
+         aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator) &&
+         (!p->out || (aligned16(p->out) && p->out_stride_s % 4 == 0 && p->out_stride_b % 4 == 0));
 }
 
 int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
@@ -1605,6 +1667,7 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
+  a.out = (uint16_t*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool keep = p->mask.keep_bits_k != nullptr;      // packed form checked by attn_fwd_mfma_supported
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
@@ -1626,7 +1689,10 @@ bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
          keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0 &&
          p->dkv_stride_s % 4 == 0 && p->dkv_stride_b % 4 == 0 && aligned16(p->q) && aligned16(p->k) &&
-         aligned16(p->v) && aligned16(p->g) && aligned16(p->dq) && aligned16(p->dk) && aligned16(p->dv);
+         aligned16(p->v) && aligned16(p->g) && aligned16(p->dq) && aligned16(p->dk) && aligned16(p->dv) &&
+         (!p->dq_out || (aligned16(p->dq_out) && p->dq_out_stride_s % 4 == 0 && p->dq_out_stride_b % 4 == 0)) &&
+         (!p->dk_out || (aligned16(p->dk_out) && aligned16(p->dv_out) && p->dkv_out_stride_s % 4 == 0 &&
+                         p->dkv_out_stride_b % 4 == 0));
 }
 
 int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
@@ -1638,6 +1704,11 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
   a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.dq = p->dq; a.dq_sb = p->dq_stride_b; a.dq_ss = p->dq_stride_s;
   a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
+  a.dq_initial = (p->grads_are_initial & RA_GRAD_INIT_DQ) != 0;
+  a.dkv_initial = (p->grads_are_initial & RA_GRAD_INIT_DKV) != 0;
+  a.dq_out = (uint16_t*)p->dq_out; a.dqo_sb = p->dq_out_stride_b; a.dqo_ss = p->dq_out_stride_s;
+  a.dk_out = (uint16_t*)p->dk_out; a.dv_out = (uint16_t*)p->dv_out;
+  a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   const long long nq = (long long)(p->Sq / FBM) * p->H * p->B, nk = (long long)(p->Skv / KBN) * p->H * p->B;

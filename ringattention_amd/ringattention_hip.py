@@ -365,9 +365,11 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
                              causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
                              dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
                              precision=None, prevent_cse=True, cache_idx=None, _mask_inputs=None,
-                             _cfg=None, _carry_is_initial=False, **extra):
+                             _cfg=None, _carry_is_initial=False, _out=None, **extra):
     """ringattention_jax.py:99-179.  ``carry`` = (numerator (B,Sq,H,D), denominator (B,H,Sq),
-    max_score (B,H,Sq)), fp32, updated IN PLACE and returned."""
+    max_score (B,H,Sq)), fp32, updated IN PLACE and returned.  With ``_out`` (B,Sq,H,D in q's dtype) the step is
+    the last one of its device: out = numerator / denominator (:52) is written there instead of the numerator,
+    which may then be None if the carry is initial."""
     cfg = _cfg or _Config(dict(causal_block_size=causal_block_size, query_chunk_size=query_chunk_size,
                                key_chunk_size=key_chunk_size, deterministic=deterministic,
                                attn_pdrop=attn_pdrop, dtype=dtype, **extra))
@@ -385,8 +387,16 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
     p.kv_stride_b, p.kv_stride_s = _rows(k)
     if _rows(v) != _rows(k):
         raise ValueError("k and v must share strides")
-    p.numerator = num.data_ptr()
-    p.num_stride_b, p.num_stride_s = _rows(num)
+    if num is not None:
+        p.numerator = num.data_ptr()
+        p.num_stride_b, p.num_stride_s = _rows(num)
+    else:
+        p.num_stride_b, p.num_stride_s = Sq * H * D, H * D
+    if _out is not None:
+        if _out.dtype != q.dtype:
+            raise ValueError("out must have the dtype of q")
+        p.out = _out.data_ptr()
+        p.out_stride_b, p.out_stride_s = _rows(_out)
     p.denominator, p.max_score = den.data_ptr(), mx.data_ptr()
     if den.stride() != mx.stride() or den.stride(2) != 1:
         raise ValueError("denominator / max_score must share strides and be dense in the last dim")
@@ -410,9 +420,12 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
                              causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
                              dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
                              precision=None, prevent_cse=True, cache_idx=None, _mask_inputs=None,
-                             _cfg=None, _delta=None, **extra):
+                             _cfg=None, _delta=None, _grads_initial=0, _dq_out=None, _dkv_out=None, **extra):
     """ringattention_jax.py:181-270.  ``carry`` = (dq, dk, dv, output, denominator, max_score); the
-    fp32 accumulators dq, dk, dv are added into IN PLACE and returned."""
+    fp32 accumulators dq, dk, dv are added into IN PLACE and returned.  ``_grads_initial`` (RA_GRAD_INIT_*) marks
+    accumulators that hold zeros by definition (not read; may be None with the matching output); ``_dq_out`` /
+    ``_dkv_out = (dk_out, dv_out)`` in q's dtype mark the last call that adds into them: the sum is written there
+    (the cast of :89) and the accumulator is left alone."""
     cfg = _cfg or _Config(dict(causal_block_size=causal_block_size, query_chunk_size=query_chunk_size,
                                key_chunk_size=key_chunk_size, deterministic=deterministic,
                                attn_pdrop=attn_pdrop, dtype=dtype, **extra))
@@ -439,12 +452,30 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
     if not (delta.stride() == den.stride() == mx.stride()):
         raise ValueError("delta / denominator / max_score must share strides")
     p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
-    p.dq = dq.data_ptr()
-    p.dq_stride_b, p.dq_stride_s = _rows(dq)
-    p.dk, p.dv = dk.data_ptr(), dv.data_ptr()
-    p.dkv_stride_b, p.dkv_stride_s = _rows(dk)
-    if _rows(dv) != _rows(dk):
-        raise ValueError("dk and dv must share strides")
+    if dq is not None:
+        p.dq = dq.data_ptr()
+        p.dq_stride_b, p.dq_stride_s = _rows(dq)
+    else:
+        p.dq_stride_b, p.dq_stride_s = Sq * H * D, H * D
+    if dk is not None:
+        p.dk, p.dv = dk.data_ptr(), dv.data_ptr()
+        p.dkv_stride_b, p.dkv_stride_s = _rows(dk)
+        if _rows(dv) != _rows(dk):
+            raise ValueError("dk and dv must share strides")
+    else:
+        p.dkv_stride_b, p.dkv_stride_s = Skv * H * D, H * D
+    p.grads_are_initial = _grads_initial
+    if _dq_out is not None:
+        if _dq_out.dtype != q.dtype:
+            raise ValueError("dq_out must have the dtype of q")
+        p.dq_out = _dq_out.data_ptr()
+        p.dq_out_stride_b, p.dq_out_stride_s = _rows(_dq_out)
+    if _dkv_out is not None:
+        dko, dvo = _dkv_out
+        if dko.dtype != q.dtype or dvo.dtype != q.dtype or _rows(dko) != _rows(dvo):
+            raise ValueError("dk_out and dv_out must have the dtype of q and share strides")
+        p.dk_out, p.dv_out = dko.data_ptr(), dvo.data_ptr()
+        p.dkv_out_stride_b, p.dkv_out_stride_s = _rows(dko)
     if mi.cache_idx_host is not None:
         q_chunk_idx_start = mi.cache_idx_host // cfg.qc
     skip = cfg.skip_masked_tiles
@@ -540,30 +571,45 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
         if cache_idx is not None:
             raise NotImplementedError("attention dropout together with cache_idx is not supported")
         cfg.skip_masked_tiles = False      # dropout can leave a row without any allowed key
-    num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)      # :22
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)         # :23
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)          # :49
-    for dev in range(n):
+    out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
+    plan = _ring_plan(cfg, mi, n, q_len, kv_len)
+    # the numerator carry (:22) only exists between the steps of a device: its first step starts it (nothing is
+    # read), its last step writes out = numerator / denominator (:52) instead
+    num = None
+    if any(len(steps) != 1 for steps in plan):
+        num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
+    for dev, steps in enumerate(plan):
         qs = slice(dev * q_len, (dev + 1) * q_len)
-        carry = (num[:, qs], den[:, :, qs], mx[:, :, qs])
-        started = False
-        for idx in range(n):                                                          # :50-51
-            k_blk = (dev - idx) % n                                                   # :36
-            k_start = k_blk * (kv_len // cfg.kc)                                      # :37
-            q_start = _q_start(cfg, mi, dev, q_len)
-            if not _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
-                continue
+        carry = (num[:, qs] if num is not None else None, den[:, :, qs], mx[:, :, qs])
+        for j, (q_start, k_blk, k_start) in enumerate(steps):
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
             _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, q_start, k_start, None, None,
                                      cfg.cbs, cfg.qc, cfg.kc, _mask_inputs=mi, _cfg=cfg,
-                                     _carry_is_initial=not started, cache_idx=cache_idx)
-            started = True
-        if not started:
+                                     _carry_is_initial=j == 0, cache_idx=cache_idx,
+                                     _out=out[:, qs] if j == len(steps) - 1 else None)
+        if not steps:                       # no tile runs for this device: 0 / 0
             _carry_init(*carry)
-    out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
-    _finalize(num, den, out)                                                          # :52
+            _finalize(carry[0], carry[1], out[:, qs])
     del num
     return out, (out, q, k, v, mi, cfg, n, den, mx)
+
+
+def _ring_plan(cfg, mi, n, q_len, kv_len):
+    """For every device of the virtual ring the steps that run, in ring order (:50-51): (q_chunk_idx_start,
+    index of the K/V shard that has arrived (:36), k_chunk_idx_start (:37))."""
+    plan = []
+    for dev in range(n):
+        steps = []
+        for idx in range(n):
+            k_blk = (dev - idx) % n
+            k_start = k_blk * (kv_len // cfg.kc)
+            q_start = _q_start(cfg, mi, dev, q_len)
+            if _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
+                steps.append((q_start, k_blk, k_start))
+        plan.append(steps)
+    return plan
 
 
 def _ring_attention_bwd(res, g):
@@ -575,24 +621,48 @@ def _ring_attention_bwd(res, g):
     q_len, kv_len = q_total // n, kv_total // n
     g = g.to(q.dtype).contiguous()
     delta = _bwd_delta(g, out)
-    dq = torch.zeros((B, q_total, H, D), dtype=torch.float32, device=q.device)        # :61
-    dk = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)       # :62
-    dv = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)       # :63
-    for dev in range(n):
+    plan = _ring_plan(cfg, mi, n, q_len, kv_len)
+    # the calls that add into each K/V shard's dk, dv, in program order (they ride with the shard, :85-86)
+    last_for_shard, count_for_shard = {}, {}
+    for dev, steps in enumerate(plan):
+        for j, (_, k_blk, _) in enumerate(steps):
+            last_for_shard[k_blk] = (dev, j)
+            count_for_shard[k_blk] = count_for_shard.get(k_blk, 0) + 1
+    # fp32 accumulators (:61-63) exist only where more than one call adds into a gradient: the first call starts
+    # them (nothing is read, so no zero fill), the last one writes the sum in the primal dtype (:89)
+    dq_out = torch.empty((B, q_total, H, D), dtype=q.dtype, device=q.device)
+    dk_out = torch.empty((B, kv_total, H, D), dtype=k.dtype, device=q.device)
+    dv_out = torch.empty((B, kv_total, H, D), dtype=v.dtype, device=q.device)
+    dq = dk = dv = None
+    if any(len(steps) > 1 for steps in plan):
+        dq = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
+    if any(c > 1 for c in count_for_shard.values()):
+        dk = torch.empty((B, kv_total, H, D), dtype=torch.float32, device=q.device)
+        dv = torch.empty((B, kv_total, H, D), dtype=torch.float32, device=q.device)
+    seen_shard = set()
+    for dev, steps in enumerate(plan):
         qs = slice(dev * q_len, (dev + 1) * q_len)
-        for idx in range(n):                                                          # :88
-            k_blk = (dev - idx) % n
-            k_start = k_blk * (kv_len // cfg.kc)
-            q_start = _q_start(cfg, mi, dev, q_len)
-            if not _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
-                continue
+        if not steps:
+            dq_out[:, qs].zero_()
+        for j, (q_start, k_blk, k_start) in enumerate(steps):
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
-            # the dk/dv partials ride with their K/V shard (:85-86): accumulate at the shard's home
+            initial = (L.RA_GRAD_INIT_DQ if j == 0 else 0) | (L.RA_GRAD_INIT_DKV if k_blk not in seen_shard else 0)
+            seen_shard.add(k_blk)
+            last_dq = j == len(steps) - 1
+            last_dkv = last_for_shard[k_blk] == (dev, j)
             _blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], g[:, qs],
-                                     (dq[:, qs], dk[:, ks], dv[:, ks], out[:, qs], den[:, :, qs], mx[:, :, qs]),
+                                     (dq[:, qs] if dq is not None else None, dk[:, ks] if dk is not None else None,
+                                      dv[:, ks] if dv is not None else None, out[:, qs], den[:, :, qs], mx[:, :, qs]),
                                      q_start, k_start, None, None, cfg.cbs, cfg.qc, cfg.kc,
-                                     _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs])
-    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
+                                     _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs], _grads_initial=initial,
+                                     _dq_out=dq_out[:, qs] if last_dq else None,
+                                     _dkv_out=(dk_out[:, ks], dv_out[:, ks]) if last_dkv else None)
+    for k_blk in range(n):
+        if k_blk not in seen_shard:
+            ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            dk_out[:, ks].zero_()
+            dv_out[:, ks].zero_()
+    return dq_out, dk_out, dv_out
 
 
 class _RingAttentionFn(torch.autograd.Function):
