@@ -4,8 +4,9 @@ are multiples of 256 run on the MFMA kernels, which read the mask in a packed fo
 anything else runs on the fp32 vector-ALU kernels."""
 import torch
 
+from . import _lib as L
 from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, _blockwise_attention_fwd,
-                                _bwd_delta, _check_qkv, _finalize, axis_size)
+                                _bwd_delta, _check_qkv, axis_size)
 
 
 def _inference_cfg(q, q_len, kv_len, float32_logits):
@@ -35,20 +36,22 @@ def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
     # tiles without a kept pair may be skipped unless some row attends to nothing at all (its logits stay
     # equal at finfo.min and its weights uniform, ringattention_inference.py:22-24)
     cfg.skip_masked_tiles = not mi.keep_has_empty_row
-    num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)   # :13
+    # the numerator (:13) lives between the steps of a device only: the first step starts it, the last one writes
+    # out = numerator / denominator (:34) instead
+    num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device) if n > 1 else None
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)      # :14
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)       # :31
+    out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
     for dev in range(n):
         qs = slice(dev * q_len, (dev + 1) * q_len)
         mi.keep_row0 = dev * q_len                  # the device's rows of a mask that is sharded like q
-        carry = (num[:, qs], den[:, :, qs], mx[:, :, qs])
+        carry = (num[:, qs] if num is not None else None, den[:, :, qs], mx[:, :, qs])
         for idx in range(n):                                                      # :32-33
             k_blk = (dev - idx) % n                                               # :20
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
             _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, dev, k_blk, None, None,
-                                     None, q_len, kv_len, _mask_inputs=mi, _cfg=cfg, _carry_is_initial=(idx == 0))
-    out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
-    _finalize(num, den, out)                                                      # :34
+                                     None, q_len, kv_len, _mask_inputs=mi, _cfg=cfg, _carry_is_initial=(idx == 0),
+                                     _out=out[:, qs] if idx == n - 1 else None)
     return out, (out, q, k, v, mi, cfg, n, den, mx)
 
 
@@ -59,20 +62,27 @@ def _bwd(res, g):
     q_len, kv_len = q_total // n, kv_total // n
     g = g.to(q.dtype).contiguous()
     delta = _bwd_delta(g, out)                                                    # :55
-    dq = torch.zeros((B, q_total, H, D), dtype=torch.float32, device=q.device)    # :42
-    dk = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)   # :43
-    dv = torch.zeros((B, kv_total, H, D), dtype=torch.float32, device=q.device)   # :44
+    # fp32 accumulators (:42-44) between the calls that add into a gradient only: every device adds into its dq
+    # n times (first idx 0, last idx n - 1) and into every K/V shard once (first device 0, last device n - 1)
+    mk = lambda t: torch.empty(t.shape, dtype=torch.float32, device=q.device) if n > 1 else None
+    dq, dk, dv = mk(q), mk(k), mk(v)
+    dq_out, dk_out, dv_out = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    part = lambda t, sl: t[:, sl] if t is not None else None
     for dev in range(n):
         qs = slice(dev * q_len, (dev + 1) * q_len)
         mi.keep_row0 = dev * q_len
         for idx in range(n):
             k_blk = (dev - idx) % n                                               # :50
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            initial = (L.RA_GRAD_INIT_DQ if idx == 0 else 0) | (L.RA_GRAD_INIT_DKV if dev == 0 else 0)
             _blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], g[:, qs],
-                                     (dq[:, qs], dk[:, ks], dv[:, ks], out[:, qs], den[:, :, qs], mx[:, :, qs]),
+                                     (part(dq, qs), part(dk, ks), part(dv, ks), out[:, qs], den[:, :, qs],
+                                      mx[:, :, qs]),
                                      dev, k_blk, None, None, None, q_len, kv_len,
-                                     _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs])
-    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)                         # :62
+                                     _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs], _grads_initial=initial,
+                                     _dq_out=dq_out[:, qs] if idx == n - 1 else None,
+                                     _dkv_out=(dk_out[:, ks], dv_out[:, ks]) if dev == n - 1 else None)
+    return dq_out, dk_out, dv_out                                                 # :62
 
 
 class _RingAttentionInferenceFn(torch.autograd.Function):
