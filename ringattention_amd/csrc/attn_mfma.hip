@@ -1135,6 +1135,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   __shared__ __attribute__((aligned(16))) uint16_t Ds[4][2][WS_PD];        // [pair][buffer] P^T as [q][key]
   __shared__ float al[4][2][32];     // [pair][buffer][query]: factor the consumer applies to O before adding the block
   __shared__ float fixs[4][32];      // [pair][query]: final factor (lazy reference max -> exact max)
+  __shared__ float dens[4][32];      // [pair][query]: final denominator, for the step that writes out
   __shared__ int seg_ks[3][FBN];
   __shared__ float bias_ks[3][FBN];
 
@@ -1187,7 +1188,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
       float* np0 = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
       uint16_t* op0 = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
       if (role == 1) {
-        const float rd = 1.f / (a.carry_is_initial ? 0.f : a.den[st0]);      // 0 / 0 = NaN, as :52
+        const float den0 = a.carry_is_initial ? 0.f : a.den[st0];            // 0 / 0 = NaN, as :52
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -1196,7 +1197,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
             if (!a.carry_is_initial) t = *(const f32x4*)(np0 + db * 32 + g * 8);
             if (a.out) {
 #pragma unroll
-              for (int e = 0; e < 4; e++) t[e] *= rd;
+              for (int e = 0; e < 4; e++) t[e] /= den0;
               store_bf16x4(op0 + db * 32 + g * 8, t);
             } else {
               *(f32x4*)(np0 + db * 32 + g * 8) = t;
@@ -1509,8 +1510,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     m2 = m_true;
     l *= fix;
     l += xor32(l);
-    // the last step of the device hands over fix / denominator: the consumer then writes out = numerator / denominator
-    if (hi == 0) fixs[pair][lo] = a.out ? fix / l : fix;
+    // the last step of the device hands over the denominator too: the consumer then writes numerator / denominator
+    if (hi == 0) { fixs[pair][lo] = fix; dens[pair][lo] = l; }
     __syncthreads();
     if (hi == 0) {
       a.den[st] = l;
@@ -1620,6 +1621,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 
     __syncthreads();      // the producer's final factor
     const float fix = fixs[pair][lo];
+    const float den_row = dens[pair][lo];
     uint16_t* outp = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
     for (int db = 0; db < 4; db++)
@@ -1628,8 +1630,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
         f32x4 t4;
 #pragma unroll
         for (int e = 0; e < 4; e++) t4[e] = acc[db][g * 4 + e] * fix;
-        if (a.out) store_bf16x4(outp + db * 32 + g * 8, t4);
-        else *(f32x4*)(nump + db * 32 + g * 8) = t4;
+        if (a.out) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) t4[e] /= den_row;               // :52
+          store_bf16x4(outp + db * 32 + g * 8, t4);
+        } else {
+          *(f32x4*)(nump + db * 32 + g * 8) = t4;
+        }
       }
   }
 #undef RA_WS_LOAD_K

@@ -281,3 +281,72 @@ def test_frozen_vectors(dtype):
         if grads is not None:
             for nm, gr in zip(("dq", "dk", "dv"), grads):
                 assert_close(gr, c["out"][nm], dtype, name + " " + nm)
+
+
+@pytest.mark.parametrize("impl,dtype,S,D,qc", [("generic", torch.float32, 128, 32, 16), ("generic", torch.bfloat16, 128, 64, 32),
+                                                ("mfma", torch.bfloat16, 1024, 128, 256)])
+def test_first_and_last_step_modes_give_the_bits_of_the_separate_passes(impl, dtype, S, D, qc):
+    """Two ring steps of one device (own shard, then the shard before it), once with explicit fp32 carries, a
+    finalize pass and a cast, once with the first step starting the carries (uninitialised memory behind them) and
+    the last step writing out / dq / dk / dv in the primal dtype.  Same fp32 sums, one rounding: equal bits."""
+    from ringattention_amd import _lib as L
+    from ringattention_amd import ringattention_hip as rh
+    B, H = 1, 2
+    q, k, v, do = make_qkv(B, 2 * S, H, D, dtype=dtype, seed=31, scale=D ** -0.25)
+    q, k, v, do = (t.to(DEV) for t in (q, k, v, do))
+    kw = dict(causal_block_size=1, query_chunk_size=qc, key_chunk_size=qc, impl=impl)
+    nq = S // qc
+    qs = slice(S, 2 * S)                                   # the second device of a ring of two
+    steps = [(nq, slice(S, 2 * S), nq), (nq, slice(0, S), 0)]
+    f32 = lambda *shape: torch.full(shape, float("nan"), dtype=torch.float32, device=DEV)
+
+    # reference way: carry initialised, every step reads and writes it, finalize, delta, zeroed accumulators, cast
+    num, den, mx = f32(B, S, H, D), f32(B, H, S), f32(B, H, S)
+    rh._carry_init(num, den, mx)
+    for q_start, ks, k_start in steps:
+        ra._blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], (num, den, mx), q_start, k_start, None, None, **kw)
+    out_a = torch.empty(B, S, H, D, dtype=dtype, device=DEV)
+    rh._finalize(num, den, out_a)
+    delta = rh._bwd_delta(do[:, qs].contiguous(), out_a)
+    dq = torch.zeros(B, S, H, D, dtype=torch.float32, device=DEV)
+    dk, dv = (torch.zeros(B, 2 * S, H, D, dtype=torch.float32, device=DEV) for _ in range(2))
+    for q_start, ks, k_start in steps:
+        ra._blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], do[:, qs], (dq, dk[:, ks], dv[:, ks], out_a, den, mx),
+                                    q_start, k_start, None, None, _delta=delta, **kw)
+    ref = (out_a, dq.to(dtype), dk.to(dtype), dv.to(dtype))
+
+    # first / last modes: NaN-filled carries prove that the first step reads nothing
+    num2, den2, mx2 = f32(B, S, H, D), f32(B, H, S), f32(B, H, S)
+    out_b = torch.empty(B, S, H, D, dtype=dtype, device=DEV)
+    for j, (q_start, ks, k_start) in enumerate(steps):
+        ra._blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], (num2, den2, mx2), q_start, k_start, None, None,
+                                    _carry_is_initial=j == 0, _out=out_b if j == 1 else None, **kw)
+    assert torch.equal(den2, den) and torch.equal(mx2, mx)
+    dq2 = f32(B, S, H, D)
+    dq_o = torch.empty(B, S, H, D, dtype=dtype, device=DEV)
+    dk_o, dv_o = (torch.empty(B, 2 * S, H, D, dtype=dtype, device=DEV) for _ in range(2))
+    for j, (q_start, ks, k_start) in enumerate(steps):
+        # every K/V shard gets one call here: it is the first and the last one for its dk, dv (no fp32 array at all)
+        ra._blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], do[:, qs], (dq2, None, None, out_b, den2, mx2),
+                                    q_start, k_start, None, None, _delta=delta,
+                                    _grads_initial=(L.RA_GRAD_INIT_DQ if j == 0 else 0) | L.RA_GRAD_INIT_DKV,
+                                    _dq_out=dq_o if j == 1 else None, _dkv_out=(dk_o[:, ks], dv_o[:, ks]), **kw)
+    torch.cuda.synchronize()
+    for name, a, b in zip(("out", "dq", "dk", "dv"), ref, (out_b, dq_o, dk_o, dv_o)):
+        assert torch.equal(torch.nan_to_num(a.float()), torch.nan_to_num(b.float())), name
+
+
+def test_first_and_last_step_modes_reject_missing_buffers():
+    from ringattention_amd import ringattention_hip as rh
+    q, k, v, do = (t.to(DEV) for t in make_qkv(1, 64, 2, 32, dtype=torch.float32, seed=32))
+    den, mx = (torch.empty(1, 2, 64, dtype=torch.float32, device=DEV) for _ in range(2))
+    kw = dict(causal_block_size=1, query_chunk_size=16, key_chunk_size=16)
+    with pytest.raises(ValueError):       # no numerator, but the carry is not initial
+        ra._blockwise_attention_fwd(q, k, v, (None, den, mx), 0, 0, None, None, _out=torch.empty_like(q), **kw)
+    with pytest.raises(ValueError):       # no numerator and no out
+        ra._blockwise_attention_fwd(q, k, v, (None, den, mx), 0, 0, None, None, _carry_is_initial=True, **kw)
+    out = torch.empty_like(q)
+    delta = torch.zeros_like(den)
+    with pytest.raises(ValueError):       # dq missing although it is not the first call
+        ra._blockwise_attention_bwd(q, k, v, do, (None, torch.zeros_like(q), torch.zeros_like(q), out, den, mx), 0, 0,
+                                    None, None, _delta=delta, _dq_out=torch.empty_like(q), **kw)
