@@ -276,10 +276,11 @@ def bench_ffn(args):
         x.grad = None
         for p in ff.parameters():
             p.grad = None
-        y = ra.blockwise_feedforward(ff, x, chunk)
+        y = ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy)
         y.backward(dy)
 
     ms = _time_steps(step, args.steps, args.warmup)
+    kept = ra.feedforward._save_preactivations(args.ffn_policy, T, f, x.device)
     flops = 18.0 * T * d * f
     value = flops / (ms * 1e-3) / 1e12
     # dominant kernel: the GEMM a = x w1 of one launch (tokens_per_launch x hidden x intermediate), timed alone
@@ -309,6 +310,7 @@ def bench_ffn(args):
         "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "config": {"workload": "ffn", "tokens": T, "hidden": d, "intermediate": f, "chunk_size": chunk,
                    "tokens_per_launch": ra.feedforward._slab_tokens(chunk, T // chunk),
+                   "policy": args.ffn_policy, "preactivations": "kept (%.1f GB)" % (4e-9 * T * f) if kept else "recomputed",
                    "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
         "roofline": {"bound": "mfma", "kernel": "gemm_bf16_w4_kernel<false, false> (a = x w1 of one launch)",
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
@@ -503,6 +505,8 @@ def main():
                                                               "dropout32k"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--ffn-policy", default=None, choices=["nothing_saveable", "save_preactivations"],
+                    help="ffn workload: what blockwise_feedforward keeps for the backward pass (default: by size)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the ring is virtual); run with --gpus 1", file=sys.stderr)

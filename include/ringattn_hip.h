@@ -227,7 +227,7 @@ int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream);
  * SwiGLU feed-forward on one chunk of tokens, the body that blockwise_feedforward
  * (ringattention_jax.py:333-352) scans: y = (silu(x w1) * (x w3)) w2, bf16, fp32 accumulation.
  * x (T,d) ; w1,w3 (d,f) ; w2 (f,d) ; row-major.  a,b (T,f) bf16 are written by the forward
- * (pre-activations, recomputed or kept by the caller) and read by the backward.
+ * (pre-activations) and read by the backward, which recomputes them first unless preact_saved is set.
  */
 typedef struct ra_swiglu_params {
   int32_t T, d, f;
@@ -240,6 +240,9 @@ typedef struct ra_swiglu_params {
   float* dw1; float* dw2; float* dw3;   /* fp32 accumulators, added into (weights are broadcast
                                            over the scan, so their gradients sum over chunks) */
   void* da; void* db;             /* (T,f) bf16 scratch */
+  int32_t preact_saved;           /* backward: 1 = a and b still hold what the forward wrote for these tokens (the
+                                     caller kept them: `policy` other than nothing_saveable, ringattention_jax.py:334);
+                                     0 = recompute them from x (the reference's default policy) */
 } ra_swiglu_params;
 
 int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream);

@@ -77,6 +77,7 @@ class RaSwigluParams(C.Structure):
         ("x", vp), ("w1", vp), ("w2", vp), ("w3", vp),
         ("a", vp), ("b", vp), ("h", vp), ("y", vp),
         ("dy", vp), ("dx", vp), ("dw1", vp), ("dw2", vp), ("dw3", vp), ("da", vp), ("db", vp),
+        ("preact_saved", i32),
     ]
 
 

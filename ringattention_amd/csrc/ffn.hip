@@ -549,11 +549,13 @@ int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s) {
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s) {
   if (int rc = check_ffn_shape(p, "swiglu_bwd")) return rc;
   const int T = p->T, d = p->d, f = p->f;
-  // recompute the pre-activations (nothing_saveable), then
+  // recompute the pre-activations (nothing_saveable) unless the caller kept them, then
   //   dh = dy w2^T ; da, db from the activation ; dx = da w1^T + db w3^T
   //   dw1 += x^T da ; dw3 += x^T db ; dw2 += h^T dy
-  if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
-  if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
+  if (!p->preact_saved) {
+    if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
+    if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
+  }
   // dh goes into the da buffer first, the activation backward then rewrites it in place
   if (int rc = gemm_bf16(p->dy, p->w2, p->da, T, f, d, 0, 1, RA_BF16, 0, s)) return rc;
   const int64_t n8 = (int64_t)T * f / 8;

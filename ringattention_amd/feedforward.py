@@ -61,14 +61,20 @@ class _SwiGLUFn(torch.autograd.Function):
 class _BlockwiseSwiGLUFn(torch.autograd.Function):
     """The whole scan of blockwise_feedforward over a SwiGLU MLP as one autograd node: chunk after chunk
     through the same scratch buffers; in the backward pass the weight gradients of all chunks
-    accumulate in fp32 inside the GEMM epilogue and are rounded to the weights' dtype once."""
+    accumulate in fp32 inside the GEMM epilogue and are rounded to the weights' dtype once.
+    With ``save_preact`` the pre-activations x w1, x w3 of every chunk stay in memory for the backward pass
+    (2 * tokens * intermediate bf16 values); otherwise they are recomputed, the reference's default policy
+    (nothing_saveable, ringattention_jax.py:334).  The results are the same bits either way."""
 
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, chunk_tokens):
+    def forward(ctx, x, w1, w2, w3, chunk_tokens, save_preact):
         T, d = x.shape
         f = w1.shape[1]
         bf = dict(dtype=torch.bfloat16, device=x.device)
-        a, b, h = (torch.empty((chunk_tokens, f), **bf) for _ in range(3))
+        save_preact = bool(save_preact) and any(ctx.needs_input_grad[:4])
+        rows = T if save_preact else chunk_tokens
+        a, b = (torch.empty((rows, f), **bf) for _ in range(2))
+        h = torch.empty((chunk_tokens, f), **bf)
         y = torch.empty((T, d), **bf)
         lib, stream = L.load(), _stream()
         p = L.RaSwigluParams()
@@ -77,9 +83,12 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
         p.a, p.b, p.h = a.data_ptr(), b.data_ptr(), h.data_ptr()
         for t0 in range(0, T, chunk_tokens):
             p.x, p.y = x[t0:].data_ptr(), y[t0:].data_ptr()
+            if save_preact:
+                p.a, p.b = a[t0:].data_ptr(), b[t0:].data_ptr()
             L.check(lib.ra_swiglu_fwd(ctypes.byref(p), stream), "ra_swiglu_fwd")
         ctx.save_for_backward(x, w1, w2, w3)
         ctx.chunk_tokens = chunk_tokens
+        ctx.preact = (a, b) if save_preact else None
         return y
 
     @staticmethod
@@ -91,7 +100,10 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
         dev = x.device
         dy = dy.to(torch.bfloat16).contiguous()
         bf = dict(dtype=torch.bfloat16, device=dev)
-        a, b, h, da, db = (torch.empty((ct, f), **bf) for _ in range(5))
+        saved = ctx.preact is not None
+        a, b = ctx.preact if saved else (torch.empty((ct, f), **bf) for _ in range(2))
+        ctx.preact = None
+        h, da, db = (torch.empty((ct, f), **bf) for _ in range(3))
         dx = torch.empty((T, d), **bf)
         dw1 = torch.zeros((d, f), dtype=torch.float32, device=dev)
         dw3 = torch.zeros((d, f), dtype=torch.float32, device=dev)
@@ -103,10 +115,13 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
         p.a, p.b, p.h, p.y = a.data_ptr(), b.data_ptr(), h.data_ptr(), None
         p.dw1, p.dw2, p.dw3 = dw1.data_ptr(), dw2.data_ptr(), dw3.data_ptr()
         p.da, p.db = da.data_ptr(), db.data_ptr()
+        p.preact_saved = 1 if saved else 0
         for t0 in range(0, T, ct):
             p.x, p.dy, p.dx = x[t0:].data_ptr(), dy[t0:].data_ptr(), dx[t0:].data_ptr()
+            if saved:
+                p.a, p.b = a[t0:].data_ptr(), b[t0:].data_ptr()
             L.check(lib.ra_swiglu_bwd(ctypes.byref(p), stream), "ra_swiglu_bwd")
-        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None
+        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None, None
 
 
 # Tokens are independent in a token-wise MLP, so several consecutive chunks may share one launch: the
@@ -114,6 +129,27 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
 # accumulators are read and written once per slab instead of once per chunk.  The scratch of a slab
 # (five (tokens, intermediate) bf16 buffers) is what bounds it: 16384 tokens x 11008 is 1.8 GB.
 MAX_SLAB_TOKENS = 16384
+
+# policy=None keeps the pre-activations of the whole scan for the backward pass when they are small next to the
+# device's memory: at most this many bytes and at most a quarter of what is free.  65536 tokens x 11008 are 2.9 GB.
+PREACT_BUDGET_BYTES = 32 << 30
+
+
+def _save_preactivations(policy, tokens, intermediate, device):
+    """What ``policy`` (ringattention_jax.py:334) means here: "nothing_saveable" (the reference's default object,
+    by name) recomputes x w1 and x w3 in the backward pass; "save_preactivations" keeps them; None decides by
+    size.  Either way the same bits come out; only memory (4 * tokens * intermediate bytes) and two GEMMs per
+    chunk in the backward pass differ."""
+    if policy is None:
+        need = 4 * tokens * intermediate
+        free, _ = torch.cuda.mem_get_info(device)
+        return need <= PREACT_BUDGET_BYTES and need <= free // 4
+    name = policy if isinstance(policy, str) else getattr(policy, "__name__", "")
+    if name == "nothing_saveable":
+        return False
+    if name in ("save_preactivations", "everything_saveable"):
+        return True
+    raise ValueError("policy must be None, 'nothing_saveable' or 'save_preactivations'")
 
 
 def _slab_tokens(chunk_size, n_chunks):
@@ -153,8 +189,10 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
     The reference groups tokens with 'b (c n) d -> b c n d', c=chunk_size and scans over n, so step
     j sees the strided token set {ci * n + j}.  A generic callable gets exactly those groups.  A
     ``SwiGLU`` instance is token-wise, so it is fed contiguous slabs of chunk_size tokens instead:
-    the same number of steps and the same result, with dense memory access.  ``policy`` /
-    ``pre_remat`` / ``static_argnums`` steer XLA rematerialisation only; SwiGLU always recomputes."""
+    the same number of steps and the same result, with dense memory access.  ``policy`` selects what the
+    SwiGLU scan keeps for its backward pass (see _save_preactivations: the reference's default recomputes
+    everything to save memory; with None the pre-activations are kept when they are small next to the device's
+    memory); ``pre_remat`` / ``static_argnums`` steer XLA rematerialisation only."""
     b, s, d = inputs.shape
     if s % chunk_size:
         raise ValueError("sequence length %d must divide by chunk_size %d" % (s, chunk_size))
@@ -167,7 +205,8 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
         # contiguous slabs of chunk_size tokens (batch rows one after the other: a token-wise MLP does not see the
         # difference), one autograd node for the whole scan
         y = _BlockwiseSwiGLUFn.apply(inputs.reshape(b * s, d).contiguous(), feedforward.w1, feedforward.w2,
-                                     feedforward.w3, _slab_tokens(chunk_size, b * n))
+                                     feedforward.w3, _slab_tokens(chunk_size, b * n),
+                                     _save_preactivations(policy, b * s, feedforward.w1.shape[1], inputs.device))
         return y.reshape(b, s, y.shape[-1])
     x = inputs.reshape(b, chunk_size, n, d)
     outs = [feedforward(x[:, :, j, :]) for j in range(n)]

@@ -130,3 +130,36 @@ def test_blockwise_feedforward_single_batch_scan_gradients():
     rel_ok(ff.w1.grad, w1.grad, "dw1")
     rel_ok(ff.w2.grad, w2.grad, "dw2")
     rel_ok(ff.w3.grad, w3.grad, "dw3")
+
+
+def test_blockwise_feedforward_policies_give_the_same_bits(monkeypatch):
+    """policy="nothing_saveable" (the reference's default: the backward pass recomputes x w1 and x w3), policy=
+    "save_preactivations" (they stay in memory) and policy=None (decided by size) differ in memory and in two GEMMs
+    per chunk, not in a single bit of y, dx or the weight gradients."""
+    from ringattention_amd import feedforward as F
+    S, d, f, chunk = 2048, 256, 512, 256
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(2, S, d, generator=g).bfloat16().to(DEV)
+    dy = torch.randn(2, S, d, generator=g).bfloat16().to(DEV)
+    ff = ra.SwiGLU(d, f, device=DEV, init_std=0.05)
+    monkeypatch.setattr(F, "MAX_SLAB_TOKENS", 1024)        # several slabs, so that the kept buffers are sliced
+    res = {}
+    for policy in ("nothing_saveable", "save_preactivations", None):
+        for prm in ff.parameters():
+            prm.grad = None
+        xd = x.clone().requires_grad_(True)
+        y = ra.blockwise_feedforward(ff, xd, chunk, policy=policy)
+        y.backward(dy)
+        res[policy] = (y.detach(), xd.grad, ff.w1.grad.clone(), ff.w2.grad.clone(), ff.w3.grad.clone())
+    for policy in ("save_preactivations", None):
+        for a, b in zip(res[policy], res["nothing_saveable"]):
+            assert torch.equal(a, b), policy
+    # the decision by size
+    assert F._save_preactivations(None, 65536, 11008, x.device) is True
+    monkeypatch.setattr(F, "PREACT_BUDGET_BYTES", 1 << 20)
+    assert F._save_preactivations(None, 65536, 11008, x.device) is False
+    with pytest.raises(ValueError):
+        ra.blockwise_feedforward(ff, x, chunk, policy="dots_saveable")
+    # no gradient wanted: nothing is kept
+    with torch.no_grad():
+        assert torch.equal(ra.blockwise_feedforward(ff, x, chunk, policy="save_preactivations"), res[None][0])
