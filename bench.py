@@ -23,7 +23,7 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters'
 # reading for the 1 GiB copy of --workload copy) at the default sizes of each workload
-MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.47e9, "attn_bwd_dkv_ws_kernel": 5.79e9, "attn_bwd_dq_ws_kernel": 4.44e9,
+MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.37e9, "attn_bwd_dkv_ws_kernel": 4.25e9, "attn_bwd_dq_ws_kernel": 3.47e9,
                     "decode_split_kernel": 68.88e9, "gemm_bf16_w4_kernel<false, false>": 2.55e9,
                     "rmsnorm_fwd_kernel": 2.15e9}
 
@@ -134,23 +134,25 @@ def bench_attention(args, ring, dropout=False):
         with torch.no_grad():
             cfg = rh._Config(kw)
             mi = rh._MaskInputs(cfg, None, None, None, B, q.device, S)
-            num = torch.empty(B, S, H, D, dtype=torch.float32, device=dev)
+            # the launches of the step: one ring step that is the first and the last of its device, so there is no
+            # fp32 numerator or gradient array: out and dq / dk / dv are written once, in bf16
+            from ringattention_amd import _lib as L
             den = torch.empty(B, H, S, dtype=torch.float32, device=dev)
             mx = torch.empty(B, H, S, dtype=torch.float32, device=dev)
             qd, kd, vd = q.detach(), k.detach(), v.detach()
-            fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (num, den, mx), 0, 0, None, None, 1, 512, 512,
-                                                      _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True)
+            out = torch.empty_like(qd)
+            fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (None, den, mx), 0, 0, None, None, 1, 512, 512,
+                                                      _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True, _out=out)
             fwd()            # under dropout the first call draws and packs the mask, which stays with mi
             kern["attn_fwd_ws_kernel"] = (_event_ms(fwd, 5), flops_fwd)
-            out = torch.empty_like(qd)
-            rh._finalize(num, den, out)
             delta = rh._bwd_delta(do, out)
-            dq = torch.zeros(B, S, H, D, dtype=torch.float32, device=dev)
-            dk, dv = torch.zeros_like(dq), torch.zeros_like(dq)
+            dq_o, dk_o, dv_o = (torch.empty_like(qd) for _ in range(3))
             for which, share in (("dkv", 8.0), ("dq", 2.0)):
                 cfg1 = rh._Config(dict(kw, bwd_only=which))
-                bw = lambda: rh._blockwise_attention_bwd(qd, kd, vd, do, (dq, dk, dv, out, den, mx), 0, 0, None, None,
-                                                         1, 512, 512, _mask_inputs=mi, _cfg=cfg1, _delta=delta)
+                bw = lambda: rh._blockwise_attention_bwd(qd, kd, vd, do, (None, None, None, out, den, mx), 0, 0, None,
+                                                         None, 1, 512, 512, _mask_inputs=mi, _cfg=cfg1, _delta=delta,
+                                                         _grads_initial=L.RA_GRAD_INIT_DQ | L.RA_GRAD_INIT_DKV,
+                                                         _dq_out=dq_o, _dkv_out=(dk_o, dv_o))
                 kern["attn_bwd_%s_ws_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
             if dropout:
                 def draw():
