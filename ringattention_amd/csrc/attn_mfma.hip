@@ -185,6 +185,15 @@ __device__ __forceinline__ void store_bf16x4(uint16_t* p, const f32x4& t) {
   for (int e = 0; e < 4; e++) o[e] = (__bf16)t[e];
   *(bf16x4_t*)p = o;
 }
+// 16-byte loads through a buffer descriptor: scalar base, scalar offset, one 32-bit byte offset per lane
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const uint16_t* p) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
+  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
+  return uint4{v[0], v[1], v[2], v[3]};
+}
 // The rows of a gradient that a workgroup owns but has nothing to add to (rows x HD floats from acc / out, which
 // point at row 0, head h): hand the accumulator on as bf16, or set it to the zeros it holds by definition.
 __device__ __forceinline__ void pass_rows(float* acc, int64_t acc_ss, uint16_t* out, int64_t out_ss, int rows,
@@ -311,10 +320,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   // ---- staging of the Q / dO tiles through registers: producers bring Q, consumers dO and the statistics
   const int srow = (tid & 255) >> 4, schunk = tid & 15;
   const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const uint16_t* sg = (role == 0 ? a.q : a.g) + (int64_t)b * a.q_sb + (int64_t)h * HD + schunk * 8 +
-                       (int64_t)(qt_first * KBM + srow) * a.q_ss;
+  // a tile is read through a buffer descriptor at its first row (scalar registers) with one 32-bit byte offset per
+  // lane: half the address data of 64-bit pointers per lane, and two registers less
+  const uint16_t* sg = (role == 0 ? a.q : a.g) + (int64_t)b * a.q_sb + (int64_t)h * HD + (int64_t)(qt_first * KBM) * a.q_ss;
+  const uint32_t sg_lane = 2u * (uint32_t)(schunk * 8 + srow * (int)a.q_ss);
+  const uint32_t row16b = 2u * 16u * (uint32_t)a.q_ss;
   uint16_t* sl = (role == 0 ? Qs : Gs) + s_off;
-  const int64_t row16 = 16 * a.q_ss;
   uint4 sr0, sr1, sr2, sr3;
   float r_m = 0.f, r_den = 1.f, r_delta = 0.f;
   int r_seg = 0;
@@ -325,9 +336,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #define RA_WS_LOAD(T)                                                                                   \
   {                                                                                                     \
     const int t_ = min((T), ntq - 1);                                                                   \
-    const uint16_t* p_ = sg + (int64_t)t_ * KBM * a.q_ss;                                               \
-    sr0 = *(const uint4*)(p_); sr1 = *(const uint4*)(p_ + row16);                                       \
-    sr2 = *(const uint4*)(p_ + 2 * row16); sr3 = *(const uint4*)(p_ + 3 * row16);                       \
+    const __amdgpu_buffer_rsrc_t rs_ = tile_rsrc(sg + (int64_t)t_ * KBM * a.q_ss);                      \
+    sr0 = ld_buf(rs_, sg_lane, 0); sr1 = ld_buf(rs_, sg_lane, row16b);                                  \
+    sr2 = ld_buf(rs_, sg_lane, 2 * row16b); sr3 = ld_buf(rs_, sg_lane, 3 * row16b);                     \
     if (tid >= 256 && tid < 256 + KBM) {                                                                \
       const int row_ = (qt_first + t_) * KBM + tid - 256;                                               \
       const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
@@ -742,10 +753,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   // stored to LDS two tiles (four steps) later
   const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
   const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const int64_t sg_off = (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
-  const uint16_t* sgk = a.k + sg_off;
-  const uint16_t* sgv = a.v + sg_off;
-  const int64_t row16 = 16 * a.kv_ss;
+  // a tile is read through a buffer descriptor at its first row (scalar registers) with one 32-bit byte offset per
+  // lane: half the address data of 64-bit pointers per lane, and two registers less
+  const int64_t sg_base = (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
+  const uint32_t sg_lane = 2u * (uint32_t)(schunk * 8 + srow * (int)a.kv_ss);
+  const uint32_t row16b = 2u * 16u * (uint32_t)a.kv_ss;
   uint4 Ak0, Ak1, Ak2, Ak3, Av0, Av1, Av2, Av3, Bk0, Bk1, Bk2, Bk3, Bv0, Bv1, Bv2, Bv3;
   int Aseg = 0, Bseg = 0;
   float Abias = 0.f, Bbias = 0.f;
@@ -758,9 +770,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #define RA_WS_LOAD_K(S, T)                                                                               \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
-    const uint16_t* pk_ = sgk + (int64_t)t_ * FBN * a.kv_ss;                                            \
-    S##k0 = *(const uint4*)(pk_); S##k1 = *(const uint4*)(pk_ + row16);                                 \
-    S##k2 = *(const uint4*)(pk_ + 2 * row16); S##k3 = *(const uint4*)(pk_ + 3 * row16);                 \
+    const __amdgpu_buffer_rsrc_t rk_ = tile_rsrc(a.k + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
+    S##k0 = ld_buf(rk_, sg_lane, 0); S##k1 = ld_buf(rk_, sg_lane, row16b);                              \
+    S##k2 = ld_buf(rk_, sg_lane, 2 * row16b); S##k3 = ld_buf(rk_, sg_lane, 3 * row16b);                 \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
@@ -775,9 +787,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #define RA_WS_LOAD_V(S, T)                                                                               \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
-    const uint16_t* pv_ = sgv + (int64_t)t_ * FBN * a.kv_ss;                                            \
-    S##v0 = *(const uint4*)(pv_); S##v1 = *(const uint4*)(pv_ + row16);                                 \
-    S##v2 = *(const uint4*)(pv_ + 2 * row16); S##v3 = *(const uint4*)(pv_ + 3 * row16);                 \
+    const __amdgpu_buffer_rsrc_t rv_ = tile_rsrc(a.v + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
+    S##v0 = ld_buf(rv_, sg_lane, 0); S##v1 = ld_buf(rv_, sg_lane, row16b);                              \
+    S##v2 = ld_buf(rv_, sg_lane, 2 * row16b); S##v3 = ld_buf(rv_, sg_lane, 3 * row16b);                 \
   }
 #define RA_WS_STORE_K(S, BUF)                                                                            \
   {                                                                                                     \
@@ -1220,10 +1232,11 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   // LDS stores waited for L2 misses often enough to cost the forward kernel 16 %.
   const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
   const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
-  const int64_t sg_off = (int64_t)b * a.kv_sb + (int64_t)h * HD + schunk * 8 + (int64_t)(k_base + srow) * a.kv_ss;
-  const uint16_t* sgk = a.k + sg_off;
-  const uint16_t* sgv = a.v + sg_off;
-  const int64_t row16 = 16 * a.kv_ss;
+  // a tile is read through a buffer descriptor at its first row (scalar registers) with one 32-bit byte offset per
+  // lane: half the address data of 64-bit pointers per lane, and two registers less
+  const int64_t sg_base = (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
+  const uint32_t sg_lane = 2u * (uint32_t)(schunk * 8 + srow * (int)a.kv_ss);
+  const uint32_t row16b = 2u * 16u * (uint32_t)a.kv_ss;
   uint4 Ak0, Ak1, Ak2, Ak3, Av0, Av1, Av2, Av3, Bk0, Bk1, Bk2, Bk3, Bv0, Bv1, Bv2, Bv3;
   int Aseg = 0, Bseg = 0;
   float Abias = 0.f, Bbias = 0.f;
@@ -1236,9 +1249,9 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #define RA_WS_LOAD_K(S, T)                                                                               \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
-    const uint16_t* pk_ = sgk + (int64_t)t_ * FBN * a.kv_ss;                                            \
-    S##k0 = *(const uint4*)(pk_); S##k1 = *(const uint4*)(pk_ + row16);                                 \
-    S##k2 = *(const uint4*)(pk_ + 2 * row16); S##k3 = *(const uint4*)(pk_ + 3 * row16);                 \
+    const __amdgpu_buffer_rsrc_t rk_ = tile_rsrc(a.k + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
+    S##k0 = ld_buf(rk_, sg_lane, 0); S##k1 = ld_buf(rk_, sg_lane, row16b);                              \
+    S##k2 = ld_buf(rk_, sg_lane, 2 * row16b); S##k3 = ld_buf(rk_, sg_lane, 3 * row16b);                 \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
@@ -1253,9 +1266,9 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #define RA_WS_LOAD_V(S, T)                                                                               \
   {                                                                                                     \
     const int t_ = min((T), ntiles - 1);                                                                \
-    const uint16_t* pv_ = sgv + (int64_t)t_ * FBN * a.kv_ss;                                            \
-    S##v0 = *(const uint4*)(pv_); S##v1 = *(const uint4*)(pv_ + row16);                                 \
-    S##v2 = *(const uint4*)(pv_ + 2 * row16); S##v3 = *(const uint4*)(pv_ + 3 * row16);                 \
+    const __amdgpu_buffer_rsrc_t rv_ = tile_rsrc(a.v + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
+    S##v0 = ld_buf(rv_, sg_lane, 0); S##v1 = ld_buf(rv_, sg_lane, row16b);                              \
+    S##v2 = ld_buf(rv_, sg_lane, 2 * row16b); S##v3 = ld_buf(rv_, sg_lane, 3 * row16b);                 \
   }
 #define RA_WS_STORE_K(S, BUF)                                                                            \
   {                                                                                                     \
