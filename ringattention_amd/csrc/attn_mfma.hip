@@ -443,7 +443,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       float x = SC[(G) * 4 + e] * c;                                                                    \
       bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
       if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
-      if (HAS_KEEP == 2) {                                                                              \
+      if (HAS_KEEP == 2 && HAS_SEG) {                                                                   \
+        /* as below, with the segment ids: a pair of two documents counts as masked once more */        \
+        const bool sne_ = st_seg[BUF][qrow0 + e] != seg_k;                                              \
+        x = (((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) && !sne_) ? x : kMask2;                       \
+        x = (((kw_some >> ((BLK) * 32 + (G) * 8 + e)) & 1) &&                                           \
+             (((kw_k >> ((BLK) * 32 + (G) * 8 + e)) & 1) || !sne_)) ? x : RA_NEG_INF;                   \
+      } else if (HAS_KEEP == 2) {                                                                       \
         /* dropout adds mask_min (:321).  kw_cur: pairs kept and causally allowed; kw_some: at least    \
            one of the two, so a clear bit there is mask_min added twice = -inf */                       \
         x = ((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) ? x : kMask2;                                  \
@@ -494,8 +500,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     // packed keep mask: this lane's word (bits over the 64 rows of a query tile) and this pair's summary byte
     const uint64_t* kw_ptr = nullptr;
     const uint8_t* ks_ptr = nullptr;
-    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0;
-    (void)kw_some;
+    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0, kw_k = 0;     // kw_k: the kept bits before the causal limit is folded in
+    (void)kw_some; (void)kw_k;
     int ks_cur = 2, ks_nxt = 2;
     if (HAS_KEEP) {
       kw_ptr = mv.kbits_q + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
@@ -540,6 +546,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
         if (HAS_KEEP == 2) {               // fold this key's causal limit (rows before qlim are masked) into the words
           const int nmask = (int)max(0LL, min(64LL, (long long)qlim - gq_tile));
           const uint64_t cw = (nmask >= 64 ? 0ULL : (~0ULL << nmask)) >> (4 * hi);
+          kw_k = kw_cur;
           kw_some = kw_cur | cw;
           kw_cur &= cw;
         }
@@ -887,7 +894,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
         float x = SC[(G) * 4 + e] * c;                                                                  \
         bool masked = (gk_tile + kr_ >= klim);                                                          \
         if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
-        if (HAS_KEEP == 2) {                                                                            \
+        if (HAS_KEEP == 2 && HAS_SEG) {                                                                 \
+          /* as below, with the segment ids: a pair of two documents counts as masked once more */      \
+          const bool sne_ = seg_ks[BUF][kr_] != seg_q;                                                  \
+          x = (((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) && !sne_) ? x : kMask2;                     \
+          x = (((kw_some >> ((BLK) * 32 + (G) * 8 + e)) & 1) &&                                         \
+               (((kw_k >> ((BLK) * 32 + (G) * 8 + e)) & 1) || !sne_)) ? x : RA_NEG_INF;                 \
+        } else if (HAS_KEEP == 2) {                                                                     \
           /* dropout adds mask_min (:321).  kw_cur: pairs kept and causally allowed; kw_some: at least  \
              one of the two, so a clear bit there is mask_min added twice = -inf */                     \
           x = ((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) ? x : kMask2;                                \
@@ -945,8 +958,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     const int t_causal = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
     const uint64_t* kw_ptr = nullptr;
     const uint8_t* ks_ptr = nullptr;
-    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0;
-    (void)kw_some;
+    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0, kw_k = 0;     // kw_k: the kept bits before the causal limit is folded in
+    (void)kw_some; (void)kw_k;
     if (HAS_KEEP) {
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
                (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + (gk0 - mv.keep_k0) / 64;
@@ -1002,6 +1015,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       if (HAS_KEEP == 2) {             /* fold this row's causal limit into the words */                \
         const int nall_ = max(0, min(64, klim - gk_tile));                                              \
         const uint64_t cw_ = (nall_ >= 64 ? ~0ULL : ((1ULL << nall_) - 1ULL)) >> (4 * hi);              \
+        kw_k = kw_cur;                                                                                  \
         kw_some = kw_cur | cw_;                                                                         \
         kw_cur &= cw_;                                                                                  \
       }                                                                                                 \
@@ -1366,7 +1380,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
         float x_ = SC[r] * c;                                                                           \
         bool masked_ = (gk_tile + kr_ >= klim);                                                         \
         if (HAS_SEG) masked_ = masked_ || (seg_ks[BUF][kr_] != seg_q);                                  \
-        if (HAS_KEEP == 2) {                                                                            \
+        if (HAS_KEEP == 2 && HAS_SEG) {                                                                 \
+          /* as below, with the segment ids: a pair of two documents counts as masked once more */      \
+          const bool sne_ = seg_ks[BUF][kr_] != seg_q;                                                  \
+          x_ = (((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) && !sne_) ? x_ : kMask2;        \
+          x_ = (((kw_some >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) &&                             \
+                (((kw_k >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) || !sne_)) ? x_ : RA_NEG_INF;    \
+        } else if (HAS_KEEP == 2) {                                                                     \
           /* dropout adds mask_min (:321).  kw_cur: pairs kept and causally allowed; kw_some: at least  \
              one of the two, so a clear bit there is mask_min added twice = -inf */                     \
           x_ = ((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) ? x_ : kMask2;                   \
@@ -1438,8 +1458,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const int t_causal = (int)max(0LL, min((long long)ntiles, ((long long)klim_wave - gk0) / FBN));
     const uint64_t* kw_ptr = nullptr;
     const uint8_t* ks_ptr = nullptr;
-    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0;
-    (void)kw_some;
+    uint64_t kw_cur = 0, kw_nxt = 0, kw_some = 0, kw_k = 0;     // kw_k: the kept bits before the causal limit is folded in
+    (void)kw_some; (void)kw_k;
     if (HAS_KEEP) {
       ks_ptr = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh +
                (int64_t)((mv.keep_q0 + q0 + pair * 32) / 64) * (mv.keep_K / 64) + (gk0 - mv.keep_k0) / 64;
@@ -1495,6 +1515,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
       if (HAS_KEEP == 2) {             /* fold this row's causal limit into the words */                \
         const int nall_ = max(0, min(64, klim - gk_tile));                                              \
         const uint64_t cw_ = (nall_ >= 64 ? ~0ULL : ((1ULL << nall_) - 1ULL)) >> (4 * hi);              \
+        kw_k = kw_cur;                                                                                  \
         kw_some = kw_cur | cw_;                                                                         \
         kw_cur &= cw_;                                                                                  \
       }                                                                                                 \
@@ -1661,11 +1682,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 // ------------------------------------------------------------------ host side
 static bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
-// a boolean keep mask is taken in packed form only, next to a causal block size at most (no bias or segment ids:
-// ring_attention_inference has neither, and the generic kernels serve any combination)
+// a boolean keep mask is taken in packed form only; the attn_mask of ring_attention_inference next to a causal block
+// size at most (it has no bias or segment ids there; the generic kernels serve any combination), the dropout mask
+// next to everything
 static bool keep_ok(const ra_mask& m) {
   if (!m.keep && !m.keep_bits_k) return true;
-  return m.keep_bits_k && m.keep_bits_q && m.keep_summary && !m.bias && !m.segment_ids;
+  if (!(m.keep_bits_k && m.keep_bits_q && m.keep_summary)) return false;
+  return m.keep_mode == RA_KEEP_DROPOUT || (!m.bias && !m.segment_ids);
 }
 
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
@@ -1693,8 +1716,12 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
   RA_REQUIRE(nwg3 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
   dim3 grid3((unsigned)((nwg3 + 7) / 8 * 8)), block3(512);
-  if (keep && p->mask.keep_mode == RA_KEEP_DROPOUT) attn_fwd_ws_kernel<false, false, 2><<<grid3, block3, 0, s>>>(a);
-  else if (keep) attn_fwd_ws_kernel<false, false, 1><<<grid3, block3, 0, s>>>(a);
+  if (keep && p->mask.keep_mode == RA_KEEP_DROPOUT) {
+    if (seg && bias) attn_fwd_ws_kernel<true, true, 2><<<grid3, block3, 0, s>>>(a);
+    else if (seg) attn_fwd_ws_kernel<true, false, 2><<<grid3, block3, 0, s>>>(a);
+    else if (bias) attn_fwd_ws_kernel<false, true, 2><<<grid3, block3, 0, s>>>(a);
+    else attn_fwd_ws_kernel<false, false, 2><<<grid3, block3, 0, s>>>(a);
+  } else if (keep) attn_fwd_ws_kernel<false, false, 1><<<grid3, block3, 0, s>>>(a);
   else if (seg && bias) attn_fwd_ws_kernel<true, true><<<grid3, block3, 0, s>>>(a);
   else if (seg) attn_fwd_ws_kernel<true, false><<<grid3, block3, 0, s>>>(a);
   else if (bias) attn_fwd_ws_kernel<false, true><<<grid3, block3, 0, s>>>(a);
@@ -1741,8 +1768,12 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
     if (do_dkv) attn_bwd_dkv_ws_kernel<__VA_ARGS__><<<gk, block, 0, s>>>(a);             \
     if (do_dq) attn_bwd_dq_ws_kernel<__VA_ARGS__><<<gq, block, 0, s>>>(a);               \
   } while (0)
-  if (p->mask.keep_bits_k && p->mask.keep_mode == RA_KEEP_DROPOUT) RA_LAUNCH_BWD(false, false, 2);
-  else if (p->mask.keep_bits_k) RA_LAUNCH_BWD(false, false, 1);      // packed boolean mask
+  if (p->mask.keep_bits_k && p->mask.keep_mode == RA_KEEP_DROPOUT) {
+    if (seg && bias) RA_LAUNCH_BWD(true, true, 2);
+    else if (seg) RA_LAUNCH_BWD(true, false, 2);
+    else if (bias) RA_LAUNCH_BWD(false, true, 2);
+    else RA_LAUNCH_BWD(false, false, 2);
+  } else if (p->mask.keep_bits_k) RA_LAUNCH_BWD(false, false, 1);      // packed boolean mask
   else if (seg && bias) RA_LAUNCH_BWD(true, true);
   else if (seg) RA_LAUNCH_BWD(true, false);
   else if (bias) RA_LAUNCH_BWD(false, true);
