@@ -177,9 +177,14 @@ int ra_dropout_keep(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32
                     ra_stream_t stream);
 /* The same mask written directly in the packed form of ra_keep_pack (Q and K multiples of 64), without the byte
  * array: what ra_keep_pack would make of ra_dropout_keep's output.  The attention entry points take the packed
- * form alone (ra_mask.keep null). */
+ * form alone (ra_mask.keep null).  With causal_block_size > 0 (and the chunk sizes and chunk starts of the ring step
+ * the mask is for, as in ra_mask) only the 64 x 64 tiles of chunk pairs that below_or_on_diag lets run
+ * (ringattention_jax.py:324-331) are written - about half of them in causal self-attention - and the others are left
+ * as they are: no kernel reads them.  The bits of a position do not depend on which tiles are written. */
 int ra_dropout_keep_packed(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K,
-                           uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, ra_stream_t stream);
+                           uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, int32_t causal_block_size,
+                           int32_t query_chunk_size, int32_t key_chunk_size, int32_t q_chunk_idx_start,
+                           int32_t k_chunk_idx_start, ra_stream_t stream);
 
 /* Carry initialisation (ringattention_jax.py:22-23,:49): numerator = 0, denominator = 0, max = -inf. */
 int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s,

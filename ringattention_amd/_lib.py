@@ -106,7 +106,7 @@ SYMBOLS = {
     "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
     "ra_keep_pack": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]),
     "ra_dropout_keep": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp]),
-    "ra_dropout_keep_packed": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp, vp, vp]),
+    "ra_dropout_keep_packed": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),

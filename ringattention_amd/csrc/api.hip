@@ -30,7 +30,8 @@ int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
 int keep_pack(const uint8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, uint64_t*, uint64_t*, uint8_t*, hipStream_t);
 int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hipStream_t s);
 int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, int K, uint64_t* bits_k,
-                        uint64_t* bits_q, uint8_t* summary, hipStream_t s);
+                        uint64_t* bits_q, uint8_t* summary, int cbs, int qc, int kc, int q_start, int k_start,
+                        hipStream_t s);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
@@ -180,15 +181,25 @@ int ra_dropout_keep(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32
 }
 
 int ra_dropout_keep_packed(uint64_t seed, float attn_pdrop, int32_t B, int32_t H, int32_t Q, int32_t K,
-                           uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, ra_stream_t stream) {
+                           uint64_t* bits_k, uint64_t* bits_q, uint8_t* summary, int32_t causal_block_size,
+                           int32_t query_chunk_size, int32_t key_chunk_size, int32_t q_chunk_idx_start,
+                           int32_t k_chunk_idx_start, ra_stream_t stream) {
   RA_REQUIRE(bits_k && bits_q && summary, RA_ERR_INVALID, "dropout_keep_packed: null pointer");
   RA_REQUIRE(B > 0 && H > 0 && (long long)B * H <= 65535, RA_ERR_INVALID, "dropout_keep_packed: bad plane count");
   RA_REQUIRE(Q > 0 && K > 0 && Q % 64 == 0 && K % 64 == 0 && Q / 64 <= 65535, RA_ERR_UNSUPPORTED,
              "dropout_keep_packed: Q and K must be positive multiples of 64 (got %d, %d)", Q, K);
   RA_REQUIRE(attn_pdrop > 0.f && attn_pdrop < 1.f, RA_ERR_INVALID,
              "dropout_keep_packed: attn_pdrop must lie in (0, 1)");
+  if (causal_block_size > 0) {
+    const int cbs = causal_block_size, qc = query_chunk_size, kc = key_chunk_size;
+    RA_REQUIRE(qc > 0 && kc > 0 && Q % qc == 0 && K % kc == 0 && q_chunk_idx_start >= 0 && k_chunk_idx_start >= 0 &&
+                   (cbs <= qc || cbs % qc == 0) && (cbs <= kc || cbs % kc == 0),
+               RA_ERR_INVALID, "dropout_keep_packed: chunk sizes must divide Q and K, and a causal_block_size larger "
+                               "than a chunk must be a multiple of it");
+  }
   return dropout_keep_packed(seed, dropout_threshold(attn_pdrop), B * H, Q, K, bits_k, bits_q, summary,
-                             (hipStream_t)stream);
+                             causal_block_size, query_chunk_size, key_chunk_size, q_chunk_idx_start,
+                             k_chunk_idx_start, (hipStream_t)stream);
 }
 
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {

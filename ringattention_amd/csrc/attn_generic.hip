@@ -514,8 +514,11 @@ int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hi
 // blocks) and the columns' words come from 64 ballots.  Writes what keep_pack_kernel would write for the byte form.
 __global__ __launch_bounds__(64) void dropout_keep_packed_kernel(uint32_t k0, uint32_t k1, uint32_t threshold, int Q,
                                                                  int K, uint64_t* bits_k, uint64_t* bits_q,
-                                                                 uint8_t* summary) {
+                                                                 uint8_t* summary, MaskView run) {
   const int kt = blockIdx.x, qt = blockIdx.y, plane = blockIdx.z, i = threadIdx.x;
+  // under a causal block size only the chunk pairs that run (:324-331) are ever read: leave the other tiles alone.
+  // (The chunk of the tile's last row runs the longest key prefix of the tile's rows.)
+  if (run.cbs > 0 && kt * 64 >= run.run_prefix_keys((qt * 64 + 63) / run.qc, K)) return;
   const int64_t e0 = ((int64_t)plane * Q + qt * 64 + i) * K + (int64_t)kt * 64;
   uint64_t wrow = 0;
 #pragma unroll
@@ -535,10 +538,13 @@ __global__ __launch_bounds__(64) void dropout_keep_packed_kernel(uint32_t k0, ui
 }
 
 int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, int K, uint64_t* bits_k,
-                        uint64_t* bits_q, uint8_t* summary, hipStream_t s) {
+                        uint64_t* bits_q, uint8_t* summary, int cbs, int qc, int kc, int q_start, int k_start,
+                        hipStream_t s) {
   dim3 grid(K / 64, Q / 64, planes);
+  MaskView run{};
+  run.cbs = cbs; run.qc = qc; run.kc = kc; run.q_start = q_start; run.k_start = k_start;
   dropout_keep_packed_kernel<<<grid, 64, 0, s>>>((uint32_t)seed, (uint32_t)(seed >> 32), threshold, Q, K, bits_k,
-                                                 bits_q, summary);
+                                                 bits_q, summary, run);
   RA_CHECK_LAUNCH("dropout_keep_packed");
   return RA_OK;
 }

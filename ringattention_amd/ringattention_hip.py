@@ -264,9 +264,11 @@ class _MaskInputs:
             bits_k = torch.empty((batch, heads, words), dtype=torch.int64, device=device)
             bits_q = torch.empty((batch, heads, words), dtype=torch.int64, device=device)
             summ = torch.empty((batch, heads, words // 64), dtype=torch.uint8, device=device)
+            # (only the tiles of chunk pairs that run under the causal block size: nothing else is read)
             L.check(L.load().ra_dropout_keep_packed(cfg.seed, cfg.pdrop, batch, heads, q_len, kv_len,
                                                     bits_k.data_ptr(), bits_q.data_ptr(), summ.data_ptr(),
-                                                    _stream()), "ra_dropout_keep_packed")
+                                                    cfg.cbs or 0, cfg.qc, cfg.kc, 0, 0, _stream()),
+                    "ra_dropout_keep_packed")
             self._drop_steps[key] = (None, (bits_k, bits_q, summ, q_len, kv_len))
         if key not in self._drop_steps:
             if self._drop_base is None:

@@ -44,11 +44,24 @@ def test_packed_dropout_mask_equals_packing_the_byte_mask(shape, seed, p):
     a, b = mk(), mk()
     L.check(lib.ra_keep_pack(keep.data_ptr(), keep.stride(0), keep.stride(1), keep.stride(2), keep.stride(3), B, H, Q,
                              K, a[0].data_ptr(), a[1].data_ptr(), a[2].data_ptr(), None), "ra_keep_pack")
-    L.check(lib.ra_dropout_keep_packed(seed, p, B, H, Q, K, b[0].data_ptr(), b[1].data_ptr(), b[2].data_ptr(), None),
-            "ra_dropout_keep_packed")
+    L.check(lib.ra_dropout_keep_packed(seed, p, B, H, Q, K, b[0].data_ptr(), b[1].data_ptr(), b[2].data_ptr(),
+                                       0, 0, 0, 0, 0, None), "ra_dropout_keep_packed")
     torch.cuda.synchronize()
     for x, y in zip(a, b):
         assert torch.equal(x, y)
+    # under a causal block size only the tiles of chunk pairs that run are written, with the same bits
+    c = mk()
+    L.check(lib.ra_dropout_keep_packed(seed, p, B, H, Q, K, c[0].data_ptr(), c[1].data_ptr(), c[2].data_ptr(),
+                                       1, 64, 64, 0, 0, None), "ra_dropout_keep_packed")
+    torch.cuda.synchronize()
+    qt, kt = Q // 64, K // 64
+    run = torch.tensor([[ra.below_or_on_diag(i, 64, j, 64, 1) for j in range(kt)] for i in range(qt)], device=DEV)
+    summ_full, summ_run = b[2].view(B, H, qt, kt), c[2].view(B, H, qt, kt)
+    assert torch.equal(summ_run[:, :, run], summ_full[:, :, run]) and bool((summ_run[:, :, ~run] == 9).all())
+    wk_full, wk_run = b[0].view(B, H, kt, qt, 64), c[0].view(B, H, kt, qt, 64)       # [kt][q] words
+    assert torch.equal(wk_run[:, :, run.t()], wk_full[:, :, run.t()]) and bool((wk_run[:, :, ~run.t()] == 0).all())
+    wq_full, wq_run = b[1].view(B, H, qt, kt, 64), c[1].view(B, H, qt, kt, 64)       # [qt][k] words
+    assert torch.equal(wq_run[:, :, run], wq_full[:, :, run]) and bool((wq_run[:, :, ~run] == 0).all())
 
 
 def test_dropout_mask_rejects():
