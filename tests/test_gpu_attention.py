@@ -47,7 +47,7 @@ def check_case(B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, dtype, impl="auto"
             assert_close(a, b, dtype, name)
 
 
-# --- BASELINE config 1: the reference's own CPU-runnable case
+# --- B1 H8 S2048 D64 fp32, chunks 512 / 512: the case the reference itself can run on a CPU
 def test_config1_fp32_fwd_bwd():
     B, S, H, D = 1, 2048, 8, 64
     q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=0)
