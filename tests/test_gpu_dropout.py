@@ -71,6 +71,13 @@ def test_dropout_mask_rejects():
     assert lib.ra_dropout_keep(0, 0.0, 1, 1, 8, 8, keep.data_ptr(), None) == L.RA_ERR_INVALID
     assert lib.ra_dropout_keep(0, 1.0, 1, 1, 8, 8, keep.data_ptr(), None) == L.RA_ERR_INVALID
     assert lib.ra_dropout_keep(0, 0.5, 1, 1, 8, 8, None, None) == L.RA_ERR_INVALID
+    w = torch.empty(4096, dtype=torch.int64, device=DEV)
+    args = (w.data_ptr(), w.data_ptr(), keep.data_ptr())
+    assert lib.ra_dropout_keep_packed(0, 0.5, 1, 1, 96, 64, *args, 0, 0, 0, 0, 0, None) == L.RA_ERR_UNSUPPORTED  # Q % 64
+    assert lib.ra_dropout_keep_packed(0, 0.5, 1, 1, 64, 64, None, None, None, 0, 0, 0, 0, 0, None) == L.RA_ERR_INVALID
+    assert lib.ra_dropout_keep_packed(0, 1.5, 1, 1, 64, 64, *args, 0, 0, 0, 0, 0, None) == L.RA_ERR_INVALID
+    # chunk sizes that do not divide the mask, under a causal block size
+    assert lib.ra_dropout_keep_packed(0, 0.5, 1, 1, 128, 128, *args, 1, 48, 64, 0, 0, None) == L.RA_ERR_INVALID
 
 
 def _run(q, k, v, do, bias, seg, n, kw):
