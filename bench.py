@@ -23,6 +23,10 @@ PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters'
 # reading for the 1 GiB copy of --workload copy) at the default sizes of each workload
+# rocprofv3's MfmaUtil (MFMA busy cycles / elapsed cycles, in per cent) of the same launches, from
+# profiles/mfma_utilisation_pmc.txt; the clock under these loads is 1.75-1.95 GHz, not the 2.4 GHz of the nominal peak
+MEASURED_MFMA_UTIL = {"attn_fwd_ws_kernel": 45.5, "attn_bwd_dkv_ws_kernel": 56.3, "attn_bwd_dq_ws_kernel": 59.9,
+                      "attn32k_step": 54.5, "gemm_bf16_w4_kernel<false, false>": 65.0}
 MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.37e9, "attn_bwd_dkv_ws_kernel": 4.25e9, "attn_bwd_dq_ws_kernel": 3.47e9,
                     "decode_split_kernel": 68.88e9, "gemm_bf16_w4_kernel<false, false>": 2.55e9,
                     "rmsnorm_fwd_kernel": 2.15e9}
@@ -166,6 +170,8 @@ def bench_attention(args, ring, dropout=False):
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
                 "traffic": MEASURED_TRAFFIC.get(dom) if S == 32768 else None,
+                "mfma_util_pmc": ({"kernel": MEASURED_MFMA_UTIL.get(dom), "step": MEASURED_MFMA_UTIL["attn32k_step"]}
+                                  if S == 32768 and not dropout else None),
                 "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
                 "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
         if dropout:
@@ -318,6 +324,7 @@ def bench_ffn(args):
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC["gemm_bf16_w4_kernel<false, false>"] if (T, chunk) == (65536, 2048) else None,
+                     "mfma_util_pmc": {"kernel": MEASURED_MFMA_UTIL["gemm_bf16_w4_kernel<false, false>"]},
                      "kernel_ms": {"gemm_bf16_w4_kernel<false, false>": round(gemm_ms, 3)}},
         "cpu_baseline": cpu,
     }
