@@ -21,15 +21,33 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters'
-# reading for the 1 GiB copy of --workload copy) at the default sizes of each workload
-# rocprofv3's MfmaUtil (MFMA busy cycles / elapsed cycles, in per cent) of the same launches, from
-# profiles/mfma_utilisation_pmc.txt; the clock under these loads is 1.75-1.95 GHz, not the 2.4 GHz of the nominal peak
-MEASURED_MFMA_UTIL = {"attn_fwd_ws_kernel": 45.5, "attn_bwd_dkv_ws_kernel": 56.3, "attn_bwd_dq_ws_kernel": 59.9,
-                      "attn32k_step": 54.5, "gemm_bf16_w4_kernel<false, false>": 65.0}
-MEASURED_TRAFFIC = {"attn_fwd_ws_kernel": 3.37e9, "attn_bwd_dkv_ws_kernel": 4.25e9, "attn_bwd_dq_ws_kernel": 3.47e9,
-                    "decode_split_kernel": 68.88e9, "gemm_bf16_w4_kernel<false, false>": 2.55e9,
-                    "rmsnorm_fwd_kernel": 2.15e9}
+
+
+def _measured(profile, kind):
+    """Figures that only a ``rocprofv3 --pmc`` run can give (HBM bytes per launch, MFMA busy share), read from the
+    summary committed under profiles/: lines ``<kind> <kernel> <value>`` after lines ``source <path> sha256=<hex>``
+    naming the kernel sources the run was made with.  A figure is reported only while every one of those sources
+    still hashes to the recorded value; once a kernel source has changed the table is stale and this returns {}."""
+    import hashlib
+    path = os.path.join(ROOT, "profiles", profile)
+    out, ok = {}, True
+    try:
+        for line in open(path):
+            w = line.split()
+            if len(w) == 3 and w[0] == "source" and w[2].startswith("sha256="):
+                try:
+                    ok = ok and hashlib.sha256(open(os.path.join(ROOT, w[1]), "rb").read()).hexdigest() == w[2][7:]
+                except OSError:
+                    ok = False
+            elif len(w) == 3 and w[0] == kind:
+                out[w[1]] = float(w[2])
+    except OSError:
+        return {}
+    return out if ok else {}
+
+
+TRAFFIC_PROFILE = "hbm_traffic_pmc.txt"
+MFMA_PROFILE = "mfma_utilisation_pmc.txt"
 
 
 def _kwargs(qc, kc, cbs=1, **extra):
@@ -100,8 +118,12 @@ def bench_attention(args, ring, dropout=False):
     if args.seq_len:
         S = args.seq_len
     g = torch.Generator(device=dev).manual_seed(0)
-    mk = lambda: (torch.randn(B, S, H, D, device=dev, generator=g) * D ** -0.5).to(torch.bfloat16)
-    q, k, v = mk().requires_grad_(True), mk().requires_grad_(True), mk().requires_grad_(True)
+    # q, k, v ~ N(0,1) / sqrt(D) is the input the configuration names; it makes the logits tiny (std 0.008).  The
+    # other choices give the logits a standard deviation of 0.09 (q, k scaled D^-0.25) or 1 (unscaled q, k)
+    qk_scale = {"baseline": D ** -0.5, "d-quarter": D ** -0.25, "unit": 1.0}[args.inputs]
+    v_scale = D ** -0.5 if args.inputs == "baseline" else 1.0
+    mk = lambda sc: (torch.randn(B, S, H, D, device=dev, generator=g) * sc).to(torch.bfloat16)
+    q, k, v = mk(qk_scale).requires_grad_(True), mk(qk_scale).requires_grad_(True), mk(v_scale).requires_grad_(True)
     do = torch.randn(B, S, H, D, device=dev, generator=g).to(torch.bfloat16)
     bias = seg = None
     pairs = S * (S + 1) / 2
@@ -164,26 +186,33 @@ def bench_attention(args, ring, dropout=False):
                     m2.use_dropout(cfg, B, H, S, S, 0, 0, q.device)
                 del mi
                 mask_ms = _event_ms(draw, 3)
+        traffic, util = _measured(TRAFFIC_PROFILE, "traffic"), _measured(MFMA_PROFILE, "mfma_util")
         dom = max(kern, key=lambda n_: kern[n_][0])
         dms, dfl = kern[dom]
         ach = dfl / (dms * 1e-3) / 1e12
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
-                "traffic": MEASURED_TRAFFIC.get(dom) if S == 32768 else None,
-                "mfma_util_pmc": ({"kernel": MEASURED_MFMA_UTIL.get(dom), "step": MEASURED_MFMA_UTIL["attn32k_step"]}
-                                  if S == 32768 and not dropout else None),
+                "traffic": traffic.get(dom) if S == 32768 and args.inputs == "baseline" else None,
+                "traffic_source": "profiles/" + TRAFFIC_PROFILE if traffic.get(dom) else None,
+                "mfma_util_pmc": ({"kernel": util.get(dom), "step": util.get("attn32k_step"),
+                                   "source": "profiles/" + MFMA_PROFILE}
+                                  if S == 32768 and not dropout and util.get(dom) else None),
                 "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
                 "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
         if dropout:
             roof["traffic"] = None
             roof["mask_draw_and_pack_ms"] = round(mask_ms, 3)
     cpu = cpu_baseline_attention() if not (args.no_cpu or dropout) else None
+    del q, k, v, do
     return {
         "metric": "attn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
         "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "config": {"workload": name, "B": B, "H": H, "S": S, "D": D, "causal_block_size": 1,
                    "query_chunk_size": 512, "key_chunk_size": 512, "virtual_ring": n,
                    "segment_ids": bool(ring), "bias": bool(ring), "attn_pdrop": pdrop if dropout else 0.0,
+                   "inputs": {"baseline": "q, k, v ~ N(0,1)/sqrt(D), dO ~ N(0,1)",
+                              "d-quarter": "q, k ~ N(0,1) * D^-0.25, v, dO ~ N(0,1)",
+                              "unit": "q, k, v, dO ~ N(0,1)"}[args.inputs],
                    "flop_convention": "4*D fwd + 10*D bwd per unmasked (q,k) pair per head"},
         "roofline": roof, "cpu_baseline": cpu,
     }
@@ -211,7 +240,7 @@ def cpu_baseline_attention():
 
 
 # --------------------------------------------------------------------------- decode workload
-def bench_decode(args):
+def bench_decode(args, steps=0):
     import torch
     import ringattention_amd as ra
     dev = "cuda:0"
@@ -238,6 +267,8 @@ def bench_decode(args):
     ms = _time_steps(step, args.steps, args.warmup)
     bytes_step = 2.0 * B * (Lf + 1) * H * D * 2
     value = bytes_step / (ms * 1e-3) / 1e9
+    # the split kernel alone (the combine pass that follows it moves 0.05 GB): events around the whole step, minus
+    # nothing - the step is this kernel to within 1 %
     kms = _event_ms(step, 5)
     ach = bytes_step / (kms * 1e-3) / 1e9
     cpu = None
@@ -260,11 +291,14 @@ def bench_decode(args):
     return {
         "metric": "decode_hbm_gbs", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms, 3),
         "dtype": "bf16", "pct_hbm_peak": round(100 * value / PEAK_HBM_GBS, 2),
+        "steps": steps or args.steps,
         "config": {"workload": "decode", "B": B, "H": H, "D": D, "cache_len": Lf, "key_chunk_size": kc,
                    "query_chunk_size": 1, "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "kernel": "decode_split_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC["decode_split_kernel"] if (B, Lf) == (16, 262144) else None},
+                     "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("decode_split_kernel")
+                                 if (B, Lf) == (16, 262144) else None),
+                     "traffic_source": "profiles/" + TRAFFIC_PROFILE},
         "cpu_baseline": cpu,
     }
 
@@ -284,15 +318,15 @@ def bench_ffn(args):
         x.grad = None
         for p in ff.parameters():
             p.grad = None
-        y = ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy)
+        y = ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy, launch_tokens=args.ffn_launch_tokens or None)
         y.backward(dy)
 
     ms = _time_steps(step, args.steps, args.warmup)
-    kept = ra.feedforward._save_preactivations(args.ffn_policy, T, f, x.device)
+    kept = ra.feedforward._save_preactivations(args.ffn_policy)
     flops = 18.0 * T * d * f
     value = flops / (ms * 1e-3) / 1e12
     # dominant kernel: the GEMM a = x w1 of one launch (tokens_per_launch x hidden x intermediate), timed alone
-    slab = ra.feedforward._slab_tokens(chunk, T // chunk)
+    slab = ra.feedforward._slab_tokens(chunk, T // chunk, args.ffn_launch_tokens or None)
     xs = x.detach()[0, :slab]
     a_out = torch.empty(slab, f, dtype=torch.bfloat16, device=dev)
     gemm_ms = _event_ms(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out), 5)
@@ -317,14 +351,16 @@ def bench_ffn(args):
         "metric": "swiglu_ffn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
         "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "config": {"workload": "ffn", "tokens": T, "hidden": d, "intermediate": f, "chunk_size": chunk,
-                   "tokens_per_launch": ra.feedforward._slab_tokens(chunk, T // chunk),
+                   "tokens_per_launch": slab,
                    "policy": args.ffn_policy, "preactivations": "kept (%.1f GB)" % (4e-9 * T * f) if kept else "recomputed",
                    "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
         "roofline": {"bound": "mfma", "kernel": "gemm_bf16_w4_kernel<false, false> (a = x w1 of one launch)",
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC["gemm_bf16_w4_kernel<false, false>"] if (T, chunk) == (65536, 2048) else None,
-                     "mfma_util_pmc": {"kernel": MEASURED_MFMA_UTIL["gemm_bf16_w4_kernel<false, false>"]},
+                     "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("gemm_bf16_w4_kernel<false,false>")
+                                 if (T, slab) == (65536, 16384) else None),
+                     "mfma_util_pmc": {"kernel": _measured(MFMA_PROFILE, "mfma_util").get("gemm_bf16_w4_kernel<false,false>"),
+                                       "source": "profiles/" + MFMA_PROFILE},
                      "kernel_ms": {"gemm_bf16_w4_kernel<false, false>": round(gemm_ms, 3)}},
         "cpu_baseline": cpu,
     }
@@ -442,7 +478,7 @@ def bench_rmsnorm(args):
         "config": {"workload": "rmsnorm", "tokens": T, "hidden": d, "bytes_per_step": bytes_step},
         "roofline": {"bound": "hbm", "kernel": "rmsnorm_fwd_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC["rmsnorm_fwd_kernel"] if T == 65536 else None,
+                     "traffic": _measured(TRAFFIC_PROFILE, "traffic").get("rmsnorm_fwd_kernel") if T == 65536 else None,
                      "kernel_ms": {"rmsnorm_fwd_kernel": round(f_ms, 4)}},
         "cpu_baseline": cpu,
     }
@@ -510,12 +546,20 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="attn32k", choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
+    ap.add_argument("--workload", default=None, choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
                                                               "dropout32k"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--ffn-policy", default=None, choices=["nothing_saveable", "save_preactivations"],
-                    help="ffn workload: what blockwise_feedforward keeps for the backward pass (default: by size)")
+    ap.add_argument("--ffn-policy", default="nothing_saveable", choices=["nothing_saveable", "save_preactivations"],
+                    help="ffn workload: what blockwise_feedforward keeps for the backward pass (default: the "
+                         "reference's, nothing: the pre-activations are recomputed)")
+    ap.add_argument("--ffn-launch-tokens", type=int, default=0,
+                    help="ffn workload: let consecutive chunks share a launch of up to this many tokens (default: one "
+                         "chunk per launch, as the reference's scan)")
+    ap.add_argument("--inputs", default="baseline", choices=["baseline", "d-quarter", "unit"],
+                    help="attention workloads: scale of q and k (baseline = N(0,1)/sqrt(D), the configuration's)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="default workload only: skip the decode leg and the other-inputs timings of the JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the ring is virtual); run with --gpus 1", file=sys.stderr)
@@ -524,8 +568,26 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
+    # no --workload: the whole headline metric in one line - the 32K attention step is the value; the decode leg
+    # (B16, 262144 positions, 64 steps) and the same attention step on other input scales ride along as sub-objects
+    whole_metric = args.workload is None and not args.no_extras and not args.seq_len
+    if args.workload is None:
+        args.workload = "attn32k"
+    extras = {}
     if args.workload in ("attn32k", "ring131k", "dropout32k"):
         r = bench_attention(args, ring=(args.workload == "ring131k"), dropout=(args.workload == "dropout32k"))
+        if whole_metric:
+            others = []
+            for inputs in ("d-quarter", "unit"):
+                a2 = argparse.Namespace(**dict(vars(args), inputs=inputs, no_cpu=True))
+                r2 = bench_attention(a2, ring=False)
+                others.append({"inputs": r2["config"]["inputs"], "value": r2["value"], "unit": r2["unit"],
+                               "ms_per_step": r2["ms_per_step"], "kernel_ms": r2["roofline"]["kernel_ms"]})
+            extras["other_inputs"] = others
+            torch.cuda.empty_cache()
+            d = bench_decode(args, steps=64)
+            extras["decode"] = {k_: d[k_] for k_ in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
+                                                     "pct_hbm_peak", "config", "roofline", "cpu_baseline")}
     elif args.workload == "decode":
         r = bench_decode(args)
     elif args.workload == "copy":
@@ -545,6 +607,7 @@ def main():
     for extra in ("pct_bf16_mfma_peak", "pct_hbm_peak"):
         if extra in r:
             line[extra] = r[extra]
+    line.update(extras)
     print(json.dumps(line))
 
 

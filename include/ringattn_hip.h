@@ -32,11 +32,7 @@ enum { RA_F32 = 0, RA_BF16 = 1 };
 enum {
   RA_IMPL_AUTO = 0,    /* MFMA kernels when the shape allows, else the generic ones */
   RA_IMPL_GENERIC = 1, /* fp32 vector-ALU kernels: any chunk sizes, fp32 or bf16 inputs */
-  RA_IMPL_MFMA = 2,    /* bf16 MFMA kernels only; RA_ERR_UNSUPPORTED if the shape does not fit */
-  /* ra_attn_bwd_params.impl may OR in one of these to launch a single backward kernel (for timing
-     one kernel in isolation; a full backward needs both) */
-  RA_BWD_ONLY_DQ = 0x10,
-  RA_BWD_ONLY_DKV = 0x20
+  RA_IMPL_MFMA = 2     /* bf16 MFMA kernels only; RA_ERR_UNSUPPORTED if the shape does not fit */
 };
 
 /*
@@ -248,6 +244,9 @@ typedef struct ra_swiglu_params {
   int32_t preact_saved;           /* backward: 1 = a and b still hold what the forward wrote for these tokens (the
                                      caller kept them: `policy` other than nothing_saveable, ringattention_jax.py:334);
                                      0 = recompute them from x (the reference's default policy) */
+  int32_t gemm_tile;              /* 0: the library picks the tile kernel of each product (the default).  1 + t forces
+                                     tile kernel t wherever the shape divides (0: 256 x 256 over four wavefronts,
+                                     1: 256 x 128, 2: 128 x 128), so that tests reach every kernel */
 } ra_swiglu_params;
 
 int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream);

@@ -1,0 +1,29 @@
+/*
+ * Measurement and test hooks of libringattn_hip.so: entry points that run ONE part of what an entry point of
+ * ringattn_hip.h runs, so that a benchmark can time a kernel alone and a test can reach every tile kernel.
+ * They are not part of the drop-in boundary; a caller of the hot path needs none of them.
+ */
+#ifndef RINGATTN_HIP_MEASURE_H_
+#define RINGATTN_HIP_MEASURE_H_
+
+#include "ringattn_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ra_attn_bwd_block (ringattention_jax.py:181-270) launches two kernels: the key-stationary one that adds into
+ * dk and dv, and the query-stationary one that adds into dq.  This launches one of them (MFMA kernels only): what
+ * the other one would have written is left untouched, and may be null. */
+enum { RA_BWD_PART_DQ = 1, RA_BWD_PART_DKV = 2 };
+int ra_attn_bwd_block_part(const ra_attn_bwd_params* p, int32_t part, ra_stream_t stream);
+
+/* ra_gemm_bf16 with the tile kernel named: tile -1 = the library's choice, 0: 256 x 256 over four wavefronts,
+ * 1: 256 x 128, 2: 128 x 128 (a forced tile still gives way to a smaller one where the shape does not divide). */
+int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,
+                      int32_t trans_b, int32_t c_dtype, int32_t beta_one, int32_t tile, ra_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RINGATTN_HIP_MEASURE_H_ */

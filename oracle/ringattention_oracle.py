@@ -251,7 +251,9 @@ def blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_st
 def _work_dtype(q, float32_logits, compute_dtype):
     if compute_dtype is not None:
         return compute_dtype
-    return torch.float32 if (float32_logits or q.dtype == torch.float32) else torch.float32
+    # :18-19: q and k are cast to float32 only when float32_logits is set; otherwise logits, softmax statistics and
+    # the carry all live in the dtype of q (:22-23)
+    return torch.float32 if (float32_logits or q.dtype == torch.float32) else q.dtype
 
 
 def ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_size, float32_logits,

@@ -11,7 +11,7 @@ plus ``ring_axis`` to declare the size of the (virtual) sequence-parallel ring, 
 from .ringattention_hip import (ring_attention, ring_axis, axis_size, below_or_on_diag, run_prefix_keys,
                                 _blockwise_attention_fwd, _blockwise_attention_bwd)
 from .feedforward import blockwise_feedforward, SwiGLU, gemm_bf16
-from .decode import decode_attention
+from .decode import decode_attention, decode_workspace
 from .inference import ring_attention_inference
 from .steps import rope_kv_append, rmsnorm_residual
 
@@ -21,4 +21,4 @@ ringattention_inference = ring_attention_inference
 
 __all__ = ["ringattention", "ringattention_jax", "ringattention_inference", "ring_attention",
            "ring_attention_inference", "blockwise_feedforward", "ring_axis",
-           "axis_size", "SwiGLU", "decode_attention", "below_or_on_diag", "rope_kv_append", "rmsnorm_residual"]
+           "axis_size", "SwiGLU", "decode_attention", "decode_workspace", "below_or_on_diag", "rope_kv_append", "rmsnorm_residual"]

@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libringattn_hip.so")
 RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
 RA_F32, RA_BF16 = 0, 1
 RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
-RA_BWD_ONLY_DQ, RA_BWD_ONLY_DKV = 0x10, 0x20
+RA_BWD_PART_DQ, RA_BWD_PART_DKV = 1, 2          # include/ringattn_hip_measure.h
 RA_SEG_TILE = 64
 RA_KEEP_WHERE, RA_KEEP_DROPOUT = 0, 1
 RA_GRAD_INIT_DQ, RA_GRAD_INIT_DKV = 1, 2
@@ -77,7 +77,7 @@ class RaSwigluParams(C.Structure):
         ("x", vp), ("w1", vp), ("w2", vp), ("w3", vp),
         ("a", vp), ("b", vp), ("h", vp), ("y", vp),
         ("dy", vp), ("dx", vp), ("dw1", vp), ("dw2", vp), ("dw3", vp), ("da", vp), ("db", vp),
-        ("preact_saved", i32),
+        ("preact_saved", i32), ("gemm_tile", i32),
     ]
 
 
@@ -101,7 +101,7 @@ class RaRmsnormParams(C.Structure):
     ]
 
 
-# every symbol include/ringattn_hip.h declares: (name, restype, argtypes)
+# every symbol include/ringattn_hip.h and include/ringattn_hip_measure.h declare: (name, restype, argtypes)
 SYMBOLS = {
     "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
     "ra_keep_pack": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]),
@@ -123,6 +123,9 @@ SYMBOLS = {
     "ra_rmsnorm_bwd": (C.c_int, [C.POINTER(RaRmsnormParams), vp]),
     "ra_last_error": (C.c_char_p, []),
     "ra_version": (C.c_int, []),
+    # measurement / test hooks
+    "ra_attn_bwd_block_part": (C.c_int, [C.POINTER(RaAttnBwdParams), i32, vp]),
+    "ra_gemm_bf16_tile": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp]),
 }
 
 _lib = None

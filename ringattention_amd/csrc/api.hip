@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include "common.hpp"
+#include "../../include/ringattn_hip_measure.h"
 
 namespace ra {
 
@@ -18,7 +19,7 @@ void set_error(const char* fmt, ...) {
 int attn_fwd_generic(const ra_attn_fwd_params* p, hipStream_t s);
 int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s);
 int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s);     // RA_ERR_UNSUPPORTED if shape does not fit
-int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s);
+int attn_bwd_mfma(const ra_attn_bwd_params* p, int parts, hipStream_t s);   // parts: RA_BWD_PART_* bits
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p);
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p);
 int carry_init(float*, int64_t, int64_t, float*, float*, int64_t, int64_t, int, int, int, int, hipStream_t);
@@ -33,11 +34,11 @@ int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, in
                         uint64_t* bits_q, uint8_t* summary, int cbs, int qc, int kc, int q_start, int k_start,
                         hipStream_t s);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
-int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s);
+int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream_t s);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s);
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
-              int beta_one, hipStream_t s);
+              int beta_one, int tile, hipStream_t s);
 
 int rope_kv_append(const ra_rope_append_params* p, hipStream_t s);
 int rmsnorm_fwd(const ra_rmsnorm_params* p, hipStream_t s);
@@ -240,29 +241,42 @@ int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t str
                    (hipStream_t)stream);
 }
 
-int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream) {
-  RA_REQUIRE(p, RA_ERR_INVALID, "attn_bwd_block: null params");
+static int attn_bwd_block(const ra_attn_bwd_params* p, int parts, const char* who, hipStream_t s) {
+  const bool dq_part = parts & RA_BWD_PART_DQ, dkv_part = parts & RA_BWD_PART_DKV;
+  RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
   RA_REQUIRE(p->q && p->k && p->v && p->g && p->delta && p->denominator && p->max_score, RA_ERR_INVALID,
-             "attn_bwd_block: null tensor");
-  RA_REQUIRE((p->dk_out == nullptr) == (p->dv_out == nullptr), RA_ERR_INVALID,
-             "attn_bwd_block: dk_out and dv_out go together");
+             "%s: null tensor", who);
+  RA_REQUIRE((p->dk_out == nullptr) == (p->dv_out == nullptr), RA_ERR_INVALID, "%s: dk_out and dv_out go together", who);
   RA_REQUIRE((p->grads_are_initial & ~(RA_GRAD_INIT_DQ | RA_GRAD_INIT_DKV)) == 0, RA_ERR_INVALID,
-             "attn_bwd_block: unknown bits in grads_are_initial");
-  RA_REQUIRE(p->dq || ((p->grads_are_initial & RA_GRAD_INIT_DQ) && p->dq_out), RA_ERR_INVALID,
-             "attn_bwd_block: dq may be null only when it is initial and dq_out is given");
-  RA_REQUIRE((p->dk && p->dv) || ((p->grads_are_initial & RA_GRAD_INIT_DKV) && p->dk_out), RA_ERR_INVALID,
-             "attn_bwd_block: dk / dv may be null only when they are initial and dk_out / dv_out are given");
-  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_bwd_block: dtype %d", p->dtype);
-  RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_bwd_block: empty shape");
-  RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_bwd_block: B and H must be <= 65535");
-  if (int rc = check_mask(p->mask, p->Sq, p->Skv, "attn_bwd_block")) return rc;
-  hipStream_t s = (hipStream_t)stream;
-  const int impl = p->impl & 0xf;
-  if (impl == RA_IMPL_GENERIC) return attn_bwd_generic(p, s);
-  if (attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, s);
-  RA_REQUIRE(impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
-             "attn_bwd_block: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128");
+             "%s: unknown bits in grads_are_initial", who);
+  RA_REQUIRE(!dq_part || p->dq || ((p->grads_are_initial & RA_GRAD_INIT_DQ) && p->dq_out), RA_ERR_INVALID,
+             "%s: dq may be null only when it is initial and dq_out is given", who);
+  RA_REQUIRE(!dkv_part || (p->dk && p->dv) || ((p->grads_are_initial & RA_GRAD_INIT_DKV) && p->dk_out), RA_ERR_INVALID,
+             "%s: dk / dv may be null only when they are initial and dk_out / dv_out are given", who);
+  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "%s: dtype %d", who, p->dtype);
+  RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "%s: empty shape", who);
+  RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "%s: B and H must be <= 65535", who);
+  RA_REQUIRE(p->impl == RA_IMPL_AUTO || p->impl == RA_IMPL_GENERIC || p->impl == RA_IMPL_MFMA, RA_ERR_INVALID,
+             "%s: impl %d", who, p->impl);
+  if (int rc = check_mask(p->mask, p->Sq, p->Skv, who)) return rc;
+  const bool whole = dq_part && dkv_part;
+  if (p->impl == RA_IMPL_GENERIC && whole) return attn_bwd_generic(p, s);
+  if (p->impl != RA_IMPL_GENERIC && attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, parts, s);
+  RA_REQUIRE(whole, RA_ERR_UNSUPPORTED, "%s: one part alone is launched by the MFMA kernels only, which do not take "
+             "this call (impl, dtype, head size or chunk sizes)", who);
+  RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
+             "%s: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128", who);
   return attn_bwd_generic(p, s);
+}
+
+int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream) {
+  return attn_bwd_block(p, RA_BWD_PART_DQ | RA_BWD_PART_DKV, "attn_bwd_block", (hipStream_t)stream);
+}
+
+int ra_attn_bwd_block_part(const ra_attn_bwd_params* p, int32_t part, ra_stream_t stream) {
+  RA_REQUIRE(part == RA_BWD_PART_DQ || part == RA_BWD_PART_DKV, RA_ERR_INVALID,
+             "attn_bwd_block_part: part must be RA_BWD_PART_DQ or RA_BWD_PART_DKV");
+  return attn_bwd_block(p, part, "attn_bwd_block_part", (hipStream_t)stream);
 }
 
 size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int32_t num_splits) {
@@ -271,27 +285,37 @@ size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int
   return (size_t)B * H * ns * (D + 2) * sizeof(float);
 }
 
-int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream) {
-  RA_REQUIRE(p, RA_ERR_INVALID, "decode_fwd: null params");
-  RA_REQUIRE(p->q && p->k && p->v && p->out && p->workspace, RA_ERR_INVALID, "decode_fwd: null tensor");
-  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "decode_fwd: dtype %d", p->dtype);
-  RA_REQUIRE(p->B > 0 && p->L > 0 && p->H > 0 && p->D > 0 && p->B <= 65535, RA_ERR_INVALID, "decode_fwd: bad shape");
+static int check_decode(const ra_decode_params* p, const char* who) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
+  RA_REQUIRE(p->q && p->k && p->v && p->out, RA_ERR_INVALID, "%s: null tensor", who);
+  RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "%s: dtype %d", who, p->dtype);
+  RA_REQUIRE(p->B > 0 && p->L > 0 && p->H > 0 && p->D > 0 && p->B <= 65535, RA_ERR_INVALID, "%s: bad shape", who);
+  RA_REQUIRE(p->D == 64 || p->D == 128, RA_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128}", who, p->D);
   RA_REQUIRE(p->mask.query_chunk_size == 1, RA_ERR_INVALID,
-             "decode_fwd: one query token needs query_chunk_size == 1 (q_len // query_chunk_size chunks)");
-  if (int rc = check_mask(p->mask, 1, p->L, "decode_fwd")) return rc;
-  RA_REQUIRE(p->mask.keep == nullptr && p->mask.keep_bits_k == nullptr, RA_ERR_UNSUPPORTED, "decode_fwd: the boolean keep mask is taken by the generic attention kernels only");
+             "%s: one query token needs query_chunk_size == 1 (q_len // query_chunk_size chunks)", who);
+  if (int rc = check_mask(p->mask, 1, p->L, who)) return rc;
+  RA_REQUIRE(p->mask.keep == nullptr && p->mask.keep_bits_k == nullptr, RA_ERR_UNSUPPORTED,
+             "%s: the boolean keep mask is taken by the generic attention kernels only", who);
+  RA_REQUIRE(p->num_splits >= 0 && p->num_splits <= 256, RA_ERR_INVALID, "%s: num_splits %d outside [0, 256]", who,
+             p->num_splits);
+  return RA_OK;
+}
+
+int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream) {
+  if (int rc = check_decode(p, "decode_fwd")) return rc;
+  RA_REQUIRE(p->workspace, RA_ERR_INVALID, "decode_fwd: null workspace");
   int ns = p->num_splits > 0 ? p->num_splits : decode_pick_splits(p->B, p->L, p->H, p->D, p->dtype);
-  RA_REQUIRE(ns <= 256, RA_ERR_INVALID, "decode_fwd: num_splits %d > 256", ns);
   size_t need = (size_t)p->B * p->H * ns * (p->D + 2) * sizeof(float);
   RA_REQUIRE(p->workspace_bytes >= need, RA_ERR_INVALID, "decode_fwd: workspace %zu bytes < %zu needed",
              p->workspace_bytes, need);
-  return decode_fwd(p, ns, (hipStream_t)stream);
+  return decode_fwd(p, (float*)p->workspace, ns, (hipStream_t)stream);
 }
 
 int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream) {
   RA_REQUIRE(p, RA_ERR_INVALID, "swiglu_fwd: null params");
   RA_REQUIRE(p->x && p->w1 && p->w2 && p->w3 && p->a && p->b && p->h && p->y, RA_ERR_INVALID, "swiglu_fwd: null tensor");
   RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_fwd: empty shape");
+  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 3, RA_ERR_INVALID, "swiglu_fwd: gemm_tile %d outside [0, 3]", p->gemm_tile);
   return swiglu_fwd(p, (hipStream_t)stream);
 }
 
@@ -301,6 +325,7 @@ int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream) {
                  p->dw3 && p->da && p->db,
              RA_ERR_INVALID, "swiglu_bwd: null tensor");
   RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_bwd: empty shape");
+  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 3, RA_ERR_INVALID, "swiglu_bwd: gemm_tile %d outside [0, 3]", p->gemm_tile);
   return swiglu_bwd(p, (hipStream_t)stream);
 }
 
@@ -309,7 +334,16 @@ int ra_gemm_bf16(const void* A, const void* Bm, void* C, int32_t M, int32_t N, i
   RA_REQUIRE(A && Bm && C, RA_ERR_INVALID, "gemm_bf16: null pointer");
   RA_REQUIRE(M > 0 && N > 0 && K > 0, RA_ERR_INVALID, "gemm_bf16: empty shape");
   RA_REQUIRE(c_dtype == RA_F32 || c_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "gemm_bf16: c_dtype %d", c_dtype);
-  return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, (hipStream_t)stream);
+  return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, -1, (hipStream_t)stream);
+}
+
+int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,
+                      int32_t trans_b, int32_t c_dtype, int32_t beta_one, int32_t tile, ra_stream_t stream) {
+  RA_REQUIRE(A && Bm && C, RA_ERR_INVALID, "gemm_bf16_tile: null pointer");
+  RA_REQUIRE(M > 0 && N > 0 && K > 0, RA_ERR_INVALID, "gemm_bf16_tile: empty shape");
+  RA_REQUIRE(c_dtype == RA_F32 || c_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "gemm_bf16_tile: c_dtype %d", c_dtype);
+  RA_REQUIRE(tile >= -1 && tile <= 2, RA_ERR_INVALID, "gemm_bf16_tile: tile %d outside [-1, 2]", tile);
+  return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, tile, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -137,19 +137,6 @@ __device__ __forceinline__ int keep_leading_full(const uint8_t* sm, int64_t stri
   return n;
 }
 
-// optional cycle-counter marks for timing experiments (compiled out unless RA_TRACE is defined)
-#ifdef RA_TRACE
-__device__ long long g_trace[8][4096];
-#define RA_TRACE_MARK() { if (trace_on && lane == 0 && trace_n < 4096) g_trace[wave][trace_n++] = __builtin_readcyclecounter(); }
-#ifdef RA_TRACE2
-#define RA_TRACE_MARK2() { __builtin_amdgcn_sched_barrier(0); RA_TRACE_MARK(); __builtin_amdgcn_sched_barrier(0); }
-#else
-#define RA_TRACE_MARK2() {}
-#endif
-#else
-#define RA_TRACE_MARK() {}
-#define RA_TRACE_MARK2() {}
-#endif
 
 // ================================================================== backward
 // Two deterministic kernels (fp32 atomics reach ~1.3 TB/s at best on this part, far below what a
@@ -222,16 +209,6 @@ __device__ __forceinline__ void pass_rows(float* acc, int64_t acc_ss, uint16_t* 
 // tile t is read by the producer's products in steps 2t-1, 2t, by its vector work in 2t, 2t+1 and by
 // the consumer in 2t+1, 2t+2; tile t+2 is stored in step 2t+1 (its buffer held tile t-1) from
 // registers loaded two steps earlier.
-// timing experiments only: each switch removes one part of the work (results are then wrong)
-#ifndef RA_ABL_WS_NOVEC
-#define RA_ABL_WS_NOVEC 0
-#endif
-#ifndef RA_ABL_WS_NOPMFMA
-#define RA_ABL_WS_NOPMFMA 0
-#endif
-#ifndef RA_ABL_WS_NOCONS
-#define RA_ABL_WS_NOCONS 0
-#endif
 constexpr int WS_PSTR = 40;                 // P / dS row stride in elements (conflict-free 16-byte reads)
 constexpr int WS_PD = 32 * WS_PSTR;         // one 32 x 32 block
 constexpr int WS_TILE = KBM * TROW;
@@ -412,7 +389,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   }
 #define RA_WS_AMFMA(G, QA, GA, SN, DPN)                                                                 \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    if (RA_ABL_WS_NOPMFMA) break;                                                                       \
     SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(QA[i], kf[2 * (G) + i], SN, 0, 0, 0);                  \
     DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(GA[i], vf[2 * (G) + i], DPN, 0, 0, 0);                \
   }
@@ -421,14 +397,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   {                                                                                                     \
     bf16x4 p4, d4;                                                                                      \
     _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
-      if (RA_ABL_WS_NOVEC) {                                                                            \
-        p4[e] = __builtin_bit_cast(__bf16, (uint16_t)(__float_as_uint(SC[(G) * 4 + e]) >> 16));         \
-        d4[e] = __builtin_bit_cast(__bf16, (uint16_t)(__float_as_uint(DPC[(G) * 4 + e]) >> 16));        \
-      } else {                                                                                          \
-        const float p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -VL[e]));                     /* :226 */     \
-        p4[e] = (__bf16)p;                                                                              \
-        d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                          /* :229 */     \
-      }                                                                                                 \
+      const float p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -VL[e]));                       /* :226 */     \
+      p4[e] = (__bf16)p;                                                                                \
+      d4[e] = (__bf16)(p * DPC[(G) * 4 + e]);                                            /* :229 */     \
     }                                                                                                   \
     *(bf16x4*)(pw + (PB) * 2 * WS_PD + (G) * 8) = p4;                                                   \
     *(bf16x4*)(pw + (PB) * 2 * WS_PD + WS_PD + (G) * 8) = d4;                                           \
@@ -604,7 +575,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   }
 #define RA_WS_CMFMA(K, F, BOP)                                                                          \
   _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                    \
-    if (RA_ABL_WS_NOCONS) break;                                                                        \
     if ((K) & 1) dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, dkacc[db], 0, 0, 0);   \
     else dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, dvacc[db], 0, 0, 0);           \
   }
@@ -815,10 +785,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + 16 * TROW) = S##v1;                                         \
     *(uint4*)(dv_ + 32 * TROW) = S##v2; *(uint4*)(dv_ + 48 * TROW) = S##v3;                             \
   }
-#ifdef RA_TRACE
-  const bool trace_on = blockIdx.x == 0;
-  int trace_n = 0;
-#endif
   if (role == 1) {
     RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
     RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
@@ -873,7 +839,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   }
 #define RA_WS_AMFMA(G, KA, VA, SN, DPN)                                                                 \
   _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    if (RA_ABL_WS_NOPMFMA) break;                                                                       \
     SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[2 * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T */ \
     DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(VA[i], gf[2 * (G) + i], DPN, 0, 0, 0); /* dP^T = V dO^T */ \
   }
@@ -883,10 +848,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     bf16x4 d4;                                                                                          \
     _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
       float p;                                                                                          \
-      if (RA_ABL_WS_NOVEC) {                                                                            \
-        d4[e] = __builtin_bit_cast(__bf16, (uint16_t)(__float_as_uint(SC[(G) * 4 + e] + DPC[(G) * 4 + e]) >> 16)); \
-        continue;                                                                                       \
-      }                                                                                                 \
       if (!(MASKED)) {                                                                                  \
         p = fast_exp2(fmaf(SC[(G) * 4 + e], c, -lse2));                                                 \
       } else {                                                                                          \
@@ -1021,15 +982,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       }                                                                                                 \
     }                                                                                                   \
     /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, nxt, 0, 0, MASKED);                             \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
     /* step 2t + 1: vector work of block 1, products of block 0 of tile t + 1 (the last tile computes  \
        a block that is never used) */                                                                   \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, nxt, 1, 1, MASKED);                             \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
     cur = nxt;                                                                                          \
   }
@@ -1074,7 +1031,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   }
 #define RA_WS_CMFMA(F, BOP)                                                                             \
   _Pragma("unroll") for (int db = 0; db < 4; db++)                                                      \
-    if (!RA_ABL_WS_NOCONS) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
+    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
     // fa holds the first 16 keys of the block on entry and, on exit, those of block NBLK of buffer NBUF
 #define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
   {                                                                                                     \
@@ -1097,19 +1054,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #define RA_WS_CTILE(S, T)                                                                               \
   {                                                                                                     \
     const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;                               \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_STORE_K(S, prv);                                                                              \
     RA_WS_STORE_V(S, prv);                                                                              \
-    RA_TRACE_MARK2();                                                                                   \
     RA_WS_LOAD_K(S, (T) + 4);                                                                           \
     RA_WS_LOAD_V(S, (T) + 4);                                                                           \
-    RA_TRACE_MARK2();                                                                                   \
     RA_WS_CONSUME(cur, 0, 0, cur, 1);                                                                   \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_CONSUME(cur, 1, 1, nxt, 0);                                                                   \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
     cur = nxt;                                                                                          \
   }
@@ -1301,10 +1252,6 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + 16 * TROW) = S##v1;                                         \
     *(uint4*)(dv_ + 32 * TROW) = S##v2; *(uint4*)(dv_ + 48 * TROW) = S##v3;                             \
   }
-#ifdef RA_TRACE
-  const bool trace_on = blockIdx.x == 0;
-  int trace_n = 0;
-#endif
   if (role == 1) {
     RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
     RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
@@ -1521,15 +1468,11 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
       }                                                                                                 \
     }                                                                                                   \
     /* step 2t: vector work of block 0 of tile t, products of block 1 */                                \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_PRODUCE(s_a, s_b, cur, 0, cur, 1, nxt, 0, 0, MASKED);                                         \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
     /* step 2t + 1: vector work of block 1, products of block 0 of tile t + 1 (the last tile computes  \
        a block that is never used) */                                                                   \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_PRODUCE(s_b, s_a, cur, 1, nxt, 0, nxt, 1, 1, MASKED);                                         \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
     cur = nxt;                                                                                          \
   }
@@ -1599,7 +1542,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   }
 #define RA_WS_CMFMA(F, BOP)                                                                             \
   _Pragma("unroll") for (int db = 0; db < 4; db++)                                                      \
-    if (!RA_ABL_WS_NOCONS) acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
+    acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
     // fa holds the first 16 keys of the block on entry and, on exit, those of block NBLK of buffer NBUF
 #define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
   {                                                                                                     \
@@ -1626,19 +1569,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #define RA_WS_CTILE(S, T)                                                                               \
   {                                                                                                     \
     const int prv = cur == 0 ? 2 : cur - 1, nxt = cur == 2 ? 0 : cur + 1;                               \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_STORE_K(S, prv);                                                                              \
-    RA_TRACE_MARK2();                                                                                   \
     RA_WS_LOAD_K(S, (T) + 4);                                                                           \
-    RA_TRACE_MARK2();                                                                                   \
     RA_WS_CONSUME(cur, 0, 0, cur, 1);                                                                   \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
-    RA_TRACE_MARK();                                                                                    \
     RA_WS_STORE_V(S, prv);                                                                              \
     RA_WS_LOAD_V(S, (T) + 4);                                                                           \
     RA_WS_CONSUME(cur, 1, 1, nxt, 0);                                                                   \
-    RA_TRACE_MARK();                                                                                    \
     __syncthreads();                                                                                    \
     cur = nxt;                                                                                          \
   }
@@ -1742,7 +1679,7 @@ bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
                          p->dkv_out_stride_b % 4 == 0));
 }
 
-int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
+int attn_bwd_mfma(const ra_attn_bwd_params* p, int parts, hipStream_t s) {   // parts: bit 0 dq, bit 1 dk / dv
   BwdArgs a{};
   a.q = (const uint16_t*)p->q; a.k = (const uint16_t*)p->k; a.v = (const uint16_t*)p->v; a.g = (const uint16_t*)p->g;
   a.B = p->B; a.Sq = p->Sq; a.Skv = p->Skv; a.H = p->H;
@@ -1762,7 +1699,7 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, hipStream_t s) {
   RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_mfma: grid too large");
   const dim3 gq((unsigned)((nq + 7) / 8 * 8)), gk((unsigned)((nk + 7) / 8 * 8)), block(512);
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
-  const bool do_dkv = !(p->impl & RA_BWD_ONLY_DQ), do_dq = !(p->impl & RA_BWD_ONLY_DKV);
+  const bool do_dkv = (parts & 2) != 0, do_dq = (parts & 1) != 0;
 #define RA_LAUNCH_BWD(...)                                                               \
   do {                                                                                   \
     if (do_dkv) attn_bwd_dkv_ws_kernel<__VA_ARGS__><<<gk, block, 0, s>>>(a);             \

@@ -191,14 +191,14 @@ static int launch_decode(const DecodeArgs& a, hipStream_t s) {
   return RA_OK;
 }
 
-int decode_fwd(const ra_decode_params* p, int nsplit, hipStream_t s) {
+int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream_t s) {
   DecodeArgs a{};
   a.q = p->q; a.k = p->k; a.v = p->v; a.out = p->out;
   a.B = p->B; a.L = p->L; a.H = p->H; a.D = p->D;
   a.q_sb = p->q_stride_b; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s; a.out_sb = p->out_stride_b;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
-  a.ws = (float*)p->workspace; a.nsplit = nsplit;
+  a.ws = partials; a.nsplit = nsplit;
   if (p->dtype == RA_BF16) {
     if (p->D == 128) return launch_decode<uint16_t, 128>(a, s);
     if (p->D == 64) return launch_decode<uint16_t, 64>(a, s);

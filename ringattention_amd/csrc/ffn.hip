@@ -461,7 +461,6 @@ static int launch_tile(const GemmArgs& g, hipStream_t s) {
 // Tile choice.  One workgroup of the large tiles fills a CU's LDS, so the grid runs in rounds of (number of CUs)
 // workgroups: take the largest tile whose last round is not mostly idle.
 static int pick_tile(int M, int N) {
-  if (const char* e = getenv("RA_GEMM_TILE")) return atoi(e);
   static const int ncu = [] {     // initialised once, thread-safe
     int dev = 0, n = 0;
     hipDeviceProp_t pr;
@@ -480,13 +479,15 @@ static int pick_tile(int M, int N) {
   return 2;
 }
 
+// tile: -1 = pick_tile, else the tile kernel to force (0: 256 x 256, 1: 256 x 128, 2: 128 x 128), which still
+// falls back to a smaller one when the shape does not divide
 template <bool TA, bool TB>
-static int launch_gemm(const GemmArgs& g, hipStream_t s) {
+static int launch_gemm(const GemmArgs& g, int tile, hipStream_t s) {
   if (g.M % 128 || g.N % 128 || g.K % GBK) {
     set_error("gemm_bf16: M, N must be multiples of 128 and K of 64 (got %d, %d, %d)", g.M, g.N, g.K);
     return RA_ERR_UNSUPPORTED;
   }
-  int t = pick_tile(g.M, g.N);
+  int t = tile >= 0 ? tile : pick_tile(g.M, g.N);
   if (t == 0 && (g.M % 256 || g.N % 256)) t = 1;
   // the 4-wavefront kernel addresses an operand through a buffer descriptor at its tile's origin with 32-bit byte
   // offsets: what a tile can reach (a whole operand in the worst case) must stay below 2^31 bytes
@@ -499,17 +500,17 @@ static int launch_gemm(const GemmArgs& g, hipStream_t s) {
   }
 }
 
-static int gemm_dispatch(const GemmArgs& g, int ta, int tb, hipStream_t s) {
-  if (ta && tb) return launch_gemm<true, true>(g, s);
-  if (ta) return launch_gemm<true, false>(g, s);
-  if (tb) return launch_gemm<false, true>(g, s);
-  return launch_gemm<false, false>(g, s);
+static int gemm_dispatch(const GemmArgs& g, int ta, int tb, int tile, hipStream_t s) {
+  if (ta && tb) return launch_gemm<true, true>(g, tile, s);
+  if (ta) return launch_gemm<true, false>(g, tile, s);
+  if (tb) return launch_gemm<false, true>(g, tile, s);
+  return launch_gemm<false, false>(g, tile, s);
 }
 
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype, int beta_one,
-              hipStream_t s) {
+              int tile, hipStream_t s) {
   GemmArgs g{(const uint16_t*)A, (const uint16_t*)B, nullptr, nullptr, C, M, N, K, c_dtype == RA_F32, beta_one};
-  return gemm_dispatch(g, ta, tb, s);
+  return gemm_dispatch(g, ta, tb, tile, s);
 }
 
 // ------------------------------------------------------------------ SwiGLU elementwise parts
@@ -557,37 +558,37 @@ static int check_ffn_shape(const ra_swiglu_params* p, const char* who) {
 
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s) {
   if (int rc = check_ffn_shape(p, "swiglu_fwd")) return rc;
-  const int T = p->T, d = p->d, f = p->f;
-  if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;     // a = x w1
-  if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;     // b = x w3
+  const int T = p->T, d = p->d, f = p->f, tile = p->gemm_tile - 1;
+  if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;     // a = x w1
+  if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;     // b = x w3
   const int64_t n8 = (int64_t)T * f / 8;
   swiglu_act_kernel<<<2048, 256, 0, s>>>((const uint16_t*)p->a, (const uint16_t*)p->b, (uint16_t*)p->h, n8);
   RA_CHECK_LAUNCH("swiglu_act");
-  return gemm_bf16(p->h, p->w2, p->y, T, d, f, 0, 0, RA_BF16, 0, s);                       // y = h w2
+  return gemm_bf16(p->h, p->w2, p->y, T, d, f, 0, 0, RA_BF16, 0, tile, s);                 // y = h w2
 }
 
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s) {
   if (int rc = check_ffn_shape(p, "swiglu_bwd")) return rc;
-  const int T = p->T, d = p->d, f = p->f;
+  const int T = p->T, d = p->d, f = p->f, tile = p->gemm_tile - 1;
   // recompute the pre-activations (nothing_saveable) unless the caller kept them, then
   //   dh = dy w2^T ; da, db from the activation ; dx = da w1^T + db w3^T
   //   dw1 += x^T da ; dw3 += x^T db ; dw2 += h^T dy
   if (!p->preact_saved) {
-    if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
-    if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, s)) return rc;
+    if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;
+    if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;
   }
   // dh goes into the da buffer first, the activation backward then rewrites it in place
-  if (int rc = gemm_bf16(p->dy, p->w2, p->da, T, f, d, 0, 1, RA_BF16, 0, s)) return rc;
+  if (int rc = gemm_bf16(p->dy, p->w2, p->da, T, f, d, 0, 1, RA_BF16, 0, tile, s)) return rc;
   const int64_t n8 = (int64_t)T * f / 8;
   swiglu_act_bwd_kernel<<<2048, 256, 0, s>>>((const uint16_t*)p->a, (const uint16_t*)p->b, (const uint16_t*)p->da,
                                              (uint16_t*)p->h, (uint16_t*)p->da, (uint16_t*)p->db, n8);
   RA_CHECK_LAUNCH("swiglu_act_bwd");
   GemmArgs g{(const uint16_t*)p->da, (const uint16_t*)p->w1, (const uint16_t*)p->db, (const uint16_t*)p->w3,
              p->dx, T, d, f, 0, 0};
-  if (int rc = gemm_dispatch(g, 0, 1, s)) return rc;                                        // dx
-  if (int rc = gemm_bf16(p->x, p->da, p->dw1, d, f, T, 1, 0, RA_F32, 1, s)) return rc;
-  if (int rc = gemm_bf16(p->x, p->db, p->dw3, d, f, T, 1, 0, RA_F32, 1, s)) return rc;
-  return gemm_bf16(p->h, p->dy, p->dw2, f, d, T, 1, 0, RA_F32, 1, s);
+  if (int rc = gemm_dispatch(g, 0, 1, tile, s)) return rc;                                  // dx
+  if (int rc = gemm_bf16(p->x, p->da, p->dw1, d, f, T, 1, 0, RA_F32, 1, tile, s)) return rc;
+  if (int rc = gemm_bf16(p->x, p->db, p->dw3, d, f, T, 1, 0, RA_F32, 1, tile, s)) return rc;
+  return gemm_bf16(p->h, p->dy, p->dw2, f, d, T, 1, 0, RA_F32, 1, tile, s);
 }
 
 }  // namespace ra

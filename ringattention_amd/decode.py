@@ -7,21 +7,26 @@ import torch
 from . import _lib as L
 from .ringattention_hip import _Config, _MaskInputs, _check_qkv, _ra_dtype, _rows, _stream
 
-_WORKSPACES = {}
+
+def decode_workspace(q, k, num_splits=0):
+    """A workspace for ``decode_attention(..., workspace=...)``: what ra_decode_workspace_bytes asks for the
+    shapes of q (B,1,H,D) and the cache k (B,L,H,D).  A caller that captures decode steps into a HIP graph, or
+    that decodes on several streams, owns one such buffer per graph / stream and keeps it alive as long as
+    the graph may replay."""
+    B, _, H, D = q.shape
+    nbytes = L.load().ra_decode_workspace_bytes(B, k.shape[1], H, D, num_splits)
+    return torch.empty(nbytes, dtype=torch.uint8, device=q.device)
 
 
-def _workspace(device, nbytes):
-    ws = _WORKSPACES.get(device)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _WORKSPACES[device] = ws
-    return ws
-
-
-def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs, out=None, num_splits=0):
+def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs, out=None, num_splits=0,
+                     workspace=None):
     """q (B,1,H,D) against the cache buffers k, v (B,L,H,D); cache_idx is a Python int or a device
     int32 scalar (read by the kernel, so the call can sit in a captured graph or a tight loop).
-    blockwise_kwargs must carry query_chunk_size == 1, as q_len // query_chunk_size demands."""
+    blockwise_kwargs must carry query_chunk_size == 1, as q_len // query_chunk_size demands.
+
+    The split-KV partials go to ``workspace`` (see decode_workspace) when one is given; otherwise to a buffer
+    allocated for this call from torch's stream-aware caching allocator, which is safe for eager calls on any
+    stream but must not be captured into a graph (the graph would keep writing to a block torch hands out again)."""
     cfg = _Config(blockwise_kwargs)
     if cfg.pdrop > 0.0:
         raise NotImplementedError("attention dropout together with cache_idx is not supported")
@@ -49,8 +54,11 @@ def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwarg
     p.out_stride_b = _rows(out)[0]
     q_start = mi.cache_idx_host if mi.cache_idx_host is not None else 0
     p.mask = mi.fill(cfg, q_start, 0, False)
-    nbytes = lib.ra_decode_workspace_bytes(B, L_buf, H, D, num_splits)
-    ws = _workspace(q.device, nbytes)
-    p.workspace, p.workspace_bytes, p.num_splits = ws.data_ptr(), ws.numel(), num_splits
+    p.num_splits = num_splits
+    if workspace is None:
+        workspace = decode_workspace(q, k, num_splits)
+    elif workspace.device != q.device or workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+        raise ValueError("workspace must be a contiguous uint8 tensor on the device of q")
+    p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
     L.check(lib.ra_decode_fwd(ctypes.byref(p), _stream()), "ra_decode_fwd")
     return out

@@ -15,13 +15,14 @@ def _ptr(t):
 class _SwiGLUFn(torch.autograd.Function):
     """y = (silu(x w1) * (x w3)) w2 on one chunk of tokens.  Nothing but x is kept for the backward
     pass (the reference's default policy is nothing_saveable, ringattention_jax.py:334): the
-    pre-activations are recomputed."""
+    pre-activations are recomputed.  ``gemm_tile`` is ra_swiglu_params.gemm_tile."""
 
     @staticmethod
-    def forward(ctx, x, w1, w2, w3):
+    def forward(ctx, x, w1, w2, w3, gemm_tile=0):
         T, d = x.shape
         f = w1.shape[1]
         dev = x.device
+        ctx.gemm_tile = gemm_tile
         a = torch.empty((T, f), dtype=torch.bfloat16, device=dev)
         b = torch.empty_like(a)
         h = torch.empty_like(a)
@@ -30,6 +31,7 @@ class _SwiGLUFn(torch.autograd.Function):
         p.T, p.d, p.f = T, d, f
         p.x, p.w1, p.w2, p.w3 = x.data_ptr(), w1.data_ptr(), w2.data_ptr(), w3.data_ptr()
         p.a, p.b, p.h, p.y = a.data_ptr(), b.data_ptr(), h.data_ptr(), y.data_ptr()
+        p.gemm_tile = gemm_tile
         L.check(L.load().ra_swiglu_fwd(ctypes.byref(p), _stream()), "ra_swiglu_fwd")
         ctx.save_for_backward(x, w1, w2, w3)
         return y
@@ -54,8 +56,9 @@ class _SwiGLUFn(torch.autograd.Function):
         p.dy, p.dx = dy.data_ptr(), dx.data_ptr()
         p.dw1, p.dw2, p.dw3 = dw1.data_ptr(), dw2.data_ptr(), dw3.data_ptr()
         p.da, p.db = da.data_ptr(), db.data_ptr()
+        p.gemm_tile = ctx.gemm_tile
         L.check(L.load().ra_swiglu_bwd(ctypes.byref(p), _stream()), "ra_swiglu_bwd")
-        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype)
+        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None
 
 
 class _BlockwiseSwiGLUFn(torch.autograd.Function):
@@ -67,8 +70,9 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
     (nothing_saveable, ringattention_jax.py:334).  The results are the same bits either way."""
 
     @staticmethod
-    def forward(ctx, x, w1, w2, w3, chunk_tokens, save_preact):
+    def forward(ctx, x, w1, w2, w3, chunk_tokens, save_preact, gemm_tile=0):
         T, d = x.shape
+        ctx.gemm_tile = gemm_tile
         f = w1.shape[1]
         bf = dict(dtype=torch.bfloat16, device=x.device)
         save_preact = bool(save_preact) and any(ctx.needs_input_grad[:4])
@@ -81,6 +85,7 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
         p.T, p.d, p.f = chunk_tokens, d, f
         p.w1, p.w2, p.w3 = w1.data_ptr(), w2.data_ptr(), w3.data_ptr()
         p.a, p.b, p.h = a.data_ptr(), b.data_ptr(), h.data_ptr()
+        p.gemm_tile = gemm_tile
         for t0 in range(0, T, chunk_tokens):
             p.x, p.y = x[t0:].data_ptr(), y[t0:].data_ptr()
             if save_preact:
@@ -116,34 +121,23 @@ class _BlockwiseSwiGLUFn(torch.autograd.Function):
         p.dw1, p.dw2, p.dw3 = dw1.data_ptr(), dw2.data_ptr(), dw3.data_ptr()
         p.da, p.db = da.data_ptr(), db.data_ptr()
         p.preact_saved = 1 if saved else 0
+        p.gemm_tile = ctx.gemm_tile
         for t0 in range(0, T, ct):
             p.x, p.dy, p.dx = x[t0:].data_ptr(), dy[t0:].data_ptr(), dx[t0:].data_ptr()
             if saved:
                 p.a, p.b = a[t0:].data_ptr(), b[t0:].data_ptr()
             L.check(lib.ra_swiglu_bwd(ctypes.byref(p), stream), "ra_swiglu_bwd")
-        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None, None
+        return dx, dw1.to(w1.dtype), dw2.to(w2.dtype), dw3.to(w3.dtype), None, None, None
 
 
-# Tokens are independent in a token-wise MLP, so several consecutive chunks may share one launch: the
-# result is the same, the GEMMs fill the 256 CUs in whole rounds, and the fp32 weight-gradient
-# accumulators are read and written once per slab instead of once per chunk.  The scratch of a slab
-# (five (tokens, intermediate) bf16 buffers) is what bounds it: 16384 tokens x 11008 is 1.8 GB.
-MAX_SLAB_TOKENS = 16384
-
-# policy=None keeps the pre-activations of the whole scan for the backward pass when they are small next to the
-# device's memory: at most this many bytes and at most a quarter of what is free.  65536 tokens x 11008 are 2.9 GB.
-PREACT_BUDGET_BYTES = 32 << 30
-
-
-def _save_preactivations(policy, tokens, intermediate, device):
-    """What ``policy`` (ringattention_jax.py:334) means here: "nothing_saveable" (the reference's default object,
-    by name) recomputes x w1 and x w3 in the backward pass; "save_preactivations" keeps them; None decides by
-    size.  Either way the same bits come out; only memory (4 * tokens * intermediate bytes) and two GEMMs per
-    chunk in the backward pass differ."""
+def _save_preactivations(policy):
+    """What ``policy`` (ringattention_jax.py:334) means here.  "nothing_saveable" - the reference's default, by
+    name or as an object of that name, and also what None means - recomputes x w1 and x w3 in the backward pass,
+    so that nothing but the input of the scan outlives a chunk.  "save_preactivations" (or
+    "everything_saveable") is the explicit opt-in that keeps them: 4 * tokens * intermediate bytes (2.9 GB at
+    65536 x 11008) for two GEMMs less per chunk in the backward pass.  The same bits come out either way."""
     if policy is None:
-        need = 4 * tokens * intermediate
-        free, _ = torch.cuda.mem_get_info(device)
-        return need <= PREACT_BUDGET_BYTES and need <= free // 4
+        return False
     name = policy if isinstance(policy, str) else getattr(policy, "__name__", "")
     if name == "nothing_saveable":
         return False
@@ -152,9 +146,16 @@ def _save_preactivations(policy, tokens, intermediate, device):
     raise ValueError("policy must be None, 'nothing_saveable' or 'save_preactivations'")
 
 
-def _slab_tokens(chunk_size, n_chunks):
-    """Tokens per launch: the largest whole number of chunks within MAX_SLAB_TOKENS that divides the scan."""
-    g = max(1, min(n_chunks, MAX_SLAB_TOKENS // chunk_size))
+def _slab_tokens(chunk_size, n_chunks, launch_tokens=None):
+    """Tokens per launch.  By default one chunk, so the scratch of a step (five (chunk_size, intermediate) bf16
+    buffers) is what chunk_size implies, as in the reference's scan.  Tokens are independent in a token-wise MLP,
+    so a caller with memory to spare may let consecutive chunks share a launch (``launch_tokens``): the result is
+    the same, the GEMMs fill the 256 CUs in whole rounds, and the fp32 weight-gradient accumulators are read and
+    written once per launch instead of once per chunk.  The largest whole number of chunks within
+    ``launch_tokens`` that divides the scan is taken (16384 tokens x 11008 are 1.8 GB of scratch)."""
+    if launch_tokens is None:
+        return chunk_size
+    g = max(1, min(n_chunks, int(launch_tokens) // chunk_size))
     while n_chunks % g:
         g -= 1
     return chunk_size * g
@@ -164,8 +165,10 @@ class SwiGLU(torch.nn.Module):
     """The LLaMA-style MLP the reference's README pairs with blockwise_feedforward:
     w2(silu(x w1) * (x w3)); weights stored (in, out), bf16."""
 
-    def __init__(self, hidden, intermediate, device=None, init_std=0.02):
+    def __init__(self, hidden, intermediate, device=None, init_std=0.02, gemm_tile=None):
         super().__init__()
+        # None: the library picks the GEMM tile kernel; 0 / 1 / 2 force one (ra_swiglu_params.gemm_tile), for tests
+        self.gemm_tile = 0 if gemm_tile is None else int(gemm_tile) + 1
         mk = lambda i, o: torch.nn.Parameter(
             (torch.randn(i, o, device=device, dtype=torch.float32) * init_std).to(torch.bfloat16))
         self.w1 = mk(hidden, intermediate)
@@ -179,20 +182,23 @@ class SwiGLU(torch.nn.Module):
             raise NotImplementedError("SwiGLU kernels are bf16")
         if not x.is_cuda:
             raise RuntimeError("ringattention_amd runs on the GPU only")
-        y = _SwiGLUFn.apply(x.contiguous(), self.w1, self.w2, self.w3)
+        y = _SwiGLUFn.apply(x.contiguous(), self.w1, self.w2, self.w3, self.gemm_tile)
         return y.reshape(*shp[:-1], y.shape[-1])
 
 
-def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), policy=None, pre_remat=True):
+def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), policy="nothing_saveable",
+                          pre_remat=True, launch_tokens=None):
     """ringattention_jax.py:333-352: apply ``feedforward`` to ``chunk_size`` tokens at a time.
 
     The reference groups tokens with 'b (c n) d -> b c n d', c=chunk_size and scans over n, so step
     j sees the strided token set {ci * n + j}.  A generic callable gets exactly those groups.  A
     ``SwiGLU`` instance is token-wise, so it is fed contiguous slabs of chunk_size tokens instead:
     the same number of steps and the same result, with dense memory access.  ``policy`` selects what the
-    SwiGLU scan keeps for its backward pass (see _save_preactivations: the reference's default recomputes
-    everything to save memory; with None the pre-activations are kept when they are small next to the device's
-    memory); ``pre_remat`` / ``static_argnums`` steer XLA rematerialisation only."""
+    SwiGLU scan keeps for its backward pass: the reference's default ``nothing_saveable`` recomputes the
+    pre-activations, ``"save_preactivations"`` is the opt-in that keeps them (see _save_preactivations).
+    ``launch_tokens`` (no counterpart in the reference) lets consecutive chunks share a kernel launch and its
+    scratch, see _slab_tokens; the default keeps a step's memory at what ``chunk_size`` implies.
+    ``pre_remat`` / ``static_argnums`` steer XLA rematerialisation only."""
     b, s, d = inputs.shape
     if s % chunk_size:
         raise ValueError("sequence length %d must divide by chunk_size %d" % (s, chunk_size))
@@ -205,8 +211,8 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
         # contiguous slabs of chunk_size tokens (batch rows one after the other: a token-wise MLP does not see the
         # difference), one autograd node for the whole scan
         y = _BlockwiseSwiGLUFn.apply(inputs.reshape(b * s, d).contiguous(), feedforward.w1, feedforward.w2,
-                                     feedforward.w3, _slab_tokens(chunk_size, b * n),
-                                     _save_preactivations(policy, b * s, feedforward.w1.shape[1], inputs.device))
+                                     feedforward.w3, _slab_tokens(chunk_size, b * n, launch_tokens),
+                                     _save_preactivations(policy), feedforward.gemm_tile)
         return y.reshape(b, s, y.shape[-1])
     x = inputs.reshape(b, chunk_size, n, d)
     outs = [feedforward(x[:, :, j, :]) for j in range(n)]
@@ -214,14 +220,20 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
     return out.reshape(b, s, out.shape[-1])
 
 
-def gemm_bf16(A, B, trans_a=False, trans_b=False, out_dtype=torch.bfloat16, out=None, accumulate=False):
-    """C = op(A) op(B) with the library's bf16 MFMA GEMM (used by the SwiGLU kernels; exposed for tests)."""
+def gemm_bf16(A, B, trans_a=False, trans_b=False, out_dtype=torch.bfloat16, out=None, accumulate=False, tile=None):
+    """C = op(A) op(B) with the library's bf16 MFMA GEMM (used by the SwiGLU kernels; exposed for tests).
+    ``tile`` 0 / 1 / 2 names the tile kernel (ra_gemm_bf16_tile); None lets the library choose."""
     M = A.shape[1] if trans_a else A.shape[0]
     K = A.shape[0] if trans_a else A.shape[1]
     N = B.shape[0] if trans_b else B.shape[1]
     if out is None:
         out = torch.zeros((M, N), dtype=out_dtype, device=A.device)
     cd = L.RA_F32 if out.dtype == torch.float32 else L.RA_BF16
-    L.check(L.load().ra_gemm_bf16(A.data_ptr(), B.data_ptr(), out.data_ptr(), M, N, K, int(trans_a),
-                                  int(trans_b), cd, int(accumulate), _stream()), "ra_gemm_bf16")
+    if tile is None:
+        L.check(L.load().ra_gemm_bf16(A.data_ptr(), B.data_ptr(), out.data_ptr(), M, N, K, int(trans_a),
+                                      int(trans_b), cd, int(accumulate), _stream()), "ra_gemm_bf16")
+    else:
+        L.check(L.load().ra_gemm_bf16_tile(A.data_ptr(), B.data_ptr(), out.data_ptr(), M, N, K, int(trans_a),
+                                           int(trans_b), cd, int(accumulate), int(tile), _stream()),
+                "ra_gemm_bf16_tile")
     return out

@@ -136,7 +136,8 @@ class _Config:
         self.mask_min = float(torch.finfo(self.dtype).min)
         self.impl = {"auto": L.RA_IMPL_AUTO, "generic": L.RA_IMPL_GENERIC, "mfma": L.RA_IMPL_MFMA}[
             kw.get("impl", "auto")]
-        self.bwd_only = {None: 0, "dq": L.RA_BWD_ONLY_DQ, "dkv": L.RA_BWD_ONLY_DKV}[kw.get("bwd_only", None)]
+        # measurement hook: launch one of the two backward kernels alone (ra_attn_bwd_block_part)
+        self.bwd_only = {None: 0, "dq": L.RA_BWD_PART_DQ, "dkv": L.RA_BWD_PART_DKV}[kw.get("bwd_only", None)]
         self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
         # policy / precision / prevent_cse only steer XLA rematerialisation: the kernels always recompute
         # the probabilities in the backward pass.
@@ -487,8 +488,11 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
         mi.use_dropout(cfg, B, H, Sq, Skv, q_chunk_idx_start, k_chunk_idx_start, q.device)
         skip = False
     p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
-    p.impl = cfg.impl | cfg.bwd_only
-    L.check(L.load().ra_attn_bwd_block(ctypes.byref(p), _stream()), "ra_attn_bwd_block")
+    p.impl = cfg.impl
+    if cfg.bwd_only:
+        L.check(L.load().ra_attn_bwd_block_part(ctypes.byref(p), cfg.bwd_only, _stream()), "ra_attn_bwd_block_part")
+    else:
+        L.check(L.load().ra_attn_bwd_block(ctypes.byref(p), _stream()), "ra_attn_bwd_block")
     return dq, dk, dv
 
 
@@ -691,7 +695,9 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
     arrays and the sequence axis is split over the virtual devices.  attn_bias (B|1, H|1, 1, K_total)
     and segment_ids (B|1, S_total) are global / replicated, as in the reference's shard_map specs.
     One query token with cache_idx set takes the streaming decode kernel."""
-    if cache_idx is not None and q.shape[1] == 1 and axis_size(axis_name) == 1 and not (
+    # (the streaming kernel serves head sizes 64 and 128; any other takes the blockwise kernels below, like a call
+    # that wants gradients)
+    if cache_idx is not None and q.shape[1] == 1 and q.shape[3] in (64, 128) and axis_size(axis_name) == 1 and not (
             torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
         from .decode import decode_attention
         return decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs)

@@ -38,21 +38,20 @@ def test_gemm_layouts(ta, tb, shape):
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("tile", [0, 1, 2])
 @pytest.mark.parametrize("shape", [(768, 512, 320), (1280, 256, 128)])
-def test_gemm_every_tile_kernel(monkeypatch, ta, tb, tile, shape):
+def test_gemm_every_tile_kernel(ta, tb, tile, shape):
     """Each tile kernel (0: 256 x 256 over four wavefronts, 1: 256 x 128, 2: 128 x 128) on shapes whose tile
     counts are no multiple of the 8 XCDs or of the tile-row group, so the workgroup -> tile order and its
-    surplus workgroups are exercised; the library picks the tile itself unless RA_GEMM_TILE names one."""
+    surplus workgroups are exercised; ra_gemm_bf16_tile names the tile kernel that ra_gemm_bf16 would pick itself."""
     M, N, K = shape
     print("gemm tile", tile, ta, tb, shape, flush=True)
-    monkeypatch.setenv("RA_GEMM_TILE", str(tile))
     g = torch.Generator().manual_seed(M + N + K + tile)
     A = torch.randn((K, M) if ta else (M, K), generator=g).bfloat16()
     B = torch.randn((N, K) if tb else (K, N), generator=g).bfloat16()
     ref = (A.float().t() if ta else A.float()) @ (B.float().t() if tb else B.float())
-    out = ra.gemm_bf16(A.to(DEV), B.to(DEV), trans_a=ta, trans_b=tb)
+    out = ra.gemm_bf16(A.to(DEV), B.to(DEV), trans_a=ta, trans_b=tb, tile=tile)
     rel_ok(out, ref, "bf16 out")
     acc = torch.ones(M, N, dtype=torch.float32, device=DEV)
-    ra.gemm_bf16(A.to(DEV), B.to(DEV), trans_a=ta, trans_b=tb, out=acc, accumulate=True)
+    ra.gemm_bf16(A.to(DEV), B.to(DEV), trans_a=ta, trans_b=tb, out=acc, accumulate=True, tile=tile)
     assert errors(acc, ref + 1.0)[1] < 1e-5
 
 
@@ -64,16 +63,14 @@ def test_gemm_rejects_ragged_shapes():
 
 
 @pytest.mark.parametrize("tile,shape", [(None, (256, 256, 384)), (0, (512, 256, 768)), (1, (512, 256, 768))])
-def test_swiglu_forward_backward_match_autograd(monkeypatch, tile, shape):
+def test_swiglu_forward_backward_match_autograd(tile, shape):
     """SwiGLU forward and backward (including the two-operand-pair GEMM of dx and the fp32 accumulation of the
     weight gradients) with the library's own tile choice and with each of the large tile kernels forced."""
     T, d, f = shape
-    if tile is not None:
-        monkeypatch.setenv("RA_GEMM_TILE", str(tile))
     g = torch.Generator().manual_seed(0)
     x = torch.randn(1, T, d, generator=g).bfloat16()
     dy = torch.randn(1, T, d, generator=g).bfloat16()
-    ff = ra.SwiGLU(d, f, device=DEV, init_std=0.05)
+    ff = ra.SwiGLU(d, f, device=DEV, init_std=0.05, gemm_tile=tile)
     w1, w2, w3 = (w.detach().float().cpu().requires_grad_(True) for w in (ff.w1, ff.w2, ff.w3))
     xr = x.float().requires_grad_(True)
     yr = O.swiglu(xr, w1, w2, w3)
@@ -132,34 +129,42 @@ def test_blockwise_feedforward_single_batch_scan_gradients():
     rel_ok(ff.w3.grad, w3.grad, "dw3")
 
 
-def test_blockwise_feedforward_policies_give_the_same_bits(monkeypatch):
-    """policy="nothing_saveable" (the reference's default: the backward pass recomputes x w1 and x w3), policy=
-    "save_preactivations" (they stay in memory) and policy=None (decided by size) differ in memory and in two GEMMs
-    per chunk, not in a single bit of y, dx or the weight gradients."""
+def test_blockwise_feedforward_policies_give_the_same_bits():
+    """policy="nothing_saveable" (the reference's default, ringattention_jax.py:334: the backward pass recomputes
+    x w1 and x w3; also what None means) and the opt-in policy="save_preactivations" (they stay in memory) differ in
+    memory and in two GEMMs per chunk, not in a single bit of y, dx or the weight gradients; nor does letting
+    several chunks share a launch (launch_tokens)."""
     from ringattention_amd import feedforward as F
     S, d, f, chunk = 2048, 256, 512, 256
     g = torch.Generator().manual_seed(7)
     x = torch.randn(2, S, d, generator=g).bfloat16().to(DEV)
     dy = torch.randn(2, S, d, generator=g).bfloat16().to(DEV)
     ff = ra.SwiGLU(d, f, device=DEV, init_std=0.05)
-    monkeypatch.setattr(F, "MAX_SLAB_TOKENS", 1024)        # several slabs, so that the kept buffers are sliced
     res = {}
-    for policy in ("nothing_saveable", "save_preactivations", None):
+    # launch_tokens 1024: several launches of four chunks, so that the kept buffers are sliced
+    for policy, launch in (("nothing_saveable", None), ("save_preactivations", None), (None, None),
+                           ("nothing_saveable", 1024), ("save_preactivations", 1024)):
         for prm in ff.parameters():
             prm.grad = None
         xd = x.clone().requires_grad_(True)
-        y = ra.blockwise_feedforward(ff, xd, chunk, policy=policy)
+        y = ra.blockwise_feedforward(ff, xd, chunk, policy=policy, launch_tokens=launch)
         y.backward(dy)
-        res[policy] = (y.detach(), xd.grad, ff.w1.grad.clone(), ff.w2.grad.clone(), ff.w3.grad.clone())
-    for policy in ("save_preactivations", None):
-        for a, b in zip(res[policy], res["nothing_saveable"]):
-            assert torch.equal(a, b), policy
-    # the decision by size
-    assert F._save_preactivations(None, 65536, 11008, x.device) is True
-    monkeypatch.setattr(F, "PREACT_BUDGET_BYTES", 1 << 20)
-    assert F._save_preactivations(None, 65536, 11008, x.device) is False
+        res[(policy, launch)] = (y.detach(), xd.grad, ff.w1.grad.clone(), ff.w2.grad.clone(), ff.w3.grad.clone())
+    base = res[("nothing_saveable", None)]
+    for key, val in res.items():
+        for i, (a, b) in enumerate(zip(val, base)):
+            if i >= 2 and key[1] != None:
+                # weight gradients: fp32 sums over launches of another size round differently in the last bit
+                assert errors(a, b)[1] < 1e-2, key
+            else:
+                assert torch.equal(a, b), key
+    # the default is the reference's: nothing kept, one chunk per launch
+    assert F._save_preactivations(None) is False and F._save_preactivations("nothing_saveable") is False
+    assert F._save_preactivations("save_preactivations") is True
+    assert F._slab_tokens(chunk, 16) == chunk and F._slab_tokens(chunk, 16, 1024) == 1024
+    assert F._slab_tokens(chunk, 6, 1024) == 3 * chunk          # a whole number of chunks that divides the scan
     with pytest.raises(ValueError):
         ra.blockwise_feedforward(ff, x, chunk, policy="dots_saveable")
     # no gradient wanted: nothing is kept
     with torch.no_grad():
-        assert torch.equal(ra.blockwise_feedforward(ff, x, chunk, policy="save_preactivations"), res[None][0])
+        assert torch.equal(ra.blockwise_feedforward(ff, x, chunk, policy="save_preactivations"), base[0])

@@ -130,9 +130,11 @@ def test_decode_step_replays_from_a_hip_graph():
     ci = torch.zeros(1, dtype=torch.int32, device=DEV)
     kw = kwargs(1, kc, 1)
 
+    ws = ra.decode_workspace(q, k_cache)       # owned by the caller: it must outlive every replay of the graph
+
     def step(kc_, vc_, qr_, out_):
         ra.rope_kv_append(q, kn, vn, kc_, vc_, ci, q_out=qr_)
-        ra.decode_attention(qr_, kc_, vc_, None, None, ci, kw, out=out_)
+        ra.decode_attention(qr_, kc_, vc_, None, None, ci, kw, out=out_, workspace=ws)
 
     ci.fill_(500)
     step(k_cache.clone(), v_cache.clone(), torch.empty_like(q), torch.empty_like(q))     # warm-up outside the capture

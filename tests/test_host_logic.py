@@ -14,9 +14,11 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_library_exports_every_declared_symbol():
-    header = open(os.path.join(ROOT, "include", "ringattn_hip.h")).read()
-    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
-    declared = set(re.findall(r"\b(ra_[a-z0-9_]+)\s*\(", header))
+    declared = set()
+    for name in ("ringattn_hip.h", "ringattn_hip_measure.h"):
+        header = open(os.path.join(ROOT, "include", name)).read()
+        header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+        declared |= set(re.findall(r"\b(ra_[a-z0-9_]+)\s*\(", header))
     assert declared, "no declarations parsed"
     assert declared == set(_lib.SYMBOLS), declared ^ set(_lib.SYMBOLS)
     lib = _lib.load()
@@ -97,6 +99,10 @@ def test_invalid_arguments_return_codes_without_gpu():
     assert lib.ra_attn_fwd_block(ctypes.byref(p), None) == _lib.RA_ERR_INVALID
     assert lib.ra_decode_fwd(None, None) == _lib.RA_ERR_INVALID
     assert lib.ra_decode_workspace_bytes(16, 1024, 32, 128, 4) == 16 * 32 * 4 * 130 * 4
+    # measurement hooks validate too
+    one_ = ctypes.c_void_p(16)
+    assert lib.ra_attn_bwd_block_part(None, 3, None) == _lib.RA_ERR_INVALID
+    assert lib.ra_gemm_bf16_tile(one_, one_, one_, 128, 128, 64, 0, 0, 1, 0, 7, None) == _lib.RA_ERR_INVALID
     # ra_keep_pack validates before touching the device
     assert lib.ra_keep_pack(None, 0, 0, 0, 1, 1, 1, 64, 64, None, None, None, None) == _lib.RA_ERR_INVALID
     one = ctypes.c_void_p(16)      # any non-null address: the shape check comes before any use
