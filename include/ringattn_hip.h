@@ -225,6 +225,22 @@ size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int
 int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream);
 
 /*
+ * ra_decode_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same computation and same kernels as
+ * ra_decode_fwd, but the split-KV partials go to a buffer that lives inside the library (a file-scope device array
+ * of RA_DECODE_STATIC_SCRATCH_BYTES per GPU, held until the process ends) instead of p->workspace, which is ignored
+ * together with p->workspace_bytes.  The call allocates and frees nothing.  The number of key splits is
+ * p->num_splits, or the automatic choice, lowered to what fits the buffer:
+ *   B * H * splits * (D + 2) * sizeof(float) <= RA_DECODE_STATIC_SCRATCH_BYTES;
+ * a shape whose single split does not fit (B * H * (D + 2) * 4 bytes above the limit) is refused with
+ * RA_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's buffer: two calls that overlap in time on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered.  Nothing in the buffer has to start at zero: every
+ * partial a call reads was written by that call.
+ */
+enum { RA_DECODE_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024 };
+int ra_decode_fwd_static(const ra_decode_params* p, ra_stream_t stream);
+
+/*
  * SwiGLU feed-forward on one chunk of tokens, the body that blockwise_feedforward
  * (ringattention_jax.py:333-352) scans: y = (silu(x w1) * (x w3)) w2, bf16, fp32 accumulation.
  * x (T,d) ; w1,w3 (d,f) ; w2 (f,d) ; row-major.  a,b (T,f) bf16 are written by the forward

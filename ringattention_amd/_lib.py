@@ -13,6 +13,7 @@ RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
 RA_F32, RA_BF16 = 0, 1
 RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
 RA_BWD_PART_DQ, RA_BWD_PART_DKV = 1, 2          # include/ringattn_hip_measure.h
+RA_DECODE_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 RA_SEG_TILE = 64
 RA_KEEP_WHERE, RA_KEEP_DROPOUT = 0, 1
 RA_GRAD_INIT_DQ, RA_GRAD_INIT_DKV = 1, 2
@@ -114,6 +115,7 @@ SYMBOLS = {
     "ra_attn_bwd_block": (C.c_int, [C.POINTER(RaAttnBwdParams), vp]),
     "ra_decode_workspace_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
     "ra_decode_fwd": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
+    "ra_decode_fwd_static": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
     "ra_swiglu_fwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
     "ra_swiglu_bwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
     "ra_gemm_bf16": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp]),

@@ -35,6 +35,7 @@ int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, in
                         hipStream_t s);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream_t s);
+int decode_static_scratch(float** ptr);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s);
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
@@ -309,6 +310,20 @@ int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->workspace_bytes >= need, RA_ERR_INVALID, "decode_fwd: workspace %zu bytes < %zu needed",
              p->workspace_bytes, need);
   return decode_fwd(p, (float*)p->workspace, ns, (hipStream_t)stream);
+}
+
+int ra_decode_fwd_static(const ra_decode_params* p, ra_stream_t stream) {
+  if (int rc = check_decode(p, "decode_fwd_static")) return rc;
+  const size_t per_split = (size_t)p->B * p->H * (p->D + 2) * sizeof(float);
+  RA_REQUIRE(per_split <= (size_t)RA_DECODE_STATIC_SCRATCH_BYTES, RA_ERR_UNSUPPORTED,
+             "decode_fwd_static: B * H * (D + 2) * 4 = %zu bytes exceed the built-in scratch buffer of %d bytes; "
+             "use ra_decode_fwd with a workspace", per_split, (int)RA_DECODE_STATIC_SCRATCH_BYTES);
+  int ns = p->num_splits > 0 ? p->num_splits : decode_pick_splits(p->B, p->L, p->H, p->D, p->dtype);
+  const int fit = (int)((size_t)RA_DECODE_STATIC_SCRATCH_BYTES / per_split);
+  if (ns > fit) ns = fit;
+  float* scratch = nullptr;
+  if (int rc = decode_static_scratch(&scratch)) return rc;
+  return decode_fwd(p, scratch, ns, (hipStream_t)stream);
 }
 
 int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream) {

@@ -11,6 +11,7 @@
 // key chunks run iff below_or_on_diag (:324-331) says so, keys inside a chunk
 // that runs are masked with finfo.min (:301-309), bias is added after the
 // 1/sqrt(D) scaling and clamped to <= 0 when a mask is on (:134-136,:299,:309).
+#include <mutex>
 #include "common.hpp"
 
 namespace ra {
@@ -188,6 +189,36 @@ static int launch_decode(const DecodeArgs& a, hipStream_t s) {
   RA_CHECK_LAUNCH("decode_split");
   decode_combine_kernel<T, D><<<dim3(a.H, a.B), D, 0, s>>>(a);
   RA_CHECK_LAUNCH("decode_combine");
+  return RA_OK;
+}
+
+// ---- the buffer of ra_decode_fwd_static: split-KV partials for callers that cannot allocate.  Each GPU holds its
+// own copy of the array at its own address; in host code the array's name is only a handle for
+// hipGetSymbolAddress, never a device address, so every launch takes the pointer looked up here.
+static __device__ __align__(256) unsigned char decode_scratch[RA_DECODE_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static float* g_scratch_ptr[kMaxDevices];     // per device, filled on the first call with that device current
+
+int decode_static_scratch(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("decode_fwd_static: no usable current device (%s, device %d)", hipGetErrorString(e), dev);
+    return RA_ERR_LAUNCH;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(decode_scratch));
+    if (e != hipSuccess || !sym) {
+      set_error("decode_fwd_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return RA_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = (float*)sym;
+  }
+  *ptr = g_scratch_ptr[dev];
   return RA_OK;
 }
 

@@ -1,5 +1,5 @@
 """Decode through cache_idx (ringattention_jax.py:31-35 with one query token): host wrapper of the
-streaming kernel ra_decode_fwd."""
+streaming kernels ra_decode_fwd / ra_decode_fwd_static."""
 import ctypes
 
 import torch
@@ -19,14 +19,16 @@ def decode_workspace(q, k, num_splits=0):
 
 
 def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs, out=None, num_splits=0,
-                     workspace=None):
+                     workspace=None, static_scratch=False):
     """q (B,1,H,D) against the cache buffers k, v (B,L,H,D); cache_idx is a Python int or a device
     int32 scalar (read by the kernel, so the call can sit in a captured graph or a tight loop).
     blockwise_kwargs must carry query_chunk_size == 1, as q_len // query_chunk_size demands.
 
     The split-KV partials go to ``workspace`` (see decode_workspace) when one is given; otherwise to a buffer
     allocated for this call from torch's stream-aware caching allocator, which is safe for eager calls on any
-    stream but must not be captured into a graph (the graph would keep writing to a block torch hands out again)."""
+    stream but must not be captured into a graph (the graph would keep writing to a block torch hands out again).
+    ``static_scratch=True`` takes ra_decode_fwd_static instead: no allocation at all, the partials go to the
+    library's built-in 16 MiB buffer of the GPU; calls that overlap in time on one GPU must not use it."""
     cfg = _Config(blockwise_kwargs)
     if cfg.pdrop > 0.0:
         raise NotImplementedError("attention dropout together with cache_idx is not supported")
@@ -55,6 +57,11 @@ def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwarg
     q_start = mi.cache_idx_host if mi.cache_idx_host is not None else 0
     p.mask = mi.fill(cfg, q_start, 0, False)
     p.num_splits = num_splits
+    if static_scratch:
+        if workspace is not None:
+            raise ValueError("static_scratch and workspace exclude each other")
+        L.check(lib.ra_decode_fwd_static(ctypes.byref(p), _stream()), "ra_decode_fwd_static")
+        return out
     if workspace is None:
         workspace = decode_workspace(q, k, num_splits)
     elif workspace.device != q.device or workspace.dtype != torch.uint8 or not workspace.is_contiguous():

@@ -99,10 +99,19 @@ def test_invalid_arguments_return_codes_without_gpu():
     assert lib.ra_attn_fwd_block(ctypes.byref(p), None) == _lib.RA_ERR_INVALID
     assert lib.ra_decode_fwd(None, None) == _lib.RA_ERR_INVALID
     assert lib.ra_decode_workspace_bytes(16, 1024, 32, 128, 4) == 16 * 32 * 4 * 130 * 4
+    # the entry point that allocates nothing refuses what its built-in buffer cannot hold, before any device call
+    assert lib.ra_decode_fwd_static(None, None) == _lib.RA_ERR_INVALID
+    d = _lib.RaDecodeParams()
+    d.q = d.k = d.v = d.out = 16
+    d.dtype, d.B, d.L, d.H, d.D = _lib.RA_BF16, 1024, 512, 64, 128       # 1024 * 64 * 130 * 4 bytes > 16 MiB
+    d.mask.query_chunk_size, d.mask.key_chunk_size = 1, 512
+    assert lib.ra_decode_fwd_static(ctypes.byref(d), None) == _lib.RA_ERR_UNSUPPORTED
+    assert b"scratch" in lib.ra_last_error()
+    d.D = 96
+    assert lib.ra_decode_fwd_static(ctypes.byref(d), None) == _lib.RA_ERR_UNSUPPORTED
     # measurement hooks validate too
-    one_ = ctypes.c_void_p(16)
     assert lib.ra_attn_bwd_block_part(None, 3, None) == _lib.RA_ERR_INVALID
-    assert lib.ra_gemm_bf16_tile(one_, one_, one_, 128, 128, 64, 0, 0, 1, 0, 7, None) == _lib.RA_ERR_INVALID
+    assert lib.ra_gemm_bf16_tile(one_ := ctypes.c_void_p(16), one_, one_, 128, 128, 64, 0, 0, 1, 0, 7, None) == _lib.RA_ERR_INVALID
     # ra_keep_pack validates before touching the device
     assert lib.ra_keep_pack(None, 0, 0, 0, 1, 1, 1, 64, 64, None, None, None, None) == _lib.RA_ERR_INVALID
     one = ctypes.c_void_p(16)      # any non-null address: the shape check comes before any use
