@@ -205,6 +205,30 @@ int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t str
 int ra_attn_bwd_block(const ra_attn_bwd_params* p, ra_stream_t stream);
 
 /*
+ * One step of the ring loop for EVERY device of a ring whose devices all live on this GPU: the body of the
+ * lax.scan at ringattention_jax.py:29-51 (forward) / :65-88 (backward) as the devices of a mesh run it side by side,
+ * in one launch per kernel instead of one per device.  In step idx device d holds the K/V shard
+ * (d - idx) mod n_dev (:36, :72).  The params describe the GLOBAL arrays: Sq and Skv are the whole sequence lengths
+ * (n_dev shards of Sq / n_dev and Skv / n_dev positions, device d owning query shard d), mask.q_chunk_idx_start /
+ * k_chunk_idx_start are ignored (each device gets d * q_len / query_chunk_size and shard * kv_len / key_chunk_size,
+ * :32-33, :37), and carry_is_initial / grads_are_initial / the nullness of out, dq_out, dk_out, dv_out as "last step"
+ * markers are replaced by the per-device bits below (the output pointers must be non-null when any bit asks for
+ * them).  Results are bit-identical to the n_dev separate ra_attn_fwd_block / ra_attn_bwd_block calls.
+ * MFMA kernels only (RA_ERR_UNSUPPORTED otherwise: fall back to the per-device calls); no keep mask, no cache_idx.
+ */
+typedef struct ra_ring_step {
+  int32_t n_dev;      /* ring size, 1 .. 64 */
+  int32_t idx;        /* scan index, 0 .. n_dev - 1 */
+  uint64_t run;       /* bit d: device d runs this step; the rows of the others are left untouched */
+  uint64_t first;     /* bit d: forward, the carry of device d is initial; backward, its dq is initial */
+  uint64_t last;      /* bit d: forward, device d writes out; backward, it writes dq_out */
+  uint64_t kv_first;  /* backward, bit s: dk / dv of K/V SHARD s (held by device (s + idx) mod n_dev) are initial */
+  uint64_t kv_last;   /* backward, bit s: dk_out / dv_out of shard s are written */
+} ra_ring_step;
+int ra_attn_fwd_ring_step(const ra_attn_fwd_params* p, const ra_ring_step* ring, ra_stream_t stream);
+int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring, ra_stream_t stream);
+
+/*
  * Decode: the cache_idx path (ringattention_jax.py:31-35 with q_len == 1): one query token per
  * batch row against the whole KV cache buffer, streamed once.  Same mask semantics as above with
  * query_chunk_size == 1.  workspace: ra_decode_workspace_bytes() bytes of device memory.

@@ -63,6 +63,13 @@ class RaAttnBwdParams(C.Structure):
     ]
 
 
+class RaRingStep(C.Structure):
+    _fields_ = [
+        ("n_dev", i32), ("idx", i32), ("run", C.c_uint64), ("first", C.c_uint64), ("last", C.c_uint64),
+        ("kv_first", C.c_uint64), ("kv_last", C.c_uint64),
+    ]
+
+
 class RaDecodeParams(C.Structure):
     _fields_ = [
         ("q", vp), ("k", vp), ("v", vp), ("out", vp), ("dtype", i32),
@@ -113,6 +120,8 @@ SYMBOLS = {
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_bwd_delta": (C.c_int, [vp, vp, i32, i64, i64, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_bwd_block": (C.c_int, [C.POINTER(RaAttnBwdParams), vp]),
+    "ra_attn_fwd_ring_step": (C.c_int, [C.POINTER(RaAttnFwdParams), C.POINTER(RaRingStep), vp]),
+    "ra_attn_bwd_ring_step": (C.c_int, [C.POINTER(RaAttnBwdParams), C.POINTER(RaRingStep), vp]),
     "ra_decode_workspace_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
     "ra_decode_fwd": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
     "ra_decode_fwd_static": (C.c_int, [C.POINTER(RaDecodeParams), vp]),

@@ -18,8 +18,8 @@ void set_error(const char* fmt, ...) {
 
 int attn_fwd_generic(const ra_attn_fwd_params* p, hipStream_t s);
 int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s);
-int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s);     // RA_ERR_UNSUPPORTED if shape does not fit
-int attn_bwd_mfma(const ra_attn_bwd_params* p, int parts, hipStream_t s);   // parts: RA_BWD_PART_* bits
+int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* ring, hipStream_t s);   // ring: nullable
+int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* ring, int parts, hipStream_t s);   // parts: RA_BWD_PART_* bits
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p);
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p);
 int carry_init(float*, int64_t, int64_t, float*, float*, int64_t, int64_t, int, int, int, int, hipStream_t);
@@ -215,7 +215,7 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   if (int rc = check_mask(p->mask, p->Sq, p->Skv, "attn_fwd_block")) return rc;
   hipStream_t s = (hipStream_t)stream;
   if (p->impl == RA_IMPL_GENERIC) return attn_fwd_generic(p, s);
-  if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, s);
+  if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, nullptr, s);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
              "attn_fwd_block: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128");
   return attn_fwd_generic(p, s);
@@ -262,7 +262,7 @@ static int attn_bwd_block(const ra_attn_bwd_params* p, int parts, const char* wh
   if (int rc = check_mask(p->mask, p->Sq, p->Skv, who)) return rc;
   const bool whole = dq_part && dkv_part;
   if (p->impl == RA_IMPL_GENERIC && whole) return attn_bwd_generic(p, s);
-  if (p->impl != RA_IMPL_GENERIC && attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, parts, s);
+  if (p->impl != RA_IMPL_GENERIC && attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, nullptr, parts, s);
   RA_REQUIRE(whole, RA_ERR_UNSUPPORTED, "%s: one part alone is launched by the MFMA kernels only, which do not take "
              "this call (impl, dtype, head size or chunk sizes)", who);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
@@ -278,6 +278,66 @@ int ra_attn_bwd_block_part(const ra_attn_bwd_params* p, int32_t part, ra_stream_
   RA_REQUIRE(part == RA_BWD_PART_DQ || part == RA_BWD_PART_DKV, RA_ERR_INVALID,
              "attn_bwd_block_part: part must be RA_BWD_PART_DQ or RA_BWD_PART_DKV");
   return attn_bwd_block(p, part, "attn_bwd_block_part", (hipStream_t)stream);
+}
+
+// The checks the two ring-step entry points share; q_len / kv_len: one device's shard lengths
+static int check_ring(const ra_ring_step* r, const ra_mask& m, int Sq, int Skv, int impl, const char* who) {
+  RA_REQUIRE(r, RA_ERR_INVALID, "%s: null ring step", who);
+  RA_REQUIRE(r->n_dev >= 1 && r->n_dev <= 64 && r->idx >= 0 && r->idx < r->n_dev, RA_ERR_INVALID,
+             "%s: ring of %d devices, step %d", who, r->n_dev, r->idx);
+  RA_REQUIRE(Sq % r->n_dev == 0 && Skv % r->n_dev == 0, RA_ERR_INVALID,
+             "%s: sequence lengths (%d, %d) must divide by the ring size %d", who, Sq, Skv, r->n_dev);
+  const uint64_t all = r->n_dev == 64 ? ~0ULL : ((1ULL << r->n_dev) - 1ULL);
+  RA_REQUIRE(((r->run | r->first | r->last | r->kv_first | r->kv_last) & ~all) == 0, RA_ERR_INVALID,
+             "%s: bits set beyond device %d", who, r->n_dev - 1);
+  RA_REQUIRE(impl != RA_IMPL_GENERIC, RA_ERR_UNSUPPORTED, "%s: the MFMA kernels only", who);
+  RA_REQUIRE(!m.keep && !m.keep_bits_k && !m.cache_idx, RA_ERR_UNSUPPORTED,
+             "%s: no keep mask and no cache_idx in a ring-step launch", who);
+  return check_mask(m, Sq / r->n_dev, Skv / r->n_dev, who);
+}
+
+int ra_attn_fwd_ring_step(const ra_attn_fwd_params* p, const ra_ring_step* ring, ra_stream_t stream) {
+  const char* who = "attn_fwd_ring_step";
+  RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
+  RA_REQUIRE(p->q && p->k && p->v && p->denominator && p->max_score, RA_ERR_INVALID, "%s: null tensor", who);
+  RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "%s: empty shape", who);
+  RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "%s: B and H must be <= 65535", who);
+  if (int rc = check_ring(ring, p->mask, p->Sq, p->Skv, p->impl, who)) return rc;
+  // a device that neither starts its carry here nor writes out needs the numerator in both directions
+  RA_REQUIRE(p->numerator || (ring->run & ~(ring->first & ring->last)) == 0, RA_ERR_INVALID,
+             "%s: the numerator may be null only when every running device both starts and ends here", who);
+  RA_REQUIRE(p->out || (ring->run & ring->last) == 0, RA_ERR_INVALID, "%s: a device writes out but out is null", who);
+  ra_attn_fwd_params dev = *p;        // the shape one device sees: what the kernels' chunk grid has to fit
+  dev.Sq = p->Sq / ring->n_dev; dev.Skv = p->Skv / ring->n_dev;
+  RA_REQUIRE(attn_fwd_mfma_supported(&dev), RA_ERR_UNSUPPORTED,
+             "%s: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128", who);
+  return attn_fwd_mfma(p, ring, (hipStream_t)stream);
+}
+
+int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring, ra_stream_t stream) {
+  const char* who = "attn_bwd_ring_step";
+  RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
+  RA_REQUIRE(p->q && p->k && p->v && p->g && p->delta && p->denominator && p->max_score, RA_ERR_INVALID,
+             "%s: null tensor", who);
+  RA_REQUIRE((p->dk_out == nullptr) == (p->dv_out == nullptr), RA_ERR_INVALID, "%s: dk_out and dv_out go together", who);
+  RA_REQUIRE((p->dk == nullptr) == (p->dv == nullptr), RA_ERR_INVALID, "%s: dk and dv go together", who);
+  RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "%s: empty shape", who);
+  RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "%s: B and H must be <= 65535", who);
+  if (int rc = check_ring(ring, p->mask, p->Sq, p->Skv, p->impl, who)) return rc;
+  uint64_t shards = 0;                // the K/V shards that the running devices hold in this step
+  for (int d = 0; d < ring->n_dev; d++)
+    if ((ring->run >> d) & 1ULL) shards |= 1ULL << ((d - ring->idx + ring->n_dev) % ring->n_dev);
+  RA_REQUIRE(p->dq || (ring->run & ~(ring->first & ring->last)) == 0, RA_ERR_INVALID,
+             "%s: dq may be null only when every running device both starts and ends its dq here", who);
+  RA_REQUIRE(p->dk || (shards & ~(ring->kv_first & ring->kv_last)) == 0, RA_ERR_INVALID,
+             "%s: dk / dv may be null only when every shard in use both starts and ends here", who);
+  RA_REQUIRE(p->dq_out || (ring->run & ring->last) == 0, RA_ERR_INVALID, "%s: dq_out is null but a device writes it", who);
+  RA_REQUIRE(p->dk_out || (shards & ring->kv_last) == 0, RA_ERR_INVALID, "%s: dk_out is null but a shard writes it", who);
+  ra_attn_bwd_params dev = *p;
+  dev.Sq = p->Sq / ring->n_dev; dev.Skv = p->Skv / ring->n_dev;
+  RA_REQUIRE(attn_bwd_mfma_supported(&dev), RA_ERR_UNSUPPORTED,
+             "%s: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128", who);
+  return attn_bwd_mfma(p, ring, RA_BWD_PART_DQ | RA_BWD_PART_DKV, (hipStream_t)stream);
 }
 
 size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int32_t num_splits) {

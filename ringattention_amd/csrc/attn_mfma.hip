@@ -27,6 +27,13 @@ constexpr int FBN = 64;          // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// One launch for every device of a ring held on this GPU (ra_ring_step): the arrays are then the global ones and
+// a workgroup first rebinds its arguments to the device (and K/V shard) its tile belongs to.
+struct RingView {
+  int n, idx;
+  unsigned long long run, first, last, kv_first, kv_last;
+};
+
 struct FwdArgs {
   const uint16_t* q; const uint16_t* k; const uint16_t* v;
   int B, Sq, Skv, H;
@@ -38,6 +45,7 @@ struct FwdArgs {
   const int32_t* cache_idx;
   int carry_is_initial;
   uint16_t* out; int64_t out_sb, out_ss;      // nullable: last step of the device, out = num / den instead of num
+  RingView ring;                              // n == 0: one device per launch
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -163,7 +171,72 @@ struct BwdArgs {
   int dq_initial, dkv_initial;                 // the fp32 accumulator holds zeros by definition: not read
   uint16_t* dq_out; int64_t dqo_sb, dqo_ss;    // nullable: last call that adds into it, the sum goes here as bf16
   uint16_t* dk_out; uint16_t* dv_out; int64_t dkvo_sb, dkvo_ss;
+  RingView ring;                               // n == 0: one device per launch
 };
+
+// Rebinds the arguments of a query-stationary workgroup (forward, dQ) to the ring device that owns the global
+// 128-row query tile qt; false when that device does not run this ring step.
+template <typename Args>
+__device__ __forceinline__ bool ring_bind_common(Args& a, MaskView& mv, int dev, int shard) {
+  const int n = a.ring.n, q_len = a.Sq / n, kv_len = a.Skv / n;
+  a.q += (int64_t)dev * q_len * a.q_ss;
+  a.k += (int64_t)shard * kv_len * a.kv_ss;
+  a.v += (int64_t)shard * kv_len * a.kv_ss;
+  a.den += (int64_t)dev * q_len;
+  a.mx += (int64_t)dev * q_len;
+  a.Sq = q_len; a.Skv = kv_len;
+  mv.q_start = dev * (q_len / mv.qc);        // :32-33
+  mv.k_start = shard * (kv_len / mv.kc);     // :37
+  return true;
+}
+__device__ __forceinline__ bool ring_bind(FwdArgs& a, MaskView& mv, int& qt) {
+  const int n = a.ring.n, tiles_dev = (a.Sq / n) / FBM;
+  const int dev = qt / tiles_dev;
+  if (!((a.ring.run >> dev) & 1ULL)) return false;
+  const int shard = (dev - a.ring.idx + n) % n;                  // :36
+  const int64_t r0 = (int64_t)dev * (a.Sq / n);
+  if (a.num) a.num += r0 * a.num_ss;
+  a.out = ((a.ring.last >> dev) & 1ULL) ? a.out + r0 * a.out_ss : nullptr;
+  a.carry_is_initial = (int)((a.ring.first >> dev) & 1ULL);
+  ring_bind_common(a, mv, dev, shard);
+  qt -= dev * tiles_dev;
+  return true;
+}
+__device__ __forceinline__ void ring_bind_bwd_rows(BwdArgs& a, int dev, int shard) {
+  const int n = a.ring.n;
+  const int64_t r0 = (int64_t)dev * (a.Sq / n), s0 = (int64_t)shard * (a.Skv / n);
+  a.g += r0 * a.q_ss;
+  a.delta += r0;
+  if (a.dq) a.dq += r0 * a.dq_ss;
+  a.dq_out = ((a.ring.last >> dev) & 1ULL) ? a.dq_out + r0 * a.dqo_ss : nullptr;
+  a.dq_initial = (int)((a.ring.first >> dev) & 1ULL);
+  if (a.dk) { a.dk += s0 * a.dkv_ss; a.dv += s0 * a.dkv_ss; }
+  if ((a.ring.kv_last >> shard) & 1ULL) { a.dk_out += s0 * a.dkvo_ss; a.dv_out += s0 * a.dkvo_ss; }
+  else { a.dk_out = nullptr; a.dv_out = nullptr; }
+  a.dkv_initial = (int)((a.ring.kv_first >> shard) & 1ULL);
+}
+// dQ kernel: global 128-row query tile qt
+__device__ __forceinline__ bool ring_bind_q(BwdArgs& a, MaskView& mv, int& qt) {
+  const int n = a.ring.n, tiles_dev = (a.Sq / n) / FBM;
+  const int dev = qt / tiles_dev;
+  if (!((a.ring.run >> dev) & 1ULL)) return false;
+  const int shard = (dev - a.ring.idx + n) % n;
+  ring_bind_bwd_rows(a, dev, shard);
+  ring_bind_common(a, mv, dev, shard);
+  qt -= dev * tiles_dev;
+  return true;
+}
+// dK/dV kernel: global 128-key block kt; its shard is held by device (shard + idx) mod n (:72)
+__device__ __forceinline__ bool ring_bind_k(BwdArgs& a, MaskView& mv, int& kt) {
+  const int n = a.ring.n, blocks_shard = (a.Skv / n) / 128;
+  const int shard = kt / blocks_shard;
+  const int dev = (shard + a.ring.idx) % n;
+  if (!((a.ring.run >> dev) & 1ULL)) return false;
+  ring_bind_bwd_rows(a, dev, shard);
+  ring_bind_common(a, mv, dev, shard);
+  kt -= shard * blocks_shard;
+  return true;
+}
 
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void store_bf16x4(uint16_t* p, const f32x4& t) {
@@ -181,17 +254,36 @@ __device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t vo
   const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
   return uint4{v[0], v[1], v[2], v[3]};
 }
-// The rows of a gradient that a workgroup owns but has nothing to add to (rows x HD floats from acc / out, which
-// point at row 0, head h): hand the accumulator on as bf16, or set it to the zeros it holds by definition.
-__device__ __forceinline__ void pass_rows(float* acc, int64_t acc_ss, uint16_t* out, int64_t out_ss, int rows,
-                                          int initial, int tid) {
+// The 128 rows of a gradient that a workgroup owns but has nothing to add to (HD floats each, from acc / out, which
+// point at row 0, head h): hand the accumulator on as bf16, or set it to the zeros it holds by definition.  In a ring
+// step most workgroups may do nothing else (a later shard meets few of a device's documents), so this is written
+// as a copy kernel: 16 bytes per lane, a row per 32 lanes, all eight requests of a lane in flight before the first
+// store.  den (nullable, one value per row): the forward's out = numerator / denominator.
+__device__ __forceinline__ void pass_rows(const float* acc, float* acc_w, int64_t acc_ss, uint16_t* out, int64_t out_ss,
+                                          const float* den, int initial, int tid) {
   if (!out && !initial) return;
-  for (int i = tid; i < rows * (HD / 4); i += 512) {
-    const int r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
-    f32x4 t = {0.f, 0.f, 0.f, 0.f};
-    if (!initial) t = *(const f32x4*)(acc + (int64_t)r * acc_ss + c4);
-    if (out) store_bf16x4(out + (int64_t)r * out_ss + c4, t);
-    else *(f32x4*)(acc + (int64_t)r * acc_ss + c4) = t;
+  constexpr int PER = 128 * (HD / 4) / 512;
+  f32x4 t[PER];
+  float d[PER];
+#pragma unroll
+  for (int j = 0; j < PER; j++) {
+    const int i = tid + j * 512, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+    t[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    d[j] = 0.f;
+    if (!initial) {
+      t[j] = *(const f32x4*)(acc + (int64_t)r * acc_ss + c4);
+      if (den) d[j] = den[r];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < PER; j++) {
+    const int i = tid + j * 512, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+    if (den) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) t[j][e] /= d[j];               // 0 / 0 = NaN when nothing ran at all, as :52
+    }
+    if (out) store_bf16x4(out + (int64_t)r * out_ss + c4, t[j]);
+    else *(f32x4*)(acc_w + (int64_t)r * acc_ss + c4) = t[j];
   }
 }
 
@@ -238,9 +330,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   const int per_xcd = (a.B * a.H * nkt + 7) >> 3;
   int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (wg >= a.B * a.H * nkt) return;
-  const int kt = wg % nkt;
+  int kt = wg % nkt;
   wg /= nkt;
   const int h = wg % a.H, b = wg / a.H;
+  if (a.ring.n && !ring_bind_k(a, mv, kt)) return;
   const int k0 = kt * KBN;
   const int krow = k0 + pair * 32 + lo;    // this lane's key row (local)
 
@@ -284,8 +377,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   if (qt_first >= qt_end) {                // nothing to add for these keys
     const int64_t o = (int64_t)b * a.dkv_sb + (int64_t)k0 * a.dkv_ss + (int64_t)h * HD;
     const int64_t oo = (int64_t)b * a.dkvo_sb + (int64_t)k0 * a.dkvo_ss + (int64_t)h * HD;
-    pass_rows(a.dk ? a.dk + o : nullptr, a.dkv_ss, a.dk_out ? a.dk_out + oo : nullptr, a.dkvo_ss, KBN, a.dkv_initial, tid);
-    pass_rows(a.dv ? a.dv + o : nullptr, a.dkv_ss, a.dv_out ? a.dv_out + oo : nullptr, a.dkvo_ss, KBN, a.dkv_initial, tid);
+    pass_rows(a.dk ? a.dk + o : nullptr, a.dk ? a.dk + o : nullptr, a.dkv_ss, a.dk_out ? a.dk_out + oo : nullptr, a.dkvo_ss,
+              nullptr, a.dkv_initial, tid);
+    pass_rows(a.dv ? a.dv + o : nullptr, a.dv ? a.dv + o : nullptr, a.dkv_ss, a.dv_out ? a.dv_out + oo : nullptr, a.dkvo_ss,
+              nullptr, a.dkv_initial, tid);
     return;
   }
   const int ntq = qt_end - qt_first;       // query tiles of 64 rows
@@ -681,9 +776,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   const int per_xcd = (a.B * a.H * nqt + 7) >> 3;
   int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (wg >= a.B * a.H * nqt) return;
-  const int qt = nqt - 1 - (wg % nqt);     // latest query tiles (most keys under causal) first
+  int qt = nqt - 1 - (wg % nqt);           // latest query tiles (most keys under causal) first
   wg /= nqt;
   const int h = wg % a.H, b = wg / a.H;
+  if (a.ring.n && !ring_bind_q(a, mv, qt)) return;
   const int q0 = qt * FBM;
   const int qrow = q0 + pair * 32 + lo;
 
@@ -715,9 +811,10 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     ntiles = t_last - t_first;
   }
   if (ntiles == 0) {           // nothing to add to dq
-    pass_rows(a.dq ? a.dq + (int64_t)b * a.dq_sb + (int64_t)q0 * a.dq_ss + (int64_t)h * HD : nullptr, a.dq_ss,
+    float* const dq0 = a.dq ? a.dq + (int64_t)b * a.dq_sb + (int64_t)q0 * a.dq_ss + (int64_t)h * HD : nullptr;
+    pass_rows(dq0, dq0, a.dq_ss,
               a.dq_out ? a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)q0 * a.dqo_ss + (int64_t)h * HD : nullptr,
-              a.dqo_ss, FBM, a.dq_initial, tid);
+              a.dqo_ss, nullptr, a.dq_initial, tid);
     return;
   }
   const int gk0 = gk0_shard + k_base;
@@ -1126,9 +1223,10 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   const int per_xcd = (a.B * a.H * nqt + 7) >> 3;
   int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (wg >= a.B * a.H * nqt) return;
-  const int qt = nqt - 1 - (wg % nqt);     // latest query tiles (most keys under causal) first
+  int qt = nqt - 1 - (wg % nqt);           // latest query tiles (most keys under causal) first
   wg /= nqt;
   const int h = wg % a.H, b = wg / a.H;
+  if (a.ring.n && !ring_bind(a, mv, qt)) return;
   const int q0 = qt * FBM;
   const int qrow = q0 + pair * 32 + lo;
 
@@ -1161,28 +1259,12 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   }
   if (ntiles == 0) {           // no key tile runs for these rows: the carry stays as it is
     if (a.carry_is_initial || a.out) {
-      const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
-      float* np0 = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
-      uint16_t* op0 = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
-      if (role == 1) {
-        const float den0 = a.carry_is_initial ? 0.f : a.den[st0];            // 0 / 0 = NaN, as :52
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-          for (int g = 0; g < 4; g++) {
-            f32x4 t = {0.f, 0.f, 0.f, 0.f};
-            if (!a.carry_is_initial) t = *(const f32x4*)(np0 + db * 32 + g * 8);
-            if (a.out) {
-#pragma unroll
-              for (int e = 0; e < 4; e++) t[e] /= den0;
-              store_bf16x4(op0 + db * 32 + g * 8, t);
-            } else {
-              *(f32x4*)(np0 + db * 32 + g * 8) = t;
-            }
-          }
-      } else if (hi == 0 && a.carry_is_initial) {
-        a.den[st0] = 0.f; a.mx[st0] = RA_NEG_INF;
-      }
+      const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + q0;
+      float* const np0 = a.num ? a.num + (int64_t)b * a.num_sb + (int64_t)q0 * a.num_ss + (int64_t)h * HD : nullptr;
+      pass_rows(np0, np0, a.num_ss,
+                a.out ? a.out + (int64_t)b * a.out_sb + (int64_t)q0 * a.out_ss + (int64_t)h * HD : nullptr, a.out_ss,
+                a.out ? a.den + st0 : nullptr, a.carry_is_initial, tid);
+      if (a.carry_is_initial && tid < FBM) { a.den[st0 + tid] = 0.f; a.mx[st0 + tid] = RA_NEG_INF; }
     }
     return;
   }
@@ -1637,8 +1719,17 @@ bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
          (!p->out || (aligned16(p->out) && p->out_stride_s % 4 == 0 && p->out_stride_b % 4 == 0));
 }
 
-int attn_fwd_mfma(const ra_attn_fwd_params* p, hipStream_t s) {
+static RingView ring_view(const ra_ring_step* r) {
+  RingView v{};
+  if (r) { v.n = r->n_dev; v.idx = r->idx; v.run = r->run; v.first = r->first; v.last = r->last;
+           v.kv_first = r->kv_first; v.kv_last = r->kv_last; }
+  return v;
+}
+
+// r: nullable; all devices of a ring in one launch (p then describes the global arrays)
+int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* r, hipStream_t s) {
   FwdArgs a{};
+  a.ring = ring_view(r);
   a.q = (const uint16_t*)p->q; a.k = (const uint16_t*)p->k; a.v = (const uint16_t*)p->v;
   a.B = p->B; a.Sq = p->Sq; a.Skv = p->Skv; a.H = p->H;
   a.q_sb = p->q_stride_b; a.q_ss = p->q_stride_s; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s;
@@ -1679,8 +1770,9 @@ bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
                          p->dkv_out_stride_b % 4 == 0));
 }
 
-int attn_bwd_mfma(const ra_attn_bwd_params* p, int parts, hipStream_t s) {   // parts: bit 0 dq, bit 1 dk / dv
+int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* r, int parts, hipStream_t s) {   // parts: bit 0 dq, bit 1 dk / dv
   BwdArgs a{};
+  a.ring = ring_view(r);
   a.q = (const uint16_t*)p->q; a.k = (const uint16_t*)p->k; a.v = (const uint16_t*)p->v; a.g = (const uint16_t*)p->g;
   a.B = p->B; a.Sq = p->Sq; a.Skv = p->Skv; a.H = p->H;
   a.q_sb = p->q_stride_b; a.q_ss = p->q_stride_s; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s;

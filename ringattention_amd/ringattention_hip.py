@@ -14,9 +14,11 @@ Tensors are torch tensors in device memory (torch only owns memory and streams).
 arrays a ``shard_map`` caller holds, and every device's program is run in turn on the one GPU
 with the K/V shard that the ring would have delivered at each step.  No bytes move.
 """
+import collections
 import contextlib
 import ctypes
 import math
+import weakref
 
 import torch
 
@@ -109,6 +111,9 @@ def run_prefix_keys(q_chunk_global, qc, kc, cbs, k_chunk_idx_start, kv_len):
     return min(nloc * kc, kv_len)
 
 
+_SEG_CACHE = collections.OrderedDict()    # per segment_ids tensor: [weakref, int32 ids, tile ranges, host copy]
+
+
 class _Config:
     """blockwise_kwargs (ringattention_jax.py:99-100) reduced to what the kernels need."""
 
@@ -139,6 +144,11 @@ class _Config:
         # measurement hook: launch one of the two backward kernels alone (ra_attn_bwd_block_part)
         self.bwd_only = {None: 0, "dq": L.RA_BWD_PART_DQ, "dkv": L.RA_BWD_PART_DKV}[kw.get("bwd_only", None)]
         self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
+        # "step": a scan step of all virtual devices goes out as one launch per kernel when the kernels allow;
+        # "device": one launch per device and step
+        self.ring_launch = kw.get("ring_launch", "step")
+        if self.ring_launch not in ("step", "device"):
+            raise ValueError("ring_launch must be 'step' or 'device'")
         # policy / precision / prevent_cse only steer XLA rematerialisation: the kernels always recompute
         # the probabilities in the backward pass.
 
@@ -170,16 +180,32 @@ class _MaskInputs:
         if segment_ids is not None:
             if segment_ids.dim() != 2:
                 raise ValueError("segment_ids must be 2-D (B, S)")
-            s = segment_ids.detach().to(device=device, dtype=torch.int32).contiguous()
+            # the int32 copy, the per-tile id ranges and their host copy are kept per segment_ids tensor (same
+            # storage, same version counter): a later call with the tensor unchanged launches nothing for them and
+            # copies nothing to the host, so it can be captured into a HIP graph
+            key = (segment_ids.data_ptr(), segment_ids._version, tuple(segment_ids.shape), segment_ids.dtype,
+                   str(segment_ids.device), str(device))
+            hit = _SEG_CACHE.get(key)
+            if hit is not None and hit[0]() is segment_ids:
+                _SEG_CACHE.move_to_end(key)
+                self._seg_entry = hit
+            else:
+                s = segment_ids.detach().to(device=device, dtype=torch.int32).contiguous()
+                # per-64-position (min, max) ids: lets the MFMA kernels skip tiles of foreign segments
+                tiles = (s.shape[1] + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
+                mm = torch.empty((s.shape[0], tiles, 2), dtype=torch.int32, device=device)
+                L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], s.shape[1],
+                                                        mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
+                self._seg_entry = [weakref.ref(segment_ids), s, mm, None]
+                _SEG_CACHE[key] = self._seg_entry
+                while len(_SEG_CACHE) > 8:
+                    _SEG_CACHE.popitem(last=False)
+            s = self._seg_entry[1]
             self.seg = s
             self.seg_stride_b = 0 if s.shape[0] == 1 else s.stride(0)
             self.seg_len = s.shape[1]
-            # per-64-position (min, max) ids: lets the MFMA kernels skip tiles of foreign segments
             self.seg_tiles = (self.seg_len + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
-            self.seg_mm = torch.empty((s.shape[0], self.seg_tiles, 2), dtype=torch.int32, device=device)
-            L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], self.seg_len,
-                                                    self.seg_mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
-            self._seg_mm_host = None
+            self.seg_mm = self._seg_entry[2]
         self.keep = None                   # boolean mask: ring_attention_inference (set_keep) or dropout
         self.keep_strides = (0, 0, 0, 0)
         self.keep_row0 = 0
@@ -331,12 +357,12 @@ class _MaskInputs:
     def segments_meet(self, q_lo, q_hi, k_lo, k_hi):
         """False when no batch row has a segment id present both in global query positions
         [q_lo, q_hi) and in global key positions [k_lo, k_hi) (conservative: id ranges are compared).
-        Costs one device->host copy of the per-tile ranges per call of ring_attention."""
+        Costs one device->host copy of the per-tile ranges per segment_ids tensor (kept while it is unchanged)."""
         if self.seg_mm is None:
             return True
-        if self._seg_mm_host is None:
-            self._seg_mm_host = self.seg_mm.cpu().numpy()
-        mm = self._seg_mm_host
+        if self._seg_entry[3] is None:
+            self._seg_entry[3] = self.seg_mm.cpu().numpy()
+        mm = self._seg_entry[3]
         t = L.RA_SEG_TILE
         qs = mm[:, q_lo // t:max(q_lo // t + 1, -(-q_hi // t))]
         ks = mm[:, k_lo // t:max(k_lo // t + 1, -(-k_hi // t))]
@@ -584,18 +610,29 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     # the numerator carry (:22) only exists between the steps of a device: its first step starts it (nothing is
     # read), its last step writes out = numerator / denominator (:52) instead
     num = None
-    if any(len(steps) != 1 for steps in plan):
+    if any(len(steps) > 1 for steps in plan.values()):
         num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
-    for dev, steps in enumerate(plan):
-        qs = slice(dev * q_len, (dev + 1) * q_len)
-        carry = (num[:, qs] if num is not None else None, den[:, :, qs], mx[:, :, qs])
-        for j, (q_start, k_blk, k_start) in enumerate(steps):
+    whole = _ring_step_launches(cfg, mi, n)
+    for idx in range(n):                    # the scan of :29-51; all devices run a step side by side
+        devs = [dev for dev in range(n) if idx in plan[dev]]
+        if whole and devs:
+            whole = _fwd_ring_step(q, k, v, (num, den, mx), out, cfg, mi, n, idx, plan, devs)
+            if whole:
+                continue
+        for dev in devs:
+            qs = slice(dev * q_len, (dev + 1) * q_len)
+            q_start, k_blk, k_start = plan[dev][idx]
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+            carry = (num[:, qs] if num is not None else None, den[:, :, qs], mx[:, :, qs])
             _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, q_start, k_start, None, None,
                                      cfg.cbs, cfg.qc, cfg.kc, _mask_inputs=mi, _cfg=cfg,
-                                     _carry_is_initial=j == 0, cache_idx=cache_idx,
-                                     _out=out[:, qs] if j == len(steps) - 1 else None)
-        if not steps:                       # no tile runs for this device: 0 / 0
+                                     _carry_is_initial=idx == min(plan[dev]), cache_idx=cache_idx,
+                                     _out=out[:, qs] if idx == max(plan[dev]) else None)
+    for dev in range(n):
+        if not plan[dev]:                   # no tile runs for this device: 0 / 0
+            qs = slice(dev * q_len, (dev + 1) * q_len)
+            carry = (num[:, qs] if num is not None else torch.empty((B, q_len, H, D), dtype=torch.float32,
+                                                                    device=q.device), den[:, :, qs], mx[:, :, qs])
             _carry_init(*carry)
             _finalize(carry[0], carry[1], out[:, qs])
     del num
@@ -603,19 +640,71 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
 
 
 def _ring_plan(cfg, mi, n, q_len, kv_len):
-    """For every device of the virtual ring the steps that run, in ring order (:50-51): (q_chunk_idx_start,
-    index of the K/V shard that has arrived (:36), k_chunk_idx_start (:37))."""
-    plan = []
+    """For every device of the virtual ring the scan steps that run: {dev: {idx: (q_chunk_idx_start, index of the
+    K/V shard that has arrived (:36), k_chunk_idx_start (:37))}}, idx ascending (:50-51)."""
+    plan = {}
     for dev in range(n):
-        steps = []
+        steps = {}
         for idx in range(n):
             k_blk = (dev - idx) % n
             k_start = k_blk * (kv_len // cfg.kc)
             q_start = _q_start(cfg, mi, dev, q_len)
             if _step_runs(cfg, mi, q_start, q_len, k_start, kv_len):
-                steps.append((q_start, k_blk, k_start))
-        plan.append(steps)
+                steps[idx] = (q_start, k_blk, k_start)
+        plan[dev] = steps
     return plan
+
+
+def _ring_step_launches(cfg, mi, n):
+    """Whether a scan step of all devices may go out as one launch per kernel (ra_attn_*_ring_step): a ring of 2 to
+    64 devices, the MFMA kernels, no boolean / dropout mask, no cache_idx.  blockwise_kwargs["ring_launch"] =
+    "device" keeps one launch per device."""
+    return (1 < n <= 64 and cfg.ring_launch != "device" and cfg.impl != L.RA_IMPL_GENERIC and cfg.pdrop == 0.0
+            and mi.keep is None and mi.keep_packed is None and mi.cache_idx_host is None and mi.cache_idx_dev is None
+            and not cfg.bwd_only)
+
+
+def _ring_bits(devs):
+    bits = 0
+    for d in devs:
+        bits |= 1 << d
+    return bits
+
+
+def _fwd_ring_step(q, k, v, carry, out, cfg, mi, n, idx, plan, devs):
+    """Scan step idx of every device in `devs` as one launch; False when the shape does not fit the MFMA kernels
+    (nothing was launched then)."""
+    num, den, mx = carry
+    B, q_total, H, D = q.shape
+    p = L.RaAttnFwdParams()
+    p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    p.dtype = _ra_dtype(q)
+    p.B, p.Sq, p.Skv, p.H, p.D = B, q_total, k.shape[1], H, D
+    p.q_stride_b, p.q_stride_s = _rows(q)
+    p.kv_stride_b, p.kv_stride_s = _rows(k)
+    if _rows(v) != _rows(k):
+        raise ValueError("k and v must share strides")
+    if num is not None:
+        p.numerator = num.data_ptr()
+        p.num_stride_b, p.num_stride_s = _rows(num)
+    else:
+        p.num_stride_b, p.num_stride_s = q_total * H * D, H * D
+    p.out = out.data_ptr()
+    p.out_stride_b, p.out_stride_s = _rows(out)
+    p.denominator, p.max_score = den.data_ptr(), mx.data_ptr()
+    p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
+    p.mask = mi.fill(cfg, 0, 0, cfg.skip_masked_tiles)
+    p.impl = cfg.impl
+    r = L.RaRingStep()
+    r.n_dev, r.idx = n, idx
+    r.run = _ring_bits(devs)
+    r.first = _ring_bits(d for d in devs if idx == min(plan[d]))
+    r.last = _ring_bits(d for d in devs if idx == max(plan[d]))
+    rc = L.load().ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), _stream())
+    if rc == L.RA_ERR_UNSUPPORTED and cfg.impl == L.RA_IMPL_AUTO:
+        return False
+    L.check(rc, "ra_attn_fwd_ring_step")
+    return True
 
 
 def _ring_attention_bwd(res, g):
@@ -628,34 +717,36 @@ def _ring_attention_bwd(res, g):
     g = g.to(q.dtype).contiguous()
     delta = _bwd_delta(g, out)
     plan = _ring_plan(cfg, mi, n, q_len, kv_len)
-    # the calls that add into each K/V shard's dk, dv, in program order (they ride with the shard, :85-86)
-    last_for_shard, count_for_shard = {}, {}
-    for dev, steps in enumerate(plan):
-        for j, (_, k_blk, _) in enumerate(steps):
-            last_for_shard[k_blk] = (dev, j)
-            count_for_shard[k_blk] = count_for_shard.get(k_blk, 0) + 1
+    # the scan steps that add into each K/V shard's dk, dv (they ride with the shard, :85-86): shard s is with
+    # device (s + idx) mod n in step idx
+    shard_steps = {s: [idx for idx in range(n) if idx in plan[(s + idx) % n]] for s in range(n)}
     # fp32 accumulators (:61-63) exist only where more than one call adds into a gradient: the first call starts
     # them (nothing is read, so no zero fill), the last one writes the sum in the primal dtype (:89)
     dq_out = torch.empty((B, q_total, H, D), dtype=q.dtype, device=q.device)
     dk_out = torch.empty((B, kv_total, H, D), dtype=k.dtype, device=q.device)
     dv_out = torch.empty((B, kv_total, H, D), dtype=v.dtype, device=q.device)
     dq = dk = dv = None
-    if any(len(steps) > 1 for steps in plan):
+    if any(len(steps) > 1 for steps in plan.values()):
         dq = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
-    if any(c > 1 for c in count_for_shard.values()):
+    if any(len(steps) > 1 for steps in shard_steps.values()):
         dk = torch.empty((B, kv_total, H, D), dtype=torch.float32, device=q.device)
         dv = torch.empty((B, kv_total, H, D), dtype=torch.float32, device=q.device)
-    seen_shard = set()
-    for dev, steps in enumerate(plan):
-        qs = slice(dev * q_len, (dev + 1) * q_len)
-        if not steps:
-            dq_out[:, qs].zero_()
-        for j, (q_start, k_blk, k_start) in enumerate(steps):
+    whole = _ring_step_launches(cfg, mi, n)
+    for idx in range(n):                    # the scan of :65-88
+        devs = [dev for dev in range(n) if idx in plan[dev]]
+        if whole and devs:
+            whole = _bwd_ring_step(q, k, v, g, delta, den, mx, (dq, dk, dv), (dq_out, dk_out, dv_out), cfg, mi, n,
+                                   idx, plan, shard_steps, devs)
+            if whole:
+                continue
+        for dev in devs:
+            qs = slice(dev * q_len, (dev + 1) * q_len)
+            q_start, k_blk, k_start = plan[dev][idx]
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
-            initial = (L.RA_GRAD_INIT_DQ if j == 0 else 0) | (L.RA_GRAD_INIT_DKV if k_blk not in seen_shard else 0)
-            seen_shard.add(k_blk)
-            last_dq = j == len(steps) - 1
-            last_dkv = last_for_shard[k_blk] == (dev, j)
+            initial = (L.RA_GRAD_INIT_DQ if idx == min(plan[dev]) else 0) | (
+                L.RA_GRAD_INIT_DKV if idx == shard_steps[k_blk][0] else 0)
+            last_dq = idx == max(plan[dev])
+            last_dkv = idx == shard_steps[k_blk][-1]
             _blockwise_attention_bwd(q[:, qs], k[:, ks], v[:, ks], g[:, qs],
                                      (dq[:, qs] if dq is not None else None, dk[:, ks] if dk is not None else None,
                                       dv[:, ks] if dv is not None else None, out[:, qs], den[:, :, qs], mx[:, :, qs]),
@@ -663,12 +754,65 @@ def _ring_attention_bwd(res, g):
                                      _mask_inputs=mi, _cfg=cfg, _delta=delta[:, :, qs], _grads_initial=initial,
                                      _dq_out=dq_out[:, qs] if last_dq else None,
                                      _dkv_out=(dk_out[:, ks], dv_out[:, ks]) if last_dkv else None)
-    for k_blk in range(n):
-        if k_blk not in seen_shard:
-            ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
+    for dev in range(n):
+        if not plan[dev]:
+            dq_out[:, dev * q_len:(dev + 1) * q_len].zero_()
+    for s in range(n):
+        if not shard_steps[s]:
+            ks = slice(s * kv_len, (s + 1) * kv_len)
             dk_out[:, ks].zero_()
             dv_out[:, ks].zero_()
     return dq_out, dk_out, dv_out
+
+
+def _bwd_ring_step(q, k, v, g, delta, den, mx, acc, outs, cfg, mi, n, idx, plan, shard_steps, devs):
+    """Scan step idx of the backward pass of every device in `devs` as one launch per kernel; False when the shape
+    does not fit the MFMA kernels (nothing was launched then)."""
+    dq, dk, dv = acc
+    dq_out, dk_out, dv_out = outs
+    B, q_total, H, D = q.shape
+    kv_total = k.shape[1]
+    if _rows(g) != _rows(q):
+        raise ValueError("g must share q's strides")
+    p = L.RaAttnBwdParams()
+    p.q, p.k, p.v, p.g = q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr()
+    p.dtype = _ra_dtype(q)
+    p.B, p.Sq, p.Skv, p.H, p.D = B, q_total, kv_total, H, D
+    p.q_stride_b, p.q_stride_s = _rows(q)
+    p.kv_stride_b, p.kv_stride_s = _rows(k)
+    p.delta, p.denominator, p.max_score = delta.data_ptr(), den.data_ptr(), mx.data_ptr()
+    if not (delta.stride() == den.stride() == mx.stride()):
+        raise ValueError("delta / denominator / max_score must share strides")
+    p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
+    if dq is not None:
+        p.dq = dq.data_ptr()
+        p.dq_stride_b, p.dq_stride_s = _rows(dq)
+    else:
+        p.dq_stride_b, p.dq_stride_s = q_total * H * D, H * D
+    if dk is not None:
+        p.dk, p.dv = dk.data_ptr(), dv.data_ptr()
+        p.dkv_stride_b, p.dkv_stride_s = _rows(dk)
+    else:
+        p.dkv_stride_b, p.dkv_stride_s = kv_total * H * D, H * D
+    p.dq_out = dq_out.data_ptr()
+    p.dq_out_stride_b, p.dq_out_stride_s = _rows(dq_out)
+    p.dk_out, p.dv_out = dk_out.data_ptr(), dv_out.data_ptr()
+    p.dkv_out_stride_b, p.dkv_out_stride_s = _rows(dk_out)
+    p.mask = mi.fill(cfg, 0, 0, cfg.skip_masked_tiles)
+    p.impl = cfg.impl
+    r = L.RaRingStep()
+    r.n_dev, r.idx = n, idx
+    r.run = _ring_bits(devs)
+    r.first = _ring_bits(d for d in devs if idx == min(plan[d]))
+    r.last = _ring_bits(d for d in devs if idx == max(plan[d]))
+    shards = [(d - idx) % n for d in devs]
+    r.kv_first = _ring_bits(s for s in shards if idx == shard_steps[s][0])
+    r.kv_last = _ring_bits(s for s in shards if idx == shard_steps[s][-1])
+    rc = L.load().ra_attn_bwd_ring_step(ctypes.byref(p), ctypes.byref(r), _stream())
+    if rc == L.RA_ERR_UNSUPPORTED and cfg.impl == L.RA_IMPL_AUTO:
+        return False
+    L.check(rc, "ra_attn_bwd_ring_step")
+    return True
 
 
 class _RingAttentionFn(torch.autograd.Function):

@@ -350,3 +350,47 @@ def test_first_and_last_step_modes_reject_missing_buffers():
     with pytest.raises(ValueError):       # dq missing although it is not the first call
         ra._blockwise_attention_bwd(q, k, v, do, (None, torch.zeros_like(q), torch.zeros_like(q), out, den, mx), 0, 0,
                                     None, None, _delta=delta, _dq_out=torch.empty_like(q), **kw)
+
+
+# --- a scan step of all virtual devices as one launch per kernel (ra_attn_*_ring_step) against one launch per device
+@pytest.mark.parametrize("n,cbs,use_seg,use_bias", [(2, 1, False, False), (4, 1, True, True), (8, 1, True, False),
+                                                    (4, None, False, True), (8, 256, True, True)])
+def test_ring_step_launch_equals_device_launches_bitwise(n, cbs, use_seg, use_bias):
+    B, S, H, D = 2, 4096, 2, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=n, scale=1.0)
+    g = torch.Generator().manual_seed(n + 50)
+    bias = torch.randn(B, H, 1, S, generator=g) if use_bias else None
+    seg = packed_segment_ids(B, S, 700, seed=n + 3) if use_seg else None
+    res = {}
+    for mode in ("step", "device"):
+        kw = kwargs(128, 128, cbs, dtype=torch.float32, impl="mfma", ring_launch=mode)
+        out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+        res[mode] = (out,) + grads
+    for name, a, b in zip(("out", "dq", "dk", "dv"), res["step"], res["device"]):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16)), name
+    # and the oracle, so that both are right and not only equal
+    kw = kwargs(128, 128, cbs, dtype=torch.float32)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    for name, a, b in zip(("out", "dq", "dk", "dv"), res["step"], (ref_out,) + tuple(ref_grads)):
+        assert_close(a, b, torch.bfloat16, name)
+
+
+def test_ring_step_entry_points_refuse_what_they_do_not_take():
+    import ctypes
+    from ringattention_amd import _lib as L
+    lib = L.load()
+    p, r = L.RaAttnFwdParams(), L.RaRingStep()
+    r.n_dev, r.idx = 4, 4
+    x = torch.zeros(1, 512, 1, 128, dtype=torch.bfloat16, device=DEV)
+    st = torch.zeros(1, 1, 512, device=DEV)
+    p.q = p.k = p.v = x.data_ptr()
+    p.denominator = p.max_score = st.data_ptr()
+    p.B, p.Sq, p.Skv, p.H, p.D, p.dtype = 1, 512, 512, 1, 128, L.RA_BF16
+    p.mask.query_chunk_size = p.mask.key_chunk_size = 128
+    assert lib.ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), None) == L.RA_ERR_INVALID    # idx == n_dev
+    r.idx, r.run = 0, 1 << 5
+    assert lib.ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), None) == L.RA_ERR_INVALID    # bit beyond the ring
+    r.run = 1
+    assert lib.ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), None) == L.RA_ERR_INVALID    # numerator needed
+    p.impl = L.RA_IMPL_GENERIC
+    assert lib.ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), None) == L.RA_ERR_UNSUPPORTED

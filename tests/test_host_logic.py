@@ -31,17 +31,17 @@ def test_struct_sizes_match_a_c_compiler(tmp_path):
     import ctypes
     import subprocess
     src = tmp_path / "sz.c"
-    src.write_text('#include <stdio.h>\n#include "%s"\nint main(){printf("%%zu %%zu %%zu %%zu %%zu %%zu %%zu\\n",'
+    src.write_text('#include <stdio.h>\n#include "%s"\nint main(){printf("%%zu %%zu %%zu %%zu %%zu %%zu %%zu %%zu\\n",'
                    'sizeof(ra_mask),sizeof(ra_attn_fwd_params),sizeof(ra_attn_bwd_params),'
                    'sizeof(ra_decode_params),sizeof(ra_swiglu_params),sizeof(ra_rope_append_params),'
-                   'sizeof(ra_rmsnorm_params));return 0;}\n'
+                   'sizeof(ra_rmsnorm_params),sizeof(ra_ring_step));return 0;}\n'
                    % os.path.join(ROOT, "include", "ringattn_hip.h"))
     exe = tmp_path / "sz"
     subprocess.check_call(["gcc", str(src), "-o", str(exe)])
     sizes = [int(x) for x in subprocess.check_output([str(exe)]).split()]
     mine = [ctypes.sizeof(c) for c in (_lib.RaMask, _lib.RaAttnFwdParams, _lib.RaAttnBwdParams,
                                        _lib.RaDecodeParams, _lib.RaSwigluParams, _lib.RaRopeAppendParams,
-                                       _lib.RaRmsnormParams)]
+                                       _lib.RaRmsnormParams, _lib.RaRingStep)]
     assert sizes == mine
 
 
