@@ -109,6 +109,8 @@ def bench_attention(args, ring, dropout=False):
     from ringattention_amd import ringattention_hip as rh
     dev = "cuda:0"
     D, H, B = 128, 32, 1
+    if args.head_dim:
+        D, H = args.head_dim, 32 * 128 // args.head_dim      # the same model width
     if ring:
         S, n, name = 131072, 8, "ring131k"
     else:
@@ -549,6 +551,8 @@ def main():
     ap.add_argument("--workload", default=None, choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
                                                               "dropout32k"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
+    ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
+                    help="attention workloads: head size (the number of heads follows, H * D = 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--ffn-policy", default="nothing_saveable", choices=["nothing_saveable", "save_preactivations"],
                     help="ffn workload: what blockwise_feedforward keeps for the backward pass (default: the "

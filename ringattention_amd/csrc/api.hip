@@ -217,7 +217,7 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   if (p->impl == RA_IMPL_GENERIC) return attn_fwd_generic(p, s);
   if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, nullptr, s);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
-             "attn_fwd_block: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128");
+             "attn_fwd_block: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128");
   return attn_fwd_generic(p, s);
 }
 
@@ -266,7 +266,7 @@ static int attn_bwd_block(const ra_attn_bwd_params* p, int parts, const char* wh
   RA_REQUIRE(whole, RA_ERR_UNSUPPORTED, "%s: one part alone is launched by the MFMA kernels only, which do not take "
              "this call (impl, dtype, head size or chunk sizes)", who);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
-             "%s: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128", who);
+             "%s: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128", who);
   return attn_bwd_generic(p, s);
 }
 
@@ -310,7 +310,7 @@ int ra_attn_fwd_ring_step(const ra_attn_fwd_params* p, const ra_ring_step* ring,
   ra_attn_fwd_params dev = *p;        // the shape one device sees: what the kernels' chunk grid has to fit
   dev.Sq = p->Sq / ring->n_dev; dev.Skv = p->Skv / ring->n_dev;
   RA_REQUIRE(attn_fwd_mfma_supported(&dev), RA_ERR_UNSUPPORTED,
-             "%s: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128", who);
+             "%s: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128", who);
   return attn_fwd_mfma(p, ring, (hipStream_t)stream);
 }
 
@@ -336,7 +336,7 @@ int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring,
   ra_attn_bwd_params dev = *p;
   dev.Sq = p->Sq / ring->n_dev; dev.Skv = p->Skv / ring->n_dev;
   RA_REQUIRE(attn_bwd_mfma_supported(&dev), RA_ERR_UNSUPPORTED,
-             "%s: MFMA kernels need bf16, D=128, chunk sizes that are multiples of 128", who);
+             "%s: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128", who);
   return attn_bwd_mfma(p, ring, RA_BWD_PART_DQ | RA_BWD_PART_DKV, (hipStream_t)stream);
 }
 

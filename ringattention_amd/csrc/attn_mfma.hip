@@ -1,4 +1,4 @@
-// bf16 MFMA blockwise attention for gfx950, head size 128: forward, dK/dV and dQ of one ring step
+// bf16 MFMA blockwise attention for gfx950, head size 128 or 64 (a template parameter): forward, dK/dV and dQ of one ring step
 // (carry in / carry out; ringattention_jax.py:130-145 forward, :147-209 backward).
 //
 // All three kernels share one structure.  A workgroup of 8 wavefronts owns 128 rows of one
@@ -21,7 +21,6 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int HD = 128;          // head size
 constexpr int FBM = 128;         // query rows per workgroup
 constexpr int FBN = 64;          // keys per tile
 constexpr float kLog2e = 1.4426950408889634f;
@@ -69,8 +68,11 @@ __device__ __forceinline__ float max_from_log2(float m2, float mask_min) { retur
 // of row r is stored at slot c ^ swz(r): sixteen consecutive rows then put a given logical slot in
 // sixteen different bank groups (conflict-free 16-byte row reads), and four consecutive rows put four
 // adjacent slots in sixteen different bank groups (conflict-free 4-row transpose reads).
-__device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
-constexpr int TROW = HD;          // elements per LDS tile row
+// With head size 64 a row is 128 bytes (8 slots, two rows per 256 bytes): rows of equal parity two apart swap the
+// halves of the slot range and rows four apart shift by one slot, which serves the same two read shapes.
+template <int HD> __device__ __forceinline__ int swz(int r) {
+  return HD == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+}
 
 // Hull [first, last+1) of the 64-position tiles, among the n tiles starting at global tile gt0, whose
 // segment-id range meets [lo, hi] (ids from ra_segment_tile_ranges).  Conservative: a tile outside the
@@ -259,6 +261,7 @@ __device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t vo
 // step most workgroups may do nothing else (a later shard meets few of a device's documents), so this is written
 // as a copy kernel: 16 bytes per lane, a row per 32 lanes, all eight requests of a lane in flight before the first
 // store.  den (nullable, one value per row): the forward's out = numerator / denominator.
+template <int HD>
 __device__ __forceinline__ void pass_rows(const float* acc, float* acc_w, int64_t acc_ss, uint16_t* out, int64_t out_ss,
                                           const float* den, int initial, int tid) {
   if (!out && !initial) return;
@@ -303,10 +306,13 @@ __device__ __forceinline__ void pass_rows(const float* acc, float* acc_w, int64_
 // registers loaded two steps earlier.
 constexpr int WS_PSTR = 40;                 // P / dS row stride in elements (conflict-free 16-byte reads)
 constexpr int WS_PD = 32 * WS_PSTR;         // one 32 x 32 block
-constexpr int WS_TILE = KBM * TROW;
 
-template <bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
+template <int HD, bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HD: head size, 64 or 128; HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
 __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
+  // head size: elements per LDS tile row, a 64-row tile, contraction steps of 16 (per quarter of a block's products),
+  // output blocks of 32, 16-byte chunks per row, rows per staging pass of 256 threads, passes per tile
+  constexpr int TROW = HD, WS_TILE = 64 * HD, NK = HD / 16, KPG = HD / 64, NDB = HD / 32, CH = HD / 8;
+  constexpr int SRP = 256 / CH, SNP = 64 / SRP;
   // Q tiles then dO tiles in one array: a dO address is the Q address plus a constant (an immediate offset)
   __shared__ __attribute__((aligned(16))) uint16_t QGs[6 * WS_TILE];
   uint16_t* const Qs = QGs;
@@ -377,9 +383,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   if (qt_first >= qt_end) {                // nothing to add for these keys
     const int64_t o = (int64_t)b * a.dkv_sb + (int64_t)k0 * a.dkv_ss + (int64_t)h * HD;
     const int64_t oo = (int64_t)b * a.dkvo_sb + (int64_t)k0 * a.dkvo_ss + (int64_t)h * HD;
-    pass_rows(a.dk ? a.dk + o : nullptr, a.dk ? a.dk + o : nullptr, a.dkv_ss, a.dk_out ? a.dk_out + oo : nullptr, a.dkvo_ss,
+    pass_rows<HD>(a.dk ? a.dk + o : nullptr, a.dk ? a.dk + o : nullptr, a.dkv_ss, a.dk_out ? a.dk_out + oo : nullptr, a.dkvo_ss,
               nullptr, a.dkv_initial, tid);
-    pass_rows(a.dv ? a.dv + o : nullptr, a.dv ? a.dv + o : nullptr, a.dkv_ss, a.dv_out ? a.dv_out + oo : nullptr, a.dkvo_ss,
+    pass_rows<HD>(a.dv ? a.dv + o : nullptr, a.dv ? a.dv + o : nullptr, a.dkv_ss, a.dv_out ? a.dv_out + oo : nullptr, a.dkvo_ss,
               nullptr, a.dkv_initial, tid);
     return;
   }
@@ -390,15 +396,15 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   const float kMask2 = mv.mask_min;
 
   // ---- staging of the Q / dO tiles through registers: producers bring Q, consumers dO and the statistics
-  const int srow = (tid & 255) >> 4, schunk = tid & 15;
-  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const int srow = (tid & 255) / CH, schunk = tid & (CH - 1);
+  const int s_off = srow * TROW + ((schunk ^ swz<HD>(srow)) << 3);
   // a tile is read through a buffer descriptor at its first row (scalar registers) with one 32-bit byte offset per
   // lane: half the address data of 64-bit pointers per lane, and two registers less
   const uint16_t* sg = (role == 0 ? a.q : a.g) + (int64_t)b * a.q_sb + (int64_t)h * HD + (int64_t)(qt_first * KBM) * a.q_ss;
   const uint32_t sg_lane = 2u * (uint32_t)(schunk * 8 + srow * (int)a.q_ss);
-  const uint32_t row16b = 2u * 16u * (uint32_t)a.q_ss;
+  const uint32_t row16b = 2u * SRP * (uint32_t)a.q_ss;        // one staging pass further
   uint16_t* sl = (role == 0 ? Qs : Gs) + s_off;
-  uint4 sr0, sr1, sr2, sr3;
+  uint4 sr0, sr1, sr2 = {}, sr3 = {};
   float r_m = 0.f, r_den = 1.f, r_delta = 0.f;
   int r_seg = 0;
   // query chunk index and offset inside the chunk of the first row of the next tile to request (tiles are requested
@@ -410,7 +416,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     const int t_ = min((T), ntq - 1);                                                                   \
     const __amdgpu_buffer_rsrc_t rs_ = tile_rsrc(sg + (int64_t)t_ * KBM * a.q_ss);                      \
     sr0 = ld_buf(rs_, sg_lane, 0); sr1 = ld_buf(rs_, sg_lane, row16b);                                  \
-    sr2 = ld_buf(rs_, sg_lane, 2 * row16b); sr3 = ld_buf(rs_, sg_lane, 3 * row16b);                     \
+    if (SNP == 4) { sr2 = ld_buf(rs_, sg_lane, 2 * row16b); sr3 = ld_buf(rs_, sg_lane, 3 * row16b); }   \
     if (tid >= 256 && tid < 256 + KBM) {                                                                \
       const int row_ = (qt_first + t_) * KBM + tid - 256;                                               \
       const int64_t st_ = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + row_;                           \
@@ -425,8 +431,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #define RA_WS_STORE(BUF)                                                                                \
   {                                                                                                     \
     uint16_t* d_ = sl + (BUF) * WS_TILE;                                                                \
-    *(uint4*)(d_) = sr0; *(uint4*)(d_ + 16 * TROW) = sr1;                                               \
-    *(uint4*)(d_ + 32 * TROW) = sr2; *(uint4*)(d_ + 48 * TROW) = sr3;                                   \
+    *(uint4*)(d_) = sr0; *(uint4*)(d_ + SRP * TROW) = sr1;                                              \
+    if (SNP == 4) { *(uint4*)(d_ + 2 * SRP * TROW) = sr2; *(uint4*)(d_ + 3 * SRP * TROW) = sr3; }       \
     if (tid >= 256 && tid < 256 + KBM) {                                                                \
       const float m2_ = max_to_log2(r_m, kMask2);                                                       \
       st_m2[BUF][tid - 256] = m2_; st_rden[BUF][tid - 256] = 1.f / r_den;                               \
@@ -457,15 +463,15 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       bias2 = bv * kLog2e / c;          // the S accumulators start from it
     }
     const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
-    bf16x8 kf[8], vf[8];
+    bf16x8 kf[NK], vf[NK];
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
+    for (int t = 0; t < NK; t++) {
       kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
       vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
     }
-    int n_off[8];
+    int n_off[NK];
 #pragma unroll
-    for (int t = 0; t < 8; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);
+    for (int t = 0; t < NK; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz<HD>(lo)) << 3);
     uint16_t* const pw = &Ps[pair][0][0][lo * WS_PSTR + hi * 4];
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
@@ -477,15 +483,15 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   }
     // A operands of two contraction steps (32 of the 128 head dimensions) of block BLK of buffer BUF
 #define RA_WS_AREAD(G, QA, GA, BUF, BLK)                                                                \
-  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    const uint16_t* p_ = Qs + (BUF) * WS_TILE + n_off[2 * (G) + i];                                     \
+  _Pragma("unroll") for (int i = 0; i < KPG; i++) {                                                       \
+    const uint16_t* p_ = Qs + (BUF) * WS_TILE + n_off[KPG * (G) + i];                                     \
     QA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW);                                                   \
     GA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW + 3 * WS_TILE);                                     \
   }
 #define RA_WS_AMFMA(G, QA, GA, SN, DPN)                                                                 \
-  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(QA[i], kf[2 * (G) + i], SN, 0, 0, 0);                  \
-    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(GA[i], vf[2 * (G) + i], DPN, 0, 0, 0);                \
+  _Pragma("unroll") for (int i = 0; i < KPG; i++) {                                                       \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(QA[i], kf[KPG * (G) + i], SN, 0, 0, 0);                  \
+    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(GA[i], vf[KPG * (G) + i], DPN, 0, 0, 0);                \
   }
     // eight rows (registers 4G .. 4G+3 of both halves) of P and dS, no masking: VL = lse2 of the rows
 #define RA_WS_VECTOR_PLAIN(G, SC, DPC, VL, PB)                                                          \
@@ -536,7 +542,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     // the operands of a group are requested from LDS one group ahead
 #define RA_WS_PRODUCE(SC, DPC, SN, DPN, BUF, BLK, NBUF, NBLK, PB, MASKED)                               \
   {                                                                                                     \
-    bf16x8 qa_[2][2], ga_[2][2];                                                                        \
+    bf16x8 qa_[2][KPG], ga_[2][KPG];                                                                        \
     f32x4 vl_[2];                                                                                       \
     RA_WS_AREAD(0, qa_[0], ga_[0], NBUF, NBLK);                                                         \
     if (!(MASKED)) vl_[0] = *(const f32x4*)&st_lse2[BUF][(BLK) * 32 + hi * 4];                          \
@@ -558,7 +564,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     RA_WS_INIT(s_a, dp_a, 0, 0);
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-      bf16x8 qa_[2], ga_[2];
+      bf16x8 qa_[KPG], ga_[KPG];
       RA_WS_AREAD(g, qa_, ga_, 0, 0);
       RA_WS_AMFMA(g, qa_, ga_, s_a, dp_a);
     }
@@ -639,19 +645,19 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     __syncthreads();      // step 2 ntq: the consumer's last block
   } else {
     // =========================== consumer: dV^T += dO^T P, dK^T += Q^T dS
-    f32x16 dkacc[4], dvacc[4];
+    f32x16 dkacc[NDB], dvacc[NDB];
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < NDB; db++)
 #pragma unroll
       for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
     // transpose reads with the natural contraction order: rows 8 hi + (i >> 2) (+4 for the second read)
-    int t_off[4][2];
+    int t_off[NDB][2];
     {
       const int i = lane & 15, rr = (i >> 2) + 8 * hi, c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
 #pragma unroll
-      for (int db = 0; db < 4; db++) {
-        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz(rr)) << 3) + half * 4;
-        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz(rr + 4)) << 3) + half * 4;
+      for (int db = 0; db < NDB; db++) {
+        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz<HD>(rr)) << 3) + half * 4;
+        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz<HD>(rr + 4)) << 3) + half * 4;
       }
     }
     const uint16_t* const pr = &Ps[pair][0][0][lo * WS_PSTR + hi * 8];   // B operand: key column lo, 8 query rows
@@ -662,14 +668,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #define RA_WS_CREAD(K, F, BUF, BLK)                                                                     \
   {                                                                                                     \
     const uint16_t* tp_ = (((K) & 1) ? Qs : Gs) + (BUF) * WS_TILE + ((BLK) * 32 + ((K) >> 1) * 16) * TROW; \
-    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+    _Pragma("unroll") for (int db = 0; db < NDB; db++) {                                                  \
       const s16x4 x0_ = lds_read_tr(tp_ + t_off[db][0]);                                                \
       const s16x4 x1_ = lds_read_tr(tp_ + t_off[db][1]);                                                \
       F[db] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0_, x1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
   }
 #define RA_WS_CMFMA(K, F, BOP)                                                                          \
-  _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                    \
+  _Pragma("unroll") for (int db = 0; db < NDB; db++) {                                                    \
     if ((K) & 1) dkacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, dkacc[db], 0, 0, 0);   \
     else dvacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, dvacc[db], 0, 0, 0);           \
   }
@@ -694,7 +700,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     __builtin_amdgcn_sched_barrier(0);                                                                  \
     RA_WS_CMFMA(3, fb, d1_);                                                                            \
   }
-    bf16x8 fa[4], fb[4];
+    bf16x8 fa[NDB], fb[NDB];
     int cur = 0;
     RA_WS_CREAD(0, fa, 0, 0);
     __syncthreads();      // step 0
@@ -716,7 +722,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
     const int64_t oout = (int64_t)b * a.dkvo_sb + (int64_t)krow * a.dkvo_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < NDB; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         float* pk = a.dk + ooff + db * 32 + g * 8;
@@ -756,8 +762,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #ifndef WS_DQ_VALU_PER_MFMA
 #define WS_DQ_VALU_PER_MFMA 5
 #endif
-template <bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
+template <int HD, bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HD: head size, 64 or 128; HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
 __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
+  // head size: elements per LDS tile row, a 64-row tile, contraction steps of 16 (per quarter of a block's products),
+  // output blocks of 32, 16-byte chunks per row, rows per staging pass of 256 threads, passes per tile
+  constexpr int TROW = HD, WS_TILE = 64 * HD, NK = HD / 16, KPG = HD / 64, NDB = HD / 32, CH = HD / 8;
+  constexpr int SRP = 256 / CH, SNP = 64 / SRP;
   // K tiles then V tiles in one array: a V address is the K address plus a constant (an immediate offset)
   __shared__ __attribute__((aligned(16))) uint16_t KVs[6 * WS_TILE];
   uint16_t* const Ks = KVs;
@@ -812,7 +822,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   }
   if (ntiles == 0) {           // nothing to add to dq
     float* const dq0 = a.dq ? a.dq + (int64_t)b * a.dq_sb + (int64_t)q0 * a.dq_ss + (int64_t)h * HD : nullptr;
-    pass_rows(dq0, dq0, a.dq_ss,
+    pass_rows<HD>(dq0, dq0, a.dq_ss,
               a.dq_out ? a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)q0 * a.dqo_ss + (int64_t)h * HD : nullptr,
               a.dqo_ss, nullptr, a.dq_initial, tid);
     return;
@@ -825,14 +835,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   // ---- staging of the K / V tiles through registers, by the consumer waves (which have registers and
   // issue slots to spare), in two register sets A and B: tile T lives in set T & 1 from its request until it is
   // stored to LDS two tiles (four steps) later
-  const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
-  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const int srow = (tid & 255) / CH, schunk = tid & (CH - 1), stid = tid & 255;
+  const int s_off = srow * TROW + ((schunk ^ swz<HD>(srow)) << 3);
   // a tile is read through a buffer descriptor at its first row (scalar registers) with one 32-bit byte offset per
   // lane: half the address data of 64-bit pointers per lane, and two registers less
   const int64_t sg_base = (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
   const uint32_t sg_lane = 2u * (uint32_t)(schunk * 8 + srow * (int)a.kv_ss);
-  const uint32_t row16b = 2u * 16u * (uint32_t)a.kv_ss;
-  uint4 Ak0, Ak1, Ak2, Ak3, Av0, Av1, Av2, Av3, Bk0, Bk1, Bk2, Bk3, Bv0, Bv1, Bv2, Bv3;
+  const uint32_t row16b = 2u * SRP * (uint32_t)a.kv_ss;       // one staging pass further
+  uint4 Ak0, Ak1, Ak2 = {}, Ak3 = {}, Av0, Av1, Av2 = {}, Av3 = {}, Bk0, Bk1, Bk2 = {}, Bk3 = {}, Bv0, Bv1, Bv2 = {}, Bv3 = {};
   int Aseg = 0, Bseg = 0;
   float Abias = 0.f, Bbias = 0.f;
   // key chunk index and offset inside the chunk of the first key of the next tile to request (tiles are requested
@@ -846,7 +856,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     const int t_ = min((T), ntiles - 1);                                                                \
     const __amdgpu_buffer_rsrc_t rk_ = tile_rsrc(a.k + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
     S##k0 = ld_buf(rk_, sg_lane, 0); S##k1 = ld_buf(rk_, sg_lane, row16b);                              \
-    S##k2 = ld_buf(rk_, sg_lane, 2 * row16b); S##k3 = ld_buf(rk_, sg_lane, 3 * row16b);                 \
+    if (SNP == 4) { S##k2 = ld_buf(rk_, sg_lane, 2 * row16b); S##k3 = ld_buf(rk_, sg_lane, 3 * row16b); } \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
@@ -863,13 +873,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     const int t_ = min((T), ntiles - 1);                                                                \
     const __amdgpu_buffer_rsrc_t rv_ = tile_rsrc(a.v + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
     S##v0 = ld_buf(rv_, sg_lane, 0); S##v1 = ld_buf(rv_, sg_lane, row16b);                              \
-    S##v2 = ld_buf(rv_, sg_lane, 2 * row16b); S##v3 = ld_buf(rv_, sg_lane, 3 * row16b);                 \
+    if (SNP == 4) { S##v2 = ld_buf(rv_, sg_lane, 2 * row16b); S##v3 = ld_buf(rv_, sg_lane, 3 * row16b); } \
   }
 #define RA_WS_STORE_K(S, BUF)                                                                            \
   {                                                                                                     \
     uint16_t* dk_ = Ks + (BUF) * WS_TILE + s_off;                                                       \
-    *(uint4*)(dk_) = S##k0; *(uint4*)(dk_ + 16 * TROW) = S##k1;                                         \
-    *(uint4*)(dk_ + 32 * TROW) = S##k2; *(uint4*)(dk_ + 48 * TROW) = S##k3;                             \
+    *(uint4*)(dk_) = S##k0; *(uint4*)(dk_ + SRP * TROW) = S##k1;                                        \
+    if (SNP == 4) { *(uint4*)(dk_ + 2 * SRP * TROW) = S##k2; *(uint4*)(dk_ + 3 * SRP * TROW) = S##k3; } \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       if (HAS_SEG) seg_ks[BUF][stid] = S##seg;                                                          \
       /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
@@ -879,8 +889,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #define RA_WS_STORE_V(S, BUF)                                                                            \
   {                                                                                                     \
     uint16_t* dv_ = Vs + (BUF) * WS_TILE + s_off;                                                       \
-    *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + 16 * TROW) = S##v1;                                         \
-    *(uint4*)(dv_ + 32 * TROW) = S##v2; *(uint4*)(dv_ + 48 * TROW) = S##v3;                             \
+    *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + SRP * TROW) = S##v1;                                        \
+    if (SNP == 4) { *(uint4*)(dv_ + 2 * SRP * TROW) = S##v2; *(uint4*)(dv_ + 3 * SRP * TROW) = S##v3; } \
   }
   if (role == 1) {
     RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
@@ -904,9 +914,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
     }
     const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-    bf16x8 qf[8], gf[8];
+    bf16x8 qf[NK], gf[NK];
 #pragma unroll
-    for (int t = 0; t < 8; t++) {
+    for (int t = 0; t < NK; t++) {
       qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
       gf[t] = *(const bf16x8*)(a.g + qoff + t * 16);
     }
@@ -916,9 +926,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     const float rden = 1.f / den;
     const float lse2 = m2 + __log2f(den);
     const float ndelta = -a.delta[st];
-    int n_off[8];
+    int n_off[NK];
 #pragma unroll
-    for (int t = 0; t < 8; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);
+    for (int t = 0; t < NK; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz<HD>(lo)) << 3);
     uint16_t* const dw = &Ds[pair][0][lo * WS_PSTR + hi * 4];
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
@@ -929,15 +939,15 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = b4_[e]; DPN[g * 4 + e] = ndelta; }  \
   }
 #define RA_WS_AREAD(G, KA, VA, BUF, BLK)                                                                \
-  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    const uint16_t* p_ = Ks + (BUF) * WS_TILE + n_off[2 * (G) + i];                                     \
+  _Pragma("unroll") for (int i = 0; i < KPG; i++) {                                                       \
+    const uint16_t* p_ = Ks + (BUF) * WS_TILE + n_off[KPG * (G) + i];                                     \
     KA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW);                                                   \
     VA[i] = *(const bf16x8*)(p_ + (BLK) * 32 * TROW + 3 * WS_TILE);                                     \
   }
 #define RA_WS_AMFMA(G, KA, VA, SN, DPN)                                                                 \
-  _Pragma("unroll") for (int i = 0; i < 2; i++) {                                                       \
-    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[2 * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T */ \
-    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(VA[i], gf[2 * (G) + i], DPN, 0, 0, 0); /* dP^T = V dO^T */ \
+  _Pragma("unroll") for (int i = 0; i < KPG; i++) {                                                       \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[KPG * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T */ \
+    DPN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(VA[i], gf[KPG * (G) + i], DPN, 0, 0, 0); /* dP^T = V dO^T */ \
   }
     // eight keys (registers 4G .. 4G+3 of both halves) of dS^T
 #define RA_WS_VECTOR(G, SC, DPC, BUF, BLK, PB, MASKED)                                                  \
@@ -987,8 +997,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       RA_WS_AMFMA(g, ka[g], va[g], SN, DPN);                                                            \
       RA_WS_VECTOR(g, SC, DPC, BUF, BLK, PB, MASKED);                                                   \
       /* issue order: the LDS reads, then each product followed by a share of the vector work */        \
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);                                                \
-      _Pragma("unroll") for (int i_ = 0; i_ < 4; i_++) {                                                \
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * KPG, 0);                                          \
+      _Pragma("unroll") for (int i_ = 0; i_ < 2 * KPG; i_++) {                                                \
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                              \
         __builtin_amdgcn_sched_group_barrier(0x002, WS_DQ_VALU_PER_MFMA, 0);                            \
       }                                                                                                 \
@@ -997,7 +1007,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   }
 
     f32x16 s_a, dp_a, s_b, dp_b;
-    bf16x8 ka[4][2], va[4][2];
+    bf16x8 ka[4][KPG], va[4][KPG];
     RA_WS_INIT(s_a, dp_a, 0, 0);
 #pragma unroll
     for (int g = 0; g < 4; g++) {
@@ -1100,18 +1110,18 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #undef RA_WS_PRODUCE
   } else {
     // =========================== consumer: dQ^T += K^T dS^T
-    f32x16 acc[4];
+    f32x16 acc[NDB];
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < NDB; db++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
-    int t_off[4][2];
+    int t_off[NDB][2];
     {
       const int i = lane & 15, rr = (i >> 2) + 8 * hi, c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
 #pragma unroll
-      for (int db = 0; db < 4; db++) {
-        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz(rr)) << 3) + half * 4;
-        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz(rr + 4)) << 3) + half * 4;
+      for (int db = 0; db < NDB; db++) {
+        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz<HD>(rr)) << 3) + half * 4;
+        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz<HD>(rr + 4)) << 3) + half * 4;
       }
     }
     const uint16_t* const dr = &Ds[pair][0][lo * WS_PSTR + hi * 8];   // B operand: query column lo, 8 keys
@@ -1120,14 +1130,14 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #define RA_WS_CREAD(K, F, BUF, BLK)                                                                     \
   {                                                                                                     \
     const uint16_t* tp_ = Ks + (BUF) * WS_TILE + ((BLK) * 32 + (K) * 16) * TROW;                        \
-    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+    _Pragma("unroll") for (int db = 0; db < NDB; db++) {                                                  \
       const s16x4 x0_ = lds_read_tr(tp_ + t_off[db][0]);                                                \
       const s16x4 x1_ = lds_read_tr(tp_ + t_off[db][1]);                                                \
       F[db] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0_, x1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
   }
 #define RA_WS_CMFMA(F, BOP)                                                                             \
-  _Pragma("unroll") for (int db = 0; db < 4; db++)                                                      \
+  _Pragma("unroll") for (int db = 0; db < NDB; db++)                                                      \
     acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
     // fa holds the first 16 keys of the block on entry and, on exit, those of block NBLK of buffer NBUF
 #define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
@@ -1141,7 +1151,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     __builtin_amdgcn_sched_barrier(0);                                                                  \
     RA_WS_CMFMA(fb, d1_);                                                                               \
   }
-    bf16x8 fa[4], fb[4];
+    bf16x8 fa[NDB], fb[NDB];
     int cur = 0;
     RA_WS_CREAD(0, fa, 0, 0);
     __syncthreads();      // step 0
@@ -1177,7 +1187,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
     uint16_t* dqo = a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)qrow * a.dqo_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < NDB; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         f32x4 t = {0.f, 0.f, 0.f, 0.f};
@@ -1200,8 +1210,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 // per-lane scalars: a lane owns a query column) and leaves P^T, rounded to bf16, in LDS together with the
 // factor by which the output accumulator has to shrink when the reference max moved; the consumer runs
 // O^T += V^T P^T one block of 32 keys behind.
-template <bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
+template <int HD, bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>   // HD: head size, 64 or 128; HAS_KEEP: 0 no keep mask, 1 where(keep, w, min), 2 dropout
 __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
+  // head size: elements per LDS tile row, a 64-row tile, contraction steps of 16 (per quarter of a block's products),
+  // output blocks of 32, 16-byte chunks per row, rows per staging pass of 256 threads, passes per tile
+  constexpr int TROW = HD, WS_TILE = 64 * HD, NK = HD / 16, KPG = HD / 64, NDB = HD / 32, CH = HD / 8;
+  constexpr int SRP = 256 / CH, SNP = 64 / SRP;
   // K tiles then V tiles in one array: a V address is the K address plus a constant (an immediate offset)
   __shared__ __attribute__((aligned(16))) uint16_t KVs[6 * WS_TILE];
   uint16_t* const Ks = KVs;
@@ -1261,7 +1275,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     if (a.carry_is_initial || a.out) {
       const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + q0;
       float* const np0 = a.num ? a.num + (int64_t)b * a.num_sb + (int64_t)q0 * a.num_ss + (int64_t)h * HD : nullptr;
-      pass_rows(np0, np0, a.num_ss,
+      pass_rows<HD>(np0, np0, a.num_ss,
                 a.out ? a.out + (int64_t)b * a.out_sb + (int64_t)q0 * a.out_ss + (int64_t)h * HD : nullptr, a.out_ss,
                 a.out ? a.den + st0 : nullptr, a.carry_is_initial, tid);
       if (a.carry_is_initial && tid < FBM) { a.den[st0 + tid] = 0.f; a.mx[st0 + tid] = RA_NEG_INF; }
@@ -1277,14 +1291,14 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   // issue slots to spare), in two register sets A and B: tile T lives in set T & 1 from its request until it is
   // stored to LDS two tiles (four steps, about 3.5 us) later.  With one set - a tile in flight for two steps - the
   // LDS stores waited for L2 misses often enough to cost the forward kernel 16 %.
-  const int srow = (tid & 255) >> 4, schunk = tid & 15, stid = tid & 255;
-  const int s_off = srow * TROW + ((schunk ^ swz(srow)) << 3);
+  const int srow = (tid & 255) / CH, schunk = tid & (CH - 1), stid = tid & 255;
+  const int s_off = srow * TROW + ((schunk ^ swz<HD>(srow)) << 3);
   // a tile is read through a buffer descriptor at its first row (scalar registers) with one 32-bit byte offset per
   // lane: half the address data of 64-bit pointers per lane, and two registers less
   const int64_t sg_base = (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
   const uint32_t sg_lane = 2u * (uint32_t)(schunk * 8 + srow * (int)a.kv_ss);
-  const uint32_t row16b = 2u * 16u * (uint32_t)a.kv_ss;
-  uint4 Ak0, Ak1, Ak2, Ak3, Av0, Av1, Av2, Av3, Bk0, Bk1, Bk2, Bk3, Bv0, Bv1, Bv2, Bv3;
+  const uint32_t row16b = 2u * SRP * (uint32_t)a.kv_ss;       // one staging pass further
+  uint4 Ak0, Ak1, Ak2 = {}, Ak3 = {}, Av0, Av1, Av2 = {}, Av3 = {}, Bk0, Bk1, Bk2 = {}, Bk3 = {}, Bv0, Bv1, Bv2 = {}, Bv3 = {};
   int Aseg = 0, Bseg = 0;
   float Abias = 0.f, Bbias = 0.f;
   // key chunk index and offset inside the chunk of the first key of the next tile to request (tiles are requested
@@ -1298,7 +1312,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const int t_ = min((T), ntiles - 1);                                                                \
     const __amdgpu_buffer_rsrc_t rk_ = tile_rsrc(a.k + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
     S##k0 = ld_buf(rk_, sg_lane, 0); S##k1 = ld_buf(rk_, sg_lane, row16b);                              \
-    S##k2 = ld_buf(rk_, sg_lane, 2 * row16b); S##k3 = ld_buf(rk_, sg_lane, 3 * row16b);                 \
+    if (SNP == 4) { S##k2 = ld_buf(rk_, sg_lane, 2 * row16b); S##k3 = ld_buf(rk_, sg_lane, 3 * row16b); } \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       const int kj_ = k_base + t_ * FBN + stid;                                                         \
       if (HAS_SEG) {                                                                                    \
@@ -1315,13 +1329,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const int t_ = min((T), ntiles - 1);                                                                \
     const __amdgpu_buffer_rsrc_t rv_ = tile_rsrc(a.v + sg_base + (int64_t)t_ * FBN * a.kv_ss);          \
     S##v0 = ld_buf(rv_, sg_lane, 0); S##v1 = ld_buf(rv_, sg_lane, row16b);                              \
-    S##v2 = ld_buf(rv_, sg_lane, 2 * row16b); S##v3 = ld_buf(rv_, sg_lane, 3 * row16b);                 \
+    if (SNP == 4) { S##v2 = ld_buf(rv_, sg_lane, 2 * row16b); S##v3 = ld_buf(rv_, sg_lane, 3 * row16b); } \
   }
 #define RA_WS_STORE_K(S, BUF)                                                                            \
   {                                                                                                     \
     uint16_t* dk_ = Ks + (BUF) * WS_TILE + s_off;                                                       \
-    *(uint4*)(dk_) = S##k0; *(uint4*)(dk_ + 16 * TROW) = S##k1;                                         \
-    *(uint4*)(dk_ + 32 * TROW) = S##k2; *(uint4*)(dk_ + 48 * TROW) = S##k3;                             \
+    *(uint4*)(dk_) = S##k0; *(uint4*)(dk_ + SRP * TROW) = S##k1;                                        \
+    if (SNP == 4) { *(uint4*)(dk_ + 2 * SRP * TROW) = S##k2; *(uint4*)(dk_ + 3 * SRP * TROW) = S##k3; } \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       if (HAS_SEG) seg_ks[BUF][stid] = S##seg;                                                          \
       /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
@@ -1331,8 +1345,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #define RA_WS_STORE_V(S, BUF)                                                                            \
   {                                                                                                     \
     uint16_t* dv_ = Vs + (BUF) * WS_TILE + s_off;                                                       \
-    *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + 16 * TROW) = S##v1;                                         \
-    *(uint4*)(dv_ + 32 * TROW) = S##v2; *(uint4*)(dv_ + 48 * TROW) = S##v3;                             \
+    *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + SRP * TROW) = S##v1;                                        \
+    if (SNP == 4) { *(uint4*)(dv_ + 2 * SRP * TROW) = S##v2; *(uint4*)(dv_ + 3 * SRP * TROW) = S##v3; } \
   }
   if (role == 1) {
     RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
@@ -1356,9 +1370,9 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
       seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
     }
     const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-    bf16x8 qf[8];
+    bf16x8 qf[NK];
 #pragma unroll
-    for (int t = 0; t < 8; t++) qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
+    for (int t = 0; t < NK; t++) qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
     const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
     // running max (log2 domain; m2 is the lazy reference the probabilities are taken against, m_true the
     // exact one) and this half-row's share of the running sum
@@ -1369,9 +1383,9 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     }
     float m_true = m2, ps = 0.f;
     constexpr float kLazy = 16.f;
-    int n_off[8];
+    int n_off[NK];
 #pragma unroll
-    for (int t = 0; t < 8; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz(lo)) << 3);
+    for (int t = 0; t < NK; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz<HD>(lo)) << 3);
     uint16_t* const dw = &Ds[pair][0][lo * WS_PSTR + hi * 4];
     typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
@@ -1382,11 +1396,11 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     _Pragma("unroll") for (int e = 0; e < 4; e++) SN[g * 4 + e] = b4_[e];                               \
   }
 #define RA_WS_AREAD(G, KA, BUF, BLK)                                                                    \
-  _Pragma("unroll") for (int i = 0; i < 2; i++)                                                         \
-    KA[i] = *(const bf16x8*)(Ks + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[2 * (G) + i]);
+  _Pragma("unroll") for (int i = 0; i < KPG; i++)                                                         \
+    KA[i] = *(const bf16x8*)(Ks + (BUF) * WS_TILE + (BLK) * 32 * TROW + n_off[KPG * (G) + i]);
 #define RA_WS_AMFMA(G, KA, SN)                                                                          \
-  _Pragma("unroll") for (int i = 0; i < 2; i++)                                                         \
-    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[2 * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T (:134) */
+  _Pragma("unroll") for (int i = 0; i < KPG; i++)                                                         \
+    SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(KA[i], qf[KPG * (G) + i], SN, 0, 0, 0);   /* S^T = K Q^T (:134) */
     // The block's 32 keys x this lane's query: the running max first (group 0), then eight keys
     // (registers 4G .. 4G+3 of both halves) of P^T per group.  (:138-144)
 #define RA_WS_ROWMAX(SC, BUF, BLK, PB, MASKED)                                                          \
@@ -1468,7 +1482,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   }
 
     f32x16 s_a, s_b;
-    bf16x8 ka[4][2];
+    bf16x8 ka[4][KPG];
     RA_WS_INIT(s_a, 0, 0);
 #pragma unroll
     for (int g = 0; g < 4; g++) {
@@ -1584,16 +1598,16 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #undef RA_WS_PRODUCE
   } else {
     // =========================== consumer: O^T += V^T P^T   (:141-143)
-    f32x16 acc[4];
+    f32x16 acc[NDB];
     float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
     if (a.carry_is_initial) {
 #pragma unroll
-      for (int db = 0; db < 4; db++)
+      for (int db = 0; db < NDB; db++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
     } else {
 #pragma unroll
-      for (int db = 0; db < 4; db++)
+      for (int db = 0; db < NDB; db++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
           const f32x4 t4 = *(const f32x4*)(nump + db * 32 + g * 8);
@@ -1601,13 +1615,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
           for (int e = 0; e < 4; e++) acc[db][g * 4 + e] = t4[e];
         }
     }
-    int t_off[4][2];
+    int t_off[NDB][2];
     {
       const int i = lane & 15, rr = (i >> 2) + 8 * hi, c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
 #pragma unroll
-      for (int db = 0; db < 4; db++) {
-        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz(rr)) << 3) + half * 4;
-        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz(rr + 4)) << 3) + half * 4;
+      for (int db = 0; db < NDB; db++) {
+        t_off[db][0] = rr * TROW + (((4 * db + c0) ^ swz<HD>(rr)) << 3) + half * 4;
+        t_off[db][1] = (rr + 4) * TROW + (((4 * db + c0) ^ swz<HD>(rr + 4)) << 3) + half * 4;
       }
     }
     const uint16_t* const dr = &Ds[pair][0][lo * WS_PSTR + hi * 8];   // B operand: query column lo, 8 keys
@@ -1616,14 +1630,14 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #define RA_WS_CREAD(K, F, BUF, BLK)                                                                     \
   {                                                                                                     \
     const uint16_t* tp_ = Vs + (BUF) * WS_TILE + ((BLK) * 32 + (K) * 16) * TROW;                        \
-    _Pragma("unroll") for (int db = 0; db < 4; db++) {                                                  \
+    _Pragma("unroll") for (int db = 0; db < NDB; db++) {                                                  \
       const s16x4 x0_ = lds_read_tr(tp_ + t_off[db][0]);                                                \
       const s16x4 x1_ = lds_read_tr(tp_ + t_off[db][1]);                                                \
       F[db] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0_, x1_, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
   }
 #define RA_WS_CMFMA(F, BOP)                                                                             \
-  _Pragma("unroll") for (int db = 0; db < 4; db++)                                                      \
+  _Pragma("unroll") for (int db = 0; db < NDB; db++)                                                      \
     acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[db], BOP, acc[db], 0, 0, 0);
     // fa holds the first 16 keys of the block on entry and, on exit, those of block NBLK of buffer NBUF
 #define RA_WS_CONSUME(BUF, BLK, PB, NBUF, NBLK)                                                         \
@@ -1632,7 +1646,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const bf16x8 d1_ = *(const bf16x8*)(dr + (PB) * WS_PD + 16);                                        \
     const float alpha_ = al[pair][PB][lo];                                                              \
     if (__builtin_amdgcn_ballot_w64(alpha_ != 1.f) != 0) {                                              \
-      _Pragma("unroll") for (int db = 0; db < 4; db++)                                                  \
+      _Pragma("unroll") for (int db = 0; db < NDB; db++)                                                  \
         _Pragma("unroll") for (int r = 0; r < 16; r++) acc[db][r] *= alpha_;                            \
     }                                                                                                   \
     RA_WS_CREAD(1, fb, BUF, BLK);                                                                       \
@@ -1642,7 +1656,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     __builtin_amdgcn_sched_barrier(0);                                                                  \
     RA_WS_CMFMA(fb, d1_);                                                                               \
   }
-    bf16x8 fa[4], fb[4];
+    bf16x8 fa[NDB], fb[NDB];
     int cur = 0;
     RA_WS_CREAD(0, fa, 0, 0);
     __syncthreads();      // step 0
@@ -1677,7 +1691,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     const float den_row = dens[pair][lo];
     uint16_t* outp = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < NDB; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         f32x4 t4;
@@ -1712,7 +1726,7 @@ static bool keep_ok(const ra_mask& m) {
 
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
   const ra_mask& m = p->mask;
-  return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
+  return p->dtype == RA_BF16 && (p->D == 128 || p->D == 64) && m.query_chunk_size % FBM == 0 && m.key_chunk_size % FBN == 0 &&
          keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
          aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator) &&
@@ -1744,23 +1758,29 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* r, hipStream_
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;
   RA_REQUIRE(nwg3 < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_mfma: grid too large");
   dim3 grid3((unsigned)((nwg3 + 7) / 8 * 8)), block3(512);
+#define RA_LAUNCH_FWD(...)                                                               \
+  do {                                                                                   \
+    if (p->D == 128) attn_fwd_ws_kernel<128, __VA_ARGS__><<<grid3, block3, 0, s>>>(a);   \
+    else attn_fwd_ws_kernel<64, __VA_ARGS__><<<grid3, block3, 0, s>>>(a);                \
+  } while (0)
   if (keep && p->mask.keep_mode == RA_KEEP_DROPOUT) {
-    if (seg && bias) attn_fwd_ws_kernel<true, true, 2><<<grid3, block3, 0, s>>>(a);
-    else if (seg) attn_fwd_ws_kernel<true, false, 2><<<grid3, block3, 0, s>>>(a);
-    else if (bias) attn_fwd_ws_kernel<false, true, 2><<<grid3, block3, 0, s>>>(a);
-    else attn_fwd_ws_kernel<false, false, 2><<<grid3, block3, 0, s>>>(a);
-  } else if (keep) attn_fwd_ws_kernel<false, false, 1><<<grid3, block3, 0, s>>>(a);
-  else if (seg && bias) attn_fwd_ws_kernel<true, true><<<grid3, block3, 0, s>>>(a);
-  else if (seg) attn_fwd_ws_kernel<true, false><<<grid3, block3, 0, s>>>(a);
-  else if (bias) attn_fwd_ws_kernel<false, true><<<grid3, block3, 0, s>>>(a);
-  else attn_fwd_ws_kernel<false, false><<<grid3, block3, 0, s>>>(a);
+    if (seg && bias) RA_LAUNCH_FWD(true, true, 2);
+    else if (seg) RA_LAUNCH_FWD(true, false, 2);
+    else if (bias) RA_LAUNCH_FWD(false, true, 2);
+    else RA_LAUNCH_FWD(false, false, 2);
+  } else if (keep) RA_LAUNCH_FWD(false, false, 1);
+  else if (seg && bias) RA_LAUNCH_FWD(true, true);
+  else if (seg) RA_LAUNCH_FWD(true, false);
+  else if (bias) RA_LAUNCH_FWD(false, true);
+  else RA_LAUNCH_FWD(false, false);
+#undef RA_LAUNCH_FWD
   RA_CHECK_LAUNCH("attn_fwd_ws");
   return RA_OK;
 }
 
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p) {
   const ra_mask& m = p->mask;
-  return p->dtype == RA_BF16 && p->D == HD && m.query_chunk_size % FBM == 0 && m.key_chunk_size % KBN == 0 &&
+  return p->dtype == RA_BF16 && (p->D == 128 || p->D == 64) && m.query_chunk_size % FBM == 0 && m.key_chunk_size % KBN == 0 &&
          keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0 &&
          p->dkv_stride_s % 4 == 0 && p->dkv_stride_b % 4 == 0 && aligned16(p->q) && aligned16(p->k) &&
@@ -1794,8 +1814,13 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* r, int parts,
   const bool do_dkv = (parts & 2) != 0, do_dq = (parts & 1) != 0;
 #define RA_LAUNCH_BWD(...)                                                               \
   do {                                                                                   \
-    if (do_dkv) attn_bwd_dkv_ws_kernel<__VA_ARGS__><<<gk, block, 0, s>>>(a);             \
-    if (do_dq) attn_bwd_dq_ws_kernel<__VA_ARGS__><<<gq, block, 0, s>>>(a);               \
+    if (p->D == 128) {                                                                   \
+      if (do_dkv) attn_bwd_dkv_ws_kernel<128, __VA_ARGS__><<<gk, block, 0, s>>>(a);      \
+      if (do_dq) attn_bwd_dq_ws_kernel<128, __VA_ARGS__><<<gq, block, 0, s>>>(a);        \
+    } else {                                                                             \
+      if (do_dkv) attn_bwd_dkv_ws_kernel<64, __VA_ARGS__><<<gk, block, 0, s>>>(a);       \
+      if (do_dq) attn_bwd_dq_ws_kernel<64, __VA_ARGS__><<<gq, block, 0, s>>>(a);         \
+    }                                                                                    \
   } while (0)
   if (p->mask.keep_bits_k && p->mask.keep_mode == RA_KEEP_DROPOUT) {
     if (seg && bias) RA_LAUNCH_BWD(true, true, 2);

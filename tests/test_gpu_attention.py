@@ -153,7 +153,7 @@ def test_invalid_shapes_raise():
         ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1))
 
 
-# --------------------------------------------------------------------------- MFMA kernels (bf16, D=128)
+# --------------------------------------------------------------------------- MFMA kernels (bf16, D = 128 or 64)
 MFMA_FWD_CASES = [
     # B, S, H, qc, kc, cbs, n, bias, seg
     (1, 256, 1, 128, 64, 1, 1, False, False),
@@ -169,10 +169,11 @@ MFMA_FWD_CASES = [
 ]
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("case", MFMA_FWD_CASES)
-def test_mfma_forward_matches_oracle(case):
+def test_mfma_forward_matches_oracle(case, D):
     B, S, H, qc, kc, cbs, n, use_bias, use_seg = case
-    check_case(B, S, H, 128, qc, kc, cbs, n, use_bias, use_seg, torch.bfloat16, impl="mfma", bwd=False,
+    check_case(B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, torch.bfloat16, impl="mfma", bwd=False,
                seg_mean=S // 5)
 
 
@@ -212,15 +213,17 @@ MFMA_BWD_CASES = [
 ]
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("case", MFMA_BWD_CASES)
-def test_mfma_backward_matches_oracle(case):
+def test_mfma_backward_matches_oracle(case, D):
     B, S, H, qc, kc, cbs, n, use_bias, use_seg = case
-    check_case(B, S, H, 128, qc, kc, cbs, n, use_bias, use_seg, torch.bfloat16, impl="mfma", bwd=True,
+    check_case(B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, torch.bfloat16, impl="mfma", bwd=True,
                seg_mean=S // 5)
 
 
-def test_mfma_backward_matches_generic_kernels_at_4k():
-    B, S, H, D = 1, 4096, 2, 128
+@pytest.mark.parametrize("D", [128, 64])
+def test_mfma_backward_matches_generic_kernels_at_4k(D):
+    B, S, H = 1, 4096, 2
     q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=D ** -0.25)
     seg = packed_segment_ids(B, S, 700, seed=22)
     res = {}
