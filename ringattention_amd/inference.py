@@ -5,8 +5,8 @@ anything else runs on the fp32 vector-ALU kernels."""
 import torch
 
 from . import _lib as L
-from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, _blockwise_attention_fwd,
-                                _bwd_delta, _check_qkv, axis_size)
+from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, _blockwise_attention_fwd, _bwd_delta,
+                                _check_qkv, _save_residuals, _saved_residuals, axis_size)
 
 
 def _inference_cfg(q, q_len, kv_len, float32_logits):
@@ -91,13 +91,12 @@ class _RingAttentionInferenceFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, attn_mask, axis_name, float32_logits):
         out, res = _fwd(q, k, v, attn_mask, axis_name, float32_logits)
-        ctx.res = res
+        _save_residuals(ctx, res)
         return out
 
     @staticmethod
     def backward(ctx, g):
-        dq, dk, dv = _bwd(ctx.res, g)
-        ctx.res = None
+        dq, dk, dv = _bwd(_saved_residuals(ctx), g)
         return dq, dk, dv, None, None, None
 
 

@@ -822,14 +822,28 @@ class _RingAttentionFn(torch.autograd.Function):
     def forward(ctx, q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
         out, res = _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits,
                                        blockwise_kwargs)
-        ctx.res = res
+        _save_residuals(ctx, res)
         return out
 
     @staticmethod
     def backward(ctx, g):
-        dq, dk, dv = _ring_attention_bwd(ctx.res, g)
-        ctx.res = None
+        dq, dk, dv = _ring_attention_bwd(_saved_residuals(ctx), g)
         return dq, dk, dv, None, None, None, None, None, None
+
+
+def _save_residuals(ctx, res):
+    """The tensors of the residuals (:53) go through save_for_backward - autograd then checks that none was edited
+    in place before the backward pass, frees them with the graph, and `out -> grad_fn -> ctx -> out` is no reference
+    cycle; the mask inputs and the configuration are plain attributes."""
+    out, q, k, v, mi, cfg, n, den, mx = res
+    ctx.save_for_backward(out, q, k, v, den, mx)
+    ctx.ra_extra = (mi, cfg, n)
+
+
+def _saved_residuals(ctx):
+    out, q, k, v, den, mx = ctx.saved_tensors
+    mi, cfg, n = ctx.ra_extra
+    return out, q, k, v, mi, cfg, n, den, mx
 
 
 def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):

@@ -397,3 +397,21 @@ def test_ring_step_entry_points_refuse_what_they_do_not_take():
     assert lib.ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), None) == L.RA_ERR_INVALID    # numerator needed
     p.impl = L.RA_IMPL_GENERIC
     assert lib.ra_attn_fwd_ring_step(ctypes.byref(p), ctypes.byref(r), None) == L.RA_ERR_UNSUPPORTED
+
+
+def test_residuals_are_saved_tensors():
+    """A second backward pass with retain_graph gives the same gradients; editing q in place between the forward
+    and the backward pass is refused by autograd instead of giving gradients of the wrong input."""
+    q, k, v, do = (t.to(DEV) for t in make_qkv(1, 256, 2, 128, dtype=torch.bfloat16, seed=5))
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    out = ra.ringattention(q, k, v, None, None, None, "sp", True, kwargs(128, 128, 1))
+    g1 = torch.autograd.grad(out, (q, k, v), do, retain_graph=True)
+    g2 = torch.autograd.grad(out, (q, k, v), do)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)
+    q2 = q.detach().clone().requires_grad_(True)
+    qq = q2 * 1.0
+    out = ra.ringattention(qq, k, v, None, None, None, "sp", True, kwargs(128, 128, 1))
+    qq.add_(1.0)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        out.backward(do)
