@@ -87,6 +87,46 @@ def _event_ms(fn, reps):
     return total / reps
 
 
+def _sclk_under_load(fn, seconds=2.0):
+    """Shader clock in MHz as ``rocm-smi --showclocks`` reports it while ``fn`` runs back to back for ``seconds``:
+    (median, min, max) over the samples taken under load, or None where the tool is not there.  The nominal peak
+    figures assume 2400 MHz."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    import torch
+    tool = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    if not os.path.exists(tool):
+        return None
+    samples, stop = [], threading.Event()
+
+    def poll():
+        while not stop.is_set():
+            try:
+                txt = subprocess.run([tool, "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+            except Exception:
+                return
+            m = re.search(r"sclk clock level:[^(]*\((\d+)Mhz\)", txt)
+            if m:
+                samples.append(int(m.group(1)))
+            stop.wait(0.25)
+
+    th = threading.Thread(target=poll, daemon=True)
+    t0 = time.perf_counter()
+    th.start()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+    stop.set()
+    th.join(timeout=10)
+    busy = sorted(x for x in samples if x > 500)
+    if not busy:
+        return None
+    return {"median": busy[len(busy) // 2], "min": busy[0], "max": busy[-1], "samples": len(busy)}
+
+
 def _packed_segments(S, mean_len, seed, device):
     import numpy as np
     import torch
@@ -158,6 +198,7 @@ def bench_attention(args, ring, dropout=False):
     # --- per-kernel durations (events on the launch stream), N=1 shape of one ring step
     roof = None
     kern = {}
+    sclk = None
     if not ring:
         with torch.no_grad():
             cfg = rh._Config(kw)
@@ -182,6 +223,8 @@ def bench_attention(args, ring, dropout=False):
                                                          _grads_initial=L.RA_GRAD_INIT_DQ | L.RA_GRAD_INIT_DKV,
                                                          _dq_out=dq_o, _dkv_out=(dk_o, dv_o))
                 kern["attn_bwd_%s_ws_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
+                if which == "dkv" and not (args.no_extras or dropout):
+                    sclk = _sclk_under_load(bw)       # the clock the dominant kernel actually runs at
             if dropout:
                 def draw():
                     m2 = rh._MaskInputs(cfg, None, None, None, B, q.device, S)
@@ -201,6 +244,10 @@ def bench_attention(args, ring, dropout=False):
                                   if S == 32768 and not dropout and util.get(dom) else None),
                 "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
                 "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
+        if sclk:
+            # the published peak assumes 2400 MHz; what the same matrix pipes can do at the clock the kernel runs at
+            roof["sclk_mhz_under_load"] = sclk
+            roof["frac_of_peak_at_sclk"] = round(ach / (PEAK_BF16_TFLOPS * sclk["median"] / 2400.0), 4)
         if dropout:
             roof["traffic"] = None
             roof["mask_draw_and_pack_ms"] = round(mask_ms, 3)

@@ -415,3 +415,38 @@ def test_residuals_are_saved_tensors():
     qq.add_(1.0)
     with pytest.raises(RuntimeError, match="modified by an inplace operation"):
         out.backward(do)
+
+
+def test_ring_forward_with_segment_ids_replays_from_a_hip_graph():
+    """The ring forward with segment ids and a bias, captured once after a first eager call (which fills the
+    per-tensor cache of the segment tile ranges, so that nothing is copied to the host under capture) and replayed
+    with new q / k / v contents: every replay equals the eager result on the same inputs."""
+    B, S, H, D, n = 1, 2048, 2, 128, 4
+    kw = kwargs(256, 256, 1, impl="mfma")
+    seg = packed_segment_ids(B, S, 500, seed=2).to(DEV)
+    bias = torch.randn(1, 1, 1, S, generator=torch.Generator().manual_seed(3)).to(DEV)
+    qs, ks, vs = (torch.zeros(B, S, H, D, dtype=torch.bfloat16, device=DEV) for _ in range(3))
+
+    def call():
+        with ra.ring_axis("sp", n):
+            return ra.ringattention(qs, ks, vs, bias, seg, None, axis_name="sp", float32_logits=True,
+                                    blockwise_kwargs=kw)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.no_grad(), torch.cuda.graph(graph):
+        out_graph = call()
+    for seed in (1, 2, 3):
+        q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=seed)
+        qs.copy_(q), ks.copy_(k), vs.copy_(v)
+        graph.replay()
+        torch.cuda.synchronize()
+        with torch.no_grad():
+            eager = call()
+        torch.cuda.synchronize()
+        assert torch.equal(out_graph.view(torch.int16), eager.view(torch.int16)), seed
+        assert float(eager.float().abs().max()) > 0
