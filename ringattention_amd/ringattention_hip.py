@@ -603,6 +603,7 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
         if cache_idx is not None:
             raise NotImplementedError("attention dropout together with cache_idx is not supported")
         cfg.skip_masked_tiles = False      # dropout can leave a row without any allowed key
+    _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total)
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)         # :23
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)          # :49
     out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
@@ -637,6 +638,37 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
             _finalize(carry[0], carry[1], out[:, qs])
     del num
     return out, (out, q, k, v, mi, cfg, n, den, mx)
+
+
+def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=128):
+    """Chunk sizes the MFMA kernels do not tile (they want multiples of 128) are replaced by 128 where that cannot
+    change the result.  The chunk sizes enter the reference's result in four places only: which chunk pairs run
+    (below_or_on_diag, :324-331), the clamped slices of segment_ids (:286-295) and of the dropout mask (:311-320),
+    and the rows of a per-row bias (:279-283).  With causal_block_size 1 and even chunk sizes - or a block size that
+    divides both chunk sizes - a chunk pair that does not run holds causally masked pairs only (its last row lies
+    before its first key, and a tie is impossible), and a masked pair weighs exp(finfo.min - max) = 0 exactly as
+    long as its row has an unmasked key, which is what skip_masked_tiles already asks for; so both chunkings sum
+    over the same pairs.  Without a causal block size every chunk pair runs.  The slices are not clamped when the
+    segment ids cover every position, there is no dropout here, and a per-row bias takes the generic kernels."""
+    if cfg.impl == L.RA_IMPL_GENERIC or q.dtype != torch.bfloat16 or q.shape[3] not in (64, 128):
+        return
+    if cfg.qc % grid == 0 and cfg.kc % grid == 0:
+        return
+    if q_len % grid or kv_len % grid or cfg.pdrop > 0.0 or not cfg.skip_masked_tiles:
+        return
+    if mi.cache_idx_host is not None or mi.cache_idx_dev is not None or mi.keep is not None:
+        return
+    if mi.bias is not None and mi.bias_strides[2] != 0:
+        return
+    if mi.seg is not None and mi.seg_len < max(q_total, kv_total):
+        return
+    if cfg.cbs is not None:
+        if cfg.cbs == 1:
+            if cfg.qc % 2 or cfg.kc % 2:
+                return
+        elif cfg.qc % cfg.cbs or cfg.kc % cfg.cbs or grid % cfg.cbs:
+            return
+    cfg.qc = cfg.kc = grid
 
 
 def _ring_plan(cfg, mi, n, q_len, kv_len):

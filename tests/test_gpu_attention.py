@@ -450,3 +450,33 @@ def test_ring_forward_with_segment_ids_replays_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(out_graph.view(torch.int16), eager.view(torch.int16)), seed
         assert float(eager.float().abs().max()) > 0
+
+
+# --- chunk sizes off the 128-grid of the MFMA kernels: served by them with 128 x 128 chunks where that sums over the
+# same pairs (even sizes under causal_block_size 1, a block size dividing both, or no causal mask at all)
+@pytest.mark.parametrize("qc,kc,cbs,n,use_seg", [(64, 64, 1, 1, False), (192, 64, 1, 2, True), (32, 96, 1, 1, True),
+                                                  (384, 192, None, 2, False), (64, 192, 32, 1, False),
+                                                  (96, 96, 1, 4, True)])
+def test_mfma_serves_chunk_sizes_off_its_grid(qc, kc, cbs, n, use_seg):
+    B, S, H, D = 1, 1536, 2, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=qc + kc, scale=1.0)
+    seg = packed_segment_ids(B, S, 400, seed=5) if use_seg else None
+    kw = kwargs(qc, kc, cbs, dtype=torch.float32, impl="mfma")       # "mfma": raises if the generic kernels were needed
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, None, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, None, seg, None, n, kw)
+    assert_close(out, ref_out, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, torch.bfloat16, name)
+
+
+def test_mfma_refuses_chunk_sizes_whose_chunking_matters():
+    """Odd chunk sizes under a causal mask (the reference then drops the diagonal pair of some chunk corners,
+    :324-331) stay with the generic kernels: impl="mfma" refuses, "auto" matches the oracle."""
+    B, S, H, D = 1, 384, 1, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=3, scale=1.0)
+    with pytest.raises(NotImplementedError):
+        run_hip(q, k, v, None, None, None, None, 1, kwargs(3, 3, 1, impl="mfma"))
+    kw = kwargs(3, 3, 1)
+    ref_out, _ = oracle_fwd_bwd(q, k, v, None, None, None, None, 1, kw)
+    out, _ = run_hip(q, k, v, None, None, None, None, 1, kw)
+    assert_close(out, ref_out, torch.bfloat16, "out")
