@@ -87,30 +87,48 @@ def _event_ms(fn, reps):
     return total / reps
 
 
+def _sclk_files():
+    """pp_dpm_sclk of the GPU this process uses (matched by PCI address where torch gives one; else every card)."""
+    import glob
+    import torch
+    files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    try:
+        pr = torch.cuda.get_device_properties(0)
+        addr = "%04x:%02x:%02x" % (getattr(pr, "pci_domain_id", 0), pr.pci_bus_id, pr.pci_device_id)
+        mine = [f for f in files if addr in os.path.realpath(os.path.dirname(f))]
+        if mine:
+            return mine
+    except Exception:
+        pass
+    return files
+
+
 def _sclk_under_load(fn, seconds=2.0):
-    """Shader clock in MHz as ``rocm-smi --showclocks`` reports it while ``fn`` runs back to back for ``seconds``:
-    (median, min, max) over the samples taken under load, or None where the tool is not there.  The nominal peak
-    figures assume 2400 MHz."""
+    """Shader clock in MHz (the level the driver marks current in sysfs pp_dpm_sclk, what rocm-smi --showclocks
+    prints) sampled from a thread while ``fn`` runs back to back for ``seconds``: median, min and max of the samples
+    taken under load, or None where the file is not readable.  Plain file reads: no child process is started.
+    The nominal peak figures assume 2400 MHz."""
     import re
-    import shutil
-    import subprocess
     import threading
     import torch
-    tool = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
-    if not os.path.exists(tool):
+    files = _sclk_files()
+    if not files:
         return None
     samples, stop = [], threading.Event()
 
     def poll():
         while not stop.is_set():
-            try:
-                txt = subprocess.run([tool, "--showclocks"], capture_output=True, text=True, timeout=5).stdout
-            except Exception:
-                return
-            m = re.search(r"sclk clock level:[^(]*\((\d+)Mhz\)", txt)
-            if m:
-                samples.append(int(m.group(1)))
-            stop.wait(0.25)
+            best = 0
+            for f in files:
+                try:
+                    m = re.search(r"(\d+)Mhz \*", open(f).read())
+                except OSError:
+                    m = None
+                if m:
+                    best = max(best, int(m.group(1)))
+            if best:
+                samples.append(best)
+            stop.wait(0.1)
 
     th = threading.Thread(target=poll, daemon=True)
     t0 = time.perf_counter()
