@@ -129,3 +129,47 @@ def test_invalid_arguments_return_codes_without_gpu():
     n.T, n.d = 4, 100
     assert lib.ra_rmsnorm_fwd(ctypes.byref(n), None) == _lib.RA_ERR_UNSUPPORTED
     assert lib.ra_rmsnorm_workspace_bytes(65536, 4096) == 4096 * 4096 * 4
+
+
+# --- chunk sizes off the 128-grid: what _fit_chunks_to_mfma_grid relies on, by brute force against the predicate
+@pytest.mark.parametrize("qc,kc,cbs", [(64, 64, 1), (192, 64, 1), (32, 96, 1), (96, 96, 1), (2, 6, 1), (64, 192, 32),
+                                       (24, 8, 4), (128, 128, 1), (128, 128, 32)])
+def test_a_chunk_pair_that_does_not_run_holds_masked_pairs_only(qc, kc, cbs):
+    """Even chunk sizes under causal_block_size 1, or a block size that divides both: every causally allowed pair
+    (q // cbs >= k // cbs) lies in a chunk pair that below_or_on_diag lets run, so two such chunkings sum over the
+    same pairs."""
+    S = 384
+    for q in range(S):
+        ks = torch.arange(0, S)
+        allowed = (q // cbs) >= (ks // cbs)
+        runs = torch.tensor([bool(O.below_or_on_diag(q // qc, qc, int(k) // kc, kc, cbs)) for k in range(0, S, kc)])
+        runs = runs.repeat_interleave(kc)[:S]
+        assert bool((runs | ~allowed).all()), (q, qc, kc, cbs)
+
+
+def test_odd_chunk_sizes_can_drop_an_allowed_pair():
+    """What keeps odd sizes away from the remapping: with query chunks of 3 and key chunks of 2 the causally allowed
+    pair (q, k) = (2, 2) sits in key chunk 1 (keys 2-3), which does not run for query chunk 0 (rows 0-2): the
+    predicate compares the last row with the first key strictly (ringattention_jax.py:331)."""
+    assert not O.below_or_on_diag(0, 3, 1, 2, 1)
+    assert 2 // 1 >= 2 // 1
+
+
+class _FakeMaskInputs:
+    cache_idx_host = cache_idx_dev = keep = bias = seg = None
+    bias_strides = (0, 0, 0, 0)
+    seg_len = 0
+
+
+@pytest.mark.parametrize("qc,kc,cbs,skip,expect", [
+    (64, 64, 1, True, 128), (192, 64, 1, True, 128), (3, 3, 1, True, 3), (64, 64, 1, False, 64),
+    (384, 192, None, True, 128), (64, 192, 32, True, 128), (64, 192, 48, True, 64), (256, 256, 1, True, 256)])
+def test_fit_chunks_to_mfma_grid_decisions(qc, kc, cbs, skip, expect):
+    from ringattention_amd import ringattention_hip as rh
+    cfg = rh._Config(dict(query_chunk_size=qc, key_chunk_size=kc, causal_block_size=cbs))
+    cfg.skip_masked_tiles = skip
+    q = torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16)
+    rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), q, 768, 768, 768, 768)
+    assert cfg.qc == expect, (cfg.qc, cfg.kc)
+    if expect == 128:
+        assert cfg.kc == 128
