@@ -356,10 +356,11 @@ def test_first_and_last_step_modes_reject_missing_buffers():
 
 
 # --- a scan step of all virtual devices as one launch per kernel (ra_attn_*_ring_step) against one launch per device
-@pytest.mark.parametrize("n,cbs,use_seg,use_bias", [(2, 1, False, False), (4, 1, True, True), (8, 1, True, False),
-                                                    (4, None, False, True), (8, 256, True, True)])
-def test_ring_step_launch_equals_device_launches_bitwise(n, cbs, use_seg, use_bias):
-    B, S, H, D = 2, 4096, 2, 128
+@pytest.mark.parametrize("n,cbs,use_seg,use_bias,D", [(2, 1, False, False, 128), (4, 1, True, True, 128),
+                                                      (8, 1, True, False, 128), (4, None, False, True, 128),
+                                                      (8, 256, True, True, 128), (4, 1, True, True, 64)])
+def test_ring_step_launch_equals_device_launches_bitwise(n, cbs, use_seg, use_bias, D):
+    B, S, H = 2, 4096, 2
     q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=n, scale=1.0)
     g = torch.Generator().manual_seed(n + 50)
     bias = torch.randn(B, H, 1, S, generator=g) if use_bias else None

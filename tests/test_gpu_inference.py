@@ -120,7 +120,7 @@ def _structured_mask(B, H, S, kind, seed):
 
 
 MFMA_CASES = [
-    # B, S, H, n, mask kind   (bf16, D = 128, shards of a multiple of 256 rows: the MFMA kernels run)
+    # B, S, H, n, mask kind   (bf16, D = 128 or 64, shards of a multiple of 256 rows: the MFMA kernels run)
     (1, 512, 2, 1, "causal"),
     (1, 1024, 2, 2, "causal"),
     (2, 1024, 2, 2, "causal_padding"),
@@ -129,10 +129,10 @@ MFMA_CASES = [
 ]
 
 
+@pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("case", MFMA_CASES)
-def test_inference_mfma_path_matches_oracle(case):
+def test_inference_mfma_path_matches_oracle(case, D):
     B, S, H, n, kind = case
-    D = 128
     q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=D ** -0.25)
     mask = _structured_mask(B, H, S, kind, 22)
     out, grads = _run(q, k, v, do, mask, n)
