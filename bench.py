@@ -87,34 +87,49 @@ def _event_ms(fn, reps):
     return total / reps
 
 
-def _sclk_files():
-    """pp_dpm_sclk of the GPU this process uses (matched by PCI address where torch gives one; else every card)."""
+def _gpu_sysfs_dirs():
+    """sysfs device directories of the GPU this process uses (matched by PCI address where torch gives one; else
+    every card)."""
     import glob
     import torch
-    files = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    dirs = sorted(os.path.dirname(f) for f in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
     try:
         pr = torch.cuda.get_device_properties(0)
         addr = "%04x:%02x:%02x" % (getattr(pr, "pci_domain_id", 0), pr.pci_bus_id, pr.pci_device_id)
-        mine = [f for f in files if addr in os.path.realpath(os.path.dirname(f))]
+        mine = [d for d in dirs if addr in os.path.realpath(d)]
         if mine:
             return mine
     except Exception:
         pass
-    return files
+    return dirs
+
+
+def _read_int(path):
+    try:
+        return int(open(path).read().split()[0])
+    except (OSError, ValueError, IndexError):
+        return None
 
 
 def _sclk_under_load(fn, seconds=2.0):
     """Shader clock in MHz (the level the driver marks current in sysfs pp_dpm_sclk, what rocm-smi --showclocks
-    prints) sampled from a thread while ``fn`` runs back to back for ``seconds``: median, min and max of the samples
-    taken under load, or None where the file is not readable.  Plain file reads: no child process is started.
-    The nominal peak figures assume 2400 MHz."""
+    prints) and board power in W (hwmon power1_input / power1_average, next to the limit in power1_cap) sampled from
+    a thread while ``fn`` runs back to back for ``seconds``: median, min and max of the samples taken under load, or
+    None where the files are not readable.  Plain file reads: no child process is started.  The nominal peak figures
+    assume 2400 MHz; the samples of the first half second (the ramp from idle) are left out of the power figures."""
+    import glob
     import re
     import threading
     import torch
-    files = _sclk_files()
-    if not files:
+    dirs = _gpu_sysfs_dirs()
+    if not dirs:
         return None
-    samples, stop = [], threading.Event()
+    files = [os.path.join(d, "pp_dpm_sclk") for d in dirs]
+    pfiles = [p for d in dirs for p in glob.glob(os.path.join(d, "hwmon/hwmon*/power1_input")) +
+              glob.glob(os.path.join(d, "hwmon/hwmon*/power1_average"))][:1]
+    cap = _read_int(pfiles[0].rsplit("/", 1)[0] + "/power1_cap") if pfiles else None
+    samples, watts, stop = [], [], threading.Event()
+    t0 = time.perf_counter()
 
     def poll():
         while not stop.is_set():
@@ -128,10 +143,12 @@ def _sclk_under_load(fn, seconds=2.0):
                     best = max(best, int(m.group(1)))
             if best:
                 samples.append(best)
+            w = _read_int(pfiles[0]) if pfiles else None
+            if w and time.perf_counter() - t0 > 0.5:
+                watts.append(w * 1e-6)
             stop.wait(0.1)
 
     th = threading.Thread(target=poll, daemon=True)
-    t0 = time.perf_counter()
     th.start()
     while time.perf_counter() - t0 < seconds:
         for _ in range(4):
@@ -142,7 +159,12 @@ def _sclk_under_load(fn, seconds=2.0):
     busy = sorted(x for x in samples if x > 500)
     if not busy:
         return None
-    return {"median": busy[len(busy) // 2], "min": busy[0], "max": busy[-1], "samples": len(busy)}
+    res = {"median": busy[len(busy) // 2], "min": busy[0], "max": busy[-1], "samples": len(busy)}
+    if watts:
+        watts.sort()
+        res["power_w"] = {"median": round(watts[len(watts) // 2], 1), "max": round(watts[-1], 1),
+                          "cap": round(cap * 1e-6, 1) if cap else None}
+    return res
 
 
 def _packed_segments(S, mean_len, seed, device):
@@ -264,6 +286,7 @@ def bench_attention(args, ring, dropout=False):
                 "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
         if sclk:
             # the published peak assumes 2400 MHz; what the same matrix pipes can do at the clock the kernel runs at
+            roof["power_w_under_load"] = sclk.pop("power_w", None)
             roof["sclk_mhz_under_load"] = sclk
             roof["frac_of_peak_at_sclk"] = round(ach / (PEAK_BF16_TFLOPS * sclk["median"] / 2400.0), 4)
         if dropout:
@@ -398,6 +421,7 @@ def bench_ffn(args):
     a_out = torch.empty(slab, f, dtype=torch.bfloat16, device=dev)
     gemm_ms = _event_ms(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out), 5)
     gemm_tf = 2.0 * slab * d * f / (gemm_ms * 1e-3) / 1e12
+    sclk = None if args.no_extras else _sclk_under_load(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out))
     cpu = None
     if not args.no_cpu:
         from oracle import ringattention_oracle as O
@@ -428,7 +452,11 @@ def bench_ffn(args):
                                  if (T, slab) == (65536, 16384) else None),
                      "mfma_util_pmc": {"kernel": _measured(MFMA_PROFILE, "mfma_util").get("gemm_bf16_w4_kernel<false,false>"),
                                        "source": "profiles/" + MFMA_PROFILE},
-                     "kernel_ms": {"gemm_bf16_w4_kernel<false, false>": round(gemm_ms, 3)}},
+                     "kernel_ms": {"gemm_bf16_w4_kernel<false, false>": round(gemm_ms, 3)},
+                     "power_w_under_load": sclk.pop("power_w", None) if sclk else None,
+                     "sclk_mhz_under_load": sclk,
+                     "frac_of_peak_at_sclk": (round(gemm_tf / (PEAK_BF16_TFLOPS * sclk["median"] / 2400.0), 4)
+                                              if sclk else None)},
         "cpu_baseline": cpu,
     }
 
