@@ -115,6 +115,10 @@ typedef struct ra_attn_fwd_params {
                                  residuals, :53).  Saves the numerator's round trip through memory and
                                  ra_attn_finalize */
   int64_t out_stride_b, out_stride_s;
+  float* out_f32;             /* nullable, only together with `out`: the same quotient BEFORE it is rounded to `dtype`,
+                                 (B,Sq,H,D) fp32 with the element strides of `out`.  It is the `output` the reference
+                                 keeps as a residual (:53) and multiplies with the cotangent in its backward pass
+                                 (:218); ra_attn_bwd_delta takes it in place of the rounded `out` */
 } ra_attn_fwd_params;
 
 /* _blockwise_attention_bwd (ringattention_jax.py:181-270): adds this step's gradients into the
@@ -196,9 +200,11 @@ int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_s
                      void* out, int32_t out_dtype, int64_t out_stride_b, int64_t out_stride_s,
                      int32_t B, int32_t Sq, int32_t H, int32_t D, ra_stream_t stream);
 
-/* delta[b,h,s] = sum_d g*out (ringattention_jax.py:218).  g, out: same dtype, same strides. */
-int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t stride_b, int64_t stride_s,
-                      float* delta, int64_t stat_stride_b, int64_t stat_stride_h,
+/* delta[b,h,s] = sum_d g*out (ringattention_jax.py:218).  g: the cotangent in `dtype`; out: the forward output,
+ * either rounded (out_dtype == dtype) or the un-rounded fp32 quotient (out_dtype RA_F32, from out_f32 of the last
+ * forward step: what the reference multiplies, :53).  Same element strides for both. */
+int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int32_t out_dtype, int64_t stride_b,
+                      int64_t stride_s, float* delta, int64_t stat_stride_b, int64_t stat_stride_h,
                       int32_t B, int32_t Sq, int32_t H, int32_t D, ra_stream_t stream);
 
 /* _blockwise_attention_bwd, ringattention_jax.py:181-270 (called at :76-84). */

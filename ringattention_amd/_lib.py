@@ -45,7 +45,7 @@ class RaAttnFwdParams(C.Structure):
         ("numerator", vp), ("num_stride_b", i64), ("num_stride_s", i64),
         ("denominator", vp), ("max_score", vp), ("stat_stride_b", i64), ("stat_stride_h", i64),
         ("mask", RaMask), ("impl", i32), ("carry_is_initial", i32),
-        ("out", vp), ("out_stride_b", i64), ("out_stride_s", i64),
+        ("out", vp), ("out_stride_b", i64), ("out_stride_s", i64), ("out_f32", vp),
     ]
 
 
@@ -118,7 +118,7 @@ SYMBOLS = {
     "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),
-    "ra_attn_bwd_delta": (C.c_int, [vp, vp, i32, i64, i64, vp, i64, i64, i32, i32, i32, i32, vp]),
+    "ra_attn_bwd_delta": (C.c_int, [vp, vp, i32, i32, i64, i64, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_bwd_block": (C.c_int, [C.POINTER(RaAttnBwdParams), vp]),
     "ra_attn_fwd_ring_step": (C.c_int, [C.POINTER(RaAttnFwdParams), C.POINTER(RaRingStep), vp]),
     "ra_attn_bwd_ring_step": (C.c_int, [C.POINTER(RaAttnBwdParams), C.POINTER(RaRingStep), vp]),

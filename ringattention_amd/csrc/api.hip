@@ -25,7 +25,7 @@ bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p);
 int carry_init(float*, int64_t, int64_t, float*, float*, int64_t, int64_t, int, int, int, int, hipStream_t);
 int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, void*, int, int64_t, int64_t, int,
              int, int, int, hipStream_t);
-int bwd_delta(const void*, const void*, int, int64_t, int64_t, float*, int64_t, int64_t, int, int, int, int,
+int bwd_delta(const void*, const void*, int, int, int64_t, int64_t, float*, int64_t, int64_t, int, int, int, int,
               hipStream_t);
 int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
 int keep_pack(const uint8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, uint64_t*, uint64_t*, uint8_t*, hipStream_t);
@@ -209,6 +209,7 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->q && p->k && p->v && p->denominator && p->max_score, RA_ERR_INVALID, "attn_fwd_block: null tensor");
   RA_REQUIRE(p->numerator || (p->carry_is_initial && p->out), RA_ERR_INVALID,
              "attn_fwd_block: the numerator may be null only when carry_is_initial is set and out is given");
+  RA_REQUIRE(!p->out_f32 || p->out, RA_ERR_INVALID, "attn_fwd_block: out_f32 goes with out");
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_fwd_block: dtype %d", p->dtype);
   RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_fwd_block: empty shape");
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_fwd_block: B and H must be <= 65535");
@@ -232,13 +233,15 @@ int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_s
                   out_stride_b, out_stride_s, B, Sq, H, D, (hipStream_t)stream);
 }
 
-int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int64_t stride_b, int64_t stride_s, float* delta,
-                      int64_t stat_stride_b, int64_t stat_stride_h, int32_t B, int32_t Sq, int32_t H, int32_t D,
-                      ra_stream_t stream) {
+int ra_attn_bwd_delta(const void* g, const void* out, int32_t dtype, int32_t out_dtype, int64_t stride_b,
+                      int64_t stride_s, float* delta, int64_t stat_stride_b, int64_t stat_stride_h, int32_t B,
+                      int32_t Sq, int32_t H, int32_t D, ra_stream_t stream) {
   RA_REQUIRE(g && out && delta, RA_ERR_INVALID, "bwd_delta: null pointer");
   RA_REQUIRE(dtype == RA_F32 || dtype == RA_BF16, RA_ERR_UNSUPPORTED, "bwd_delta: dtype %d", dtype);
+  RA_REQUIRE(out_dtype == dtype || out_dtype == RA_F32, RA_ERR_UNSUPPORTED,
+             "bwd_delta: out is either in the cotangent's dtype or fp32 (got %d)", out_dtype);
   RA_REQUIRE(B > 0 && Sq > 0 && H > 0 && D > 0 && B <= 65535, RA_ERR_INVALID, "bwd_delta: bad shape");
-  return bwd_delta(g, out, dtype, stride_b, stride_s, delta, stat_stride_b, stat_stride_h, B, Sq, H, D,
+  return bwd_delta(g, out, dtype, out_dtype, stride_b, stride_s, delta, stat_stride_b, stat_stride_h, B, Sq, H, D,
                    (hipStream_t)stream);
 }
 
@@ -307,6 +310,7 @@ int ra_attn_fwd_ring_step(const ra_attn_fwd_params* p, const ra_ring_step* ring,
   RA_REQUIRE(p->numerator || (ring->run & ~(ring->first & ring->last)) == 0, RA_ERR_INVALID,
              "%s: the numerator may be null only when every running device both starts and ends here", who);
   RA_REQUIRE(p->out || (ring->run & ring->last) == 0, RA_ERR_INVALID, "%s: a device writes out but out is null", who);
+  RA_REQUIRE(!p->out_f32 || p->out, RA_ERR_INVALID, "%s: out_f32 goes with out", who);
   ra_attn_fwd_params dev = *p;        // the shape one device sees: what the kernels' chunk grid has to fit
   dev.Sq = p->Sq / ring->n_dev; dev.Skv = p->Skv / ring->n_dev;
   RA_REQUIRE(attn_fwd_mfma_supported(&dev), RA_ERR_UNSUPPORTED,

@@ -23,6 +23,7 @@ struct GenericArgs {
   const int32_t* cache_idx;
   int carry_is_initial;
   void* out; int64_t out_sb, out_ss;             // forward, nullable: out = num / den instead of the numerator
+  float* out32;                                  // forward, nullable: the same quotient un-rounded, strides of out
   int dq_initial, dkv_initial;                   // backward: that accumulator holds zeros by definition
   void* dq_out; int64_t dqo_sb, dqo_ss;          // backward, nullable: the sum goes here in the primal dtype
   void* dk_out; void* dv_out; int64_t dkvo_sb, dkvo_ss;
@@ -193,9 +194,14 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs 
   if (valid) {
     const float nan = poison ? __builtin_nanf("") : 0.f;
     if (a.out) {                       // last step of the device: out = numerator / denominator (:52)
-      T* op = (T*)a.out + (int64_t)b * a.out_sb + (int64_t)rrow * a.out_ss + (int64_t)h * D;
+      const int64_t oo = (int64_t)b * a.out_sb + (int64_t)rrow * a.out_ss + (int64_t)h * D;
+      T* op = (T*)a.out + oo;
 #pragma unroll
       for (int d = 0; d < D; d++) store_from_f32<T>(op + d, poison ? nan : acc[d] / l);
+      if (a.out32) {                   // the residual of :53
+#pragma unroll
+        for (int d = 0; d < D; d++) a.out32[oo + d] = poison ? nan : acc[d] / l;
+      }
     } else {
 #pragma unroll
       for (int d = 0; d < D; d++) nump[d] = poison ? nan : acc[d];
@@ -386,8 +392,8 @@ __global__ void finalize_kernel(const float* num, int64_t num_sb, int64_t num_ss
   }
 }
 
-template <typename T>
-__global__ void delta_kernel(const T* g, const T* o, int64_t sb, int64_t ss, float* delta, int64_t st_sb,
+template <typename T, typename TO>
+__global__ void delta_kernel(const T* g, const TO* o, int64_t sb, int64_t ss, float* delta, int64_t st_sb,
                              int64_t st_sh, int Sq, int H, int D) {
   // one wavefront per (b, row, h)
   const int b = blockIdx.z, row = blockIdx.x;
@@ -395,7 +401,7 @@ __global__ void delta_kernel(const T* g, const T* o, int64_t sb, int64_t ss, flo
   for (int h = wave; h < H; h += nw) {
     const int64_t off = (int64_t)b * sb + (int64_t)row * ss + (int64_t)h * D;
     float s = 0.f;
-    for (int d = lane; d < D; d += 64) s = fmaf(load_f32<T>(g + off + d), load_f32<T>(o + off + d), s);
+    for (int d = lane; d < D; d += 64) s = fmaf(load_f32<T>(g + off + d), load_f32<TO>(o + off + d), s);
     for (int x = 32; x > 0; x >>= 1) s += __shfl_xor(s, x);
     if (lane == 0) delta[(int64_t)b * st_sb + (int64_t)h * st_sh + row] = s;   // :218
   }
@@ -560,7 +566,7 @@ static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
-  a.out = p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s;
+  a.out = p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   return a;
 }
 
@@ -643,15 +649,18 @@ int finalize(const float* num, int64_t num_sb, int64_t num_ss, const float* den,
   return RA_OK;
 }
 
-int bwd_delta(const void* g, const void* o, int dtype, int64_t sb, int64_t ss, float* delta, int64_t st_sb,
-              int64_t st_sh, int B, int Sq, int H, int D, hipStream_t s) {
+int bwd_delta(const void* g, const void* o, int dtype, int out_dtype, int64_t sb, int64_t ss, float* delta,
+              int64_t st_sb, int64_t st_sh, int B, int Sq, int H, int D, hipStream_t s) {
   dim3 grid(Sq, 1, B);
   if (dtype == RA_F32)
-    delta_kernel<float><<<grid, 256, 0, s>>>((const float*)g, (const float*)o, sb, ss, delta, st_sb, st_sh, Sq,
-                                            H, D);
+    delta_kernel<float, float><<<grid, 256, 0, s>>>((const float*)g, (const float*)o, sb, ss, delta, st_sb, st_sh,
+                                                   Sq, H, D);
+  else if (out_dtype == RA_F32)
+    delta_kernel<uint16_t, float><<<grid, 256, 0, s>>>((const uint16_t*)g, (const float*)o, sb, ss, delta, st_sb,
+                                                      st_sh, Sq, H, D);
   else
-    delta_kernel<uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)o, sb, ss, delta, st_sb,
-                                               st_sh, Sq, H, D);
+    delta_kernel<uint16_t, uint16_t><<<grid, 256, 0, s>>>((const uint16_t*)g, (const uint16_t*)o, sb, ss, delta,
+                                                         st_sb, st_sh, Sq, H, D);
   RA_CHECK_LAUNCH("bwd_delta");
   return RA_OK;
 }

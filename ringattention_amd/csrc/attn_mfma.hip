@@ -44,6 +44,7 @@ struct FwdArgs {
   const int32_t* cache_idx;
   int carry_is_initial;
   uint16_t* out; int64_t out_sb, out_ss;      // nullable: last step of the device, out = num / den instead of num
+  float* out32;                               // nullable, with out: the quotient before rounding, strides of out
   RingView ring;                              // n == 0: one device per launch
 };
 
@@ -199,6 +200,7 @@ __device__ __forceinline__ bool ring_bind(FwdArgs& a, MaskView& mv, int& qt) {
   const int64_t r0 = (int64_t)dev * (a.Sq / n);
   if (a.num) a.num += r0 * a.num_ss;
   a.out = ((a.ring.last >> dev) & 1ULL) ? a.out + r0 * a.out_ss : nullptr;
+  if (a.out32) a.out32 += r0 * a.out_ss;
   a.carry_is_initial = (int)((a.ring.first >> dev) & 1ULL);
   ring_bind_common(a, mv, dev, shard);
   qt -= dev * tiles_dev;
@@ -260,10 +262,11 @@ __device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t vo
 // point at row 0, head h): hand the accumulator on as bf16, or set it to the zeros it holds by definition.  In a ring
 // step most workgroups may do nothing else (a later shard meets few of a device's documents), so this is written
 // as a copy kernel: 16 bytes per lane, a row per 32 lanes, all eight requests of a lane in flight before the first
-// store.  den (nullable, one value per row): the forward's out = numerator / denominator.
+// store.  den (nullable, one value per row): the forward's out = numerator / denominator, which out32 (nullable, the
+// strides of out) takes un-rounded as well.
 template <int HD>
 __device__ __forceinline__ void pass_rows(const float* acc, float* acc_w, int64_t acc_ss, uint16_t* out, int64_t out_ss,
-                                          const float* den, int initial, int tid) {
+                                          const float* den, int initial, int tid, float* out32 = nullptr) {
   if (!out && !initial) return;
   constexpr int PER = 128 * (HD / 4) / 512;
   f32x4 t[PER];
@@ -285,8 +288,12 @@ __device__ __forceinline__ void pass_rows(const float* acc, float* acc_w, int64_
 #pragma unroll
       for (int e = 0; e < 4; e++) t[j][e] /= d[j];               // 0 / 0 = NaN when nothing ran at all, as :52
     }
-    if (out) store_bf16x4(out + (int64_t)r * out_ss + c4, t[j]);
-    else *(f32x4*)(acc_w + (int64_t)r * acc_ss + c4) = t[j];
+    if (out) {
+      store_bf16x4(out + (int64_t)r * out_ss + c4, t[j]);
+      if (out32) *(f32x4*)(out32 + (int64_t)r * out_ss + c4) = t[j];
+    } else {
+      *(f32x4*)(acc_w + (int64_t)r * acc_ss + c4) = t[j];
+    }
   }
 }
 
@@ -1277,7 +1284,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
       float* const np0 = a.num ? a.num + (int64_t)b * a.num_sb + (int64_t)q0 * a.num_ss + (int64_t)h * HD : nullptr;
       pass_rows<HD>(np0, np0, a.num_ss,
                 a.out ? a.out + (int64_t)b * a.out_sb + (int64_t)q0 * a.out_ss + (int64_t)h * HD : nullptr, a.out_ss,
-                a.out ? a.den + st0 : nullptr, a.carry_is_initial, tid);
+                a.out ? a.den + st0 : nullptr, a.carry_is_initial, tid,
+                (a.out && a.out32) ? a.out32 + (int64_t)b * a.out_sb + (int64_t)q0 * a.out_ss + (int64_t)h * HD : nullptr);
       if (a.carry_is_initial && tid < FBM) { a.den[st0 + tid] = 0.f; a.mx[st0 + tid] = RA_NEG_INF; }
     }
     return;
@@ -1689,7 +1697,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     __syncthreads();      // the producer's final factor
     const float fix = fixs[pair][lo];
     const float den_row = dens[pair][lo];
-    uint16_t* outp = a.out + (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
+    const int64_t ooff = (int64_t)b * a.out_sb + (int64_t)qrow * a.out_ss + (int64_t)h * HD + hi * 4;
+    uint16_t* outp = a.out + ooff;
 #pragma unroll
     for (int db = 0; db < NDB; db++)
 #pragma unroll
@@ -1701,6 +1710,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #pragma unroll
           for (int e = 0; e < 4; e++) t4[e] /= den_row;               // :52
           store_bf16x4(outp + db * 32 + g * 8, t4);
+          if (a.out32) *(f32x4*)(a.out32 + ooff + db * 32 + g * 8) = t4;   // the residual of :53
         } else {
           *(f32x4*)(nump + db * 32 + g * 8) = t4;
         }
@@ -1730,7 +1740,8 @@ bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p) {
          keep_ok(m) && (m.bias == nullptr || m.bias_stride_q == 0) && p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 &&
          p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0 &&
          aligned16(p->q) && aligned16(p->k) && aligned16(p->v) && aligned16(p->numerator) &&
-         (!p->out || (aligned16(p->out) && p->out_stride_s % 4 == 0 && p->out_stride_b % 4 == 0));
+         (!p->out || (aligned16(p->out) && p->out_stride_s % 4 == 0 && p->out_stride_b % 4 == 0)) &&
+         aligned16(p->out_f32);
 }
 
 static RingView ring_view(const ra_ring_step* r) {
@@ -1752,7 +1763,7 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* r, hipStream_
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
-  a.out = (uint16_t*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s;
+  a.out = (uint16_t*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool keep = p->mask.keep_bits_k != nullptr;      // packed form checked by attn_fwd_mfma_supported
   const long long nwg3 = (long long)(p->Sq / FBM) * p->H * p->B;

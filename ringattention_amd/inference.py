@@ -42,6 +42,10 @@ def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)      # :14
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)       # :31
     out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
+    # the residual `output` of :35 is the quotient before it is rounded to v's dtype (it meets the cotangent at :55)
+    out32 = None
+    if out.dtype != torch.float32:
+        out32 = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
     for dev in range(n):
         qs = slice(dev * q_len, (dev + 1) * q_len)
         mi.keep_row0 = dev * q_len                  # the device's rows of a mask that is sharded like q
@@ -51,8 +55,9 @@ def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
             ks = slice(k_blk * kv_len, (k_blk + 1) * kv_len)
             _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, dev, k_blk, None, None,
                                      None, q_len, kv_len, _mask_inputs=mi, _cfg=cfg, _carry_is_initial=(idx == 0),
-                                     _out=out[:, qs] if idx == n - 1 else None)
-    return out, (out, q, k, v, mi, cfg, n, den, mx)
+                                     _out=out[:, qs] if idx == n - 1 else None,
+                                     _out_f32=out32[:, qs] if out32 is not None and idx == n - 1 else None)
+    return out, (out if out32 is None else out32, q, k, v, mi, cfg, n, den, mx)
 
 
 def _bwd(res, g):

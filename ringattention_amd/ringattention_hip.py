@@ -149,6 +149,12 @@ class _Config:
         self.ring_launch = kw.get("ring_launch", "step")
         if self.ring_launch not in ("step", "device"):
             raise ValueError("ring_launch must be 'step' or 'device'")
+        # what the backward pass multiplies with the cotangent (:218): "fp32", the un-rounded output the reference
+        # keeps as a residual (:53; 4 bytes per element next to the returned output), or "rounded", the returned
+        # output itself (no extra memory; differs from the reference by the rounding of the output)
+        self.output_residual = kw.get("output_residual", "fp32")
+        if self.output_residual not in ("fp32", "rounded"):
+            raise ValueError("output_residual must be 'fp32' or 'rounded'")
         # policy / precision / prevent_cse only steer XLA rematerialisation: the kernels always recompute
         # the probabilities in the backward pass.
 
@@ -394,11 +400,12 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
                              causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
                              dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
                              precision=None, prevent_cse=True, cache_idx=None, _mask_inputs=None,
-                             _cfg=None, _carry_is_initial=False, _out=None, **extra):
+                             _cfg=None, _carry_is_initial=False, _out=None, _out_f32=None, **extra):
     """ringattention_jax.py:99-179.  ``carry`` = (numerator (B,Sq,H,D), denominator (B,H,Sq),
     max_score (B,H,Sq)), fp32, updated IN PLACE and returned.  With ``_out`` (B,Sq,H,D in q's dtype) the step is
     the last one of its device: out = numerator / denominator (:52) is written there instead of the numerator,
-    which may then be None if the carry is initial."""
+    which may then be None if the carry is initial; ``_out_f32`` (fp32, the strides of ``_out``) takes the same
+    quotient before it is rounded (the residual of :53)."""
     cfg = _cfg or _Config(dict(causal_block_size=causal_block_size, query_chunk_size=query_chunk_size,
                                key_chunk_size=key_chunk_size, deterministic=deterministic,
                                attn_pdrop=attn_pdrop, dtype=dtype, **extra))
@@ -426,6 +433,10 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
             raise ValueError("out must have the dtype of q")
         p.out = _out.data_ptr()
         p.out_stride_b, p.out_stride_s = _rows(_out)
+        if _out_f32 is not None:
+            if _out_f32.dtype != torch.float32 or _rows(_out_f32) != _rows(_out):
+                raise ValueError("out_f32 must be fp32 with the strides of out")
+            p.out_f32 = _out_f32.data_ptr()
     p.denominator, p.max_score = den.data_ptr(), mx.data_ptr()
     if den.stride() != mx.stride() or den.stride(2) != 1:
         raise ValueError("denominator / max_score must share strides and be dense in the last dim")
@@ -523,17 +534,18 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
 
 
 def _bwd_delta(g, output):
-    """dl_part of ringattention_jax.py:218: sum_d g * output, (B, H, Sq) fp32."""
+    """dl_part of ringattention_jax.py:218: sum_d g * output, (B, H, Sq) fp32.  ``output`` is the forward output in
+    g's dtype or, as in the reference (:53), un-rounded in fp32."""
     B, Sq, H, D = g.shape
-    if output.dtype != g.dtype:
+    if output.dtype not in (g.dtype, torch.float32):
         output = output.to(g.dtype)
     if _rows(output) != _rows(g):
         output = output.contiguous()
         g = g.contiguous()
     delta = torch.empty((B, H, Sq), dtype=torch.float32, device=g.device)
     sb, ss = _rows(g)
-    L.check(L.load().ra_attn_bwd_delta(g.data_ptr(), output.data_ptr(), _ra_dtype(g), sb, ss, delta.data_ptr(),
-                                       delta.stride(0), delta.stride(1), B, Sq, H, D, _stream()),
+    L.check(L.load().ra_attn_bwd_delta(g.data_ptr(), output.data_ptr(), _ra_dtype(g), _ra_dtype(output), sb, ss,
+                                       delta.data_ptr(), delta.stride(0), delta.stride(1), B, Sq, H, D, _stream()),
             "ra_attn_bwd_delta")
     return delta
 
@@ -607,6 +619,10 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)         # :23
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)          # :49
     out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
+    # the residual `output` of :53 is the quotient before it is rounded to v's dtype
+    out32 = None
+    if cfg.output_residual == "fp32" and out.dtype != torch.float32:
+        out32 = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
     plan = _ring_plan(cfg, mi, n, q_len, kv_len)
     # the numerator carry (:22) only exists between the steps of a device: its first step starts it (nothing is
     # read), its last step writes out = numerator / denominator (:52) instead
@@ -617,7 +633,7 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     for idx in range(n):                    # the scan of :29-51; all devices run a step side by side
         devs = [dev for dev in range(n) if idx in plan[dev]]
         if whole and devs:
-            whole = _fwd_ring_step(q, k, v, (num, den, mx), out, cfg, mi, n, idx, plan, devs)
+            whole = _fwd_ring_step(q, k, v, (num, den, mx), out, out32, cfg, mi, n, idx, plan, devs)
             if whole:
                 continue
         for dev in devs:
@@ -628,7 +644,8 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
             _blockwise_attention_fwd(q[:, qs], k[:, ks], v[:, ks], carry, q_start, k_start, None, None,
                                      cfg.cbs, cfg.qc, cfg.kc, _mask_inputs=mi, _cfg=cfg,
                                      _carry_is_initial=idx == min(plan[dev]), cache_idx=cache_idx,
-                                     _out=out[:, qs] if idx == max(plan[dev]) else None)
+                                     _out=out[:, qs] if idx == max(plan[dev]) else None,
+                                     _out_f32=out32[:, qs] if out32 is not None and idx == max(plan[dev]) else None)
     for dev in range(n):
         if not plan[dev]:                   # no tile runs for this device: 0 / 0
             qs = slice(dev * q_len, (dev + 1) * q_len)
@@ -636,8 +653,10 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
                                                                     device=q.device), den[:, :, qs], mx[:, :, qs])
             _carry_init(*carry)
             _finalize(carry[0], carry[1], out[:, qs])
+            if out32 is not None:
+                _finalize(carry[0], carry[1], out32[:, qs])
     del num
-    return out, (out, q, k, v, mi, cfg, n, den, mx)
+    return out, (out if out32 is None else out32, q, k, v, mi, cfg, n, den, mx)
 
 
 def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=128):
@@ -703,7 +722,7 @@ def _ring_bits(devs):
     return bits
 
 
-def _fwd_ring_step(q, k, v, carry, out, cfg, mi, n, idx, plan, devs):
+def _fwd_ring_step(q, k, v, carry, out, out32, cfg, mi, n, idx, plan, devs):
     """Scan step idx of every device in `devs` as one launch; False when the shape does not fit the MFMA kernels
     (nothing was launched then)."""
     num, den, mx = carry
@@ -723,6 +742,8 @@ def _fwd_ring_step(q, k, v, carry, out, cfg, mi, n, idx, plan, devs):
         p.num_stride_b, p.num_stride_s = q_total * H * D, H * D
     p.out = out.data_ptr()
     p.out_stride_b, p.out_stride_s = _rows(out)
+    if out32 is not None:
+        p.out_f32 = out32.data_ptr()
     p.denominator, p.max_score = den.data_ptr(), mx.data_ptr()
     p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
     p.mask = mi.fill(cfg, 0, 0, cfg.skip_masked_tiles)

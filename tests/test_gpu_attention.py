@@ -481,3 +481,65 @@ def test_mfma_refuses_chunk_sizes_whose_chunking_matters():
     ref_out, _ = oracle_fwd_bwd(q, k, v, None, None, None, None, 1, kw)
     out, _ = run_hip(q, k, v, None, None, None, None, 1, kw)
     assert_close(out, ref_out, torch.bfloat16, "out")
+
+
+# --- the residual `output` of the reference (ringattention_jax.py:53) is the quotient before it is rounded
+@pytest.mark.parametrize("impl,D,n,use_seg,mode", [("mfma", 128, 1, False, "step"), ("mfma", 64, 4, True, "step"),
+                                                   ("mfma", 128, 4, True, "device"), ("generic", 64, 2, False, "step")])
+def test_output_residual_is_the_unrounded_quotient(impl, D, n, use_seg, mode):
+    """bf16 inputs: the forward pass keeps numerator / denominator in fp32 next to the rounded output; rounding it
+    gives the returned output bit for bit, and it matches the oracle's fp32 output and residual product
+    delta = sum_d g * output (:218) to what the bf16 rounding of the probabilities inside the MFMA kernels leaves
+    (the generic kernels keep them in fp32)."""
+    from ringattention_amd import ringattention_hip as rh
+    from oracle import ringattention_oracle as O
+    from tests.util import oracle_kwargs
+    B, S, H = 1, 1024 if impl == "mfma" else 256, 2
+    qc = 128 if impl == "mfma" else 32
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=11, scale=1.0)
+    seg = packed_segment_ids(B, S, 300, seed=5) if use_seg else None      # documents shorter than a shard: rows
+    kw = kwargs(qc, qc, 1, dtype=torch.float32, impl=impl, ring_launch=mode)   # of later shards are passed through
+    with ra.ring_axis("sp", n):
+        out, res = rh._ring_attention_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None, None if seg is None else seg.to(DEV),
+                                          None, "sp", True, kw)
+    out32 = res[0]
+    assert out32.dtype == torch.float32 and out.dtype == torch.bfloat16
+    assert torch.equal(out32.to(torch.bfloat16).view(torch.int16), out.view(torch.int16))
+    ref_out, ref_res = O.ring_attention_fwd(q, k, v, None, seg, None, n, True, oracle_kwargs(kw))
+    tol = 3e-3 if impl == "mfma" else 1e-5
+    ma, rl = errors(out32, ref_res[0])
+    print("un-rounded output against the oracle's: max-abs %.2e, rel-L2 %.2e" % (ma, rl), flush=True)
+    assert rl <= tol, (ma, rl)
+    delta = rh._bwd_delta(do.to(DEV), out32)
+    ref_delta = (do.float() * ref_res[0].float()).sum(-1).permute(0, 2, 1)
+    ma, rl = errors(delta, ref_delta)
+    print("delta against the oracle's: max-abs %.2e, rel-L2 %.2e" % (ma, rl), flush=True)
+    assert rl <= tol, (ma, rl)
+    # the kernel's sum is the plain fp32 one of these very numbers
+    mine = (do.to(DEV).float() * out32).sum(-1).permute(0, 2, 1)
+    assert errors(delta, mine)[1] <= 1e-6
+    # the rounded output as residual stays available and is what it says
+    with ra.ring_axis("sp", n):
+        out_r, res_r = rh._ring_attention_fwd(q.to(DEV), k.to(DEV), v.to(DEV), None,
+                                              None if seg is None else seg.to(DEV), None, "sp", True,
+                                              dict(kw, output_residual="rounded"))
+    assert res_r[0].dtype == torch.bfloat16 and torch.equal(res_r[0].view(torch.int16), out.view(torch.int16))
+
+
+def test_gradients_with_the_fp32_residual_match_the_oracle_more_closely():
+    """What the residual is for: with output values of order one and a cotangent correlated with them, delta carries
+    the output's rounding error (2^-9 relative) into dS when it is taken from the rounded output."""
+    B, S, H, D = 1, 1024, 2, 128
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=1.0)
+    v = (v.float() + 4.0).to(torch.bfloat16)            # outputs near 4: large delta, visible rounding
+    do = torch.ones(B, S, H, D, dtype=torch.bfloat16)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, None, None, None, 1, kwargs(128, 128, 1))
+    errs = {}
+    for mode in ("fp32", "rounded"):
+        kw = kwargs(128, 128, 1, dtype=torch.float32, impl="mfma", output_residual=mode)
+        _, grads = run_hip(q, k, v, do, None, None, None, 1, kw)
+        errs[mode] = [errors(a, b)[1] for a, b in zip(grads, ref_grads)]
+        assert_close(grads[2], ref_grads[2], torch.bfloat16, "dv")
+    print("relative L2 error of dq, dk, dv:", errs, flush=True)
+    # a stress case (dP - delta cancels to a fortieth of either term): no fixed bar, the comparison is the point
+    assert errs["fp32"][0] < errs["rounded"][0] and errs["fp32"][1] < errs["rounded"][1]
