@@ -250,11 +250,13 @@ def bench_attention(args, ring, dropout=False):
             mx = torch.empty(B, H, S, dtype=torch.float32, device=dev)
             qd, kd, vd = q.detach(), k.detach(), v.detach()
             out = torch.empty_like(qd)
+            out32 = torch.empty(qd.shape, dtype=torch.float32, device=dev)      # the fp32 residual the step keeps
             fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (None, den, mx), 0, 0, None, None, 1, 512, 512,
-                                                      _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True, _out=out)
+                                                      _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True, _out=out,
+                                                      _out_f32=out32)
             fwd()            # under dropout the first call draws and packs the mask, which stays with mi
             kern["attn_fwd_ws_kernel"] = (_event_ms(fwd, 5), flops_fwd)
-            delta = rh._bwd_delta(do, out)
+            delta = rh._bwd_delta(do, out32)
             dq_o, dk_o, dv_o = (torch.empty_like(qd) for _ in range(3))
             for which, share in (("dkv", 8.0), ("dq", 2.0)):
                 cfg1 = rh._Config(dict(kw, bwd_only=which))
