@@ -294,6 +294,14 @@ def bench_attention(args, ring, dropout=False):
         if dropout:
             roof["traffic"] = None
             roof["mask_draw_and_pack_ms"] = round(mask_ms, 3)
+    if ring and not args.no_extras:
+        # clock and board power over whole steps: what tells a power-limited step from a stall-limited one
+        whole = _sclk_under_load(step)
+        if whole:
+            roof = {"bound": "mfma", "kernel": None, "achieved": round(value, 1), "peak": PEAK_BF16_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                    "scope": "whole step (six attention launches), FLOP of unmasked pairs",
+                    "power_w_under_load": whole.pop("power_w", None), "sclk_mhz_under_load": whole}
     cpu = cpu_baseline_attention() if not (args.no_cpu or dropout) else None
     del q, k, v, do
     return {
