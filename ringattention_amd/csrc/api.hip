@@ -22,6 +22,10 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* ring, hipStre
 int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* ring, int parts, hipStream_t s);   // parts: RA_BWD_PART_* bits
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p);
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p);
+int attn_fwd_f32(const ra_attn_fwd_params* p, hipStream_t s);                  // fp32 inputs on the matrix cores
+int attn_bwd_f32(const ra_attn_bwd_params* p, int parts, hipStream_t s);
+bool attn_fwd_f32_supported(const ra_attn_fwd_params* p);
+bool attn_bwd_f32_supported(const ra_attn_bwd_params* p);
 int carry_init(float*, int64_t, int64_t, float*, float*, int64_t, int64_t, int, int, int, int, hipStream_t);
 int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, void*, int, int64_t, int64_t, int,
              int, int, int, hipStream_t);
@@ -217,8 +221,9 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   hipStream_t s = (hipStream_t)stream;
   if (p->impl == RA_IMPL_GENERIC) return attn_fwd_generic(p, s);
   if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, nullptr, s);
+  if (attn_fwd_f32_supported(p)) return attn_fwd_f32(p, s);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
-             "attn_fwd_block: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128");
+             "attn_fwd_block: MFMA kernels need bf16 or fp32, head size 64 or 128, chunk sizes that are multiples of 128");
   return attn_fwd_generic(p, s);
 }
 
@@ -266,10 +271,11 @@ static int attn_bwd_block(const ra_attn_bwd_params* p, int parts, const char* wh
   const bool whole = dq_part && dkv_part;
   if (p->impl == RA_IMPL_GENERIC && whole) return attn_bwd_generic(p, s);
   if (p->impl != RA_IMPL_GENERIC && attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, nullptr, parts, s);
+  if (p->impl != RA_IMPL_GENERIC && attn_bwd_f32_supported(p)) return attn_bwd_f32(p, parts, s);
   RA_REQUIRE(whole, RA_ERR_UNSUPPORTED, "%s: one part alone is launched by the MFMA kernels only, which do not take "
              "this call (impl, dtype, head size or chunk sizes)", who);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
-             "%s: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128", who);
+             "%s: MFMA kernels need bf16 or fp32, head size 64 or 128, chunk sizes that are multiples of 128", who);
   return attn_bwd_generic(p, s);
 }
 

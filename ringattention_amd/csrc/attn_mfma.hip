@@ -75,34 +75,6 @@ template <int HD> __device__ __forceinline__ int swz(int r) {
   return HD == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
 
-// Hull [first, last+1) of the 64-position tiles, among the n tiles starting at global tile gt0, whose
-// segment-id range meets [lo, hi] (ids from ra_segment_tile_ranges).  Conservative: a tile outside the
-// hull holds no key (query) of a segment present in the rows at hand; tiles inside may still be fully
-// masked.  Every thread of the workgroup must call it; hull2 points at two ints of LDS.
-__device__ __forceinline__ void seg_tile_hull(const MaskView& mv, int b, int gt0, int n, int lo, int hi, int* hull2,
-                                              int tid, int nthreads, int& first, int& last) {
-  if (tid == 0) { hull2[0] = n; hull2[1] = 0; }
-  __syncthreads();
-  const int32_t* mm = mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2;
-  for (int t = tid; t < n; t += nthreads) {
-    const int g = min(gt0 + t, mv.seg_tiles - 1);
-    const int mn = mm[2 * g], mx = mm[2 * g + 1];
-    if (mx >= lo && mn <= hi) { atomicMin(&hull2[0], t); atomicMax(&hull2[1], t + 1); }
-  }
-  __syncthreads();
-  first = hull2[0]; last = hull2[1];
-  if (last < first) { first = 0; last = 0; }
-}
-// segment-id range of the rows [g0, g0 + rows) (global positions, multiples of 64)
-__device__ __forceinline__ void seg_rows_range(const MaskView& mv, int b, int g0, int rows, int& lo, int& hi) {
-  const int32_t* mm = mv.seg_mm + (int64_t)(mv.seg_sb ? b : 0) * mv.seg_tiles * 2;
-  lo = 0x7fffffff; hi = -0x7fffffff - 1;
-  for (int t = g0 / RA_SEG_TILE; t < (g0 + rows) / RA_SEG_TILE; t++) {
-    const int g = min(t, mv.seg_tiles - 1);
-    lo = min(lo, mm[2 * g]); hi = max(hi, mm[2 * g + 1]);
-  }
-}
-
 // ---- boolean keep mask in packed form (ra_keep_pack): 64-bit words and a per-64x64-tile summary
 // (0 none kept, 1 mixed, 2 all kept).  Hull of the key tiles [gkt0, gkt0 + n) that hold a kept pair for
 // any of the nrows summary rows starting at qt64 (every thread of the workgroup must call it).

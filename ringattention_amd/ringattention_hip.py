@@ -629,7 +629,7 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     num = None
     if any(len(steps) > 1 for steps in plan.values()):
         num = torch.empty((B, q_total, H, D), dtype=torch.float32, device=q.device)
-    whole = _ring_step_launches(cfg, mi, n)
+    whole = _ring_step_launches(cfg, mi, n) and q.dtype == torch.bfloat16      # those entry points take bf16 only
     for idx in range(n):                    # the scan of :29-51; all devices run a step side by side
         devs = [dev for dev in range(n) if idx in plan[dev]]
         if whole and devs:
@@ -669,7 +669,7 @@ def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=
     long as its row has an unmasked key, which is what skip_masked_tiles already asks for; so both chunkings sum
     over the same pairs.  Without a causal block size every chunk pair runs.  The slices are not clamped when the
     segment ids cover every position, there is no dropout here, and a per-row bias takes the generic kernels."""
-    if cfg.impl == L.RA_IMPL_GENERIC or q.dtype != torch.bfloat16 or q.shape[3] not in (64, 128):
+    if cfg.impl == L.RA_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float32) or q.shape[3] not in (64, 128):
         return
     if cfg.qc % grid == 0 and cfg.kc % grid == 0:
         return
@@ -784,7 +784,7 @@ def _ring_attention_bwd(res, g):
     if any(len(steps) > 1 for steps in shard_steps.values()):
         dk = torch.empty((B, kv_total, H, D), dtype=torch.float32, device=q.device)
         dv = torch.empty((B, kv_total, H, D), dtype=torch.float32, device=q.device)
-    whole = _ring_step_launches(cfg, mi, n)
+    whole = _ring_step_launches(cfg, mi, n) and q.dtype == torch.bfloat16      # those entry points take bf16 only
     for idx in range(n):                    # the scan of :65-88
         devs = [dev for dev in range(n) if idx in plan[dev]]
         if whole and devs:

@@ -287,7 +287,8 @@ def test_frozen_vectors(dtype):
 
 
 @pytest.mark.parametrize("impl,dtype,S,D,qc", [("generic", torch.float32, 128, 32, 16), ("generic", torch.bfloat16, 128, 64, 32),
-                                                ("mfma", torch.bfloat16, 1024, 128, 256)])
+                                                ("mfma", torch.bfloat16, 1024, 128, 256),
+                                                ("mfma", torch.float32, 512, 64, 128), ("mfma", torch.float32, 512, 128, 256)])
 def test_first_and_last_step_modes_give_the_bits_of_the_separate_passes(impl, dtype, S, D, qc):
     """Two ring steps of one device (own shard, then the shard before it), once with explicit fp32 carries, a
     finalize pass and a cast, once with the first step starting the carries (uninitialised memory behind them) and
@@ -543,3 +544,58 @@ def test_gradients_with_the_fp32_residual_match_the_oracle_more_closely():
     print("relative L2 error of dq, dk, dv:", errs, flush=True)
     # a stress case (dP - delta cancels to a fortieth of either term): no fixed bar, the comparison is the point
     assert errs["fp32"][0] < errs["rounded"][0] and errs["fp32"][1] < errs["rounded"][1]
+
+
+# --- fp32 inputs on the matrix cores (v_mfma_f32_32x32x2_f32): head size 64 or 128, chunk sizes on the 128-grid
+F32_MFMA_CASES = [
+    # B, S, H, D, qc, kc, cbs, n, bias, seg
+    (1, 2048, 8, 64, 512, 512, 1, 1, True, True),          # the reference's CPU-runnable configuration
+    (2, 512, 2, 128, 128, 128, 1, 1, False, False),
+    (1, 1024, 3, 128, 256, 128, 1, 2, True, True),
+    (2, 1024, 2, 64, 128, 256, 1, 4, True, False),
+    (1, 1024, 2, 128, 128, 128, None, 2, False, True),
+    (1, 1024, 2, 64, 128, 128, None, 1, True, False),
+    (1, 2048, 2, 128, 256, 256, 64, 2, False, True),
+    (1, 2048, 1, 64, 128, 128, 512, 4, True, True),
+    (1, 1024, 2, 128, 64, 64, 1, 2, False, True),           # off the grid: served as 128 x 128 chunks
+]
+
+
+@pytest.mark.parametrize("case", F32_MFMA_CASES)
+def test_fp32_mfma_kernels_match_oracle(case):
+    B, S, H, D, qc, kc, cbs, n, use_bias, use_seg = case
+    impl = "mfma" if qc % 128 == 0 and kc % 128 == 0 else "auto"
+    check_case(B, S, H, D, qc, kc, cbs, n, use_bias, use_seg, torch.float32, impl=impl, seg_mean=200)
+
+
+@pytest.mark.parametrize("D,n,cbs,use_seg,use_bias", [(128, 1, 1, False, False), (64, 2, 1, True, True),
+                                                      (128, 4, 256, True, False), (64, 1, None, False, True)])
+def test_fp32_mfma_kernels_agree_with_the_vector_kernels(D, n, cbs, use_seg, use_bias):
+    """Same inputs through the fp32 matrix-core kernels and the one-row-per-lane kernels: both sum in fp32, so they
+    agree to a few ulp of the largest term."""
+    B, S, H = 2, 1024, 2
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=3, scale=1.0)
+    g = torch.Generator().manual_seed(9)
+    bias = torch.randn(B, H, 1, S, generator=g) if use_bias else None
+    seg = packed_segment_ids(B, S, 150, seed=4) if use_seg else None
+    res = {}
+    for impl in ("mfma", "generic"):
+        out, grads = run_hip(q, k, v, do, bias, seg, None, n, kwargs(128, 128, cbs, dtype=torch.float32, impl=impl))
+        res[impl] = (out,) + grads
+    for name, a, b in zip(("out", "dq", "dk", "dv"), res["mfma"], res["generic"]):
+        ma, rl = errors(a, b)
+        assert ma <= 2e-5 and rl <= 1e-5, (name, ma, rl)
+
+
+def test_fp32_mfma_kernels_refuse_what_they_do_not_take():
+    """A per-row bias and head sizes other than 64 / 128 stay with the vector kernels; asking for the matrix-core
+    kernels by name then is an error, not a silent fallback."""
+    q, k, v, _ = make_qkv(1, 256, 1, 32, dtype=torch.float32, seed=1)
+    with pytest.raises(NotImplementedError):
+        run_hip(q, k, v, None, None, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32, impl="mfma"))
+    q, k, v, _ = make_qkv(1, 256, 1, 64, dtype=torch.float32, seed=1)
+    bias = torch.zeros(1, 1, 128, 256)
+    with pytest.raises(NotImplementedError):
+        run_hip(q, k, v, None, bias, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32, impl="mfma"))
+    out, _ = run_hip(q, k, v, None, bias, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32))   # auto: served
+    assert torch.isfinite(out).all()
