@@ -20,6 +20,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6      # MI355X dense bf16 MFMA
+PEAK_F32_TFLOPS = 157.3        # MI355X dense fp32 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 
 
@@ -204,9 +205,13 @@ def bench_attention(args, ring, dropout=False):
     # other choices give the logits a standard deviation of 0.09 (q, k scaled D^-0.25) or 1 (unscaled q, k)
     qk_scale = {"baseline": D ** -0.5, "d-quarter": D ** -0.25, "unit": 1.0}[args.inputs]
     v_scale = D ** -0.5 if args.inputs == "baseline" else 1.0
-    mk = lambda sc: (torch.randn(B, S, H, D, device=dev, generator=g) * sc).to(torch.bfloat16)
+    fp32 = getattr(args, "dtype", "bf16") == "fp32"
+    tdt = torch.float32 if fp32 else torch.bfloat16
+    peak = PEAK_F32_TFLOPS if fp32 else PEAK_BF16_TFLOPS
+    sfx = "_f32_kernel" if fp32 else "_ws_kernel"
+    mk = lambda sc: (torch.randn(B, S, H, D, device=dev, generator=g) * sc).to(tdt)
     q, k, v = mk(qk_scale).requires_grad_(True), mk(qk_scale).requires_grad_(True), mk(v_scale).requires_grad_(True)
-    do = torch.randn(B, S, H, D, device=dev, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, S, H, D, device=dev, generator=g).to(tdt)
     bias = seg = None
     pairs = S * (S + 1) / 2
     if ring:
@@ -214,6 +219,8 @@ def bench_attention(args, ring, dropout=False):
         seg, lens = _packed_segments(S, 4096, 0, dev)
         pairs = float(sum(l * (l + 1) / 2 for l in lens))
     kw = _kwargs(512, 512, 1)
+    if fp32:
+        kw["dtype"] = torch.float32
     pdrop = 0.1
     if dropout:
         # attention dropout: a fresh seed every step, so drawing and packing the mask is part of the step; only the
@@ -250,13 +257,14 @@ def bench_attention(args, ring, dropout=False):
             mx = torch.empty(B, H, S, dtype=torch.float32, device=dev)
             qd, kd, vd = q.detach(), k.detach(), v.detach()
             out = torch.empty_like(qd)
-            out32 = torch.empty(qd.shape, dtype=torch.float32, device=dev)      # the fp32 residual the step keeps
+            # the fp32 residual the step keeps next to a bf16 output
+            out32 = torch.empty(qd.shape, dtype=torch.float32, device=dev) if not fp32 else None
             fwd = lambda: rh._blockwise_attention_fwd(qd, kd, vd, (None, den, mx), 0, 0, None, None, 1, 512, 512,
                                                       _mask_inputs=mi, _cfg=cfg, _carry_is_initial=True, _out=out,
                                                       _out_f32=out32)
             fwd()            # under dropout the first call draws and packs the mask, which stays with mi
-            kern["attn_fwd_ws_kernel"] = (_event_ms(fwd, 5), flops_fwd)
-            delta = rh._bwd_delta(do, out32)
+            kern["attn_fwd" + sfx] = (_event_ms(fwd, 5), flops_fwd)
+            delta = rh._bwd_delta(do, out32 if out32 is not None else out)
             dq_o, dk_o, dv_o = (torch.empty_like(qd) for _ in range(3))
             for which, share in (("dkv", 8.0), ("dq", 2.0)):
                 cfg1 = rh._Config(dict(kw, bwd_only=which))
@@ -264,7 +272,7 @@ def bench_attention(args, ring, dropout=False):
                                                          None, 1, 512, 512, _mask_inputs=mi, _cfg=cfg1, _delta=delta,
                                                          _grads_initial=L.RA_GRAD_INIT_DQ | L.RA_GRAD_INIT_DKV,
                                                          _dq_out=dq_o, _dkv_out=(dk_o, dv_o))
-                kern["attn_bwd_%s_ws_kernel" % which] = (_event_ms(bw, 5), share * D * pairs * B * H)
+                kern["attn_bwd_%s%s" % (which, sfx)] = (_event_ms(bw, 5), share * D * pairs * B * H)
                 if which == "dkv" and not (args.no_extras or dropout):
                     sclk = _sclk_under_load(bw)       # the clock the dominant kernel actually runs at
             if dropout:
@@ -277,8 +285,8 @@ def bench_attention(args, ring, dropout=False):
         dom = max(kern, key=lambda n_: kern[n_][0])
         dms, dfl = kern[dom]
         ach = dfl / (dms * 1e-3) / 1e12
-        roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
+        roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": peak,
+                "unit": "TFLOP/s", "frac": round(ach / peak, 4),
                 "traffic": traffic.get(dom) if S == 32768 and args.inputs == "baseline" else None,
                 "traffic_source": "profiles/" + TRAFFIC_PROFILE if traffic.get(dom) else None,
                 "mfma_util_pmc": ({"kernel": util.get(dom), "step": util.get("attn32k_step"),
@@ -290,7 +298,7 @@ def bench_attention(args, ring, dropout=False):
             # the published peak assumes 2400 MHz; what the same matrix pipes can do at the clock the kernel runs at
             roof["power_w_under_load"] = sclk.pop("power_w", None)
             roof["sclk_mhz_under_load"] = sclk
-            roof["frac_of_peak_at_sclk"] = round(ach / (PEAK_BF16_TFLOPS * sclk["median"] / 2400.0), 4)
+            roof["frac_of_peak_at_sclk"] = round(ach / (peak * sclk["median"] / 2400.0), 4)
         if dropout:
             roof["traffic"] = None
             roof["mask_draw_and_pack_ms"] = round(mask_ms, 3)
@@ -298,15 +306,16 @@ def bench_attention(args, ring, dropout=False):
         # clock and board power over whole steps: what tells a power-limited step from a stall-limited one
         whole = _sclk_under_load(step)
         if whole:
-            roof = {"bound": "mfma", "kernel": None, "achieved": round(value, 1), "peak": PEAK_BF16_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None,
+            roof = {"bound": "mfma", "kernel": None, "achieved": round(value, 1), "peak": peak,
+                    "unit": "TFLOP/s", "frac": round(value / peak, 4), "traffic": None,
                     "scope": "whole step (six attention launches), FLOP of unmasked pairs",
                     "power_w_under_load": whole.pop("power_w", None), "sclk_mhz_under_load": whole}
     cpu = cpu_baseline_attention() if not (args.no_cpu or dropout) else None
     del q, k, v, do
+    pct_key = "pct_f32_mfma_peak" if fp32 else "pct_bf16_mfma_peak"
     return {
         "metric": "attn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
-        "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+        "dtype": "f32" if fp32 else "bf16", pct_key: round(100 * value / peak, 2),
         "config": {"workload": name, "B": B, "H": H, "S": S, "D": D, "causal_block_size": 1,
                    "query_chunk_size": 512, "key_chunk_size": 512, "virtual_ring": n,
                    "segment_ids": bool(ring), "bias": bool(ring), "attn_pdrop": pdrop if dropout else 0.0,
@@ -656,6 +665,9 @@ def main():
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
                     help="attention workloads: head size (the number of heads follows, H * D = 4096)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"],
+                    help="attention workloads: dtype of q, k, v (fp32 runs on v_mfma_f32_32x32x2_f32; its roofline is the "
+                         "fp32 matrix peak)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--ffn-policy", default="nothing_saveable", choices=["nothing_saveable", "save_preactivations"],
                     help="ffn workload: what blockwise_feedforward keeps for the backward pass (default: the "
@@ -711,7 +723,7 @@ def main():
             "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": r["dtype"], "data": "synthetic", "config": r["config"],
             "roofline": r["roofline"], "cpu_baseline": r["cpu_baseline"]}
-    for extra in ("pct_bf16_mfma_peak", "pct_hbm_peak"):
+    for extra in ("pct_bf16_mfma_peak", "pct_f32_mfma_peak", "pct_hbm_peak"):
         if extra in r:
             line[extra] = r[extra]
     line.update(extras)
