@@ -311,3 +311,23 @@ def test_float32_logits_false_is_accepted():
     # chunk step): it sits this far from its own fp32 run, so the bar is looser than the fp32-logit one
     ma, rl = errors(a, ref)
     assert ma <= 6e-2 and rl <= 3e-2, (ma, rl)
+
+
+def test_fp32_16k_ring4_matches_oracle():
+    """fp32 q, k, v on the matrix-core kernels at B1 H2 S16384 D128, ring of 4, packed documents and a bias, chunks
+    512/512: the fp32 bar (max-abs 1e-4, relative L2 1e-2) at a length where every workgroup streams hundreds of
+    tiles."""
+    B, S, H, D, n = 1, 16384, 2, 128, 4
+    print("oracle parity, fp32 16k ring 4", flush=True)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=44, scale=D ** -0.25)
+    seg = packed_segment_ids(B, S, 3000, seed=45)
+    bias = torch.randn(1, 1, 1, S, generator=torch.Generator().manual_seed(46))
+    kw = kwargs(512, 512, 1, dtype=torch.float32, impl="mfma")
+    t0 = time.time()
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    secs = time.time() - t0
+    out, grads = _hip(q, k, v, do, bias, seg, n, kw)
+    rows = [("out",) + assert_close(out, ref_out, torch.float32, "fp32 16k out")]
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        rows.append((name,) + assert_close(a, b, torch.float32, "fp32 16k " + name))
+    print("fp32 16k ring 4: oracle %.1f s;" % secs, "; ".join("%s max-abs %.2e rel-L2 %.2e" % r for r in rows), flush=True)
