@@ -184,7 +184,7 @@ def _packed_segments(S, mean_len, seed, device):
 
 
 # --------------------------------------------------------------------------- attention workloads
-def bench_attention(args, ring, dropout=False):
+def bench_attention(args, ring, dropout=False, c1=False):
     import torch
     import ringattention_amd as ra
     from ringattention_amd import ringattention_hip as rh
@@ -198,6 +198,10 @@ def bench_attention(args, ring, dropout=False):
         S, n, name = 32768, 1, "attn32k"
     if dropout:
         name = "dropout32k"
+    if c1:
+        # the reference's own CPU-runnable configuration: B1 H8 S2048 D64 fp32, N(0,1) inputs, a zero bias, one document
+        S, n, name, D, H = 2048, 1, "c1", 64, 8
+        args = argparse.Namespace(**dict(vars(args), dtype="fp32", inputs="unit"))
     if args.seq_len:
         S = args.seq_len
     g = torch.Generator(device=dev).manual_seed(0)
@@ -218,6 +222,9 @@ def bench_attention(args, ring, dropout=False):
         bias = torch.randn(1, 1, 1, S, device=dev, generator=g)
         seg, lens = _packed_segments(S, 4096, 0, dev)
         pairs = float(sum(l * (l + 1) / 2 for l in lens))
+    if c1:
+        bias = torch.zeros(1, 1, 1, S, device=dev)
+        seg = torch.zeros(1, S, dtype=torch.int32, device=dev)
     kw = _kwargs(512, 512, 1)
     if fp32:
         kw["dtype"] = torch.float32
@@ -246,7 +253,7 @@ def bench_attention(args, ring, dropout=False):
     roof = None
     kern = {}
     sclk = None
-    if not ring:
+    if not ring and not c1:
         with torch.no_grad():
             cfg = rh._Config(kw)
             mi = rh._MaskInputs(cfg, None, None, None, B, q.device, S)
@@ -310,7 +317,15 @@ def bench_attention(args, ring, dropout=False):
                     "unit": "TFLOP/s", "frac": round(value / peak, 4), "traffic": None,
                     "scope": "whole step (six attention launches), FLOP of unmasked pairs",
                     "power_w_under_load": whole.pop("power_w", None), "sclk_mhz_under_load": whole}
-    cpu = cpu_baseline_attention() if not (args.no_cpu or dropout) else None
+    if c1:
+        roof = {"bound": "mfma", "kernel": None, "achieved": round(value, 2), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(value / peak, 4), "traffic": None,
+                "scope": "whole step: 128 forward and dQ workgroups on 256 CUs, launch-bound"}
+    cpu = None
+    if c1 and not args.no_cpu:
+        cpu = cpu_baseline_c1(q.detach().cpu(), k.detach().cpu(), v.detach().cpu(), do.cpu(), kw)
+    elif not (args.no_cpu or dropout):
+        cpu = cpu_baseline_attention()
     del q, k, v, do
     pct_key = "pct_f32_mfma_peak" if fp32 else "pct_bf16_mfma_peak"
     return {
@@ -318,13 +333,32 @@ def bench_attention(args, ring, dropout=False):
         "dtype": "f32" if fp32 else "bf16", pct_key: round(100 * value / peak, 2),
         "config": {"workload": name, "B": B, "H": H, "S": S, "D": D, "causal_block_size": 1,
                    "query_chunk_size": 512, "key_chunk_size": 512, "virtual_ring": n,
-                   "segment_ids": bool(ring), "bias": bool(ring), "attn_pdrop": pdrop if dropout else 0.0,
+                   "segment_ids": seg is not None, "bias": bias is not None, "attn_pdrop": pdrop if dropout else 0.0,
                    "inputs": {"baseline": "q, k, v ~ N(0,1)/sqrt(D), dO ~ N(0,1)",
                               "d-quarter": "q, k ~ N(0,1) * D^-0.25, v, dO ~ N(0,1)",
                               "unit": "q, k, v, dO ~ N(0,1)"}[args.inputs],
                    "flop_convention": "4*D fwd + 10*D bwd per unmasked (q,k) pair per head"},
         "roofline": roof, "cpu_baseline": cpu,
     }
+
+
+def cpu_baseline_c1(q, k, v, do, kw):
+    """The CPU oracle on the whole of the reference's CPU-runnable configuration, forward + backward."""
+    import torch
+    from oracle import ringattention_oracle as O
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    S, H, D = q.shape[1], q.shape[2], q.shape[3]
+    bias, seg = torch.zeros(1, 1, 1, S), torch.zeros(1, S, dtype=torch.int32)
+    reps, t0 = 0, time.perf_counter()
+    while reps < 3 or time.perf_counter() - t0 < 10.0:
+        out, res = O.ring_attention_fwd(q, k, v, bias, seg, None, 1, True, kw)
+        O.ring_attention_bwd(1, True, kw, res, do)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    flops = 14.0 * D * (S * (S + 1) / 2) * H
+    return {"value": round(flops / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "the whole configuration, fwd+bwd, %d repetitions of %.3f s" % (reps, dt)}
 
 
 def cpu_baseline_attention():
@@ -661,7 +695,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default=None, choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
-                                                              "dropout32k"])
+                                                              "dropout32k", "c1"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
                     help="attention workloads: head size (the number of heads follows, H * D = 4096)")
@@ -693,8 +727,9 @@ def main():
     if args.workload is None:
         args.workload = "attn32k"
     extras = {}
-    if args.workload in ("attn32k", "ring131k", "dropout32k"):
-        r = bench_attention(args, ring=(args.workload == "ring131k"), dropout=(args.workload == "dropout32k"))
+    if args.workload in ("attn32k", "ring131k", "dropout32k", "c1"):
+        r = bench_attention(args, ring=(args.workload == "ring131k"), dropout=(args.workload == "dropout32k"),
+                            c1=(args.workload == "c1"))
         if whole_metric:
             others = []
             for inputs in ("d-quarter", "unit"):
