@@ -111,8 +111,8 @@ __device__ __forceinline__ void f32_pass_rows(const float* acc, float* acc_w, in
   }
 
 // key range [k_base, k_base + 64 ntiles) of the shard that a 128-row query tile has to visit (forward, dQ)
-template <bool HAS_SEG>
-__device__ __forceinline__ void f32_key_range(const MaskView& mv, int b, int q0, int Skv, int tid, int* hull2,
+template <bool HAS_SEG, bool HAS_KEEP>
+__device__ __forceinline__ void f32_key_range(const MaskView& mv, int b, int h, int q0, int Skv, int tid, int* hull2,
                                               int& k_base, int& ntiles) {
   const int qi = q0 / mv.qc;
   int kend = mv.run_prefix_keys(qi, Skv);
@@ -132,6 +132,13 @@ __device__ __forceinline__ void f32_key_range(const MaskView& mv, int b, int q0,
     k_base = t_first * XBN;
     ntiles = t_last - t_first;
   }
+  if (HAS_KEEP && mv.skip_tiles && ntiles > 0) {     // key tiles that hold an attended pair for any of the 128 rows
+    int t_first, t_last;
+    keep_ktile_hull(mv, b, h, (mv.keep_q0 + q0) / 64, XBM / 64, (gk0_shard + k_base - mv.keep_k0) / 64, ntiles, hull2, tid, 256,
+                    t_first, t_last);
+    k_base += t_first * XBN;
+    ntiles = t_last - t_first;
+  }
 }
 
 // segment id and (clamped) bias of local key kj, as the reference slices them (:279-295)
@@ -149,7 +156,7 @@ __device__ __forceinline__ void f32_key_info(const MaskView& mv, int b, int h, i
 }
 
 // ------------------------------------------------------------------ forward
-template <int HD, bool HAS_SEG, bool HAS_BIAS>
+template <int HD, bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>   // HAS_KEEP: where(keep, logit, mask_min), packed mask
 __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) float Ks[XBN * (HD + 4)];
   __shared__ __attribute__((aligned(16))) float Vs[XBN * (HD + 4)];
@@ -166,7 +173,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
   qt = nqt - 1 - qt;                       // latest query tiles (most keys under a causal mask) first
   const int q0 = qt * XBM, qrow = q0 + wave * 32 + lo;
   int k_base, ntiles;
-  f32_key_range<HAS_SEG>(mv, b, q0, a.Skv, tid, hull2, k_base, ntiles);
+  f32_key_range<HAS_SEG, HAS_KEEP>(mv, b, h, q0, a.Skv, tid, hull2, k_base, ntiles);
   const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + q0;
   if (ntiles == 0) {                       // no key tile runs for these rows: the carry stays as it is
     if (a.carry_is_initial || a.out) {
@@ -202,6 +209,15 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
     const int idx = clamp_seg_index(((long long)mv.q_start + q0 / mv.qc) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
     seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
   }
+  // packed boolean mask: one 64-bit word per query row and key tile (bit i = key i of the tile is attended)
+  const uint64_t* kw_ptr = nullptr;
+  uint64_t kw = 0, kw_nxt = 0;
+  if (HAS_KEEP) {
+    kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
+             (int64_t)((gk0 - mv.keep_k0) / 64) * mv.keep_Q + mv.keep_q0 + qrow;
+    kw_nxt = kw_ptr[0];
+  }
+  (void)kw;
   // O^T accumulators: block db, row i is head dimension NDB i + db; this lane's query is the column
   f32x16 acc[NDB];
   float* nump = a.num ? a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD : nullptr;
@@ -228,6 +244,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
   if (tid < XBN) { seg_ks[tid] = s_seg; bias_ks[tid] = s_bias; }
   __syncthreads();
   for (int t = 0; t < ntiles; t++) {
+    if (HAS_KEEP) { kw = kw_nxt; kw_nxt = kw_ptr[(int64_t)min(t + 1, ntiles - 1) * mv.keep_Q]; }
     if (t + 1 < ntiles) {                  // the next tile travels while this one is worked on
       RA_F32_LOAD(kg, vg, (t + 1) * XBN, a.kv_ss)
       if (tid < XBN) f32_key_info<HAS_SEG, HAS_BIAS>(mv, b, h, k_base + (t + 1) * XBN + tid, s_seg, s_bias);
@@ -249,12 +266,15 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
       }
       // logits of this lane's query against its 16 keys of the block (:134-136, :272-322)
       const int gkb = gk0 + t * XBN + blk * 32;
+      const uint32_t kwb = HAS_KEEP ? (uint32_t)(kw >> (blk * 32)) >> (4 * hi) : 0u;   // this lane's keys of the block
+      (void)kwb;
       float x[16], mloc = RA_NEG_INF;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int kr = blk * 32 + crow(r, hi);
         bool masked = gkb + crow(r, hi) >= klim;
         if (HAS_SEG) masked = masked || seg_ks[kr] != seg_q;
+        if (HAS_KEEP) masked = masked || !((kwb >> (8 * (r >> 2) + (r & 3))) & 1u);   /* ringattention_inference.py:22 */
         const float add = masked ? mv.mask_min : (HAS_BIAS ? bias_ks[kr] : 0.f);
         x[r] = (s0[r] + s1[r]) * rscale + add;
         mloc = fmaxf(mloc, x[r]);
@@ -316,7 +336,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
 }
 
 // ------------------------------------------------------------------ backward, dQ (query-stationary)
-template <int HD, bool HAS_SEG, bool HAS_BIAS>
+template <int HD, bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) float Ks[XBN * (HD + 4)];
   __shared__ __attribute__((aligned(16))) float Vs[XBN * (HD + 4)];
@@ -333,7 +353,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
   qt = nqt - 1 - qt;
   const int q0 = qt * XBM, qrow = q0 + wave * 32 + lo;
   int k_base, ntiles;
-  f32_key_range<HAS_SEG>(mv, b, q0, a.Skv, tid, hull2, k_base, ntiles);
+  f32_key_range<HAS_SEG, HAS_KEEP>(mv, b, h, q0, a.Skv, tid, hull2, k_base, ntiles);
   if (ntiles == 0) {                       // nothing to add to dq
     float* const dq0 = a.dq ? a.dq + (int64_t)b * a.dq_sb + (int64_t)q0 * a.dq_ss + (int64_t)h * HD : nullptr;
     f32_pass_rows<HD>(dq0, dq0, a.dq_ss,
@@ -364,6 +384,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
     const int idx = clamp_seg_index(((long long)mv.q_start + q0 / mv.qc) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
     seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
   }
+  // packed boolean mask: one 64-bit word per query row and key tile (bit i = key i of the tile is attended)
+  const uint64_t* kw_ptr = nullptr;
+  uint64_t kw = 0, kw_nxt = 0;
+  if (HAS_KEEP) {
+    kw_ptr = mv.kbits_k + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
+             (int64_t)((gk0 - mv.keep_k0) / 64) * mv.keep_Q + mv.keep_q0 + qrow;
+    kw_nxt = kw_ptr[0];
+  }
+  (void)kw;
   const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
   const float m = a.mx[st], rden = 1.f / a.den[st], delta = a.delta[st];
   f32x16 acc[NDB];
@@ -378,6 +407,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
   if (tid < XBN) { seg_ks[tid] = s_seg; bias_ks[tid] = s_bias; }
   __syncthreads();
   for (int t = 0; t < ntiles; t++) {
+    if (HAS_KEEP) { kw = kw_nxt; kw_nxt = kw_ptr[(int64_t)min(t + 1, ntiles - 1) * mv.keep_Q]; }
     if (t + 1 < ntiles) {
       RA_F32_LOAD(kg, vg, (t + 1) * XBN, a.kv_ss)
       if (tid < XBN) f32_key_info<HAS_SEG, HAS_BIAS>(mv, b, h, k_base + (t + 1) * XBN + tid, s_seg, s_bias);
@@ -400,12 +430,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
         }
       }
       const int gkb = gk0 + t * XBN + blk * 32;
+      const uint32_t kwb = HAS_KEEP ? (uint32_t)(kw >> (blk * 32)) >> (4 * hi) : 0u;   // this lane's keys of the block
+      (void)kwb;
       float ds[16];
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int kr = blk * 32 + crow(r, hi);
         bool masked = gkb + crow(r, hi) >= klim;
         if (HAS_SEG) masked = masked || seg_ks[kr] != seg_q;
+        if (HAS_KEEP) masked = masked || !((kwb >> (8 * (r >> 2) + (r & 3))) & 1u);   /* ringattention_inference.py:22 */
         const float add = masked ? mv.mask_min : (HAS_BIAS ? bias_ks[kr] : 0.f);
         const float p = __expf(s[r] * rscale + add - m) * rden;    // :226
         ds[r] = (dp[r] - delta) * p;                               // :229
@@ -443,7 +476,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
 }
 
 // ------------------------------------------------------------------ backward, dK and dV (key-stationary)
-template <int HD, bool HAS_SEG, bool HAS_BIAS>
+template <int HD, bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
 __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) float Qs[XBN * (HD + 4)];
   __shared__ __attribute__((aligned(16))) float Gs[XBN * (HD + 4)];
@@ -489,6 +522,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
     qt_end = qt_first + t_last;
     qt_first += t_first;
   }
+  if (HAS_KEEP && mv.skip_tiles && qt_first < qt_end) {
+    int t_first, t_last;
+    keep_qtile_hull(mv, b, h, (gk0 - mv.keep_k0) / 64, XBM / 64, mv.keep_q0 / 64 + qt_first, qt_end - qt_first, hull2, tid, 256,
+                    t_first, t_last);
+    qt_end = qt_first + t_last;
+    qt_first += t_first;
+  }
   if (qt_first >= qt_end) {                // nothing to add for these keys
     const int64_t o = (int64_t)b * a.dkv_sb + (int64_t)k0 * a.dkv_ss + (int64_t)h * HD;
     const int64_t oo = (int64_t)b * a.dkvo_sb + (int64_t)k0 * a.dkvo_ss + (int64_t)h * HD;
@@ -518,6 +558,15 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   for (int db = 0; db < NDB; db++)
 #pragma unroll
     for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+  // packed boolean mask: one 64-bit word per key and query tile (bit i = row i of the tile attends to this key)
+  const uint64_t* kw_ptr = nullptr;
+  uint64_t kw = 0, kw_nxt = 0;
+  if (HAS_KEEP) {
+    kw_ptr = mv.kbits_q + (int64_t)b * mv.kpack_sb + (int64_t)h * mv.kpack_sh +
+             (int64_t)(mv.keep_q0 / 64 + qt_first) * mv.keep_K + gk - mv.keep_k0;
+    kw_nxt = kw_ptr[0];
+  }
+  (void)kw;
 
   const float* qg = a.q + (int64_t)b * a.q_sb + (int64_t)h * HD + (int64_t)(qt_first * XBN) * a.q_ss;
   const float* gg = a.g + (int64_t)b * a.q_sb + (int64_t)h * HD + (int64_t)(qt_first * XBN) * a.q_ss;
@@ -541,6 +590,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   RA_F32_ROWSTATS_STORE
   __syncthreads();
   for (int t = 0; t < ntq; t++) {
+    if (HAS_KEEP) { kw = kw_nxt; kw_nxt = kw_ptr[(int64_t)min(t + 1, ntq - 1) * mv.keep_K]; }
     if (t + 1 < ntq) {
       RA_F32_LOAD(qg, gg, (t + 1) * XBN, a.q_ss)
       RA_F32_ROWSTATS(t + 1)
@@ -564,6 +614,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
         }
       }
       float p[16], ds[16];
+      const uint32_t kwb = HAS_KEEP ? (uint32_t)(kw >> (blk * 32)) >> (4 * hi) : 0u;     // this lane's rows of the block
+      (void)kwb;
 #pragma unroll
       for (int g4 = 0; g4 < 4; g4++) {
         const int row0 = blk * 32 + 8 * g4 + 4 * hi;               // rows of registers 4 g4 .. 4 g4 + 3
@@ -573,6 +625,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
           const int r = 4 * g4 + e;
           bool masked = gq_tile + row0 + e < qlim;
           if (HAS_SEG) masked = masked || st_seg[row0 + e] != seg_k;
+          if (HAS_KEEP) masked = masked || !((kwb >> (8 * g4 + e)) & 1u);
           const float add = masked ? mv.mask_min : (HAS_BIAS ? bias_k : 0.f);
           p[r] = __expf(s[r] * rscale + add - vm[e]) * vr[e];      // :226
           ds[r] = (dp[r] - vd[e]) * p[r];                          // :229
@@ -627,8 +680,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
 // ------------------------------------------------------------------ host side
 static bool al16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
+// a boolean mask is taken in packed form, with the where() semantics of ring_attention_inference and nothing next to
+// it but a causal block size (the dropout mask and every other combination stay with the vector kernels)
 static bool f32_mask_ok(const ra_mask& m) {
-  return !m.keep && !m.keep_bits_k && (m.bias == nullptr || m.bias_stride_q == 0);
+  if ((m.keep || m.keep_bits_k) &&
+      !(m.keep_bits_k && m.keep_bits_q && m.keep_summary && m.keep_mode == RA_KEEP_WHERE && !m.bias && !m.segment_ids))
+    return false;
+  return m.bias == nullptr || m.bias_stride_q == 0;
 }
 
 bool attn_fwd_f32_supported(const ra_attn_fwd_params* p) {
@@ -655,7 +713,10 @@ bool attn_bwd_f32_supported(const ra_attn_bwd_params* p) {
 
 #define RA_F32_DISPATCH(KERNEL, GRID)                                                    \
   do {                                                                                   \
-    if (p->D == 128) {                                                                   \
+    if (keep) {                                                                          \
+      if (p->D == 128) KERNEL<128, false, false, true><<<GRID, 256, 0, s>>>(a);          \
+      else KERNEL<64, false, false, true><<<GRID, 256, 0, s>>>(a);                       \
+    } else if (p->D == 128) {                                                            \
       if (seg && bias) KERNEL<128, true, true><<<GRID, 256, 0, s>>>(a);                  \
       else if (seg) KERNEL<128, true, false><<<GRID, 256, 0, s>>>(a);                    \
       else if (bias) KERNEL<128, false, true><<<GRID, 256, 0, s>>>(a);                   \
@@ -679,7 +740,7 @@ int attn_fwd_f32(const ra_attn_fwd_params* p, hipStream_t s) {
   a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
   a.out = (float*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
-  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
+  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr, keep = p->mask.keep_bits_k != nullptr;
   const long long nwg = (long long)(p->Sq / XBM) * p->H * p->B;
   RA_REQUIRE(nwg < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_fwd_f32: grid too large");
   const dim3 grid((unsigned)((nwg + 7) / 8 * 8));
@@ -704,7 +765,7 @@ int attn_bwd_f32(const ra_attn_bwd_params* p, int parts, hipStream_t s) {   // p
   a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.cache_idx = p->mask.cache_idx;
-  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
+  const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr, keep = p->mask.keep_bits_k != nullptr;
   const long long nq = (long long)(p->Sq / XBM) * p->H * p->B, nk = (long long)(p->Skv / XBM) * p->H * p->B;
   RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_f32: grid too large");
   const dim3 gq((unsigned)((nq + 7) / 8 * 8)), gk((unsigned)((nk + 7) / 8 * 8));

@@ -75,40 +75,6 @@ template <int HD> __device__ __forceinline__ int swz(int r) {
   return HD == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
 
-// ---- boolean keep mask in packed form (ra_keep_pack): 64-bit words and a per-64x64-tile summary
-// (0 none kept, 1 mixed, 2 all kept).  Hull of the key tiles [gkt0, gkt0 + n) that hold a kept pair for
-// any of the nrows summary rows starting at qt64 (every thread of the workgroup must call it).
-__device__ __forceinline__ void keep_ktile_hull(const MaskView& mv, int b, int h, int qt64, int nrows, int gkt0, int n,
-                                                int* hull2, int tid, int nthreads, int& first, int& last) {
-  if (tid == 0) { hull2[0] = n; hull2[1] = 0; }
-  __syncthreads();
-  const int KT = mv.keep_K / 64;
-  const uint8_t* sm = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh + (int64_t)qt64 * KT + gkt0;
-  for (int t = tid; t < n; t += nthreads) {
-    int any = 0;
-    for (int r = 0; r < nrows; r++) any |= sm[(int64_t)r * KT + t];
-    if (any) { atomicMin(&hull2[0], t); atomicMax(&hull2[1], t + 1); }
-  }
-  __syncthreads();
-  first = hull2[0]; last = hull2[1];
-  if (last < first) { first = 0; last = 0; }
-}
-// the same over the query tiles [gqt0, gqt0 + n) for the ncols summary columns starting at kt64
-__device__ __forceinline__ void keep_qtile_hull(const MaskView& mv, int b, int h, int kt64, int ncols, int gqt0, int n,
-                                                int* hull2, int tid, int nthreads, int& first, int& last) {
-  if (tid == 0) { hull2[0] = n; hull2[1] = 0; }
-  __syncthreads();
-  const int KT = mv.keep_K / 64;
-  const uint8_t* sm = mv.ksum + (int64_t)b * mv.ksum_sb + (int64_t)h * mv.ksum_sh + (int64_t)gqt0 * KT + kt64;
-  for (int t = tid; t < n; t += nthreads) {
-    int any = 0;
-    for (int cidx = 0; cidx < ncols; cidx++) any |= sm[(int64_t)t * KT + cidx];
-    if (any) { atomicMin(&hull2[0], t); atomicMax(&hull2[1], t + 1); }
-  }
-  __syncthreads();
-  first = hull2[0]; last = hull2[1];
-  if (last < first) { first = 0; last = 0; }
-}
 // number of leading tiles of a summary row (or column, with the given stride) that are "all kept"
 __device__ __forceinline__ int keep_leading_full(const uint8_t* sm, int64_t stride, int n, int lane) {
   for (int base = 0; base < n; base += 64) {

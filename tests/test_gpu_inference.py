@@ -129,18 +129,46 @@ MFMA_CASES = [
 ]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("D", [128, 64])
 @pytest.mark.parametrize("case", MFMA_CASES)
-def test_inference_mfma_path_matches_oracle(case, D):
+def test_inference_mfma_path_matches_oracle(case, D, dtype):
+    """bf16 on the bf16 MFMA kernels, fp32 on the fp32 ones (both read the packed mask)."""
     B, S, H, n, kind = case
-    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=21, scale=D ** -0.25)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=21, scale=D ** -0.25)
     mask = _structured_mask(B, H, S, kind, 22)
     out, grads = _run(q, k, v, do, mask, n)
     ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
     ref_grads = O.ring_attention_inference_bwd(n, res, do)
-    assert_close(out, ref_out, torch.bfloat16, "out")
+    assert_close(out, ref_out, dtype, "out")
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
-        assert_close(a, b, torch.bfloat16, name)
+        assert_close(a, b, dtype, name)
+
+
+def test_inference_fp32_matrix_core_and_vector_kernels_agree():
+    """fp32 inputs: the same call with the packed mask (fp32 matrix-core kernels) and without it (vector kernels),
+    including a row that attends to nothing."""
+    from ringattention_amd import ringattention_hip as rh
+    B, S, H, D, n = 2, 1024, 2, 128, 2
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float32, seed=27, scale=D ** -0.25)
+    mask = _structured_mask(B, H, S, "causal_padding", 28)
+    mask[:, :, 700, :] = False
+    out, grads = _run(q, k, v, do, mask, n)
+    orig = rh._MaskInputs.set_keep
+
+    def no_pack(self, *a, **kw):
+        orig(self, *a, **kw)
+        self.keep_packed = None
+
+    rh._MaskInputs.set_keep = no_pack
+    try:
+        out_g, grads_g = _run(q, k, v, do, mask, n)
+    finally:
+        rh._MaskInputs.set_keep = orig
+    assert torch.allclose(out[:, 700], v.mean(dim=1), atol=1e-5)
+    for name, a, b in zip(("out", "dq", "dk", "dv"), (out,) + grads, (out_g,) + grads_g):
+        assert_close(a, b, torch.float32, name)
+        assert float((a - b).abs().max()) <= 2e-5, name
 
 
 def test_inference_mfma_path_with_a_row_that_attends_to_nothing():
