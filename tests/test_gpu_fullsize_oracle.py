@@ -272,9 +272,16 @@ def test_blockwise_q_len_differs_from_kv_len(impl):
         ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, None, None, None, 1, kw)
         out, grads = _hip(q, k, v, do, None, None, 1, kw)
         _compare("q %d kv %d %s" % (Sq, Skv, impl), out, grads, ref_out, ref_grads, 0.0)
+        if impl == "mfma":                  # the same lengths in fp32, on the fp32 matrix-core kernels
+            qf, kf, vf, dof = (t.float() for t in (q, k, v, do))
+            ref_out, ref_grads = oracle_fwd_bwd(qf, kf, vf, dof, None, None, None, 1, kw)
+            out, grads = _hip(qf, kf, vf, dof, None, None, 1, dict(kw, dtype=torch.float32))
+            assert_close(out, ref_out, torch.float32, "fp32 out")
+            for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+                assert_close(a, b, torch.float32, "fp32 " + name)
 
 
-@pytest.mark.parametrize("impl,dtype", [("mfma", torch.bfloat16), ("generic", torch.float32)])
+@pytest.mark.parametrize("impl,dtype", [("mfma", torch.bfloat16), ("generic", torch.float32), ("mfma", torch.float32)])
 @pytest.mark.parametrize("cache_idx", [0, 300, 512, 1000, 1536])
 def test_cache_idx_with_several_query_tokens(cache_idx, impl, dtype):
     """cache_idx with q_len > 1 (ringattention_jax.py:34-35): the query chunks start at global chunk
