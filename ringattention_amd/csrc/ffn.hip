@@ -19,10 +19,6 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-#ifndef RA_W4_ABL
-// timing experiments only (results are wrong): 1 = no global loads, 2 = no LDS stores, 4 = no LDS reads, 8 = no barrier
-#define RA_W4_ABL 0
-#endif
 constexpr int GBK = 64;               // K step of the 8-wavefront tiles (and the granularity required of K)
 
 struct GemmArgs {
@@ -388,15 +384,15 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   // which goes to the other buffer, and is then reloaded with slab NEXT_T
 #define RA_W4_STEP(CUR, S, NEXT_T)                                                                      \
   {                                                                                                     \
-    if (!(RA_W4_ABL & 4)) { RA_W4_FRAGS(G, CUR, 1); }                                                   \
-    if (!(RA_W4_ABL & 2)) { RA_W4_STORE(S, (CUR) ^ 1); }                                                \
-    if (!(RA_W4_ABL & 1)) { RA_W4_LOAD_A(S, NEXT_T); }                                                  \
+    RA_W4_FRAGS(G, CUR, 1);                                                                             \
+    RA_W4_STORE(S, (CUR) ^ 1);                                                                          \
+    RA_W4_LOAD_A(S, NEXT_T);                                                                            \
     RA_W4_MFMA(F);                                                                                      \
     RA_W4_SCHED(8, 4);                                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
-    if (!(RA_W4_ABL & 8)) __syncthreads();                                                              \
-    if (!(RA_W4_ABL & 4)) { RA_W4_FRAGS(F, (CUR) ^ 1, 0); }                                             \
-    if (!(RA_W4_ABL & 1)) { RA_W4_LOAD_B(S, NEXT_T); }                                                  \
+    __syncthreads();                                                                                    \
+    RA_W4_FRAGS(F, (CUR) ^ 1, 0);                                                                       \
+    RA_W4_LOAD_B(S, NEXT_T);                                                                            \
     RA_W4_MFMA(G);                                                                                      \
     RA_W4_SCHED(0, 4);                                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
