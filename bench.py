@@ -689,13 +689,44 @@ def bench_inference(args):
             "cpu_baseline": None}
 
 
+def bench_mfma_probe(args):
+    """What the matrix pipes sustain on bf16 MFMAs alone, by operand activity (ra_mfma_rate_probe): the rate, the
+    clock and the board power of a two-second run each.  The value is the rate on random operands: the ceiling a
+    bf16 kernel on real data has on this board, next to the published peak."""
+    import torch
+    from ringattention_amd import _lib as L
+    dev = "cuda:0"
+    wgs, iters = 256, 8192                      # one workgroup per CU, 64 * iters MFMAs per wavefront
+    sink = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    flop = wgs * 4 * iters * 64 * 32768.0
+    rows = {}
+    for mode, name in ((0, "one value everywhere"), (1, "a value per lane, constant in time"), (2, "random operands")):
+        fn = lambda: L.check(L.load().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, mode, stream), "ra_mfma_rate_probe")
+        fn()
+        torch.cuda.synchronize()
+        clk = _sclk_under_load(fn, seconds=2.5)
+        ms = _event_ms(fn, 10)
+        rows[name] = {"tflops": round(flop / (ms * 1e-3) / 1e12, 1), "ms": round(ms, 3),
+                      "power_w": clk.pop("power_w", None) if clk else None, "sclk_mhz": clk}
+        time.sleep(1.0)
+    value = rows["random operands"]["tflops"]
+    return {"metric": "mfma_only_tflops", "value": value, "unit": "TFLOP/s", "ms_per_step": rows["random operands"]["ms"],
+            "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+            "config": {"workload": "mfma_probe", "workgroups": wgs, "mfma_per_wavefront": iters * 64,
+                       "instruction": "v_mfma_f32_32x32x16_bf16", "by_operands": rows},
+            "roofline": {"bound": "mfma", "kernel": "mfma_probe_kernel", "achieved": value, "peak": PEAK_BF16_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(value / PEAK_BF16_TFLOPS, 4), "traffic": None},
+            "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default=None, choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
-                                                              "dropout32k", "c1"])
+                                                              "dropout32k", "c1", "mfma_probe"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
                     help="attention workloads: head size (the number of heads follows, H * D = 4096)")
@@ -752,6 +783,8 @@ def main():
         r = bench_rmsnorm(args)
     elif args.workload == "inference":
         r = bench_inference(args)
+    elif args.workload == "mfma_probe":
+        r = bench_mfma_probe(args)
     else:
         r = bench_ffn(args)
     line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,

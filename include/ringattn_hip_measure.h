@@ -23,6 +23,13 @@ int ra_attn_bwd_block_part(const ra_attn_bwd_params* p, int32_t part, ra_stream_
 int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,
                       int32_t trans_b, int32_t c_dtype, int32_t beta_one, int32_t tile, ra_stream_t stream);
 
+/* What the matrix pipes sustain on bf16 MFMAs alone (v_mfma_f32_32x32x16_bf16, four independent accumulators per
+ * wavefront, four wavefronts per workgroup): every wavefront issues 64 * iters instructions of 32768 FLOP each.
+ * operands 0: one value everywhere; 1: a value per lane, the same in every instruction; 2: random values, consecutive
+ * instructions see different operand pairs.  sink: workgroups * 256 floats of device memory (written once).  The rate
+ * depends on the operands because the clock is set by a power / current limit, not by the instruction stream. */
+int ra_mfma_rate_probe(float* sink, int32_t workgroups, int32_t iters, int32_t operands, ra_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

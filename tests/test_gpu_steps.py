@@ -153,3 +153,20 @@ def test_decode_step_replays_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(torch.nan_to_num(out), torch.nan_to_num(out_ref))
         assert torch.equal(qr, qr_ref) and torch.equal(k_cache, k_ref) and torch.equal(v_cache, v_ref)
+
+
+def test_mfma_rate_probe_computes_what_it_says():
+    """The measurement probe really issues its MFMAs: with 0.5 and 0.25 everywhere an instruction adds 16 * 0.125 = 2
+    to each of its 1024 results, an accumulator takes 16 instructions per iteration, and a lane sums 4 x 16 results."""
+    from ringattention_amd import _lib as L
+    iters, wgs = 4, 8
+    sink = torch.zeros(wgs * 256, dtype=torch.float32, device=DEV)
+    L.check(L.load().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, 0, torch.cuda.current_stream().cuda_stream),
+            "ra_mfma_rate_probe")
+    torch.cuda.synchronize()
+    assert bool((sink == 2.0 * 16 * iters * 64).all())
+    for mode in (1, 2):
+        L.check(L.load().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, mode, torch.cuda.current_stream().cuda_stream),
+                "ra_mfma_rate_probe")
+        torch.cuda.synchronize()
+        assert bool(torch.isfinite(sink).all()) and float(sink.abs().max()) > 0

@@ -112,6 +112,8 @@ def test_invalid_arguments_return_codes_without_gpu():
     # measurement hooks validate too
     assert lib.ra_attn_bwd_block_part(None, 3, None) == _lib.RA_ERR_INVALID
     assert lib.ra_gemm_bf16_tile(one_ := ctypes.c_void_p(16), one_, one_, 128, 128, 64, 0, 0, 1, 0, 7, None) == _lib.RA_ERR_INVALID
+    assert lib.ra_mfma_rate_probe(None, 1, 1, 0, None) == _lib.RA_ERR_INVALID
+    assert lib.ra_mfma_rate_probe(ctypes.c_void_p(16), 1, 1, 3, None) == _lib.RA_ERR_INVALID
     # ra_keep_pack validates before touching the device
     assert lib.ra_keep_pack(None, 0, 0, 0, 1, 1, 1, 64, 64, None, None, None, None) == _lib.RA_ERR_INVALID
     one = ctypes.c_void_p(16)      # any non-null address: the shape check comes before any use
