@@ -769,6 +769,13 @@ def main():
                 others.append({"inputs": r2["config"]["inputs"], "value": r2["value"], "unit": r2["unit"],
                                "ms_per_step": r2["ms_per_step"], "kernel_ms": r2["roofline"]["kernel_ms"]})
             extras["other_inputs"] = others
+            # the rate of the matrix pipes on MFMAs alone, same board, same run: what "peak" means for real data here
+            pr = bench_mfma_probe(args)
+            extras["mfma_probe"] = {"metric": pr["metric"], "value": pr["value"], "unit": pr["unit"],
+                                    "by_operands": pr["config"]["by_operands"]}
+            if r.get("roofline") and pr["value"]:
+                r["roofline"]["frac_of_mfma_only_rate_on_random_operands"] = round(
+                    r["roofline"]["achieved"] / pr["value"], 4)
             torch.cuda.empty_cache()
             d = bench_decode(args, steps=64)
             extras["decode"] = {k_: d[k_] for k_ in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
