@@ -111,7 +111,7 @@ __device__ __forceinline__ void f32_pass_rows(const float* acc, float* acc_w, in
   }
 
 // key range [k_base, k_base + 64 ntiles) of the shard that a 128-row query tile has to visit (forward, dQ)
-template <bool HAS_SEG, bool HAS_KEEP>
+template <bool HAS_SEG, int HAS_KEEP>
 __device__ __forceinline__ void f32_key_range(const MaskView& mv, int b, int h, int q0, int Skv, int tid, int* hull2,
                                               int& k_base, int& ntiles) {
   const int qi = q0 / mv.qc;
@@ -155,8 +155,22 @@ __device__ __forceinline__ void f32_key_info(const MaskView& mv, int b, int h, i
   }
 }
 
+// Logit of one pair from its scaled dot product (:134-136, :272-322).  masked: the causal or segment mask hits the
+// pair; kept: its bit of the boolean mask (only read when KEEP is set); bias: the key's clamped bias.
+template <int KEEP>
+__device__ __forceinline__ float f32_logit(float dot_scaled, bool masked, bool kept, float bias, float mask_min) {
+  if (KEEP == 2) {
+    if (kept) return dot_scaled + (masked ? mask_min : bias);
+    return masked ? RA_NEG_INF : mask_min;          // dropped: mask_min added once absorbs logit and bias, twice overflows
+  }
+  if (KEEP == 1) masked = masked || !kept;
+  return dot_scaled + (masked ? mask_min : bias);
+}
+
 // ------------------------------------------------------------------ forward
-template <int HD, bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>   // HAS_KEEP: where(keep, logit, mask_min), packed mask
+// HAS_KEEP (packed boolean mask): 0 none, 1 where(keep, logit, mask_min) (ringattention_inference.py:22), 2 dropout:
+// mask_min is ADDED for a dropped pair (ringattention_jax.py:321), so a pair that is masked as well becomes -inf
+template <int HD, bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>
 __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) float Ks[XBN * (HD + 4)];
   __shared__ __attribute__((aligned(16))) float Vs[XBN * (HD + 4)];
@@ -274,9 +288,8 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
         const int kr = blk * 32 + crow(r, hi);
         bool masked = gkb + crow(r, hi) >= klim;
         if (HAS_SEG) masked = masked || seg_ks[kr] != seg_q;
-        if (HAS_KEEP) masked = masked || !((kwb >> (8 * (r >> 2) + (r & 3))) & 1u);   /* ringattention_inference.py:22 */
-        const float add = masked ? mv.mask_min : (HAS_BIAS ? bias_ks[kr] : 0.f);
-        x[r] = (s0[r] + s1[r]) * rscale + add;
+        const bool kept = HAS_KEEP ? ((kwb >> (8 * (r >> 2) + (r & 3))) & 1u) != 0 : true;
+        x[r] = f32_logit<HAS_KEEP>((s0[r] + s1[r]) * rscale, masked, kept, HAS_BIAS ? bias_ks[kr] : 0.f, mv.mask_min);
         mloc = fmaxf(mloc, x[r]);
       }
       mloc = fmaxf(mloc, xor32f(mloc));
@@ -336,7 +349,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
 }
 
 // ------------------------------------------------------------------ backward, dQ (query-stationary)
-template <int HD, bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
+template <int HD, bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>
 __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) float Ks[XBN * (HD + 4)];
   __shared__ __attribute__((aligned(16))) float Vs[XBN * (HD + 4)];
@@ -438,9 +451,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
         const int kr = blk * 32 + crow(r, hi);
         bool masked = gkb + crow(r, hi) >= klim;
         if (HAS_SEG) masked = masked || seg_ks[kr] != seg_q;
-        if (HAS_KEEP) masked = masked || !((kwb >> (8 * (r >> 2) + (r & 3))) & 1u);   /* ringattention_inference.py:22 */
-        const float add = masked ? mv.mask_min : (HAS_BIAS ? bias_ks[kr] : 0.f);
-        const float p = __expf(s[r] * rscale + add - m) * rden;    // :226
+        const bool kept = HAS_KEEP ? ((kwb >> (8 * (r >> 2) + (r & 3))) & 1u) != 0 : true;
+        const float x_ = f32_logit<HAS_KEEP>(s[r] * rscale, masked, kept, HAS_BIAS ? bias_ks[kr] : 0.f, mv.mask_min);
+        const float p = __expf(x_ - m) * rden;                     // :226
         ds[r] = (dp[r] - delta) * p;                               // :229
       }
       // dQ^T += K^T dS^T (:230)
@@ -476,7 +489,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
 }
 
 // ------------------------------------------------------------------ backward, dK and dV (key-stationary)
-template <int HD, bool HAS_SEG, bool HAS_BIAS, bool HAS_KEEP = false>
+template <int HD, bool HAS_SEG, bool HAS_BIAS, int HAS_KEEP = 0>
 __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) float Qs[XBN * (HD + 4)];
   __shared__ __attribute__((aligned(16))) float Gs[XBN * (HD + 4)];
@@ -625,9 +638,9 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
           const int r = 4 * g4 + e;
           bool masked = gq_tile + row0 + e < qlim;
           if (HAS_SEG) masked = masked || st_seg[row0 + e] != seg_k;
-          if (HAS_KEEP) masked = masked || !((kwb >> (8 * g4 + e)) & 1u);
-          const float add = masked ? mv.mask_min : (HAS_BIAS ? bias_k : 0.f);
-          p[r] = __expf(s[r] * rscale + add - vm[e]) * vr[e];      // :226
+          const bool kept = HAS_KEEP ? ((kwb >> (8 * g4 + e)) & 1u) != 0 : true;
+          const float x_ = f32_logit<HAS_KEEP>(s[r] * rscale, masked, kept, HAS_BIAS ? bias_k : 0.f, mv.mask_min);
+          p[r] = __expf(x_ - vm[e]) * vr[e];                       // :226
           ds[r] = (dp[r] - vd[e]) * p[r];                          // :229
         }
       }
@@ -680,11 +693,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
 // ------------------------------------------------------------------ host side
 static bool al16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
-// a boolean mask is taken in packed form, with the where() semantics of ring_attention_inference and nothing next to
-// it but a causal block size (the dropout mask and every other combination stay with the vector kernels)
+// a boolean mask is taken in packed form only; the attn_mask of ring_attention_inference next to a causal block size
+// at most (it has no bias or segment ids there), the dropout mask next to everything
 static bool f32_mask_ok(const ra_mask& m) {
   if ((m.keep || m.keep_bits_k) &&
-      !(m.keep_bits_k && m.keep_bits_q && m.keep_summary && m.keep_mode == RA_KEEP_WHERE && !m.bias && !m.segment_ids))
+      !(m.keep_bits_k && m.keep_bits_q && m.keep_summary &&
+        (m.keep_mode == RA_KEEP_DROPOUT || (!m.bias && !m.segment_ids))))
     return false;
   return m.bias == nullptr || m.bias_stride_q == 0;
 }
@@ -713,9 +727,21 @@ bool attn_bwd_f32_supported(const ra_attn_bwd_params* p) {
 
 #define RA_F32_DISPATCH(KERNEL, GRID)                                                    \
   do {                                                                                   \
-    if (keep) {                                                                          \
-      if (p->D == 128) KERNEL<128, false, false, true><<<GRID, 256, 0, s>>>(a);          \
-      else KERNEL<64, false, false, true><<<GRID, 256, 0, s>>>(a);                       \
+    if (keep && p->mask.keep_mode == RA_KEEP_DROPOUT) {                                  \
+      if (p->D == 128) {                                                                 \
+        if (seg && bias) KERNEL<128, true, true, 2><<<GRID, 256, 0, s>>>(a);             \
+        else if (seg) KERNEL<128, true, false, 2><<<GRID, 256, 0, s>>>(a);               \
+        else if (bias) KERNEL<128, false, true, 2><<<GRID, 256, 0, s>>>(a);              \
+        else KERNEL<128, false, false, 2><<<GRID, 256, 0, s>>>(a);                       \
+      } else {                                                                           \
+        if (seg && bias) KERNEL<64, true, true, 2><<<GRID, 256, 0, s>>>(a);              \
+        else if (seg) KERNEL<64, true, false, 2><<<GRID, 256, 0, s>>>(a);                \
+        else if (bias) KERNEL<64, false, true, 2><<<GRID, 256, 0, s>>>(a);               \
+        else KERNEL<64, false, false, 2><<<GRID, 256, 0, s>>>(a);                        \
+      }                                                                                  \
+    } else if (keep) {                                                                   \
+      if (p->D == 128) KERNEL<128, false, false, 1><<<GRID, 256, 0, s>>>(a);             \
+      else KERNEL<64, false, false, 1><<<GRID, 256, 0, s>>>(a);                          \
     } else if (p->D == 128) {                                                            \
       if (seg && bias) KERNEL<128, true, true><<<GRID, 256, 0, s>>>(a);                  \
       else if (seg) KERNEL<128, true, false><<<GRID, 256, 0, s>>>(a);                    \

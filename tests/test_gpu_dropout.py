@@ -129,25 +129,28 @@ def test_dropout_with_segments_and_bias_matches_oracle():
     (2, 1024, 512, 512, 256, 0.2),
 ])
 @pytest.mark.parametrize("D", [128, 64])
-def test_dropout_mfma_bf16_matches_oracle(n, S, qc, kc, cbs, p, D):
-    """bf16, D 128 or 64, chunk sizes the MFMA kernels take: the packed mask, next to the causal block size."""
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_dropout_mfma_bf16_matches_oracle(n, S, qc, kc, cbs, p, D, dtype):
+    """D 128 or 64, chunk sizes the MFMA kernels take (bf16 and fp32 family alike): the packed mask, next to the
+    causal block size."""
     B, H = 1, 2
-    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=13, scale=D ** -0.25)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=13, scale=D ** -0.25)
     kw = kwargs(qc, kc, cbs, deterministic=False, dropout_rng=7, attn_pdrop=p, impl="mfma")
-    _compare(q, k, v, do, None, None, n, kw, torch.bfloat16, "mfma n%d S%d %d/%d cbs %s p %.1f" % (n, S, qc, kc, cbs, p))
+    _compare(q, k, v, do, None, None, n, kw, dtype, "mfma n%d S%d %d/%d cbs %s p %.1f" % (n, S, qc, kc, cbs, p))
 
 
 @pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("use_seg,use_bias,n", [(True, False, 1), (False, True, 2), (True, True, 2), (True, True, 4)])
-def test_dropout_mfma_with_documents_and_bias_matches_oracle(use_seg, use_bias, n, D):
+def test_dropout_mfma_with_documents_and_bias_matches_oracle(use_seg, use_bias, n, D, dtype):
     """The dropout mask next to segment ids and a bias on the MFMA kernels: a pair of two documents counts as masked
     once (finfo.min), masked and dropped as twice (-inf), and the bias is clamped at 0 under a mask as always."""
     B, S, H = 2, 1024, 2
-    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=17, scale=D ** -0.25)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=17, scale=D ** -0.25)
     seg = packed_segment_ids(B, S, 200, seed=6) if use_seg else None
     bias = torch.randn(B, H, 1, S, generator=torch.Generator().manual_seed(8)) if use_bias else None
     kw = kwargs(256, 256, 1, deterministic=False, dropout_rng=11, attn_pdrop=0.3, impl="mfma")
-    _compare(q, k, v, do, bias, seg, n, kw, torch.bfloat16, "mfma seg %s bias %s n%d" % (use_seg, use_bias, n))
+    _compare(q, k, v, do, bias, seg, n, kw, dtype, "mfma seg %s bias %s n%d" % (use_seg, use_bias, n))
 
 
 def test_dropout_mfma_equals_generic():
