@@ -168,10 +168,24 @@ class _FakeMaskInputs:
     (384, 192, None, True, 128), (64, 192, 32, True, 128), (64, 192, 48, True, 64), (256, 256, 1, True, 256)])
 def test_fit_chunks_to_mfma_grid_decisions(qc, kc, cbs, skip, expect):
     from ringattention_amd import ringattention_hip as rh
+    for dtype in (torch.bfloat16, torch.float32):           # both matrix-core families tile on the same grid
+        cfg = rh._Config(dict(query_chunk_size=qc, key_chunk_size=kc, causal_block_size=cbs))
+        cfg.skip_masked_tiles = skip
+        q = torch.zeros(1, 1, 1, 128, dtype=dtype)
+        rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), q, 768, 768, 768, 768)
+        assert cfg.qc == expect, (cfg.qc, cfg.kc)
+        if expect == 128:
+            assert cfg.kc == 128
     cfg = rh._Config(dict(query_chunk_size=qc, key_chunk_size=kc, causal_block_size=cbs))
     cfg.skip_masked_tiles = skip
-    q = torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16)
-    rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), q, 768, 768, 768, 768)
-    assert cfg.qc == expect, (cfg.qc, cfg.kc)
-    if expect == 128:
-        assert cfg.kc == 128
+    rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 32, dtype=torch.bfloat16), 768, 768, 768, 768)
+    assert (cfg.qc, cfg.kc) == (qc, kc)                      # head size 32: the vector kernels, chunk sizes untouched
+
+
+def test_output_residual_option():
+    from ringattention_amd.ringattention_hip import _Config
+    base = dict(causal_block_size=1, query_chunk_size=128, key_chunk_size=128)
+    assert _Config(base).output_residual == "fp32"                          # the reference's residual (:53)
+    assert _Config(dict(base, output_residual="rounded")).output_residual == "rounded"
+    with pytest.raises(ValueError):
+        _Config(dict(base, output_residual="bf16"))
