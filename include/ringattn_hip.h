@@ -32,7 +32,9 @@ enum { RA_F32 = 0, RA_BF16 = 1 };
 enum {
   RA_IMPL_AUTO = 0,    /* MFMA kernels when the shape allows, else the generic ones */
   RA_IMPL_GENERIC = 1, /* fp32 vector-ALU kernels: any chunk sizes, fp32 or bf16 inputs */
-  RA_IMPL_MFMA = 2     /* bf16 MFMA kernels only; RA_ERR_UNSUPPORTED if the shape does not fit */
+  RA_IMPL_MFMA = 2     /* matrix-core kernels only (bf16 inputs: v_mfma_f32_32x32x16_bf16, fp32 inputs:
+                          v_mfma_f32_32x32x2_f32; head size 64 or 128, chunk sizes multiples of 128);
+                          RA_ERR_UNSUPPORTED if the shape does not fit */
 };
 
 /*
