@@ -268,6 +268,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   __shared__ __attribute__((aligned(16))) float st_lse2[3][KBM];
   __shared__ __attribute__((aligned(16))) float st_delta[3][KBM];   // holds -delta
   __shared__ __attribute__((aligned(16))) int st_seg[3][KBM];
+  __shared__ float st_bias[4][64];           // [pair][lane]: the lane's key's clamped, scaled bias
 
   MaskView mv = a.mv;
   if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
@@ -406,6 +407,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)gk * mv.bias_sk];
       if (mv.any_mask) bv = fminf(bv, 0.f);
       bias2 = bv * kLog2e / c;          // the S accumulators start from it
+      st_bias[pair][lane] = bias2;      // kept in LDS, not in a register: every lane reads back its own slot
     }
     const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
     bf16x8 kf[NK], vf[NK];
@@ -424,7 +426,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
 #define RA_WS_INIT(SN, DPN, BUF, BLK)                                                                   \
   _Pragma("unroll") for (int g = 0; g < 4; g++) {                                                       \
     const f32x4 d_ = *(const f32x4*)&st_delta[BUF][(BLK) * 32 + g * 8 + hi * 4];                        \
-    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = HAS_BIAS ? bias2 : 0.f; DPN[g * 4 + e] = d_[e]; } \
+    const float b0_ = HAS_BIAS ? st_bias[pair][lane] : 0.f;                                                \
+    _Pragma("unroll") for (int e = 0; e < 4; e++) { SN[g * 4 + e] = b0_; DPN[g * 4 + e] = d_[e]; } \
   }
     // A operands of two contraction steps (32 of the 128 head dimensions) of block BLK of buffer BUF
 #define RA_WS_AREAD(G, QA, GA, BUF, BLK)                                                                \
