@@ -776,6 +776,11 @@ def main():
             if r.get("roofline") and pr["value"]:
                 r["roofline"]["frac_of_mfma_only_rate_on_random_operands"] = round(
                     r["roofline"]["achieved"] / pr["value"], 4)
+            # the reference's own CPU-runnable configuration (fp32, on the fp32 matrix-core kernels) next to the CPU
+            # oracle timed on the whole of it
+            c1 = bench_attention(argparse.Namespace(**dict(vars(args), steps=50, warmup=5)), ring=False, c1=True)
+            extras["c1"] = {k_: c1[k_] for k_ in ("metric", "value", "unit", "ms_per_step", "dtype", "config",
+                                                    "roofline", "cpu_baseline")}
             torch.cuda.empty_cache()
             d = bench_decode(args, steps=64)
             extras["decode"] = {k_: d[k_] for k_ in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
