@@ -259,14 +259,18 @@ __device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t vo
 template <bool TA, bool TB>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   constexpr int BM = 256, BN = 256, BK = 32, NT = 256, WM = 128, WN = 128;
-  // A row-wise read tile has rows of 32 elements = four 16-byte chunks and no padding; chunk c of row r sits at
-  // chunk c ^ ((r >> 2) & 3): sixteen consecutive rows then put a given chunk in sixteen different bank groups
-  // (conflict-free fragment reads), and a row stays one contiguous 64 bytes (conflict-free staging writes).
-  constexpr int NAT_STR = BK;
-  constexpr int A_STR = TA ? BM + 32 : NAT_STR, B_STR = TB ? NAT_STR : BN + 32;
+  // An operand whose rows run along K ("row-wise": A unless TA, B if TB) is fetched in whole 128-byte lines: a
+  // staging unit of such an operand is 128 of the tile's 256 rows times 64 K positions, so that two consecutive K
+  // steps bring in one slab of two K steps (unit u = slab u / 2, row half u % 2) and every request that reaches the
+  // L2 is a full line, where rows of one K step would be 64-byte halves requested twice.  In LDS such a slab is 256
+  // rows of eight 16-byte chunks, chunk c of row r at position c ^ ((r >> 1) & 7): sixteen consecutive rows then
+  // put a given chunk in sixteen different bank groups (conflict-free fragment reads), and a row stays one
+  // contiguous 128 bytes (conflict-free staging writes).  It is stored two K steps before its first use, the unit
+  // of an operand that is staged as it lies (32 K rows of the tile's 256 columns) one step before.
+  constexpr int WIDE_STR = 64;
+  constexpr int A_STR = TA ? BM + 32 : WIDE_STR, B_STR = TB ? WIDE_STR : BN + 32;
   constexpr int A_ROWS = TA ? BK : BM, B_ROWS = TB ? BN : BK;
-  constexpr int A_CPR = (TA ? BM : BK) / 8, B_CPR = (TB ? BK : BN) / 8;
-  static_assert(A_ROWS * A_CPR == 4 * NT && B_ROWS * B_CPR == 4 * NT, "four 16-byte chunks per thread and operand");
+  constexpr int A_CPR = TA ? BM / 8 : 8, B_CPR = TB ? 8 : BN / 8;
   // one array per buffer and operand: reads of one buffer and writes of the other can then be reordered freely
   __shared__ __attribute__((aligned(16))) uint16_t As0[A_ROWS * A_STR];
   __shared__ __attribute__((aligned(16))) uint16_t As1[A_ROWS * A_STR];
@@ -274,6 +278,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) uint16_t Bs1[B_ROWS * B_STR];
 #define RA_W4_AS(BUF) ((BUF) ? As1 : As0)
 #define RA_W4_BS(BUF) ((BUF) ? Bs1 : Bs0)
+  // where the unit of K step U (known modulo 4) lives: buffer and offset of its row half
+#define RA_W4_ABUF(U) (TA ? ((U) & 1) : (((U) >> 1) & 1))
+#define RA_W4_BBUF(U) (TB ? (((U) >> 1) & 1) : ((U) & 1))
+#define RA_W4_AHALF(U) (TA ? 0 : ((U) & 1) * 128 * WIDE_STR)
+#define RA_W4_BHALF(U) (TB ? ((U) & 1) * 128 * WIDE_STR : 0)
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
@@ -289,14 +298,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  // four sets of staging registers: slab j lives in set j % 4 from its request until it is stored to LDS four K
+  // four sets of staging registers: unit j lives in set j % 4 from its request until it is stored to LDS four K
   // steps later (about 2 us: an L2 miss served from HBM under load takes that long)
   uint4 Pa0, Pa1, Pa2, Pa3, Pb0, Pb1, Pb2, Pb3, Qa0, Qa1, Qa2, Qa3, Qb0, Qb1, Qb2, Qb3;
   uint4 Ra0, Ra1, Ra2, Ra3, Rb0, Rb1, Rb2, Rb3, Ta0, Ta1, Ta2, Ta3, Tb0, Tb1, Tb2, Tb3;
   const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
   const int nk = g.K / BK;
   const int total = nk * (g.A2 ? 2 : 1);
-  // this thread's four chunks of a slab: global offsets (without the K position) and LDS offsets
+  // this thread's four chunks of a unit: global offsets (without the K position) and LDS offsets
   // The global address of a chunk is a wave-uniform base (operand, tile origin, K position: scalar registers) plus a
   // 32-bit byte offset per lane: that form of load sends half the address data of a 64-bit pointer per lane and
   // measured 5-7 % more 16-byte loads per clock and CU.  (A tile spans at most 255 rows: the offset stays below 2^31.)
@@ -305,14 +314,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   const int64_t tile_a = TA ? (int64_t)m0 : (int64_t)m0 * lda, tile_b = TB ? (int64_t)n0 * ldb : (int64_t)n0;
 #pragma unroll
   for (int c = 0; c < 4; c++) {
-    const int ia = c * NT + tid, ib = c * NT + tid;
-    ga[c] = 2u * (uint32_t)((ia / A_CPR) * lda + (ia % A_CPR) * 8);
-    gb[c] = 2u * (uint32_t)((ib / B_CPR) * ldb + (ib % B_CPR) * 8);
-    la[c] = (ia / A_CPR) * A_STR + (TA ? ia % A_CPR : (ia % A_CPR) ^ ((ia / A_CPR >> 2) & 3)) * 8;
-    lb[c] = (ib / B_CPR) * B_STR + (TB ? (ib % B_CPR) ^ ((ib / B_CPR >> 2) & 3) : ib % B_CPR) * 8;
+    const int i = c * NT + tid;
+    const int ra_ = i / A_CPR, ca_ = i % A_CPR, rb_ = i / B_CPR, cb_ = i % B_CPR;
+    ga[c] = 2u * (uint32_t)(ra_ * lda + ca_ * 8);
+    gb[c] = 2u * (uint32_t)(rb_ * ldb + cb_ * 8);
+    la[c] = ra_ * A_STR + (TA ? ca_ : ca_ ^ ((ra_ >> 1) & 7)) * 8;
+    lb[c] = rb_ * B_STR + (TB ? cb_ ^ ((rb_ >> 1) & 7) : cb_) * 8;
   }
-  // buffer descriptors that start at the tile's origin; the K position goes into the scalar offset (bytes)
-  const uint32_t ka2 = 2u * (uint32_t)(TA ? lda : 1), kb2 = 2u * (uint32_t)(TB ? 1 : ldb);
+  // buffer descriptors that start at the tile's origin; the unit's position goes into the scalar offset (bytes):
+  // K step u of an operand staged as it lies starts u * 32 rows down, unit u of a row-wise one 64 (u / 2) elements
+  // along the rows and 128 (u % 2) rows down
+  const uint32_t ka2 = 2u * (uint32_t)lda * (TA ? BK : 128), kb2 = 2u * (uint32_t)ldb * (TB ? 128 : BK);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)(g.A + tile_a), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + tile_b), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_a2 = __builtin_amdgcn_make_buffer_rsrc((void*)((g.A2 ? g.A2 : g.A) + tile_a), 0, 0x7fffffff, 0x00020000);
@@ -321,7 +333,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   {                                                                                                     \
     const int t_ = min((T), total - 1);                                                                 \
     const __amdgpu_buffer_rsrc_t ra_ = t_ >= nk ? rsrc_a2 : rsrc_a;                                     \
-    const uint32_t so_ = (uint32_t)((t_ >= nk ? t_ - nk : t_) * BK) * ka2;                              \
+    const int u_ = t_ >= nk ? t_ - nk : t_;                                                             \
+    const uint32_t so_ = TA ? (uint32_t)u_ * ka2 : (uint32_t)(u_ >> 1) * 128u + (uint32_t)(u_ & 1) * ka2; \
     S##a0 = ld_buf(ra_, ga[0], so_); S##a1 = ld_buf(ra_, ga[1], so_);                                   \
     S##a2 = ld_buf(ra_, ga[2], so_); S##a3 = ld_buf(ra_, ga[3], so_);                                   \
   }
@@ -329,38 +342,47 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   {                                                                                                     \
     const int t_ = min((T), total - 1);                                                                 \
     const __amdgpu_buffer_rsrc_t rb_ = t_ >= nk ? rsrc_b2 : rsrc_b;                                     \
-    const uint32_t so_ = (uint32_t)((t_ >= nk ? t_ - nk : t_) * BK) * kb2;                              \
+    const int u_ = t_ >= nk ? t_ - nk : t_;                                                             \
+    const uint32_t so_ = TB ? (uint32_t)(u_ >> 1) * 128u + (uint32_t)(u_ & 1) * kb2 : (uint32_t)u_ * kb2; \
     S##b0 = ld_buf(rb_, gb[0], so_); S##b1 = ld_buf(rb_, gb[1], so_);                                   \
     S##b2 = ld_buf(rb_, gb[2], so_); S##b3 = ld_buf(rb_, gb[3], so_);                                   \
   }
 #define RA_W4_LOAD(S, T) { RA_W4_LOAD_A(S, T); RA_W4_LOAD_B(S, T); }
-#define RA_W4_STORE(S, BUF)                                                                             \
+  // set S holds the unit of K step U (modulo 4)
+#define RA_W4_STORE_A(S, U)                                                                             \
   {                                                                                                     \
-    *(uint4*)(&RA_W4_AS(BUF)[la[0]]) = S##a0; *(uint4*)(&RA_W4_AS(BUF)[la[1]]) = S##a1;                             \
-    *(uint4*)(&RA_W4_AS(BUF)[la[2]]) = S##a2; *(uint4*)(&RA_W4_AS(BUF)[la[3]]) = S##a3;                             \
-    *(uint4*)(&RA_W4_BS(BUF)[lb[0]]) = S##b0; *(uint4*)(&RA_W4_BS(BUF)[lb[1]]) = S##b1;                             \
-    *(uint4*)(&RA_W4_BS(BUF)[lb[2]]) = S##b2; *(uint4*)(&RA_W4_BS(BUF)[lb[3]]) = S##b3;                             \
+    uint16_t* const d_ = &RA_W4_AS(RA_W4_ABUF(U))[RA_W4_AHALF(U)];                                      \
+    *(uint4*)(d_ + la[0]) = S##a0; *(uint4*)(d_ + la[1]) = S##a1;                                       \
+    *(uint4*)(d_ + la[2]) = S##a2; *(uint4*)(d_ + la[3]) = S##a3;                                       \
+  }
+#define RA_W4_STORE_B(S, U)                                                                             \
+  {                                                                                                     \
+    uint16_t* const d_ = &RA_W4_BS(RA_W4_BBUF(U))[RA_W4_BHALF(U)];                                      \
+    *(uint4*)(d_ + lb[0]) = S##b0; *(uint4*)(d_ + lb[1]) = S##b1;                                       \
+    *(uint4*)(d_ + lb[2]) = S##b2; *(uint4*)(d_ + lb[3]) = S##b3;                                       \
   }
   const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wm * WM;
   const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wn * WN;
-  // row-wise fragment of K slice kk: row lo, chunk (2 kk + hi) ^ ((lo >> 2) & 3)
-  const int nsw = hi ^ ((lo >> 2) & 3);
-  const int natA0 = (wm * WM + lo) * A_STR + nsw * 8, natA1 = (wm * WM + lo) * A_STR + (nsw ^ 2) * 8;
-  const int natB0 = (wn * WN + lo) * B_STR + nsw * 8, natB1 = (wn * WN + lo) * B_STR + (nsw ^ 2) * 8;
-  // the eight fragments of K slice KK of buffer BUF into set F (F##a[0..3], F##b[0..3])
-#define RA_W4_FRAGS(F, BUF, KK)                                                                         \
+  // row-wise fragment of K slice k' (0-3) of a slab: row lo, chunk (2 k' + hi) ^ ((lo >> 1) & 7)
+  const int nsw = (hi ^ ((lo >> 1) & 7)) * 8;
+  const int natA0 = (wm * WM + lo) * WIDE_STR + nsw, natB0 = (wn * WN + lo) * WIDE_STR + nsw;
+  const int natA1 = natA0 ^ 16, natA2 = natA0 ^ 32, natA3 = natA0 ^ 48;
+  const int natB1 = natB0 ^ 16, natB2 = natB0 ^ 32, natB3 = natB0 ^ 48;
+#define RA_W4_NAT(X, Q) ((Q) == 0 ? nat##X##0 : (Q) == 1 ? nat##X##1 : (Q) == 2 ? nat##X##2 : nat##X##3)
+  // the eight fragments of K slice KK (0 or 1) of K step U (modulo 4) into set F (F##a[0..3], F##b[0..3])
+#define RA_W4_FRAGS(F, U, KK)                                                                           \
   _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                       \
     if (!TA) {                                                                                          \
-      F##a[i] = *(const bf16x8*)(&RA_W4_AS(BUF)[((KK) ? natA1 : natA0) + i * 32 * A_STR]);                          \
+      F##a[i] = *(const bf16x8*)(&RA_W4_AS(RA_W4_ABUF(U))[RA_W4_NAT(A, 2 * ((U) & 1) + (KK)) + i * 32 * WIDE_STR]); \
     } else {                                                                                            \
-      const uint16_t* p = &RA_W4_AS(BUF)[(KK) * 16 * A_STR + trA + i * 32];                                   \
+      const uint16_t* p = &RA_W4_AS(RA_W4_ABUF(U))[(KK) * 16 * A_STR + trA + i * 32];                   \
       s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);                                                 \
       F##a[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
     if (TB) {                                                                                           \
-      F##b[i] = *(const bf16x8*)(&RA_W4_BS(BUF)[((KK) ? natB1 : natB0) + i * 32 * B_STR]);                          \
+      F##b[i] = *(const bf16x8*)(&RA_W4_BS(RA_W4_BBUF(U))[RA_W4_NAT(B, 2 * ((U) & 1) + (KK)) + i * 32 * WIDE_STR]); \
     } else {                                                                                            \
-      const uint16_t* p = &RA_W4_BS(BUF)[(KK) * 16 * B_STR + trB + i * 32];                                   \
+      const uint16_t* p = &RA_W4_BS(RA_W4_BBUF(U))[(KK) * 16 * B_STR + trB + i * 32];                   \
       s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);                                                 \
       F##b[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
@@ -369,8 +391,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   _Pragma("unroll") for (int i = 0; i < 4; i++)                                                         \
     _Pragma("unroll") for (int j = 0; j < 4; j++)                                                       \
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F##a[i], F##b[j], acc[i][j], 0, 0, 0);
-  // one K step: slab in buffer CUR (its slice 0 already in set F); set S of staging registers holds the next slab,
-  // which goes to the other buffer, and is then reloaded with slab NEXT_T
   // A single wavefront per SIMD issues in order: the MFMA pipe only stays busy if every MFMA is followed by at most
   // a few other instructions.  Sixteen groups of one MFMA, one LDS read and one LDS write or global load.
 #define RA_W4_SCHED(WRITES, LOADS)                                                                      \
@@ -380,19 +400,21 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
     if (m_ < (WRITES)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                               \
     else if (m_ < (WRITES) + (LOADS)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                \
   }
-  // one K step: slab in buffer CUR (its slice 0 already in set F); set S of staging registers holds the next slab,
-  // which goes to the other buffer, and is then reloaded with slab NEXT_T
-#define RA_W4_STEP(CUR, S, NEXT_T)                                                                      \
+  // K step U (modulo 4; its slice 0 already in set F), T0 its index.  S1 is the register set of step U + 1, S2 that
+  // of step U + 2: a row-wise operand's unit goes to LDS from S2, the other kind's from S1, and the set is then
+  // requested again for four K steps later.
+#define RA_W4_STEP(U, S1, S2, T0)                                                                       \
   {                                                                                                     \
-    RA_W4_FRAGS(G, CUR, 1);                                                                             \
-    RA_W4_STORE(S, (CUR) ^ 1);                                                                          \
-    RA_W4_LOAD_A(S, NEXT_T);                                                                            \
+    RA_W4_FRAGS(G, U, 1);                                                                               \
+    if (TA) { RA_W4_STORE_A(S1, ((U) + 1) & 3); } else { RA_W4_STORE_A(S2, ((U) + 2) & 3); }            \
+    if (TB) { RA_W4_STORE_B(S2, ((U) + 2) & 3); } else { RA_W4_STORE_B(S1, ((U) + 1) & 3); }            \
+    if (TA) { RA_W4_LOAD_A(S1, (T0) + 5); } else { RA_W4_LOAD_A(S2, (T0) + 6); }                        \
     RA_W4_MFMA(F);                                                                                      \
     RA_W4_SCHED(8, 4);                                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
     __syncthreads();                                                                                    \
-    RA_W4_FRAGS(F, (CUR) ^ 1, 0);                                                                       \
-    RA_W4_LOAD_B(S, NEXT_T);                                                                            \
+    RA_W4_FRAGS(F, ((U) + 1) & 3, 0);                                                                   \
+    if (TB) { RA_W4_LOAD_B(S2, (T0) + 6); } else { RA_W4_LOAD_B(S1, (T0) + 5); }                        \
     RA_W4_MFMA(G);                                                                                      \
     RA_W4_SCHED(0, 4);                                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
@@ -402,28 +424,37 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   RA_W4_LOAD(Q, 1);
   RA_W4_LOAD(R, 2);
   RA_W4_LOAD(T, 3);
-  RA_W4_STORE(P, 0);
+  RA_W4_STORE_A(P, 0);
+  RA_W4_STORE_B(P, 0);
   RA_W4_LOAD(P, 4);
+  if (!TA) { RA_W4_STORE_A(Q, 1); RA_W4_LOAD_A(Q, 5); }
+  if (TB) { RA_W4_STORE_B(Q, 1); RA_W4_LOAD_B(Q, 5); }
   __syncthreads();
   RA_W4_FRAGS(F, 0, 0);
-  // K is a multiple of 64: an even number of slabs; four steps per trip, two more when that leaves a remainder
+  // K is a multiple of 64: an even number of K steps; four steps per trip, two more when that leaves a remainder
   int it = 0;
   for (; it + 4 <= total; it += 4) {
-    RA_W4_STEP(0, Q, it + 5);
-    RA_W4_STEP(1, R, it + 6);
-    RA_W4_STEP(0, T, it + 7);
-    RA_W4_STEP(1, P, it + 8);
+    RA_W4_STEP(0, Q, R, it);
+    RA_W4_STEP(1, R, T, it + 1);
+    RA_W4_STEP(2, T, P, it + 2);
+    RA_W4_STEP(3, P, Q, it + 3);
   }
   if (it < total) {
-    RA_W4_STEP(0, Q, it + 5);
-    RA_W4_STEP(1, R, it + 6);
+    RA_W4_STEP(0, Q, R, it);
+    RA_W4_STEP(1, R, T, it + 1);
   }
 #undef RA_W4_STEP
 #undef RA_W4_AS
 #undef RA_W4_BS
+#undef RA_W4_ABUF
+#undef RA_W4_BBUF
+#undef RA_W4_AHALF
+#undef RA_W4_BHALF
+#undef RA_W4_NAT
 #undef RA_W4_MFMA
 #undef RA_W4_FRAGS
-#undef RA_W4_STORE
+#undef RA_W4_STORE_A
+#undef RA_W4_STORE_B
 #undef RA_W4_LOAD
 #undef RA_W4_LOAD_A
 #undef RA_W4_LOAD_B
