@@ -486,11 +486,11 @@ def bench_ffn(args):
     a_out = torch.empty(slab, f, dtype=torch.bfloat16, device=dev)
     gemm_ms = _event_ms(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out), 5)
     gemm_tf = 2.0 * slab * d * f / (gemm_ms * 1e-3) / 1e12
-    # the tile kernel the library picks for (slab, f): the 256 x 256 one when its grid fills at least 80 % of the last
-    # round of 256 CUs, else the 256 x 128 one (the shapes here divide both)
-    n256 = (slab // 256) * (f // 256)
-    gemm_name = ("gemm_bf16_w4_kernel<false, false>" if n256 / (math.ceil(n256 / 256.0) * 256.0) >= 0.8
-                 else "gemm_bf16_kernel<false, false, 256, 128, 4, 2, true>")
+    # the tile kernel the library picks for (slab, f): 256 x 256 or 256 x 128 over four wavefronts, whichever takes
+    # fewer rounds of 256 CUs weighted by the cost of a round (1.62 : 1); the shapes here divide both
+    r256 = math.ceil((slab // 256) * (f // 256) / 256.0) * 1.62
+    r128 = math.ceil((slab // 256) * (f // 128) / 256.0) * 1.0
+    gemm_name = "gemm_bf16_w4_kernel<false, false, %d>" % (256 if r256 <= r128 else 128)
     sclk = None if args.no_extras else _sclk_under_load(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out))
     cpu = None
     if not args.no_cpu:
@@ -519,9 +519,9 @@ def bench_ffn(args):
         "roofline": {"bound": "mfma", "kernel": "%s (a = x w1 of one launch)" % gemm_name,
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
-                     "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("gemm_bf16_w4_kernel<false,false>")
+                     "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("gemm_bf16_w4_kernel<false,false,256>")
                                  if (T, slab) == (65536, 16384) else None),
-                     "mfma_util_pmc": {"kernel": (_measured(MFMA_PROFILE, "mfma_util").get("gemm_bf16_w4_kernel<false,false>")
+                     "mfma_util_pmc": {"kernel": (_measured(MFMA_PROFILE, "mfma_util").get("gemm_bf16_w4_kernel<false,false,256>")
                                                   if (T, slab) == (65536, 16384) else None),
                                        "source": "profiles/" + MFMA_PROFILE},
                      "kernel_ms": {gemm_name: round(gemm_ms, 3)},

@@ -294,7 +294,8 @@ typedef struct ra_swiglu_params {
                                      0 = recompute them from x (the reference's default policy) */
   int32_t gemm_tile;              /* 0: the library picks the tile kernel of each product (the default).  1 + t forces
                                      tile kernel t wherever the shape divides (0: 256 x 256 over four wavefronts,
-                                     1: 256 x 128, 2: 128 x 128), so that tests reach every kernel */
+                                     1: 256 x 128 over eight, 2: 128 x 128, 3: 256 x 128 over four), so that tests reach every
+                                     kernel */
 } ra_swiglu_params;
 
 int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream);

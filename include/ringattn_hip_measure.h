@@ -19,7 +19,8 @@ enum { RA_BWD_PART_DQ = 1, RA_BWD_PART_DKV = 2 };
 int ra_attn_bwd_block_part(const ra_attn_bwd_params* p, int32_t part, ra_stream_t stream);
 
 /* ra_gemm_bf16 with the tile kernel named: tile -1 = the library's choice, 0: 256 x 256 over four wavefronts,
- * 1: 256 x 128, 2: 128 x 128 (a forced tile still gives way to a smaller one where the shape does not divide). */
+ * 1: 256 x 128 over eight, 2: 128 x 128, 3: 256 x 128 over four (a forced tile still gives way to another one where
+ * the shape does not divide). */
 int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,
                       int32_t trans_b, int32_t c_dtype, int32_t beta_one, int32_t tile, ra_stream_t stream);
 

@@ -401,7 +401,7 @@ int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream) {
   RA_REQUIRE(p, RA_ERR_INVALID, "swiglu_fwd: null params");
   RA_REQUIRE(p->x && p->w1 && p->w2 && p->w3 && p->a && p->b && p->h && p->y, RA_ERR_INVALID, "swiglu_fwd: null tensor");
   RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_fwd: empty shape");
-  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 3, RA_ERR_INVALID, "swiglu_fwd: gemm_tile %d outside [0, 3]", p->gemm_tile);
+  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 4, RA_ERR_INVALID, "swiglu_fwd: gemm_tile %d outside [0, 4]", p->gemm_tile);
   return swiglu_fwd(p, (hipStream_t)stream);
 }
 
@@ -411,7 +411,7 @@ int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream) {
                  p->dw3 && p->da && p->db,
              RA_ERR_INVALID, "swiglu_bwd: null tensor");
   RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_bwd: empty shape");
-  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 3, RA_ERR_INVALID, "swiglu_bwd: gemm_tile %d outside [0, 3]", p->gemm_tile);
+  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 4, RA_ERR_INVALID, "swiglu_bwd: gemm_tile %d outside [0, 4]", p->gemm_tile);
   return swiglu_bwd(p, (hipStream_t)stream);
 }
 
@@ -428,7 +428,7 @@ int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t
   RA_REQUIRE(A && Bm && C, RA_ERR_INVALID, "gemm_bf16_tile: null pointer");
   RA_REQUIRE(M > 0 && N > 0 && K > 0, RA_ERR_INVALID, "gemm_bf16_tile: empty shape");
   RA_REQUIRE(c_dtype == RA_F32 || c_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "gemm_bf16_tile: c_dtype %d", c_dtype);
-  RA_REQUIRE(tile >= -1 && tile <= 2, RA_ERR_INVALID, "gemm_bf16_tile: tile %d outside [-1, 2]", tile);
+  RA_REQUIRE(tile >= -1 && tile <= 3, RA_ERR_INVALID, "gemm_bf16_tile: tile %d outside [-1, 3]", tile);
   return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, tile, (hipStream_t)stream);
 }
 

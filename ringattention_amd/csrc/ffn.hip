@@ -2,10 +2,10 @@
 // blockwise_feedforward (ringattention_jax.py:333-352) scans over chunks of tokens.
 //
 // GEMM: C (M,N) = op(A) op(B) [+ op(A2) op(B2)], fp32 accumulation in v_mfma_f32_32x32x16_bf16.
-//   The tile is chosen per problem: 256 x 256 over 4 wavefronts (gemm_bf16_w4_kernel: each wavefront
-//   128 x 128, eight operand fragments from LDS per sixteen MFMAs) when that still gives every CU work;
-//   otherwise gemm_bf16_kernel with WGM x WGN wavefronts on a BM x BN tile (256 x 128 over 8, 128 x 128
-//   over 4), K step 64, LDS double buffered.
+//   The tile is chosen per problem: 256 x 256 or 256 x 128 over 4 wavefronts, one per SIMD (gemm_bf16_w4_kernel:
+//   each wavefront 128 x 128 or 128 x 64; eight or six operand fragments from LDS per sixteen or eight MFMAs),
+//   whichever fills the CUs in fewer weighted rounds; gemm_bf16_kernel with WGM x WGN wavefronts on a BM x BN tile
+//   (256 x 128 over 8, 128 x 128 over 4; K step 64, LDS double buffered) for what those do not divide or reach.
 //   An operand whose contraction index is contiguous in memory is staged row-major and read with
 //   16-byte LDS reads; one whose contraction index is the slow axis is staged as it lies in memory
 //   and read with ds_read_b64_tr_b16, so no layout ever needs a transposing copy.
@@ -256,9 +256,11 @@ __device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t vo
   const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
   return uint4{v[0], v[1], v[2], v[3]};
 }
-template <bool TA, bool TB>
+template <bool TA, bool TB, int BN>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
-  constexpr int BM = 256, BN = 256, BK = 32, NT = 256, WM = 128, WN = 128;
+  static_assert(BN == 256 || BN == 128, "tile width");
+  // NJ: 32-column blocks of a wavefront's part of C; NBC: 16-byte chunks per thread and staging unit of B
+  constexpr int BM = 256, BK = 32, NT = 256, WM = 128, WN = BN / 2, NJ = WN / 32, NBC = BN / 64;
   // An operand whose rows run along K ("row-wise": A unless TA, B if TB) is fetched in whole 128-byte lines: a
   // staging unit of such an operand is 128 of the tile's 256 rows times 64 K positions, so that two consecutive K
   // steps bring in one slab of two K steps (unit u = slab u / 2, row half u % 2) and every request that reaches the
@@ -282,7 +284,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
 #define RA_W4_ABUF(U) (TA ? ((U) & 1) : (((U) >> 1) & 1))
 #define RA_W4_BBUF(U) (TB ? (((U) >> 1) & 1) : ((U) & 1))
 #define RA_W4_AHALF(U) (TA ? 0 : ((U) & 1) * 128 * WIDE_STR)
-#define RA_W4_BHALF(U) (TB ? ((U) & 1) * 128 * WIDE_STR : 0)
+#define RA_W4_BHALF(U) (TB ? ((U) & 1) * (BN / 2) * WIDE_STR : 0)
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
@@ -290,11 +292,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   if (!tile_of_block(g.M / BM, g.N / BN, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
 
-  f32x16 acc[4][4];
+  f32x16 acc[4][NJ];
 #pragma unroll
   for (int i = 0; i < 4; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NJ; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   // buffer descriptors that start at the tile's origin; the unit's position goes into the scalar offset (bytes):
   // K step u of an operand staged as it lies starts u * 32 rows down, unit u of a row-wise one 64 (u / 2) elements
   // along the rows and 128 (u % 2) rows down
-  const uint32_t ka2 = 2u * (uint32_t)lda * (TA ? BK : 128), kb2 = 2u * (uint32_t)ldb * (TB ? 128 : BK);
+  const uint32_t ka2 = 2u * (uint32_t)lda * (TA ? BK : 128), kb2 = 2u * (uint32_t)ldb * (TB ? BN / 2 : BK);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)(g.A + tile_a), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + tile_b), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_a2 = __builtin_amdgcn_make_buffer_rsrc((void*)((g.A2 ? g.A2 : g.A) + tile_a), 0, 0x7fffffff, 0x00020000);
@@ -345,7 +347,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
     const int u_ = t_ >= nk ? t_ - nk : t_;                                                             \
     const uint32_t so_ = TB ? (uint32_t)(u_ >> 1) * 128u + (uint32_t)(u_ & 1) * kb2 : (uint32_t)u_ * kb2; \
     S##b0 = ld_buf(rb_, gb[0], so_); S##b1 = ld_buf(rb_, gb[1], so_);                                   \
-    S##b2 = ld_buf(rb_, gb[2], so_); S##b3 = ld_buf(rb_, gb[3], so_);                                   \
+    if (NBC == 4) { S##b2 = ld_buf(rb_, gb[2], so_); S##b3 = ld_buf(rb_, gb[3], so_); }                 \
   }
 #define RA_W4_LOAD(S, T) { RA_W4_LOAD_A(S, T); RA_W4_LOAD_B(S, T); }
   // set S holds the unit of K step U (modulo 4)
@@ -359,7 +361,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   {                                                                                                     \
     uint16_t* const d_ = &RA_W4_BS(RA_W4_BBUF(U))[RA_W4_BHALF(U)];                                      \
     *(uint4*)(d_ + lb[0]) = S##b0; *(uint4*)(d_ + lb[1]) = S##b1;                                       \
-    *(uint4*)(d_ + lb[2]) = S##b2; *(uint4*)(d_ + lb[3]) = S##b3;                                       \
+    if (NBC == 4) { *(uint4*)(d_ + lb[2]) = S##b2; *(uint4*)(d_ + lb[3]) = S##b3; }                     \
   }
   const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wm * WM;
   const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wn * WN;
@@ -379,6 +381,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
       s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);                                                 \
       F##a[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
+    if (i >= NJ) continue;                                                                              \
     if (TB) {                                                                                           \
       F##b[i] = *(const bf16x8*)(&RA_W4_BS(RA_W4_BBUF(U))[RA_W4_NAT(B, 2 * ((U) & 1) + (KK)) + i * 32 * WIDE_STR]); \
     } else {                                                                                            \
@@ -389,16 +392,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   }
 #define RA_W4_MFMA(F)                                                                                   \
   _Pragma("unroll") for (int i = 0; i < 4; i++)                                                         \
-    _Pragma("unroll") for (int j = 0; j < 4; j++)                                                       \
+    _Pragma("unroll") for (int j = 0; j < NJ; j++)                                                      \
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F##a[i], F##b[j], acc[i][j], 0, 0, 0);
   // A single wavefront per SIMD issues in order: the MFMA pipe only stays busy if every MFMA is followed by at most
-  // a few other instructions.  Sixteen groups of one MFMA, one LDS read and one LDS write or global load.
+  // a few other instructions.  One group per MFMA: the MFMA, its share of the LDS reads, and one LDS write or,
+  // once the writes are out, its share of the global loads.
+  constexpr int NM = 4 * NJ, RD = (TA ? 8 : 4) + (TB ? NJ : 2 * NJ), RPG = (RD + NM - 1) / NM;
 #define RA_W4_SCHED(WRITES, LOADS)                                                                      \
-  _Pragma("unroll") for (int m_ = 0; m_ < 16; m_++) {                                                   \
+  _Pragma("unroll") for (int m_ = 0; m_ < NM; m_++) {                                                   \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                  \
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                                  \
+    __builtin_amdgcn_sched_group_barrier(0x100, RPG, 0);                                                \
     if (m_ < (WRITES)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                               \
-    else if (m_ < (WRITES) + (LOADS)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                \
+    else if ((m_ - (WRITES)) * (((LOADS) + NM - (WRITES) - 1) / (NM - (WRITES))) < (LOADS))             \
+      __builtin_amdgcn_sched_group_barrier(0x020, ((LOADS) + NM - (WRITES) - 1) / (NM - (WRITES)), 0);  \
   }
   // K step U (modulo 4; its slice 0 already in set F), T0 its index.  S1 is the register set of step U + 1, S2 that
   // of step U + 2: a row-wise operand's unit goes to LDS from S2, the other kind's from S1, and the set is then
@@ -410,16 +416,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
     if (TB) { RA_W4_STORE_B(S2, ((U) + 2) & 3); } else { RA_W4_STORE_B(S1, ((U) + 1) & 3); }            \
     if (TA) { RA_W4_LOAD_A(S1, (T0) + 5); } else { RA_W4_LOAD_A(S2, (T0) + 6); }                        \
     RA_W4_MFMA(F);                                                                                      \
-    RA_W4_SCHED(8, 4);                                                                                  \
+    RA_W4_SCHED(4 + NBC, 4);                                                                                \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
     __syncthreads();                                                                                    \
     RA_W4_FRAGS(F, ((U) + 1) & 3, 0);                                                                   \
     if (TB) { RA_W4_LOAD_B(S2, (T0) + 6); } else { RA_W4_LOAD_B(S1, (T0) + 5); }                        \
     RA_W4_MFMA(G);                                                                                      \
-    RA_W4_SCHED(0, 4);                                                                                  \
+    RA_W4_SCHED(0, NBC);                                                                                \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
-  bf16x8 Fa[4], Fb[4], Ga[4], Gb[4];
+  bf16x8 Fa[4], Fb[NJ], Ga[4], Gb[NJ];
   RA_W4_LOAD(P, 0);
   RA_W4_LOAD(Q, 1);
   RA_W4_LOAD(R, 2);
@@ -469,10 +475,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   else if (!g.beta_one) store_tile<1>(acc, patch, patch + 32 * 36, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
   else store_tile<2>(acc, patch, patch + 32 * 36, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
 }
-template <bool TA, bool TB>
+template <bool TA, bool TB, int BN>
 static int launch_w4(const GemmArgs& g, hipStream_t s) {
-  const long long nwg = ((long long)(g.M / 256) * (g.N / 256) + 7) / 8 * 8;
-  gemm_bf16_w4_kernel<TA, TB><<<dim3((unsigned)nwg), 256, 0, s>>>(g);
+  const long long nwg = ((long long)(g.M / 256) * (g.N / BN) + 7) / 8 * 8;
+  gemm_bf16_w4_kernel<TA, TB, BN><<<dim3((unsigned)nwg), 256, 0, s>>>(g);
   RA_CHECK_LAUNCH("gemm_bf16_w4");
   return RA_OK;
 }
@@ -485,43 +491,46 @@ static int launch_tile(const GemmArgs& g, hipStream_t s) {
   return RA_OK;
 }
 
-// Tile choice.  One workgroup of the large tiles fills a CU's LDS, so the grid runs in rounds of (number of CUs)
-// workgroups: take the largest tile whose last round is not mostly idle.
-static int pick_tile(int M, int N) {
+// Tile choice.  One workgroup of the large tiles fills a CU, so the grid runs in rounds of (number of CUs)
+// workgroups: take the tile whose rounds, weighted by what a round of it costs (measured on full grids: a round of
+// 256 x 256 tiles takes 1.62 times one of 256 x 128 over four wavefronts, which does half the work), take least.
+static bool w4_reach_ok(int M, int N, int K) {
+  // the 4-wavefront kernels address an operand through a buffer descriptor at its tile's origin with 32-bit byte
+  // offsets: what a tile can reach (a whole operand in the worst case) must stay below 2^31 bytes
+  return M % 256 == 0 && (int64_t)M * K < (1LL << 30) && (int64_t)N * K < (1LL << 30);
+}
+static int pick_tile(int M, int N, int K) {
   static const int ncu = [] {     // initialised once, thread-safe
     int dev = 0, n = 0;
     hipDeviceProp_t pr;
     if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&pr, dev) == hipSuccess) n = pr.multiProcessorCount;
     return n > 0 ? n : 256;
   }();
-  auto eff = [&](int bm, int bn) {
-    if (M % bm || N % bn) return 0.0;
-    const double n = (double)(M / bm) * (N / bn);
-    return n / (ceil(n / ncu) * ncu);
-  };
-  if (eff(256, 256) >= 0.8) return 0;
-  if (eff(256, 128) >= 0.8) return 1;
-  if (eff(256, 256) >= 0.66) return 0;
-  if (eff(256, 128) >= 0.66) return 1;
-  return 2;
+  auto rounds = [&](int bm, int bn) { return ceil((double)(M / bm) * (N / bn) / ncu); };
+  const bool w4 = w4_reach_ok(M, N, K);
+  int best = 2;
+  double cost = rounds(128, 128) * 0.70;
+  if (M % 256 == 0 && rounds(256, 128) * 1.16 < cost) { best = 1; cost = rounds(256, 128) * 1.16; }
+  if (w4 && rounds(256, 128) * 1.00 < cost) { best = 3; cost = rounds(256, 128) * 1.00; }
+  if (w4 && N % 256 == 0 && rounds(256, 256) * 1.62 <= cost) { best = 0; cost = rounds(256, 256) * 1.62; }
+  return best;
 }
 
-// tile: -1 = pick_tile, else the tile kernel to force (0: 256 x 256, 1: 256 x 128, 2: 128 x 128), which still
-// falls back to a smaller one when the shape does not divide
+// tile: -1 = pick_tile, else the tile kernel to force (0: 256 x 256 over four wavefronts, 1: 256 x 128 over eight,
+// 2: 128 x 128, 3: 256 x 128 over four), which still falls back to another one when the shape does not divide
 template <bool TA, bool TB>
 static int launch_gemm(const GemmArgs& g, int tile, hipStream_t s) {
   if (g.M % 128 || g.N % 128 || g.K % GBK) {
     set_error("gemm_bf16: M, N must be multiples of 128 and K of 64 (got %d, %d, %d)", g.M, g.N, g.K);
     return RA_ERR_UNSUPPORTED;
   }
-  int t = tile >= 0 ? tile : pick_tile(g.M, g.N);
-  if (t == 0 && (g.M % 256 || g.N % 256)) t = 1;
-  // the 4-wavefront kernel addresses an operand through a buffer descriptor at its tile's origin with 32-bit byte
-  // offsets: what a tile can reach (a whole operand in the worst case) must stay below 2^31 bytes
-  if (t == 0 && ((int64_t)g.M * g.K >= (1LL << 30) || (int64_t)g.N * g.K >= (1LL << 30))) t = 1;
+  int t = tile >= 0 ? tile : pick_tile(g.M, g.N, g.K);
+  if (t == 0 && g.N % 256) t = 3;
+  if ((t == 0 || t == 3) && !w4_reach_ok(g.M, g.N, g.K)) t = 1;
   if (t == 1 && g.M % 256) t = 2;
   switch (t) {
-    case 0: return launch_w4<TA, TB>(g, s);
+    case 0: return launch_w4<TA, TB, 256>(g, s);
+    case 3: return launch_w4<TA, TB, 128>(g, s);
     case 1: return launch_tile<TA, TB, 256, 128, 4, 2, true>(g, s);
     default: return launch_tile<TA, TB, 128, 128, 2, 2, false>(g, s);
   }

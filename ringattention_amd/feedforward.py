@@ -167,7 +167,7 @@ class SwiGLU(torch.nn.Module):
 
     def __init__(self, hidden, intermediate, device=None, init_std=0.02, gemm_tile=None):
         super().__init__()
-        # None: the library picks the GEMM tile kernel; 0 / 1 / 2 force one (ra_swiglu_params.gemm_tile), for tests
+        # None: the library picks the GEMM tile kernel; 0 - 3 force one (ra_swiglu_params.gemm_tile), for tests
         self.gemm_tile = 0 if gemm_tile is None else int(gemm_tile) + 1
         mk = lambda i, o: torch.nn.Parameter(
             (torch.randn(i, o, device=device, dtype=torch.float32) * init_std).to(torch.bfloat16))
@@ -222,7 +222,7 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
 
 def gemm_bf16(A, B, trans_a=False, trans_b=False, out_dtype=torch.bfloat16, out=None, accumulate=False, tile=None):
     """C = op(A) op(B) with the library's bf16 MFMA GEMM (used by the SwiGLU kernels; exposed for tests).
-    ``tile`` 0 / 1 / 2 names the tile kernel (ra_gemm_bf16_tile); None lets the library choose."""
+    ``tile`` 0 - 3 names the tile kernel (ra_gemm_bf16_tile); None lets the library choose."""
     M = A.shape[1] if trans_a else A.shape[0]
     K = A.shape[0] if trans_a else A.shape[1]
     N = B.shape[0] if trans_b else B.shape[1]

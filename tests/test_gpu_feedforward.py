@@ -36,10 +36,10 @@ def test_gemm_layouts(ta, tb, shape):
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("tile", [0, 1, 2])
-@pytest.mark.parametrize("shape", [(768, 512, 320), (1280, 256, 128)])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("shape", [(768, 512, 320), (1280, 256, 128), (512, 384, 448)])
 def test_gemm_every_tile_kernel(ta, tb, tile, shape):
-    """Each tile kernel (0: 256 x 256 over four wavefronts, 1: 256 x 128, 2: 128 x 128) on shapes whose tile
+    """Each tile kernel (0: 256 x 256 over four wavefronts, 1: 256 x 128 over eight, 2: 128 x 128, 3: 256 x 128 over four) on shapes whose tile
     counts are no multiple of the 8 XCDs or of the tile-row group, so the workgroup -> tile order and its
     surplus workgroups are exercised; ra_gemm_bf16_tile names the tile kernel that ra_gemm_bf16 would pick itself."""
     M, N, K = shape
@@ -62,7 +62,7 @@ def test_gemm_rejects_ragged_shapes():
         ra.gemm_bf16(A, B)
 
 
-@pytest.mark.parametrize("tile,shape", [(None, (256, 256, 384)), (0, (512, 256, 768)), (1, (512, 256, 768))])
+@pytest.mark.parametrize("tile,shape", [(None, (256, 256, 384)), (0, (512, 256, 768)), (1, (512, 256, 768)), (3, (512, 256, 768))])
 def test_swiglu_forward_backward_match_autograd(tile, shape):
     """SwiGLU forward and backward (including the two-operand-pair GEMM of dx and the fp32 accumulation of the
     weight gradients) with the library's own tile choice and with each of the large tile kernels forced."""
