@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the ring-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|inference|copy|decode_step|rmsnorm|dropout32k]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload attn32k|ring131k|ffn|decode|inference|copy|decode_step|rmsnorm|dropout32k|c1|mfma_probe|vendor_sdpa]
 
 One step = one pass of the hot path over one batch of synthetic input already resident in HBM.
 Default workload ``attn32k`` is the configuration the headline metric is quoted on: blockwise
@@ -708,6 +708,47 @@ def bench_inference(args):
             "cpu_baseline": None}
 
 
+def bench_vendor_sdpa(args):
+    """The attn32k shape through torch's scaled_dot_product_attention (the fused attention kernels the ROCm build of
+    PyTorch ships), timed the same way: a yardstick measured on the same box, not part of the library."""
+    import torch
+    import torch.nn.functional as F
+    from torch.nn.attention import sdpa_kernel, SDPBackend
+    dev = "cuda:0"
+    B, H, S, D = 1, 32, args.seq_len or 32768, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    q, k, v = ((torch.randn(B, H, S, D, device=dev, generator=g) / D ** 0.5).to(torch.bfloat16).requires_grad_(True)
+               for _ in range(3))
+    do = torch.randn(B, H, S, D, device=dev, generator=g).to(torch.bfloat16)
+    flops = 14.0 * D * (S * (S + 1) / 2.0) * B * H
+    res = {}
+    for name, be in (("flash", SDPBackend.FLASH_ATTENTION), ("efficient", SDPBackend.EFFICIENT_ATTENTION)):
+        try:
+            with sdpa_kernel(be):
+                def step():
+                    q.grad = k.grad = v.grad = None
+                    F.scaled_dot_product_attention(q, k, v, is_causal=True).backward(do)
+
+                def fwd():
+                    with torch.no_grad():
+                        F.scaled_dot_product_attention(q, k, v, is_causal=True)
+                ms = _time_steps(step, args.steps, args.warmup)
+                ms_f = _time_steps(fwd, args.steps, args.warmup)
+            res[name] = {"ms_per_step": round(ms, 3), "tflops": round(flops / (ms * 1e-3) / 1e12, 1),
+                         "fwd_ms": round(ms_f, 3)}
+        except Exception as e:                     # a backend this build does not have
+            res[name] = {"error": repr(e)[:200]}
+    ok = [r for r in res.values() if "ms_per_step" in r]
+    if not ok:
+        raise RuntimeError("no fused attention backend of torch ran: %r" % res)
+    best = min(ok, key=lambda r: r["ms_per_step"])
+    return {"metric": "vendor_sdpa_fwd_bwd_tflops", "value": best["tflops"], "unit": "TFLOP/s",
+            "ms_per_step": best["ms_per_step"], "dtype": "bf16",
+            "config": {"workload": "vendor_sdpa", "B": B, "H": H, "S": S, "D": D, "is_causal": True, "backends": res,
+                       "flop_convention": "4*D fwd + 10*D bwd per unmasked (q,k) pair per head"},
+            "roofline": None, "cpu_baseline": None}
+
+
 def bench_mfma_probe(args):
     """What the matrix pipes sustain on bf16 MFMAs alone, by operand activity (ra_mfma_rate_probe): the rate, the
     clock and the board power of a two-second run each.  The value is the rate on random operands: the ceiling a
@@ -745,7 +786,7 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default=None, choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
-                                                              "dropout32k", "c1", "mfma_probe"])
+                                                              "dropout32k", "c1", "mfma_probe", "vendor_sdpa"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
                     help="attention workloads: head size (the number of heads follows, H * D = 4096)")
@@ -816,6 +857,8 @@ def main():
         r = bench_inference(args)
     elif args.workload == "mfma_probe":
         r = bench_mfma_probe(args)
+    elif args.workload == "vendor_sdpa":
+        r = bench_vendor_sdpa(args)
     else:
         r = bench_ffn(args)
     line = {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "n_gpus": 1, "steps": args.steps,
