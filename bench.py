@@ -487,8 +487,8 @@ def bench_ffn(args):
     gemm_ms = _event_ms(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out), 5)
     gemm_tf = 2.0 * slab * d * f / (gemm_ms * 1e-3) / 1e12
     # the tile kernel the library picks for (slab, f): 256 x 256 or 256 x 128 over four wavefronts, whichever takes
-    # fewer rounds of 256 CUs weighted by the cost of a round (1.62 : 1); the shapes here divide both
-    r256 = math.ceil((slab // 256) * (f // 256) / 256.0) * 1.62
+    # fewer rounds of 256 CUs weighted by the cost of a round (1.72 : 1); the shapes here divide both
+    r256 = math.ceil((slab // 256) * (f // 256) / 256.0) * 1.72
     r128 = math.ceil((slab // 256) * (f // 128) / 256.0) * 1.0
     gemm_name = "gemm_bf16_w4_kernel<false, false, %d>" % (256 if r256 <= r128 else 128)
     sclk = None if args.no_extras else _sclk_under_load(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out))

@@ -244,49 +244,39 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_bf16_kernel(GemmArgs g) {
   else store_tile<2>(acc, patch, patch, g.C, g.N, m0 + wm * WM, n0 + wn * WN, lane);
 }
 
-// 256 x 256 tile over FOUR wavefronts (2 x 2), one per SIMD with all 512 registers: each wavefront owns 128 x 128
-// of C (256 accumulator registers), so a K slice of 16 takes eight operand fragments from LDS for sixteen MFMAs -
-// half the LDS bytes per MFMA of the eight-wavefront tile, which is LDS-bound.  With a single wavefront per SIMD
-// nothing hides latency but the wavefront's own pipelining: K step 32 = two slices; the fragments of a slice are
-// requested from LDS one slice (sixteen MFMAs) before their use, across the barrier of the K step; a K slab stays
-// in flight from global memory for four K steps in one of four register sets.
-// a 16-byte load through a buffer descriptor: scalar base and scalar offset, one 32-bit byte offset per lane
-typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ uint4 ld_buf(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
-  const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, soff, 0);
-  return uint4{v[0], v[1], v[2], v[3]};
-}
+// 256 x BN tile (BN 256 or 128) over FOUR wavefronts (2 x 2), one per SIMD with all 512 registers: each wavefront
+// owns 128 x BN/2 of C (256 accumulator registers at BN = 256), so a K slice of 16 takes eight operand fragments from
+// LDS for sixteen MFMAs - half the LDS bytes per MFMA of the eight-wavefront tile.  With a single wavefront per SIMD
+// nothing hides latency but the wavefront's own pipelining, and what the loop costs beside its MFMAs is mostly the
+// energy of moving operands (the board runs it at its power limit), so:
+//   * operands go from global memory straight into LDS (buffer_load ... lds: sixteen bytes a lane, the 64 lanes of
+//     an instruction fill 1 KB of consecutive LDS): no staging registers, no LDS writes by the wavefronts;
+//   * the unit is a slab of 64 K positions (four K slices) of the whole tile, 32 KB an operand at BN = 256, fetched
+//     as whole 128-byte lines whichever way the operand lies;
+//   * A has three slab buffers and B two (160 KB at BN = 256), so that a slab step can issue its loads evenly - B's
+//     in its first and last quarter, A's in the second and third, four a wavefront and quarter - and every load has
+//     between 2.5 quarters and a whole slab step to land;
+//   * the barrier between slabs is a bare s_barrier behind an s_waitcnt that leaves the eight newest loads (the slab
+//     after next of A) in flight; __syncthreads() would wait for all of them.
+// LDS layout of a slab.  Row-wise operand (rows run along K: A unless TA, B if TB): one row of 64 elements = eight
+// 16-byte chunks per tile row, chunk c of row r at position c ^ ((r >> 1) & 7).  K-major operand (stored (K, M) or
+// (K, N)): 64 rows of W = 256 or BN elements, chunk c of row r at position c ^ ((r & 3) << 2).  Both make the
+// fragment reads (16-byte reads of a row-wise slab, ds_read_b64_tr_b16 of a K-major one) conflict-free without
+// padding, and the permutation is done by the loads: lane l of a load fetches the chunk that belongs at position l.
 template <bool TA, bool TB, int BN>
 __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   static_assert(BN == 256 || BN == 128, "tile width");
-  // NJ: 32-column blocks of a wavefront's part of C; NBC: 16-byte chunks per thread and staging unit of B
-  constexpr int BM = 256, BK = 32, NT = 256, WM = 128, WN = BN / 2, NJ = WN / 32, NBC = BN / 64;
-  // An operand whose rows run along K ("row-wise": A unless TA, B if TB) is fetched in whole 128-byte lines: a
-  // staging unit of such an operand is 128 of the tile's 256 rows times 64 K positions, so that two consecutive K
-  // steps bring in one slab of two K steps (unit u = slab u / 2, row half u % 2) and every request that reaches the
-  // L2 is a full line, where rows of one K step would be 64-byte halves requested twice.  In LDS such a slab is 256
-  // rows of eight 16-byte chunks, chunk c of row r at position c ^ ((r >> 1) & 7): sixteen consecutive rows then
-  // put a given chunk in sixteen different bank groups (conflict-free fragment reads), and a row stays one
-  // contiguous 128 bytes (conflict-free staging writes).  It is stored two K steps before its first use, the unit
-  // of an operand that is staged as it lies (32 K rows of the tile's 256 columns) one step before.
-  constexpr int WIDE_STR = 64;
-  constexpr int A_STR = TA ? BM + 32 : WIDE_STR, B_STR = TB ? WIDE_STR : BN + 32;
-  constexpr int A_ROWS = TA ? BK : BM, B_ROWS = TB ? BN : BK;
-  constexpr int A_CPR = TA ? BM / 8 : 8, B_CPR = TB ? 8 : BN / 8;
-  // one array per buffer and operand: reads of one buffer and writes of the other can then be reordered freely
-  __shared__ __attribute__((aligned(16))) uint16_t As0[A_ROWS * A_STR];
-  __shared__ __attribute__((aligned(16))) uint16_t As1[A_ROWS * A_STR];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs0[B_ROWS * B_STR];
-  __shared__ __attribute__((aligned(16))) uint16_t Bs1[B_ROWS * B_STR];
-#define RA_W4_AS(BUF) ((BUF) ? As1 : As0)
+  // NJ: 32-column blocks of a wavefront's part of C; NBC: loads per wavefront for half a slab of B
+  constexpr int BM = 256, WM = 128, WN = BN / 2, NJ = WN / 32, NBC = BN / 64, SK = 64, WS = 64;
+  __shared__ __attribute__((aligned(16))) uint16_t As0[BM * SK];
+  __shared__ __attribute__((aligned(16))) uint16_t As1[BM * SK];
+  __shared__ __attribute__((aligned(16))) uint16_t As2[BM * SK];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs0[BN * SK];
+  __shared__ __attribute__((aligned(16))) uint16_t Bs1[BN * SK];
+#define RA_W4_AS(BUF) ((BUF) == 0 ? As0 : (BUF) == 1 ? As1 : As2)
 #define RA_W4_BS(BUF) ((BUF) ? Bs1 : Bs0)
-  // where the unit of K step U (known modulo 4) lives: buffer and offset of its row half
-#define RA_W4_ABUF(U) (TA ? ((U) & 1) : (((U) >> 1) & 1))
-#define RA_W4_BBUF(U) (TB ? (((U) >> 1) & 1) : ((U) & 1))
-#define RA_W4_AHALF(U) (TA ? 0 : ((U) & 1) * 128 * WIDE_STR)
-#define RA_W4_BHALF(U) (TB ? ((U) & 1) * (BN / 2) * WIDE_STR : 0)
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
   if (!tile_of_block(g.M / BM, g.N / BN, tm, tn)) return;
@@ -300,93 +290,79 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  // four sets of staging registers: unit j lives in set j % 4 from its request until it is stored to LDS four K
-  // steps later (about 2 us: an L2 miss served from HBM under load takes that long)
-  uint4 Pa0, Pa1, Pa2, Pa3, Pb0, Pb1, Pb2, Pb3, Qa0, Qa1, Qa2, Qa3, Qb0, Qb1, Qb2, Qb3;
-  uint4 Ra0, Ra1, Ra2, Ra3, Rb0, Rb1, Rb2, Rb3, Ta0, Ta1, Ta2, Ta3, Tb0, Tb1, Tb2, Tb3;
   const int lda = TA ? g.M : g.K, ldb = TB ? g.K : g.N;
-  const int nk = g.K / BK;
-  const int total = nk * (g.A2 ? 2 : 1);
-  // this thread's four chunks of a unit: global offsets (without the K position) and LDS offsets
-  // The global address of a chunk is a wave-uniform base (operand, tile origin, K position: scalar registers) plus a
-  // 32-bit byte offset per lane: that form of load sends half the address data of a 64-bit pointer per lane and
-  // measured 5-7 % more 16-byte loads per clock and CU.  (A tile spans at most 255 rows: the offset stays below 2^31.)
-  uint32_t ga[4], gb[4];
-  int la[4], lb[4];
+  const int nk = g.K / SK;                         // slabs per operand pair
+  const int nslab = nk * (g.A2 ? 2 : 1);
+  // Load c of a wavefront for half a slab.  Row-wise: rows (4 c + wave) 8 .. + 7 of the half's 128 (BN / 2) tile
+  // rows, lane l row l / 8, position l % 8.  K-major: the half's 32 K rows, RPI = 64 / (W / 8) rows an instruction,
+  // lane l row l / (W / 8), position l % (W / 8).  The lane offset (bytes) is the same for every c but for the rows.
+  constexpr int A_CPR = TA ? BM / 8 : 8, B_CPR = TB ? 8 : BN / 8;         // chunks per LDS row
+  constexpr int A_RPI = 64 / A_CPR, B_RPI = 64 / B_CPR;                   // rows per load instruction
+  const int ar = lane / A_CPR, br = lane / B_CPR;
+  const int a_sw = TA ? ((wave * A_RPI + ar) & 3) << 2 : (((wave * 8 + ar) >> 1) & 7);
+  const int b_sw = TB ? (((wave * 8 + br) >> 1) & 7) : ((wave * B_RPI + br) & 3) << 2;
+  const uint32_t ga0 = 2u * (uint32_t)((wave * A_RPI + ar) * lda + ((lane % A_CPR) ^ a_sw) * 8);
+  const uint32_t gb0 = 2u * (uint32_t)((wave * B_RPI + br) * ldb + ((lane % B_CPR) ^ b_sw) * 8);
+  const uint32_t ga_c = 2u * (uint32_t)(4 * A_RPI * lda), gb_c = 2u * (uint32_t)(4 * B_RPI * ldb);   // per c
+  // scalar offsets (bytes): of a slab along K, and of its second half
+  const uint32_t a_slab = TA ? 2u * (uint32_t)lda * SK : 2u * SK, a_half = TA ? 2u * (uint32_t)lda * 32 : 2u * (uint32_t)lda * 128;
+  const uint32_t b_slab = TB ? 2u * SK : 2u * (uint32_t)ldb * SK, b_half = TB ? 2u * (uint32_t)ldb * (BN / 2) : 2u * (uint32_t)ldb * 32;
   const int64_t tile_a = TA ? (int64_t)m0 : (int64_t)m0 * lda, tile_b = TB ? (int64_t)n0 * ldb : (int64_t)n0;
-#pragma unroll
-  for (int c = 0; c < 4; c++) {
-    const int i = c * NT + tid;
-    const int ra_ = i / A_CPR, ca_ = i % A_CPR, rb_ = i / B_CPR, cb_ = i % B_CPR;
-    ga[c] = 2u * (uint32_t)(ra_ * lda + ca_ * 8);
-    gb[c] = 2u * (uint32_t)(rb_ * ldb + cb_ * 8);
-    la[c] = ra_ * A_STR + (TA ? ca_ : ca_ ^ ((ra_ >> 1) & 7)) * 8;
-    lb[c] = rb_ * B_STR + (TB ? cb_ ^ ((rb_ >> 1) & 7) : cb_) * 8;
-  }
-  // buffer descriptors that start at the tile's origin; the unit's position goes into the scalar offset (bytes):
-  // K step u of an operand staged as it lies starts u * 32 rows down, unit u of a row-wise one 64 (u / 2) elements
-  // along the rows and 128 (u % 2) rows down
-  const uint32_t ka2 = 2u * (uint32_t)lda * (TA ? BK : 128), kb2 = 2u * (uint32_t)ldb * (TB ? BN / 2 : BK);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)(g.A + tile_a), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + tile_b), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_a2 = __builtin_amdgcn_make_buffer_rsrc((void*)((g.A2 ? g.A2 : g.A) + tile_a), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b2 = __builtin_amdgcn_make_buffer_rsrc((void*)((g.B2 ? g.B2 : g.B) + tile_b), 0, 0x7fffffff, 0x00020000);
-#define RA_W4_LOAD_A(S, T)                                                                              \
+  typedef __attribute__((address_space(3))) void* lds_ptr;
+  // half HF of slab J into buffer BUF (J past the end: the last slab again, into a buffer nobody reads any more)
+#define RA_W4_LOAD_A(BUF, J, HF)                                                                        \
   {                                                                                                     \
-    const int t_ = min((T), total - 1);                                                                 \
-    const __amdgpu_buffer_rsrc_t ra_ = t_ >= nk ? rsrc_a2 : rsrc_a;                                     \
-    const int u_ = t_ >= nk ? t_ - nk : t_;                                                             \
-    const uint32_t so_ = TA ? (uint32_t)u_ * ka2 : (uint32_t)(u_ >> 1) * 128u + (uint32_t)(u_ & 1) * ka2; \
-    S##a0 = ld_buf(ra_, ga[0], so_); S##a1 = ld_buf(ra_, ga[1], so_);                                   \
-    S##a2 = ld_buf(ra_, ga[2], so_); S##a3 = ld_buf(ra_, ga[3], so_);                                   \
+    const int j_ = min((J), nslab - 1);                                                                 \
+    const bool second_ = j_ >= nk;                                                                      \
+    const __amdgpu_buffer_rsrc_t r_ = second_ ? rsrc_a2 : rsrc_a;                                       \
+    const uint32_t so_ = (uint32_t)(second_ ? j_ - nk : j_) * a_slab + (HF) * a_half;                   \
+    _Pragma("unroll") for (int c = 0; c < 4; c++)                                                       \
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                         \
+          r_, (lds_ptr)&RA_W4_AS(BUF)[(HF) * (BM * SK / 2) + (4 * c + wave) * 512], 16, ga0 + c * ga_c, so_, 0, 0); \
   }
-#define RA_W4_LOAD_B(S, T)                                                                              \
+#define RA_W4_LOAD_B(BUF, J, HF)                                                                        \
   {                                                                                                     \
-    const int t_ = min((T), total - 1);                                                                 \
-    const __amdgpu_buffer_rsrc_t rb_ = t_ >= nk ? rsrc_b2 : rsrc_b;                                     \
-    const int u_ = t_ >= nk ? t_ - nk : t_;                                                             \
-    const uint32_t so_ = TB ? (uint32_t)(u_ >> 1) * 128u + (uint32_t)(u_ & 1) * kb2 : (uint32_t)u_ * kb2; \
-    S##b0 = ld_buf(rb_, gb[0], so_); S##b1 = ld_buf(rb_, gb[1], so_);                                   \
-    if (NBC == 4) { S##b2 = ld_buf(rb_, gb[2], so_); S##b3 = ld_buf(rb_, gb[3], so_); }                 \
+    const int j_ = min((J), nslab - 1);                                                                 \
+    const bool second_ = j_ >= nk;                                                                      \
+    const __amdgpu_buffer_rsrc_t r_ = second_ ? rsrc_b2 : rsrc_b;                                       \
+    const uint32_t so_ = (uint32_t)(second_ ? j_ - nk : j_) * b_slab + (HF) * b_half;                   \
+    _Pragma("unroll") for (int c = 0; c < NBC; c++)                                                     \
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                         \
+          r_, (lds_ptr)&RA_W4_BS(BUF)[(HF) * (BN * SK / 2) + (4 * c + wave) * 512], 16, gb0 + c * gb_c, so_, 0, 0); \
   }
-#define RA_W4_LOAD(S, T) { RA_W4_LOAD_A(S, T); RA_W4_LOAD_B(S, T); }
-  // set S holds the unit of K step U (modulo 4)
-#define RA_W4_STORE_A(S, U)                                                                             \
-  {                                                                                                     \
-    uint16_t* const d_ = &RA_W4_AS(RA_W4_ABUF(U))[RA_W4_AHALF(U)];                                      \
-    *(uint4*)(d_ + la[0]) = S##a0; *(uint4*)(d_ + la[1]) = S##a1;                                       \
-    *(uint4*)(d_ + la[2]) = S##a2; *(uint4*)(d_ + la[3]) = S##a3;                                       \
-  }
-#define RA_W4_STORE_B(S, U)                                                                             \
-  {                                                                                                     \
-    uint16_t* const d_ = &RA_W4_BS(RA_W4_BBUF(U))[RA_W4_BHALF(U)];                                      \
-    *(uint4*)(d_ + lb[0]) = S##b0; *(uint4*)(d_ + lb[1]) = S##b1;                                       \
-    if (NBC == 4) { *(uint4*)(d_ + lb[2]) = S##b2; *(uint4*)(d_ + lb[3]) = S##b3; }                     \
-  }
-  const int trA = (8 * hi + ((lane & 15) >> 2)) * A_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wm * WM;
-  const int trB = (8 * hi + ((lane & 15) >> 2)) * B_STR + 16 * ((lane >> 4) & 1) + 4 * (lane & 3) + wn * WN;
-  // row-wise fragment of K slice k' (0-3) of a slab: row lo, chunk (2 k' + hi) ^ ((lo >> 1) & 7)
-  const int nsw = (hi ^ ((lo >> 1) & 7)) * 8;
-  const int natA0 = (wm * WM + lo) * WIDE_STR + nsw, natB0 = (wn * WN + lo) * WIDE_STR + nsw;
-  const int natA1 = natA0 ^ 16, natA2 = natA0 ^ 32, natA3 = natA0 ^ 48;
-  const int natB1 = natB0 ^ 16, natB2 = natB0 ^ 32, natB3 = natB0 ^ 48;
-#define RA_W4_NAT(X, Q) ((Q) == 0 ? nat##X##0 : (Q) == 1 ? nat##X##1 : (Q) == 2 ? nat##X##2 : nat##X##3)
-  // the eight fragments of K slice KK (0 or 1) of K step U (modulo 4) into set F (F##a[0..3], F##b[0..3])
-#define RA_W4_FRAGS(F, U, KK)                                                                           \
+  // fragment addresses (elements).  Row-wise, K slice q: row lo, chunk (2 q + hi) ^ ((lo >> 1) & 7): q only flips
+  // bits 4 and 5.  K-major, block i: rows 16 q + 8 hi + r4 (and + 4), r4 = (lane & 15) >> 2, columns 32 i + 16 x + 4 y:
+  // block b = 32 i / 32 + (the wavefront's first block) of the row, chunk 4 b + 2 x + y / 2 at position
+  // ((b ^ r4) << 2) + 2 x + y / 2: one address per block.
+  const int r4 = (lane & 15) >> 2, cl = 2 * ((lane >> 4) & 1) + ((lane >> 1) & 1);
+  const int natA = (wm * WM + lo) * WS + (hi ^ ((lo >> 1) & 7)) * 8, natB = (wn * WN + lo) * WS + (hi ^ ((lo >> 1) & 7)) * 8;
+  const int trA_ = (8 * hi + r4) * BM + cl * 8 + 4 * (lane & 1), trB_ = (8 * hi + r4) * BN + cl * 8 + 4 * (lane & 1);
+  const int ba = wm * 4, bb = wn * NJ;             // first 32-column block of this wavefront in a row of the slab
+  const int trA0 = trA_ + (((ba + 0) ^ r4) << 5), trA1 = trA_ + (((ba + 1) ^ r4) << 5);
+  const int trA2 = trA_ + (((ba + 2) ^ r4) << 5), trA3 = trA_ + (((ba + 3) ^ r4) << 5);
+  const int trB0 = trB_ + (((bb + 0) ^ r4) << 5), trB1 = trB_ + (((bb + 1) ^ r4) << 5);
+  const int trB2 = trB_ + (((bb + 2) ^ r4) << 5), trB3 = trB_ + (((bb + 3) ^ r4) << 5);
+#define RA_W4_SEL(X, I) ((I) == 0 ? X##0 : (I) == 1 ? X##1 : (I) == 2 ? X##2 : X##3)
+  // the fragments of K slice Q (0-3) of the slabs in buffers ABUF, BBUF into set F (F##a[0..3], F##b[0..NJ-1])
+#define RA_W4_FRAGS(F, ABUF, BBUF, Q)                                                                   \
   _Pragma("unroll") for (int i = 0; i < 4; i++) {                                                       \
     if (!TA) {                                                                                          \
-      F##a[i] = *(const bf16x8*)(&RA_W4_AS(RA_W4_ABUF(U))[RA_W4_NAT(A, 2 * ((U) & 1) + (KK)) + i * 32 * WIDE_STR]); \
+      F##a[i] = *(const bf16x8*)(&RA_W4_AS(ABUF)[(natA ^ ((Q) << 4)) + i * 32 * WS]);                   \
     } else {                                                                                            \
-      const uint16_t* p = &RA_W4_AS(RA_W4_ABUF(U))[(KK) * 16 * A_STR + trA + i * 32];                   \
-      s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * A_STR);                                                 \
+      const uint16_t* p = &RA_W4_AS(ABUF)[RA_W4_SEL(trA, i) + (Q) * 16 * BM];                           \
+      s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * BM);                                                    \
       F##a[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
     if (i >= NJ) continue;                                                                              \
     if (TB) {                                                                                           \
-      F##b[i] = *(const bf16x8*)(&RA_W4_BS(RA_W4_BBUF(U))[RA_W4_NAT(B, 2 * ((U) & 1) + (KK)) + i * 32 * WIDE_STR]); \
+      F##b[i] = *(const bf16x8*)(&RA_W4_BS(BBUF)[(natB ^ ((Q) << 4)) + i * 32 * WS]);                   \
     } else {                                                                                            \
-      const uint16_t* p = &RA_W4_BS(RA_W4_BBUF(U))[(KK) * 16 * B_STR + trB + i * 32];                   \
-      s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * B_STR);                                                 \
+      const uint16_t* p = &RA_W4_BS(BBUF)[RA_W4_SEL(trB, i) + (Q) * 16 * BN];                           \
+      s16x4 x0 = lds_tr(p), x1 = lds_tr(p + 4 * BN);                                                    \
       F##b[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));    \
     }                                                                                                   \
   }
@@ -395,79 +371,76 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
     _Pragma("unroll") for (int j = 0; j < NJ; j++)                                                      \
       acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F##a[i], F##b[j], acc[i][j], 0, 0, 0);
   // A single wavefront per SIMD issues in order: the MFMA pipe only stays busy if every MFMA is followed by at most
-  // a few other instructions.  One group per MFMA: the MFMA, its share of the LDS reads, and one LDS write or,
-  // once the writes are out, its share of the global loads.
+  // a few other instructions.  One group per MFMA of a quarter: the MFMA, its share of the quarter's LDS reads, and
+  // every (NM / LOADS)-th a load.
   constexpr int NM = 4 * NJ, RD = (TA ? 8 : 4) + (TB ? NJ : 2 * NJ), RPG = (RD + NM - 1) / NM;
-#define RA_W4_SCHED(WRITES, LOADS)                                                                      \
+#define RA_W4_SCHED(LOADS)                                                                              \
   _Pragma("unroll") for (int m_ = 0; m_ < NM; m_++) {                                                   \
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                                  \
-    __builtin_amdgcn_sched_group_barrier(0x100, RPG, 0);                                                \
-    if (m_ < (WRITES)) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                               \
-    else if ((m_ - (WRITES)) * (((LOADS) + NM - (WRITES) - 1) / (NM - (WRITES))) < (LOADS))             \
-      __builtin_amdgcn_sched_group_barrier(0x020, ((LOADS) + NM - (WRITES) - 1) / (NM - (WRITES)), 0);  \
+    if (m_ * RPG < RD) __builtin_amdgcn_sched_group_barrier(0x100, RPG, 0);                             \
+    if (m_ % (NM / (LOADS)) == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                    \
   }
-  // K step U (modulo 4; its slice 0 already in set F), T0 its index.  S1 is the register set of step U + 1, S2 that
-  // of step U + 2: a row-wise operand's unit goes to LDS from S2, the other kind's from S1, and the set is then
-  // requested again for four K steps later.
-#define RA_W4_STEP(U, S1, S2, T0)                                                                       \
+  // slab J: A in buffer AC (of three), B in buffer BC (of two); its slice 0 already in set F
+#define RA_W4_STEP(AC, BC, J)                                                                           \
   {                                                                                                     \
-    RA_W4_FRAGS(G, U, 1);                                                                               \
-    if (TA) { RA_W4_STORE_A(S1, ((U) + 1) & 3); } else { RA_W4_STORE_A(S2, ((U) + 2) & 3); }            \
-    if (TB) { RA_W4_STORE_B(S2, ((U) + 2) & 3); } else { RA_W4_STORE_B(S1, ((U) + 1) & 3); }            \
-    if (TA) { RA_W4_LOAD_A(S1, (T0) + 5); } else { RA_W4_LOAD_A(S2, (T0) + 6); }                        \
+    RA_W4_FRAGS(G, AC, BC, 1);                                                                          \
+    RA_W4_LOAD_B((BC) ^ 1, (J) + 1, 1);                                                                 \
     RA_W4_MFMA(F);                                                                                      \
-    RA_W4_SCHED(4 + NBC, 4);                                                                                \
+    RA_W4_SCHED(NBC);                                                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
-    __syncthreads();                                                                                    \
-    RA_W4_FRAGS(F, ((U) + 1) & 3, 0);                                                                   \
-    if (TB) { RA_W4_LOAD_B(S2, (T0) + 6); } else { RA_W4_LOAD_B(S1, (T0) + 5); }                        \
+    RA_W4_FRAGS(F, AC, BC, 2);                                                                          \
+    RA_W4_LOAD_A(((AC) + 2) % 3, (J) + 2, 0);                                                           \
     RA_W4_MFMA(G);                                                                                      \
-    RA_W4_SCHED(0, NBC);                                                                                \
+    RA_W4_SCHED(4);                                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    RA_W4_FRAGS(G, AC, BC, 3);                                                                          \
+    RA_W4_LOAD_A(((AC) + 2) % 3, (J) + 2, 1);                                                           \
+    RA_W4_MFMA(F);                                                                                      \
+    RA_W4_SCHED(4);                                                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                                  \
+    /* everything but the slab after next of A (the eight newest loads) has landed, in every wavefront */ \
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");                            \
+    RA_W4_FRAGS(F, ((AC) + 1) % 3, (BC) ^ 1, 0);                                                        \
+    RA_W4_LOAD_B(BC, (J) + 2, 0);                                                                       \
+    RA_W4_MFMA(G);                                                                                      \
+    RA_W4_SCHED(NBC);                                                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                  \
   }
   bf16x8 Fa[4], Fb[NJ], Ga[4], Gb[NJ];
-  RA_W4_LOAD(P, 0);
-  RA_W4_LOAD(Q, 1);
-  RA_W4_LOAD(R, 2);
-  RA_W4_LOAD(T, 3);
-  RA_W4_STORE_A(P, 0);
-  RA_W4_STORE_B(P, 0);
-  RA_W4_LOAD(P, 4);
-  if (!TA) { RA_W4_STORE_A(Q, 1); RA_W4_LOAD_A(Q, 5); }
-  if (TB) { RA_W4_STORE_B(Q, 1); RA_W4_LOAD_B(Q, 5); }
-  __syncthreads();
-  RA_W4_FRAGS(F, 0, 0);
-  // K is a multiple of 64: an even number of K steps; four steps per trip, two more when that leaves a remainder
-  int it = 0;
-  for (; it + 4 <= total; it += 4) {
-    RA_W4_STEP(0, Q, R, it);
-    RA_W4_STEP(1, R, T, it + 1);
-    RA_W4_STEP(2, T, P, it + 2);
-    RA_W4_STEP(3, P, Q, it + 3);
+  RA_W4_LOAD_A(0, 0, 0); RA_W4_LOAD_A(0, 0, 1);
+  RA_W4_LOAD_B(0, 0, 0); RA_W4_LOAD_B(0, 0, 1);
+  RA_W4_LOAD_A(1, 1, 0); RA_W4_LOAD_A(1, 1, 1);
+  RA_W4_LOAD_B(1, 1, 0);
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  RA_W4_FRAGS(F, 0, 0, 0);
+  // the buffers come round every six slabs
+  int j = 0;
+  for (; j + 6 <= nslab; j += 6) {
+    RA_W4_STEP(0, 0, j);
+    RA_W4_STEP(1, 1, j + 1);
+    RA_W4_STEP(2, 0, j + 2);
+    RA_W4_STEP(0, 1, j + 3);
+    RA_W4_STEP(1, 0, j + 4);
+    RA_W4_STEP(2, 1, j + 5);
   }
-  if (it < total) {
-    RA_W4_STEP(0, Q, R, it);
-    RA_W4_STEP(1, R, T, it + 1);
-  }
+  if (j < nslab) RA_W4_STEP(0, 0, j);
+  if (j + 1 < nslab) RA_W4_STEP(1, 1, j + 1);
+  if (j + 2 < nslab) RA_W4_STEP(2, 0, j + 2);
+  if (j + 3 < nslab) RA_W4_STEP(0, 1, j + 3);
+  if (j + 4 < nslab) RA_W4_STEP(1, 0, j + 4);
 #undef RA_W4_STEP
 #undef RA_W4_AS
 #undef RA_W4_BS
-#undef RA_W4_ABUF
-#undef RA_W4_BBUF
-#undef RA_W4_AHALF
-#undef RA_W4_BHALF
-#undef RA_W4_NAT
+#undef RA_W4_SEL
 #undef RA_W4_MFMA
 #undef RA_W4_FRAGS
-#undef RA_W4_STORE_A
-#undef RA_W4_STORE_B
-#undef RA_W4_LOAD
 #undef RA_W4_LOAD_A
 #undef RA_W4_LOAD_B
 #undef RA_W4_SCHED
 
-  // epilogue through two LDS patches per wavefront, one operand array each (the operand tiles are dead by now)
-  __syncthreads();
+  // epilogue through two LDS patches per wavefront (the operand slabs are dead by now, and no load may land in
+  // them any more)
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
   static_assert(sizeof(As0) >= (size_t)2 * 32 * 36 * sizeof(float) && sizeof(Bs0) >= (size_t)2 * 32 * 36 * sizeof(float),
                 "operand tile too small for two epilogue patches");
   float* patch = (float*)(wave == 0 ? &As0[0] : wave == 1 ? &As1[0] : wave == 2 ? &Bs0[0] : &Bs1[0]);
@@ -493,7 +466,7 @@ static int launch_tile(const GemmArgs& g, hipStream_t s) {
 
 // Tile choice.  One workgroup of the large tiles fills a CU, so the grid runs in rounds of (number of CUs)
 // workgroups: take the tile whose rounds, weighted by what a round of it costs (measured on full grids: a round of
-// 256 x 256 tiles takes 1.62 times one of 256 x 128 over four wavefronts, which does half the work), take least.
+// 256 x 256 tiles takes 1.72 times one of 256 x 128 over four wavefronts, which does half the work), take least.
 static bool w4_reach_ok(int M, int N, int K) {
   // the 4-wavefront kernels address an operand through a buffer descriptor at its tile's origin with 32-bit byte
   // offsets: what a tile can reach (a whole operand in the worst case) must stay below 2^31 bytes
@@ -512,7 +485,7 @@ static int pick_tile(int M, int N, int K) {
   double cost = rounds(128, 128) * 0.70;
   if (M % 256 == 0 && rounds(256, 128) * 1.16 < cost) { best = 1; cost = rounds(256, 128) * 1.16; }
   if (w4 && rounds(256, 128) * 1.00 < cost) { best = 3; cost = rounds(256, 128) * 1.00; }
-  if (w4 && N % 256 == 0 && rounds(256, 256) * 1.62 <= cost) { best = 0; cost = rounds(256, 256) * 1.62; }
+  if (w4 && N % 256 == 0 && rounds(256, 256) * 1.72 <= cost) { best = 0; cost = rounds(256, 256) * 1.72; }
   return best;
 }
 
