@@ -37,11 +37,13 @@ def test_gemm_layouts(ta, tb, shape):
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
 @pytest.mark.parametrize("tile", [0, 1, 2, 3])
-@pytest.mark.parametrize("shape", [(768, 512, 320), (1280, 256, 128), (512, 384, 448)])
+@pytest.mark.parametrize("shape", [(768, 512, 320), (1280, 256, 128), (512, 384, 448), (256, 256, 64), (256, 512, 192),
+                                   (512, 256, 256), (256, 256, 576)])
 def test_gemm_every_tile_kernel(ta, tb, tile, shape):
     """Each tile kernel (0: 256 x 256 over four wavefronts, 1: 256 x 128 over eight, 2: 128 x 128, 3: 256 x 128 over four) on shapes whose tile
     counts are no multiple of the 8 XCDs or of the tile-row group, so the workgroup -> tile order and its
-    surplus workgroups are exercised; ra_gemm_bf16_tile names the tile kernel that ra_gemm_bf16 would pick itself."""
+    surplus workgroups are exercised, and on K of 1 to 9 slabs of 64 (the 4-wavefront kernels rotate their LDS buffers
+    every six slabs and finish with up to five single steps); ra_gemm_bf16_tile names the tile kernel that ra_gemm_bf16 would pick itself."""
     M, N, K = shape
     print("gemm tile", tile, ta, tb, shape, flush=True)
     g = torch.Generator().manual_seed(M + N + K + tile)
