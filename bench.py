@@ -845,6 +845,17 @@ def main():
             d = bench_decode(args, steps=64)
             extras["decode"] = {k_: d[k_] for k_ in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
                                                      "pct_hbm_peak", "config", "roofline", "cpu_baseline")}
+            # the other two configurations: the virtual ring of eight over 131072 positions with packed documents and a
+            # bias, and the SwiGLU feed-forward over 65536 tokens (one chunk per launch, and 16384 tokens per launch)
+            torch.cuda.empty_cache()
+            rg = bench_attention(argparse.Namespace(**dict(vars(args), no_cpu=True, no_extras=True, steps=3, warmup=1)),
+                                 ring=True)
+            extras["ring131k"] = {k_: rg[k_] for k_ in ("metric", "value", "unit", "ms_per_step", "dtype", "config")}
+            torch.cuda.empty_cache()
+            ff = bench_ffn(argparse.Namespace(**dict(vars(args), no_cpu=True, steps=3, warmup=1)))
+            extras["ffn"] = {k_: ff[k_] for k_ in ("metric", "value", "unit", "ms_per_step", "dtype", "config",
+                                                   "launch_tokens_16384")}
+            extras["ffn"]["gemm"] = {k_: ff["roofline"][k_] for k_ in ("kernel", "achieved", "unit", "frac")}
     elif args.workload == "decode":
         r = bench_decode(args)
     elif args.workload == "copy":
