@@ -304,22 +304,26 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   const uint32_t ga0 = 2u * (uint32_t)((wave * A_RPI + ar) * lda + ((lane % A_CPR) ^ a_sw) * 8);
   const uint32_t gb0 = 2u * (uint32_t)((wave * B_RPI + br) * ldb + ((lane % B_CPR) ^ b_sw) * 8);
   const uint32_t ga_c = 2u * (uint32_t)(4 * A_RPI * lda), gb_c = 2u * (uint32_t)(4 * B_RPI * ldb);   // per c
-  // scalar offsets (bytes): of a slab along K, and of its second half
-  const uint32_t a_slab = TA ? 2u * (uint32_t)lda * SK : 2u * SK, a_half = TA ? 2u * (uint32_t)lda * 32 : 2u * (uint32_t)lda * 128;
-  const uint32_t b_slab = TB ? 2u * SK : 2u * (uint32_t)ldb * SK, b_half = TB ? 2u * (uint32_t)ldb * (BN / 2) : 2u * (uint32_t)ldb * 32;
+  // A slab is read through a buffer descriptor at its own origin in the tile (64-bit scalar arithmetic), so the 32-bit
+  // lane and scalar offsets only span one slab - at most 256 rows of a row-wise operand, 64 of a K-major one - and
+  // an operand may be of any size.  Elements from one slab to the next, and bytes to a slab's second half:
+  const int64_t a_slab = TA ? (int64_t)lda * SK : SK, b_slab = TB ? SK : (int64_t)ldb * SK;
+  const uint32_t a_half = TA ? 2u * (uint32_t)lda * 32 : 2u * (uint32_t)lda * 128;
+  const uint32_t b_half = TB ? 2u * (uint32_t)ldb * (BN / 2) : 2u * (uint32_t)ldb * 32;
   const int64_t tile_a = TA ? (int64_t)m0 : (int64_t)m0 * lda, tile_b = TB ? (int64_t)n0 * ldb : (int64_t)n0;
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)(g.A + tile_a), 0, 0x7fffffff, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void*)(g.B + tile_b), 0, 0x7fffffff, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_a2 = __builtin_amdgcn_make_buffer_rsrc((void*)((g.A2 ? g.A2 : g.A) + tile_a), 0, 0x7fffffff, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b2 = __builtin_amdgcn_make_buffer_rsrc((void*)((g.B2 ? g.B2 : g.B) + tile_b), 0, 0x7fffffff, 0x00020000);
+  const uint16_t* const a_tile = g.A + tile_a;
+  const uint16_t* const b_tile = g.B + tile_b;
+  const uint16_t* const a2_tile = (g.A2 ? g.A2 : g.A) + tile_a;
+  const uint16_t* const b2_tile = (g.B2 ? g.B2 : g.B) + tile_b;
   typedef __attribute__((address_space(3))) void* lds_ptr;
   // half HF of slab J into buffer BUF (J past the end: the last slab again, into a buffer nobody reads any more)
 #define RA_W4_LOAD_A(BUF, J, HF)                                                                        \
   {                                                                                                     \
     const int j_ = min((J), nslab - 1);                                                                 \
     const bool second_ = j_ >= nk;                                                                      \
-    const __amdgpu_buffer_rsrc_t r_ = second_ ? rsrc_a2 : rsrc_a;                                       \
-    const uint32_t so_ = (uint32_t)(second_ ? j_ - nk : j_) * a_slab + (HF) * a_half;                   \
+    const __amdgpu_buffer_rsrc_t r_ = __builtin_amdgcn_make_buffer_rsrc(                               \
+        (void*)((second_ ? a2_tile : a_tile) + (second_ ? j_ - nk : j_) * a_slab), 0, 0x7fffffff, 0x00020000); \
+    const uint32_t so_ = (HF) * a_half;                                                                 \
     _Pragma("unroll") for (int c = 0; c < 4; c++)                                                       \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                         \
           r_, (lds_ptr)&RA_W4_AS(BUF)[(HF) * (BM * SK / 2) + (4 * c + wave) * 512], 16, ga0 + c * ga_c, so_, 0, 0); \
@@ -328,8 +332,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   {                                                                                                     \
     const int j_ = min((J), nslab - 1);                                                                 \
     const bool second_ = j_ >= nk;                                                                      \
-    const __amdgpu_buffer_rsrc_t r_ = second_ ? rsrc_b2 : rsrc_b;                                       \
-    const uint32_t so_ = (uint32_t)(second_ ? j_ - nk : j_) * b_slab + (HF) * b_half;                   \
+    const __amdgpu_buffer_rsrc_t r_ = __builtin_amdgcn_make_buffer_rsrc(                               \
+        (void*)((second_ ? b2_tile : b_tile) + (second_ ? j_ - nk : j_) * b_slab), 0, 0x7fffffff, 0x00020000); \
+    const uint32_t so_ = (HF) * b_half;                                                                 \
     _Pragma("unroll") for (int c = 0; c < NBC; c++)                                                     \
       __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                         \
           r_, (lds_ptr)&RA_W4_BS(BUF)[(HF) * (BN * SK / 2) + (4 * c + wave) * 512], 16, gb0 + c * gb_c, so_, 0, 0); \
@@ -468,9 +473,9 @@ static int launch_tile(const GemmArgs& g, hipStream_t s) {
 // workgroups: take the tile whose rounds, weighted by what a round of it costs (measured on full grids: a round of
 // 256 x 256 tiles takes 1.72 times one of 256 x 128 over four wavefronts, which does half the work), take least.
 static bool w4_reach_ok(int M, int N, int K) {
-  // the 4-wavefront kernels address an operand through a buffer descriptor at its tile's origin with 32-bit byte
-  // offsets: what a tile can reach (a whole operand in the worst case) must stay below 2^31 bytes
-  return M % 256 == 0 && (int64_t)M * K < (1LL << 30) && (int64_t)N * K < (1LL << 30);
+  // the 4-wavefront kernels address a slab through a buffer descriptor at its origin with 32-bit byte offsets: 256
+  // rows of a row-wise operand (512 K bytes) or 64 rows of a K-major one (128 M or 128 N bytes) must stay below 2^31
+  return M % 256 == 0 && K < (1 << 21) && M < (1 << 23) && N < (1 << 23);
 }
 static int pick_tile(int M, int N, int K) {
   static const int ncu = [] {     // initialised once, thread-safe

@@ -57,6 +57,30 @@ def test_gemm_every_tile_kernel(ta, tb, tile, shape):
     assert errors(acc, ref + 1.0)[1] < 1e-5
 
 
+def test_gemm_operand_beyond_two_gib():
+    """A K-major operand of 2.3 GB (a weight gradient over 98304 tokens): the 4-wavefront kernels read every slab
+    through a descriptor of its own, so the size of an operand does not matter; checked against fp32 sums of
+    torch's products of 8192-row slices."""
+    K, M, N = 98304, 11776, 256
+    g = torch.Generator(device=DEV).manual_seed(5)
+    A = torch.randn(K, M, device=DEV, generator=g).to(torch.bfloat16)          # stored (K, M): trans_a
+    B = torch.randn(K, N, device=DEV, generator=g).to(torch.bfloat16)
+    assert A.numel() * 2 > 2 ** 31
+    ref = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+    for k0 in range(0, K, 8192):
+        ref += A[k0:k0 + 8192].float().t() @ B[k0:k0 + 8192].float()
+    for tile in (0, 3):
+        out = torch.zeros(M, N, dtype=torch.float32, device=DEV)
+        ra.gemm_bf16(A, B, trans_a=True, out=out, accumulate=True, tile=tile)
+        assert errors(out, ref)[1] < 1e-5, (tile, errors(out, ref))
+    # the other side: a row-wise B of 2.3 GB
+    Bt = A                                                                      # as (N' = K, K' = M): stored (N, K)
+    A2 = torch.randn(256, M, device=DEV, generator=g).to(torch.bfloat16)
+    ref2 = A2.float() @ Bt[:16384].float().t()
+    out2 = ra.gemm_bf16(A2, Bt, trans_b=True, tile=0)
+    rel_ok(out2[:, :16384], ref2, "row-wise B beyond 2 GiB")
+
+
 def test_gemm_rejects_ragged_shapes():
     A = torch.zeros(100, 64, dtype=torch.bfloat16, device=DEV)
     B = torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV)
