@@ -57,6 +57,29 @@ def test_gemm_every_tile_kernel(ta, tb, tile, shape):
     assert errors(acc, ref + 1.0)[1] < 1e-5
 
 
+def test_gemm_random_shapes():
+    """Sixty seeded random shapes (M, N multiples of 128 up to 1536, K of 1 to 40 slabs of 64), layouts, tile kernels
+    and output modes against torch's fp32 product."""
+    import random
+    rnd = random.Random(7)
+    for case in range(60):
+        M, N, K = 128 * rnd.randint(1, 12), 128 * rnd.randint(1, 12), 64 * rnd.randint(1, 40)
+        ta, tb = rnd.random() < 0.5, rnd.random() < 0.5
+        tile = rnd.choice([None, 0, 1, 2, 3])
+        acc = rnd.random() < 0.4
+        g = torch.Generator().manual_seed(case)
+        A = torch.randn((K, M) if ta else (M, K), generator=g).bfloat16().to(DEV)
+        B = torch.randn((N, K) if tb else (K, N), generator=g).bfloat16().to(DEV)
+        ref = (A.float().t() if ta else A.float()) @ (B.float().t() if tb else B.float())
+        what = "case %d: %d x %d x %d ta %s tb %s tile %s acc %s" % (case, M, N, K, ta, tb, tile, acc)
+        if acc:
+            out = torch.full((M, N), 0.5, dtype=torch.float32, device=DEV)
+            ra.gemm_bf16(A, B, trans_a=ta, trans_b=tb, out=out, accumulate=True, tile=tile)
+            assert errors(out - 0.5, ref)[1] < 1e-5, what
+        else:
+            rel_ok(ra.gemm_bf16(A, B, trans_a=ta, trans_b=tb, tile=tile), ref, what)
+
+
 def test_gemm_operand_beyond_two_gib():
     """A K-major operand of 2.3 GB (a weight gradient over 98304 tokens): the 4-wavefront kernels read every slab
     through a descriptor of its own, so the size of an operand does not matter; checked against fp32 sums of
