@@ -60,11 +60,32 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[MB][NB], float* patch0,
                                            int row0, int col0, int lane) {
   const int lo = lane & 31, hi = lane >> 5;
   const int er = lane >> 3, ec = (lane & 7) * 4;          // this lane's row (of 8 per pass) and first column
+  // MODE 2 adds into C: the old values of a block are requested PF blocks ahead, before the stores of the block in
+  // hand.  (Requested inside the block that uses them, every block waited a memory latency and, the counter of
+  // outstanding memory operations being in order, for the stores of the block before: sixteen such waits were a third
+  // of a workgroup's time at K = 2048.)
+  constexpr int PF = 2, NBLK = MB * NB;
+  float4 old[PF][4] = {};
+#define RA_ST_REQUEST(BI)                                                                               \
+  _Pragma("unroll") for (int pass = 0; pass < 4; pass++)                                                \
+    old[(BI) % PF][pass] = *(const float4*)((const float*)C + (int64_t)(row0 + ((BI) / NB) * 32 + pass * 8 + er) * ldc + \
+                                            col0 + ((BI) % NB) * 32 + ec);
+  if (MODE == 2) {
+#pragma unroll
+    for (int bi = 0; bi < PF && bi < NBLK; bi++) RA_ST_REQUEST(bi)
+  }
 #pragma unroll
   for (int i = 0; i < MB; i++)
 #pragma unroll
     for (int j = 0; j < NB; j++) {
-      float* patch = ((i * NB + j) & 1) ? patch1 : patch0;
+      const int bi = i * NB + j;
+      float* patch = (bi & 1) ? patch1 : patch0;
+      float4 cur[4] = {};
+      if (MODE == 2) {
+#pragma unroll
+        for (int pass = 0; pass < 4; pass++) cur[pass] = old[bi % PF][pass];
+        if (bi + PF < NBLK) RA_ST_REQUEST(bi + PF)
+      }
 #pragma unroll
       for (int r = 0; r < 16; r++) patch[((r >> 2) * 8 + hi * 4 + (r & 3)) * 36 + lo] = acc[i][j][r];
 #pragma unroll
@@ -80,11 +101,12 @@ __device__ __forceinline__ void store_tile(f32x16 (&acc)[MB][NB], float* patch0,
         } else {
           float4* c = (float4*)((float*)C + o);
           float4 w = v;
-          if (MODE == 2) { const float4 old = *c; w.x += old.x; w.y += old.y; w.z += old.z; w.w += old.w; }
+          if (MODE == 2) { w.x += cur[pass].x; w.y += cur[pass].y; w.z += cur[pass].z; w.w += cur[pass].w; }
           *c = w;
         }
       }
     }
+#undef RA_ST_REQUEST
 }
 
 // TA: A is stored (K,M).  TB: B is stored (N,K).
