@@ -669,23 +669,31 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     const float rscale = 1.f / sqrtf((float)HD);
     const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
     const int64_t oout = (int64_t)b * a.dkvo_sb + (int64_t)krow * a.dkvo_ss + (int64_t)h * HD + hi * 4;
+    // dk, then dv; all the old values of one are requested before its first store (a load issued after a store is
+    // not waited for until that store has completed too: one in-order counter)
 #pragma unroll
-    for (int db = 0; db < NDB; db++)
+    for (int which = 0; which < 2; which++) {
+      float* const pacc = (which == 0 ? a.dk : a.dv) + ooff;
+      uint16_t* const pout = (which == 0 ? a.dk_out : a.dv_out) + oout;
+      f32x4 old[NDB][4];
 #pragma unroll
-      for (int g = 0; g < 4; g++) {
-        float* pk = a.dk + ooff + db * 32 + g * 8;
-        float* pv = a.dv + ooff + db * 32 + g * 8;
-        f32x4 tk = {0.f, 0.f, 0.f, 0.f}, tv = {0.f, 0.f, 0.f, 0.f};
-        if (!a.dkv_initial) { tk = *(const f32x4*)pk; tv = *(const f32x4*)pv; }
+      for (int db = 0; db < NDB; db++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) { tk[e] += dkacc[db][g * 4 + e] * rscale; tv[e] += dvacc[db][g * 4 + e]; }
-        if (a.dk_out) {                  // last call for these keys: the sum as bf16 (:89)
-          store_bf16x4(a.dk_out + oout + db * 32 + g * 8, tk);
-          store_bf16x4(a.dv_out + oout + db * 32 + g * 8, tv);
-        } else {
-          *(f32x4*)pk = tk; *(f32x4*)pv = tv;
+        for (int g = 0; g < 4; g++) {
+          old[db][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+          if (!a.dkv_initial) old[db][g] = *(const f32x4*)(pacc + db * 32 + g * 8);
         }
-      }
+#pragma unroll
+      for (int db = 0; db < NDB; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          f32x4 t = old[db][g];
+#pragma unroll
+          for (int e = 0; e < 4; e++) t[e] += which == 0 ? dkacc[db][g * 4 + e] * rscale : dvacc[db][g * 4 + e];
+          if (a.dk_out) store_bf16x4(pout + db * 32 + g * 8, t);     // last call for these keys: the sum as bf16 (:89)
+          else *(f32x4*)(pacc + db * 32 + g * 8) = t;
+        }
+    }
   }
 #undef RA_WS_LOAD
 #undef RA_WS_STORE
@@ -1134,12 +1142,21 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     const float rscale = 1.f / sqrtf((float)HD);
     float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
     uint16_t* dqo = a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)qrow * a.dqo_ss + (int64_t)h * HD + hi * 4;
+    // all the old values are requested before the first store: a load issued after a store is not waited for until
+    // that store has completed too (one in-order counter), and sixteen such round trips in a row cost tens of us
+    f32x4 old[NDB][4];
 #pragma unroll
     for (int db = 0; db < NDB; db++)
 #pragma unroll
       for (int g = 0; g < 4; g++) {
-        f32x4 t = {0.f, 0.f, 0.f, 0.f};
-        if (!a.dq_initial) t = *(const f32x4*)(dqp + db * 32 + g * 8);
+        old[db][g] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (!a.dq_initial) old[db][g] = *(const f32x4*)(dqp + db * 32 + g * 8);
+      }
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        f32x4 t = old[db][g];
 #pragma unroll
         for (int e = 0; e < 4; e++) t[e] += acc[db][g * 4 + e] * rscale;
         if (a.dq_out) store_bf16x4(dqo + db * 32 + g * 8, t);      // last call for these rows: the sum as bf16 (:89)
