@@ -477,12 +477,19 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
   // dq += acc / sqrt(D) (:230)
   float* dqp = a.dq ? a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD : nullptr;
   float* dqo = a.dq_out ? a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)qrow * a.dqo_ss + (int64_t)h * HD : nullptr;
+  // all the old values are requested before the first store (a load issued after a store is not waited for until
+  // that store has completed too: one in-order counter of outstanding memory operations)
+  float old[16][NDB];
+#pragma unroll
+  for (int r = 0; r < 16; r++)
+#pragma unroll
+    for (int db = 0; db < NDB; db++) old[r][db] = a.dq_initial ? 0.f : dqp[NDB * crow(r, hi) + db];
 #pragma unroll
   for (int r = 0; r < 16; r++)
 #pragma unroll
     for (int db = 0; db < NDB; db++) {
       const int d = NDB * crow(r, hi) + db;
-      const float t_ = (a.dq_initial ? 0.f : dqp[d]) + acc[db][r] * rscale;
+      const float t_ = old[r][db] + acc[db][r] * rscale;
       if (dqo) dqo[d] = t_;                // last call for these rows (:89)
       else dqp[d] = t_;
     }
@@ -675,13 +682,23 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   // dk += acc / sqrt(D) (:231), dv += acc (:232)
   const int64_t o = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD;
   const int64_t oo = (int64_t)b * a.dkvo_sb + (int64_t)krow * a.dkvo_ss + (int64_t)h * HD;
+  // all the old values are requested before the first store (see the dQ kernel)
+  float oldk[16][NDB], oldv[16][NDB];
 #pragma unroll
   for (int r = 0; r < 16; r++)
 #pragma unroll
     for (int db = 0; db < NDB; db++) {
       const int d = NDB * crow(r, hi) + db;
-      const float tk = (a.dkv_initial ? 0.f : a.dk[o + d]) + dkacc[db][r] * rscale;
-      const float tv = (a.dkv_initial ? 0.f : a.dv[o + d]) + dvacc[db][r];
+      oldk[r][db] = a.dkv_initial ? 0.f : a.dk[o + d];
+      oldv[r][db] = a.dkv_initial ? 0.f : a.dv[o + d];
+    }
+#pragma unroll
+  for (int r = 0; r < 16; r++)
+#pragma unroll
+    for (int db = 0; db < NDB; db++) {
+      const int d = NDB * crow(r, hi) + db;
+      const float tk = oldk[r][db] + dkacc[db][r] * rscale;
+      const float tv = oldv[r][db] + dvacc[db][r];
       if (a.dk_out) { a.dk_out[oo + d] = tk; a.dv_out[oo + d] = tv; }      // last call for these keys (:89)
       else { a.dk[o + d] = tk; a.dv[o + d] = tv; }
     }
