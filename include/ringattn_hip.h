@@ -25,6 +25,10 @@ extern "C" {
 
 typedef struct ihipStream_t* ra_stream_t; /* == hipStream_t */
 
+/* Version of this interface: bumped whenever a struct below grows or a signature changes.  ra_version() returns the
+ * value the library was built with; a binding compares the two before its first call (the ctypes binding does). */
+#define RA_ABI_VERSION 2
+
 enum { RA_OK = 0, RA_ERR_INVALID = 1, RA_ERR_UNSUPPORTED = 2, RA_ERR_LAUNCH = 3 };
 enum { RA_F32 = 0, RA_BF16 = 1 };
 
@@ -57,6 +61,13 @@ typedef struct ra_mask {
   int32_t q_chunk_idx_start;  /* :33 ; ignored when cache_idx is given */
   int32_t k_chunk_idx_start;  /* :37 */
   const int32_t* cache_idx;   /* nullable device scalar: q_chunk_idx_start = *cache_idx / query_chunk_size (:35) */
+  const int32_t* chunk_starts; /* nullable device pair {q_chunk_idx_start, k_chunk_idx_start}: read by the kernels in
+                                 place of the two host ints above.  Under jit both come from lax.axis_index
+                                 (:31-37, :69-75), a traced value that a custom call receives as a buffer and cannot
+                                 read without a sync; the kernels derive which tiles run from it themselves, so a
+                                 call whose every tile is skipped still launches (and passes its rows on).  cache_idx,
+                                 when given too, still decides the query start.  Not together with a keep mask (its
+                                 slices are laid out by the host) and not in a ring-step launch. */
   float mask_min;             /* finfo(blockwise_kwargs["dtype"]).min (:298,:308) */
   int32_t skip_masked_tiles;  /* 1: kernels may also skip sub-tiles whose every pair is masked; exact
                                  unless a query row has no unmasked key at all in the whole ring */
@@ -251,9 +262,24 @@ typedef struct ra_decode_params {
   ra_mask mask;               /* query_chunk_size must be 1; cache_idx pointer or q_chunk_idx_start */
   void* workspace; size_t workspace_bytes;
   int32_t num_splits;         /* 0 = choose */
+  /* One step of a ring whose K/V cache is sharded over the sequence axis (ringattention_jax.py:31-37 with cache_idx
+     and an axis size above one): k, v are then the shard that has arrived, mask.k_chunk_idx_start its first chunk
+     (:37), and the step's result is merged into the carry of the device's one query row instead of being
+     normalised - numerator (B,1,H,D) fp32, denominator and max_score (B,H,1) fp32, updated in place as
+     _blockwise_attention_fwd does (:138-144); the max is the natural-domain one, as in ra_attn_fwd_params.  All three
+     null: no carry, out = the normalised result (a ring of one).  With a carry, out may be null (the step hands the
+     carry on); when given, the step is the last one of its device and out = numerator / denominator (:52). */
+  float* carry_numerator; float* carry_denominator; float* carry_max_score;
+  int64_t carry_num_stride_b;   /* elements; head stride D */
+  int64_t carry_stat_stride_b;  /* elements; head stride 1 */
+  int32_t carry_is_initial;     /* 1: the carry holds (0, 0, -inf) by definition and is not read */
 } ra_decode_params;
 
+/* num_splits == 0: the size for the largest split count the library may choose (256); a caller that wants no more
+ * than the automatic choice needs asks ra_decode_auto_splits first and passes that count here and in the params. */
 size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int32_t num_splits);
+/* The split count ra_decode_fwd picks for num_splits == 0 (0 for a shape it does not take). */
+int ra_decode_auto_splits(int32_t B, int32_t L, int32_t H, int32_t D, int32_t dtype);
 int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream);
 
 /*
@@ -268,6 +294,9 @@ int ra_decode_fwd(const ra_decode_params* p, ra_stream_t stream);
  * RA_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's buffer: two calls that overlap in time on one GPU (two
  * streams, two threads) race; calls on one stream are ordered.  Nothing in the buffer has to start at zero: every
  * partial a call reads was written by that call.
+ * The first call on a GPU looks the array's address up (hipGetSymbolAddress, which may load the code object, under a
+ * mutex): make one eager call per GPU before capturing this entry point into a HIP graph; later calls only launch.
+ * The GPU that owns `stream` must be the current device (refused otherwise): each GPU has its own copy of the array.
  */
 enum { RA_DECODE_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024 };
 int ra_decode_fwd_static(const ra_decode_params* p, ra_stream_t stream);

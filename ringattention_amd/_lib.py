@@ -9,6 +9,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libringattn_hip.so")
 
+RA_ABI_VERSION = 2          # include/ringattn_hip.h; load() refuses a library built for another one
 RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
 RA_F32, RA_BF16 = 0, 1
 RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
@@ -26,7 +27,8 @@ class RaMask(C.Structure):
         ("bias", vp), ("bias_stride_b", i64), ("bias_stride_h", i64), ("bias_stride_q", i64),
         ("bias_stride_k", i64), ("segment_ids", vp), ("seg_stride_b", i64), ("seg_len", i32),
         ("causal_block_size", i32), ("query_chunk_size", i32), ("key_chunk_size", i32),
-        ("q_chunk_idx_start", i32), ("k_chunk_idx_start", i32), ("cache_idx", vp), ("mask_min", f32),
+        ("q_chunk_idx_start", i32), ("k_chunk_idx_start", i32), ("cache_idx", vp), ("chunk_starts", vp),
+        ("mask_min", f32),
         ("skip_masked_tiles", i32), ("seg_tile_minmax", vp), ("seg_tiles", i32),
         ("keep", vp), ("keep_stride_b", i64), ("keep_stride_h", i64), ("keep_stride_q", i64),
         ("keep_stride_k", i64),
@@ -76,6 +78,8 @@ class RaDecodeParams(C.Structure):
         ("B", i32), ("L", i32), ("H", i32), ("D", i32),
         ("q_stride_b", i64), ("kv_stride_b", i64), ("kv_stride_s", i64), ("out_stride_b", i64),
         ("mask", RaMask), ("workspace", vp), ("workspace_bytes", C.c_size_t), ("num_splits", i32),
+        ("carry_numerator", vp), ("carry_denominator", vp), ("carry_max_score", vp),
+        ("carry_num_stride_b", i64), ("carry_stat_stride_b", i64), ("carry_is_initial", i32),
     ]
 
 
@@ -123,6 +127,7 @@ SYMBOLS = {
     "ra_attn_fwd_ring_step": (C.c_int, [C.POINTER(RaAttnFwdParams), C.POINTER(RaRingStep), vp]),
     "ra_attn_bwd_ring_step": (C.c_int, [C.POINTER(RaAttnBwdParams), C.POINTER(RaRingStep), vp]),
     "ra_decode_workspace_bytes": (C.c_size_t, [i32, i32, i32, i32, i32]),
+    "ra_decode_auto_splits": (C.c_int, [i32, i32, i32, i32, i32]),
     "ra_decode_fwd": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
     "ra_decode_fwd_static": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
     "ra_swiglu_fwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
@@ -157,6 +162,9 @@ def load():
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
+    if lib.ra_version() != RA_ABI_VERSION:
+        raise RuntimeError("ringattention_amd: %s speaks interface version %d, this binding version %d; rebuild it "
+                           "with `python -m ringattention_amd.build`" % (LIB_PATH, lib.ra_version(), RA_ABI_VERSION))
     _lib = lib
     return lib
 

@@ -40,7 +40,7 @@ int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, in
                         hipStream_t s);
 int decode_pick_splits(int B, int L, int H, int D, int dtype);
 int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream_t s);
-int decode_static_scratch(float** ptr);
+int decode_static_scratch(float** ptr, hipStream_t stream);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s);
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
@@ -66,6 +66,8 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
                RA_ERR_INVALID, "%s: causal_block_size %d larger than a chunk must be a multiple of it", who, cbs);
   }
   RA_REQUIRE(m.q_chunk_idx_start >= 0 && m.k_chunk_idx_start >= 0, RA_ERR_INVALID, "%s: negative chunk start", who);
+  RA_REQUIRE(!m.chunk_starts || (!m.keep && !m.keep_bits_k && !m.keep_bits_q && !m.keep_summary), RA_ERR_UNSUPPORTED,
+             "%s: chunk starts in device memory do not go with a keep mask (the host lays out its slices)", who);
   if (m.segment_ids) RA_REQUIRE(m.seg_len > 0, RA_ERR_INVALID, "%s: segment_ids given with seg_len 0", who);
   if (m.seg_tile_minmax)
     RA_REQUIRE(m.segment_ids && m.seg_tiles == (m.seg_len + RA_SEG_TILE - 1) / RA_SEG_TILE, RA_ERR_INVALID,
@@ -144,7 +146,7 @@ int ra_rmsnorm_bwd(const ra_rmsnorm_params* p, ra_stream_t stream) {
 }
 
 const char* ra_last_error(void) { return g_err; }
-int ra_version(void) { return 1; }
+int ra_version(void) { return RA_ABI_VERSION; }
 
 int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_stride_s, float* denominator,
                        float* max_score, int64_t stat_stride_b, int64_t stat_stride_h, int32_t B, int32_t Sq,
@@ -301,8 +303,8 @@ static int check_ring(const ra_ring_step* r, const ra_mask& m, int Sq, int Skv, 
   RA_REQUIRE(((r->run | r->first | r->last | r->kv_first | r->kv_last) & ~all) == 0, RA_ERR_INVALID,
              "%s: bits set beyond device %d", who, r->n_dev - 1);
   RA_REQUIRE(impl != RA_IMPL_GENERIC, RA_ERR_UNSUPPORTED, "%s: the MFMA kernels only", who);
-  RA_REQUIRE(!m.keep && !m.keep_bits_k && !m.cache_idx, RA_ERR_UNSUPPORTED,
-             "%s: no keep mask and no cache_idx in a ring-step launch", who);
+  RA_REQUIRE(!m.keep && !m.keep_bits_k && !m.cache_idx && !m.chunk_starts, RA_ERR_UNSUPPORTED,
+             "%s: no keep mask, no cache_idx and no device-side chunk starts in a ring-step launch", who);
   return check_mask(m, Sq / r->n_dev, Skv / r->n_dev, who);
 }
 
@@ -351,6 +353,11 @@ int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring,
   return attn_bwd_mfma(p, ring, RA_BWD_PART_DQ | RA_BWD_PART_DKV, (hipStream_t)stream);
 }
 
+int ra_decode_auto_splits(int32_t B, int32_t L, int32_t H, int32_t D, int32_t dtype) {
+  if (B <= 0 || L <= 0 || H <= 0 || (D != 64 && D != 128) || (dtype != RA_F32 && dtype != RA_BF16)) return 0;
+  return decode_pick_splits(B, L, H, D, dtype);
+}
+
 size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int32_t num_splits) {
   if (B <= 0 || L <= 0 || H <= 0 || D <= 0) return 0;
   int ns = num_splits > 0 ? num_splits : 256;   // upper bound of the automatic choice
@@ -359,7 +366,11 @@ size_t ra_decode_workspace_bytes(int32_t B, int32_t L, int32_t H, int32_t D, int
 
 static int check_decode(const ra_decode_params* p, const char* who) {
   RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
-  RA_REQUIRE(p->q && p->k && p->v && p->out, RA_ERR_INVALID, "%s: null tensor", who);
+  RA_REQUIRE(p->q && p->k && p->v, RA_ERR_INVALID, "%s: null tensor", who);
+  const bool carry = p->carry_numerator || p->carry_denominator || p->carry_max_score;
+  RA_REQUIRE(!carry || (p->carry_numerator && p->carry_denominator && p->carry_max_score), RA_ERR_INVALID,
+             "%s: the carry is numerator, denominator and max_score together", who);
+  RA_REQUIRE(p->out || carry, RA_ERR_INVALID, "%s: out may be null only in a ring step that hands on a carry", who);
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "%s: dtype %d", who, p->dtype);
   RA_REQUIRE(p->B > 0 && p->L > 0 && p->H > 0 && p->D > 0 && p->B <= 65535, RA_ERR_INVALID, "%s: bad shape", who);
   RA_REQUIRE(p->D == 64 || p->D == 128, RA_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128}", who, p->D);
@@ -393,7 +404,7 @@ int ra_decode_fwd_static(const ra_decode_params* p, ra_stream_t stream) {
   const int fit = (int)((size_t)RA_DECODE_STATIC_SCRATCH_BYTES / per_split);
   if (ns > fit) ns = fit;
   float* scratch = nullptr;
-  if (int rc = decode_static_scratch(&scratch)) return rc;
+  if (int rc = decode_static_scratch(&scratch, (hipStream_t)stream)) return rc;
   return decode_fwd(p, scratch, ns, (hipStream_t)stream);
 }
 

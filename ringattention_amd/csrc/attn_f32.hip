@@ -37,7 +37,6 @@ struct F32Args {
   float* dq; int64_t dq_sb, dq_ss;
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
-  const int32_t* cache_idx;
   int carry_is_initial;
   float* out; int64_t out_sb, out_ss;           // forward, nullable: out = num / den instead of the numerator
   float* out32;                                  // forward, nullable: the same once more (strides of out)
@@ -178,7 +177,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
   __shared__ float bias_ks[XBN];
   __shared__ int hull2[2];
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  mv.resolve();
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   RA_F32_STAGE_DECL
   const int nqt = a.Sq / XBM;
@@ -357,7 +356,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
   __shared__ float bias_ks[XBN];
   __shared__ int hull2[2];
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  mv.resolve();
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   RA_F32_STAGE_DECL
   const int nqt = a.Sq / XBM;
@@ -506,7 +505,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   __shared__ __attribute__((aligned(16))) int st_seg[XBN];
   __shared__ int hull2[2];
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  mv.resolve();
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   RA_F32_STAGE_DECL
   const int nkt = a.Skv / XBM;
@@ -780,7 +779,6 @@ int attn_fwd_f32(const ra_attn_fwd_params* p, hipStream_t s) {
   a.num = p->numerator; a.num_sb = p->num_stride_b; a.num_ss = p->num_stride_s;
   a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
   a.out = (float*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr, keep = p->mask.keep_bits_k != nullptr;
@@ -807,7 +805,6 @@ int attn_bwd_f32(const ra_attn_bwd_params* p, int parts, hipStream_t s) {   // p
   a.dk_out = (float*)p->dk_out; a.dv_out = (float*)p->dv_out;
   a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr, keep = p->mask.keep_bits_k != nullptr;
   const long long nq = (long long)(p->Sq / XBM) * p->H * p->B, nk = (long long)(p->Skv / XBM) * p->H * p->B;
   RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_f32: grid too large");

@@ -20,7 +20,6 @@ struct GenericArgs {
   float* dq; int64_t dq_sb, dq_ss;
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
-  const int32_t* cache_idx;
   int carry_is_initial;
   void* out; int64_t out_sb, out_ss;             // forward, nullable: out = num / den instead of the numerator
   float* out32;                                  // forward, nullable: the same quotient un-rounded, strides of out
@@ -31,7 +30,7 @@ struct GenericArgs {
 
 __device__ __forceinline__ MaskView resolve_mask(const GenericArgs& a) {
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;   // ringattention_jax.py:35
+  mv.resolve();
   return mv;
 }
 
@@ -564,7 +563,6 @@ static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
   a.num = p->numerator; a.num_sb = p->num_stride_b; a.num_ss = p->num_stride_s;
   a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
   a.out = p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   return a;
@@ -623,7 +621,6 @@ int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s) {
   a.dq_out = p->dq_out; a.dqo_sb = p->dq_out_stride_b; a.dqo_ss = p->dq_out_stride_s;
   a.dk_out = p->dk_out; a.dv_out = p->dv_out; a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   return p->dtype == RA_F32 ? launch_bwd_T<float>(a, s) : launch_bwd_T<uint16_t>(a, s);
 }
 

@@ -41,7 +41,6 @@ struct FwdArgs {
   float* den; float* mx;
   int64_t st_sb, st_sh;
   MaskView mv;
-  const int32_t* cache_idx;
   int carry_is_initial;
   uint16_t* out; int64_t out_sb, out_ss;      // nullable: last step of the device, out = num / den instead of num
   float* out32;                               // nullable, with out: the quotient before rounding, strides of out
@@ -108,7 +107,6 @@ struct BwdArgs {
   float* dq; int64_t dq_sb, dq_ss;
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
-  const int32_t* cache_idx;
   int dq_initial, dkv_initial;                 // the fp32 accumulator holds zeros by definition: not read
   uint16_t* dq_out; int64_t dqo_sb, dqo_ss;    // nullable: last call that adds into it, the sum goes here as bf16
   uint16_t* dk_out; uint16_t* dv_out; int64_t dkvo_sb, dkvo_ss;
@@ -271,7 +269,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   __shared__ float st_bias[4][64];           // [pair][lane]: the lane's key's clamped, scaled bias
 
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  mv.resolve();
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
   const int nkt = a.Skv / KBN;
@@ -733,7 +731,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   __shared__ float bias_ks[3][FBN];
 
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  mv.resolve();
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
   const int nqt = a.Sq / FBM;
@@ -1193,7 +1191,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   __shared__ float bias_ks[3][FBN];
 
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = (*a.cache_idx) / mv.qc;
+  mv.resolve();
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int role = __builtin_amdgcn_readfirstlane(wave >> 2), pair = wave & 3;
   const int nqt = a.Sq / FBM;
@@ -1719,7 +1717,6 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* r, hipStream_
   a.num = p->numerator; a.num_sb = p->num_stride_b; a.num_ss = p->num_stride_s;
   a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   a.carry_is_initial = p->carry_is_initial;
   a.out = (uint16_t*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
@@ -1775,7 +1772,6 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* r, int parts,
   a.dk_out = (uint16_t*)p->dk_out; a.dv_out = (uint16_t*)p->dv_out;
   a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   const long long nq = (long long)(p->Sq / FBM) * p->H * p->B, nk = (long long)(p->Skv / KBN) * p->H * p->B;
   RA_REQUIRE(nq < (1LL << 31) && nk < (1LL << 31), RA_ERR_UNSUPPORTED, "attn_bwd_mfma: grid too large");
   const dim3 gq((unsigned)((nq + 7) / 8 * 8)), gk((unsigned)((nk + 7) / 8 * 8)), block(512);

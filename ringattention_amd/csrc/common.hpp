@@ -71,6 +71,8 @@ struct MaskView {
   int64_t kpack_sb, kpack_sh, ksum_sb, ksum_sh;
   int keep_Q, keep_K, keep_q0, keep_k0;
   int keep_drop;           // 1: dropout semantics (mask_min added: a pair masked twice becomes -inf)
+  const int32_t* cache_idx;     // nullable device scalar (ringattention_jax.py:35)
+  const int32_t* chunk_starts;  // nullable device pair (q_chunk_idx_start, k_chunk_idx_start) (:31-37, :69-75)
 
   __host__ __device__ static MaskView make(const ra_mask& m, int q_chunk_idx_start) {
     MaskView v;
@@ -90,7 +92,16 @@ struct MaskView {
     v.ksum_sb = m.keep_sum_stride_b; v.ksum_sh = m.keep_sum_stride_h;
     v.keep_Q = m.keep_q_total; v.keep_K = m.keep_k_total; v.keep_q0 = m.keep_q0;
     v.keep_k0 = m.keep_k0; v.keep_drop = m.keep_mode == RA_KEEP_DROPOUT;
+    v.cache_idx = m.cache_idx; v.chunk_starts = m.chunk_starts;
     return v;
+  }
+
+  // The chunk starts a kernel works with: the host ints of ra_mask unless the caller left them in device memory -
+  // under jit lax.axis_index and cache_idx are traced values (:31-37), which a custom call receives as buffers.
+  // Every thread of a kernel calls this first (uniform loads).
+  __device__ __forceinline__ void resolve() {
+    if (chunk_starts) { q_start = chunk_starts[0]; k_start = chunk_starts[1]; }
+    if (cache_idx) q_start = *cache_idx / qc;                        // :35
   }
 
   // Number of leading local keys (out of skv) whose chunk runs against local query chunk qi.

@@ -21,9 +21,12 @@ struct DecodeArgs {
   int B, L, H, D;
   int64_t q_sb, kv_sb, kv_ss, out_sb;
   MaskView mv;
-  const int32_t* cache_idx;
   float* ws;          // [B][H][nsplit][D + 2]
   int nsplit;
+  // ring step: the carry of ringattention_jax.py:22-23,:49 for the one query row, merged in place (nullable)
+  float* c_num; float* c_den; float* c_max;
+  int64_t c_num_sb, c_stat_sb;
+  int carry_is_initial;
 };
 
 constexpr int DEC_THREADS = 512;
@@ -53,7 +56,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
   constexpr int LPH = D / EPL;            // lanes per head
   constexpr int HP = DEC_THREADS / LPH;   // heads per workgroup
   MaskView mv = a.mv;
-  if (a.cache_idx) mv.q_start = *a.cache_idx;          // query_chunk_size == 1 (:35)
+  mv.resolve();                      // query_chunk_size == 1: q_start = cache_idx (:35)
   const int tid = threadIdx.x, b = blockIdx.z, split = blockIdx.x;
   const int h = blockIdx.y * HP + tid / LPH;
   const int dl = tid % LPH;
@@ -150,13 +153,30 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
   }
 }
 
+// Merges the split partials - and, in a ring step, the incoming carry - in a fixed order.  Without a carry the
+// result is the normalised output; with one, (numerator, denominator, max_score) are updated in place as
+// _blockwise_attention_fwd does per key chunk (:138-144), and out (nullable then) is written when the step is the
+// last one of its device (:52).
 template <typename T, int D>
 __global__ void decode_combine_kernel(DecodeArgs a) {
   const int b = blockIdx.y, h = blockIdx.x, d = threadIdx.x;
   const float* w = a.ws + ((int64_t)b * a.H + h) * a.nsplit * (D + 2);
   float M = RA_NEG_INF;
   for (int s = 0; s < a.nsplit; s++) M = fmaxf(M, w[s * (D + 2) + D]);
+  const bool merge = a.c_num && !a.carry_is_initial;
+  float m_in = RA_NEG_INF, num_in = 0.f, den_in = 0.f;
+  if (merge) {
+    m_in = a.c_max[(int64_t)b * a.c_stat_sb + h];
+    den_in = a.c_den[(int64_t)b * a.c_stat_sb + h];
+    num_in = a.c_num[(int64_t)b * a.c_num_sb + (int64_t)h * D + d];
+    M = fmaxf(M, m_in);
+  }
   float num = 0.f, den = 0.f;
+  if (merge && m_in != RA_NEG_INF) {
+    const float c = expf(m_in - M);
+    num = c * num_in;
+    den = c * den_in;
+  }
   for (int s = 0; s < a.nsplit; s++) {
     const float ms = w[s * (D + 2) + D];
     if (ms == RA_NEG_INF) continue;
@@ -164,8 +184,15 @@ __global__ void decode_combine_kernel(DecodeArgs a) {
     num = fmaf(c, w[s * (D + 2) + d], num);
     den = fmaf(c, w[s * (D + 2) + D + 1], den);
   }
+  if (a.c_num) {
+    a.c_num[(int64_t)b * a.c_num_sb + (int64_t)h * D + d] = num;
+    if (d == 0) {
+      a.c_den[(int64_t)b * a.c_stat_sb + h] = den;
+      a.c_max[(int64_t)b * a.c_stat_sb + h] = M;
+    }
+  }
   // no key ran at all: 0/0 = NaN, as numerator/denominator in ringattention_jax.py:52
-  store_from_f32<T>((T*)a.out + (int64_t)b * a.out_sb + (int64_t)h * D + d, num / den);
+  if (a.out) store_from_f32<T>((T*)a.out + (int64_t)b * a.out_sb + (int64_t)h * D + d, num / den);
 }
 
 int decode_pick_splits(int B, int L, int H, int D, int dtype) {
@@ -201,9 +228,16 @@ constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mutex;
 static float* g_scratch_ptr[kMaxDevices];     // per device, filled on the first call with that device current
 
-int decode_static_scratch(float** ptr) {
+int decode_static_scratch(float** ptr, hipStream_t stream) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess && stream) {          // each GPU has its own copy of the array: the stream's GPU must be current
+    hipDevice_t sdev = -1;
+    if (hipStreamGetDevice(stream, &sdev) == hipSuccess && (int)sdev != dev) {
+      set_error("decode_fwd_static: the stream belongs to device %d but device %d is current", (int)sdev, dev);
+      return RA_ERR_INVALID;
+    }
+  }
   if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
     set_error("decode_fwd_static: no usable current device (%s, device %d)", hipGetErrorString(e), dev);
     return RA_ERR_LAUNCH;
@@ -228,8 +262,10 @@ int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream
   a.B = p->B; a.L = p->L; a.H = p->H; a.D = p->D;
   a.q_sb = p->q_stride_b; a.kv_sb = p->kv_stride_b; a.kv_ss = p->kv_stride_s; a.out_sb = p->out_stride_b;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
-  a.cache_idx = p->mask.cache_idx;
   a.ws = partials; a.nsplit = nsplit;
+  a.c_num = p->carry_numerator; a.c_den = p->carry_denominator; a.c_max = p->carry_max_score;
+  a.c_num_sb = p->carry_num_stride_b; a.c_stat_sb = p->carry_stat_stride_b;
+  a.carry_is_initial = p->carry_is_initial;
   if (p->dtype == RA_BF16) {
     if (p->D == 128) return launch_decode<uint16_t, 128>(a, s);
     if (p->D == 64) return launch_decode<uint16_t, 64>(a, s);

@@ -146,6 +146,9 @@ class _Config:
         self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
         # "step": a scan step of all virtual devices goes out as one launch per kernel when the kernels allow;
         # "device": one launch per device and step
+        # False: never reuse the int32 copy / tile ranges of a segment_ids tensor seen before (for callers that edit
+        # the ids through a numpy alias or .data, which the tensor's version counter does not see)
+        self.cache_segment_ids = bool(kw.get("cache_segment_ids", True))
         self.ring_launch = kw.get("ring_launch", "step")
         if self.ring_launch not in ("step", "device"):
             raise ValueError("ring_launch must be 'step' or 'device'")
@@ -188,24 +191,29 @@ class _MaskInputs:
                 raise ValueError("segment_ids must be 2-D (B, S)")
             # the int32 copy, the per-tile id ranges and their host copy are kept per segment_ids tensor (same
             # storage, same version counter): a later call with the tensor unchanged launches nothing for them and
-            # copies nothing to the host, so it can be captured into a HIP graph
-            key = (segment_ids.data_ptr(), segment_ids._version, tuple(segment_ids.shape), segment_ids.dtype,
-                   str(segment_ids.device), str(device))
-            hit = _SEG_CACHE.get(key)
-            if hit is not None and hit[0]() is segment_ids:
+            # copies nothing to the host, so it can be captured into a HIP graph.  The version counter does not see
+            # edits through a numpy alias (torch.from_numpy) or through .data: such callers pass
+            # blockwise_kwargs["cache_segment_ids"] = False.  Tensors made under torch.inference_mode() have no
+            # version counter and are never cached.  An entry is reused on the stream that produced it, and on any
+            # other stream once its host copy exists (that copy waited for the kernels that wrote the entry).
+            key = None
+            cur_stream = torch.cuda.current_stream(device).cuda_stream if torch.device(device).type == "cuda" else 0
+            if cfg.cache_segment_ids:
+                try:
+                    key = (segment_ids.data_ptr(), segment_ids._version, tuple(segment_ids.shape), segment_ids.dtype,
+                           str(segment_ids.device), str(device))
+                except RuntimeError:          # inference tensors do not track a version counter
+                    key = None
+            hit = _SEG_CACHE.get(key) if key is not None else None
+            if hit is not None and hit[0]() is segment_ids and (hit[4] == cur_stream or hit[3] is not None):
                 _SEG_CACHE.move_to_end(key)
                 self._seg_entry = hit
             else:
-                s = segment_ids.detach().to(device=device, dtype=torch.int32).contiguous()
-                # per-64-position (min, max) ids: lets the MFMA kernels skip tiles of foreign segments
-                tiles = (s.shape[1] + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
-                mm = torch.empty((s.shape[0], tiles, 2), dtype=torch.int32, device=device)
-                L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], s.shape[1],
-                                                        mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
-                self._seg_entry = [weakref.ref(segment_ids), s, mm, None]
-                _SEG_CACHE[key] = self._seg_entry
-                while len(_SEG_CACHE) > 8:
-                    _SEG_CACHE.popitem(last=False)
+                self._seg_entry = self._segment_entry(segment_ids, device) + [cur_stream]
+                if key is not None:
+                    _SEG_CACHE[key] = self._seg_entry
+                    while len(_SEG_CACHE) > 8:
+                        _SEG_CACHE.popitem(last=False)
             s = self._seg_entry[1]
             self.seg = s
             self.seg_stride_b = 0 if s.shape[0] == 1 else s.stride(0)
@@ -231,6 +239,24 @@ class _MaskInputs:
                     self.cache_idx_host = int(cache_idx)
             else:
                 self.cache_idx_host = int(cache_idx)
+
+    @staticmethod
+    def _segment_entry(segment_ids, device):
+        """[weakref, int32 ids on the device, per-64-position (min, max) id ranges, host copy of the ranges (lazy)];
+        the caller appends the stream that produced them."""
+        s = segment_ids.detach().to(device=device, dtype=torch.int32).contiguous()
+        tiles = (s.shape[1] + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
+        mm = torch.empty((s.shape[0], tiles, 2), dtype=torch.int32, device=device)
+        if s.is_cuda:
+            # lets the MFMA kernels skip tiles of foreign segments
+            L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], s.shape[1],
+                                                    mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
+        else:                                  # host logic only (tests without a GPU): same ranges with torch ops
+            pad = tiles * L.RA_SEG_TILE - s.shape[1]
+            sp = torch.nn.functional.pad(s, (0, pad), mode="replicate") if pad else s
+            sp = sp.view(s.shape[0], tiles, L.RA_SEG_TILE)
+            mm = torch.stack((sp.amin(dim=2), sp.amax(dim=2)), dim=2).to(torch.int32)
+        return [weakref.ref(segment_ids), s, mm, None]
 
     def set_keep(self, attn_mask, device, q_total, k_total):
         """attn_mask (B|1, H|1, Q|1, K_total), nonzero = attend (ringattention_inference.py:19-22).
@@ -327,8 +353,12 @@ class _MaskInputs:
         self.keep_k0 = k_chunk_idx_start * cfg.kc
         self.keep_mode = L.RA_KEEP_DROPOUT
 
-    def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip):
+    def fill(self, cfg, q_chunk_idx_start, k_chunk_idx_start, skip, chunk_starts=None):
         m = L.RaMask()
+        if chunk_starts is not None:            # int32[2] in device memory: the kernels read the starts there
+            self._chunk_starts = chunk_starts   # kept alive with the mask inputs
+            m.chunk_starts = chunk_starts.data_ptr()
+            q_chunk_idx_start = k_chunk_idx_start = 0
         m.bias = self.bias.data_ptr() if self.bias is not None else None
         m.bias_stride_b, m.bias_stride_h, m.bias_stride_q, m.bias_stride_k = self.bias_strides
         m.segment_ids = self.seg.data_ptr() if self.seg is not None else None
@@ -396,6 +426,25 @@ def _rows(t):
 
 
 # --------------------------------------------------------------------------- one ring step
+def _device_chunk_starts(q_chunk_idx_start, k_chunk_idx_start, device):
+    """The chunk starts as the kernels take them from device memory (ra_mask.chunk_starts), or None when both are
+    Python ints.  Under jit the reference computes them from lax.axis_index (:31-37, :69-75), a traced value; the
+    counterpart here is a device tensor: either one int32 tensor of two elements passed as q_chunk_idx_start (with
+    k_chunk_idx_start None: no kernel is launched to pack them, so the call can be captured into a HIP graph and
+    replayed with other values in the tensor), or two scalars of which at least one is a device tensor."""
+    qt, kt = isinstance(q_chunk_idx_start, torch.Tensor), isinstance(k_chunk_idx_start, torch.Tensor)
+    if not qt and not kt:
+        return None
+    if qt and k_chunk_idx_start is None:
+        cs = q_chunk_idx_start
+        if cs.numel() != 2 or cs.dtype != torch.int32 or not cs.is_cuda or not cs.is_contiguous():
+            raise ValueError("chunk starts in one tensor: a contiguous int32 device tensor of two elements")
+        return cs.reshape(2)
+    parts = [t.to(device=device, dtype=torch.int32).reshape(1) if isinstance(t, torch.Tensor)
+             else torch.tensor([int(t)], dtype=torch.int32, device=device) for t in (q_chunk_idx_start, k_chunk_idx_start)]
+    return torch.cat(parts)
+
+
 def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_start, bias, segment_ids,
                              causal_block_size, query_chunk_size, key_chunk_size, deterministic=True,
                              dropout_rng=None, attn_pdrop=0.0, dtype=torch.float32, policy=None,
@@ -412,8 +461,13 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
     _check_qkv(q, k, v)
     B, Sq, H, D = q.shape
     Skv = k.shape[1]
+    starts_dev = _device_chunk_starts(q_chunk_idx_start, k_chunk_idx_start, q.device)
+    if starts_dev is not None:
+        q_chunk_idx_start = k_chunk_idx_start = 0      # unknown to the host: nothing below may depend on them
+        if cfg.pdrop > 0.0:
+            raise NotImplementedError("attention dropout needs chunk starts the host knows")
     mi = _mask_inputs or _MaskInputs(cfg, bias, segment_ids, cache_idx, B, q.device,
-                                     k_chunk_idx_start * cfg.kc + Skv)
+                                     (k_chunk_idx_start * cfg.kc + Skv) if starts_dev is None else 0)
     num, den, mx = carry
     p = L.RaAttnFwdParams()
     p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
@@ -449,7 +503,7 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
     if cfg.pdrop > 0.0:
         mi.use_dropout(cfg, B, H, Sq, Skv, q_chunk_idx_start, k_chunk_idx_start, q.device)
         skip = False        # a row may lose every allowed key: its masked tiles then carry its (uniform) weights
-    p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
+    p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip, starts_dev)
     p.impl = cfg.impl
     p.carry_is_initial = 1 if _carry_is_initial else 0
     L.check(L.load().ra_attn_fwd_block(ctypes.byref(p), _stream()), "ra_attn_fwd_block")
@@ -472,8 +526,13 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
     _check_qkv(q, k, v)
     B, Sq, H, D = q.shape
     Skv = k.shape[1]
+    starts_dev = _device_chunk_starts(q_chunk_idx_start, k_chunk_idx_start, q.device)
+    if starts_dev is not None:
+        q_chunk_idx_start = k_chunk_idx_start = 0
+        if cfg.pdrop > 0.0:
+            raise NotImplementedError("attention dropout needs chunk starts the host knows")
     mi = _mask_inputs or _MaskInputs(cfg, bias, segment_ids, cache_idx, B, q.device,
-                                     k_chunk_idx_start * cfg.kc + Skv)
+                                     (k_chunk_idx_start * cfg.kc + Skv) if starts_dev is None else 0)
     dq, dk, dv, output, den, mx = carry
     if g.dtype != q.dtype:
         g = g.to(q.dtype)
@@ -524,7 +583,7 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
     if cfg.pdrop > 0.0:
         mi.use_dropout(cfg, B, H, Sq, Skv, q_chunk_idx_start, k_chunk_idx_start, q.device)
         skip = False
-    p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip)
+    p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip, starts_dev)
     p.impl = cfg.impl
     if cfg.bwd_only:
         L.check(L.load().ra_attn_bwd_block_part(ctypes.byref(p), cfg.bwd_only, _stream()), "ra_attn_bwd_block_part")
@@ -908,9 +967,16 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
     One query token with cache_idx set takes the streaming decode kernel."""
     # (the streaming kernel serves head sizes 64 and 128; any other takes the blockwise kernels below, like a call
     # that wants gradients)
-    if cache_idx is not None and q.shape[1] == 1 and q.shape[3] in (64, 128) and axis_size(axis_name) == 1 and not (
-            torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
-        from .decode import decode_attention
-        return decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs)
+    n = axis_size(axis_name)
+    if cache_idx is not None and q.shape[1] == n and q.shape[3] in (64, 128) and not (
+            torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) \
+            and int(dict(blockwise_kwargs)["query_chunk_size"]) == 1:
+        from .decode import decode_attention, decode_attention_ring
+        if n == 1:
+            return decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs)
+        # one query token per virtual device and the cache sharded over the ring: every shard is streamed with
+        # the split kernel and merged into the device's carry
+        if k.shape[1] % n == 0 and (k.shape[1] // n) % int(dict(blockwise_kwargs)["key_chunk_size"]) == 0:
+            return decode_attention_ring(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwargs, n)
     return _RingAttentionFn.apply(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits,
                                   blockwise_kwargs)

@@ -60,3 +60,66 @@ def test_decode_split_counts_agree():
     outs = [ra.decode_attention(qd, kd, vd, None, None, 1999, kw, num_splits=ns).float() for ns in (1, 3, 8, 64)]
     for o in outs[1:]:
         assert errors(o, outs[0])[0] < 1e-2
+
+
+@pytest.mark.parametrize("n", [2, 4, 8])
+@pytest.mark.parametrize("cache_idx", [65535, 40000, 8192])
+def test_ring_sharded_decode_matches_oracle(n, cache_idx):
+    """cache_idx with an axis size above one (ringattention_jax.py:31-37): one query token per virtual device, the
+    cache of 65536 positions sharded over the ring; every shard goes through the streaming kernel with a carry.
+    8192 is the edge at which the query's own key chunk does not run (:324-331) and, on rings of 8, a shard start."""
+    B, L, H, D, kc = 1, 65536, 4, 128, 512
+    print("ring decode", n, cache_idx, flush=True)
+    q, k, v, _ = make_qkv(B, n, H, D, dtype=torch.bfloat16, seed=n, Skv=L, scale=D ** -0.25)
+    g = torch.Generator().manual_seed(11)
+    bias = torch.randn(B, 1, 1, L, generator=g)
+    seg = packed_segment_ids(B, L, 20000, seed=12)
+    kw = kwargs(1, kc, 1)
+    ref = O.ring_attention(q, k, v, bias, seg, cache_idx, n, True, oracle_kwargs(kw))
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention(qd, kd, vd, bias.to(DEV), seg.to(DEV), cache_idx, axis_name="sp", float32_logits=True,
+                               blockwise_kwargs=kw)
+        # the same call through the blockwise kernels (wanting gradients keeps it off the streaming kernel)
+        slow = ra.ringattention(qd.clone().requires_grad_(True), kd, vd, bias.to(DEV), seg.to(DEV), cache_idx,
+                                axis_name="sp", float32_logits=True, blockwise_kwargs=kw)
+    assert_close(out, ref, torch.bfloat16, "ring decode")
+    assert errors(out, slow)[0] <= 2e-2
+
+
+def test_ring_sharded_decode_position_zero_is_nan_everywhere():
+    n, B, L, H, D, kc = 4, 1, 2048, 2, 64, 128
+    q, k, v, _ = make_qkv(B, n, H, D, dtype=torch.float32, seed=1, Skv=L)
+    kw = kwargs(1, kc, 1)
+    ref = O.ring_attention(q, k, v, None, None, 0, n, True, oracle_kwargs(kw))
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention(q.to(DEV), k.to(DEV), v.to(DEV), None, None, 0, axis_name="sp", float32_logits=True,
+                               blockwise_kwargs=kw)
+    assert torch.isnan(ref).all() and torch.isnan(out).all()
+
+
+def test_decode_carry_of_one_step_equals_the_plain_call_bitwise():
+    """A ring of one through the carry form: numerator / denominator of the single step is the plain result."""
+    B, L, H, D, kc = 2, 4096, 4, 128, 256
+    q, k, v, _ = make_qkv(B, 1, H, D, dtype=torch.bfloat16, seed=9, Skv=L)
+    kw = kwargs(1, kc, 1)
+    qd, kd, vd = (t.to(DEV) for t in (q, k, v))
+    plain = ra.decode_attention(qd, kd, vd, None, None, 3000, kw)
+    num = torch.empty((B, 1, H, D), dtype=torch.float32, device=DEV)
+    den = torch.empty((B, H, 1), dtype=torch.float32, device=DEV)
+    mx = torch.empty((B, H, 1), dtype=torch.float32, device=DEV)
+    out = ra.decode_attention(qd, kd, vd, None, None, 3000, kw, carry=(num, den, mx), carry_is_initial=True)
+    assert torch.equal(plain, out)
+    assert torch.equal((num / den.reshape(B, 1, H, 1)).to(torch.bfloat16), plain)
+
+
+def test_default_workspace_is_sized_for_the_automatic_split_count():
+    from ringattention_amd import _lib
+    from ringattention_amd.decode import decode_workspace
+    B, L, H, D = 4, 8192, 32, 128
+    q = torch.empty((B, 1, H, D), dtype=torch.bfloat16, device=DEV)
+    k = torch.empty((B, L, H, D), dtype=torch.bfloat16, device=DEV)
+    ns = _lib.load().ra_decode_auto_splits(B, L, H, D, _lib.RA_BF16)
+    assert 1 <= ns <= 256
+    assert decode_workspace(q, k).numel() == B * H * ns * (D + 2) * 4
+    assert decode_workspace(q, k).numel() < _lib.load().ra_decode_workspace_bytes(B, L, H, D, 0)

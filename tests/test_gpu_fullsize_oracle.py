@@ -338,3 +338,47 @@ def test_fp32_16k_ring4_matches_oracle():
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
         rows.append((name,) + assert_close(a, b, torch.float32, "fp32 16k " + name))
     print("fp32 16k ring 4: oracle %.1f s;" % secs, "; ".join("%s max-abs %.2e rel-L2 %.2e" % r for r in rows), flush=True)
+
+
+_SWIGLU_ORACLE = {}     # tokens -> the oracle's (y, dx, dw1, dw2, dw3) and wall time: the cases of a size share inputs
+
+
+@pytest.mark.parametrize("tokens,chunk,launch,policy,tile", [
+    (2048, 2048, None, "nothing_saveable", None),          # one 2048-token chunk per launch: the library picks 256 x 128
+    (2048, 2048, None, "save_preactivations", 0),          # the same chunk with the 256 x 256 tile kernel forced
+    (16384, 2048, 16384, "nothing_saveable", None),        # eight chunks sharing one launch: 256 x 256 tiles
+    (16384, 2048, 16384, "save_preactivations", 3),        # ... and with the 256 x 128 tile kernel forced
+])
+def test_swiglu_llama7b_shape_matches_oracle(tokens, chunk, launch, policy, tile):
+    """blockwise_feedforward over SwiGLU(4096, 11008) - the shape of BASELINE configuration 4, K = 11008 being 172
+    slabs of 64 and 43 column tiles of 256 - forward and backward against the oracle's formula under fp32 autograd
+    on the CPU (ringattention_jax.py:333-352): bf16 outputs of fp32-accumulated products, relative L2 <= 1e-2 and
+    max-abs within 2e-2 of the output's scale."""
+    from tests.test_gpu_feedforward import rel_ok
+    d, f = 4096, 11008
+    print("swiglu case", dict(tokens=tokens, chunk=chunk, launch=launch, policy=policy, tile=tile), flush=True)
+    g = torch.Generator().manual_seed(tokens)
+    x = torch.randn(1, tokens, d, generator=g).bfloat16()
+    dy = torch.randn(1, tokens, d, generator=g).bfloat16()
+    torch.manual_seed(4096 + tokens)                       # the weights are drawn on the device from the global stream
+    ff = ra.SwiGLU(d, f, device=DEV, init_std=0.02, gemm_tile=tile)
+    xd = x.to(DEV).requires_grad_(True)
+    y = ra.blockwise_feedforward(ff, xd, chunk, policy=policy, launch_tokens=launch)
+    y.backward(dy.to(DEV))
+    torch.cuda.synchronize()
+    if tokens not in _SWIGLU_ORACLE:
+        t0 = time.time()
+        w1, w2, w3 = (w.detach().float().cpu().requires_grad_(True) for w in (ff.w1, ff.w2, ff.w3))
+        xr = x.float().requires_grad_(True)
+        yr = O.blockwise_feedforward(lambda h: O.swiglu(h, w1, w2, w3), xr, chunk)
+        yr.backward(dy.float())
+        _SWIGLU_ORACLE.clear()                             # one size at a time: a gigabyte of gradients each
+        _SWIGLU_ORACLE[tokens] = ((yr.detach(), xr.grad, w1.grad, w2.grad, w3.grad), time.time() - t0,
+                                  ff.w1.detach().clone())
+    ref, secs, w1_seen = _SWIGLU_ORACLE[tokens]
+    assert torch.equal(w1_seen, ff.w1.detach()), "the cases of one size must share their weights"
+    print("  oracle %.1f s" % secs, flush=True)
+    for name, a, b in zip(("y", "dx", "dw1", "dw2", "dw3"), (y, xd.grad, ff.w1.grad, ff.w2.grad, ff.w3.grad), ref):
+        ma, rl = errors(a, b)
+        print("  %-3s max-abs %.3e rel-L2 %.3e (scale %.3e)" % (name, ma, rl, float(b.abs().max())), flush=True)
+        rel_ok(a, b, name)

@@ -24,7 +24,8 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert getattr(lib, name) is not None
-    assert lib.ra_version() >= 1
+    macro = int(re.search(r"#define\s+RA_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "ringattn_hip.h")).read()).group(1))
+    assert lib.ra_version() == macro == _lib.RA_ABI_VERSION
 
 
 def test_struct_sizes_match_a_c_compiler(tmp_path):
@@ -189,3 +190,37 @@ def test_output_residual_option():
     assert _Config(dict(base, output_residual="rounded")).output_residual == "rounded"
     with pytest.raises(ValueError):
         _Config(dict(base, output_residual="bf16"))
+
+
+def test_mask_inputs_accept_segment_ids_made_under_inference_mode():
+    """Inference tensors have no version counter: the per-tensor cache of the int32 ids and tile ranges is bypassed
+    for them instead of raising, and the ranges equal those of an ordinary tensor."""
+    from ringattention_amd import ringattention_hip as R
+    cfg = R._Config(dict(query_chunk_size=128, key_chunk_size=128, causal_block_size=1))
+    ids = torch.arange(300) // 70
+    with torch.inference_mode():
+        seg = ids.clone().reshape(1, -1)
+        with pytest.raises(RuntimeError):
+            seg._version
+        mi = R._MaskInputs(cfg, None, seg, None, 1, "cpu", 300)
+    ref = R._MaskInputs(cfg, None, ids.reshape(1, -1), None, 1, "cpu", 300)
+    assert torch.equal(mi.seg_mm, ref.seg_mm) and torch.equal(mi.seg, ref.seg)
+    assert mi.seg_mm.shape == (1, 5, 2)
+    assert mi.seg_mm[0, 1].tolist() == [0, 1] and mi.seg_mm[0, 4].tolist() == [3, 4]
+    assert mi.segments_meet(0, 64, 256, 300) is False and mi.segments_meet(0, 128, 64, 128) is True
+
+
+def test_segment_cache_follows_the_version_counter_and_the_opt_out():
+    from ringattention_amd import ringattention_hip as R
+    cfg = R._Config(dict(query_chunk_size=128, key_chunk_size=128, causal_block_size=1))
+    seg = (torch.arange(256) // 100).reshape(1, -1)
+    a = R._MaskInputs(cfg, None, seg, None, 1, "cpu", 256)
+    b = R._MaskInputs(cfg, None, seg, None, 1, "cpu", 256)
+    assert a._seg_entry is b._seg_entry                  # unchanged tensor: one entry
+    seg[0, 0] = 7                                        # in-place edit bumps the version: recomputed
+    c = R._MaskInputs(cfg, None, seg, None, 1, "cpu", 256)
+    assert c._seg_entry is not a._seg_entry and c.seg_mm[0, 0].tolist() == [0, 7]
+    seg.numpy()[0, 1] = 9                                # an edit the counter does not see needs the opt-out
+    cfg2 = R._Config(dict(query_chunk_size=128, key_chunk_size=128, causal_block_size=1, cache_segment_ids=False))
+    d = R._MaskInputs(cfg2, None, seg, None, 1, "cpu", 256)
+    assert d.seg_mm[0, 0].tolist() == [0, 9]

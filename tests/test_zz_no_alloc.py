@@ -86,3 +86,35 @@ def test_static_scratch_entry_rejects_what_cannot_fit():
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     assert lib.ra_decode_fwd_static(ctypes.byref(p), stream) == L.RA_ERR_UNSUPPORTED
     assert b"scratch" in lib.ra_last_error()
+
+
+def test_static_scratch_decode_replays_from_a_graph():
+    """decode_attention(static_scratch=True) after one eager warm-up call (which looks the buffer's address up),
+    captured into a graph and replayed for several positions - the position sits in device memory - with eager
+    work between the replays; every replay must give the bits of the workspace path."""
+    import ringattention_amd as ra
+    from tests.util import kwargs
+    B, Lc, H, D, kc = 2, 4096, 8, 128, 128
+    g = torch.Generator(device=DEV).manual_seed(31)
+    q = torch.randn(B, 1, H, D, device=DEV, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Lc, H, D, device=DEV, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Lc, H, D, device=DEV, generator=g).to(torch.bfloat16)
+    kw = kwargs(1, kc, 1)
+    pos = torch.tensor(100, dtype=torch.int32, device=DEV)
+    out = torch.empty_like(q)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ra.decode_attention(q, k, v, None, None, pos, kw, out=out, static_scratch=True)       # warm-up
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ra.decode_attention(q, k, v, None, None, pos, kw, out=out, static_scratch=True)
+    for p in (100, 4095, 777, 128, 2048):
+        pos.fill_(p)
+        want = ra.decode_attention(q, k, v, None, None, p, kw)        # eager, workspace path, between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(want, out), p
