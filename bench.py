@@ -310,14 +310,42 @@ def bench_attention(args, ring, dropout=False, c1=False):
         if dropout:
             roof["traffic"] = None
             roof["mask_draw_and_pack_ms"] = round(mask_ms, 3)
-    if ring and not args.no_extras:
-        # clock and board power over whole steps: what tells a power-limited step from a stall-limited one
-        whole = _sclk_under_load(step)
-        if whole:
-            roof = {"bound": "mfma", "kernel": None, "achieved": round(value, 1), "peak": peak,
-                    "unit": "TFLOP/s", "frac": round(value / peak, 4), "traffic": None,
-                    "scope": "whole step (six attention launches), FLOP of unmasked pairs",
-                    "power_w_under_load": whole.pop("power_w", None), "sclk_mhz_under_load": whole}
+    if ring:
+        # per kernel: the sum of its launches over the scan steps of one pass (two steps have work: every device
+        # against its own shard, then the documents that straddle a shard boundary), events on the launch stream
+        import copy
+        with torch.no_grad(), ra.ring_axis("sp", n):
+            qd, kd, vd = q.detach(), k.detach(), v.detach()
+            fwd = lambda: rh._ring_attention_fwd(qd, kd, vd, bias, seg, None, "sp", True, kw)
+            res = fwd()[1]
+            kern["attn_fwd_ws_kernel"] = (_event_ms(fwd, 3), flops_fwd)
+            t_delta = _event_ms(lambda: rh._bwd_delta(do, res[0]), 3)
+            for which, share in (("dkv", 8.0), ("dq", 2.0)):
+                cfg_p = copy.copy(res[5])
+                cfg_p.bwd_only = {"dq": 1, "dkv": 2}[which]        # RA_BWD_PART_*
+                res_p = res[:5] + (cfg_p,) + res[6:]
+                t = _event_ms(lambda: rh._ring_attention_bwd(res_p, do), 3) - t_delta
+                kern["attn_bwd_%s_ws_kernel" % which] = (t, share * D * pairs * B * H)
+            del res, res_p
+        util = _measured(MFMA_PROFILE, "mfma_util")
+        dom = max(kern, key=lambda n_: kern[n_][0])
+        dms, dfl = kern[dom]
+        ach = dfl / (dms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s",
+                "frac": round(ach / peak, 4), "traffic": None,
+                "scope": "the kernel's launches of one pass summed (one per scan step with work, host launch gaps "
+                         "included), FLOP of unmasked pairs: 8*D per pair for dK/dV, 2*D for dQ, 4*D forward",
+                "mfma_util_pmc": ({"kernel": util.get("ring131k:" + dom), "step": util.get("ring131k_step"),
+                                   "source": "profiles/" + MFMA_PROFILE}
+                                  if S == 131072 and util.get("ring131k:" + dom) else None),
+                "kernel_ms": {n_: round(t, 3) for n_, (t, _) in kern.items()},
+                "kernel_tflops": {n_: round(f / (t * 1e-3) / 1e12, 1) for n_, (t, f) in kern.items()}}
+        if not args.no_extras:
+            # clock and board power over whole steps: what tells a power-limited step from a stall-limited one
+            whole = _sclk_under_load(step)
+            if whole:
+                roof["power_w_under_load"] = whole.pop("power_w", None)
+                roof["sclk_mhz_under_load"] = whole
     if c1:
         roof = {"bound": "mfma", "kernel": None, "achieved": round(value, 2), "peak": peak, "unit": "TFLOP/s",
                 "frac": round(value / peak, 4), "traffic": None,
@@ -325,6 +353,8 @@ def bench_attention(args, ring, dropout=False, c1=False):
     cpu = None
     if c1 and not args.no_cpu:
         cpu = cpu_baseline_c1(q.detach().cpu(), k.detach().cpu(), v.detach().cpu(), do.cpu(), kw)
+    elif ring and not args.no_cpu:
+        cpu = cpu_baseline_ring(lens)
     elif not (args.no_cpu or dropout):
         cpu = cpu_baseline_attention()
     del q, k, v, do
@@ -383,6 +413,32 @@ def cpu_baseline_attention():
             "sample": "8 heads (of 32) at full S=32768, fwd+bwd, %.1f s" % dt}
 
 
+def cpu_baseline_ring(lens):
+    """The CPU oracle on a slice of the ring131k workload: one head (of 32) over the first 65536 positions (of
+    131072) as a ring of four shards of 16384, the same packed documents and a per-key bias, forward + backward."""
+    import numpy as np
+    import torch
+    from oracle import ringattention_oracle as O
+    S, D, n = 65536, 128, 4
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    q, k, v, do = (torch.randn(1, S, 1, D, generator=g) * (D ** -0.5 if i < 3 else 1.0) for i in range(4))
+    bias = torch.randn(1, 1, 1, S, generator=g)
+    ids = np.repeat(np.arange(len(lens)), lens)[:S].astype(np.int32)
+    seg = torch.from_numpy(ids).reshape(1, S)
+    cut = np.bincount(ids).astype(np.float64)                    # document lengths inside the slice
+    pairs = float((cut * (cut + 1) / 2).sum())
+    kw = _kwargs(512, 512, 1)
+    t0 = time.perf_counter()
+    out, res = O.ring_attention_fwd(q, k, v, bias, seg, None, n, True, kw)
+    O.ring_attention_bwd(n, True, kw, res, do)
+    dt = time.perf_counter() - t0
+    return {"value": round(14.0 * D * pairs / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "1 head (of 32), the first 65536 positions (of 131072) as a ring of 4, documents + bias, "
+                      "fwd+bwd, FLOP of unmasked pairs, %.1f s" % dt}
+
+
 # --------------------------------------------------------------------------- decode workload
 def bench_decode(args, steps=0):
     import torch
@@ -411,8 +467,8 @@ def bench_decode(args, steps=0):
     ms = _time_steps(step, args.steps, args.warmup)
     bytes_step = 2.0 * B * (Lf + 1) * H * D * 2
     value = bytes_step / (ms * 1e-3) / 1e9
-    # the split kernel alone (the combine pass that follows it moves 0.05 GB): events around the whole step, minus
-    # nothing - the step is this kernel to within 1 %
+    # events around the whole step: the fill of the position scalar, the split kernel and the combine pass that merges
+    # its partials (0.05 GB); the split kernel is 98.9 % of that by the kernel trace
     kms = _event_ms(step, 5)
     ach = bytes_step / (kms * 1e-3) / 1e9
     cpu = None
@@ -438,8 +494,10 @@ def bench_decode(args, steps=0):
         "steps": steps or args.steps,
         "config": {"workload": "decode", "B": B, "H": H, "D": D, "cache_len": Lf, "key_chunk_size": kc,
                    "query_chunk_size": 1, "bytes_per_step": bytes_step},
-        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4),
+        "roofline": {"bound": "hbm", "kernel": "decode_split_kernel + decode_combine_kernel", "achieved": round(ach, 1),
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4),
+                     "scope": "algorithmic bytes of a step / events around the whole step on the launch stream "
+                              "(position fill + split kernel + combine kernel)",
                      "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("decode_split_kernel")
                                  if (B, Lf) == (16, 262144) else None),
                      "traffic_source": "profiles/" + TRAFFIC_PROFILE},
@@ -521,8 +579,10 @@ def bench_ffn(args):
                      "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
                      "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("gemm_bf16_w4_kernel<false,false,256>")
                                  if (T, slab) == (65536, 16384) else None),
-                     "mfma_util_pmc": {"kernel": (_measured(MFMA_PROFILE, "mfma_util").get("gemm_bf16_w4_kernel<false,false,256>")
-                                                  if (T, slab) == (65536, 16384) else None),
+                     "mfma_util_pmc": {"kernel": (_measured(MFMA_PROFILE, "mfma_util").get(
+                                           "gemm_bf16_w4_kernel<false,false,256>" if slab == 16384
+                                           else "ffn2048:gemm_bf16_w4_kernel<false,false,128>")
+                                                  if T == 65536 and slab in (2048, 16384) else None),
                                        "source": "profiles/" + MFMA_PROFILE},
                      "kernel_ms": {gemm_name: round(gemm_ms, 3)},
                      "power_w_under_load": sclk.pop("power_w", None) if sclk else None,
@@ -848,14 +908,13 @@ def main():
             # the other two configurations: the virtual ring of eight over 131072 positions with packed documents and a
             # bias, and the SwiGLU feed-forward over 65536 tokens (one chunk per launch, and 16384 tokens per launch)
             torch.cuda.empty_cache()
-            rg = bench_attention(argparse.Namespace(**dict(vars(args), no_cpu=True, no_extras=True, steps=3, warmup=1)),
-                                 ring=True)
-            extras["ring131k"] = {k_: rg[k_] for k_ in ("metric", "value", "unit", "ms_per_step", "dtype", "config")}
+            rg = bench_attention(argparse.Namespace(**dict(vars(args), no_extras=True, steps=3, warmup=1)), ring=True)
+            extras["ring131k"] = {k_: rg[k_] for k_ in ("metric", "value", "unit", "ms_per_step", "dtype", "config",
+                                                        "roofline", "cpu_baseline")}
             torch.cuda.empty_cache()
-            ff = bench_ffn(argparse.Namespace(**dict(vars(args), no_cpu=True, steps=3, warmup=1)))
+            ff = bench_ffn(argparse.Namespace(**dict(vars(args), steps=3, warmup=1)))
             extras["ffn"] = {k_: ff[k_] for k_ in ("metric", "value", "unit", "ms_per_step", "dtype", "config",
-                                                   "launch_tokens_16384")}
-            extras["ffn"]["gemm"] = {k_: ff["roofline"][k_] for k_ in ("kernel", "achieved", "unit", "frac")}
+                                                   "launch_tokens_16384", "roofline", "cpu_baseline")}
     elif args.workload == "decode":
         r = bench_decode(args)
     elif args.workload == "copy":

@@ -17,6 +17,8 @@ extern "C" {
  * the other one would have written is left untouched, and may be null. */
 enum { RA_BWD_PART_DQ = 1, RA_BWD_PART_DKV = 2 };
 int ra_attn_bwd_block_part(const ra_attn_bwd_params* p, int32_t part, ra_stream_t stream);
+/* The same for ra_attn_bwd_ring_step: one of its two kernels for every device of the ring. */
+int ra_attn_bwd_ring_step_part(const ra_attn_bwd_params* p, const ra_ring_step* ring, int32_t part, ra_stream_t stream);
 
 /* ra_gemm_bf16 with the tile kernel named: tile -1 = the library's choice, 0: 256 x 256 over four wavefronts,
  * 1: 256 x 128 over eight, 2: 128 x 128, 3: 256 x 128 over four (a forced tile still gives way to another one where

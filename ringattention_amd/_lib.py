@@ -141,6 +141,7 @@ SYMBOLS = {
     "ra_version": (C.c_int, []),
     # measurement / test hooks
     "ra_attn_bwd_block_part": (C.c_int, [C.POINTER(RaAttnBwdParams), i32, vp]),
+    "ra_attn_bwd_ring_step_part": (C.c_int, [C.POINTER(RaAttnBwdParams), C.POINTER(RaRingStep), i32, vp]),
     "ra_gemm_bf16_tile": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp]),
     "ra_mfma_rate_probe": (C.c_int, [vp, i32, i32, i32, vp]),
 }

@@ -327,8 +327,9 @@ int ra_attn_fwd_ring_step(const ra_attn_fwd_params* p, const ra_ring_step* ring,
   return attn_fwd_mfma(p, ring, (hipStream_t)stream);
 }
 
-int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring, ra_stream_t stream) {
-  const char* who = "attn_bwd_ring_step";
+static int attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring, int parts, const char* who,
+                              hipStream_t stream) {
+  const bool dq_part = parts & RA_BWD_PART_DQ, dkv_part = parts & RA_BWD_PART_DKV;
   RA_REQUIRE(p, RA_ERR_INVALID, "%s: null params", who);
   RA_REQUIRE(p->q && p->k && p->v && p->g && p->delta && p->denominator && p->max_score, RA_ERR_INVALID,
              "%s: null tensor", who);
@@ -340,17 +341,27 @@ int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring,
   uint64_t shards = 0;                // the K/V shards that the running devices hold in this step
   for (int d = 0; d < ring->n_dev; d++)
     if ((ring->run >> d) & 1ULL) shards |= 1ULL << ((d - ring->idx + ring->n_dev) % ring->n_dev);
-  RA_REQUIRE(p->dq || (ring->run & ~(ring->first & ring->last)) == 0, RA_ERR_INVALID,
+  RA_REQUIRE(!dq_part || p->dq || (ring->run & ~(ring->first & ring->last)) == 0, RA_ERR_INVALID,
              "%s: dq may be null only when every running device both starts and ends its dq here", who);
-  RA_REQUIRE(p->dk || (shards & ~(ring->kv_first & ring->kv_last)) == 0, RA_ERR_INVALID,
+  RA_REQUIRE(!dkv_part || p->dk || (shards & ~(ring->kv_first & ring->kv_last)) == 0, RA_ERR_INVALID,
              "%s: dk / dv may be null only when every shard in use both starts and ends here", who);
-  RA_REQUIRE(p->dq_out || (ring->run & ring->last) == 0, RA_ERR_INVALID, "%s: dq_out is null but a device writes it", who);
-  RA_REQUIRE(p->dk_out || (shards & ring->kv_last) == 0, RA_ERR_INVALID, "%s: dk_out is null but a shard writes it", who);
+  RA_REQUIRE(!dq_part || p->dq_out || (ring->run & ring->last) == 0, RA_ERR_INVALID, "%s: dq_out is null but a device writes it", who);
+  RA_REQUIRE(!dkv_part || p->dk_out || (shards & ring->kv_last) == 0, RA_ERR_INVALID, "%s: dk_out is null but a shard writes it", who);
   ra_attn_bwd_params dev = *p;
   dev.Sq = p->Sq / ring->n_dev; dev.Skv = p->Skv / ring->n_dev;
   RA_REQUIRE(attn_bwd_mfma_supported(&dev), RA_ERR_UNSUPPORTED,
              "%s: MFMA kernels need bf16, head size 64 or 128, chunk sizes that are multiples of 128", who);
-  return attn_bwd_mfma(p, ring, RA_BWD_PART_DQ | RA_BWD_PART_DKV, (hipStream_t)stream);
+  return attn_bwd_mfma(p, ring, parts, stream);
+}
+
+int ra_attn_bwd_ring_step(const ra_attn_bwd_params* p, const ra_ring_step* ring, ra_stream_t stream) {
+  return attn_bwd_ring_step(p, ring, RA_BWD_PART_DQ | RA_BWD_PART_DKV, "attn_bwd_ring_step", (hipStream_t)stream);
+}
+
+int ra_attn_bwd_ring_step_part(const ra_attn_bwd_params* p, const ra_ring_step* ring, int32_t part, ra_stream_t stream) {
+  RA_REQUIRE(part == RA_BWD_PART_DQ || part == RA_BWD_PART_DKV, RA_ERR_INVALID,
+             "attn_bwd_ring_step_part: part must be RA_BWD_PART_DQ or RA_BWD_PART_DKV");
+  return attn_bwd_ring_step(p, ring, part, "attn_bwd_ring_step_part", (hipStream_t)stream);
 }
 
 int ra_decode_auto_splits(int32_t B, int32_t L, int32_t H, int32_t D, int32_t dtype) {

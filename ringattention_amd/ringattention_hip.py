@@ -770,8 +770,7 @@ def _ring_step_launches(cfg, mi, n):
     64 devices, the MFMA kernels, no boolean / dropout mask, no cache_idx.  blockwise_kwargs["ring_launch"] =
     "device" keeps one launch per device."""
     return (1 < n <= 64 and cfg.ring_launch != "device" and cfg.impl != L.RA_IMPL_GENERIC and cfg.pdrop == 0.0
-            and mi.keep is None and mi.keep_packed is None and mi.cache_idx_host is None and mi.cache_idx_dev is None
-            and not cfg.bwd_only)
+            and mi.keep is None and mi.keep_packed is None and mi.cache_idx_host is None and mi.cache_idx_dev is None)
 
 
 def _ring_bits(devs):
@@ -920,7 +919,10 @@ def _bwd_ring_step(q, k, v, g, delta, den, mx, acc, outs, cfg, mi, n, idx, plan,
     shards = [(d - idx) % n for d in devs]
     r.kv_first = _ring_bits(s for s in shards if idx == shard_steps[s][0])
     r.kv_last = _ring_bits(s for s in shards if idx == shard_steps[s][-1])
-    rc = L.load().ra_attn_bwd_ring_step(ctypes.byref(p), ctypes.byref(r), _stream())
+    if cfg.bwd_only:      # measurement hook: one of the two kernels alone
+        rc = L.load().ra_attn_bwd_ring_step_part(ctypes.byref(p), ctypes.byref(r), cfg.bwd_only, _stream())
+    else:
+        rc = L.load().ra_attn_bwd_ring_step(ctypes.byref(p), ctypes.byref(r), _stream())
     if rc == L.RA_ERR_UNSUPPORTED and cfg.impl == L.RA_IMPL_AUTO:
         return False
     L.check(rc, "ra_attn_bwd_ring_step")
