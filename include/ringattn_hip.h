@@ -128,6 +128,10 @@ typedef struct ra_attn_fwd_params {
                                  residuals, :53).  Saves the numerator's round trip through memory and
                                  ra_attn_finalize */
   int64_t out_stride_b, out_stride_s;
+  int32_t logit_dim;          /* the head size whose square root divides the logits (:118, :134); 0 = D.  For callers
+                                 that hand over q, k, v zero-padded along D to a head size the matrix-core kernels
+                                 take (the products are those of the un-padded rows, the scale must stay the
+                                 original's) */
   float* out_f32;             /* nullable, only together with `out`: the same quotient BEFORE it is rounded to `dtype`,
                                  (B,Sq,H,D) fp32 with the element strides of `out`.  It is the `output` the reference
                                  keeps as a residual (:53) and multiplies with the cotangent in its backward pass
@@ -157,6 +161,7 @@ typedef struct ra_attn_bwd_params {
   int64_t dq_out_stride_b, dq_out_stride_s;
   void* dk_out; void* dv_out; /* the same for dk and dv (both or neither), (B,Skv,H,D) */
   int64_t dkv_out_stride_b, dkv_out_stride_s;
+  int32_t logit_dim;          /* as in ra_attn_fwd_params; 0 = D */
 } ra_attn_bwd_params;
 
 enum { RA_GRAD_INIT_DQ = 1, RA_GRAD_INIT_DKV = 2 };
@@ -206,6 +211,14 @@ int ra_attn_carry_init(float* numerator, int64_t num_stride_b, int64_t num_strid
 
 /* _blockwise_attention_fwd, ringattention_jax.py:99-179 (called at :38-46). */
 int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream);
+
+/* Which kernel family ra_attn_fwd_block / ra_attn_bwd_block would run for these params (nothing is launched), or 0
+ * when the call would be refused.  The generic kernels serve every shape but run on the vector ALU, two orders of
+ * magnitude below the matrix-core kernels on long sequences: a caller that lets RA_IMPL_AUTO choose can ask here
+ * what it got (the Python layer warns once when a large problem lands on them). */
+enum { RA_FAMILY_GENERIC = 1, RA_FAMILY_MFMA_BF16 = 2, RA_FAMILY_MFMA_F32 = 3 };
+int ra_attn_fwd_family(const ra_attn_fwd_params* p);
+int ra_attn_bwd_family(const ra_attn_bwd_params* p);
 
 /* output = numerator / denominator, cast (ringattention_jax.py:52-53).  out_dtype RA_F32|RA_BF16. */
 int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_stride_s,

@@ -6,10 +6,11 @@ per backend; here there is one backend, the gfx950 HIP kernels):
     ringattention, ringattention_jax, ringattention_inference, blockwise_feedforward
 
 plus ``ring_axis`` to declare the size of the (virtual) sequence-parallel ring, ``SwiGLU``,
-``decode_attention`` and the two steps either side of the path, ``rope_kv_append`` and ``rmsnorm_residual``.
+``decode_attention``, the two steps either side of the path, ``rope_kv_append`` and ``rmsnorm_residual``, and
+``kernel_family_of_last_call`` (which kernels the automatic choice took).
 """
 from .ringattention_hip import (ring_attention, ring_axis, axis_size, below_or_on_diag, run_prefix_keys,
-                                _blockwise_attention_fwd, _blockwise_attention_bwd)
+                                kernel_family_of_last_call, _blockwise_attention_fwd, _blockwise_attention_bwd)
 from .feedforward import blockwise_feedforward, SwiGLU, gemm_bf16
 from .decode import decode_attention, decode_workspace
 from .inference import ring_attention_inference
@@ -21,4 +22,5 @@ ringattention_inference = ring_attention_inference
 
 __all__ = ["ringattention", "ringattention_jax", "ringattention_inference", "ring_attention",
            "ring_attention_inference", "blockwise_feedforward", "ring_axis",
-           "axis_size", "SwiGLU", "decode_attention", "decode_workspace", "below_or_on_diag", "rope_kv_append", "rmsnorm_residual"]
+           "axis_size", "SwiGLU", "decode_attention", "decode_workspace", "below_or_on_diag", "rope_kv_append", "rmsnorm_residual",
+           "kernel_family_of_last_call"]

@@ -18,6 +18,7 @@ RA_DECODE_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 RA_SEG_TILE = 64
 RA_KEEP_WHERE, RA_KEEP_DROPOUT = 0, 1
 RA_GRAD_INIT_DQ, RA_GRAD_INIT_DKV = 1, 2
+RA_FAMILY_GENERIC, RA_FAMILY_MFMA_BF16, RA_FAMILY_MFMA_F32 = 1, 2, 3
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 
@@ -47,7 +48,7 @@ class RaAttnFwdParams(C.Structure):
         ("numerator", vp), ("num_stride_b", i64), ("num_stride_s", i64),
         ("denominator", vp), ("max_score", vp), ("stat_stride_b", i64), ("stat_stride_h", i64),
         ("mask", RaMask), ("impl", i32), ("carry_is_initial", i32),
-        ("out", vp), ("out_stride_b", i64), ("out_stride_s", i64), ("out_f32", vp),
+        ("out", vp), ("out_stride_b", i64), ("out_stride_s", i64), ("logit_dim", i32), ("out_f32", vp),
     ]
 
 
@@ -61,7 +62,7 @@ class RaAttnBwdParams(C.Structure):
         ("dk", vp), ("dv", vp), ("dkv_stride_b", i64), ("dkv_stride_s", i64),
         ("mask", RaMask), ("impl", i32), ("grads_are_initial", i32),
         ("dq_out", vp), ("dq_out_stride_b", i64), ("dq_out_stride_s", i64),
-        ("dk_out", vp), ("dv_out", vp), ("dkv_out_stride_b", i64), ("dkv_out_stride_s", i64),
+        ("dk_out", vp), ("dv_out", vp), ("dkv_out_stride_b", i64), ("dkv_out_stride_s", i64), ("logit_dim", i32),
     ]
 
 
@@ -121,6 +122,8 @@ SYMBOLS = {
     "ra_dropout_keep_packed": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp]),
     "ra_attn_carry_init": (C.c_int, [vp, i64, i64, vp, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_fwd_block": (C.c_int, [C.POINTER(RaAttnFwdParams), vp]),
+    "ra_attn_fwd_family": (C.c_int, [C.POINTER(RaAttnFwdParams)]),
+    "ra_attn_bwd_family": (C.c_int, [C.POINTER(RaAttnBwdParams)]),
     "ra_attn_finalize": (C.c_int, [vp, i64, i64, vp, i64, i64, vp, i32, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_bwd_delta": (C.c_int, [vp, vp, i32, i32, i64, i64, vp, i64, i64, i32, i32, i32, i32, vp]),
     "ra_attn_bwd_block": (C.c_int, [C.POINTER(RaAttnBwdParams), vp]),

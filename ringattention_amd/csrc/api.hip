@@ -217,6 +217,7 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->numerator || (p->carry_is_initial && p->out), RA_ERR_INVALID,
              "attn_fwd_block: the numerator may be null only when carry_is_initial is set and out is given");
   RA_REQUIRE(!p->out_f32 || p->out, RA_ERR_INVALID, "attn_fwd_block: out_f32 goes with out");
+  RA_REQUIRE(p->logit_dim >= 0, RA_ERR_INVALID, "attn_fwd_block: negative logit_dim");
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "attn_fwd_block: dtype %d", p->dtype);
   RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "attn_fwd_block: empty shape");
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_fwd_block: B and H must be <= 65535");
@@ -228,6 +229,22 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
              "attn_fwd_block: MFMA kernels need bf16 or fp32, head size 64 or 128, chunk sizes that are multiples of 128");
   return attn_fwd_generic(p, s);
+}
+
+int ra_attn_fwd_family(const ra_attn_fwd_params* p) {
+  if (!p || (p->dtype != RA_F32 && p->dtype != RA_BF16)) return 0;
+  if (p->impl == RA_IMPL_GENERIC) return RA_FAMILY_GENERIC;
+  if (attn_fwd_mfma_supported(p)) return RA_FAMILY_MFMA_BF16;
+  if (attn_fwd_f32_supported(p)) return RA_FAMILY_MFMA_F32;
+  return p->impl == RA_IMPL_MFMA ? 0 : RA_FAMILY_GENERIC;
+}
+
+int ra_attn_bwd_family(const ra_attn_bwd_params* p) {
+  if (!p || (p->dtype != RA_F32 && p->dtype != RA_BF16)) return 0;
+  if (p->impl == RA_IMPL_GENERIC) return RA_FAMILY_GENERIC;
+  if (attn_bwd_mfma_supported(p)) return RA_FAMILY_MFMA_BF16;
+  if (attn_bwd_f32_supported(p)) return RA_FAMILY_MFMA_F32;
+  return p->impl == RA_IMPL_MFMA ? 0 : RA_FAMILY_GENERIC;
 }
 
 int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_stride_s, const float* denominator,
@@ -268,6 +285,7 @@ static int attn_bwd_block(const ra_attn_bwd_params* p, int parts, const char* wh
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "%s: dtype %d", who, p->dtype);
   RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "%s: empty shape", who);
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "%s: B and H must be <= 65535", who);
+  RA_REQUIRE(p->logit_dim >= 0, RA_ERR_INVALID, "%s: negative logit_dim", who);
   RA_REQUIRE(p->impl == RA_IMPL_AUTO || p->impl == RA_IMPL_GENERIC || p->impl == RA_IMPL_MFMA, RA_ERR_INVALID,
              "%s: impl %d", who, p->impl);
   if (int rc = check_mask(p->mask, p->Sq, p->Skv, who)) return rc;

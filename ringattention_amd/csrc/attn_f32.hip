@@ -38,6 +38,7 @@ struct F32Args {
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
   int carry_is_initial;
+  int sdim;                                      // head size that scales the logits (the un-padded one)
   float* out; int64_t out_sb, out_ss;           // forward, nullable: out = num / den instead of the numerator
   float* out32;                                  // forward, nullable: the same once more (strides of out)
   int dq_initial, dkv_initial;
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(256) void attn_fwd_f32_kernel(F32Args a) {
     }
     return;
   }
-  const float rscale = 1.f / sqrtf((float)HD);                   // :118
+  const float rscale = 1.f / sqrtf((float)a.sdim);                   // :118
   const int gk0 = (int)mv.global_k(k_base);
   const float* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
   const float* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
@@ -373,7 +374,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_f32_kernel(F32Args a) {
                       nullptr, a.dqo_ss, nullptr, a.dq_initial, tid);
     return;
   }
-  const float rscale = 1.f / sqrtf((float)HD);
+  const float rscale = 1.f / sqrtf((float)a.sdim);
   const int gk0 = (int)mv.global_k(k_base);
   const float* kg = a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
   const float* vg = a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD + (int64_t)k_base * a.kv_ss;
@@ -558,7 +559,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
     return;
   }
   const int ntq = qt_end - qt_first;
-  const float rscale = 1.f / sqrtf((float)HD);
+  const float rscale = 1.f / sqrtf((float)a.sdim);
   const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;        // masked iff gq < qlim
   int seg_k = 0; float bias_k = 0.f;
   f32_key_info<HAS_SEG, HAS_BIAS>(mv, b, h, krow, seg_k, bias_k);
@@ -780,6 +781,7 @@ int attn_fwd_f32(const ra_attn_fwd_params* p, hipStream_t s) {
   a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.carry_is_initial = p->carry_is_initial;
+  a.sdim = p->logit_dim > 0 ? p->logit_dim : p->D;
   a.out = (float*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr, keep = p->mask.keep_bits_k != nullptr;
   const long long nwg = (long long)(p->Sq / XBM) * p->H * p->B;
@@ -799,6 +801,7 @@ int attn_bwd_f32(const ra_attn_bwd_params* p, int parts, hipStream_t s) {   // p
   a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.dq = p->dq; a.dq_sb = p->dq_stride_b; a.dq_ss = p->dq_stride_s;
   a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
+  a.sdim = p->logit_dim > 0 ? p->logit_dim : p->D;
   a.dq_initial = (p->grads_are_initial & RA_GRAD_INIT_DQ) != 0;
   a.dkv_initial = (p->grads_are_initial & RA_GRAD_INIT_DKV) != 0;
   a.dq_out = (float*)p->dq_out; a.dqo_sb = p->dq_out_stride_b; a.dqo_ss = p->dq_out_stride_s;

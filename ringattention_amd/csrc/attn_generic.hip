@@ -21,6 +21,7 @@ struct GenericArgs {
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
   int carry_is_initial;
+  int sdim;                                      // head size that scales the logits (the un-padded one)
   void* out; int64_t out_sb, out_ss;             // forward, nullable: out = num / den instead of the numerator
   float* out32;                                  // forward, nullable: the same quotient un-rounded, strides of out
   int dq_initial, dkv_initial;                   // backward: that accumulator holds zeros by definition
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_fwd_generic_kernel(GenericArgs 
   const T* vbase = (const T*)a.v + (int64_t)b * a.kv_sb + (int64_t)h * D;
   float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)rrow * a.num_ss + (int64_t)h * D;
   const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rrow;
-  const float scale = sqrtf((float)D);                            // :118
+  const float scale = sqrtf((float)a.sdim);                            // :118
 
   float q[D], acc[D];
 #pragma unroll
@@ -227,7 +228,7 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_bwd_dq_generic_kernel(GenericAr
   const T* vbase = (const T*)a.v + (int64_t)b * a.kv_sb + (int64_t)h * D;
   float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)rrow * a.dq_ss + (int64_t)h * D;
   const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rrow;
-  const float scale = sqrtf((float)D);
+  const float scale = sqrtf((float)a.sdim);
 
   float q[D], g[D], dq[D];
 #pragma unroll
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(GEN_ROWS) void attn_bwd_dkv_generic_kernel(GenericA
   const T* qbase = (const T*)a.q + (int64_t)b * a.q_sb + (int64_t)h * D;
   const T* gbase = (const T*)a.g + (int64_t)b * a.q_sb + (int64_t)h * D;
   float* outp = (WANT_DK ? a.dk : a.dv) + (int64_t)b * a.dkv_sb + (int64_t)rk * a.dkv_ss + (int64_t)h * D;
-  const float scale = sqrtf((float)D);
+  const float scale = sqrtf((float)a.sdim);
 
   float k[D], v[WANT_DK ? D : 1], acc[D];
 #pragma unroll
@@ -564,6 +565,7 @@ static GenericArgs make_args_fwd(const ra_attn_fwd_params* p) {
   a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.carry_is_initial = p->carry_is_initial;
+  a.sdim = p->logit_dim > 0 ? p->logit_dim : p->D;
   a.out = p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   return a;
 }
@@ -616,6 +618,7 @@ int attn_bwd_generic(const ra_attn_bwd_params* p, hipStream_t s) {
   a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.dq = p->dq; a.dq_sb = p->dq_stride_b; a.dq_ss = p->dq_stride_s;
   a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
+  a.sdim = p->logit_dim > 0 ? p->logit_dim : p->D;
   a.dq_initial = (p->grads_are_initial & RA_GRAD_INIT_DQ) != 0;
   a.dkv_initial = (p->grads_are_initial & RA_GRAD_INIT_DKV) != 0;
   a.dq_out = p->dq_out; a.dqo_sb = p->dq_out_stride_b; a.dqo_ss = p->dq_out_stride_s;

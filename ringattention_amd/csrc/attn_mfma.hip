@@ -42,6 +42,7 @@ struct FwdArgs {
   int64_t st_sb, st_sh;
   MaskView mv;
   int carry_is_initial;
+  int sdim;                                   // head size that scales the logits (the un-padded one)
   uint16_t* out; int64_t out_sb, out_ss;      // nullable: last step of the device, out = num / den instead of num
   float* out32;                               // nullable, with out: the quotient before rounding, strides of out
   RingView ring;                              // n == 0: one device per launch
@@ -108,6 +109,7 @@ struct BwdArgs {
   float* dk; float* dv; int64_t dkv_sb, dkv_ss;
   MaskView mv;
   int dq_initial, dkv_initial;                 // the fp32 accumulator holds zeros by definition: not read
+  int sdim;                                    // head size that scales the logits (the un-padded one)
   uint16_t* dq_out; int64_t dqo_sb, dqo_ss;    // nullable: last call that adds into it, the sum goes here as bf16
   uint16_t* dk_out; uint16_t* dv_out; int64_t dkvo_sb, dkvo_ss;
   RingView ring;                               // n == 0: one device per launch
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   const int ntq = qt_end - qt_first;       // query tiles of 64 rows
   const int nblk = 2 * ntq;                // blocks of 32 rows
 
-  const float c = kLog2e / sqrtf((float)HD);
+  const float c = kLog2e / sqrtf((float)a.sdim);
   const float kMask2 = mv.mask_min;
 
   // ---- staging of the Q / dO tiles through registers: producers bring Q, consumers dO and the statistics
@@ -664,7 +666,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     }
 
     // dk += acc / sqrt(D) (:231), dv += acc (:232); this pair owns its 32 key rows
-    const float rscale = 1.f / sqrtf((float)HD);
+    const float rscale = 1.f / sqrtf((float)a.sdim);
     const int64_t ooff = (int64_t)b * a.dkv_sb + (int64_t)krow * a.dkv_ss + (int64_t)h * HD + hi * 4;
     const int64_t oout = (int64_t)b * a.dkvo_sb + (int64_t)krow * a.dkvo_ss + (int64_t)h * HD + hi * 4;
     // dk, then dv; all the old values of one are requested before its first store (a load issued after a store is
@@ -782,7 +784,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     return;
   }
   const int gk0 = gk0_shard + k_base;
-  const float c = kLog2e / sqrtf((float)HD);
+  const float c = kLog2e / sqrtf((float)a.sdim);
   const float bias_scale = kLog2e / c;
   const float kMask2 = mv.mask_min;
 
@@ -1137,7 +1139,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #undef RA_WS_CONSUME
 
     // dq += acc / sqrt(D)   (:230)
-    const float rscale = 1.f / sqrtf((float)HD);
+    const float rscale = 1.f / sqrtf((float)a.sdim);
     float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)qrow * a.dq_ss + (int64_t)h * HD + hi * 4;
     uint16_t* dqo = a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)qrow * a.dqo_ss + (int64_t)h * HD + hi * 4;
     // all the old values are requested before the first store: a load issued after a store is not waited for until
@@ -1247,7 +1249,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     return;
   }
   const int gk0 = gk0_shard + k_base;
-  const float c = kLog2e / sqrtf((float)HD);
+  const float c = kLog2e / sqrtf((float)a.sdim);
   const float bias_scale = kLog2e / c;
   const float kMask2 = mv.mask_min;
 
@@ -1718,6 +1720,7 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* r, hipStream_
   a.den = p->denominator; a.mx = p->max_score; a.st_sb = p->stat_stride_b; a.st_sh = p->stat_stride_h;
   a.mv = MaskView::make(p->mask, p->mask.q_chunk_idx_start);
   a.carry_is_initial = p->carry_is_initial;
+  a.sdim = p->logit_dim > 0 ? p->logit_dim : p->D;
   a.out = (uint16_t*)p->out; a.out_sb = p->out_stride_b; a.out_ss = p->out_stride_s; a.out32 = p->out_f32;
   const bool seg = p->mask.segment_ids != nullptr, bias = p->mask.bias != nullptr;
   const bool keep = p->mask.keep_bits_k != nullptr;      // packed form checked by attn_fwd_mfma_supported
@@ -1768,6 +1771,7 @@ int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* r, int parts,
   a.dk = p->dk; a.dv = p->dv; a.dkv_sb = p->dkv_stride_b; a.dkv_ss = p->dkv_stride_s;
   a.dq_initial = (p->grads_are_initial & RA_GRAD_INIT_DQ) != 0;
   a.dkv_initial = (p->grads_are_initial & RA_GRAD_INIT_DKV) != 0;
+  a.sdim = p->logit_dim > 0 ? p->logit_dim : p->D;
   a.dq_out = (uint16_t*)p->dq_out; a.dqo_sb = p->dq_out_stride_b; a.dqo_ss = p->dq_out_stride_s;
   a.dk_out = (uint16_t*)p->dk_out; a.dv_out = (uint16_t*)p->dv_out;
   a.dkvo_sb = p->dkv_out_stride_b; a.dkvo_ss = p->dkv_out_stride_s;

@@ -18,6 +18,7 @@ import collections
 import contextlib
 import ctypes
 import math
+import warnings
 import weakref
 
 import torch
@@ -149,6 +150,7 @@ class _Config:
         # False: never reuse the int32 copy / tile ranges of a segment_ids tensor seen before (for callers that edit
         # the ids through a numpy alias or .data, which the tensor's version counter does not see)
         self.cache_segment_ids = bool(kw.get("cache_segment_ids", True))
+        self.logit_dim = 0            # set when q, k, v were zero-padded along D: the head size that scales the logits
         self.ring_launch = kw.get("ring_launch", "step")
         if self.ring_launch not in ("step", "device"):
             raise ValueError("ring_launch must be 'step' or 'device'")
@@ -425,6 +427,47 @@ def _rows(t):
     return t.stride(0), t.stride(1)
 
 
+# --------------------------------------------------------------------------- which kernels ran
+_FAMILY_NAMES = {L.RA_FAMILY_GENERIC: "generic", L.RA_FAMILY_MFMA_BF16: "mfma_bf16", L.RA_FAMILY_MFMA_F32: "mfma_f32"}
+_LAST_FAMILY = {"forward": None, "backward": None}
+_WARNED = set()
+_GENERIC_WARN_PAIRS = 1 << 28         # B * H * q_len * kv_len from which the vector-ALU kernels take seconds
+
+
+def kernel_family_of_last_call():
+    """{"forward": ..., "backward": ...}: the kernel family ("mfma_bf16", "mfma_f32", "generic") that the last
+    attention launch of each direction ran on - what blockwise_kwargs["impl"] = "auto" (the default) chose."""
+    return dict(_LAST_FAMILY)
+
+
+def _note_family(direction, fam, cfg, q, k, mi):
+    _LAST_FAMILY[direction] = _FAMILY_NAMES.get(fam)
+    if fam != L.RA_FAMILY_GENERIC or cfg.impl != L.RA_IMPL_AUTO:
+        return
+    B, Sq, H, D = q.shape
+    if B * H * Sq * k.shape[1] < _GENERIC_WARN_PAIRS:
+        return
+    why = []
+    if q.dtype not in (torch.bfloat16, torch.float32):
+        why.append("dtype %s" % q.dtype)
+    if D not in (64, 128):
+        why.append("head size %d (64 and 128 are taken as they are, smaller ones zero-padded)" % D)
+    if cfg.qc % 128 or cfg.kc % 128:
+        why.append("chunk sizes (%d, %d) that are no multiples of 128 and cannot be re-chunked (odd sizes under a "
+                   "causal mask, a ragged shard, dropout)" % (cfg.qc, cfg.kc))
+    if mi.bias is not None and mi.bias_strides[2] != 0:
+        why.append("a bias with one row per query")
+    if mi.keep is not None and mi.keep_packed is None:
+        why.append("a boolean mask whose lengths are no multiples of 64")
+    key = (direction, tuple(why))
+    if key in _WARNED:
+        return
+    _WARNED.add(key)
+    warnings.warn("ringattention_amd: this %s call runs on the generic vector-ALU kernels, about a hundred times "
+                  "slower than the matrix-core kernels at this size, because of %s"
+                  % (direction, "; ".join(why) or "its strides or alignment"), RuntimeWarning, stacklevel=4)
+
+
 # --------------------------------------------------------------------------- one ring step
 def _device_chunk_starts(q_chunk_idx_start, k_chunk_idx_start, device):
     """The chunk starts as the kernels take them from device memory (ra_mask.chunk_starts), or None when both are
@@ -505,7 +548,9 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
         skip = False        # a row may lose every allowed key: its masked tiles then carry its (uniform) weights
     p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip, starts_dev)
     p.impl = cfg.impl
+    p.logit_dim = cfg.logit_dim
     p.carry_is_initial = 1 if _carry_is_initial else 0
+    _note_family("forward", L.load().ra_attn_fwd_family(ctypes.byref(p)), cfg, q, k, mi)
     L.check(L.load().ra_attn_fwd_block(ctypes.byref(p), _stream()), "ra_attn_fwd_block")
     return num, den, mx
 
@@ -585,6 +630,8 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
         skip = False
     p.mask = mi.fill(cfg, q_chunk_idx_start, k_chunk_idx_start, skip, starts_dev)
     p.impl = cfg.impl
+    p.logit_dim = cfg.logit_dim
+    _note_family("backward", L.load().ra_attn_bwd_family(ctypes.byref(p)), cfg, q, k, mi)
     if cfg.bwd_only:
         L.check(L.load().ra_attn_bwd_block_part(ctypes.byref(p), cfg.bwd_only, _stream()), "ra_attn_bwd_block_part")
     else:
@@ -675,6 +722,14 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
             raise NotImplementedError("attention dropout together with cache_idx is not supported")
         cfg.skip_masked_tiles = False      # dropout can leave a row without any allowed key
     _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total)
+    d_true = D
+    pad_to = _mfma_head_size(cfg, mi, q)
+    if pad_to:
+        # a head size the matrix-core kernels do not tile: q, k, v zero-padded along D (the products are those of the
+        # un-padded rows), the logits still divided by sqrt of the original head size (:118)
+        q, k, v = (torch.nn.functional.pad(t, (0, pad_to - D)) for t in (q, k, v))
+        cfg.logit_dim = D
+        D = pad_to
     den = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)         # :23
     mx = torch.empty((B, H, q_total), dtype=torch.float32, device=q.device)          # :49
     out = torch.empty((B, q_total, H, D), dtype=v.dtype, device=q.device)
@@ -715,7 +770,25 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
             if out32 is not None:
                 _finalize(carry[0], carry[1], out32[:, qs])
     del num
-    return out, (out if out32 is None else out32, q, k, v, mi, cfg, n, den, mx)
+    res = (out if out32 is None else out32, q, k, v, mi, cfg, n, den, mx)
+    if D != d_true:
+        out = out[..., :d_true].contiguous()
+    return out, res
+
+
+def _mfma_head_size(cfg, mi, q):
+    """The head size (64 or 128) to zero-pad q, k, v to so that the matrix-core kernels take a call whose own head
+    size they do not tile, or 0: when the head size is 64 or 128 already or above 128, when the generic kernels were
+    asked for, or when something else keeps the call on them anyway (chunk sizes off the 128-grid, a per-row bias, an
+    unpacked boolean mask), where padding would only add work."""
+    D = q.shape[3]
+    if D in (64, 128) or D > 128 or cfg.impl == L.RA_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float32):
+        return 0
+    if cfg.qc % 128 or cfg.kc % 128 or (mi.bias is not None and mi.bias_strides[2] != 0):
+        return 0
+    if mi.keep is not None and mi.keep_packed is None:
+        return 0
+    return 64 if D < 64 else 128
 
 
 def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=128):
@@ -728,7 +801,7 @@ def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=
     long as its row has an unmasked key, which is what skip_masked_tiles already asks for; so both chunkings sum
     over the same pairs.  Without a causal block size every chunk pair runs.  The slices are not clamped when the
     segment ids cover every position, there is no dropout here, and a per-row bias takes the generic kernels."""
-    if cfg.impl == L.RA_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float32) or q.shape[3] not in (64, 128):
+    if cfg.impl == L.RA_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float32) or q.shape[3] > 128:
         return
     if cfg.qc % grid == 0 and cfg.kc % grid == 0:
         return
@@ -806,6 +879,7 @@ def _fwd_ring_step(q, k, v, carry, out, out32, cfg, mi, n, idx, plan, devs):
     p.stat_stride_b, p.stat_stride_h = den.stride(0), den.stride(1)
     p.mask = mi.fill(cfg, 0, 0, cfg.skip_masked_tiles)
     p.impl = cfg.impl
+    p.logit_dim = cfg.logit_dim
     r = L.RaRingStep()
     r.n_dev, r.idx = n, idx
     r.run = _ring_bits(devs)
@@ -815,6 +889,7 @@ def _fwd_ring_step(q, k, v, carry, out, out32, cfg, mi, n, idx, plan, devs):
     if rc == L.RA_ERR_UNSUPPORTED and cfg.impl == L.RA_IMPL_AUTO:
         return False
     L.check(rc, "ra_attn_fwd_ring_step")
+    _LAST_FAMILY["forward"] = "mfma_bf16"
     return True
 
 
@@ -825,6 +900,9 @@ def _ring_attention_bwd(res, g):
     B, q_total, H, D = q.shape
     kv_total = k.shape[1]
     q_len, kv_len = q_total // n, kv_total // n
+    d_true = g.shape[3]
+    if d_true != D:             # q, k, v were zero-padded along D in the forward pass: the cotangent follows
+        g = torch.nn.functional.pad(g, (0, D - d_true))
     g = g.to(q.dtype).contiguous()
     delta = _bwd_delta(g, out)
     plan = _ring_plan(cfg, mi, n, q_len, kv_len)
@@ -873,6 +951,8 @@ def _ring_attention_bwd(res, g):
             ks = slice(s * kv_len, (s + 1) * kv_len)
             dk_out[:, ks].zero_()
             dv_out[:, ks].zero_()
+    if d_true != D:
+        dq_out, dk_out, dv_out = (t[..., :d_true].contiguous() for t in (dq_out, dk_out, dv_out))
     return dq_out, dk_out, dv_out
 
 
@@ -911,6 +991,7 @@ def _bwd_ring_step(q, k, v, g, delta, den, mx, acc, outs, cfg, mi, n, idx, plan,
     p.dkv_out_stride_b, p.dkv_out_stride_s = _rows(dk_out)
     p.mask = mi.fill(cfg, 0, 0, cfg.skip_masked_tiles)
     p.impl = cfg.impl
+    p.logit_dim = cfg.logit_dim
     r = L.RaRingStep()
     r.n_dev, r.idx = n, idx
     r.run = _ring_bits(devs)
@@ -926,6 +1007,7 @@ def _bwd_ring_step(q, k, v, g, delta, den, mx, acc, outs, cfg, mi, n, idx, plan,
     if rc == L.RA_ERR_UNSUPPORTED and cfg.impl == L.RA_IMPL_AUTO:
         return False
     L.check(rc, "ra_attn_bwd_ring_step")
+    _LAST_FAMILY["backward"] = "mfma_bf16"
     return True
 
 

@@ -588,14 +588,74 @@ def test_fp32_mfma_kernels_agree_with_the_vector_kernels(D, n, cbs, use_seg, use
 
 
 def test_fp32_mfma_kernels_refuse_what_they_do_not_take():
-    """A per-row bias and head sizes other than 64 / 128 stay with the vector kernels; asking for the matrix-core
-    kernels by name then is an error, not a silent fallback."""
-    q, k, v, _ = make_qkv(1, 256, 1, 32, dtype=torch.float32, seed=1)
+    """A per-row bias and head sizes above 128 stay with the vector kernels (which stop at 128 themselves); asking for
+    the matrix-core kernels by name then is an error, not a silent fallback.  Head sizes below 128 are zero-padded."""
+    q, k, v, _ = make_qkv(1, 256, 1, 256, dtype=torch.float32, seed=1)
     with pytest.raises(NotImplementedError):
         run_hip(q, k, v, None, None, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32, impl="mfma"))
+    q, k, v, _ = make_qkv(1, 256, 1, 32, dtype=torch.float32, seed=1)
+    out, _ = run_hip(q, k, v, None, None, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32, impl="mfma"))
+    assert out.shape == q.shape and ra.kernel_family_of_last_call()["forward"] == "mfma_f32"
     q, k, v, _ = make_qkv(1, 256, 1, 64, dtype=torch.float32, seed=1)
     bias = torch.zeros(1, 1, 128, 256)
     with pytest.raises(NotImplementedError):
         run_hip(q, k, v, None, bias, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32, impl="mfma"))
     out, _ = run_hip(q, k, v, None, bias, None, None, 1, kwargs(128, 128, 1, dtype=torch.float32))   # auto: served
     assert torch.isfinite(out).all()
+
+
+# --- head sizes the matrix-core kernels do not tile: q, k, v zero-padded to 64 / 128, logits scaled by the original
+# head size (ra_attn_*_params.logit_dim); the generic kernels remain the cross-check
+@pytest.mark.parametrize("D,dtype,n,use_seg", [(32, torch.bfloat16, 1, False), (32, torch.bfloat16, 2, True),
+                                               (96, torch.bfloat16, 2, True), (40, torch.bfloat16, 1, False),
+                                               (32, torch.float32, 2, True), (80, torch.float32, 1, False)])
+def test_other_head_sizes_run_on_the_mfma_kernels(D, dtype, n, use_seg):
+    B, S, H = 1, 512 * n, 2
+    print("head size case", D, dtype, n, use_seg, flush=True)
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=D, scale=D ** -0.25)
+    bias = torch.randn(B, 1, 1, S, generator=torch.Generator().manual_seed(1)) if use_seg else None
+    seg = packed_segment_ids(B, S, S // 3, seed=2) if use_seg else None
+    kw = kwargs(128, 128, 1, dtype=torch.float32)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    fam = ra.kernel_family_of_last_call()
+    want = "mfma_bf16" if dtype == torch.bfloat16 else "mfma_f32"
+    assert fam == {"forward": want, "backward": want}, fam
+    assert out.shape == q.shape and out.is_contiguous()
+    assert_close(out, ref_out, dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert a.shape == q.shape
+        assert_close(a, b, dtype, name)
+    if D == 32:         # the vector kernels take this head size as it is: same result within the parity bar
+        g_out, g_grads = run_hip(q, k, v, do, bias, seg, None, n, dict(kw, impl="generic"))
+        assert ra.kernel_family_of_last_call() == {"forward": "generic", "backward": "generic"}
+        assert_close(out, g_out, dtype, "mfma vs generic out")
+        for name, a, b in zip(("dq", "dk", "dv"), grads, g_grads):
+            assert_close(a, b, dtype, "mfma vs generic " + name)
+
+
+def test_a_large_call_on_the_generic_kernels_warns_once():
+    """RA_IMPL_AUTO falls back to the vector-ALU kernels silently for small problems; from 2^28 (query, key) pairs
+    on it says so, once per cause, and kernel_family_of_last_call tells which family ran."""
+    import warnings
+    B, S, H, D, qc = 1, 8192, 4, 64, 128
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=1, scale=D ** -0.25)
+    bias = torch.randn(1, 1, qc, S, generator=torch.Generator().manual_seed(2))       # one bias row per query of a chunk
+    kw = kwargs(qc, qc, 1)
+    qd, kd, vd, bd = (t.to(DEV) for t in (q, k, v, bias))
+    with torch.no_grad(), warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        ra.ringattention(qd, kd, vd, bd, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+        ra.ringattention(qd, kd, vd, bd, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+        torch.cuda.synchronize()
+    assert ra.kernel_family_of_last_call()["forward"] == "generic"
+    mine = [w for w in seen if issubclass(w.category, RuntimeWarning) and "generic vector-ALU kernels" in str(w.message)]
+    assert len(mine) <= 1
+    from ringattention_amd import ringattention_hip as R
+    assert any(key[0] == "forward" and any("bias with one row per query" in t for t in key[1]) for key in R._WARNED)
+    # a small call of the same kind stays silent
+    with torch.no_grad(), warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        ra.ringattention(qd[:, :256], kd[:, :256], vd[:, :256], bd[..., :256], None, None, axis_name=None,
+                         float32_logits=True, blockwise_kwargs=kw)
+    assert not [w for w in seen if "generic vector-ALU kernels" in str(w.message)]

@@ -179,8 +179,18 @@ def test_fit_chunks_to_mfma_grid_decisions(qc, kc, cbs, skip, expect):
             assert cfg.kc == 128
     cfg = rh._Config(dict(query_chunk_size=qc, key_chunk_size=kc, causal_block_size=cbs))
     cfg.skip_masked_tiles = skip
-    rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 32, dtype=torch.bfloat16), 768, 768, 768, 768)
-    assert (cfg.qc, cfg.kc) == (qc, kc)                      # head size 32: the vector kernels, chunk sizes untouched
+    rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 256, dtype=torch.bfloat16), 768, 768, 768, 768)
+    assert (cfg.qc, cfg.kc) == (qc, kc)                      # head size 256: the vector kernels, chunk sizes untouched
+    # head sizes below 128 are zero-padded to 64 / 128 for the matrix-core kernels, so they re-chunk like those
+    cfg = rh._Config(dict(query_chunk_size=qc, key_chunk_size=kc, causal_block_size=cbs))
+    cfg.skip_masked_tiles = skip
+    q32 = torch.zeros(1, 1, 1, 32, dtype=torch.bfloat16)
+    rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), q32, 768, 768, 768, 768)
+    assert cfg.qc == expect
+    assert rh._mfma_head_size(cfg, _FakeMaskInputs(), q32) == (64 if cfg.qc % 128 == 0 and cfg.kc % 128 == 0 else 0)
+    assert rh._mfma_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 96, dtype=torch.float32)) == (
+        128 if cfg.qc % 128 == 0 and cfg.kc % 128 == 0 else 0)
+    assert rh._mfma_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16)) == 0
 
 
 def test_output_residual_option():
