@@ -822,7 +822,7 @@ def bench_mfma_probe(args):
     flop = wgs * 4 * iters * 64 * 32768.0
     rows = {}
     for mode, name in ((0, "one value everywhere"), (1, "a value per lane, constant in time"), (2, "random operands")):
-        fn = lambda: L.check(L.load().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, mode, stream), "ra_mfma_rate_probe")
+        fn = lambda: L.check(L.load_probe().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, mode, stream), "ra_mfma_rate_probe")
         fn()
         torch.cuda.synchronize()
         clk = _sclk_under_load(fn, seconds=2.5)
@@ -939,7 +939,12 @@ def main():
         if extra in r:
             line[extra] = r[extra]
     line.update(extras)
-    print(json.dumps(line))
+    # give the device memory back before the line goes out: whoever reads the line may look at the GPU right away
+    import gc
+    gc.collect()
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    print(json.dumps(line), flush=True)
 
 
 if __name__ == "__main__":

@@ -146,8 +146,29 @@ SYMBOLS = {
     "ra_attn_bwd_block_part": (C.c_int, [C.POINTER(RaAttnBwdParams), i32, vp]),
     "ra_attn_bwd_ring_step_part": (C.c_int, [C.POINTER(RaAttnBwdParams), C.POINTER(RaRingStep), i32, vp]),
     "ra_gemm_bf16_tile": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp]),
+}
+# libringattn_probe.so: the MFMA rate probe of the benchmark, kept out of the product library
+PROBE_LIB_PATH = os.path.join(_HERE, "libringattn_probe.so")
+PROBE_SYMBOLS = {
     "ra_mfma_rate_probe": (C.c_int, [vp, i32, i32, i32, vp]),
 }
+_probe = None
+
+
+def load_probe():
+    """The measurement library (ringattn_hip_measure.h: ra_mfma_rate_probe); raises if it has not been built."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise RuntimeError("ringattention_amd: %s is missing. Build it with `python -m ringattention_amd.build`."
+                               % PROBE_LIB_PATH)
+        lib = C.CDLL(PROBE_LIB_PATH)
+        for name, (res, args) in PROBE_SYMBOLS.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _probe = lib
+    return _probe
 
 _lib = None
 

@@ -11,6 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libringattn_hip.so")
+PROBE_LIB = os.path.join(HERE, "libringattn_probe.so")      # measurement only (csrc/measure): not the product library
 OBJ_DIR = os.path.join(CSRC, "obj")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -44,6 +45,12 @@ def build(force=True, jobs=4):
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    probe = sorted(glob.glob(os.path.join(CSRC, "measure", "*.hip")))
+    pobjs = [_compile(s, force) for s in probe]
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBE_LIB] + pobjs,
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link of the probe library failed:\n" + r.stderr)
     return LIB
 
 

@@ -22,7 +22,6 @@ int attn_fwd_mfma(const ra_attn_fwd_params* p, const ra_ring_step* ring, hipStre
 int attn_bwd_mfma(const ra_attn_bwd_params* p, const ra_ring_step* ring, int parts, hipStream_t s);   // parts: RA_BWD_PART_* bits
 bool attn_fwd_mfma_supported(const ra_attn_fwd_params* p);
 bool attn_bwd_mfma_supported(const ra_attn_bwd_params* p);
-int mfma_probe(float* sink, int workgroups, int iters, int operands, hipStream_t s);
 int attn_fwd_f32(const ra_attn_fwd_params* p, hipStream_t s);                  // fp32 inputs on the matrix cores
 int attn_bwd_f32(const ra_attn_bwd_params* p, int parts, hipStream_t s);
 bool attn_fwd_f32_supported(const ra_attn_fwd_params* p);
@@ -470,14 +469,6 @@ int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t
   RA_REQUIRE(c_dtype == RA_F32 || c_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "gemm_bf16_tile: c_dtype %d", c_dtype);
   RA_REQUIRE(tile >= -1 && tile <= 3, RA_ERR_INVALID, "gemm_bf16_tile: tile %d outside [-1, 3]", tile);
   return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, tile, (hipStream_t)stream);
-}
-
-int ra_mfma_rate_probe(float* sink, int32_t workgroups, int32_t iters, int32_t operands, ra_stream_t stream) {
-  RA_REQUIRE(sink, RA_ERR_INVALID, "mfma_rate_probe: null sink");
-  RA_REQUIRE(workgroups > 0 && workgroups <= 65536 && iters > 0 && iters <= (1 << 22), RA_ERR_INVALID,
-             "mfma_rate_probe: %d workgroups, %d iterations", workgroups, iters);
-  RA_REQUIRE(operands >= 0 && operands <= 2, RA_ERR_INVALID, "mfma_rate_probe: operands %d outside [0, 2]", operands);
-  return mfma_probe(sink, workgroups, iters, operands, (hipStream_t)stream);
 }
 
 }  // extern "C"

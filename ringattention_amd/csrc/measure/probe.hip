@@ -1,8 +1,11 @@
 // Measurement probe: what the matrix pipes of this GPU sustain on nothing but bf16 MFMAs, as a function of how much
 // the operands change from one instruction to the next.  Under a power or current limit the clock, and with it the
 // rate, depends on that activity; the attention and GEMM kernels are judged against the rate measured here next to
-// the published peak.  Not part of the drop-in boundary (ringattn_hip_measure.h).
-#include "common.hpp"
+// the published peak.  Not part of the drop-in boundary and not part of libringattn_hip.so: it is built into
+// libringattn_probe.so, which only the benchmark and its test load (declared in ringattn_hip_measure.h).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../../include/ringattn_hip_measure.h"
 
 namespace ra {
 
@@ -48,12 +51,14 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(float* sink, int iters)
   sink[blockIdx.x * 256 + threadIdx.x] = t;
 }
 
-int mfma_probe(float* sink, int workgroups, int iters, int operands, hipStream_t s) {
-  if (operands == 0) mfma_probe_kernel<0><<<workgroups, 256, 0, s>>>(sink, iters);
-  else if (operands == 1) mfma_probe_kernel<1><<<workgroups, 256, 0, s>>>(sink, iters);
-  else mfma_probe_kernel<2><<<workgroups, 256, 0, s>>>(sink, iters);
-  RA_CHECK_LAUNCH("mfma_probe");
-  return RA_OK;
-}
-
 }  // namespace ra
+
+extern "C" int ra_mfma_rate_probe(float* sink, int32_t workgroups, int32_t iters, int32_t operands, ra_stream_t stream) {
+  if (!sink || workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 22) || operands < 0 || operands > 2)
+    return RA_ERR_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  if (operands == 0) ra::mfma_probe_kernel<0><<<workgroups, 256, 0, s>>>(sink, iters);
+  else if (operands == 1) ra::mfma_probe_kernel<1><<<workgroups, 256, 0, s>>>(sink, iters);
+  else ra::mfma_probe_kernel<2><<<workgroups, 256, 0, s>>>(sink, iters);
+  return hipGetLastError() == hipSuccess ? RA_OK : RA_ERR_LAUNCH;
+}

@@ -161,12 +161,12 @@ def test_mfma_rate_probe_computes_what_it_says():
     from ringattention_amd import _lib as L
     iters, wgs = 4, 8
     sink = torch.zeros(wgs * 256, dtype=torch.float32, device=DEV)
-    L.check(L.load().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, 0, torch.cuda.current_stream().cuda_stream),
+    L.check(L.load_probe().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, 0, torch.cuda.current_stream().cuda_stream),
             "ra_mfma_rate_probe")
     torch.cuda.synchronize()
     assert bool((sink == 2.0 * 16 * iters * 64).all())
     for mode in (1, 2):
-        L.check(L.load().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, mode, torch.cuda.current_stream().cuda_stream),
+        L.check(L.load_probe().ra_mfma_rate_probe(sink.data_ptr(), wgs, iters, mode, torch.cuda.current_stream().cuda_stream),
                 "ra_mfma_rate_probe")
         torch.cuda.synchronize()
         assert bool(torch.isfinite(sink).all()) and float(sink.abs().max()) > 0

@@ -20,10 +20,12 @@ def test_library_exports_every_declared_symbol():
         header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
         declared |= set(re.findall(r"\b(ra_[a-z0-9_]+)\s*\(", header))
     assert declared, "no declarations parsed"
-    assert declared == set(_lib.SYMBOLS), declared ^ set(_lib.SYMBOLS)
-    lib = _lib.load()
+    assert declared == set(_lib.SYMBOLS) | set(_lib.PROBE_SYMBOLS), declared ^ (set(_lib.SYMBOLS) | set(_lib.PROBE_SYMBOLS))
+    lib, probe = _lib.load(), _lib.load_probe()
     for name in declared:
-        assert getattr(lib, name) is not None
+        assert getattr(probe if name in _lib.PROBE_SYMBOLS else lib, name) is not None
+    with pytest.raises(AttributeError):           # the probe is measurement code: not in the product library
+        lib.ra_mfma_rate_probe
     macro = int(re.search(r"#define\s+RA_ABI_VERSION\s+(\d+)", open(os.path.join(ROOT, "include", "ringattn_hip.h")).read()).group(1))
     assert lib.ra_version() == macro == _lib.RA_ABI_VERSION
 
@@ -113,8 +115,8 @@ def test_invalid_arguments_return_codes_without_gpu():
     # measurement hooks validate too
     assert lib.ra_attn_bwd_block_part(None, 3, None) == _lib.RA_ERR_INVALID
     assert lib.ra_gemm_bf16_tile(one_ := ctypes.c_void_p(16), one_, one_, 128, 128, 64, 0, 0, 1, 0, 7, None) == _lib.RA_ERR_INVALID
-    assert lib.ra_mfma_rate_probe(None, 1, 1, 0, None) == _lib.RA_ERR_INVALID
-    assert lib.ra_mfma_rate_probe(ctypes.c_void_p(16), 1, 1, 3, None) == _lib.RA_ERR_INVALID
+    assert _lib.load_probe().ra_mfma_rate_probe(None, 1, 1, 0, None) == _lib.RA_ERR_INVALID
+    assert _lib.load_probe().ra_mfma_rate_probe(ctypes.c_void_p(16), 1, 1, 3, None) == _lib.RA_ERR_INVALID
     # ra_keep_pack validates before touching the device
     assert lib.ra_keep_pack(None, 0, 0, 0, 1, 1, 1, 64, 64, None, None, None, None) == _lib.RA_ERR_INVALID
     one = ctypes.c_void_p(16)      # any non-null address: the shape check comes before any use
