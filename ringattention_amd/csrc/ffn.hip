@@ -26,6 +26,10 @@ struct GemmArgs {
   void* C;
   int M, N, K;
   int c_f32, beta_one;
+  // two products that share A in one launch, C = A B and C_alt = A B_alt (both (M, N)): the grid covers the tile
+  // columns of both, so that the two together fill the CUs in fewer rounds than one after the other (4-wavefront
+  // tile kernels only; null: one product)
+  const uint16_t* B_alt; void* C_alt;
 };
 
 __device__ __forceinline__ s16x4 lds_tr(const uint16_t* p) {
@@ -301,7 +305,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
-  if (!tile_of_block(g.M / BM, g.N / BN, tm, tn)) return;
+  const int ntn1 = g.N / BN;
+  if (!tile_of_block(g.M / BM, g.B_alt ? 2 * ntn1 : ntn1, tm, tn)) return;
+  if (tn >= ntn1) { tn -= ntn1; g.B = g.B_alt; g.C = g.C_alt; }       // a tile of the second product
   const int m0 = tm * BM, n0 = tn * BN;
 
   f32x16 acc[4][NJ];
@@ -477,7 +483,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_w4_kernel(GemmArgs g) {
 }
 template <bool TA, bool TB, int BN>
 static int launch_w4(const GemmArgs& g, hipStream_t s) {
-  const long long nwg = ((long long)(g.M / 256) * (g.N / BN) + 7) / 8 * 8;
+  const long long nwg = ((long long)(g.M / 256) * (g.N / BN) * (g.B_alt ? 2 : 1) + 7) / 8 * 8;
   gemm_bf16_w4_kernel<TA, TB, BN><<<dim3((unsigned)nwg), 256, 0, s>>>(g);
   RA_CHECK_LAUNCH("gemm_bf16_w4");
   return RA_OK;
@@ -549,6 +555,22 @@ int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta
   return gemm_dispatch(g, ta, tb, tile, s);
 }
 
+// C1 = A B1 and C2 = A B2 (both (M, N), row-major, bf16 out), in one launch where the 4-wavefront tile kernels take
+// the shape, else one after the other.  Same bits either way: a tile is computed the same whichever launch holds it.
+static int gemm_bf16_pair(const void* A, const void* B1, const void* B2, void* C1, void* C2, int M, int N, int K,
+                          int tile, hipStream_t s) {
+  if (M % 256 == 0 && N % 128 == 0 && K % GBK == 0 && w4_reach_ok(M, N, K)) {
+    int t = tile >= 0 ? tile : pick_tile(M, 2 * N, K);
+    if (t == 0 && N % 256) t = 3;
+    if (t == 0 || t == 3) {
+      GemmArgs g{(const uint16_t*)A, (const uint16_t*)B1, nullptr, nullptr, C1, M, N, K, 0, 0, (const uint16_t*)B2, C2};
+      return t == 0 ? launch_w4<false, false, 256>(g, s) : launch_w4<false, false, 128>(g, s);
+    }
+  }
+  if (int rc = gemm_bf16(A, B1, C1, M, N, K, 0, 0, RA_BF16, 0, tile, s)) return rc;
+  return gemm_bf16(A, B2, C2, M, N, K, 0, 0, RA_BF16, 0, tile, s);
+}
+
 // ------------------------------------------------------------------ SwiGLU elementwise parts
 __device__ __forceinline__ float silu(float x) { return x / (1.f + __expf(-x)); }
 
@@ -595,8 +617,7 @@ static int check_ffn_shape(const ra_swiglu_params* p, const char* who) {
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s) {
   if (int rc = check_ffn_shape(p, "swiglu_fwd")) return rc;
   const int T = p->T, d = p->d, f = p->f, tile = p->gemm_tile - 1;
-  if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;     // a = x w1
-  if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;     // b = x w3
+  if (int rc = gemm_bf16_pair(p->x, p->w1, p->w3, p->a, p->b, T, f, d, tile, s)) return rc;     // a = x w1, b = x w3
   const int64_t n8 = (int64_t)T * f / 8;
   swiglu_act_kernel<<<2048, 256, 0, s>>>((const uint16_t*)p->a, (const uint16_t*)p->b, (uint16_t*)p->h, n8);
   RA_CHECK_LAUNCH("swiglu_act");
@@ -610,8 +631,7 @@ int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s) {
   //   dh = dy w2^T ; da, db from the activation ; dx = da w1^T + db w3^T
   //   dw1 += x^T da ; dw3 += x^T db ; dw2 += h^T dy
   if (!p->preact_saved) {
-    if (int rc = gemm_bf16(p->x, p->w1, p->a, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;
-    if (int rc = gemm_bf16(p->x, p->w3, p->b, T, f, d, 0, 0, RA_BF16, 0, tile, s)) return rc;
+    if (int rc = gemm_bf16_pair(p->x, p->w1, p->w3, p->a, p->b, T, f, d, tile, s)) return rc;
   }
   // dh goes into the da buffer first, the activation backward then rewrites it in place
   if (int rc = gemm_bf16(p->dy, p->w2, p->da, T, f, d, 0, 1, RA_BF16, 0, tile, s)) return rc;
