@@ -76,6 +76,12 @@ typedef struct ra_mask {
                                      skip_masked_tiles it lets kernels skip key (query) tiles whose id range
                                      cannot meet the ids of the query (key) rows at hand */
   int32_t seg_tiles;
+  const int32_t* seg_run_hulls;   /* nullable; from ra_segment_run_hulls: (B or 1, seg_runs, 2) = for every run of
+                                     2 * RA_SEG_TILE global positions the first and one-past-the-last tile (of
+                                     RA_SEG_TILE positions, over the whole sequence) whose id range meets the run's.
+                                     Lets a workgroup find its key (query) tiles with two loads instead of a scan.
+                                     Only when segment_ids covers every position the call touches */
+  int32_t seg_runs;               /* ceil(seg_tiles / 2) */
   const uint8_t* keep;        /* nullable; a boolean mask, nonzero = attend.  keep_mode says what a zero does:
                                  RA_KEEP_WHERE, the attn_mask of ring_attention_inference
                                  (ringattention_inference.py:19-22): the logit becomes mask_min;
@@ -172,6 +178,11 @@ enum { RA_SEG_TILE = 64 };
  * only feeds the tile-skipping of the kernels. */
 int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int32_t Bseg, int32_t seg_len,
                            int32_t* out, ra_stream_t stream);
+
+/* From the ranges of ra_segment_tile_ranges (minmax: (Bseg, seg_tiles, 2)) to ra_mask.seg_run_hulls:
+ * out (Bseg, ceil(seg_tiles / 2), 2).  No counterpart in the reference; only feeds the tile skipping. */
+int ra_segment_run_hulls(const int32_t* seg_tile_minmax, int32_t Bseg, int32_t seg_tiles, int32_t* out,
+                         ra_stream_t stream);
 
 /* Packs a boolean mask (nonzero = attend; byte strides, 0 broadcasts an axis) of Q x K positions, both
  * multiples of 64, into the three arrays ra_mask.keep_bits_k / keep_bits_q / keep_summary describe, for Bm x Hm

@@ -31,6 +31,7 @@ class RaMask(C.Structure):
         ("q_chunk_idx_start", i32), ("k_chunk_idx_start", i32), ("cache_idx", vp), ("chunk_starts", vp),
         ("mask_min", f32),
         ("skip_masked_tiles", i32), ("seg_tile_minmax", vp), ("seg_tiles", i32),
+        ("seg_run_hulls", vp), ("seg_runs", i32),
         ("keep", vp), ("keep_stride_b", i64), ("keep_stride_h", i64), ("keep_stride_q", i64),
         ("keep_stride_k", i64),
         ("keep_bits_k", vp), ("keep_bits_q", vp), ("keep_summary", vp),
@@ -117,6 +118,7 @@ class RaRmsnormParams(C.Structure):
 # every symbol include/ringattn_hip.h and include/ringattn_hip_measure.h declare: (name, restype, argtypes)
 SYMBOLS = {
     "ra_segment_tile_ranges": (C.c_int, [vp, i64, i32, i32, vp, vp]),
+    "ra_segment_run_hulls": (C.c_int, [vp, i32, i32, vp, vp]),
     "ra_keep_pack": (C.c_int, [vp, i64, i64, i64, i64, i32, i32, i32, i32, vp, vp, vp, vp]),
     "ra_dropout_keep": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp]),
     "ra_dropout_keep_packed": (C.c_int, [C.c_uint64, f32, i32, i32, i32, i32, vp, vp, vp, i32, i32, i32, i32, i32, vp]),

@@ -32,6 +32,7 @@ int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, voi
 int bwd_delta(const void*, const void*, int, int, int64_t, int64_t, float*, int64_t, int64_t, int, int, int, int,
               hipStream_t);
 int seg_tile_ranges(const int32_t*, int64_t, int, int, int32_t*, hipStream_t);
+int seg_run_hulls(const int32_t*, int, int, int32_t*, hipStream_t);
 int keep_pack(const uint8_t*, int64_t, int64_t, int64_t, int64_t, int, int, int, int, uint64_t*, uint64_t*, uint8_t*, hipStream_t);
 int dropout_keep(uint64_t seed, uint32_t threshold, int64_t n, uint8_t* keep, hipStream_t s);
 int dropout_keep_packed(uint64_t seed, uint32_t threshold, int planes, int Q, int K, uint64_t* bits_k,
@@ -71,6 +72,9 @@ static int check_mask(const ra_mask& m, int Sq, int Skv, const char* who) {
   if (m.seg_tile_minmax)
     RA_REQUIRE(m.segment_ids && m.seg_tiles == (m.seg_len + RA_SEG_TILE - 1) / RA_SEG_TILE, RA_ERR_INVALID,
                "%s: seg_tile_minmax needs segment_ids and seg_tiles == ceil(seg_len / %d)", who, (int)RA_SEG_TILE);
+  if (m.seg_run_hulls)
+    RA_REQUIRE(m.seg_tile_minmax && m.seg_runs == (m.seg_tiles + 1) / 2, RA_ERR_INVALID,
+               "%s: seg_run_hulls needs seg_tile_minmax and seg_runs == ceil(seg_tiles / 2)", who);
   if (m.keep_bits_k || m.keep_bits_q || m.keep_summary) {
     RA_REQUIRE(m.keep_bits_k && m.keep_bits_q && m.keep_summary, RA_ERR_INVALID,
                "%s: the packed keep mask needs keep_bits_k, keep_bits_q and keep_summary together", who);
@@ -161,6 +165,13 @@ int ra_segment_tile_ranges(const int32_t* segment_ids, int64_t seg_stride_b, int
   RA_REQUIRE(segment_ids && out, RA_ERR_INVALID, "segment_tile_ranges: null pointer");
   RA_REQUIRE(Bseg > 0 && Bseg <= 65535 && seg_len > 0, RA_ERR_INVALID, "segment_tile_ranges: bad shape");
   return seg_tile_ranges(segment_ids, seg_stride_b, Bseg, seg_len, out, (hipStream_t)stream);
+}
+
+int ra_segment_run_hulls(const int32_t* seg_tile_minmax, int32_t Bseg, int32_t seg_tiles, int32_t* out,
+                         ra_stream_t stream) {
+  RA_REQUIRE(seg_tile_minmax && out, RA_ERR_INVALID, "segment_run_hulls: null pointer");
+  RA_REQUIRE(Bseg > 0 && Bseg <= 65535 && seg_tiles > 0, RA_ERR_INVALID, "segment_run_hulls: bad shape");
+  return seg_run_hulls(seg_tile_minmax, Bseg, seg_tiles, out, (hipStream_t)stream);
 }
 
 int ra_keep_pack(const uint8_t* keep, int64_t stride_b, int64_t stride_h, int64_t stride_q, int64_t stride_k,

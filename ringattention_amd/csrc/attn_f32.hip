@@ -126,9 +126,8 @@ __device__ __forceinline__ void f32_key_range(const MaskView& mv, int b, int h, 
   ntiles = (kend + XBN - 1) / XBN;
   k_base = 0;
   if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gq0, XBM, slo, shi);
-    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 256, t_first, t_last);
+    int t_first, t_last;
+    seg_hull_of_rows(mv, b, gq0, XBM, gk0_shard / RA_SEG_TILE, ntiles, hull2, tid, 256, t_first, t_last);
     k_base = t_first * XBN;
     ntiles = t_last - t_first;
   }
@@ -536,9 +535,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_f32_kernel(F32Args a) {
   }
   int qt_end = nqt;
   if (HAS_SEG && mv.seg_mm && mv.skip_tiles && qt_first < nqt) {
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gk0, XBM, slo, shi);
-    seg_tile_hull(mv, b, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, slo, shi, hull2, tid, 256, t_first, t_last);
+    int t_first, t_last;
+    seg_hull_of_rows(mv, b, gk0, XBM, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, hull2, tid, 256, t_first, t_last);
     qt_end = qt_first + t_last;
     qt_first += t_first;
   }

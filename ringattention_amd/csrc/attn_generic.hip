@@ -427,6 +427,31 @@ int seg_tile_ranges(const int32_t* seg, int64_t seg_sb, int Bseg, int seg_len, i
   return RA_OK;
 }
 
+// For every run of 2 * RA_SEG_TILE positions: first and one-past-the-last tile (of all ntile) whose id range meets the
+// run's.  One workgroup per run; the run's own tiles always meet it, so the hull is never empty.
+__global__ __launch_bounds__(256) void seg_run_hulls_kernel(const int32_t* mm, int ntile, int nrun, int32_t* out) {
+  __shared__ int hull[2];
+  const int r = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int32_t* m = mm + (int64_t)b * ntile * 2;
+  const int t0 = 2 * r, t1 = min(2 * r + 1, ntile - 1);
+  const int lo = min(m[2 * t0], m[2 * t1]), hi = max(m[2 * t0 + 1], m[2 * t1 + 1]);
+  if (tid == 0) { hull[0] = ntile; hull[1] = 0; }
+  __syncthreads();
+  int first = ntile, last = 0;
+  for (int t = tid; t < ntile; t += 256)
+    if (m[2 * t + 1] >= lo && m[2 * t] <= hi) { first = min(first, t); last = max(last, t + 1); }
+  if (first < ntile) { atomicMin(&hull[0], first); atomicMax(&hull[1], last); }
+  __syncthreads();
+  if (tid == 0) { out[((int64_t)b * nrun + r) * 2] = hull[0]; out[((int64_t)b * nrun + r) * 2 + 1] = hull[1]; }
+}
+
+int seg_run_hulls(const int32_t* mm, int Bseg, int ntile, int32_t* out, hipStream_t s) {
+  const int nrun = (ntile + 1) / 2;
+  seg_run_hulls_kernel<<<dim3(nrun, Bseg), 256, 0, s>>>(mm, ntile, nrun, out);
+  RA_CHECK_LAUNCH("seg_run_hulls");
+  return RA_OK;
+}
+
 // One 64 x 64 tile of the boolean mask per workgroup of 64 threads: thread i writes the word of query row i
 // (bits over the tile's keys) and the word of key column i (bits over the tile's query rows).
 __global__ __launch_bounds__(64) void keep_pack_kernel(const uint8_t* keep, int64_t sb, int64_t sh, int64_t sq,

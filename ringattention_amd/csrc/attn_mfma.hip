@@ -312,9 +312,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
   int qt_end = nqt;
   if (HAS_SEG && mv.seg_mm && mv.skip_tiles && qt_first < nqt) {
     __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gk0, KBN, slo, shi);
-    seg_tile_hull(mv, b, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, slo, shi, hull2, tid, 512, t_first, t_last);
+    int t_first, t_last;
+    seg_hull_of_rows(mv, b, gk0, KBN, gq_base / RA_SEG_TILE + qt_first, nqt - qt_first, hull2, tid, 512, t_first, t_last);
     qt_end = qt_first + t_last;
     qt_first += t_first;
   }
@@ -762,9 +761,8 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
   int k_base = 0;
   if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
     __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gq0, FBM, slo, shi);
-    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
+    int t_first, t_last;
+    seg_hull_of_rows(mv, b, gq0, FBM, gk0_shard / RA_SEG_TILE, ntiles, hull2, tid, 512, t_first, t_last);
     k_base = t_first * FBN;
     ntiles = t_last - t_first;
   }
@@ -1222,9 +1220,8 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   int k_base = 0;
   if (HAS_SEG && mv.seg_mm && mv.skip_tiles && ntiles > 0) {
     __shared__ int hull2[2];
-    int slo, shi, t_first, t_last;
-    seg_rows_range(mv, b, gq0, FBM, slo, shi);
-    seg_tile_hull(mv, b, gk0_shard / RA_SEG_TILE, ntiles, slo, shi, hull2, tid, 512, t_first, t_last);
+    int t_first, t_last;
+    seg_hull_of_rows(mv, b, gq0, FBM, gk0_shard / RA_SEG_TILE, ntiles, hull2, tid, 512, t_first, t_last);
     k_base = t_first * FBN;
     ntiles = t_last - t_first;
   }

@@ -63,6 +63,8 @@ struct MaskView {
   int skip_tiles;
   const int32_t* seg_mm;   // per-64-position (min, max) segment ids, or null
   int seg_tiles;
+  const int32_t* seg_hull; // per-128-position [first, last) 64-position tile whose id range meets the run's, or null
+  int seg_runs;
   const uint8_t* keep;     // boolean mask (local query row, global key - keep_k0), or null
   int64_t keep_sb, keep_sh, keep_sq, keep_sk;
   const uint64_t* kbits_k;   // packed mask, see ra_keep_pack; all null unless the MFMA kernels take the mask
@@ -85,6 +87,7 @@ struct MaskView {
     v.any_mask = (m.segment_ids != nullptr) || (m.causal_block_size > 0);
     v.skip_tiles = m.skip_masked_tiles;
     v.seg_mm = m.seg_tile_minmax; v.seg_tiles = m.seg_tiles;
+    v.seg_hull = m.seg_run_hulls; v.seg_runs = m.seg_runs;
     v.keep = m.keep; v.keep_sb = m.keep_stride_b; v.keep_sh = m.keep_stride_h;
     v.keep_sq = m.keep_stride_q; v.keep_sk = m.keep_stride_k;
     v.kbits_k = m.keep_bits_k; v.kbits_q = m.keep_bits_q; v.ksum = m.keep_summary;
@@ -160,6 +163,26 @@ __device__ __forceinline__ void seg_rows_range(const MaskView& mv, int b, int g0
     const int g = min(t, mv.seg_tiles - 1);
     lo = min(lo, mm[2 * g]); hi = max(hi, mm[2 * g + 1]);
   }
+}
+
+// The two calls above for the rows [g_rows0, g_rows0 + rows): the hull, among the n tiles starting at global tile gt0,
+// of the tiles that can hold a position of one of the rows' segments.  With the table of ra_segment_run_hulls (one
+// entry per run of 128 positions, over ALL tiles of the sequence) this is two loads and an intersection instead of a
+// scan with two barriers - the table's hull can only be wider than the scan's (tiles between two meeting ones), which
+// adds fully masked tiles and changes no result.  Every thread of the workgroup must call it.
+__device__ __forceinline__ void seg_hull_of_rows(const MaskView& mv, int b, int g_rows0, int rows, int gt0, int n,
+                                                 int* hull2, int tid, int nthreads, int& first, int& last) {
+  if (mv.seg_hull && rows == 2 * RA_SEG_TILE && (g_rows0 % (2 * RA_SEG_TILE)) == 0) {
+    const int r = min(g_rows0 / (2 * RA_SEG_TILE), mv.seg_runs - 1);
+    const int32_t* h = mv.seg_hull + ((int64_t)(mv.seg_sb ? b : 0) * mv.seg_runs + r) * 2;
+    first = max(h[0] - gt0, 0);
+    last = min(h[1] - gt0, n);
+    if (last <= first) { first = 0; last = 0; }
+    return;
+  }
+  int lo, hi;
+  seg_rows_range(mv, b, g_rows0, rows, lo, hi);
+  seg_tile_hull(mv, b, gt0, n, lo, hi, hull2, tid, nthreads, first, last);
 }
 
 // ---- boolean keep mask in packed form (ra_keep_pack): 64-bit words and a per-64x64-tile summary

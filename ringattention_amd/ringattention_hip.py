@@ -150,6 +150,9 @@ class _Config:
         # False: never reuse the int32 copy / tile ranges of a segment_ids tensor seen before (for callers that edit
         # the ids through a numpy alias or .data, which the tensor's version counter does not see)
         self.cache_segment_ids = bool(kw.get("cache_segment_ids", True))
+        # False: the kernels scan the per-tile id ranges for their tile hulls instead of reading the per-run table
+        # (the two give the same results; for tests)
+        self.segment_hull_table = bool(kw.get("segment_hull_table", True))
         self.logit_dim = 0            # set when q, k, v were zero-padded along D: the head size that scales the logits
         self.ring_launch = kw.get("ring_launch", "step")
         if self.ring_launch not in ("step", "device"):
@@ -187,6 +190,7 @@ class _MaskInputs:
         self.seg_stride_b = 0
         self.seg_len = 0
         self.seg_mm = None
+        self.seg_hull = None
         self.seg_tiles = 0
         if segment_ids is not None:
             if segment_ids.dim() != 2:
@@ -211,7 +215,7 @@ class _MaskInputs:
                 _SEG_CACHE.move_to_end(key)
                 self._seg_entry = hit
             else:
-                self._seg_entry = self._segment_entry(segment_ids, device) + [cur_stream]
+                self._seg_entry = self._segment_entry(segment_ids, device, cur_stream)
                 if key is not None:
                     _SEG_CACHE[key] = self._seg_entry
                     while len(_SEG_CACHE) > 8:
@@ -222,6 +226,10 @@ class _MaskInputs:
             self.seg_len = s.shape[1]
             self.seg_tiles = (self.seg_len + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
             self.seg_mm = self._seg_entry[2]
+            self.seg_hull = self._seg_entry[5]
+        # set by a caller that knows that segment_ids covers every global position of its calls (no clamped slices):
+        # the kernels may then look their tile hulls up in the per-run table instead of scanning the tile ranges
+        self.seg_covers = False
         self.keep = None                   # boolean mask: ring_attention_inference (set_keep) or dropout
         self.keep_strides = (0, 0, 0, 0)
         self.keep_row0 = 0
@@ -243,22 +251,26 @@ class _MaskInputs:
                 self.cache_idx_host = int(cache_idx)
 
     @staticmethod
-    def _segment_entry(segment_ids, device):
-        """[weakref, int32 ids on the device, per-64-position (min, max) id ranges, host copy of the ranges (lazy)];
-        the caller appends the stream that produced them."""
+    def _segment_entry(segment_ids, device, stream):
+        """[weakref, int32 ids on the device, per-64-position (min, max) id ranges, host copy of the ranges (lazy),
+        the stream that produced them, per-128-position tile hulls (ra_segment_run_hulls; None without a GPU)]."""
         s = segment_ids.detach().to(device=device, dtype=torch.int32).contiguous()
         tiles = (s.shape[1] + L.RA_SEG_TILE - 1) // L.RA_SEG_TILE
         mm = torch.empty((s.shape[0], tiles, 2), dtype=torch.int32, device=device)
+        hull = None
         if s.is_cuda:
             # lets the MFMA kernels skip tiles of foreign segments
             L.check(L.load().ra_segment_tile_ranges(s.data_ptr(), s.stride(0), s.shape[0], s.shape[1],
                                                     mm.data_ptr(), _stream()), "ra_segment_tile_ranges")
+            hull = torch.empty((s.shape[0], (tiles + 1) // 2, 2), dtype=torch.int32, device=device)
+            L.check(L.load().ra_segment_run_hulls(mm.data_ptr(), s.shape[0], tiles, hull.data_ptr(), _stream()),
+                    "ra_segment_run_hulls")
         else:                                  # host logic only (tests without a GPU): same ranges with torch ops
             pad = tiles * L.RA_SEG_TILE - s.shape[1]
             sp = torch.nn.functional.pad(s, (0, pad), mode="replicate") if pad else s
             sp = sp.view(s.shape[0], tiles, L.RA_SEG_TILE)
             mm = torch.stack((sp.amin(dim=2), sp.amax(dim=2)), dim=2).to(torch.int32)
-        return [weakref.ref(segment_ids), s, mm, None]
+        return [weakref.ref(segment_ids), s, mm, None, stream, hull]
 
     def set_keep(self, attn_mask, device, q_total, k_total):
         """attn_mask (B|1, H|1, Q|1, K_total), nonzero = attend (ringattention_inference.py:19-22).
@@ -376,6 +388,9 @@ class _MaskInputs:
         m.skip_masked_tiles = 1 if skip else 0
         m.seg_tile_minmax = self.seg_mm.data_ptr() if self.seg_mm is not None else None
         m.seg_tiles = self.seg_tiles
+        if self.seg_hull is not None and self.seg_covers and chunk_starts is None:
+            m.seg_run_hulls = self.seg_hull.data_ptr()
+            m.seg_runs = (self.seg_tiles + 1) // 2
         if self.keep is not None or self.keep_packed is not None:
             if self.keep is not None:
                 m.keep = self.keep.data_ptr() + self.keep_row0 * self.keep_strides[2]
@@ -715,6 +730,8 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
         raise ValueError("per-device lengths (%d, %d) must divide by the chunk sizes (%d, %d)"
                          % (q_len, kv_len, cfg.qc, cfg.kc))
     mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, kv_total)
+    mi.seg_covers = (mi.seg is not None and cache_idx is None and mi.seg_len >= max(q_total, kv_total)
+                     and cfg.segment_hull_table)
     if cfg.skip_masked_tiles is None:
         cfg.skip_masked_tiles = bool(cfg.qc >= 2 and cache_idx is None and q_total == kv_total)
     if cfg.pdrop > 0.0:
@@ -1045,12 +1062,20 @@ def _saved_residuals(ctx):
 def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
     """Drop-in for ringattention_jax.py:92-97 (exported as ``ringattention``).
 
-    q, k, v: (B, S, H, D) device tensors, bf16 or fp32; with a declared ring axis they are the global
+    q, k, v: (B, S, H, D) device tensors, bf16, fp32 or fp16 (computed on fp32 copies); with a declared ring axis they are the global
     arrays and the sequence axis is split over the virtual devices.  attn_bias (B|1, H|1, 1, K_total)
     and segment_ids (B|1, S_total) are global / replicated, as in the reference's shard_map specs.
     One query token with cache_idx set takes the streaming decode kernel."""
     # (the streaming kernel serves head sizes 64 and 128; any other takes the blockwise kernels below, like a call
     # that wants gradients)
+    if q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16:
+        # float16 inputs: with float32_logits the reference casts q and k to fp32 (:18-19) and the products with v
+        # promote to fp32 as well, so computing on exact fp32 copies (the fp32 matrix-core kernels) and rounding the
+        # output - and, through autograd, the gradients - to float16 is its arithmetic; twice the memory of a native
+        # float16 path, which the kernels do not have
+        out = ring_attention(q.float(), k.float(), v.float(), attn_bias, segment_ids, cache_idx, axis_name,
+                             float32_logits, blockwise_kwargs)
+        return out.to(torch.float16)
     n = axis_size(axis_name)
     if cache_idx is not None and q.shape[1] == n and q.shape[3] in (64, 128) and not (
             torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) \

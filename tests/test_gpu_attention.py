@@ -659,3 +659,72 @@ def test_a_large_call_on_the_generic_kernels_warns_once():
         ra.ringattention(qd[:, :256], kd[:, :256], vd[:, :256], bd[..., :256], None, None, axis_name=None,
                          float32_logits=True, blockwise_kwargs=kw)
     assert not [w for w in seen if "generic vector-ALU kernels" in str(w.message)]
+
+
+def test_float16_inputs_are_computed_in_fp32_and_rounded():
+    """float16 q, k, v (the reference is dtype-generic, ringattention_jax.py:18-23): computed on exact fp32 copies,
+    output and gradients rounded to float16.  Bar: the oracle on the same float16 inputs, fp32 tolerance on values of
+    order one widened by the float16 rounding of the results (2^-11 relative)."""
+    B, S, H, D, n = 1, 512, 2, 64, 2
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.float16, seed=4, scale=D ** -0.25)
+    seg = packed_segment_ids(B, S, 200, seed=3)
+    kw = kwargs(128, 128, 1, dtype=torch.float32)
+    ref_out, ref_grads = oracle_fwd_bwd(q.float(), k.float(), v.float(), do.float(), None, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, None, seg, None, n, kw)
+    assert out.dtype == torch.float16 and all(g.dtype == torch.float16 for g in grads)
+    assert ra.kernel_family_of_last_call() == {"forward": "mfma_f32", "backward": "mfma_f32"}
+    for name, a, b in zip(("out", "dq", "dk", "dv"), (out,) + tuple(grads), (ref_out,) + tuple(ref_grads)):
+        ma, rl = errors(a, b)
+        assert ma <= 1e-4 + 2.0 ** -11 * float(b.abs().max()) and rl <= 1e-3, (name, ma, rl)
+
+
+def test_segment_run_hulls_equal_brute_force():
+    """ra_segment_run_hulls: for every run of 128 positions the hull of the 64-position tiles whose id range meets
+    the run's, against a double loop in numpy; packed documents (monotone ids) and ids in arbitrary order."""
+    import ctypes
+    import numpy as np
+    from ringattention_amd import _lib as L
+    S = 4096 + 64                     # an odd number of tiles: the last run has one tile
+    rng = np.random.default_rng(0)
+    packed = packed_segment_ids(2, S, 300, seed=1).numpy()
+    shuffled = rng.integers(0, 6, size=(2, S // 32)).repeat(32, axis=1).astype(np.int32)
+    for ids in (packed, shuffled):
+        seg = torch.from_numpy(ids).to(DEV)
+        tiles = (S + 63) // 64
+        mm = torch.empty((2, tiles, 2), dtype=torch.int32, device=DEV)
+        hull = torch.empty((2, (tiles + 1) // 2, 2), dtype=torch.int32, device=DEV)
+        st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        L.check(L.load().ra_segment_tile_ranges(seg.data_ptr(), seg.stride(0), 2, S, mm.data_ptr(), st), "ranges")
+        L.check(L.load().ra_segment_run_hulls(mm.data_ptr(), 2, tiles, hull.data_ptr(), st), "hulls")
+        mmh, got = mm.cpu().numpy(), hull.cpu().numpy()
+        for b in range(2):
+            for r in range((tiles + 1) // 2):
+                ts = [t for t in (2 * r, 2 * r + 1) if t < tiles]
+                lo, hi = min(mmh[b, t, 0] for t in ts), max(mmh[b, t, 1] for t in ts)
+                meet = [t for t in range(tiles) if mmh[b, t, 1] >= lo and mmh[b, t, 0] <= hi]
+                assert (got[b, r, 0], got[b, r, 1]) == (meet[0], meet[-1] + 1), (b, r)
+
+
+@pytest.mark.parametrize("dtype,ids", [(torch.bfloat16, "packed"), (torch.bfloat16, "interleaved"), (torch.float32, "packed")])
+def test_hull_table_gives_the_results_of_the_scan(dtype, ids):
+    """The per-run hull table (the default when segment_ids covers every position) against the in-kernel scan of the
+    tile ranges: the same bits for packed documents, where the two hulls coincide; with documents interleaved in
+    blocks the table's hull is wider by fully masked tiles, which add exact zeros."""
+    B, S, H, D, n = 1, 2048, 2, 128, 4
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=8, scale=D ** -0.25)
+    if ids == "packed":
+        seg = packed_segment_ids(B, S, 300, seed=5)
+    else:
+        seg = (torch.arange(S) // 192 % 3).to(torch.int32).reshape(1, S)       # three documents in alternating blocks
+    bias = torch.randn(B, 1, 1, S, generator=torch.Generator().manual_seed(6))
+    kw = kwargs(128, 128, 1, dtype=torch.float32, impl="mfma")
+    a_out, a_g = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    b_out, b_g = run_hip(q, k, v, do, bias, seg, None, n, dict(kw, segment_hull_table=False))
+    assert not torch.isnan(a_out).any()
+    assert torch.equal(a_out, b_out)
+    for x, y in zip(a_g, b_g):
+        assert torch.equal(x, y)
+    ref_out, ref_g = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    assert_close(a_out, ref_out, dtype, "out")
+    for name, x, y in zip(("dq", "dk", "dv"), a_g, ref_g):
+        assert_close(x, y, dtype, name)

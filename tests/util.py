@@ -16,7 +16,7 @@ def kwargs(qc, kc, cbs=1, dtype=torch.float32, **extra):
 
 def oracle_kwargs(kw):
     return {k: v for k, v in kw.items() if k not in ("impl", "skip_masked_tiles", "bwd_only", "ring_launch", "output_residual",
-                                                          "cache_segment_ids")}
+                                                          "cache_segment_ids", "segment_hull_table")}
 
 
 def make_qkv(B, S, H, D, dtype=torch.float32, seed=0, Skv=None, scale=1.0):
