@@ -385,15 +385,24 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       if (HAS_SEG) st_seg[BUF][tid - 256] = r_seg;                                                      \
     }                                                                                                   \
   }
-  RA_WS_LOAD(0);
-  RA_WS_STORE(0);
-  RA_WS_LOAD(1);
-  RA_WS_STORE(1);
-  RA_WS_LOAD(2);
-  __syncthreads();
+  // Both roles stage the first tiles, then meet at the first barrier, each inside its own branch: the producer's K and
+  // V fragments are requested before the staging, so that their latency runs next to it instead of after the barrier,
+  // and being defined inside the branch they take no register of the consumers
+#define RA_WS_PROLOGUE  \
+  RA_WS_LOAD(0); RA_WS_STORE(0); RA_WS_LOAD(1); RA_WS_STORE(1); RA_WS_LOAD(2); __syncthreads();
 
   if (role == 0) {
     // =========================== producer: S, dP -> P, dS
+    bf16x8 kf[NK], vf[NK];
+    {
+      const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
+#pragma unroll
+      for (int t = 0; t < NK; t++) {
+        kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
+        vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
+      }
+    }
+    RA_WS_PROLOGUE
     const int qlim = mv.cbs > 0 ? (gk / mv.cbs) * mv.cbs : -0x7fffffff;       // masked iff gq < qlim
     const int qlim_wave = __builtin_amdgcn_readfirstlane(mv.cbs > 0 ? ((gk0 + pair * 32 + 31) / mv.cbs) * mv.cbs : -0x7fffffff);
     int seg_k = 0;
@@ -407,13 +416,6 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       if (mv.any_mask) bv = fminf(bv, 0.f);
       bias2 = bv * kLog2e / c;          // the S accumulators start from it
       st_bias[pair][lane] = bias2;      // kept in LDS, not in a register: every lane reads back its own slot
-    }
-    const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)krow * a.kv_ss + (int64_t)h * HD + hi * 8;
-    bf16x8 kf[NK], vf[NK];
-#pragma unroll
-    for (int t = 0; t < NK; t++) {
-      kf[t] = *(const bf16x8*)(a.k + koff + t * 16);
-      vf[t] = *(const bf16x8*)(a.v + koff + t * 16);
     }
     int n_off[NK];
 #pragma unroll
@@ -592,6 +594,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     __syncthreads();      // step 2 ntq: the consumer's last block
   } else {
     // =========================== consumer: dV^T += dO^T P, dK^T += Q^T dS
+    RA_WS_PROLOGUE
     f32x16 dkacc[NDB], dvacc[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; db++)
@@ -694,6 +697,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
         }
     }
   }
+#undef RA_WS_PROLOGUE
 #undef RA_WS_LOAD
 #undef RA_WS_STORE
 #undef RA_WS_INIT
@@ -846,18 +850,23 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + SRP * TROW) = S##v1;                                        \
     if (SNP == 4) { *(uint4*)(dv_ + 2 * SRP * TROW) = S##v2; *(uint4*)(dv_ + 3 * SRP * TROW) = S##v3; } \
   }
-  if (role == 1) {
-    RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
-    RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
-    RA_WS_STORE_K(A, 0); RA_WS_STORE_V(A, 0);
-    RA_WS_LOAD_K(A, 2); RA_WS_LOAD_V(A, 2);
-    RA_WS_STORE_K(B, 1); RA_WS_STORE_V(B, 1);
-    RA_WS_LOAD_K(B, 3); RA_WS_LOAD_V(B, 3);
-  }
-  __syncthreads();
-
+  // The consumers stage the first tiles; meanwhile the producers request their Q / dO fragments and row statistics.
+  // The two roles meet at the first barrier, each inside its own branch.
   if (role == 0) {
     // =========================== producer: S^T, dP^T -> dS^T
+    bf16x8 qf[NK], gf[NK];
+    float st_den, st_mx, st_delta;
+    {
+      const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
+#pragma unroll
+      for (int t = 0; t < NK; t++) {
+        qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
+        gf[t] = *(const bf16x8*)(a.g + qoff + t * 16);
+      }
+      const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+      st_den = a.den[st]; st_mx = a.mx[st]; st_delta = a.delta[st];
+    }
+    __syncthreads();
     const int gq = gq0 + pair * 32 + lo;
     const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
     const int klim_wave = __builtin_amdgcn_readfirstlane(
@@ -867,19 +876,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
       int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
       seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
     }
-    const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-    bf16x8 qf[NK], gf[NK];
-#pragma unroll
-    for (int t = 0; t < NK; t++) {
-      qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
-      gf[t] = *(const bf16x8*)(a.g + qoff + t * 16);
-    }
-    const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
-    const float den = a.den[st];
-    const float m2 = max_to_log2(a.mx[st], kMask2);
+    const float den = st_den;
+    const float m2 = max_to_log2(st_mx, kMask2);
     const float rden = 1.f / den;
     const float lse2 = m2 + __log2f(den);
-    const float ndelta = -a.delta[st];
+    const float ndelta = -st_delta;
     int n_off[NK];
 #pragma unroll
     for (int t = 0; t < NK; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz<HD>(lo)) << 3);
@@ -1064,6 +1065,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
 #undef RA_WS_PRODUCE
   } else {
     // =========================== consumer: dQ^T += K^T dS^T
+    RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
+    RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
+    RA_WS_STORE_K(A, 0); RA_WS_STORE_V(A, 0);
+    RA_WS_LOAD_K(A, 2); RA_WS_LOAD_V(A, 2);
+    RA_WS_STORE_K(B, 1); RA_WS_STORE_V(B, 1);
+    RA_WS_LOAD_K(B, 3); RA_WS_LOAD_V(B, 3);
+    __syncthreads();
     f32x16 acc[NDB];
 #pragma unroll
     for (int db = 0; db < NDB; db++)
@@ -1311,18 +1319,22 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     *(uint4*)(dv_) = S##v0; *(uint4*)(dv_ + SRP * TROW) = S##v1;                                        \
     if (SNP == 4) { *(uint4*)(dv_ + 2 * SRP * TROW) = S##v2; *(uint4*)(dv_ + 3 * SRP * TROW) = S##v3; } \
   }
-  if (role == 1) {
-    RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
-    RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
-    RA_WS_STORE_K(A, 0); RA_WS_STORE_V(A, 0);
-    RA_WS_LOAD_K(A, 2); RA_WS_LOAD_V(A, 2);
-    RA_WS_STORE_K(B, 1); RA_WS_STORE_V(B, 1);
-    RA_WS_LOAD_K(B, 3); RA_WS_LOAD_V(B, 3);
-  }
-  __syncthreads();
-
+  // The consumers stage the first tiles; meanwhile the producers request their Q fragments and the carry's statistics.
+  // The two roles meet at the first barrier, each inside its own branch.
   if (role == 0) {
     // =========================== producer: S^T -> online softmax -> P^T
+    bf16x8 qf[NK];
+    float st_mx = 0.f, st_den = 0.f;
+    {
+      const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
+#pragma unroll
+      for (int t = 0; t < NK; t++) qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
+      if (!a.carry_is_initial) {
+        const int64_t st0 = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
+        st_mx = a.mx[st0]; st_den = a.den[st0];
+      }
+    }
+    __syncthreads();
     const int gq = gq0 + pair * 32 + lo;
     const int klim = mv.cbs > 0 ? (int)min((long long)(gq / mv.cbs + 1) * mv.cbs, 0x7fffffffLL) : 0x7fffffff;
     const int klim_wave = __builtin_amdgcn_readfirstlane(
@@ -1332,17 +1344,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
       int idx = clamp_seg_index(((long long)mv.q_start + qi) * mv.qc, mv.qc, mv.seg_len, qrow % mv.qc);
       seg_q = mv.seg[(int64_t)b * mv.seg_sb + idx];
     }
-    const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * HD + hi * 8;
-    bf16x8 qf[NK];
-#pragma unroll
-    for (int t = 0; t < NK; t++) qf[t] = *(const bf16x8*)(a.q + qoff + t * 16);
     const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + qrow;
     // running max (log2 domain; m2 is the lazy reference the probabilities are taken against, m_true the
     // exact one) and this half-row's share of the running sum
     float m2 = RA_NEG_INF, l = 0.f;
     if (!a.carry_is_initial) {
-      m2 = max_to_log2(a.mx[st], kMask2);
-      l = hi == 0 ? a.den[st] : 0.f;
+      m2 = max_to_log2(st_mx, kMask2);
+      l = hi == 0 ? st_den : 0.f;
     }
     float m_true = m2, ps = 0.f;
     constexpr float kLazy = 16.f;
@@ -1561,6 +1569,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
 #undef RA_WS_PRODUCE
   } else {
     // =========================== consumer: O^T += V^T P^T   (:141-143)
+    RA_WS_LOAD_K(A, 0); RA_WS_LOAD_V(A, 0);
+    RA_WS_LOAD_K(B, 1); RA_WS_LOAD_V(B, 1);
+    RA_WS_STORE_K(A, 0); RA_WS_STORE_V(A, 0);
+    RA_WS_LOAD_K(A, 2); RA_WS_LOAD_V(A, 2);
+    RA_WS_STORE_K(B, 1); RA_WS_STORE_V(B, 1);
+    RA_WS_LOAD_K(B, 3); RA_WS_LOAD_V(B, 3);
+    __syncthreads();
     f32x16 acc[NDB];
     float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)qrow * a.num_ss + (int64_t)h * HD + hi * 4;
     if (a.carry_is_initial) {
