@@ -520,7 +520,8 @@ def bench_ffn(args):
         x.grad = None
         for p in ff.parameters():
             p.grad = None
-        y = ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy, launch_tokens=args.ffn_launch_tokens or None)
+        y = ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy, launch_tokens=args.ffn_launch_tokens or None,
+                                     weight_grad_chunks=args.ffn_weight_grad_chunks)
         y.backward(dy)
 
     ms = _time_steps(step, args.steps, args.warmup)
@@ -533,7 +534,8 @@ def bench_ffn(args):
             x.grad = None
             for p in ff.parameters():
                 p.grad = None
-            ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy, launch_tokens=16384).backward(dy)
+            ra.blockwise_feedforward(ff, x, chunk, policy=args.ffn_policy, launch_tokens=16384,
+                                     weight_grad_chunks=args.ffn_weight_grad_chunks).backward(dy)
         ms_sh = _time_steps(step_shared, args.steps, args.warmup)
         shared = {"tokens_per_launch": ra.feedforward._slab_tokens(chunk, T // chunk, 16384),
                   "ms_per_step": round(ms_sh, 3), "value": round(flops / (ms_sh * 1e-3) / 1e12, 2), "unit": "TFLOP/s"}
@@ -570,7 +572,7 @@ def bench_ffn(args):
         "metric": "swiglu_ffn_fwd_bwd_tflops", "value": round(value, 2), "unit": "TFLOP/s", "ms_per_step": round(ms, 3),
         "dtype": "bf16", "pct_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "config": {"workload": "ffn", "tokens": T, "hidden": d, "intermediate": f, "chunk_size": chunk,
-                   "tokens_per_launch": slab,
+                   "tokens_per_launch": slab, "weight_grad_chunks": args.ffn_weight_grad_chunks,
                    "policy": args.ffn_policy, "preactivations": "kept (%.1f GB)" % (4e-9 * T * f) if kept else "recomputed",
                    "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
         "launch_tokens_16384": shared,
@@ -860,6 +862,9 @@ def main():
     ap.add_argument("--ffn-launch-tokens", type=int, default=0,
                     help="ffn workload: let consecutive chunks share a launch of up to this many tokens (default: one "
                          "chunk per launch, as the reference's scan)")
+    ap.add_argument("--ffn-weight-grad-chunks", type=int, default=4,
+                    help="ffn workload: chunks whose weight-gradient products share a launch in the backward pass "
+                         "(blockwise_feedforward's default is 4; 1 = one launch per chunk)")
     ap.add_argument("--inputs", default="baseline", choices=["baseline", "d-quarter", "unit"],
                     help="attention workloads: scale of q and k (baseline = N(0,1)/sqrt(D), the configuration's)")
     ap.add_argument("--no-extras", action="store_true",

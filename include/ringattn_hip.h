@@ -345,6 +345,10 @@ typedef struct ra_swiglu_params {
   int32_t preact_saved;           /* backward: 1 = a and b still hold what the forward wrote for these tokens (the
                                      caller kept them: `policy` other than nothing_saveable, ringattention_jax.py:334);
                                      0 = recompute them from x (the reference's default policy) */
+  int32_t defer_weight_grads;     /* backward: 1 = leave dw1, dw2, dw3 alone (they may be null); the caller adds them
+                                     later with ra_swiglu_weight_grads, over the tokens of several consecutive calls
+                                     at once - their h, da, db kept side by side - so that the fp32 accumulators are
+                                     read and written once per group instead of once per call */
   int32_t gemm_tile;              /* 0: the library picks the tile kernel of each product (the default).  1 + t forces
                                      tile kernel t wherever the shape divides (0: 256 x 256 over four wavefronts,
                                      1: 256 x 128 over eight, 2: 128 x 128, 3: 256 x 128 over four), so that tests reach every
@@ -353,6 +357,10 @@ typedef struct ra_swiglu_params {
 
 int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream);
 int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream);
+/* The weight gradients alone, for T tokens whose h, da, db an earlier ra_swiglu_bwd (with defer_weight_grads) left
+ * in the buffers of p: dw1 += x^T da, dw3 += x^T db, dw2 += h^T dy (the sums over chunks of ringattention_jax.py:344-350,
+ * whose weights are broadcast over the scan).  Reads x, dy, h, da, db, T, d, f, gemm_tile. */
+int ra_swiglu_weight_grads(const ra_swiglu_params* p, ra_stream_t stream);
 
 /* C (M,N) = op(A) op(B), bf16 inputs, fp32 accumulation.  trans_a: A is stored (K,M); trans_b: B is
  * stored (N,K).  c_dtype RA_BF16 (overwrite) or RA_F32 (accumulate when beta_one != 0). */

@@ -91,7 +91,7 @@ class RaSwigluParams(C.Structure):
         ("x", vp), ("w1", vp), ("w2", vp), ("w3", vp),
         ("a", vp), ("b", vp), ("h", vp), ("y", vp),
         ("dy", vp), ("dx", vp), ("dw1", vp), ("dw2", vp), ("dw3", vp), ("da", vp), ("db", vp),
-        ("preact_saved", i32), ("gemm_tile", i32),
+        ("preact_saved", i32), ("defer_weight_grads", i32), ("gemm_tile", i32),
     ]
 
 
@@ -137,6 +137,7 @@ SYMBOLS = {
     "ra_decode_fwd_static": (C.c_int, [C.POINTER(RaDecodeParams), vp]),
     "ra_swiglu_fwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
     "ra_swiglu_bwd": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
+    "ra_swiglu_weight_grads": (C.c_int, [C.POINTER(RaSwigluParams), vp]),
     "ra_gemm_bf16": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, vp]),
     "ra_rope_kv_append": (C.c_int, [C.POINTER(RaRopeAppendParams), vp]),
     "ra_rmsnorm_workspace_bytes": (C.c_size_t, [i64, i32]),

@@ -43,6 +43,7 @@ int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream
 int decode_static_scratch(float** ptr, hipStream_t stream);
 int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s);
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s);
+int swiglu_weight_grads(const ra_swiglu_params* p, hipStream_t s);
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
               int beta_one, int tile, hipStream_t s);
 
@@ -457,12 +458,21 @@ int ra_swiglu_fwd(const ra_swiglu_params* p, ra_stream_t stream) {
 
 int ra_swiglu_bwd(const ra_swiglu_params* p, ra_stream_t stream) {
   RA_REQUIRE(p, RA_ERR_INVALID, "swiglu_bwd: null params");
-  RA_REQUIRE(p->x && p->w1 && p->w2 && p->w3 && p->a && p->b && p->h && p->dy && p->dx && p->dw1 && p->dw2 &&
-                 p->dw3 && p->da && p->db,
+  RA_REQUIRE(p->x && p->w1 && p->w2 && p->w3 && p->a && p->b && p->h && p->dy && p->dx && p->da && p->db &&
+                 (p->defer_weight_grads || (p->dw1 && p->dw2 && p->dw3)),
              RA_ERR_INVALID, "swiglu_bwd: null tensor");
   RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_bwd: empty shape");
   RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 4, RA_ERR_INVALID, "swiglu_bwd: gemm_tile %d outside [0, 4]", p->gemm_tile);
   return swiglu_bwd(p, (hipStream_t)stream);
+}
+
+int ra_swiglu_weight_grads(const ra_swiglu_params* p, ra_stream_t stream) {
+  RA_REQUIRE(p, RA_ERR_INVALID, "swiglu_weight_grads: null params");
+  RA_REQUIRE(p->x && p->dy && p->h && p->da && p->db && p->dw1 && p->dw2 && p->dw3, RA_ERR_INVALID,
+             "swiglu_weight_grads: null tensor");
+  RA_REQUIRE(p->T > 0 && p->d > 0 && p->f > 0, RA_ERR_INVALID, "swiglu_weight_grads: empty shape");
+  RA_REQUIRE(p->gemm_tile >= 0 && p->gemm_tile <= 4, RA_ERR_INVALID, "swiglu_weight_grads: gemm_tile %d outside [0, 4]", p->gemm_tile);
+  return swiglu_weight_grads(p, (hipStream_t)stream);
 }
 
 int ra_gemm_bf16(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,

@@ -624,6 +624,14 @@ int swiglu_fwd(const ra_swiglu_params* p, hipStream_t s) {
   return gemm_bf16(p->h, p->w2, p->y, T, d, f, 0, 0, RA_BF16, 0, tile, s);                 // y = h w2
 }
 
+int swiglu_weight_grads(const ra_swiglu_params* p, hipStream_t s) {
+  if (int rc = check_ffn_shape(p, "swiglu_weight_grads")) return rc;
+  const int T = p->T, d = p->d, f = p->f, tile = p->gemm_tile - 1;
+  if (int rc = gemm_bf16(p->x, p->da, p->dw1, d, f, T, 1, 0, RA_F32, 1, tile, s)) return rc;
+  if (int rc = gemm_bf16(p->x, p->db, p->dw3, d, f, T, 1, 0, RA_F32, 1, tile, s)) return rc;
+  return gemm_bf16(p->h, p->dy, p->dw2, f, d, T, 1, 0, RA_F32, 1, tile, s);
+}
+
 int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s) {
   if (int rc = check_ffn_shape(p, "swiglu_bwd")) return rc;
   const int T = p->T, d = p->d, f = p->f, tile = p->gemm_tile - 1;
@@ -642,9 +650,7 @@ int swiglu_bwd(const ra_swiglu_params* p, hipStream_t s) {
   GemmArgs g{(const uint16_t*)p->da, (const uint16_t*)p->w1, (const uint16_t*)p->db, (const uint16_t*)p->w3,
              p->dx, T, d, f, 0, 0};
   if (int rc = gemm_dispatch(g, 0, 1, tile, s)) return rc;                                  // dx
-  if (int rc = gemm_bf16(p->x, p->da, p->dw1, d, f, T, 1, 0, RA_F32, 1, tile, s)) return rc;
-  if (int rc = gemm_bf16(p->x, p->db, p->dw3, d, f, T, 1, 0, RA_F32, 1, tile, s)) return rc;
-  return gemm_bf16(p->h, p->dy, p->dw2, f, d, T, 1, 0, RA_F32, 1, tile, s);
+  return p->defer_weight_grads ? RA_OK : swiglu_weight_grads(p, s);
 }
 
 }  // namespace ra

@@ -217,3 +217,32 @@ def test_blockwise_feedforward_policies_give_the_same_bits():
     # no gradient wanted: nothing is kept
     with torch.no_grad():
         assert torch.equal(ra.blockwise_feedforward(ff, x, chunk, policy="save_preactivations"), base[0])
+
+
+def test_weight_gradients_of_grouped_launches():
+    """weight_grad_chunks: the weight-gradient products of two (three, all) consecutive chunks in one launch each.
+    y and dx are the same bits as with one launch per chunk; the weight gradients are the same sums in another fp32
+    order (bar: relative L2 1e-2 against fp32 autograd, and 1e-3 against the per-chunk launches).  Seven chunks, so
+    that the last group is short."""
+    S, d, f, chunk = 7 * 256, 256, 512, 256
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(1, S, d, generator=g).bfloat16().to(DEV)
+    dy = torch.randn(1, S, d, generator=g).bfloat16().to(DEV)
+    ff = ra.SwiGLU(d, f, device=DEV, init_std=0.05)
+    res = {}
+    for grp in (1, 2, 3, 7, 100):
+        for prm in ff.parameters():
+            prm.grad = None
+        xd = x.clone().requires_grad_(True)
+        y = ra.blockwise_feedforward(ff, xd, chunk, weight_grad_chunks=grp)
+        y.backward(dy)
+        res[grp] = (y.detach(), xd.grad, ff.w1.grad.clone(), ff.w2.grad.clone(), ff.w3.grad.clone())
+    w1, w2, w3 = (w.detach().float().cpu().requires_grad_(True) for w in (ff.w1, ff.w2, ff.w3))
+    xr = x.float().cpu().requires_grad_(True)
+    O.swiglu(xr, w1, w2, w3).backward(dy.float().cpu())
+    for grp, val in res.items():
+        assert torch.equal(val[0], res[1][0]) and torch.equal(val[1], res[1][1]), grp
+        for i, ref in ((2, w1.grad), (3, w2.grad), (4, w3.grad)):
+            rel_ok(val[i], ref, "dw group %d" % grp)
+            assert errors(val[i], res[1][i])[1] < 1e-3, grp
+    assert torch.equal(res[7][2], res[100][2])          # a group beyond the scan is the whole scan
