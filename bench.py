@@ -540,18 +540,22 @@ def bench_ffn(args):
         shared = {"tokens_per_launch": ra.feedforward._slab_tokens(chunk, T // chunk, 16384),
                   "ms_per_step": round(ms_sh, 3), "value": round(flops / (ms_sh * 1e-3) / 1e12, 2), "unit": "TFLOP/s"}
     value = flops / (ms * 1e-3) / 1e12
-    # dominant kernel: the GEMM a = x w1 of one launch (tokens_per_launch x hidden x intermediate), timed alone
+    # dominant kernel: the launch that computes a = x w1 and b = x w3 together over the tile columns of both (a third
+    # of the step's time by the kernel trace), timed alone on one launch's tokens
+    from ringattention_amd.feedforward import gemm_bf16_pair
     slab = ra.feedforward._slab_tokens(chunk, T // chunk, args.ffn_launch_tokens or None)
     xs = x.detach()[0, :slab]
     a_out = torch.empty(slab, f, dtype=torch.bfloat16, device=dev)
-    gemm_ms = _event_ms(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out), 5)
-    gemm_tf = 2.0 * slab * d * f / (gemm_ms * 1e-3) / 1e12
-    # the tile kernel the library picks for (slab, f): 256 x 256 or 256 x 128 over four wavefronts, whichever takes
-    # fewer rounds of 256 CUs weighted by the cost of a round (1.72 : 1); the shapes here divide both
-    r256 = math.ceil((slab // 256) * (f // 256) / 256.0) * 1.72
-    r128 = math.ceil((slab // 256) * (f // 128) / 256.0) * 1.0
+    b_out = torch.empty(slab, f, dtype=torch.bfloat16, device=dev)
+    pair = lambda: gemm_bf16_pair(xs, ff.w1.detach(), ff.w3.detach(), a_out, b_out)
+    gemm_ms = _event_ms(pair, 5)
+    gemm_tf = 4.0 * slab * d * f / (gemm_ms * 1e-3) / 1e12
+    # the tile kernel the library picks for the pair (slab, 2 f): 256 x 256 or 256 x 128 over four wavefronts, whichever
+    # takes fewer rounds of 256 CUs weighted by the cost of a round (1.72 : 1); the shapes here divide both
+    r256 = math.ceil((slab // 256) * (2 * f // 256) / 256.0) * 1.72
+    r128 = math.ceil((slab // 256) * (2 * f // 128) / 256.0) * 1.0
     gemm_name = "gemm_bf16_w4_kernel<false, false, %d>" % (256 if r256 <= r128 else 128)
-    sclk = None if args.no_extras else _sclk_under_load(lambda: ra.gemm_bf16(xs, ff.w1.detach(), out=a_out))
+    sclk = None if args.no_extras else _sclk_under_load(pair)
     cpu = None
     if not args.no_cpu:
         from oracle import ringattention_oracle as O
@@ -576,14 +580,14 @@ def bench_ffn(args):
                    "policy": args.ffn_policy, "preactivations": "kept (%.1f GB)" % (4e-9 * T * f) if kept else "recomputed",
                    "flop_convention": "6*T*d*f fwd + 12*T*d*f bwd, recompute not counted"},
         "launch_tokens_16384": shared,
-        "roofline": {"bound": "mfma", "kernel": "%s (a = x w1 of one launch)" % gemm_name,
+        "roofline": {"bound": "mfma", "kernel": "%s (a = x w1 and b = x w3 of one launch of %d tokens)" % (gemm_name, slab),
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
                      "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("gemm_bf16_w4_kernel<false,false,256>")
                                  if (T, slab) == (65536, 16384) else None),
                      "mfma_util_pmc": {"kernel": (_measured(MFMA_PROFILE, "mfma_util").get(
                                            "gemm_bf16_w4_kernel<false,false,256>" if slab == 16384
-                                           else "ffn2048:gemm_bf16_w4_kernel<false,false,128>")
+                                           else "ffn2048:gemm_bf16_w4_kernel<false,false,256>")
                                                   if T == 65536 and slab in (2048, 16384) else None),
                                        "source": "profiles/" + MFMA_PROFILE},
                      "kernel_ms": {gemm_name: round(gemm_ms, 3)},

@@ -26,6 +26,13 @@ int ra_attn_bwd_ring_step_part(const ra_attn_bwd_params* p, const ra_ring_step* 
 int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t N, int32_t K, int32_t trans_a,
                       int32_t trans_b, int32_t c_dtype, int32_t beta_one, int32_t tile, ra_stream_t stream);
 
+/* C1 = A B1 and C2 = A B2 (all row-major bf16, C (M, N)) as ONE launch over the tile columns of both products: how
+ * ra_swiglu_fwd / ra_swiglu_bwd compute a = x w1 and b = x w3 (ringattention_jax.py:340-350 scans a feed-forward
+ * whose first two products share their input).  tile as in ra_gemm_bf16_tile; shapes the four-wavefront tile
+ * kernels do not take run as two launches. */
+int ra_gemm_bf16_pair(const void* A, const void* B1, const void* B2, void* C1, void* C2, int32_t M, int32_t N,
+                      int32_t K, int32_t tile, ra_stream_t stream);
+
 /* What the matrix pipes sustain on bf16 MFMAs alone (v_mfma_f32_32x32x16_bf16, four independent accumulators per
  * wavefront, four wavefronts per workgroup): every wavefront issues 64 * iters instructions of 32768 FLOP each.
  * operands 0: one value everywhere; 1: a value per lane, the same in every instruction; 2: random values, consecutive

@@ -148,6 +148,7 @@ SYMBOLS = {
     # measurement / test hooks
     "ra_attn_bwd_block_part": (C.c_int, [C.POINTER(RaAttnBwdParams), i32, vp]),
     "ra_attn_bwd_ring_step_part": (C.c_int, [C.POINTER(RaAttnBwdParams), C.POINTER(RaRingStep), i32, vp]),
+    "ra_gemm_bf16_pair": (C.c_int, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "ra_gemm_bf16_tile": (C.c_int, [vp, vp, vp, i32, i32, i32, i32, i32, i32, i32, i32, vp]),
 }
 # libringattn_probe.so: the MFMA rate probe of the benchmark, kept out of the product library

@@ -47,6 +47,8 @@ int swiglu_weight_grads(const ra_swiglu_params* p, hipStream_t s);
 int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta, int tb, int c_dtype,
               int beta_one, int tile, hipStream_t s);
 
+int gemm_bf16_pair(const void* A, const void* B1, const void* B2, void* C1, void* C2, int M, int N, int K, int tile,
+                   hipStream_t s);
 int rope_kv_append(const ra_rope_append_params* p, hipStream_t s);
 int rmsnorm_fwd(const ra_rmsnorm_params* p, hipStream_t s);
 int rmsnorm_bwd(const ra_rmsnorm_params* p, hipStream_t s);
@@ -490,6 +492,14 @@ int ra_gemm_bf16_tile(const void* A, const void* Bm, void* C, int32_t M, int32_t
   RA_REQUIRE(c_dtype == RA_F32 || c_dtype == RA_BF16, RA_ERR_UNSUPPORTED, "gemm_bf16_tile: c_dtype %d", c_dtype);
   RA_REQUIRE(tile >= -1 && tile <= 3, RA_ERR_INVALID, "gemm_bf16_tile: tile %d outside [-1, 3]", tile);
   return gemm_bf16(A, Bm, C, M, N, K, trans_a, trans_b, c_dtype, beta_one, tile, (hipStream_t)stream);
+}
+
+int ra_gemm_bf16_pair(const void* A, const void* B1, const void* B2, void* C1, void* C2, int32_t M, int32_t N,
+                      int32_t K, int32_t tile, ra_stream_t stream) {
+  RA_REQUIRE(A && B1 && B2 && C1 && C2, RA_ERR_INVALID, "gemm_bf16_pair: null pointer");
+  RA_REQUIRE(M > 0 && N > 0 && K > 0, RA_ERR_INVALID, "gemm_bf16_pair: empty shape");
+  RA_REQUIRE(tile >= -1 && tile <= 3, RA_ERR_INVALID, "gemm_bf16_pair: tile %d outside [-1, 3]", tile);
+  return gemm_bf16_pair(A, B1, B2, C1, C2, M, N, K, tile, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -557,7 +557,7 @@ int gemm_bf16(const void* A, const void* B, void* C, int M, int N, int K, int ta
 
 // C1 = A B1 and C2 = A B2 (both (M, N), row-major, bf16 out), in one launch where the 4-wavefront tile kernels take
 // the shape, else one after the other.  Same bits either way: a tile is computed the same whichever launch holds it.
-static int gemm_bf16_pair(const void* A, const void* B1, const void* B2, void* C1, void* C2, int M, int N, int K,
+int gemm_bf16_pair(const void* A, const void* B1, const void* B2, void* C1, void* C2, int M, int N, int K,
                           int tile, hipStream_t s) {
   if (M % 256 == 0 && N % 128 == 0 && K % GBK == 0 && w4_reach_ok(M, N, K)) {
     int t = tile >= 0 ? tile : pick_tile(M, 2 * N, K);

@@ -260,3 +260,17 @@ def gemm_bf16(A, B, trans_a=False, trans_b=False, out_dtype=torch.bfloat16, out=
                                            int(trans_b), cd, int(accumulate), int(tile), _stream()),
                 "ra_gemm_bf16_tile")
     return out
+
+
+def gemm_bf16_pair(A, B1, B2, out1=None, out2=None, tile=None):
+    """C1 = A B1 and C2 = A B2 in one launch (ra_gemm_bf16_pair: how the SwiGLU kernels compute x w1 and x w3;
+    exposed for tests and the benchmark)."""
+    M, K = A.shape
+    N = B1.shape[1]
+    if out1 is None:
+        out1 = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    if out2 is None:
+        out2 = torch.empty((M, N), dtype=torch.bfloat16, device=A.device)
+    L.check(L.load().ra_gemm_bf16_pair(A.data_ptr(), B1.data_ptr(), B2.data_ptr(), out1.data_ptr(), out2.data_ptr(),
+                                       M, N, K, -1 if tile is None else int(tile), _stream()), "ra_gemm_bf16_pair")
+    return out1, out2

@@ -246,3 +246,19 @@ def test_weight_gradients_of_grouped_launches():
             rel_ok(val[i], ref, "dw group %d" % grp)
             assert errors(val[i], res[1][i])[1] < 1e-3, grp
     assert torch.equal(res[7][2], res[100][2])          # a group beyond the scan is the whole scan
+
+
+@pytest.mark.parametrize("shape,tile", [((2048, 1536, 512), None), ((512, 768, 256), 0), ((512, 640, 192), 3), ((384, 256, 128), None)])
+def test_gemm_pair_equals_two_launches_bitwise(shape, tile):
+    """a = x w1 and b = x w3 as one launch over the tile columns of both: the bits of the two separate launches (a tile
+    is computed the same whichever launch holds it), including a shape the four-wavefront kernels do not take."""
+    from ringattention_amd.feedforward import gemm_bf16_pair
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M + N)
+    A = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    B1 = torch.randn(K, N, generator=g).bfloat16().to(DEV)
+    B2 = torch.randn(K, N, generator=g).bfloat16().to(DEV)
+    c1, c2 = gemm_bf16_pair(A, B1, B2, tile=tile)
+    assert torch.equal(c1, ra.gemm_bf16(A, B1, tile=tile)) and torch.equal(c2, ra.gemm_bf16(A, B2, tile=tile))
+    rel_ok(c1, A.float() @ B1.float(), "pair c1")
+    rel_ok(c2, A.float() @ B2.float(), "pair c2")
