@@ -78,27 +78,29 @@ def _document_dense_check(q, k, v, do, bias, ids, out, grads, heads, tag):
     starts = torch.nonzero(torch.cat([torch.ones(1, dtype=torch.bool, device=ids.device), ids[1:] != ids[:-1]]))[:, 0]
     ends = torch.cat([starts[1:], torch.tensor([S], device=ids.device)])
     lens = (ends - starts).tolist()
-    # a document of 1500..5000 positions that crosses a multiple of 16384 (a shard boundary of the ring of 8) if
-    # there is one, else the first of that length
-    pick = None
-    for s0, ln in zip(starts.tolist(), lens):
-        if 1500 <= ln <= 5000:
-            crosses = (s0 // 16384) != ((s0 + ln - 1) // 16384)
-            if pick is None or (crosses and not pick[2]):
-                pick = (s0, ln, crosses)
-    assert pick is not None
-    s0, ln, crosses = pick
-    sl = slice(s0, s0 + ln)
+    # documents of 1500..5000 positions: one that crosses a multiple of 16384 (a shard boundary of the ring of 8) if
+    # there is one, the first one that lies inside a shard, and the last one of the sequence of that length
+    docs = [(s0, ln, (s0 // 16384) != ((s0 + ln - 1) // 16384)) for s0, ln in zip(starts.tolist(), lens) if 1500 <= ln <= 5000]
+    assert docs
+    picks = []
+    for want in (lambda d: d[2], lambda d: not d[2]):
+        hit = [d for d in docs if want(d)]
+        if hit:
+            picks.append(hit[0])
+    if docs[-1] not in picks:
+        picks.append(docs[-1])
     hs = list(heads)
-    qd, kd, vd = (t[:, sl][:, :, hs].double().cpu().requires_grad_(True) for t in (q, k, v))
-    kw = oracle_kwargs(kwargs(ln, ln, 1))
-    ref = O.dense_attention(qd, kd, vd, bias[..., sl].double().cpu(), None, None, 1, kw)
-    ref.backward(do[:, sl][:, :, hs].double().cpu())
-    rows = [("out",) + assert_close(out[:, sl][:, :, hs], ref.detach(), torch.bfloat16, tag + " out")]
-    for name, a, b in zip(("dq", "dk", "dv"), grads, (qd.grad, kd.grad, vd.grad)):
-        rows.append((name,) + assert_close(a[:, sl][:, :, hs], b, torch.bfloat16, tag + " " + name))
-    print(tag, "document at %d, %d positions, crosses a shard boundary: %s;" % (s0, ln, crosses),
-          "; ".join("%s max-abs %.2e rel-L2 %.2e" % r for r in rows), flush=True)
+    for s0, ln, crosses in picks:
+        sl = slice(s0, s0 + ln)
+        qd, kd, vd = (t[:, sl][:, :, hs].double().cpu().requires_grad_(True) for t in (q, k, v))
+        kw = oracle_kwargs(kwargs(ln, ln, 1))
+        ref = O.dense_attention(qd, kd, vd, bias[..., sl].double().cpu(), None, None, 1, kw)
+        ref.backward(do[:, sl][:, :, hs].double().cpu())
+        rows = [("out",) + assert_close(out[:, sl][:, :, hs], ref.detach(), torch.bfloat16, tag + " out")]
+        for name, a, b in zip(("dq", "dk", "dv"), grads, (qd.grad, kd.grad, vd.grad)):
+            rows.append((name,) + assert_close(a[:, sl][:, :, hs], b, torch.bfloat16, tag + " " + name))
+        print(tag, "document at %d, %d positions, crosses a shard boundary: %s;" % (s0, ln, crosses),
+              "; ".join("%s max-abs %.2e rel-L2 %.2e" % r for r in rows), flush=True)
 
 
 def _sampled_rows_check(q, k, v, do, bias, ids, out, dq, n_rows, seed, tag):
@@ -128,8 +130,8 @@ def _sampled_rows_check(q, k, v, do, bias, ids, out, dq, n_rows, seed, tag):
 
 def test_packed_documents_131k_ring8_full_size():
     """B1 H32 S131072 D128 bf16, 8 virtual shards of 16384, document ids and a bias: the whole configuration,
-    forward and backward.  (1) one document (two heads) against the oracle's dense closed form and its autograd in
-    float64; (2) 64 random rows of out and dq recomputed from the definition in float64; (3) a ring of 8 agrees with
+    forward and backward.  (1) up to three documents (one across a shard boundary, one inside a shard, the last one; two
+    heads) against the oracle's dense closed form and its autograd in float64: out, dq, dk and dv; (2) 64 random rows of out and dq recomputed from the definition in float64; (3) a ring of 8 agrees with
     one device on out / dq / dk / dv; (4) documents are isolated bitwise in the gradients too: changing one
     document's keys, values and cotangents changes no other document's dq, dk or dv."""
     B, S, H, D, n = 1, 131072, 32, 128, 8
