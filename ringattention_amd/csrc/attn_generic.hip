@@ -602,7 +602,8 @@ static int launch_fwd_T(const GenericArgs& a, hipStream_t s) {
     case 32: attn_fwd_generic_kernel<T, 32><<<grid, block, 0, s>>>(a); break;
     case 64: attn_fwd_generic_kernel<T, 64><<<grid, block, 0, s>>>(a); break;
     case 128: attn_fwd_generic_kernel<T, 128><<<grid, block, 0, s>>>(a); break;
-    default: set_error("generic attention: head size %d not in {32,64,128}", a.D); return RA_ERR_UNSUPPORTED;
+    case 256: attn_fwd_generic_kernel<T, 256><<<grid, block, 0, s>>>(a); break;      // row vectors partly in scratch memory
+    default: set_error("generic attention: head size %d not in {32,64,128,256}", a.D); return RA_ERR_UNSUPPORTED;
   }
   RA_CHECK_LAUNCH("attn_fwd_generic");
   return RA_OK;
@@ -628,7 +629,8 @@ static int launch_bwd_T(const GenericArgs& a, hipStream_t s) {
     case 32: launch_bwd_TD<T, 32>(a, s); break;
     case 64: launch_bwd_TD<T, 64>(a, s); break;
     case 128: launch_bwd_TD<T, 128>(a, s); break;
-    default: set_error("generic attention: head size %d not in {32,64,128}", a.D); return RA_ERR_UNSUPPORTED;
+    case 256: launch_bwd_TD<T, 256>(a, s); break;
+    default: set_error("generic attention: head size %d not in {32,64,128,256}", a.D); return RA_ERR_UNSUPPORTED;
   }
   RA_CHECK_LAUNCH("attn_bwd_generic");
   return RA_OK;

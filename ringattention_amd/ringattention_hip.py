@@ -794,18 +794,22 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
 
 
 def _mfma_head_size(cfg, mi, q):
-    """The head size (64 or 128) to zero-pad q, k, v to so that the matrix-core kernels take a call whose own head
-    size they do not tile, or 0: when the head size is 64 or 128 already or above 128, when the generic kernels were
-    asked for, or when something else keeps the call on them anyway (chunk sizes off the 128-grid, a per-row bias, an
-    unpacked boolean mask), where padding would only add work."""
+    """The head size to zero-pad q, k, v to (the products are those of the un-padded rows; the logits keep the scale
+    of the original head size), or 0 when the kernels take the head size as it is.  The matrix-core kernels tile 64
+    and 128, the generic ones 32, 64, 128 and 256: a call that stays on the generic kernels anyway (they were asked
+    for, chunk sizes off the 128-grid, a per-row bias, an unpacked boolean mask, a head size above 128) is padded to
+    the next of those, any other to 64 or 128."""
     D = q.shape[3]
-    if D in (64, 128) or D > 128 or cfg.impl == L.RA_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float32):
-        return 0
-    if cfg.qc % 128 or cfg.kc % 128 or (mi.bias is not None and mi.bias_strides[2] != 0):
-        return 0
-    if mi.keep is not None and mi.keep_packed is None:
-        return 0
-    return 64 if D < 64 else 128
+    if D > 256:
+        raise NotImplementedError("head size %d: the kernels take head sizes up to 256" % D)
+    generic = (cfg.impl == L.RA_IMPL_GENERIC or D > 128 or q.dtype not in (torch.bfloat16, torch.float32)
+               or cfg.qc % 128 or cfg.kc % 128 or (mi.bias is not None and mi.bias_strides[2] != 0)
+               or (mi.keep is not None and mi.keep_packed is None))
+    if generic:
+        to = next(s for s in (32, 64, 128, 256) if D <= s)
+    else:
+        to = 64 if D <= 64 else 128
+    return 0 if to == D else to
 
 
 def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=128):

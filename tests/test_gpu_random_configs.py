@@ -1,0 +1,79 @@
+"""Seeded random configurations of ring_attention, HIP (through the C-ABI) against the CPU oracle.
+
+The hand-picked cases of the other files follow the kernels' known seams; these draw the whole argument space of
+ringattention_jax.py:17-97 at once - input type, head size, ring size, chunk sizes on and off the matrix-core grid,
+causal block size or none, bias broadcast or per head / batch / row, packed segment ids, unequal query and key
+lengths - so that a combination nobody thought of still meets the oracle.  Same bar as everywhere: max-abs 1e-4
+(fp32 inputs) or 2e-2 (bf16 / fp16 inputs; widened in proportion once the reference holds elements above 4, where
+rounding the result to 16 bits alone exceeds it), relative L2 1e-2, NaN rows coinciding.
+"""
+import random
+
+import pytest
+import torch
+
+import ringattention_amd as ra
+from tests.test_gpu_attention import run_hip
+from tests.util import assert_close_scaled, kwargs, make_qkv, oracle_fwd_bwd, packed_segment_ids
+
+pytestmark = pytest.mark.gpu
+
+N_CASES = 160
+
+
+def draw(seed):
+    r = random.Random(1000 + seed)
+    dtype = r.choice([torch.float32, torch.bfloat16, torch.bfloat16, torch.float16])
+    D = r.choice([16, 32, 40, 64, 64, 80, 96, 128, 128, 128, 160, 256])
+    n = r.choice([1, 1, 2, 2, 4, 8])
+    on_grid = r.random() < 0.6                      # chunk sizes the matrix-core kernels tile as they are
+    if on_grid:
+        qc, kc = r.choice([128, 128, 256]), r.choice([128, 128, 256])
+    else:
+        qc, kc = r.choice([8, 16, 32, 48, 64, 96]), r.choice([8, 16, 32, 48, 64, 96])
+    # per-device lengths: multiples of both chunk sizes, the whole ring at most 2048 positions
+    unit = qc * kc // __import__("math").gcd(qc, kc)
+    per_dev_max = max(unit, (2048 // n) // unit * unit)
+    q_len = unit * r.randint(1, max(1, min(4, per_dev_max // unit)))
+    kv_len = q_len
+    if n == 1 and r.random() < 0.3:                 # cross-length attention (one device only: a ring rotates equal shards)
+        kv_len = unit * r.randint(1, max(1, min(4, per_dev_max // unit)))
+    cbs = r.choice([1, 1, 1, None, 2, 8, 32, 128])
+    if cbs not in (None, 1) and (max(cbs, qc) % min(cbs, qc) or max(cbs, kc) % min(cbs, kc)):
+        cbs = 1                                     # :327-330 divide block size and chunk sizes by one another
+    B, H = r.choice([1, 1, 2]), r.choice([1, 2, 3])
+    bias = r.choice([None, None, "key", "key", "head", "row"])
+    seg = r.choice([None, "docs", "docs", "one"])
+    return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cbs=cbs, B=B, H=H, bias=bias, seg=seg)
+
+
+@pytest.mark.parametrize("seed", range(N_CASES))
+def test_random_configuration_matches_oracle(seed):
+    c = draw(seed)
+    print("case", seed, c, flush=True)
+    n, B, H, D = c["n"], c["B"], c["H"], c["D"]
+    S, Skv = n * c["q_len"], n * c["kv_len"]
+    q, k, v, do = make_qkv(B, S, H, D, dtype=c["dtype"], seed=seed, Skv=Skv)
+    g = torch.Generator().manual_seed(seed + 500)
+    bias = None
+    if c["bias"] == "key":
+        bias = torch.randn(1, 1, 1, Skv, generator=g)
+    elif c["bias"] == "head":
+        bias = torch.randn(B, H, 1, Skv, generator=g)
+    elif c["bias"] == "row":                        # :279-283: rows 0:qc of the bias serve every query chunk
+        bias = torch.randn(1, H, c["qc"], Skv, generator=g)
+    seg = None
+    if c["seg"] == "docs":
+        seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7)
+    elif c["seg"] == "one":
+        seg = torch.zeros(B, max(S, Skv), dtype=torch.int32)
+    kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    print("  family", ra.kernel_family_of_last_call(), flush=True)
+    tol_dtype = torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16
+    assert out.dtype == c["dtype"] and out.shape == q.shape
+    assert_close_scaled(out, ref_out, tol_dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert a.dtype == c["dtype"]
+        assert_close_scaled(a, b, tol_dtype, name)
