@@ -77,3 +77,59 @@ def test_random_configuration_matches_oracle(seed):
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
         assert a.dtype == c["dtype"]
         assert_close_scaled(a, b, tol_dtype, name)
+
+
+def draw_cache(seed):
+    r = random.Random(5000 + seed)
+    dtype = r.choice([torch.float32, torch.bfloat16, torch.bfloat16, torch.float16])
+    D = r.choice([32, 64, 64, 80, 128, 128, 128, 256])
+    n = r.choice([1, 1, 1, 2, 4])
+    qc = r.choice([1, 1, 1, 1, 2, 4, 16])
+    kc = r.choice([16, 32, 64, 128, 512])
+    q_len = qc * r.choice([1, 1, 2])                 # query tokens per device
+    kv_len = kc * r.randint(1, max(1, 2048 // (n * kc)))
+    L = n * kv_len
+    edge = r.random()
+    if edge < 0.15:
+        cache_idx = r.choice([0, 1, L - 1])
+    elif edge < 0.45:
+        cache_idx = min(L - 1, kc * r.randint(0, L // kc))        # the skip predicate's edge (:324-331)
+    else:
+        cache_idx = r.randint(0, L - 1)
+    cbs = r.choice([1, 1, 1, None])
+    B, H = r.choice([1, 2, 3]), r.choice([1, 2, 5])
+    bias = r.choice([None, None, "key", "head"])
+    seg = r.choice([None, None, "docs"])
+    device_idx = r.random() < 0.5                     # cache_idx as a device scalar (a traced value under jit)
+    return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cache_idx=cache_idx, cbs=cbs, B=B, H=H,
+                bias=bias, seg=seg, device_idx=device_idx)
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_random_cache_idx_configuration_matches_oracle(seed):
+    """The cache_idx path (ringattention_jax.py:31-35, :72-73): the query tokens sit at global positions
+    (cache_idx // query_chunk_size) * query_chunk_size + row, the keys are the whole cache."""
+    from oracle import ringattention_oracle as O
+    from tests.util import oracle_kwargs
+    c = draw_cache(seed)
+    print("cache case", seed, c, flush=True)
+    n, B, H, D = c["n"], c["B"], c["H"], c["D"]
+    S, L = n * c["q_len"], n * c["kv_len"]
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=c["dtype"], seed=seed, Skv=L)
+    g = torch.Generator().manual_seed(seed + 900)
+    bias = None
+    if c["bias"] == "key":
+        bias = torch.randn(1, 1, 1, L, generator=g)
+    elif c["bias"] == "head":
+        bias = torch.randn(B, H, 1, L, generator=g)
+    seg = packed_segment_ids(B, L, max(4, L // 3), seed=seed + 3) if c["seg"] == "docs" else None
+    kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32)
+    ref = O.ring_attention(q, k, v, bias, seg, c["cache_idx"], n, True, oracle_kwargs(kw))
+    ci = torch.tensor(c["cache_idx"], dtype=torch.int32, device="cuda") if c["device_idx"] else c["cache_idx"]
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention(q.cuda(), k.cuda(), v.cuda(), bias.cuda() if bias is not None else None,
+                               seg.cuda() if seg is not None else None, ci, axis_name="sp", float32_logits=True,
+                               blockwise_kwargs=kw)
+    torch.cuda.synchronize()
+    assert out.dtype == c["dtype"] and out.shape == q.shape
+    assert_close_scaled(out, ref, torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16, "out")
