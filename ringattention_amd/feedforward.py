@@ -176,6 +176,9 @@ def _slab_tokens(chunk_size, n_chunks, launch_tokens=None):
     return chunk_size * g
 
 
+_TOKEN_GRID = 128       # tokens per launch are a multiple of this (rows of a GEMM tile)
+
+
 class SwiGLU(torch.nn.Module):
     """The LLaMA-style MLP the reference's README pairs with blockwise_feedforward:
     w2(silu(x w1) * (x w3)); weights stored (in, out), bf16."""
@@ -197,7 +200,10 @@ class SwiGLU(torch.nn.Module):
             raise NotImplementedError("SwiGLU kernels are bf16")
         if not x.is_cuda:
             raise RuntimeError("ringattention_amd runs on the GPU only")
-        y = _SwiGLUFn.apply(x.contiguous(), self.w1, self.w2, self.w3, self.gemm_tile)
+        T = x.shape[0]
+        if T % _TOKEN_GRID:         # the GEMM tiles want whole groups of 128 tokens: zero rows, dropped again below
+            x = torch.nn.functional.pad(x, (0, 0, 0, _TOKEN_GRID - T % _TOKEN_GRID))
+        y = _SwiGLUFn.apply(x.contiguous(), self.w1, self.w2, self.w3, self.gemm_tile)[:T]
         return y.reshape(*shp[:-1], y.shape[-1])
 
 
@@ -208,7 +214,8 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
     The reference groups tokens with 'b (c n) d -> b c n d', c=chunk_size and scans over n, so step
     j sees the strided token set {ci * n + j}.  A generic callable gets exactly those groups.  A
     ``SwiGLU`` instance is token-wise, so it is fed contiguous slabs of chunk_size tokens instead:
-    the same number of steps and the same result, with dense memory access.  ``policy`` selects what the
+    the same number of steps and the same result, with dense memory access (a chunk size that is not a multiple of
+    128 is rounded up to one: fewer, slightly larger steps over the same tokens).  ``policy`` selects what the
     SwiGLU scan keeps for its backward pass: the reference's default ``nothing_saveable`` recomputes the
     pre-activations, ``"save_preactivations"`` is the opt-in that keeps them (see _save_preactivations).
     ``launch_tokens`` (no counterpart in the reference) lets consecutive chunks share a kernel launch and its
@@ -232,11 +239,20 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
             raise RuntimeError("ringattention_amd runs on the GPU only")
         # contiguous slabs of chunk_size tokens (batch rows one after the other: a token-wise MLP does not see the
         # difference), one autograd node for the whole scan
-        slab = _slab_tokens(chunk_size, b * n, launch_tokens)
-        y = _BlockwiseSwiGLUFn.apply(inputs.reshape(b * s, d).contiguous(), feedforward.w1, feedforward.w2,
+        x2 = inputs.reshape(b * s, d)
+        step, steps = chunk_size, b * n
+        if chunk_size % _TOKEN_GRID:
+            # a chunk size the GEMM tiles do not divide: the same tokens in steps of the next multiple of 128, the
+            # last one filled up with zero rows that are dropped again (tokens are independent, zero rows add
+            # nothing to the weight gradients)
+            step = -(-chunk_size // _TOKEN_GRID) * _TOKEN_GRID
+            steps = -(-b * s // step)
+            x2 = torch.nn.functional.pad(x2, (0, 0, 0, steps * step - b * s))
+        slab = _slab_tokens(step, steps, launch_tokens)
+        y = _BlockwiseSwiGLUFn.apply(x2.contiguous(), feedforward.w1, feedforward.w2,
                                      feedforward.w3, slab, _save_preactivations(policy), feedforward.gemm_tile,
-                                     max(1, int(weight_grad_chunks) * chunk_size // slab))
-        return y.reshape(b, s, y.shape[-1])
+                                     max(1, int(weight_grad_chunks) * step // slab))
+        return y[:b * s].reshape(b, s, y.shape[-1])
     x = inputs.reshape(b, chunk_size, n, d)
     outs = [feedforward(x[:, :, j, :]) for j in range(n)]
     out = torch.stack(outs, dim=2)

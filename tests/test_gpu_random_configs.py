@@ -133,3 +133,53 @@ def test_random_cache_idx_configuration_matches_oracle(seed):
     torch.cuda.synchronize()
     assert out.dtype == c["dtype"] and out.shape == q.shape
     assert_close_scaled(out, ref, torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16, "out")
+
+
+def draw_ffn(seed):
+    r = random.Random(9000 + seed)
+    d = 128 * r.choice([1, 1, 2, 3])
+    f = 128 * r.choice([1, 2, 3, 5, 7])
+    chunk = r.choice([8, 40, 100, 128, 128, 200, 256, 384, 512])
+    n = r.randint(1, 6)                              # scan steps
+    b = r.choice([1, 1, 2, 3])
+    policy = r.choice([None, "nothing_saveable", "save_preactivations"])
+    launch = r.choice([None, None, 512, 1024])
+    group = r.choice([1, 2, 4, 4])
+    tile = r.choice([None, None, None, 0, 1, 2, 3])
+    if d % 256 or f % 256 or chunk % 256:
+        tile = None                                   # a forced tile kernel wants its own multiples
+    return dict(d=d, f=f, chunk=chunk, n=n, b=b, policy=policy, launch=launch, group=group, tile=tile)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_blockwise_feedforward_matches_oracle(seed):
+    """blockwise_feedforward (ringattention_jax.py:333-352) over a SwiGLU MLP against the oracle's scan and fp32
+    autograd of the oracle's formula, relative L2 1e-2 on y, dx and the three weight gradients: chunk sizes on and
+    off the GEMM's token grid, every policy, shared launches, grouped weight gradients, every tile kernel."""
+    from oracle import ringattention_oracle as O
+    from tests.util import errors
+    c = draw_ffn(seed)
+    print("ffn case", seed, c, flush=True)
+    b, s, d, f = c["b"], c["chunk"] * c["n"], c["d"], c["f"]
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(b, s, d, generator=g).bfloat16()
+    dy = torch.randn(b, s, d, generator=g).bfloat16()
+    ff = ra.SwiGLU(d, f, device="cuda", init_std=0.05, gemm_tile=c["tile"])
+    w1, w2, w3 = (w.detach().float().cpu().requires_grad_(True) for w in (ff.w1, ff.w2, ff.w3))
+    xr = x.float().requires_grad_(True)
+    yr = O.blockwise_feedforward(lambda h: O.swiglu(h, w1, w2, w3), xr, c["chunk"])
+    yr.backward(dy.float())
+    xd = x.cuda().requires_grad_(True)
+    y = ra.blockwise_feedforward(ff, xd, c["chunk"], policy=c["policy"], launch_tokens=c["launch"],
+                                 weight_grad_chunks=c["group"])
+    y.backward(dy.cuda())
+    torch.cuda.synchronize()
+    assert y.shape == yr.shape and y.dtype == torch.bfloat16
+    for name, got, ref in (("y", y, yr), ("dx", xd.grad, xr.grad), ("dw1", ff.w1.grad, w1.grad),
+                           ("dw2", ff.w2.grad, w2.grad), ("dw3", ff.w3.grad, w3.grad)):
+        rel = errors(got, ref)[1]
+        assert rel <= 1e-2, "%s: rel-L2 %.3e" % (name, rel)
+    # the module alone, on a token count off the grid
+    t = 1 + seed * 37 % 300
+    y1 = ff(x.cuda().reshape(-1, d)[:t])
+    assert errors(y1, O.swiglu(x.float().reshape(-1, d)[:t], w1, w2, w3))[1] <= 1e-2
