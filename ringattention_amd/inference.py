@@ -9,14 +9,16 @@ from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, 
                                 _check_qkv, _save_residuals, _saved_residuals, axis_size)
 
 
-def _inference_cfg(q, q_len, kv_len, float32_logits):
+def _inference_cfg(q, q_len, kv_len, float32_logits, logit_dim=0):
     # one "chunk" per ring step (:21 is a single einsum over the shard); finfo.min of the logits' dtype (:22)
     logits_dtype = torch.float32 if (float32_logits or q.dtype == torch.float32) else q.dtype
-    return _Config(dict(causal_block_size=None, query_chunk_size=q_len, key_chunk_size=kv_len, deterministic=True,
-                        attn_pdrop=0.0, dtype=logits_dtype, impl="auto", skip_masked_tiles=False))
+    cfg = _Config(dict(causal_block_size=None, query_chunk_size=q_len, key_chunk_size=kv_len, deterministic=True,
+                       attn_pdrop=0.0, dtype=logits_dtype, impl="auto", skip_masked_tiles=False))
+    cfg.logit_dim = logit_dim       # q, k, v zero-padded along D: the head size that scales the logits (:18)
+    return cfg
 
 
-def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
+def _fwd(q, k, v, attn_mask, axis_name, float32_logits, logit_dim=0):
     _check_qkv(q, k, v)
     q, k, v = (t if (t.stride(3) == 1 and t.stride(2) == t.shape[3]) else t.contiguous() for t in (q, k, v))
     n = axis_size(axis_name)                                                     # :15
@@ -28,7 +30,7 @@ def _fwd(q, k, v, attn_mask, axis_name, float32_logits):
     if attn_mask.dim() != 4 or attn_mask.shape[3] != kv_total or attn_mask.shape[2] not in (1, q_total) or \
             attn_mask.shape[0] not in (1, B) or attn_mask.shape[1] not in (1, H):
         raise ValueError("attn_mask must be (B|1, H|1, Q|1, K) with Q = %d and K = %d" % (q_total, kv_total))
-    cfg = _inference_cfg(q, q_len, kv_len, float32_logits)
+    cfg = _inference_cfg(q, q_len, kv_len, float32_logits, logit_dim)
     mi = _MaskInputs(cfg, None, None, None, B, q.device, kv_total)
     mi.set_keep(attn_mask, q.device, q_total, kv_total)
     if q_len % 64 or kv_len % 64:
@@ -94,18 +96,33 @@ class _RingAttentionInferenceFn(torch.autograd.Function):
     """custom_vjp of ringattention_inference.py:67-73: cotangents for q, k, v; None for the mask (:64)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, attn_mask, axis_name, float32_logits):
-        out, res = _fwd(q, k, v, attn_mask, axis_name, float32_logits)
+    def forward(ctx, q, k, v, attn_mask, axis_name, float32_logits, logit_dim=0):
+        out, res = _fwd(q, k, v, attn_mask, axis_name, float32_logits, logit_dim)
         _save_residuals(ctx, res)
         return out
 
     @staticmethod
     def backward(ctx, g):
         dq, dk, dv = _bwd(_saved_residuals(ctx), g)
-        return dq, dk, dv, None, None, None
+        return dq, dk, dv, None, None, None, None
 
 
 def ring_attention_inference(q, k, v, attn_mask, axis_name, float32_logits=True):
     """ringattention_inference.py:67-70.  q, k, v are the global (B, S, H, D) arrays of the virtual ring
-    declared with ``ring_axis``; attn_mask is the global boolean mask (B|1, H|1, Q|1, K), True = attend."""
-    return _RingAttentionInferenceFn.apply(q, k, v, attn_mask, axis_name, float32_logits)
+    declared with ``ring_axis``; attn_mask is the global boolean mask (B|1, H|1, Q|1, K), True = attend.
+    bf16, fp32 or fp16 (computed on fp32 copies, as ring_attention does); a head size no kernel tiles (they take 64
+    and 128 on the matrix cores, 32, 64, 128 and 256 otherwise) is zero-padded to the next one that is, with the
+    logits still divided by the square root of the original head size."""
+    if q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16:
+        return ring_attention_inference(q.float(), k.float(), v.float(), attn_mask, axis_name,
+                                        float32_logits).to(torch.float16)
+    D = q.shape[-1]
+    if D > 256:
+        raise NotImplementedError("head size %d: the kernels take head sizes up to 256" % D)
+    n = axis_size(axis_name)
+    on_grid = q.shape[1] % (64 * n) == 0 and k.shape[1] % (64 * n) == 0 and D <= 128
+    to = (64 if D <= 64 else 128) if on_grid else next(s for s in (32, 64, 128, 256) if D <= s)
+    if to == D:
+        return _RingAttentionInferenceFn.apply(q, k, v, attn_mask, axis_name, float32_logits)
+    q, k, v = (torch.nn.functional.pad(t, (0, to - D)) for t in (q, k, v))
+    return _RingAttentionInferenceFn.apply(q, k, v, attn_mask, axis_name, float32_logits, D)[..., :D].contiguous()

@@ -183,3 +183,51 @@ def test_random_blockwise_feedforward_matches_oracle(seed):
     t = 1 + seed * 37 % 300
     y1 = ff(x.cuda().reshape(-1, d)[:t])
     assert errors(y1, O.swiglu(x.float().reshape(-1, d)[:t], w1, w2, w3))[1] <= 1e-2
+
+
+def draw_inference(seed):
+    r = random.Random(13000 + seed)
+    dtype = r.choice([torch.float32, torch.bfloat16, torch.bfloat16, torch.float16])
+    D = r.choice([32, 40, 64, 96, 128, 128, 128, 160])
+    n = r.choice([1, 2, 2, 4])
+    per_dev = r.choice([8, 24, 64, 100, 128, 256, 256, 512])
+    B, H = r.choice([1, 2]), r.choice([1, 2, 3])
+    kind = r.choice(["full", "bcast_bh", "key_only", "per_head", "per_batch"])
+    p_keep = r.choice([0.05, 0.5, 0.9])
+    empty_row = r.random() < 0.25                    # a row that attends to nothing: uniform weights (:22-24)
+    causal = r.random() < 0.4
+    return dict(dtype=dtype, D=D, n=n, per_dev=per_dev, B=B, H=H, kind=kind, p_keep=p_keep, empty_row=empty_row,
+                causal=causal)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_inference_configuration_matches_oracle(seed):
+    """ring_attention_inference (ringattention_inference.py:8-73): boolean masks of every broadcast form, sparse
+    and dense, with and without rows that attend to nothing, shards on and off the packed-mask grid."""
+    from oracle import ringattention_oracle as O
+    c = draw_inference(seed)
+    print("inference case", seed, c, flush=True)
+    n, B, H, D = c["n"], c["B"], c["H"], c["D"]
+    S = n * c["per_dev"]
+    q, k, v, do = make_qkv(B, S, H, D, dtype=c["dtype"], seed=seed, scale=D ** -0.25)
+    shape = {"full": (B, H, S, S), "bcast_bh": (1, 1, S, S), "key_only": (B, 1, 1, S), "per_head": (1, H, S, S),
+             "per_batch": (B, 1, S, S)}[c["kind"]]
+    g = torch.Generator().manual_seed(seed + 77)
+    mask = torch.rand(shape, generator=g) < c["p_keep"]
+    if c["causal"] and shape[2] == S:
+        mask = mask & torch.tril(torch.ones(S, S, dtype=torch.bool))
+    mask[..., 0] = True
+    if c["empty_row"] and shape[2] == S:
+        mask[:, :, S // 3, :] = False
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+    ref_grads = O.ring_attention_inference_bwd(n, res, do)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention_inference(qd, kd, vd, mask.cuda(), "sp", True)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+    tol_dtype = torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16
+    assert out.dtype == c["dtype"] and out.shape == q.shape
+    assert_close_scaled(out, ref_out, tol_dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), (qd.grad, kd.grad, vd.grad), ref_grads):
+        assert_close_scaled(a, b, tol_dtype, name)
