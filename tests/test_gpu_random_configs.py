@@ -231,3 +231,47 @@ def test_random_inference_configuration_matches_oracle(seed):
     assert_close_scaled(out, ref_out, tol_dtype, "out")
     for name, a, b in zip(("dq", "dk", "dv"), (qd.grad, kd.grad, vd.grad), ref_grads):
         assert_close_scaled(a, b, tol_dtype, name)
+
+
+def draw_long(seed):
+    r = random.Random(17000 + seed)
+    dtype = r.choice([torch.float32, torch.bfloat16, torch.bfloat16])
+    D = r.choice([64, 128, 128, 96])
+    n = r.choice([1, 2, 4, 8])
+    qc, kc = r.choice([128, 256, 512, 1024]), r.choice([128, 256, 512, 1024])
+    unit = max(qc, kc)
+    S = unit * n * r.randint(1, max(1, 8192 // (unit * n)))
+    cbs = r.choice([1, 1, 1, None, 256, 2048])
+    if cbs not in (None, 1) and (max(cbs, qc) % min(cbs, qc) or max(cbs, kc) % min(cbs, kc)):
+        cbs = 1
+    bias = r.choice([None, "key", "head"])
+    seg = r.choice([None, "docs", "docs", "short"])
+    return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, S=S, cbs=cbs, bias=bias, seg=seg, H=r.choice([1, 2]))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_long_configuration_matches_oracle(seed):
+    """Up to 8192 positions on the matrix-core kernels: loops of many key tiles, the tile buffers coming round, packed
+    documents from a few positions to thousands, whole-ring launches."""
+    c = draw_long(seed)
+    print("long case", seed, c, flush=True)
+    n, H, D, S = c["n"], c["H"], c["D"], c["S"]
+    q, k, v, do = make_qkv(1, S, H, D, dtype=c["dtype"], seed=seed, scale=D ** -0.25)
+    g = torch.Generator().manual_seed(seed + 300)
+    bias = {"key": lambda: torch.randn(1, 1, 1, S, generator=g), "head": lambda: torch.randn(1, H, 1, S, generator=g),
+            None: lambda: None}[c["bias"]]()
+    seg = None
+    if c["seg"] == "docs":
+        seg = packed_segment_ids(1, S, S // 6, seed=seed + 7)
+    elif c["seg"] == "short":
+        seg = packed_segment_ids(1, S, 90, seed=seed + 7)
+    kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    fam = ra.kernel_family_of_last_call()
+    print("  family", fam, flush=True)
+    assert "generic" not in str(fam)
+    tol_dtype = torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16
+    assert_close_scaled(out, ref_out, tol_dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close_scaled(a, b, tol_dtype, name)
