@@ -4,9 +4,10 @@ The hand-picked cases of the other files follow the kernels' known seams; these 
 ringattention_jax.py:17-97 at once - input type, head size, ring size, chunk sizes on and off the matrix-core grid,
 causal block size or none, bias broadcast or per head / batch / row, packed segment ids, unequal query and key
 lengths - so that a combination nobody thought of still meets the oracle.  Same bar as everywhere: max-abs 1e-4
-(fp32 inputs) or 2e-2 (bf16 / fp16 inputs; widened in proportion once the reference holds elements above 4, where
-rounding the result to 16 bits alone exceeds it), relative L2 1e-2, NaN rows coinciding.
+(fp32 inputs) or 2e-2 (bf16 / fp16 inputs; one bf16 unit in the last place of the largest reference element where
+that is more: two roundings a boundary apart differ by that much), relative L2 1e-2, NaN rows coinciding.
 """
+import os
 import random
 
 import pytest
@@ -19,6 +20,8 @@ from tests.util import assert_close_scaled, kwargs, make_qkv, oracle_fwd_bwd, pa
 pytestmark = pytest.mark.gpu
 
 N_CASES = 160
+# RA_TEST_SEED_OFFSET=1000 (say) draws another set of configurations with the same tests
+OFFSET = int(os.environ.get("RA_TEST_SEED_OFFSET", "0"))
 
 
 def draw(seed):
@@ -47,7 +50,7 @@ def draw(seed):
     return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cbs=cbs, B=B, H=H, bias=bias, seg=seg)
 
 
-@pytest.mark.parametrize("seed", range(N_CASES))
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + N_CASES))
 def test_random_configuration_matches_oracle(seed):
     c = draw(seed)
     print("case", seed, c, flush=True)
@@ -105,7 +108,7 @@ def draw_cache(seed):
                 bias=bias, seg=seg, device_idx=device_idx)
 
 
-@pytest.mark.parametrize("seed", range(96))
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + 96))
 def test_random_cache_idx_configuration_matches_oracle(seed):
     """The cache_idx path (ringattention_jax.py:31-35, :72-73): the query tokens sit at global positions
     (cache_idx // query_chunk_size) * query_chunk_size + row, the keys are the whole cache."""
@@ -151,7 +154,7 @@ def draw_ffn(seed):
     return dict(d=d, f=f, chunk=chunk, n=n, b=b, policy=policy, launch=launch, group=group, tile=tile)
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + 48))
 def test_random_blockwise_feedforward_matches_oracle(seed):
     """blockwise_feedforward (ringattention_jax.py:333-352) over a SwiGLU MLP against the oracle's scan and fp32
     autograd of the oracle's formula, relative L2 1e-2 on y, dx and the three weight gradients: chunk sizes on and
@@ -200,7 +203,7 @@ def draw_inference(seed):
                 causal=causal)
 
 
-@pytest.mark.parametrize("seed", range(64))
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + 64))
 def test_random_inference_configuration_matches_oracle(seed):
     """ring_attention_inference (ringattention_inference.py:8-73): boolean masks of every broadcast form, sparse
     and dense, with and without rows that attend to nothing, shards on and off the packed-mask grid."""
@@ -249,7 +252,7 @@ def draw_long(seed):
     return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, S=S, cbs=cbs, bias=bias, seg=seg, H=r.choice([1, 2]))
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + 24))
 def test_random_long_configuration_matches_oracle(seed):
     """Up to 8192 positions on the matrix-core kernels: loops of many key tiles, the tile buffers coming round, packed
     documents from a few positions to thousands, whole-ring launches."""
