@@ -278,3 +278,38 @@ def test_random_long_configuration_matches_oracle(seed):
     assert_close_scaled(out, ref_out, tol_dtype, "out")
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
         assert_close_scaled(a, b, tol_dtype, name)
+
+
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + 64))
+def test_random_dropout_configuration_matches_oracle(seed):
+    """The draws of the first test with attention dropout on (ringattention_jax.py:119-123, :311-321): the mask of the
+    documented Philox stream, seeded by an integer, on both sides; dropped pairs take finfo.min once more, rows may
+    lose every allowed key."""
+    c = draw(seed + 40000)
+    r = random.Random(21000 + seed)
+    p = r.choice([0.1, 0.3, 0.5, 0.9])
+    if c["dtype"] == torch.float16:
+        c["dtype"] = torch.bfloat16
+    c["bias"] = c["bias"] if c["bias"] != "row" else "head"
+    print("dropout case", seed, c, p, flush=True)
+    n, B, H, D = c["n"], c["B"], c["H"], c["D"]
+    S, Skv = n * c["q_len"], n * c["kv_len"]
+    q, k, v, do = make_qkv(B, S, H, D, dtype=c["dtype"], seed=seed, Skv=Skv)
+    g = torch.Generator().manual_seed(seed + 500)
+    bias = None
+    if c["bias"] == "key":
+        bias = torch.randn(1, 1, 1, Skv, generator=g)
+    elif c["bias"] == "head":
+        bias = torch.randn(B, H, 1, Skv, generator=g)
+    seg = None
+    if c["seg"] == "docs":
+        seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7)
+    elif c["seg"] == "one":
+        seg = torch.zeros(B, max(S, Skv), dtype=torch.int32)
+    kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32, deterministic=False, dropout_rng=seed + 1, attn_pdrop=p)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    tol_dtype = torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16
+    assert_close_scaled(out, ref_out, tol_dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close_scaled(a, b, tol_dtype, name)
