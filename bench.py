@@ -331,8 +331,10 @@ def bench_attention(args, ring, dropout=False, c1=False):
         dom = max(kern, key=lambda n_: kern[n_][0])
         dms, dfl = kern[dom]
         ach = dfl / (dms * 1e-3) / 1e12
+        ring_traffic = _measured(TRAFFIC_PROFILE, "traffic").get("ring131k:" + dom) if S == 131072 else None
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": peak, "unit": "TFLOP/s",
-                "frac": round(ach / peak, 4), "traffic": None,
+                "frac": round(ach / peak, 4), "traffic": ring_traffic,
+                "traffic_source": "profiles/" + TRAFFIC_PROFILE if ring_traffic else None,
                 "scope": "the kernel's launches of one pass summed (one per scan step with work, host launch gaps "
                          "included), FLOP of unmasked pairs: 8*D per pair for dK/dV, 2*D for dQ, 4*D forward",
                 "mfma_util_pmc": ({"kernel": util.get("ring131k:" + dom), "step": util.get("ring131k_step"),
@@ -583,8 +585,11 @@ def bench_ffn(args):
         "roofline": {"bound": "mfma", "kernel": "%s (a = x w1 and b = x w3 of one launch of %d tokens)" % (gemm_name, slab),
                      "achieved": round(gemm_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(gemm_tf / PEAK_BF16_TFLOPS, 4),
-                     "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get("gemm_bf16_w4_kernel<false,false,256>")
-                                 if (T, slab) == (65536, 16384) else None),
+                     "traffic": (_measured(TRAFFIC_PROFILE, "traffic").get(
+                                     "gemm_bf16_w4_kernel<false,false,256>" if slab == 16384
+                                     else "ffn2048:gemm_bf16_w4_kernel<false,false,256>")
+                                 if T == 65536 and slab in (2048, 16384) else None),
+                     "traffic_source": "profiles/" + TRAFFIC_PROFILE,
                      "mfma_util_pmc": {"kernel": (_measured(MFMA_PROFILE, "mfma_util").get(
                                            "gemm_bf16_w4_kernel<false,false,256>" if slab == 16384
                                            else "ffn2048:gemm_bf16_w4_kernel<false,false,256>")
