@@ -148,9 +148,11 @@ def test_invalid_shapes_raise():
     q = torch.zeros(1, 100, 1, 64, device=DEV)
     with pytest.raises(ValueError):
         ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1))
-    q = torch.zeros(1, 64, 1, 48, device=DEV)
+    q = torch.zeros(1, 64, 1, 272, device=DEV)       # head sizes above 256: no kernel family
     with pytest.raises(NotImplementedError):
         ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1))
+    q = torch.zeros(1, 64, 1, 48, device=DEV)        # any head size up to 256 runs (zero-padded to one a kernel tiles)
+    assert ra.ringattention(q, q, q, None, None, None, "sp", True, kwargs(32, 32, 1)).shape == q.shape
 
 
 # --------------------------------------------------------------------------- MFMA kernels (bf16, D = 128 or 64)
@@ -588,7 +590,7 @@ def test_fp32_mfma_kernels_agree_with_the_vector_kernels(D, n, cbs, use_seg, use
 
 
 def test_fp32_mfma_kernels_refuse_what_they_do_not_take():
-    """A per-row bias and head sizes above 128 stay with the vector kernels (which stop at 128 themselves); asking for
+    """A per-row bias and head sizes above 128 stay with the vector kernels (which stop at 256 themselves); asking for
     the matrix-core kernels by name then is an error, not a silent fallback.  Head sizes below 128 are zero-padded."""
     q, k, v, _ = make_qkv(1, 256, 1, 256, dtype=torch.float32, seed=1)
     with pytest.raises(NotImplementedError):
