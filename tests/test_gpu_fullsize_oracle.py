@@ -174,6 +174,62 @@ def test_packed_documents_131k_ring8_full_size():
         assert not torch.equal(a[:, inside], b[:, inside]), name
 
 
+def test_one_million_positions_ring8():
+    """B1 H32 S1048576 D128 bf16, causal, a ring of 8 shards of 131072 positions, chunks 512 / 512, forward and
+    backward: the context length the reference was written for, on one GPU (8.6 GB per operand; element offsets pass
+    2^32 and byte offsets 2^33, so every index of the path has to be 64-bit).  48 random rows of out and dq, and the last
+    row, recomputed from the definition in float64; dk and dv of key rows near the end of the sequence (head 31,
+    where the offsets are largest) against a float64 dense reference over the query rows that see them."""
+    B, S, H, D, n = 1, 1 << 20, 32, 128, 8
+    print("1M positions ring 8", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(51)
+    mk = lambda: torch.randn(B, S, H, D, device=DEV, generator=g).bfloat16()
+    q, k, v, do = mk(), mk(), mk(), mk()
+    kw = kwargs(512, 512, 1)
+    qd, kd, vd = (t.detach().requires_grad_(True) for t in (q, k, v))
+    t0 = time.time()
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention(qd, kd, vd, None, None, None, axis_name="sp", float32_logits=True, blockwise_kwargs=kw)
+        out.backward(do)
+    torch.cuda.synchronize()
+    print("1M positions: forward + backward %.1f s, kernels %s" % (time.time() - t0, ra.kernel_family_of_last_call()),
+          flush=True)
+    out, dq, dk, dv = out.detach(), qd.grad, kd.grad, vd.grad
+    for name, t in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert torch.isfinite(t[:, -4096:]).all() and torch.isfinite(t[:, :4096]).all(), name
+    ids = torch.zeros(S, dtype=torch.int32, device=DEV)
+    zero_bias = torch.zeros(1, 1, 1, S, device=DEV)
+    _sampled_rows_check(q, k, v, do, zero_bias, ids, out, dq, 48, 52, "1M ring 8")
+    # the last row of the last head by name
+    h, pos = H - 1, S - 1
+    kk, vv = k[0, :, h].double(), v[0, :, h].double()
+    p = torch.softmax(kk @ q[0, pos, h].double() / D ** 0.5, dim=0)
+    o = p @ vv
+    gg = do[0, pos, h].double()
+    dq_row = (p * (vv @ gg - gg @ o)) @ kk / D ** 0.5
+    assert float((out[0, pos, h].double() - o).abs().max()) <= 2e-2
+    assert float((dq[0, pos, h].double() - dq_row).abs().max()) <= 2e-2
+    # dk, dv of the last 2048 key rows of head 31: only the query rows from there on see them
+    j0 = S - 2048
+    dk_ref = torch.zeros(S - j0, D, dtype=torch.float64, device=DEV)
+    dv_ref = torch.zeros_like(dk_ref)
+    posn = torch.arange(S, device=DEV)
+    for r0 in range(j0, S, 256):
+        r1 = r0 + 256
+        qq, gg = q[0, r0:r1, h].double(), do[0, r0:r1, h].double()
+        logits = qq @ kk[:r1].T / D ** 0.5
+        logits = logits.masked_fill(posn[None, :r1] > posn[r0:r1, None], float("-inf"))
+        p = torch.softmax(logits, dim=1)
+        o = p @ vv[:r1]
+        ds = p * (gg @ vv[:r1].T - (gg * o).sum(dim=1, keepdim=True))
+        dk_ref[:r1 - j0] += ds[:, j0:].T @ qq / D ** 0.5
+        dv_ref[:r1 - j0] += p[:, j0:].T @ gg
+        del logits, p, ds
+    for name, a, b in (("dk", dk[0, j0:, h], dk_ref), ("dv", dv[0, j0:, h], dv_ref)):
+        ma, rl = assert_close(a, b, torch.bfloat16, "1M ring 8 head 31 " + name)
+        print("1M ring 8, last 2048 keys of head 31", name, "max-abs %.2e rel-L2 %.2e" % (ma, rl), flush=True)
+
+
 def test_causal_32k_all_heads_sampled_rows():
     """B1 H32 S32768 D128 bf16 causal, chunks 512/512 - all 32 heads of the headline configuration: 64 random rows of
     out and dq recomputed from the definition in float64, and head 9 (of 32) of dk / dv against a float64 dense
