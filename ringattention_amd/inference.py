@@ -6,7 +6,7 @@ import torch
 
 from . import _lib as L
 from .ringattention_hip import (_Config, _MaskInputs, _blockwise_attention_bwd, _blockwise_attention_fwd, _bwd_delta,
-                                _check_qkv, _save_residuals, _saved_residuals, axis_size)
+                                _check_qkv, _row_dense, _save_residuals, _saved_residuals, axis_size)
 
 
 def _inference_cfg(q, q_len, kv_len, float32_logits, logit_dim=0):
@@ -20,7 +20,9 @@ def _inference_cfg(q, q_len, kv_len, float32_logits, logit_dim=0):
 
 def _fwd(q, k, v, attn_mask, axis_name, float32_logits, logit_dim=0):
     _check_qkv(q, k, v)
-    q, k, v = (t if (t.stride(3) == 1 and t.stride(2) == t.shape[3]) else t.contiguous() for t in (q, k, v))
+    q, k, v = (t if _row_dense(t) else t.contiguous() for t in (q, k, v))      # other views are copied once
+    if k.stride(0) != v.stride(0):
+        k, v = k.contiguous(), v.contiguous()
     n = axis_size(axis_name)                                                     # :15
     B, q_total, H, D = q.shape
     kv_total = k.shape[1]

@@ -435,6 +435,11 @@ def _check_qkv(q, k, v):
         raise ValueError("q, k, v must share a dtype")
 
 
+def _row_dense(t):
+    """(B, S, H, D) with the last three dims laid out as one dense row of H * D elements per position."""
+    return t.stride(3) == 1 and t.stride(2) == t.shape[3] and t.stride(1) == t.shape[2] * t.shape[3]
+
+
 def _rows(t):
     """(stride_b, stride_s) of a (B, S, H, D) tensor whose last two dims are dense."""
     if t.stride(3) != 1 or t.stride(2) != t.shape[3]:
@@ -719,7 +724,12 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     Returns (out, residuals)."""
     cfg = _Config(blockwise_kwargs)
     _check_qkv(q, k, v)
-    q, k, v = (t if (t.stride(3) == 1 and t.stride(2) == t.shape[3]) else t.contiguous() for t in (q, k, v))
+    # the kernels take any batch stride, rows of H * D elements one after the other; k and v share theirs, and the
+    # cotangent and the gradients follow q.  Any other view (a slice of a fused q/k/v projection, a transposed
+    # (B, H, S, D) array) is copied once
+    q, k, v = (t if _row_dense(t) else t.contiguous() for t in (q, k, v))
+    if k.stride(0) != v.stride(0):
+        k, v = k.contiguous(), v.contiguous()
     n = axis_size(axis_name)
     B, q_total, H, D = q.shape
     kv_total = k.shape[1]

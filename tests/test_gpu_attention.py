@@ -730,3 +730,48 @@ def test_hull_table_gives_the_results_of_the_scan(dtype, ids):
     assert_close(a_out, ref_out, dtype, "out")
     for name, x, y in zip(("dq", "dk", "dv"), a_g, ref_g):
         assert_close(x, y, dtype, name)
+
+
+@pytest.mark.parametrize("dtype,D,chunk", [(torch.bfloat16, 128, 128), (torch.float32, 64, 32)])
+def test_strided_views_of_q_k_v_give_the_bits_of_contiguous_arrays(dtype, D, chunk):
+    """q, k, v as slices of one fused (B, S, 3, H, D) projection, as transposed (B, H, S, D) arrays, and k, v as
+    slices of a longer cache buffer: the results - output and, through autograd, the gradients in the layout of the
+    views - are those of contiguous copies, bit for bit (the reference's arrays have no strides to speak of)."""
+    B, S, H, n = 2, 512, 2, 2
+    g = torch.Generator().manual_seed(21)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).to(dtype).to(DEV)
+    do = torch.randn(B, S, H, D, generator=g).to(dtype).to(DEV)
+    seg = packed_segment_ids(B, S, 150, seed=22).to(DEV)
+    kw = kwargs(chunk, chunk, 1)
+
+    def run(q, k, v):
+        q, k, v = (t.detach().requires_grad_(True) for t in (q, k, v))
+        with ra.ring_axis("sp", n):
+            out = ra.ringattention(q, k, v, None, seg, None, axis_name="sp", float32_logits=True, blockwise_kwargs=kw)
+            out.backward(do)
+        return out.detach(), q.grad, k.grad, v.grad
+
+    base = run(*(qkv[:, :, i].contiguous() for i in range(3)))
+    fused = run(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2])
+    bhsd = qkv.permute(2, 0, 3, 1, 4).contiguous()                      # (3, B, H, S, D)
+    transposed = run(*(bhsd[i].transpose(1, 2) for i in range(3)))
+    cache = torch.zeros(2, B, S + 256, H, D, dtype=dtype, device=DEV)
+    cache[0, :, :S], cache[1, :, :S] = qkv[:, :, 1], qkv[:, :, 2]
+    cached = run(qkv[:, :, 0].contiguous(), cache[0, :, :S], cache[1, :, :S])
+    mixed = run(qkv[:, :, 0], cache[0, :, :S], qkv[:, :, 2].contiguous())   # k and v with different batch strides
+    for name, res in (("fused", fused), ("transposed", transposed), ("cache", cached), ("mixed", mixed)):
+        for what, a, b in zip(("out", "dq", "dk", "dv"), res, base):
+            assert a.shape == b.shape and torch.equal(a, b), (name, what)
+    # the same through the boolean-mask ring
+    mask = torch.ones(1, 1, S, S, dtype=torch.bool, device=DEV).tril()
+
+    def run_inf(q, k, v):
+        q, k, v = (t.detach().requires_grad_(True) for t in (q, k, v))
+        with ra.ring_axis("sp", n):
+            out = ra.ringattention_inference(q, k, v, mask, "sp", True)
+            out.backward(do)
+        return out.detach(), q.grad, k.grad, v.grad
+
+    base = run_inf(*(qkv[:, :, i].contiguous() for i in range(3)))
+    for what, a, b in zip(("out", "dq", "dk", "dv"), run_inf(qkv[:, :, 0], cache[0, :, :S], qkv[:, :, 2]), base):
+        assert torch.equal(a, b), ("inference", what)
