@@ -201,6 +201,9 @@ class SwiGLU(torch.nn.Module):
         if not x.is_cuda:
             raise RuntimeError("ringattention_amd runs on the GPU only")
         T = x.shape[0]
+        if T == 0:                  # nothing to launch; the zero keeps the empty result attached to its inputs
+            zero = 0.0 * (self.w1.sum() + self.w2.sum() + self.w3.sum())
+            return x.new_zeros(*shp[:-1], self.w2.shape[1]) + x.sum() + zero.to(x.dtype)
         if T % _TOKEN_GRID:         # the GEMM tiles want whole groups of 128 tokens: zero rows, dropped again below
             x = torch.nn.functional.pad(x, (0, 0, 0, _TOKEN_GRID - T % _TOKEN_GRID))
         y = _SwiGLUFn.apply(x.contiguous(), self.w1, self.w2, self.w3, self.gemm_tile)[:T]
@@ -232,6 +235,8 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
     if s % chunk_size:
         raise ValueError("sequence length %d must divide by chunk_size %d" % (s, chunk_size))
     n = s // chunk_size
+    if isinstance(feedforward, SwiGLU) and inputs.numel() == 0:
+        return feedforward(inputs)
     if isinstance(feedforward, SwiGLU):
         if inputs.dtype != torch.bfloat16:
             raise NotImplementedError("SwiGLU kernels are bf16")

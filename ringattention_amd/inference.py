@@ -118,6 +118,10 @@ def ring_attention_inference(q, k, v, attn_mask, axis_name, float32_logits=True)
     if q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16:
         return ring_attention_inference(q.float(), k.float(), v.float(), attn_mask, axis_name,
                                         float32_logits).to(torch.float16)
+    if q.numel() == 0 or k.numel() == 0:          # nothing to launch (as in ring_attention)
+        _check_qkv(q, k, v)
+        fill = float("nan") if q.numel() else 0.0
+        return torch.full_like(q, fill) + 0.0 * (q.sum() + k.sum() + v.sum()).to(q.dtype)
     D = q.shape[-1]
     if D > 256:
         raise NotImplementedError("head size %d: the kernels take head sizes up to 256" % D)

@@ -1090,6 +1090,12 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
         out = ring_attention(q.float(), k.float(), v.float(), attn_bias, segment_ids, cache_idx, axis_name,
                              float32_logits, blockwise_kwargs)
         return out.to(torch.float16)
+    if q.numel() == 0 or k.numel() == 0:
+        # nothing to launch: an empty result, or - queries without a single key - the 0 / 0 of :52; the product
+        # with zero keeps the result attached to its inputs for autograd
+        _check_qkv(q, k, v)
+        fill = float("nan") if q.numel() else 0.0
+        return torch.full_like(q, fill) + 0.0 * (q.sum() + k.sum() + v.sum()).to(q.dtype)
     n = axis_size(axis_name)
     if cache_idx is not None and q.shape[1] == n and q.shape[3] in (64, 128) and not (
             torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) \

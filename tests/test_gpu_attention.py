@@ -775,3 +775,29 @@ def test_strided_views_of_q_k_v_give_the_bits_of_contiguous_arrays(dtype, D, chu
     base = run_inf(*(qkv[:, :, i].contiguous() for i in range(3)))
     for what, a, b in zip(("out", "dq", "dk", "dv"), run_inf(qkv[:, :, 0], cache[0, :, :S], qkv[:, :, 2]), base):
         assert torch.equal(a, b), ("inference", what)
+
+
+def test_empty_inputs_give_empty_results():
+    """No batch rows, no positions, no tokens: nothing is launched and the (empty) result stays attached to its inputs
+    for autograd; queries without a single key end as the 0 / 0 of ringattention_jax.py:52."""
+    kw = kwargs(128, 128, 1)
+    for shape in ((0, 256, 2, 128), (1, 0, 2, 128)):
+        q = torch.zeros(shape, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+        out = ra.ringattention(q, q, q, None, None, None, axis_name=None, float32_logits=True, blockwise_kwargs=kw)
+        assert out.shape == q.shape and out.dtype == q.dtype
+        out.sum().backward()
+        assert q.grad.shape == q.shape
+        with ra.ring_axis("sp", 1):
+            mask = torch.ones(1, 1, shape[1], shape[1], dtype=torch.bool, device=DEV)
+            assert ra.ringattention_inference(q, q, q, mask, "sp", True).shape == q.shape
+    q = torch.zeros(1, 128, 2, 128, device=DEV, dtype=torch.bfloat16)
+    k = torch.zeros(1, 0, 2, 128, device=DEV, dtype=torch.bfloat16)
+    assert torch.isnan(ra.ringattention(q, k, k, None, None, None, axis_name=None, float32_logits=True,
+                                        blockwise_kwargs=kw)).all()
+    ff = ra.SwiGLU(128, 256, device=DEV)
+    x = torch.zeros(0, 256, 128, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    y = ra.blockwise_feedforward(ff, x, 128)
+    assert y.shape == (0, 256, 128)
+    y.sum().backward()
+    assert x.grad.shape == x.shape and ff.w1.grad is not None and not ff.w1.grad.any()
+    assert ff(torch.zeros(0, 128, device=DEV, dtype=torch.bfloat16)).shape == (0, 128)
