@@ -52,7 +52,7 @@ def decode_attention(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_kwarg
     if L_buf % cfg.kc:
         raise ValueError("cache length %d must divide by key_chunk_size %d" % (L_buf, cfg.kc))
     mi = _mask_inputs or _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device,
-                                     k_chunk_idx_start * cfg.kc + L_buf)
+                                     k_chunk_idx_start * cfg.kc + L_buf, q.shape[2])
     if out is None and (write_out or carry is None):
         out = torch.empty_like(q)
     lib = L.load()
@@ -111,7 +111,7 @@ def decode_attention_ring(q, k, v, attn_bias, segment_ids, cache_idx, blockwise_
     if L_buf % n or (L_buf // n) % cfg.kc:
         raise ValueError("cache length %d must divide into %d shards of whole key chunks (%d)" % (L_buf, n, cfg.kc))
     kv_len = L_buf // n
-    mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, L_buf)
+    mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, L_buf, H)
     out = torch.empty_like(q)
     num = torch.empty((B, n, H, D), dtype=torch.float32, device=q.device)
     den = torch.empty((B, n, H, 1), dtype=torch.float32, device=q.device)

@@ -170,13 +170,18 @@ class _Config:
 class _MaskInputs:
     """attn_bias / segment_ids / cache_idx in the form ra_mask wants (device memory kept alive here)."""
 
-    def __init__(self, cfg, attn_bias, segment_ids, cache_idx, batch, device, k_total):
+    def __init__(self, cfg, attn_bias, segment_ids, cache_idx, batch, device, k_total, heads=None):
         self.bias = None
         self.bias_strides = (0, 0, 0, 0)
         if attn_bias is not None:
             if attn_bias.dim() != 4:
                 raise ValueError("attn_bias must be 4-D (B, H, Q, K)")
             bb, hb, qb, kb = attn_bias.shape
+            # the kernels index the bias by batch row and head: a size that is neither 1 (broadcast) nor the array's
+            # own would read past its end
+            if bb not in (1, batch) or (heads is not None and hb not in (1, heads)):
+                raise ValueError("attn_bias batch / head dims %s must be 1 or those of q (%d, %s)"
+                                 % ((bb, hb), batch, heads))
             if qb != 1 and qb < cfg.qc:
                 raise ValueError("attn_bias query dim must be 1 or >= query_chunk_size")
             if kb != 1 and kb < k_total:
@@ -195,6 +200,8 @@ class _MaskInputs:
         if segment_ids is not None:
             if segment_ids.dim() != 2:
                 raise ValueError("segment_ids must be 2-D (B, S)")
+            if segment_ids.shape[0] not in (1, batch):
+                raise ValueError("segment_ids batch dim %d must be 1 or that of q (%d)" % (segment_ids.shape[0], batch))
             # the int32 copy, the per-tile id ranges and their host copy are kept per segment_ids tensor (same
             # storage, same version counter): a later call with the tensor unchanged launches nothing for them and
             # copies nothing to the host, so it can be captured into a HIP graph.  The version counter does not see
@@ -530,7 +537,7 @@ def _blockwise_attention_fwd(q, k, v, carry, q_chunk_idx_start, k_chunk_idx_star
         if cfg.pdrop > 0.0:
             raise NotImplementedError("attention dropout needs chunk starts the host knows")
     mi = _mask_inputs or _MaskInputs(cfg, bias, segment_ids, cache_idx, B, q.device,
-                                     (k_chunk_idx_start * cfg.kc + Skv) if starts_dev is None else 0)
+                                     (k_chunk_idx_start * cfg.kc + Skv) if starts_dev is None else 0, H)
     num, den, mx = carry
     p = L.RaAttnFwdParams()
     p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
@@ -597,7 +604,7 @@ def _blockwise_attention_bwd(q, k, v, g, carry, q_chunk_idx_start, k_chunk_idx_s
         if cfg.pdrop > 0.0:
             raise NotImplementedError("attention dropout needs chunk starts the host knows")
     mi = _mask_inputs or _MaskInputs(cfg, bias, segment_ids, cache_idx, B, q.device,
-                                     (k_chunk_idx_start * cfg.kc + Skv) if starts_dev is None else 0)
+                                     (k_chunk_idx_start * cfg.kc + Skv) if starts_dev is None else 0, H)
     dq, dk, dv, output, den, mx = carry
     if g.dtype != q.dtype:
         g = g.to(q.dtype)
@@ -739,7 +746,7 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     if q_len % cfg.qc or kv_len % cfg.kc:
         raise ValueError("per-device lengths (%d, %d) must divide by the chunk sizes (%d, %d)"
                          % (q_len, kv_len, cfg.qc, cfg.kc))
-    mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, kv_total)
+    mi = _MaskInputs(cfg, attn_bias, segment_ids, cache_idx, B, q.device, kv_total, H)
     mi.seg_covers = (mi.seg is not None and cache_idx is None and mi.seg_len >= max(q_total, kv_total)
                      and cfg.segment_hull_table)
     if cfg.skip_masked_tiles is None:

@@ -244,3 +244,18 @@ def test_segment_cache_follows_the_version_counter_and_the_opt_out():
     cfg2 = R._Config(dict(query_chunk_size=128, key_chunk_size=128, causal_block_size=1, cache_segment_ids=False))
     d = R._MaskInputs(cfg2, None, seg, None, 1, "cpu", 256)
     assert d.seg_mm[0, 0].tolist() == [0, 9]
+
+
+def test_bias_and_segment_ids_must_broadcast_or_match_batch_and_heads():
+    """The kernels index attn_bias by batch row and head and segment_ids by batch row: a dim that is neither 1 nor the
+    array's own would be read past its end, so the host refuses it before anything is launched."""
+    from ringattention_amd import ringattention_hip as rh
+    cfg = rh._Config(dict(query_chunk_size=8, key_chunk_size=8, causal_block_size=1, cache_segment_ids=False))
+    ok_bias = torch.zeros(1, 4, 1, 64)
+    rh._MaskInputs(cfg, ok_bias, torch.zeros(1, 64, dtype=torch.int32), None, 3, "cpu", 64, 4)
+    rh._MaskInputs(cfg, torch.zeros(3, 1, 1, 64), torch.zeros(3, 64, dtype=torch.int32), None, 3, "cpu", 64, 4)
+    for bad_bias in (torch.zeros(2, 1, 1, 64), torch.zeros(1, 3, 1, 64)):
+        with pytest.raises(ValueError):
+            rh._MaskInputs(cfg, bad_bias, None, None, 3, "cpu", 64, 4)
+    with pytest.raises(ValueError):
+        rh._MaskInputs(cfg, None, torch.zeros(2, 64, dtype=torch.int32), None, 3, "cpu", 64, 4)
