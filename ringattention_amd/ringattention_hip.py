@@ -757,7 +757,7 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
         cfg.skip_masked_tiles = False      # dropout can leave a row without any allowed key
     _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total)
     d_true = D
-    pad_to = _mfma_head_size(cfg, mi, q)
+    pad_to = _padded_head_size(cfg, mi, q)
     if pad_to:
         # a head size the matrix-core kernels do not tile: q, k, v zero-padded along D (the products are those of the
         # un-padded rows), the logits still divided by sqrt of the original head size (:118)
@@ -810,7 +810,7 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     return out, res
 
 
-def _mfma_head_size(cfg, mi, q):
+def _padded_head_size(cfg, mi, q):
     """The head size to zero-pad q, k, v to (the products are those of the un-padded rows; the logits keep the scale
     of the original head size), or 0 when the kernels take the head size as it is.  The matrix-core kernels tile 64
     and 128, the generic ones 32, 64, 128 and 256: a call that stays on the generic kernels anyway (they were asked
