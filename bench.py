@@ -61,23 +61,41 @@ def _kwargs(qc, kc, cbs=1, **extra):
     return kw
 
 
+def _note(msg):
+    """A line on stderr: a sign of life from runs whose steps take many seconds (the JSON line stays alone on stdout)."""
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
 def _time_steps(fn, steps, warmup):
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
+    if steps <= 2:          # a handful of long steps: say so as they finish (the wait costs nothing next to them)
+        for i in range(steps):
+            t1 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            if time.perf_counter() - t1 > 5.0:
+                _note("step %d of %d: %.1f s" % (i + 1, steps, time.perf_counter() - t1))
+    else:
+        for _ in range(steps):
+            fn()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
 def _event_ms(fn, reps):
-    """Average duration of ``fn`` (which launches on torch's current stream) from events on that stream."""
+    """Average duration of ``fn`` (which launches on torch's current stream) from events on that stream.  A call
+    that takes seconds is repeated once, not ``reps`` times."""
     import torch
+    t0 = time.perf_counter()
     fn()
     torch.cuda.synchronize()
+    if time.perf_counter() - t0 > 2.0:
+        _note("a launch of %.1f s: timed once more" % (time.perf_counter() - t0))
+        reps = 1
     total = 0.0
     for _ in range(reps):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -296,7 +314,8 @@ def bench_attention(args, ring, dropout=False, c1=False):
         roof = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": peak,
                 "unit": "TFLOP/s", "frac": round(ach / peak, 4),
                 "traffic": traffic.get(dom) if S == 32768 and args.inputs == "baseline" else None,
-                "traffic_source": "profiles/" + TRAFFIC_PROFILE if traffic.get(dom) else None,
+                "traffic_source": ("profiles/" + TRAFFIC_PROFILE
+                                   if traffic.get(dom) and S == 32768 and args.inputs == "baseline" else None),
                 "mfma_util_pmc": ({"kernel": util.get(dom), "step": util.get("attn32k_step"),
                                    "source": "profiles/" + MFMA_PROFILE}
                                   if S == 32768 and not dropout and util.get(dom) else None),
