@@ -230,7 +230,9 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
     for the order of the fp32 sum over tokens.  1 = per launch; the default of 4 keeps the scratch of a backward step
     at 14 (chunk, intermediate) buffers instead of 5, still independent of the sequence length (at 65536 tokens of
     4096 x 11008: 61.2 ms with 1, 57.5 with 2, 55.8 with 4, 55.0 with 8).
-    ``pre_remat`` / ``static_argnums`` steer XLA rematerialisation only."""
+    ``pre_remat=False`` (:335-336) rematerialises a generic callable here (torch.utils.checkpoint, per chunk) unless
+    ``policy`` keeps the activations; with the default True the caller has done so, or not, as in the reference.
+    ``static_argnums`` steers XLA only."""
     b, s, d = inputs.shape
     if s % chunk_size:
         raise ValueError("sequence length %d must divide by chunk_size %d" % (s, chunk_size))
@@ -258,8 +260,19 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
                                      feedforward.w3, slab, _save_preactivations(policy), feedforward.gemm_tile,
                                      max(1, int(weight_grad_chunks) * step // slab))
         return y[:b * s].reshape(b, s, y.shape[-1])
+    fn = feedforward
+    if not pre_remat and torch.is_grad_enabled():
+        # :335-336: the callable has not been rematerialised by the caller, so it is here - every chunk's forward
+        # pass runs again in the backward pass instead of keeping its activations - unless the policy keeps them
+        try:
+            keep = _save_preactivations(policy)
+        except ValueError:
+            keep = False            # another checkpoint policy of the reference's framework: recompute (same results)
+        if not keep:
+            from torch.utils.checkpoint import checkpoint
+            fn = lambda h: checkpoint(feedforward, h, use_reentrant=False)
     x = inputs.reshape(b, chunk_size, n, d)
-    outs = [feedforward(x[:, :, j, :]) for j in range(n)]
+    outs = [fn(x[:, :, j, :]) for j in range(n)]
     out = torch.stack(outs, dim=2)
     return out.reshape(b, s, out.shape[-1])
 

@@ -259,3 +259,40 @@ def test_bias_and_segment_ids_must_broadcast_or_match_batch_and_heads():
             rh._MaskInputs(cfg, bad_bias, None, None, 3, "cpu", 64, 4)
     with pytest.raises(ValueError):
         rh._MaskInputs(cfg, None, torch.zeros(2, 64, dtype=torch.int32), None, 3, "cpu", 64, 4)
+
+
+def test_blockwise_feedforward_generic_callable_groups_and_remat():
+    """A callable that is not the library's SwiGLU (ringattention_jax.py:333-352): the scan hands it the reference's
+    strided token groups {c * n + j} ('b (c n) d -> b c n d'); with pre_remat=False it is rematerialised per chunk
+    (its forward pass runs again in the backward pass), with the default True it is called once per chunk.  Same
+    values and gradients either way, equal to the un-chunked call.  Runs on the CPU: no kernel of the library is
+    involved."""
+    import ringattention_amd as ra
+    torch.manual_seed(0)
+    mlp = torch.nn.Sequential(torch.nn.Linear(16, 48), torch.nn.GELU(), torch.nn.Linear(48, 16))
+    calls = []
+
+    def ff(h):
+        calls.append(tuple(h.shape))
+        return mlp(h)
+    x = torch.randn(2, 24, 16, requires_grad=True)
+    ref = mlp(x)
+    ref.square().sum().backward()
+    gx, gw = x.grad.clone(), mlp[0].weight.grad.clone()
+    for pre_remat, n_calls in ((True, 4), (False, 8)):
+        x.grad = None
+        mlp.zero_grad()
+        calls.clear()
+        y = ra.blockwise_feedforward(ff, x, 6, pre_remat=pre_remat)
+        assert torch.allclose(y, ref, atol=1e-6)
+        y.square().sum().backward()
+        assert calls[:4] == [(2, 6, 16)] * 4 and len(calls) == n_calls
+        assert torch.allclose(x.grad, gx, atol=1e-5) and torch.allclose(mlp[0].weight.grad, gw, atol=1e-5)
+    # the groups are strided: step j sees tokens j, n + j, 2 n + j, ...
+    seen = []
+    ra.blockwise_feedforward(lambda h: (seen.append(h[0, :, 0].clone()), h)[1], torch.arange(24.).reshape(1, 24, 1), 6)
+    assert torch.equal(seen[1], torch.tensor([1., 5., 9., 13., 17., 21.]))
+    # a policy that keeps the activations switches the rematerialisation off again
+    calls.clear()
+    ra.blockwise_feedforward(ff, x, 6, pre_remat=False, policy="everything_saveable").sum().backward()
+    assert len(calls) == 4
