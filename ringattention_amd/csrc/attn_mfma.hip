@@ -411,12 +411,18 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       int idx = clamp_seg_index(((long long)mv.k_start + krow / mv.kc) * mv.kc, mv.kc, mv.seg_len, krow % mv.kc);
       seg_k = mv.seg[(int64_t)b * mv.seg_sb + idx];
     }
+    // a bias at the level of the mask value (a padding mask passed as where(keep, 0, finfo.min)) absorbs the logit in
+    // the reference and would overflow here once scaled: the key then counts as masked for every row (its accumulators
+    // start at -inf, the masked path puts the mask value itself), and its wavefront takes the masked path throughout
+    bool lane_bm = false;
     if (HAS_BIAS) {
       float bv = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + (int64_t)gk * mv.bias_sk];
       if (mv.any_mask) bv = fminf(bv, 0.f);
-      bias2 = bv * kLog2e / c;          // the S accumulators start from it
+      lane_bm = bv * kLog2e <= kMask2;
+      bias2 = lane_bm ? RA_NEG_INF : bv * kLog2e / c;          // the S accumulators start from it
       st_bias[pair][lane] = bias2;      // kept in LDS, not in a register: every lane reads back its own slot
     }
+    const bool wave_bm = HAS_BIAS && __builtin_amdgcn_ballot_w64(lane_bm) != 0ULL;
     int n_off[NK];
 #pragma unroll
     for (int t = 0; t < NK; t++) n_off[t] = lo * TROW + (((2 * t + hi) ^ swz<HD>(lo)) << 3);
@@ -463,10 +469,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
     _Pragma("unroll") for (int e = 0; e < 4; e++) {                                                     \
       float x = SC[(G) * 4 + e] * c;                                                                    \
       bool masked = (gq_tile + qrow0 + e < qlim);                                                       \
-      if (HAS_SEG) masked = masked || (st_seg[BUF][qrow0 + e] != seg_k);                                \
-      if (HAS_KEEP == 2 && HAS_SEG) {                                                                   \
-        /* as below, with the segment ids: a pair of two documents counts as masked once more */        \
-        const bool sne_ = st_seg[BUF][qrow0 + e] != seg_k;                                              \
+      /* another document, or this lane's key carries a bias at the level of the mask value */          \
+      bool sne_ = HAS_BIAS && lane_bm;                                                                  \
+      if (HAS_SEG) sne_ = sne_ || st_seg[BUF][qrow0 + e] != seg_k;                                      \
+      masked = masked || sne_;                                                                          \
+      if (HAS_KEEP == 2 && (HAS_SEG || HAS_BIAS)) {                                                     \
+        /* as below, with such pairs: they count as masked once more */                                 \
         x = (((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) && !sne_) ? x : kMask2;                       \
         x = (((kw_some >> ((BLK) * 32 + (G) * 8 + e)) & 1) &&                                           \
              (((kw_k >> ((BLK) * 32 + (G) * 8 + e)) & 1) || !sne_)) ? x : RA_NEG_INF;                   \
@@ -573,7 +581,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
         }
       }
       // step 2t: vector work of block 0 of tile t, products of block 1
-      if ((HAS_SEG && !sp_cur) || (gq_tile < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
+      if ((HAS_SEG && !sp_cur) || (gq_tile < qlim_wave) || (HAS_KEEP && ks_cur != 2) || wave_bm) {
         RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, true);
       } else {
         RA_WS_PRODUCE(s_a, dp_a, s_b, dp_b, cur, 0, cur, 1, 0, false);
@@ -583,7 +591,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkv_ws_kernel(BwdArgs a) {
       // block 0 of tile t + 1 (the last tile computes a block that is never used)
       RA_WS_STORE(prv);
       RA_WS_LOAD(t + 3);
-      if ((HAS_SEG && !sp_cur) || (gq_tile + 32 < qlim_wave) || (HAS_KEEP && ks_cur != 2)) {
+      if ((HAS_SEG && !sp_cur) || (gq_tile + 32 < qlim_wave) || (HAS_KEEP && ks_cur != 2) || wave_bm) {
         RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, true);
       } else {
         RA_WS_PRODUCE(s_b, dp_b, s_a, dp_a, cur, 1, nxt, 0, 1, false);
@@ -840,8 +848,16 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     if (SNP == 4) { *(uint4*)(dk_ + 2 * SRP * TROW) = S##k2; *(uint4*)(dk_ + 3 * SRP * TROW) = S##k3; } \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       if (HAS_SEG) seg_ks[BUF][stid] = S##seg;                                                          \
-      /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
-      if (HAS_BIAS) bias_ks[BUF][stid] = (mv.any_mask ? fminf(S##bias, 0.f) : S##bias) * bias_scale;    \
+      /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it.  A bias  \
+         at the level of the mask value (a padding mask passed as where(keep, 0, finfo.min)) absorbs    \
+         the logit in the reference and would overflow here once scaled: such a key is marked with     \
+         -inf; the masked path turns the mark into the mask value itself, the plain path gives the key  \
+         the weight exp2(-inf) = 0, which is its weight in every row that sees a real key */           \
+      if (HAS_BIAS) {                                                                                   \
+        const float bv_ = mv.any_mask ? fminf(S##bias, 0.f) : S##bias;                                  \
+        const bool bm_ = bv_ * kLog2e <= kMask2;                                                        \
+        bias_ks[BUF][stid] = bm_ ? RA_NEG_INF : bv_ * bias_scale;                                       \
+      }                                                                                                 \
     }                                                                                                   \
   }
 #define RA_WS_STORE_V(S, BUF)                                                                            \
@@ -916,10 +932,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
         const int kr_ = (BLK) * 32 + (G) * 8 + hi * 4 + e;                                              \
         float x = SC[(G) * 4 + e] * c;                                                                  \
         bool masked = (gk_tile + kr_ >= klim);                                                          \
-        if (HAS_SEG) masked = masked || (seg_ks[BUF][kr_] != seg_q);                                    \
-        if (HAS_KEEP == 2 && HAS_SEG) {                                                                 \
-          /* as below, with the segment ids: a pair of two documents counts as masked once more */      \
-          const bool sne_ = seg_ks[BUF][kr_] != seg_q;                                                  \
+        /* another document, or a key whose bias is at the level of the mask value (marked -inf) */     \
+        bool sne_ = false;                                                                              \
+        if (HAS_SEG) sne_ = seg_ks[BUF][kr_] != seg_q;                                                  \
+        if (HAS_BIAS) sne_ = sne_ || SC[(G) * 4 + e] == RA_NEG_INF;                                     \
+        masked = masked || sne_;                                                                        \
+        if (HAS_KEEP == 2 && (HAS_SEG || HAS_BIAS)) {                                                   \
+          /* as below, with such pairs: they count as masked once more */                               \
           x = (((kw_cur >> ((BLK) * 32 + (G) * 8 + e)) & 1) && !sne_) ? x : kMask2;                     \
           x = (((kw_some >> ((BLK) * 32 + (G) * 8 + e)) & 1) &&                                         \
                (((kw_k >> ((BLK) * 32 + (G) * 8 + e)) & 1) || !sne_)) ? x : RA_NEG_INF;                 \
@@ -1053,9 +1072,9 @@ __global__ __launch_bounds__(512) void attn_bwd_dq_ws_kernel(BwdArgs a) {
     cur = nxt;                                                                                          \
   }
     int t = 0;
-    for (; t < t_a; t++) RA_WS_TILE(true);
-    for (; t < t_b; t++) RA_WS_TILE(false);
-    for (; t < ntiles; t++) RA_WS_TILE(true);
+      for (; t < t_a; t++) RA_WS_TILE(true);
+      for (; t < t_b; t++) RA_WS_TILE(false);
+      for (; t < ntiles; t++) RA_WS_TILE(true);
 #undef RA_WS_TILE
     __syncthreads();      // step 2 ntiles: the consumer's last block
 #undef RA_WS_INIT
@@ -1197,6 +1216,7 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
   __shared__ float dens[4][32];      // [pair][query]: final denominator, for the step that writes out
   __shared__ int seg_ks[3][FBN];
   __shared__ float bias_ks[3][FBN];
+  __shared__ int bias_any[3];        // [buffer]: some key of the tile carries a bias at the level of the mask value
 
   MaskView mv = a.mv;
   mv.resolve();
@@ -1309,8 +1329,17 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     if (SNP == 4) { *(uint4*)(dk_ + 2 * SRP * TROW) = S##k2; *(uint4*)(dk_ + 3 * SRP * TROW) = S##k3; } \
     if ((HAS_SEG || HAS_BIAS) && stid < FBN) {                                                          \
       if (HAS_SEG) seg_ks[BUF][stid] = S##seg;                                                          \
-      /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it */          \
-      if (HAS_BIAS) bias_ks[BUF][stid] = (mv.any_mask ? fminf(S##bias, 0.f) : S##bias) * bias_scale;    \
+      /* clamped when a mask is on (:299,:309) and scaled: the S accumulators start from it.  A bias  \
+         at the level of the mask value (a padding mask passed as where(keep, 0, finfo.min)) absorbs    \
+         the logit in the reference and would overflow here once scaled: such a key is marked with     \
+         -inf and its tile takes the masked path, where the mark becomes the mask value itself */      \
+      if (HAS_BIAS) {                                                                                   \
+        const float bv_ = mv.any_mask ? fminf(S##bias, 0.f) : S##bias;                                  \
+        const bool bm_ = bv_ * kLog2e <= kMask2;                                                        \
+        bias_ks[BUF][stid] = bm_ ? RA_NEG_INF : bv_ * bias_scale;                                       \
+        const unsigned long long any_ = __builtin_amdgcn_ballot_w64(bm_);                               \
+        if (stid == 0) bias_any[BUF] = any_ != 0ULL;                                                    \
+      }                                                                                                 \
     }                                                                                                   \
   }
 #define RA_WS_STORE_V(S, BUF)                                                                            \
@@ -1393,10 +1422,13 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
         const int kr_ = (BLK) * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);                                   \
         float x_ = SC[r] * c;                                                                           \
         bool masked_ = (gk_tile + kr_ >= klim);                                                         \
-        if (HAS_SEG) masked_ = masked_ || (seg_ks[BUF][kr_] != seg_q);                                  \
-        if (HAS_KEEP == 2 && HAS_SEG) {                                                                 \
-          /* as below, with the segment ids: a pair of two documents counts as masked once more */      \
-          const bool sne_ = seg_ks[BUF][kr_] != seg_q;                                                  \
+        /* another document, or a key whose bias is at the level of the mask value (marked -inf) */     \
+        bool sne_ = false;                                                                              \
+        if (HAS_SEG) sne_ = seg_ks[BUF][kr_] != seg_q;                                                  \
+        if (HAS_BIAS) sne_ = sne_ || SC[r] == RA_NEG_INF;                                               \
+        masked_ = masked_ || sne_;                                                                      \
+        if (HAS_KEEP == 2 && (HAS_SEG || HAS_BIAS)) {                                                   \
+          /* as below, with such pairs: they count as masked once more */                               \
           x_ = (((kw_cur >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) && !sne_) ? x_ : kMask2;        \
           x_ = (((kw_some >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) &&                             \
                 (((kw_k >> ((BLK) * 32 + (r >> 2) * 8 + (r & 3))) & 1) || !sne_)) ? x_ : RA_NEG_INF;    \
@@ -1544,9 +1576,18 @@ __global__ __launch_bounds__(512) void attn_fwd_ws_kernel(FwdArgs a) {
     cur = nxt;                                                                                          \
   }
     int t = 0;
-    for (; t < t_a; t++) RA_WS_TILE(true);
-    for (; t < t_b; t++) RA_WS_TILE(false);
-    for (; t < ntiles; t++) RA_WS_TILE(true);
+    if (HAS_BIAS) {
+      // one loop: a tile inside the run still takes the masked path when one of its keys carries a bias at the level
+      // of the mask value (the flag its staging left in LDS)
+      for (; t < ntiles; t++) {
+        if (t < t_a || t >= t_b || __builtin_amdgcn_readfirstlane(bias_any[cur])) RA_WS_TILE(true)
+        else RA_WS_TILE(false)
+      }
+    } else {
+      for (; t < t_a; t++) RA_WS_TILE(true);
+      for (; t < t_b; t++) RA_WS_TILE(false);
+      for (; t < ntiles; t++) RA_WS_TILE(true);
+    }
 #undef RA_WS_TILE
     __syncthreads();      // step 2 ntiles: the consumer's last block
     // bring the carry to the exact running max (:138) and hand the factor to the consumer

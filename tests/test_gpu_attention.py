@@ -801,3 +801,39 @@ def test_empty_inputs_give_empty_results():
     y.sum().backward()
     assert x.grad.shape == x.shape and ff.w1.grad is not None and not ff.w1.grad.any()
     assert ff(torch.zeros(0, 128, device=DEV, dtype=torch.bfloat16)).shape == (0, 128)
+
+
+@pytest.mark.parametrize("skip", [False, None])
+@pytest.mark.parametrize("dtype,D,chunk,n", [(torch.bfloat16, 128, 128, 2), (torch.float32, 64, 32, 1), (torch.bfloat16, 64, 256, 4),
+                                             (torch.float32, 128, 128, 2)])
+def test_padding_mask_as_bias_matches_oracle(dtype, D, chunk, n, skip):
+    """How a model built on the reference passes its padding mask: attn_bias = where(mask, 0, finfo.min) per key,
+    (B, 1, 1, K), next to the causal mask.  A padded key's logit is absorbed by finfo.min exactly as a masked one's
+    (ringattention_jax.py:135-136), so it weighs exp(finfo.min - max) = 0 in every row that sees a real key.  Batch
+    row 1 starts with padding: its first 70 rows see padded and masked keys only and take the uniform weights of equal
+    finfo.min logits over the keys of the chunks that run (:138-144).  With skip_masked_tiles=False every tile of those
+    chunks runs here too and the whole output is the oracle's; with the default (tiles that hold masked pairs only
+    are skipped, which asks for an unmasked key in every row) the rows that see a real key are the oracle's and the
+    others stay finite.  With no cotangent on those rows - a model's loss mask - all gradients are the oracle's."""
+    B, S, H = 2, 1024, 2
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=31, scale=D ** -0.25)
+    keep = torch.ones(B, S, dtype=torch.bool)
+    keep[0, 900:] = False                 # right padding
+    keep[1, :70] = False                  # left padding
+    bias = torch.where(keep, 0.0, torch.finfo(torch.float32).min).reshape(B, 1, 1, S)
+    kw = kwargs(chunk, chunk, 1, dtype=torch.float32, skip_masked_tiles=skip)
+    do = do.clone()
+    do[1, :70] = 0                        # no cotangent on the rows that see no real key (a model's loss mask)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, None, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, None, None, n, kw)
+    print("padding mask", dtype, D, chunk, n, skip, ra.kernel_family_of_last_call(), flush=True)
+    assert torch.isfinite(out).all() and all(torch.isfinite(t).all() for t in grads)
+    if skip is None:                      # rows without a real key: defined, but not the reference's average
+        out, ref_out = out.clone(), ref_out.clone()
+        out[1, :70] = 0
+        ref_out[1, :70] = 0
+    assert_close(out, ref_out, dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, dtype, name)
+    # padded keys get no gradient from rows that see a real key as well
+    assert float(grads[1][0, 900:].abs().max()) == 0.0 and float(grads[2][0, 900:].abs().max()) == 0.0

@@ -47,6 +47,8 @@ def draw(seed):
     B, H = r.choice([1, 1, 2]), r.choice([1, 2, 3])
     bias = r.choice([None, None, "key", "key", "head", "row"])
     seg = r.choice([None, "docs", "docs", "one"])
+    if r.random() < 0.15:
+        bias = "pad"                                # a padding mask as a bias: where(keep, 0, finfo.min), padding on the right
     return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cbs=cbs, B=B, H=H, bias=bias, seg=seg)
 
 
@@ -65,11 +67,16 @@ def test_random_configuration_matches_oracle(seed):
         bias = torch.randn(B, H, 1, Skv, generator=g)
     elif c["bias"] == "row":                        # :279-283: rows 0:qc of the bias serve every query chunk
         bias = torch.randn(1, H, c["qc"], Skv, generator=g)
+    elif c["bias"] == "pad":                        # every batch row keeps a prefix of real keys, at least one
+        keep = torch.arange(Skv)[None, :] < torch.randint(1, Skv + 1, (B, 1), generator=g)
+        bias = torch.where(keep, 0.0, torch.finfo(torch.float32).min).reshape(B, 1, 1, Skv)
     seg = None
     if c["seg"] == "docs":
         seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7)
     elif c["seg"] == "one":
         seg = torch.zeros(B, max(S, Skv), dtype=torch.int32)
+    if c["bias"] == "pad" and c["seg"] == "docs":
+        seg = None                                  # a padded document's rows would see no real key at all
     kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32)
     ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
     out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
