@@ -49,7 +49,9 @@ def draw(seed):
     seg = r.choice([None, "docs", "docs", "one"])
     if r.random() < 0.15:
         bias = "pad"                                # a padding mask as a bias: where(keep, 0, finfo.min), padding on the right
-    return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cbs=cbs, B=B, H=H, bias=bias, seg=seg)
+    # blockwise_kwargs["dtype"]: the type the bias is rounded to and whose finfo.min is the mask value (:322, :298)
+    kw_dtype = r.choice([torch.float32, torch.float32, torch.bfloat16])
+    return dict(kw_dtype=kw_dtype, dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cbs=cbs, B=B, H=H, bias=bias, seg=seg)
 
 
 @pytest.mark.parametrize("seed", range(OFFSET, OFFSET + N_CASES))
@@ -69,7 +71,9 @@ def test_random_configuration_matches_oracle(seed):
         bias = torch.randn(1, H, c["qc"], Skv, generator=g)
     elif c["bias"] == "pad":                        # every batch row keeps a prefix of real keys, at least one
         keep = torch.arange(Skv)[None, :] < torch.randint(1, Skv + 1, (B, 1), generator=g)
-        bias = torch.where(keep, 0.0, torch.finfo(torch.float32).min).reshape(B, 1, 1, Skv)
+        # the mask value of the dtype the bias is rounded to (finfo(float32).min would round to -inf in bfloat16, and
+        # a first chunk of -inf logits turns the row NaN in the reference, exp(-inf - -inf); here it counts as masked)
+        bias = torch.where(keep, 0.0, torch.finfo(c["kw_dtype"]).min).reshape(B, 1, 1, Skv)
     seg = None
     if c["seg"] == "docs":
         seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7)
@@ -77,7 +81,7 @@ def test_random_configuration_matches_oracle(seed):
         seg = torch.zeros(B, max(S, Skv), dtype=torch.int32)
     if c["bias"] == "pad" and c["seg"] == "docs":
         seg = None                                  # a padded document's rows would see no real key at all
-    kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32)
+    kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=c["kw_dtype"])
     ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
     out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
     print("  family", ra.kernel_family_of_last_call(), flush=True)
