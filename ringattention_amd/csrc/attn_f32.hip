@@ -160,7 +160,9 @@ template <int KEEP>
 __device__ __forceinline__ float f32_logit(float dot_scaled, bool masked, bool kept, float bias, float mask_min) {
   if (KEEP == 2) {
     if (kept) return dot_scaled + (masked ? mask_min : bias);
-    return masked ? RA_NEG_INF : mask_min;          // dropped: mask_min added once absorbs logit and bias, twice overflows
+    // dropped: chunk_bias += mask_min (:321) before the logit is added.  Added to a bias of ordinary size it absorbs
+    // it (mask_min), added to mask_min - a masked pair, or a bias at that level: a padding mask - it overflows (-inf)
+    return dot_scaled + ((masked ? mask_min : bias) + mask_min);
   }
   if (KEEP == 1) masked = masked || !kept;
   return dot_scaled + (masked ? mask_min : bias);

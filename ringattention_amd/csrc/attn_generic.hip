@@ -81,8 +81,10 @@ __device__ __forceinline__ float logit(const MaskView& mv, const RowInfo& r, flo
     off = !((mv.kbits_k[r.kbit_off + (kk >> 6) * mv.keep_Q] >> (kk & 63)) & 1);
   }
   if (off && mv.keep_drop) {
-    // chunk_bias += dropped * finfo.min (:321): twice finfo.min overflows to -inf, once absorbs logit and bias
-    return masked ? RA_NEG_INF : mv.mask_min;
+    // chunk_bias += dropped * finfo.min (:321), before the logit is added: on top of a bias of ordinary size it
+    // absorbs bias and logit (finfo.min), on top of finfo.min - a masked pair, or a bias at that level (a padding
+    // mask) - it overflows to -inf
+    return dot / scale + ((masked ? mv.mask_min : add) + mv.mask_min);
   }
   if (off) masked = true;                  // where(mask, w, finfo.min), ringattention_inference.py:24
   if (masked) add = mv.mask_min;

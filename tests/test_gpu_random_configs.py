@@ -312,6 +312,9 @@ def test_random_dropout_configuration_matches_oracle(seed):
         bias = torch.randn(1, 1, 1, Skv, generator=g)
     elif c["bias"] == "head":
         bias = torch.randn(B, H, 1, Skv, generator=g)
+    elif c["bias"] == "pad":                        # dropped and padded: finfo.min twice, -inf (:321)
+        keep = torch.arange(Skv)[None, :] < torch.randint(1, Skv + 1, (B, 1), generator=g)
+        bias = torch.where(keep, 0.0, torch.finfo(torch.float32).min).reshape(B, 1, 1, Skv)
     seg = None
     if c["seg"] == "docs":
         seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7)
