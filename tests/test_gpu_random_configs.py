@@ -112,7 +112,7 @@ def draw_cache(seed):
         cache_idx = r.randint(0, L - 1)
     cbs = r.choice([1, 1, 1, None])
     B, H = r.choice([1, 2, 3]), r.choice([1, 2, 5])
-    bias = r.choice([None, None, "key", "head"])
+    bias = r.choice([None, None, "key", "head", "pad"])
     seg = r.choice([None, None, "docs"])
     device_idx = r.random() < 0.5                     # cache_idx as a device scalar (a traced value under jit)
     return dict(dtype=dtype, D=D, n=n, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cache_idx=cache_idx, cbs=cbs, B=B, H=H,
@@ -136,6 +136,9 @@ def test_random_cache_idx_configuration_matches_oracle(seed):
         bias = torch.randn(1, 1, 1, L, generator=g)
     elif c["bias"] == "head":
         bias = torch.randn(B, H, 1, L, generator=g)
+    elif c["bias"] == "pad":                        # a left-padded prompt: where(keep, 0, finfo.min)
+        keep = torch.arange(L)[None, :] >= torch.randint(0, L, (B, 1), generator=g)
+        bias = torch.where(keep, 0.0, torch.finfo(torch.float32).min).reshape(B, 1, 1, L)
     seg = packed_segment_ids(B, L, max(4, L // 3), seed=seed + 3) if c["seg"] == "docs" else None
     kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=torch.float32)
     ref = O.ring_attention(q, k, v, bias, seg, c["cache_idx"], n, True, oracle_kwargs(kw))
