@@ -50,6 +50,11 @@ template <> struct Vec16<float> {
   }
 };
 
+// A row of zeros: what the kernel reads in place of a cache slot behind the query's position.  Such a key is masked
+// (finfo.min absorbs its logit, :301-309) and weighs exp(finfo.min - max) = 0, but 0 times whatever an uninitialised
+// slot holds need not be 0; a cache that was zero-initialised, as the reference's is, reads the same either way.
+static __device__ __align__(16) const float dec_zero_row[256] = {};
+
 template <typename T, int D>
 __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a) {
   constexpr int EPL = Vec16<T>::N;        // elements per lane
@@ -85,18 +90,22 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
   const float scale = sqrtf((float)D);
   const T* kb = (const T*)a.k + (int64_t)b * a.kv_sb + (int64_t)hh * D + dl * EPL;
   const T* vb = (const T*)a.v + (int64_t)b * a.kv_sb + (int64_t)hh * D + dl * EPL;
+  const T* zrow = (const T*)dec_zero_row + dl * EPL;
+  // first local key behind the query's causal block (all of them when there is no causal mask)
+  const long long jd = mv.cbs > 0 ? (gq_blk + 1) * (long long)mv.cbs - mv.global_k(0) : (long long)a.L;
+  const int jdead = (int)max(0LL, min(jd, (long long)a.L));
 
   for (int j0 = ks; j0 < ke; j0 += DEC_UNROLL) {
     float kf[DEC_UNROLL][EPL], vf[DEC_UNROLL][EPL], s[DEC_UNROLL];
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
       int j = min(j0 + u, ke - 1);
-      Vec16<T>::load(kb + (int64_t)j * a.kv_ss, kf[u]);
+      Vec16<T>::load(j < jdead ? kb + (int64_t)j * a.kv_ss : zrow, kf[u]);
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
       int j = min(j0 + u, ke - 1);
-      Vec16<T>::load(vb + (int64_t)j * a.kv_ss, vf[u]);
+      Vec16<T>::load(j < jdead ? vb + (int64_t)j * a.kv_ss : zrow, vf[u]);
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {

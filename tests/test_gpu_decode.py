@@ -123,3 +123,25 @@ def test_default_workspace_is_sized_for_the_automatic_split_count():
     assert 1 <= ns <= 256
     assert decode_workspace(q, k).numel() == B * H * ns * (D + 2) * 4
     assert decode_workspace(q, k).numel() < _lib.load().ra_decode_workspace_bytes(B, L, H, D, 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cache_idx", [5, 63, 64, 700])
+def test_decode_does_not_read_cache_slots_behind_the_query(cache_idx, dtype):
+    """A cache allocated with torch.empty holds anything behind the last token written, NaN included.  Those keys are
+    masked and weigh 0, but 0 * NaN is NaN: the streaming kernel reads zeros in their place - what a zero-initialised
+    cache, the reference's kind, holds there - so the result is that of the zero-filled cache, bit for bit."""
+    B, L, H, D, kc = 2, 1024, 4, 128, 64
+    q, k, v, _ = make_qkv(B, 1, H, D, dtype=dtype, seed=cache_idx, Skv=L)
+    kw = kwargs(1, kc, 1)
+    kz, vz = k.clone(), v.clone()
+    kz[:, cache_idx + 1:] = 0
+    vz[:, cache_idx + 1:] = 0
+    kn, vn = kz.clone(), vz.clone()
+    kn[:, cache_idx + 1:] = float("nan")
+    vn[:, cache_idx + 1:] = float("inf")
+    clean = ra.ringattention(q.to(DEV), kz.to(DEV), vz.to(DEV), None, None, cache_idx, None, True, kw)
+    dirty = ra.ringattention(q.to(DEV), kn.to(DEV), vn.to(DEV), None, None, cache_idx, None, True, kw)
+    assert torch.isfinite(dirty).all() and torch.equal(clean, dirty)
+    ref = O.ring_attention(q, kz, vz, None, None, cache_idx, 1, True, oracle_kwargs(kw))
+    assert_close(dirty, ref, dtype, "decode over a dirty cache")
