@@ -179,6 +179,19 @@ def _slab_tokens(chunk_size, n_chunks, launch_tokens=None):
 _TOKEN_GRID = 128       # tokens per launch are a multiple of this (rows of a GEMM tile)
 
 
+def _check_swiglu_weights(ff, x):
+    """The kernels read the three weights as dense bf16 (in, out) arrays on x's device: anything else (a module moved
+    to fp32, a transposed view) would be read as garbage, so it is refused."""
+    d, f = ff.w1.shape
+    for name, w, shape in (("w1", ff.w1, (d, f)), ("w3", ff.w3, (d, f)), ("w2", ff.w2, (f, d))):
+        if w.dtype != torch.bfloat16:
+            raise NotImplementedError("SwiGLU kernels are bf16: %s is %s" % (name, w.dtype))
+        if tuple(w.shape) != shape or not w.is_contiguous() or w.device != x.device:
+            raise ValueError("SwiGLU weight %s must be a contiguous %s array on %s" % (name, shape, x.device))
+    if x.shape[-1] != d:
+        raise ValueError("hidden size %d of the input does not match the weights' %d" % (x.shape[-1], d))
+
+
 class SwiGLU(torch.nn.Module):
     """The LLaMA-style MLP the reference's README pairs with blockwise_feedforward:
     w2(silu(x w1) * (x w3)); weights stored (in, out), bf16."""
@@ -200,6 +213,7 @@ class SwiGLU(torch.nn.Module):
             raise NotImplementedError("SwiGLU kernels are bf16")
         if not x.is_cuda:
             raise RuntimeError("ringattention_amd runs on the GPU only")
+        _check_swiglu_weights(self, x)
         T = x.shape[0]
         if T == 0:                  # nothing to launch; the zero keeps the empty result attached to its inputs
             zero = 0.0 * (self.w1.sum() + self.w2.sum() + self.w3.sum())
@@ -246,6 +260,7 @@ def blockwise_feedforward(feedforward, inputs, chunk_size, static_argnums=(1,), 
             raise RuntimeError("ringattention_amd runs on the GPU only")
         # contiguous slabs of chunk_size tokens (batch rows one after the other: a token-wise MLP does not see the
         # difference), one autograd node for the whole scan
+        _check_swiglu_weights(feedforward, inputs)
         x2 = inputs.reshape(b * s, d)
         step, steps = chunk_size, b * n
         if chunk_size % _TOKEN_GRID:

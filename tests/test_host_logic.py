@@ -296,3 +296,19 @@ def test_blockwise_feedforward_generic_callable_groups_and_remat():
     calls.clear()
     ra.blockwise_feedforward(ff, x, 6, pre_remat=False, policy="everything_saveable").sum().backward()
     assert len(calls) == 4
+
+
+def test_swiglu_weights_must_be_dense_bf16():
+    """A module moved to fp32 or given a transposed weight would be read as garbage by kernels that take raw bf16
+    pointers: refused before anything is launched (the check runs on the host; no GPU needed)."""
+    from ringattention_amd import feedforward as F
+    ff = F.SwiGLU(128, 256, device="cpu")
+    x = torch.zeros(4, 128, dtype=torch.bfloat16)
+    F._check_swiglu_weights(ff, x)
+    with pytest.raises(ValueError):
+        F._check_swiglu_weights(ff, torch.zeros(4, 64, dtype=torch.bfloat16))
+    ff.w2.data = ff.w2.data.t().contiguous().t()
+    with pytest.raises(ValueError):
+        F._check_swiglu_weights(ff, x)
+    with pytest.raises(NotImplementedError):
+        F._check_swiglu_weights(F.SwiGLU(128, 256, device="cpu").float(), x)
