@@ -574,3 +574,48 @@ def test_rmsnorm_residual_definition_invariances_and_gradient():
     dy = rstd * gw - yd * rstd ** 3 / d * (gw * yd).sum(-1, keepdim=True) + dres
     assert torch.allclose(xx.grad, dy, rtol=1e-10, atol=1e-12)
     assert torch.allclose(ww.grad, (dn * yd * rstd).sum(0), rtol=1e-10, atol=1e-12)
+
+
+@pytest.mark.parametrize("n,qc,kc", [(1, 8, 8), (2, 8, 16), (4, 4, 4)])
+def test_padding_mask_as_bias_equals_attention_over_the_real_keys(n, qc, kc):
+    """A bias of finfo.min on padded keys (how a model passes its padding mask) must act as if those keys were not
+    there at all, for every row that sees a real key: checked against a causal softmax in float64 over the real keys
+    only, written here from the definition (keys sliced away, not masked), forward and - through autograd - backward.
+    Rows that see padded keys only (left padding) take equal weights over the keys of the chunks that run."""
+    B, S, H, D = 2, 64, 2, 8
+    q, k, v = make(B, S, H, D, seed=11, dtype=torch.float32)
+    keep = torch.ones(B, S, dtype=torch.bool)
+    keep[0, 50:] = False                                     # right padding
+    keep[1, :5] = False                                      # left padding
+    bias = torch.where(keep, 0.0, torch.finfo(torch.float32).min).reshape(B, 1, 1, S)
+    kw = kwargs(qc, kc, 1)
+    g = torch.randn(B, S, H, D, generator=torch.Generator().manual_seed(12))
+    g[1, :5] = 0                                             # no cotangent where no real key is seen
+    out, res = O.ring_attention_fwd(q, k, v, bias, None, None, n, True, kw)
+    dq, dk, dv = O.ring_attention_bwd(n, True, kw, res, g)
+    qa, ka, va = (t.double().requires_grad_(True) for t in (q, k, v))
+    ref = torch.zeros(B, S, H, D, dtype=F64)
+    rows = []
+    for b in range(B):
+        real = torch.nonzero(keep[b]).flatten()
+        for i in range(S):
+            vis = real[real <= i]
+            if vis.numel() == 0:
+                continue
+            w = torch.softmax(torch.einsum("hd,khd->hk", qa[b, i], ka[b, vis]) / D ** 0.5, dim=-1)
+            rows.append((b, i, torch.einsum("hk,khd->hd", w, va[b, vis])))
+    loss = 0.0
+    for b, i, o in rows:
+        ref[b, i] = o.detach()
+        loss = loss + (o * g[b, i].double()).sum()
+    loss.backward()
+    seen = torch.zeros(B, S, dtype=torch.bool)
+    for b, i, _ in rows:
+        seen[b, i] = True
+    assert int((~seen).sum()) == 5
+    assert float((out.double() - ref)[seen].abs().max()) < 2e-6
+    for a, r in ((dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
+        assert float((a.double() - r).abs().max()) < 2e-5
+    assert float(dk[0, 50:].abs().max()) == 0.0 and float(dv[0, 50:].abs().max()) == 0.0
+    # rows 0..4 of batch row 1: equal weights over the keys of the chunks that run for them (:138-144)
+    assert torch.isfinite(out[1, :5]).all()
