@@ -46,7 +46,7 @@ def draw(seed):
         cbs = 1                                     # :327-330 divide block size and chunk sizes by one another
     B, H = r.choice([1, 1, 2]), r.choice([1, 2, 3])
     bias = r.choice([None, None, "key", "key", "head", "row"])
-    seg = r.choice([None, "docs", "docs", "one"])
+    seg = r.choice([None, "docs", "docs", "one", "relabelled"])
     if r.random() < 0.15:
         bias = "pad"                                # a padding mask as a bias: where(keep, 0, finfo.min), padding on the right
     # blockwise_kwargs["dtype"]: the type the bias is rounded to and whose finfo.min is the mask value (:322, :298)
@@ -77,11 +77,16 @@ def test_random_configuration_matches_oracle(seed):
         # a first chunk of -inf logits turns the row NaN in the reference, exp(-inf - -inf); here it counts as masked)
         bias = torch.where(keep, 0.0, torch.finfo(c["kw_dtype"]).min).reshape(B, 1, 1, Skv)
     seg = None
-    if c["seg"] == "docs":
+    if c["seg"] in ("docs", "relabelled"):
         seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7)
     elif c["seg"] == "one":
         seg = torch.zeros(B, max(S, Skv), dtype=torch.int32)
-    if c["bias"] == "pad" and c["seg"] == "docs":
+    if c["seg"] == "relabelled":
+        # ids in no order and used more than once (the reference compares them for equality only, :294: two documents
+        # with one id see each other across what lies between), one row of ids for the whole batch
+        table = torch.randint(-3, 4, (int(seg.max()) + 1,), generator=g, dtype=torch.int32)
+        seg = table[seg[:1].long()]
+    if c["bias"] == "pad" and c["seg"] in ("docs", "relabelled"):
         seg = None                                  # a padded document's rows would see no real key at all
     kw = kwargs(c["qc"], c["kc"], c["cbs"], dtype=c["kw_dtype"])
     ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)

@@ -73,9 +73,10 @@ def assert_close(got, ref, dtype, what=""):
 def assert_close_scaled(got, ref, dtype, what=""):
     """assert_close for results that may be large (sharp softmax rows, q and k of standard deviation 3: gradients
     of 10 - 60).  The max-abs bars of 2e-2 / 1e-4 are meant for results of order one; beyond that they scale with the
-    largest reference element: for the 16-bit types two bf16 units in the last place of it (one is what two
+    largest reference element: for the 16-bit types three bf16 units in the last place of it (one is what two
     roundings a boundary apart differ by, 3.1e-2 for a value in [4, 8); the weights P and dS are themselves rounded
-    to bf16 before their second product, 2^-9 relative on the terms that dominate a sharp row), for fp32 3e-5 of it
+    to bf16 before their second product, 2^-9 relative each on the terms that dominate a sharp row, and the result is
+    rounded once more), for fp32 3e-5 of it
     (a logit of 40 carries 40 fp32 roundings' worth of error into its exponential, on either side).
     The relative L2 bar stays as it is."""
     ma, rl = errors(got, ref)
@@ -85,7 +86,7 @@ def assert_close_scaled(got, ref, dtype, what=""):
     top = float(finite.abs().max()) if finite.numel() else 0.0
     if top > 0.0:
         if dtype != torch.float32:
-            tol_abs = max(tol_abs, 2.002 * 2.0 ** (math.floor(math.log2(top)) - 7))
+            tol_abs = max(tol_abs, 3.0 * 2.0 ** (math.floor(math.log2(top)) - 7))
         else:
             tol_abs = max(tol_abs, 3e-5 * top)
     if ma <= 1e-5:
