@@ -50,11 +50,6 @@ template <> struct Vec16<float> {
   }
 };
 
-// A row of zeros: what the kernel reads in place of a cache slot behind the query's position.  Such a key is masked
-// (finfo.min absorbs its logit, :301-309) and weighs exp(finfo.min - max) = 0, but 0 times whatever an uninitialised
-// slot holds need not be 0; a cache that was zero-initialised, as the reference's is, reads the same either way.
-static __device__ __align__(16) const float dec_zero_row[256] = {};
-
 template <typename T, int D>
 __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a) {
   constexpr int EPL = Vec16<T>::N;        // elements per lane
@@ -90,8 +85,10 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
   const float scale = sqrtf((float)D);
   const T* kb = (const T*)a.k + (int64_t)b * a.kv_sb + (int64_t)hh * D + dl * EPL;
   const T* vb = (const T*)a.v + (int64_t)b * a.kv_sb + (int64_t)hh * D + dl * EPL;
-  const T* zrow = (const T*)dec_zero_row + dl * EPL;
-  // first local key behind the query's causal block (all of them when there is no causal mask)
+  // First local key behind the query's causal block (none when there is no causal mask).  From there on the cache may
+  // never have been written: such a key is masked - finfo.min absorbs its logit, so the logit is not looked at - and
+  // where its weight exp(finfo.min - max) is 0 its value is not multiplied (0 times an uninitialised slot's NaN or inf
+  // is not 0).  With finite data in those slots nothing changes, bit for bit.
   const long long jd = mv.cbs > 0 ? (gq_blk + 1) * (long long)mv.cbs - mv.global_k(0) : (long long)a.L;
   const int jdead = (int)max(0LL, min(jd, (long long)a.L));
 
@@ -100,12 +97,12 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
       int j = min(j0 + u, ke - 1);
-      Vec16<T>::load(j < jdead ? kb + (int64_t)j * a.kv_ss : zrow, kf[u]);
+      Vec16<T>::load(kb + (int64_t)j * a.kv_ss, kf[u]);
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
       int j = min(j0 + u, ke - 1);
-      Vec16<T>::load(j < jdead ? vb + (int64_t)j * a.kv_ss : zrow, vf[u]);
+      Vec16<T>::load(vb + (int64_t)j * a.kv_ss, vf[u]);
     }
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) {
@@ -135,8 +132,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
         int idx = clamp_seg_index((mv.k_start + (long long)(jj / mv.kc)) * mv.kc, mv.kc, mv.seg_len, jj % mv.kc);
         masked = masked || (mv.seg[(int64_t)b * mv.seg_sb + idx] != seg_q);
       }
-      if (masked) add = mv.mask_min;
-      s[u] = (j < ke) ? s[u] / scale + add : RA_NEG_INF;
+      s[u] = (j < ke) ? (masked ? mv.mask_min : s[u] / scale + add) : RA_NEG_INF;
       tile_max = fmaxf(tile_max, s[u]);
     }
     const float m_new = fmaxf(m, tile_max);
@@ -144,12 +140,22 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
     float psum = 0.f;
 #pragma unroll
     for (int u = 0; u < DEC_UNROLL; u++) { s[u] = expf(s[u] - m_new); psum += s[u]; }
+    if (j0 + DEC_UNROLL > jdead) {           // the few steps that reach behind the query
 #pragma unroll
-    for (int e = 0; e < EPL; e++) {
-      float t = 0.f;
+      for (int e = 0; e < EPL; e++) {
+        float t = 0.f;
 #pragma unroll
-      for (int u = 0; u < DEC_UNROLL; u++) t = fmaf(s[u], vf[u][e], t);
-      acc[e] = acc[e] * corr + t;
+        for (int u = 0; u < DEC_UNROLL; u++) t = s[u] != 0.f ? fmaf(s[u], vf[u][e], t) : t;
+        acc[e] = acc[e] * corr + t;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPL; e++) {
+        float t = 0.f;
+#pragma unroll
+        for (int u = 0; u < DEC_UNROLL; u++) t = fmaf(s[u], vf[u][e], t);
+        acc[e] = acc[e] * corr + t;
+      }
     }
     l = l * corr + psum;
     m = m_new;
@@ -181,15 +187,20 @@ __global__ void decode_combine_kernel(DecodeArgs a) {
     M = fmaxf(M, m_in);
   }
   float num = 0.f, den = 0.f;
+  // a part whose factor is 0 is left out rather than multiplied: a split that saw masked keys only (its own weights
+  // are 1 then) may have summed what uninitialised cache slots hold, and 0 times inf is not 0
   if (merge && m_in != RA_NEG_INF) {
     const float c = expf(m_in - M);
-    num = c * num_in;
-    den = c * den_in;
+    if (c != 0.f) {
+      num = c * num_in;
+      den = c * den_in;
+    }
   }
   for (int s = 0; s < a.nsplit; s++) {
     const float ms = w[s * (D + 2) + D];
     if (ms == RA_NEG_INF) continue;
     const float c = expf(ms - M);
+    if (c == 0.f) continue;
     num = fmaf(c, w[s * (D + 2) + d], num);
     den = fmaf(c, w[s * (D + 2) + D + 1], den);
   }

@@ -129,8 +129,8 @@ def test_default_workspace_is_sized_for_the_automatic_split_count():
 @pytest.mark.parametrize("cache_idx", [5, 63, 64, 700])
 def test_decode_does_not_read_cache_slots_behind_the_query(cache_idx, dtype):
     """A cache allocated with torch.empty holds anything behind the last token written, NaN included.  Those keys are
-    masked and weigh 0, but 0 * NaN is NaN: the streaming kernel reads zeros in their place - what a zero-initialised
-    cache, the reference's kind, holds there - so the result is that of the zero-filled cache, bit for bit."""
+    masked and weigh 0, but 0 * NaN is NaN: the streaming kernel neither looks at a masked key's logit nor multiplies a
+    value by a weight of 0 there, so the result is that of the zero-filled cache, bit for bit."""
     B, L, H, D, kc = 2, 1024, 4, 128, 64
     q, k, v, _ = make_qkv(B, 1, H, D, dtype=dtype, seed=cache_idx, Skv=L)
     kw = kwargs(1, kc, 1)
