@@ -212,7 +212,7 @@ def test_random_blockwise_feedforward_matches_oracle(seed):
 def draw_inference(seed):
     r = random.Random(13000 + seed)
     dtype = r.choice([torch.float32, torch.bfloat16, torch.bfloat16, torch.float16])
-    D = r.choice([32, 40, 64, 96, 128, 128, 128, 160])
+    D = r.choice([32, 40, 64, 96, 128, 128, 128, 160, 256])
     n = r.choice([1, 2, 2, 4])
     per_dev = r.choice([8, 24, 64, 100, 128, 256, 256, 512])
     B, H = r.choice([1, 2]), r.choice([1, 2, 3])
@@ -246,8 +246,17 @@ def test_random_inference_configuration_matches_oracle(seed):
     ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
     ref_grads = O.ring_attention_inference_bwd(n, res, do)
     qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    # the mask as callers hold it: boolean, or 0 / 1 in another type; dense, or a broadcast view
+    md = mask.cuda()
+    form = seed % 4
+    if form == 1:
+        md = md.to(torch.uint8)
+    elif form == 2:
+        md = md.to(torch.float32)
+    elif form == 3 and md.shape[1] == 1:
+        md = md.expand(md.shape[0], H, md.shape[2], md.shape[3])
     with ra.ring_axis("sp", n):
-        out = ra.ringattention_inference(qd, kd, vd, mask.cuda(), "sp", True)
+        out = ra.ringattention_inference(qd, kd, vd, md, "sp", True)
     out.backward(do.cuda())
     torch.cuda.synchronize()
     tol_dtype = torch.float32 if c["dtype"] == torch.float32 else torch.bfloat16
