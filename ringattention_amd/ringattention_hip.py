@@ -1080,6 +1080,53 @@ def _saved_residuals(ctx):
     return out, q, k, v, mi, cfg, n, den, mx
 
 
+def _pad_lengths_to_mfma_grid(q, k, v, attn_bias, segment_ids, cache_idx, n, axis_name, float32_logits,
+                              blockwise_kwargs, grid=128):
+    """One device, equal query and key lengths that are no multiple of 128 (a prompt of 5000 tokens in chunks of
+    500): the matrix-core kernels tile 128 positions, so such a call would take the vector kernels, a few hundred times
+    slower.  Where the chunking cannot change the result (the conditions of _fit_chunks_to_mfma_grid) the call is
+    made on arrays padded to the next multiple of 128 instead, in chunks of 128, and the result cut back:
+    the padded keys are masked for every real row - they lie behind it under a causal mask, and carry a segment id
+    of their own otherwise - so each real row sums over exactly its own pairs, and the padded rows, whose output is
+    dropped, get no cotangent.  Returns the result, or None when the call is left as it is."""
+    kw = dict(blockwise_kwargs)
+    B, S, H, D = q.shape
+    if n != 1 or cache_idx is not None or k.shape[1] != S or S % grid == 0 or D > 128:
+        return None
+    if q.dtype not in (torch.bfloat16, torch.float32) or kw.get("impl", "auto") == "generic":
+        return None
+    if kw.get("skip_masked_tiles", None) is False or kw.get("_padded", False):
+        return None
+    if (not kw.get("deterministic", True)) and float(kw.get("attn_pdrop", 0.0)) > 0.0:
+        return None                    # the dropout mask is drawn for the shape of the call
+    qc, kc, cbs = int(kw["query_chunk_size"]), int(kw["key_chunk_size"]), kw.get("causal_block_size", None)
+    if S % qc or S % kc:
+        return None                    # refused further down, with the reference's message
+    if cbs is not None:
+        cbs = int(cbs)
+        if (cbs == 1 and (qc % 2 or kc % 2)) or (cbs > 1 and (qc % cbs or kc % cbs or grid % cbs)):
+            return None
+    if attn_bias is not None and (attn_bias.dim() != 4 or attn_bias.shape[2] != 1 or attn_bias.shape[3] != S):
+        return None
+    if segment_ids is not None and (segment_ids.dim() != 2 or segment_ids.shape[1] != S):
+        return None
+    if cbs is None and segment_ids is None and attn_bias is not None:
+        return None                    # the segment ids added below would switch the clamp of the bias on (:299)
+    pad = grid - S % grid
+    qp, kp, vp = (torch.nn.functional.pad(t, (0, 0, 0, 0, 0, pad)) for t in (q, k, v))
+    bias_p = None if attn_bias is None else torch.nn.functional.pad(attn_bias.detach(), (0, pad))
+    seg_p = segment_ids
+    if cbs is None or segment_ids is not None:
+        # without a causal mask only a segment id of their own keeps the padded keys away from the real rows
+        ids = segment_ids.detach().to(torch.int32) if segment_ids is not None else \
+            torch.zeros((1, S), dtype=torch.int32, device=q.device)
+        own = (ids.max() + 1).reshape(1, 1).expand(ids.shape[0], pad)
+        seg_p = torch.cat((ids, own), dim=1)
+    kw.update(query_chunk_size=grid, key_chunk_size=grid, skip_masked_tiles=True, _padded=True)
+    out = ring_attention(qp, kp, vp, bias_p, seg_p, None, axis_name, float32_logits, kw)
+    return out[:, :S].contiguous()
+
+
 def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float32_logits, blockwise_kwargs):
     """Drop-in for ringattention_jax.py:92-97 (exported as ``ringattention``).
 
@@ -1104,6 +1151,10 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
         fill = float("nan") if q.numel() else 0.0
         return torch.full_like(q, fill) + 0.0 * (q.sum() + k.sum() + v.sum()).to(q.dtype)
     n = axis_size(axis_name)
+    padded = _pad_lengths_to_mfma_grid(q, k, v, attn_bias, segment_ids, cache_idx, n, axis_name, float32_logits,
+                                       blockwise_kwargs)
+    if padded is not None:
+        return padded
     if cache_idx is not None and q.shape[1] == n and q.shape[3] in (64, 128) and not (
             torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) \
             and int(dict(blockwise_kwargs)["query_chunk_size"]) == 1:

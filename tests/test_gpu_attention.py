@@ -837,3 +837,27 @@ def test_padding_mask_as_bias_matches_oracle(dtype, D, chunk, n, skip):
         assert_close(a, b, dtype, name)
     # padded keys get no gradient from rows that see a real key as well
     assert float(grads[1][0, 900:].abs().max()) == 0.0 and float(grads[2][0, 900:].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("S,chunk,cbs,use_bias,use_seg", [
+    (1000, 100, 1, False, False), (1000, 250, 1, True, True), (5000, 500, 1, False, True), (1000, 500, None, False, False),
+    (1000, 200, None, False, True), (1000, 200, None, True, True), (1016, 8, 8, True, False), (72, 24, 1, False, False)])
+def test_lengths_off_the_128_grid_run_on_the_matrix_cores(S, chunk, cbs, use_bias, use_seg, dtype):
+    """One device, a length that is no multiple of 128, chunk sizes that divide it (as the reference asks): the call
+    is made on arrays padded to the next multiple of 128 and cut back, where the chunking cannot change the result;
+    forward and backward against the oracle run at the original length and chunk sizes."""
+    B, H, D = 2, 2, 128 if dtype == torch.bfloat16 else 64
+    q, k, v, do = make_qkv(B, S, H, D, dtype=dtype, seed=S + chunk, scale=D ** -0.25)
+    g = torch.Generator().manual_seed(S)
+    bias = torch.randn(B, 1, 1, S, generator=g) if use_bias else None
+    seg = packed_segment_ids(B, S, S // 4, seed=S) if use_seg else None
+    kw = kwargs(chunk, chunk, cbs)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, 1, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, 1, kw)
+    fam = ra.kernel_family_of_last_call()
+    assert out.shape == q.shape and "mfma" in fam["forward"] and "mfma" in fam["backward"], fam
+    assert_close(out, ref_out, dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert a.shape == q.shape
+        assert_close(a, b, dtype, name)
