@@ -415,7 +415,9 @@ static int check_decode(const ra_decode_params* p, const char* who) {
   RA_REQUIRE(p->out || carry, RA_ERR_INVALID, "%s: out may be null only in a ring step that hands on a carry", who);
   RA_REQUIRE(p->dtype == RA_F32 || p->dtype == RA_BF16, RA_ERR_UNSUPPORTED, "%s: dtype %d", who, p->dtype);
   RA_REQUIRE(p->B > 0 && p->L > 0 && p->H > 0 && p->D > 0 && p->B <= 65535, RA_ERR_INVALID, "%s: bad shape", who);
-  RA_REQUIRE(p->D == 64 || p->D == 128, RA_ERR_UNSUPPORTED, "%s: head size %d not in {64, 128}", who, p->D);
+  RA_REQUIRE(p->D == 32 || p->D == 40 || p->D == 64 || p->D == 80 || p->D == 96 || p->D == 112 || p->D == 128 ||
+                 p->D == 160 || p->D == 192 || p->D == 256,
+             RA_ERR_UNSUPPORTED, "%s: head size %d not in {32, 40, 64, 80, 96, 112, 128, 160, 192, 256}", who, p->D);
   RA_REQUIRE(p->mask.query_chunk_size == 1, RA_ERR_INVALID,
              "%s: one query token needs query_chunk_size == 1 (q_len // query_chunk_size chunks)", who);
   if (int rc = check_mask(p->mask, 1, p->L, who)) return rc;

@@ -50,16 +50,23 @@ template <> struct Vec16<float> {
   }
 };
 
+constexpr int dec_pow2_ge(int x) { int p = 1; while (p < x) p <<= 1; return p; }
+
+// D: any multiple of the 16 bytes a lane loads (8 bf16 / 4 fp32 elements).  A head's elements take D / EPL lanes; the
+// group of lanes that reduces a logit is the next power of two, and the lanes beyond the head's (head size 96: 12 of
+// 16) go along with a zero query - they load what lane 0 loads and write nothing.
 template <typename T, int D>
 __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a) {
   constexpr int EPL = Vec16<T>::N;        // elements per lane
-  constexpr int LPH = D / EPL;            // lanes per head
+  constexpr int LPA = D / EPL;            // lanes that hold a head's elements
+  constexpr int LPH = dec_pow2_ge(LPA);   // lanes per head
   constexpr int HP = DEC_THREADS / LPH;   // heads per workgroup
   MaskView mv = a.mv;
   mv.resolve();                      // query_chunk_size == 1: q_start = cache_idx (:35)
   const int tid = threadIdx.x, b = blockIdx.z, split = blockIdx.x;
   const int h = blockIdx.y * HP + tid / LPH;
-  const int dl = tid % LPH;
+  const bool lane_on = tid % LPH < LPA;
+  const int dl = lane_on ? tid % LPH : 0;
   const bool hvalid = h < a.H;
   const int hh = hvalid ? h : a.H - 1;
 
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
   float qf[EPL], acc[EPL];
   Vec16<T>::load((const T*)a.q + (int64_t)b * a.q_sb + (int64_t)hh * D + dl * EPL, qf);
 #pragma unroll
-  for (int e = 0; e < EPL; e++) acc[e] = 0.f;
+  for (int e = 0; e < EPL; e++) { acc[e] = 0.f; if (LPA != LPH && !lane_on) qf[e] = 0.f; }
   float m = RA_NEG_INF, l = 0.f;
   const float scale = sqrtf((float)D);
   const T* kb = (const T*)a.k + (int64_t)b * a.kv_sb + (int64_t)hh * D + dl * EPL;
@@ -160,7 +167,7 @@ __global__ __launch_bounds__(DEC_THREADS) void decode_split_kernel(DecodeArgs a)
     l = l * corr + psum;
     m = m_new;
   }
-  if (hvalid) {
+  if (hvalid && lane_on) {
     float* w = a.ws + (((int64_t)b * a.H + h) * a.nsplit + split) * (D + 2);
 #pragma unroll
     for (int e = 0; e < EPL; e++) w[dl * EPL + e] = acc[e];
@@ -217,7 +224,7 @@ __global__ void decode_combine_kernel(DecodeArgs a) {
 
 int decode_pick_splits(int B, int L, int H, int D, int dtype) {
   const int epl = dtype == RA_F32 ? 4 : 8;
-  const int hp = DEC_THREADS / (D / epl);
+  const int hp = DEC_THREADS / dec_pow2_ge(D / epl);
   const int hg = (H + hp - 1) / hp;
   int want = (2048 + B * hg - 1) / (B * hg);
   int maxs = (L + 255) / 256;
@@ -229,7 +236,7 @@ int decode_pick_splits(int B, int L, int H, int D, int dtype) {
 
 template <typename T, int D>
 static int launch_decode(const DecodeArgs& a, hipStream_t s) {
-  constexpr int LPH = D / Vec16<T>::N;
+  constexpr int LPH = dec_pow2_ge(D / Vec16<T>::N);
   constexpr int HP = DEC_THREADS / LPH;
   dim3 grid(a.nsplit, (a.H + HP - 1) / HP, a.B);
   decode_split_kernel<T, D><<<grid, DEC_THREADS, 0, s>>>(a);
@@ -286,14 +293,12 @@ int decode_fwd(const ra_decode_params* p, float* partials, int nsplit, hipStream
   a.c_num = p->carry_numerator; a.c_den = p->carry_denominator; a.c_max = p->carry_max_score;
   a.c_num_sb = p->carry_num_stride_b; a.c_stat_sb = p->carry_stat_stride_b;
   a.carry_is_initial = p->carry_is_initial;
-  if (p->dtype == RA_BF16) {
-    if (p->D == 128) return launch_decode<uint16_t, 128>(a, s);
-    if (p->D == 64) return launch_decode<uint16_t, 64>(a, s);
-  } else {
-    if (p->D == 128) return launch_decode<float, 128>(a, s);
-    if (p->D == 64) return launch_decode<float, 64>(a, s);
-  }
-  set_error("decode: head size %d not in {64,128}", p->D);
+#define RA_DECODE_D(DD)                                                              \
+  if (p->D == DD) return p->dtype == RA_BF16 ? launch_decode<uint16_t, DD>(a, s) : launch_decode<float, DD>(a, s);
+  RA_DECODE_D(128) RA_DECODE_D(64) RA_DECODE_D(256) RA_DECODE_D(32) RA_DECODE_D(40) RA_DECODE_D(80) RA_DECODE_D(96)
+  RA_DECODE_D(112) RA_DECODE_D(160) RA_DECODE_D(192)
+#undef RA_DECODE_D
+  set_error("decode: head size %d not in {32,40,64,80,96,112,128,160,192,256}", p->D);
   return RA_ERR_UNSUPPORTED;
 }
 

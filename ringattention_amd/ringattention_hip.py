@@ -1080,6 +1080,9 @@ def _saved_residuals(ctx):
     return out, q, k, v, mi, cfg, n, den, mx
 
 
+_DECODE_HEAD_SIZES = (32, 40, 64, 80, 96, 112, 128, 160, 192, 256)     # what decode_split_kernel is instantiated for
+
+
 def _pad_lengths_to_mfma_grid(q, k, v, attn_bias, segment_ids, cache_idx, n, axis_name, float32_logits,
                               blockwise_kwargs, grid=128):
     """One device, equal query and key lengths that are no multiple of 128 (a prompt of 5000 tokens in chunks of
@@ -1134,8 +1137,8 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
     arrays and the sequence axis is split over the virtual devices.  attn_bias (B|1, H|1, 1, K_total)
     and segment_ids (B|1, S_total) are global / replicated, as in the reference's shard_map specs.
     One query token with cache_idx set takes the streaming decode kernel."""
-    # (the streaming kernel serves head sizes 64 and 128; any other takes the blockwise kernels below, like a call
-    # that wants gradients)
+    # (a head size the streaming kernel is not built for takes the blockwise kernels below, like a call that wants
+    # gradients)
     if q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16:
         # float16 inputs: with float32_logits the reference casts q and k to fp32 (:18-19) and the products with v
         # promote to fp32 as well, so computing on exact fp32 copies (the fp32 matrix-core kernels) and rounding the
@@ -1155,7 +1158,7 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
                                        blockwise_kwargs)
     if padded is not None:
         return padded
-    if cache_idx is not None and q.shape[1] == n and q.shape[3] in (64, 128) and not (
+    if cache_idx is not None and q.shape[1] == n and q.shape[3] in _DECODE_HEAD_SIZES and not (
             torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)) \
             and int(dict(blockwise_kwargs)["query_chunk_size"]) == 1:
         from .decode import decode_attention, decode_attention_ring

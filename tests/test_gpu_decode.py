@@ -145,3 +145,25 @@ def test_decode_does_not_read_cache_slots_behind_the_query(cache_idx, dtype):
     assert torch.isfinite(dirty).all() and torch.equal(clean, dirty)
     ref = O.ring_attention(q, kz, vz, None, None, cache_idx, 1, True, oracle_kwargs(kw))
     assert_close(dirty, ref, dtype, "decode over a dirty cache")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 40, 80, 96, 112, 160, 192, 256])
+@pytest.mark.parametrize("n", [1, 2])
+def test_decode_head_sizes(D, dtype, n):
+    """The streaming kernel at the other head sizes it is built for - among them those whose elements take a number of
+    lanes that is no power of two (96: 12 of a group of 16) -, alone and as a ring of 2."""
+    B, L, H, kc, cache_idx = 2, 2048, 3, 128, 1500
+    q, k, v, _ = make_qkv(B, n, H, D, dtype=dtype, seed=D + n, Skv=L)
+    g = torch.Generator().manual_seed(D)
+    bias = torch.randn(B, 1, 1, L, generator=g)
+    seg = packed_segment_ids(B, L, 900, seed=D)
+    kw = kwargs(1, kc, 1)
+    ref = O.ring_attention(q, k, v, bias, seg, cache_idx, n, True, oracle_kwargs(kw))
+    with ra.ring_axis("sp", n):
+        out = ra.ringattention(q.to(DEV), k.to(DEV), v.to(DEV), bias.to(DEV), seg.to(DEV), cache_idx, axis_name="sp",
+                               float32_logits=True, blockwise_kwargs=kw)
+        slow = ra.ringattention(q.to(DEV).requires_grad_(True), k.to(DEV), v.to(DEV), bias.to(DEV), seg.to(DEV),
+                                cache_idx, axis_name="sp", float32_logits=True, blockwise_kwargs=kw)
+    assert_close(out, ref, dtype, "decode D %d" % D)
+    assert errors(out, slow)[0] <= (2e-2 if dtype == torch.bfloat16 else 1e-5)
