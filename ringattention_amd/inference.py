@@ -1,7 +1,8 @@
 """ring_attention_inference (ringattention/ringattention_inference.py:8-73): the ring with a boolean
-attention mask and no chunking inside a ring step.  bf16 inputs with head size 128 and shard lengths that
-are multiples of 256 run on the MFMA kernels, which read the mask in a packed form (ra_keep_pack);
-anything else runs on the fp32 vector-ALU kernels."""
+attention mask and no chunking inside a ring step.  bf16 / fp32 / fp16 inputs with head sizes up to 128 run on
+the MFMA kernels, which read the mask in a packed form (ra_keep_pack): shard lengths that are no multiple of 128
+are padded to one (_pad_lengths) unless some row of the mask attends to nothing; that case and head sizes
+above 128 run on the fp32 vector-ALU kernels."""
 import torch
 
 from . import _lib as L
@@ -109,6 +110,38 @@ class _RingAttentionInferenceFn(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None
 
 
+def _pad_lengths(q, k, v, attn_mask, axis_name, float32_logits, n, grid=128):
+    """Lengths whose shards are no multiple of 128 (a prompt of 1000 tokens): the matrix-core kernels tile 128
+    positions and read the mask packed in words of 64, so such a call would take the vector kernels.  The mask says
+    who attends to whom and positions mean nothing else here, so q, k, v and the mask are padded at the end to the
+    next multiple of 128 per device and the result is cut back: the new keys are attended to by no real row, the new
+    rows - whose output is dropped and which get no cotangent - attend to the new keys (or to key 0 when only rows
+    were added), so no row is left without a key.  A real row that attends to nothing averages over all keys
+    (ringattention_inference.py:22-24), padded ones included: a mask with such a row is left as it is.  Returns the
+    result, or None."""
+    B, Q, H, D = q.shape
+    K = k.shape[1]
+    step = grid * n
+    if (Q % step == 0 and K % step == 0) or q.dtype not in (torch.bfloat16, torch.float32) or D > 128:
+        return None
+    if attn_mask.dim() != 4 or attn_mask.shape[3] != K or attn_mask.shape[2] not in (1, Q):
+        return None                    # refused further down, with the message for it
+    m = attn_mask if attn_mask.dtype == torch.bool else attn_mask != 0
+    if not bool(m.any(dim=-1).all()):
+        return None
+    pq, pk = -Q % step, -K % step
+    rows = m.shape[2] > 1
+    mp = torch.nn.functional.pad(m, (0, pk, 0, pq if rows else 0), value=False)
+    if rows and pq:
+        if pk:
+            mp[:, :, Q:, K:] = True
+        else:
+            mp[:, :, Q:, 0] = True
+    qp = torch.nn.functional.pad(q, (0, 0, 0, 0, 0, pq))
+    kp, vp = (torch.nn.functional.pad(t, (0, 0, 0, 0, 0, pk)) for t in (k, v))
+    return ring_attention_inference(qp, kp, vp, mp, axis_name, float32_logits)[:, :Q].contiguous()
+
+
 def ring_attention_inference(q, k, v, attn_mask, axis_name, float32_logits=True):
     """ringattention_inference.py:67-70.  q, k, v are the global (B, S, H, D) arrays of the virtual ring
     declared with ``ring_axis``; attn_mask is the global boolean mask (B|1, H|1, Q|1, K), True = attend.
@@ -126,6 +159,9 @@ def ring_attention_inference(q, k, v, attn_mask, axis_name, float32_logits=True)
     if D > 256:
         raise NotImplementedError("head size %d: the kernels take head sizes up to 256" % D)
     n = axis_size(axis_name)
+    padded = _pad_lengths(q, k, v, attn_mask, axis_name, float32_logits, n)
+    if padded is not None:
+        return padded
     on_grid = q.shape[1] % (64 * n) == 0 and k.shape[1] % (64 * n) == 0 and D <= 128
     to = (64 if D <= 64 else 128) if on_grid else next(s for s in (32, 64, 128, 256) if D <= s)
     if to == D:

@@ -232,3 +232,28 @@ def test_inference_mfma_path_is_bitwise_reproducible():
     assert torch.equal(first[0], again[0])
     for a, b in zip(first[1], again[1]):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("S,Sk,n,kind", [(1000, 1000, 1, "full"), (1000, 1000, 2, "per_head"), (900, 1024, 1, "full"),
+                                         (1024, 1000, 2, "key_only"), (200, 1000, 1, "bcast_bh")])
+def test_inference_lengths_off_the_128_grid_run_on_the_matrix_cores(S, Sk, n, kind, dtype):
+    """A prompt of 1000 tokens: q, k, v and the mask are padded to the next multiple of 128 per device (positions mean
+    nothing but what the mask says) and the result is cut back; against the oracle at the original lengths."""
+    B, H, D = 2, 2, 128
+    g = torch.Generator().manual_seed(S + Sk)
+    q = (torch.randn(B, S, H, D, generator=g) * D ** -0.25).to(dtype)
+    k = (torch.randn(B, Sk, H, D, generator=g) * D ** -0.25).to(dtype)
+    v = torch.randn(B, Sk, H, D, generator=g).to(dtype)
+    do = torch.randn(B, S, H, D, generator=g).to(dtype)
+    shape = {"full": (B, H, S, Sk), "bcast_bh": (1, 1, S, Sk), "key_only": (B, 1, 1, Sk), "per_head": (1, H, S, Sk)}[kind]
+    mask = torch.rand(shape, generator=g) < 0.5
+    mask[..., 0] = True
+    out, grads = _run(q, k, v, do, mask, n)
+    fam = ra.kernel_family_of_last_call()
+    assert "mfma" in fam["forward"] and "mfma" in fam["backward"], fam
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+    ref_grads = O.ring_attention_inference_bwd(n, res, do)
+    assert_close(out, ref_out, dtype, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close(a, b, dtype, name)
