@@ -21,7 +21,8 @@ def _inference_cfg(q, q_len, kv_len, float32_logits, logit_dim=0):
 
 def _fwd(q, k, v, attn_mask, axis_name, float32_logits, logit_dim=0):
     _check_qkv(q, k, v)
-    q, k, v = (t if _row_dense(t) else t.contiguous() for t in (q, k, v))      # other views are copied once
+    q = q.contiguous()                             # the cotangent arrives dense and shares q's strides
+    k, v = (t if _row_dense(t) else t.contiguous() for t in (k, v))            # other views are copied once
     if k.stride(0) != v.stride(0):
         k, v = k.contiguous(), v.contiguous()
     n = axis_size(axis_name)                                                     # :15

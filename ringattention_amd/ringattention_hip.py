@@ -434,7 +434,7 @@ class _MaskInputs:
 def _check_qkv(q, k, v):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("ringattention_amd runs on the GPU only: q, k, v must be device tensors")
-    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape:
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or v.shape != k.shape:
         raise ValueError("q, k, v must be (B, S, H, D) with k.shape == v.shape")
     if q.shape[0] != k.shape[0] or q.shape[2:] != k.shape[2:]:
         raise ValueError("q and k must agree in batch, heads and head size")
@@ -731,10 +731,11 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
     Returns (out, residuals)."""
     cfg = _Config(blockwise_kwargs)
     _check_qkv(q, k, v)
-    # the kernels take any batch stride, rows of H * D elements one after the other; k and v share theirs, and the
-    # cotangent and the gradients follow q.  Any other view (a slice of a fused q/k/v projection, a transposed
-    # (B, H, S, D) array) is copied once
-    q, k, v = (t if _row_dense(t) else t.contiguous() for t in (q, k, v))
+    # the kernels take any batch stride, rows of H * D elements one after the other; k and v share theirs; the
+    # cotangent arrives dense and shares q's strides, so q is dense too.  Any other view (a slice of a fused q/k/v
+    # projection, a transposed (B, H, S, D) array, the first positions of a longer q) is copied once
+    q = q.contiguous()
+    k, v = (t if _row_dense(t) else t.contiguous() for t in (k, v))
     if k.stride(0) != v.stride(0):
         k, v = k.contiguous(), v.contiguous()
     n = axis_size(axis_name)
@@ -1139,6 +1140,7 @@ def ring_attention(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, float3
     One query token with cache_idx set takes the streaming decode kernel."""
     # (a head size the streaming kernel is not built for takes the blockwise kernels below, like a call that wants
     # gradients)
+    _check_qkv(q, k, v)
     if q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16:
         # float16 inputs: with float32_logits the reference casts q and k to fp32 (:18-19) and the products with v
         # promote to fp32 as well, so computing on exact fp32 copies (the fp32 matrix-core kernels) and rounding the

@@ -759,7 +759,11 @@ def test_strided_views_of_q_k_v_give_the_bits_of_contiguous_arrays(dtype, D, chu
     cache[0, :, :S], cache[1, :, :S] = qkv[:, :, 1], qkv[:, :, 2]
     cached = run(qkv[:, :, 0].contiguous(), cache[0, :, :S], cache[1, :, :S])
     mixed = run(qkv[:, :, 0], cache[0, :, :S], qkv[:, :, 2].contiguous())   # k and v with different batch strides
-    for name, res in (("fused", fused), ("transposed", transposed), ("cache", cached), ("mixed", mixed)):
+    longer = torch.zeros(B, S + 128, H, D, dtype=dtype, device=DEV)
+    longer[:, :S] = qkv[:, :, 0]
+    prefix = run(longer[:, :S], qkv[:, :, 1], qkv[:, :, 2])                # q as the first positions of a longer array
+    for name, res in (("fused", fused), ("transposed", transposed), ("cache", cached), ("mixed", mixed),
+                      ("prefix", prefix)):
         for what, a, b in zip(("out", "dq", "dk", "dv"), res, base):
             assert a.shape == b.shape and torch.equal(a, b), (name, what)
     # the same through the boolean-mask ring
@@ -773,6 +777,8 @@ def test_strided_views_of_q_k_v_give_the_bits_of_contiguous_arrays(dtype, D, chu
         return out.detach(), q.grad, k.grad, v.grad
 
     base = run_inf(*(qkv[:, :, i].contiguous() for i in range(3)))
+    for what, a, b in zip(("out", "dq", "dk", "dv"), run_inf(longer[:, :S], cache[0, :, :S], qkv[:, :, 2]), base):
+        assert a.shape == b.shape and torch.equal(a, b), ("inference prefix", what)
     for what, a, b in zip(("out", "dq", "dk", "dv"), run_inf(qkv[:, :, 0], cache[0, :, :S], qkv[:, :, 2]), base):
         assert torch.equal(a, b), ("inference", what)
 
