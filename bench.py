@@ -223,6 +223,8 @@ def bench_attention(args, ring, dropout=False, c1=False):
         args = argparse.Namespace(**dict(vars(args), dtype="fp32", inputs="unit"))
     if args.seq_len:
         S = args.seq_len
+    if args.batch:
+        B = args.batch
     g = torch.Generator(device=dev).manual_seed(0)
     # q, k, v ~ N(0,1) / sqrt(D) is the input the configuration names; it makes the logits tiny (std 0.008).  The
     # other choices give the logits a standard deviation of 0.09 (q, k scaled D^-0.25) or 1 (unscaled q, k)
@@ -805,7 +807,7 @@ def bench_vendor_sdpa(args):
     import torch.nn.functional as F
     from torch.nn.attention import sdpa_kernel, SDPBackend
     dev = "cuda:0"
-    B, H, S, D = 1, 32, args.seq_len or 32768, 128
+    B, H, S, D = args.batch or 1, 32, args.seq_len or 32768, 128
     g = torch.Generator(device=dev).manual_seed(0)
     q, k, v = ((torch.randn(B, H, S, D, device=dev, generator=g) / D ** 0.5).to(torch.bfloat16).requires_grad_(True)
                for _ in range(3))
@@ -878,6 +880,7 @@ def main():
     ap.add_argument("--workload", default=None, choices=["attn32k", "ring131k", "ffn", "decode", "inference", "copy", "decode_step", "rmsnorm",
                                                               "dropout32k", "c1", "mfma_probe", "vendor_sdpa"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
+    ap.add_argument("--batch", type=int, default=0, help="attention workloads: batch rows (the configurations have 1)")
     ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
                     help="attention workloads: head size (the number of heads follows, H * D = 4096)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"],
@@ -907,7 +910,7 @@ def main():
         sys.exit(1)
     # no --workload: the whole headline metric in one line - the 32K attention step is the value; the decode leg
     # (B16, 262144 positions, 64 steps) and the same attention step on other input scales ride along as sub-objects
-    whole_metric = args.workload is None and not args.no_extras and not args.seq_len
+    whole_metric = args.workload is None and not args.no_extras and not args.seq_len and not args.batch
     if args.workload is None:
         args.workload = "attn32k"
     extras = {}
