@@ -352,3 +352,38 @@ def test_random_dropout_configuration_matches_oracle(seed):
     assert_close_scaled(out, ref_out, tol_dtype, "out")
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
         assert_close_scaled(a, b, tol_dtype, name)
+
+
+def draw_ring_cross(seed):
+    r = random.Random(21000 + seed)
+    n = r.choice([2, 4, 8])
+    dtype = r.choice([torch.float32, torch.bfloat16])
+    D = r.choice([64, 128])
+    qc, kc = r.choice([(128, 128), (128, 256), (256, 128), (32, 64), (64, 32), (16, 16)])
+    q_len = qc * r.randint(1, 3) * (kc // qc if kc > qc else 1)
+    kv_len = kc * r.randint(1, 3) * (qc // kc if qc > kc else 1)
+    cbs = r.choice([1, None, max(qc, kc)])
+    return dict(n=n, dtype=dtype, D=D, qc=qc, kc=kc, q_len=q_len, kv_len=kv_len, cbs=cbs, B=r.choice([1, 2]),
+                H=r.choice([1, 2]), bias=r.random() < 0.5, seg=r.random() < 0.5)
+
+
+@pytest.mark.parametrize("seed", range(OFFSET, OFFSET + 32))
+def test_random_ring_with_unequal_query_and_key_shards_matches_oracle(seed):
+    """A ring whose query shards and key shards differ in length (ringattention_jax.py:31-37 places a device's chunks
+    by its own shard lengths: query chunk start dev * q_len / qc, key chunk start src * kv_len / kc), with and without a
+    causal block size, bias and segment ids."""
+    c = draw_ring_cross(seed)
+    print("ring cross case", seed, c, flush=True)
+    n, B, H, D = c["n"], c["B"], c["H"], c["D"]
+    S, Skv = n * c["q_len"], n * c["kv_len"]
+    q, k, v, do = make_qkv(B, S, H, D, dtype=c["dtype"], seed=seed, Skv=Skv, scale=1.0)
+    g = torch.Generator().manual_seed(seed + 900)
+    bias = torch.randn(1, 1, 1, Skv, generator=g) if c["bias"] else None
+    seg = packed_segment_ids(B, max(S, Skv), max(4, S // 5), seed=seed + 7) if c["seg"] else None
+    kw = kwargs(c["qc"], c["kc"], c["cbs"])
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    print("  family", ra.kernel_family_of_last_call(), flush=True)
+    assert_close_scaled(out, ref_out, c["dtype"], "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close_scaled(a, b, c["dtype"], name)
