@@ -36,9 +36,13 @@ enum { RA_F32 = 0, RA_BF16 = 1 };
 enum {
   RA_IMPL_AUTO = 0,    /* MFMA kernels when the shape allows, else the generic ones */
   RA_IMPL_GENERIC = 1, /* fp32 vector-ALU kernels: any chunk sizes, fp32 or bf16 inputs */
-  RA_IMPL_MFMA = 2     /* matrix-core kernels only (bf16 inputs: v_mfma_f32_32x32x16_bf16, fp32 inputs:
+  RA_IMPL_MFMA = 2,    /* the tiled matrix-core kernels only (bf16 inputs: v_mfma_f32_32x32x16_bf16, fp32 inputs:
                           v_mfma_f32_32x32x2_f32; head size 64 or 128, chunk sizes multiples of 128);
                           RA_ERR_UNSUPPORTED if the shape does not fit */
+  RA_IMPL_MFMA_ANY = 3 /* the matrix-core kernels that evaluate the mask element by element only (bf16 inputs, head
+                          size 128 or 256; any chunk sizes and lengths, a bias per row, a boolean mask in bytes; no
+                          attention dropout): what RA_IMPL_AUTO falls back to before the generic kernels;
+                          RA_ERR_UNSUPPORTED if the call does not fit */
 };
 
 /*
@@ -227,7 +231,7 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream);
  * when the call would be refused.  The generic kernels serve every shape but run on the vector ALU, two orders of
  * magnitude below the matrix-core kernels on long sequences: a caller that lets RA_IMPL_AUTO choose can ask here
  * what it got (the Python layer warns once when a large problem lands on them). */
-enum { RA_FAMILY_GENERIC = 1, RA_FAMILY_MFMA_BF16 = 2, RA_FAMILY_MFMA_F32 = 3 };
+enum { RA_FAMILY_GENERIC = 1, RA_FAMILY_MFMA_BF16 = 2, RA_FAMILY_MFMA_F32 = 3, RA_FAMILY_MFMA_BF16_ANY = 4 };
 int ra_attn_fwd_family(const ra_attn_fwd_params* p);
 int ra_attn_bwd_family(const ra_attn_bwd_params* p);
 

@@ -12,13 +12,13 @@ LIB_PATH = os.path.join(_HERE, "libringattn_hip.so")
 RA_ABI_VERSION = 2          # include/ringattn_hip.h; load() refuses a library built for another one
 RA_OK, RA_ERR_INVALID, RA_ERR_UNSUPPORTED, RA_ERR_LAUNCH = 0, 1, 2, 3
 RA_F32, RA_BF16 = 0, 1
-RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA = 0, 1, 2
+RA_IMPL_AUTO, RA_IMPL_GENERIC, RA_IMPL_MFMA, RA_IMPL_MFMA_ANY = 0, 1, 2, 3
 RA_BWD_PART_DQ, RA_BWD_PART_DKV = 1, 2          # include/ringattn_hip_measure.h
 RA_DECODE_STATIC_SCRATCH_BYTES = 16 * 1024 * 1024
 RA_SEG_TILE = 64
 RA_KEEP_WHERE, RA_KEEP_DROPOUT = 0, 1
 RA_GRAD_INIT_DQ, RA_GRAD_INIT_DKV = 1, 2
-RA_FAMILY_GENERIC, RA_FAMILY_MFMA_BF16, RA_FAMILY_MFMA_F32 = 1, 2, 3
+RA_FAMILY_GENERIC, RA_FAMILY_MFMA_BF16, RA_FAMILY_MFMA_F32, RA_FAMILY_MFMA_BF16_ANY = 1, 2, 3, 4
 
 i32, i64, f32, vp = C.c_int32, C.c_int64, C.c_float, C.c_void_p
 

@@ -26,6 +26,10 @@ int attn_fwd_f32(const ra_attn_fwd_params* p, hipStream_t s);                  /
 int attn_bwd_f32(const ra_attn_bwd_params* p, int parts, hipStream_t s);
 bool attn_fwd_f32_supported(const ra_attn_fwd_params* p);
 bool attn_bwd_f32_supported(const ra_attn_bwd_params* p);
+int attn_fwd_any(const ra_attn_fwd_params* p, hipStream_t s);                  // bf16, the mask element by element
+int attn_bwd_any(const ra_attn_bwd_params* p, int parts, hipStream_t s);
+bool attn_fwd_any_supported(const ra_attn_fwd_params* p);
+bool attn_bwd_any_supported(const ra_attn_bwd_params* p);
 int carry_init(float*, int64_t, int64_t, float*, float*, int64_t, int64_t, int, int, int, int, hipStream_t);
 int finalize(const float*, int64_t, int64_t, const float*, int64_t, int64_t, void*, int, int64_t, int64_t, int,
              int, int, int, hipStream_t);
@@ -236,28 +240,43 @@ int ra_attn_fwd_block(const ra_attn_fwd_params* p, ra_stream_t stream) {
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "attn_fwd_block: B and H must be <= 65535");
   if (int rc = check_mask(p->mask, p->Sq, p->Skv, "attn_fwd_block")) return rc;
   hipStream_t s = (hipStream_t)stream;
+  RA_REQUIRE(p->impl == RA_IMPL_AUTO || p->impl == RA_IMPL_GENERIC || p->impl == RA_IMPL_MFMA ||
+             p->impl == RA_IMPL_MFMA_ANY, RA_ERR_INVALID, "attn_fwd_block: impl %d", p->impl);
   if (p->impl == RA_IMPL_GENERIC) return attn_fwd_generic(p, s);
-  if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, nullptr, s);
-  if (attn_fwd_f32_supported(p)) return attn_fwd_f32(p, s);
-  RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
-             "attn_fwd_block: MFMA kernels need bf16 or fp32, head size 64 or 128, chunk sizes that are multiples of 128");
+  if (p->impl != RA_IMPL_MFMA_ANY) {
+    if (attn_fwd_mfma_supported(p)) return attn_fwd_mfma(p, nullptr, s);
+    if (attn_fwd_f32_supported(p)) return attn_fwd_f32(p, s);
+    RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
+               "attn_fwd_block: MFMA kernels need bf16 or fp32, head size 64 or 128, chunk sizes that are multiples of 128");
+  }
+  if (attn_fwd_any_supported(p)) return attn_fwd_any(p, s);
+  RA_REQUIRE(p->impl != RA_IMPL_MFMA_ANY, RA_ERR_UNSUPPORTED,
+             "attn_fwd_block: the element-wise-mask MFMA kernels need bf16, head size 128 or 256, no attention dropout");
   return attn_fwd_generic(p, s);
 }
 
 int ra_attn_fwd_family(const ra_attn_fwd_params* p) {
   if (!p || (p->dtype != RA_F32 && p->dtype != RA_BF16)) return 0;
   if (p->impl == RA_IMPL_GENERIC) return RA_FAMILY_GENERIC;
-  if (attn_fwd_mfma_supported(p)) return RA_FAMILY_MFMA_BF16;
-  if (attn_fwd_f32_supported(p)) return RA_FAMILY_MFMA_F32;
-  return p->impl == RA_IMPL_MFMA ? 0 : RA_FAMILY_GENERIC;
+  if (p->impl != RA_IMPL_MFMA_ANY) {
+    if (attn_fwd_mfma_supported(p)) return RA_FAMILY_MFMA_BF16;
+    if (attn_fwd_f32_supported(p)) return RA_FAMILY_MFMA_F32;
+    if (p->impl == RA_IMPL_MFMA) return 0;
+  }
+  if (attn_fwd_any_supported(p)) return RA_FAMILY_MFMA_BF16_ANY;
+  return p->impl == RA_IMPL_MFMA_ANY ? 0 : RA_FAMILY_GENERIC;
 }
 
 int ra_attn_bwd_family(const ra_attn_bwd_params* p) {
   if (!p || (p->dtype != RA_F32 && p->dtype != RA_BF16)) return 0;
   if (p->impl == RA_IMPL_GENERIC) return RA_FAMILY_GENERIC;
-  if (attn_bwd_mfma_supported(p)) return RA_FAMILY_MFMA_BF16;
-  if (attn_bwd_f32_supported(p)) return RA_FAMILY_MFMA_F32;
-  return p->impl == RA_IMPL_MFMA ? 0 : RA_FAMILY_GENERIC;
+  if (p->impl != RA_IMPL_MFMA_ANY) {
+    if (attn_bwd_mfma_supported(p)) return RA_FAMILY_MFMA_BF16;
+    if (attn_bwd_f32_supported(p)) return RA_FAMILY_MFMA_F32;
+    if (p->impl == RA_IMPL_MFMA) return 0;
+  }
+  if (attn_bwd_any_supported(p)) return RA_FAMILY_MFMA_BF16_ANY;
+  return p->impl == RA_IMPL_MFMA_ANY ? 0 : RA_FAMILY_GENERIC;
 }
 
 int ra_attn_finalize(const float* numerator, int64_t num_stride_b, int64_t num_stride_s, const float* denominator,
@@ -299,17 +318,21 @@ static int attn_bwd_block(const ra_attn_bwd_params* p, int parts, const char* wh
   RA_REQUIRE(p->B > 0 && p->Sq > 0 && p->Skv > 0 && p->H > 0 && p->D > 0, RA_ERR_INVALID, "%s: empty shape", who);
   RA_REQUIRE(p->B <= 65535 && p->H <= 65535, RA_ERR_UNSUPPORTED, "%s: B and H must be <= 65535", who);
   RA_REQUIRE(p->logit_dim >= 0, RA_ERR_INVALID, "%s: negative logit_dim", who);
-  RA_REQUIRE(p->impl == RA_IMPL_AUTO || p->impl == RA_IMPL_GENERIC || p->impl == RA_IMPL_MFMA, RA_ERR_INVALID,
-             "%s: impl %d", who, p->impl);
+  RA_REQUIRE(p->impl == RA_IMPL_AUTO || p->impl == RA_IMPL_GENERIC || p->impl == RA_IMPL_MFMA ||
+             p->impl == RA_IMPL_MFMA_ANY, RA_ERR_INVALID, "%s: impl %d", who, p->impl);
   if (int rc = check_mask(p->mask, p->Sq, p->Skv, who)) return rc;
   const bool whole = dq_part && dkv_part;
   if (p->impl == RA_IMPL_GENERIC && whole) return attn_bwd_generic(p, s);
-  if (p->impl != RA_IMPL_GENERIC && attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, nullptr, parts, s);
-  if (p->impl != RA_IMPL_GENERIC && attn_bwd_f32_supported(p)) return attn_bwd_f32(p, parts, s);
-  RA_REQUIRE(whole, RA_ERR_UNSUPPORTED, "%s: one part alone is launched by the MFMA kernels only, which do not take "
-             "this call (impl, dtype, head size or chunk sizes)", who);
+  const bool tiled = p->impl == RA_IMPL_AUTO || p->impl == RA_IMPL_MFMA;
+  if (tiled && attn_bwd_mfma_supported(p)) return attn_bwd_mfma(p, nullptr, parts, s);
+  if (tiled && attn_bwd_f32_supported(p)) return attn_bwd_f32(p, parts, s);
   RA_REQUIRE(p->impl != RA_IMPL_MFMA, RA_ERR_UNSUPPORTED,
              "%s: MFMA kernels need bf16 or fp32, head size 64 or 128, chunk sizes that are multiples of 128", who);
+  if (p->impl != RA_IMPL_GENERIC && attn_bwd_any_supported(p)) return attn_bwd_any(p, parts, s);
+  RA_REQUIRE(p->impl != RA_IMPL_MFMA_ANY, RA_ERR_UNSUPPORTED,
+             "%s: the element-wise-mask MFMA kernels need bf16, head size 128 or 256, no attention dropout", who);
+  RA_REQUIRE(whole, RA_ERR_UNSUPPORTED, "%s: one part alone is launched by the MFMA kernels only, which do not take "
+             "this call (impl, dtype, head size or chunk sizes)", who);
   return attn_bwd_generic(p, s);
 }
 

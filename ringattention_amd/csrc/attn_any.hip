@@ -1,0 +1,661 @@
+// Matrix-core attention kernels that evaluate the reference's mask element by element: what the generic kernels
+// compute (any chunk sizes, any causal block size, a bias per key or per row, segment ids, a boolean mask given as
+// bytes, lengths that are no multiple of a tile), with the four matrix products on v_mfma_f32_32x32x16_bf16.  bf16
+// inputs, head size 128 or 256 (smaller ones arrive zero-padded).  They serve the calls the wave-specialised kernels
+// of attn_mfma.hip do not take; attention dropout stays with the generic kernels.
+//
+// A workgroup of four wavefronts keeps 128 rows of one operand in registers (32 per wavefront: a lane owns one of
+// them, so that row's softmax statistics are lane scalars) and streams 64-row tiles of the others through LDS, a
+// tile ahead in registers.  Products are formed transposed, S^T = K Q^T, so the C layout hands every lane its own
+// row's logits; P^T (dS^T) goes back in as a B operand from the same registers after one exchange with the partner
+// lane, and the second operand of O^T += V^T P^T comes from LDS transpose reads.  A tile whose pairs all run and
+// are not masked skips the element-wise evaluation.
+//
+// Semantics follow ringattention_jax.py:130-145 (forward tile), :220-233 (backward tile), :272-322 (bias / mask)
+// and :324-331 (skip predicate), through the same row_info() / logit() the generic kernels use.
+#include "generic_args.hpp"
+#include "../../include/ringattn_hip_measure.h"
+
+namespace ra {
+
+typedef __bf16 any_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float any_f32x16 __attribute__((ext_vector_type(16)));
+typedef float any_f32x4 __attribute__((ext_vector_type(4)));
+typedef short any_s16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned any_u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned any_u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int ANY_ROWS = 128;      // rows a workgroup keeps: four wavefronts of 32
+constexpr int ANY_TILE = 64;       // rows of the streamed operands per step
+constexpr int ANY_THREADS = 256;
+
+// LDS tiles hold rows of HD bf16 without padding; the 16-byte slot c of row r sits at slot c ^ any_swz(r), which
+// spreads a column of slots over the bank groups for the row reads and the four-row transpose reads below.
+__device__ __forceinline__ int any_swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
+__device__ __forceinline__ any_s16x4 any_read_tr(const uint16_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((any_s16x4 __attribute__((address_space(3)))*)(p));
+}
+__device__ __forceinline__ float any_max_xor32(float x) {
+  any_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float any_sum_xor32(float x) {
+  any_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// One 64-row tile of a (B, S, H, D) operand on its way to LDS: 16-byte chunks, a row's chunks on consecutive lanes.
+// Rows past `limit` repeat the last row (finite data that the mask logic never lets through).
+template <int HD>
+struct AnyStage {
+  static constexpr int SLOTS = HD / 8, NCH = ANY_TILE * SLOTS / ANY_THREADS;
+  uint4 r[NCH];
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t stride, int row0, int limit, int tid) {
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int c = tid + ANY_THREADS * i, row = c / SLOTS, slot = c % SLOTS;
+      const int gr = min(row0 + row, limit - 1);
+      r[i] = *(const uint4*)(base + (int64_t)gr * stride + slot * 8);
+    }
+  }
+  __device__ __forceinline__ void store(uint16_t* lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int c = tid + ANY_THREADS * i, row = c / SLOTS, slot = c % SLOTS;
+      *(uint4*)(lds + row * HD + ((slot ^ any_swz(row)) << 3)) = r[i];
+    }
+  }
+};
+
+// A operand of contraction step ks (16 head dimensions): row `row` of an LDS tile, this lane's eight elements
+template <int HD>
+__device__ __forceinline__ any_bf16x8 any_row_frag(const uint16_t* tile, int row, int ks, int hi) {
+  return *(const any_bf16x8*)(tile + row * HD + (((2 * ks + hi) ^ any_swz(row)) << 3));
+}
+
+// Offsets of the two transpose reads that give, for 16 consecutive tile rows starting at a multiple of 16, the A
+// operand "32 head dimensions of block db x those 16 rows": lane half hi takes rows 8 hi .. 8 hi + 7.
+template <int HD>
+struct AnyTr {
+  int off[HD / 32][2];
+  __device__ __forceinline__ void init(int lane) {
+    const int hi = lane >> 5, i = lane & 15, rr = (i >> 2) + 8 * hi;
+    const int c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
+#pragma unroll
+    for (int db = 0; db < HD / 32; db++) {
+      off[db][0] = rr * HD + (((4 * db + c0) ^ any_swz(rr)) << 3) + half * 4;
+      off[db][1] = (rr + 4) * HD + (((4 * db + c0) ^ any_swz(rr + 4)) << 3) + half * 4;
+    }
+  }
+  __device__ __forceinline__ any_bf16x8 frag(const uint16_t* rows16, int db) const {
+    const any_s16x4 x0 = any_read_tr(rows16 + off[db][0]);
+    const any_s16x4 x1 = any_read_tr(rows16 + off[db][1]);
+    return __builtin_bit_cast(any_bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
+  }
+};
+
+// A 32 x 32 product block in the C layout: the lane's column is lane % 32, register 4 g + e holds row 8 g + 4 hi + e.
+// The B operand of contraction step K over those rows (16 K .. 16 K + 15, lane half hi taking 16 K + 8 hi .. + 7)
+// is made of this lane's registers of row group g = 2 K + hi and the partner lane's registers of the same group.
+__device__ __forceinline__ any_bf16x8 any_bop(const any_f32x16& c, int K) {
+  const uint32_t x0 = f32x2_to_bf16x2(c[8 * K + 0], c[8 * K + 1]), x1 = f32x2_to_bf16x2(c[8 * K + 2], c[8 * K + 3]);
+  const uint32_t y0 = f32x2_to_bf16x2(c[8 * K + 4], c[8 * K + 5]), y1 = f32x2_to_bf16x2(c[8 * K + 6], c[8 * K + 7]);
+  // lanes 0-31 keep x and receive the partner's x; lanes 32-63 receive the partner's y and keep y
+  const any_u32x2 a = __builtin_amdgcn_permlane32_swap(x0, y0, false, false);
+  const any_u32x2 b = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
+  const any_u32x4 v = {a[0], b[0], a[1], b[1]};
+  return __builtin_bit_cast(any_bf16x8, v);
+}
+
+__device__ __forceinline__ int any_wave_max(int v) {
+  for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off));
+  return v;
+}
+__device__ __forceinline__ int any_wave_min(int v) {
+  for (int off = 32; off > 0; off >>= 1) v = min(v, __shfl_xor(v, off));
+  return v;
+}
+__device__ __forceinline__ long long any_wave_min(long long v) {
+  for (int off = 32; off > 0; off >>= 1) { const long long o = __shfl_xor(v, off); v = o < v ? o : v; }
+  return v;
+}
+
+// segment id and additive bias of key kj (clamped into the shard) for the lanes' rows: what a tile keeps in LDS
+__device__ __forceinline__ int any_key_seg(const MaskView& mv, int b, int kj) {
+  if (!mv.seg) return 0;
+  const int ki = kj / mv.kc;
+  const int idx = clamp_seg_index(((long long)mv.k_start + ki) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
+  return mv.seg[(int64_t)b * mv.seg_sb + idx];
+}
+__device__ __forceinline__ long long any_key_block(const MaskView& mv, int kj) {
+  const long long gk = mv.global_k(kj);
+  return mv.cbs > 1 ? gk / mv.cbs : gk;
+}
+
+// ------------------------------------------------------------------ forward
+template <int HD>
+__global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a) {
+  constexpr int NKS = HD / 16, NDB = HD / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[ANY_TILE * HD];
+  __shared__ int seg_ks[ANY_TILE];
+  __shared__ float bias_ks[ANY_TILE];
+  __shared__ int kend_s[4];
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int qtile = gridDim.x - 1 - blockIdx.x;              // under a causal mask the longest rows start first
+  const int row = qtile * ANY_ROWS + wave * 32 + lo;
+  const bool valid = row < a.Sq;
+  const int rrow = valid ? row : a.Sq - 1;
+  const uint16_t* qp = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)rrow * a.q_ss + (int64_t)h * HD;
+  const uint16_t* kbase = (const uint16_t*)a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD;
+  const uint16_t* vbase = (const uint16_t*)a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD;
+  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rrow;
+  const float scale = sqrtf((float)a.sdim);                            // :118
+
+  any_bf16x8 qf[NKS];                                                  // B operands: this lane's query, 8 dims per step
+#pragma unroll
+  for (int ks = 0; ks < NKS; ks++) qf[ks] = *(const any_bf16x8*)(qp + ks * 16 + hi * 8);
+
+  any_f32x16 acc[NDB];                                                 // O^T: register 4 g + e of block db = dim 32 db + 8 g + 4 hi + e
+  float m = RA_NEG_INF, l = 0.f;                                       // l: this lane's share of the denominator
+  if (a.carry_is_initial) {
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+  } else {
+    const float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)rrow * a.num_ss + (int64_t)h * HD + hi * 4;
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const any_f32x4 t4 = *(const any_f32x4*)(nump + db * 32 + g * 8);
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[db][g * 4 + e] = t4[e];
+      }
+    m = a.mx[st];
+    l = hi == 0 ? a.den[st] : 0.f;
+  }
+  RowInfo ri = row_info(mv, b, h, rrow, a.Skv);
+  if (!valid) ri.kend = 0;
+  const int kend_max_w = any_wave_max(ri.kend), kend_min_w = any_wave_min(ri.kend);
+  const long long gqblk_min_w = any_wave_min(ri.gq_blk);
+  if (lane == 0) kend_s[wave] = kend_max_w;
+  __syncthreads();
+  const int kend_wg = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
+  const int ntile = (kend_wg + ANY_TILE - 1) / ANY_TILE;
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0;
+  const bool elementwise_always = mv.seg || mv.keep || mv.kbits_k;
+
+  AnyTr<HD> tr;
+  tr.init(lane);
+  AnyStage<HD> sk, sv;
+  if (ntile > 0) {
+    sk.load(kbase, a.kv_ss, 0, a.Skv, tid);
+    sv.load(vbase, a.kv_ss, 0, a.Skv, tid);
+  }
+  for (int t = 0; t < ntile; t++) {
+    const int k0 = t * ANY_TILE;
+    __syncthreads();                                   // the tile before this one has been read by every wavefront
+    sk.store(Ks, tid);
+    sv.store(Vs, tid);
+    if (tid < ANY_TILE) {
+      const int kj = min(k0 + tid, a.Skv - 1);
+      seg_ks[tid] = any_key_seg(mv, b, kj);
+      float add = 0.f;
+      if (bias_per_key) {
+        add = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(kj) * mv.bias_sk];
+        if (mv.any_mask) add = fminf(add, 0.f);                         // minimum(), :299,:309
+      }
+      bias_ks[tid] = add;
+    }
+    __syncthreads();
+    if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
+      sk.load(kbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
+      sv.load(vbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
+    }
+    if (k0 >= kend_max_w) continue;                    // no row of this wavefront runs against these keys
+
+    any_f32x16 S[2];                                   // S^T, two blocks of 32 keys: register 4 g + e = key 8 g + 4 hi + e
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) S[blk][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ks++)
+        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Ks, blk * 32 + lo, ks, hi), qf[ks], S[blk], 0, 0, 0);   // :134
+    }
+    // every pair of the tile runs and is unmasked for every row of the wavefront: logit = dot / scale + bias
+    const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
+                       (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
+    float tmax = RA_NEG_INF;
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+        float s;
+        if (plain) {
+          float add = 0.f;
+          if (bias_per_key) add = bias_ks[kk];
+          else if (mv.bias) {
+            add = mv.bias[ri.bias_off + mv.global_k(k0 + kk) * mv.bias_sk];
+            if (mv.any_mask) add = fminf(add, 0.f);
+          }
+          s = S[blk][r] / scale + add;                                  // :134-136
+        } else {
+          s = logit(mv, ri, S[blk][r], scale, k0 + kk, seg_ks[kk]);
+        }
+        S[blk][r] = s;
+        tmax = fmaxf(tmax, s);
+      }
+    tmax = any_max_xor32(tmax);
+    const float m_new = fmaxf(m, tmax);                                 // :138
+    const float mm = m_new == RA_NEG_INF ? 0.f : m_new;                 // nothing ran for this row yet: every p is 0
+    const float corr = (m == m_new) ? 1.f : __expf(m - mm);             // :142
+    float psum = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float p = __expf(S[blk][r] - mm);                         // :140
+        S[blk][r] = p;
+        psum += p;
+      }
+    l = l * corr + psum;                                                // :144
+    m = m_new;
+    if (__builtin_amdgcn_ballot_w64(corr != 1.f) != 0) {
+#pragma unroll
+      for (int db = 0; db < NDB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] *= corr;                // :143
+    }
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int K = 0; K < 2; K++) {
+        const any_bf16x8 bop = any_bop(S[blk], K);
+        const uint16_t* rows16 = Vs + (blk * 32 + K * 16) * HD;
+#pragma unroll
+        for (int db = 0; db < NDB; db++)
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr.frag(rows16, db), bop, acc[db], 0, 0, 0);   // :141
+      }
+  }
+  if (valid) {
+    const float den = any_sum_xor32(l);
+    const int64_t ooff = (int64_t)b * a.out_sb + (int64_t)rrow * a.out_ss + (int64_t)h * HD + hi * 4;
+    float* nump = a.num + (int64_t)b * a.num_sb + (int64_t)rrow * a.num_ss + (int64_t)h * HD + hi * 4;
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        any_f32x4 t4;
+#pragma unroll
+        for (int e = 0; e < 4; e++) t4[e] = acc[db][g * 4 + e];
+        if (a.out) {                       // last step of the device: out = numerator / denominator (:52)
+#pragma unroll
+          for (int e = 0; e < 4; e++) t4[e] /= den;
+          uint2 pk = {f32x2_to_bf16x2(t4[0], t4[1]), f32x2_to_bf16x2(t4[2], t4[3])};
+          *(uint2*)((uint16_t*)a.out + ooff + db * 32 + g * 8) = pk;
+          if (a.out32) *(any_f32x4*)(a.out32 + ooff + db * 32 + g * 8) = t4;      // the residual of :53
+        } else {
+          *(any_f32x4*)(nump + db * 32 + g * 8) = t4;
+        }
+      }
+    if (hi == 0) { a.mx[st] = m; a.den[st] = den; }
+  }
+}
+
+// ------------------------------------------------------------------ backward, dq (a lane owns a query row)
+template <int HD>
+__global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArgs a) {
+  constexpr int NKS = HD / 16, NDB = HD / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[ANY_TILE * HD];
+  __shared__ int seg_ks[ANY_TILE];
+  __shared__ float bias_ks[ANY_TILE];
+  __shared__ int kend_s[4];
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int qtile = gridDim.x - 1 - blockIdx.x;
+  const int row = qtile * ANY_ROWS + wave * 32 + lo;
+  const bool valid = row < a.Sq;
+  const int rrow = valid ? row : a.Sq - 1;
+  const int64_t qoff = (int64_t)b * a.q_sb + (int64_t)rrow * a.q_ss + (int64_t)h * HD;
+  const uint16_t* qp = (const uint16_t*)a.q + qoff;
+  const uint16_t* gp = (const uint16_t*)a.g + qoff;
+  const uint16_t* kbase = (const uint16_t*)a.k + (int64_t)b * a.kv_sb + (int64_t)h * HD;
+  const uint16_t* vbase = (const uint16_t*)a.v + (int64_t)b * a.kv_sb + (int64_t)h * HD;
+  const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rrow;
+  const float scale = sqrtf((float)a.sdim);
+
+  any_bf16x8 qf[NKS], gf[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ks++) {
+    qf[ks] = *(const any_bf16x8*)(qp + ks * 16 + hi * 8);
+    gf[ks] = *(const any_bf16x8*)(gp + ks * 16 + hi * 8);
+  }
+  any_f32x16 acc[NDB];                                                 // dQ^T
+#pragma unroll
+  for (int db = 0; db < NDB; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+  const float m = a.mx[st], rden = 1.f / a.den[st], delta = a.delta[st];
+  RowInfo ri = row_info(mv, b, h, rrow, a.Skv);
+  if (!valid) ri.kend = 0;
+  const int kend_max_w = any_wave_max(ri.kend), kend_min_w = any_wave_min(ri.kend);
+  const long long gqblk_min_w = any_wave_min(ri.gq_blk);
+  if (lane == 0) kend_s[wave] = kend_max_w;
+  __syncthreads();
+  const int kend_wg = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
+  const int ntile = (kend_wg + ANY_TILE - 1) / ANY_TILE;
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0;
+  const bool elementwise_always = mv.seg || mv.keep || mv.kbits_k;
+
+  AnyTr<HD> tr;
+  tr.init(lane);
+  AnyStage<HD> sk, sv;
+  if (ntile > 0) {
+    sk.load(kbase, a.kv_ss, 0, a.Skv, tid);
+    sv.load(vbase, a.kv_ss, 0, a.Skv, tid);
+  }
+  for (int t = 0; t < ntile; t++) {
+    const int k0 = t * ANY_TILE;
+    __syncthreads();
+    sk.store(Ks, tid);
+    sv.store(Vs, tid);
+    if (tid < ANY_TILE) {
+      const int kj = min(k0 + tid, a.Skv - 1);
+      seg_ks[tid] = any_key_seg(mv, b, kj);
+      float add = 0.f;
+      if (bias_per_key) {
+        add = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(kj) * mv.bias_sk];
+        if (mv.any_mask) add = fminf(add, 0.f);
+      }
+      bias_ks[tid] = add;
+    }
+    __syncthreads();
+    if (t + 1 < ntile) {
+      sk.load(kbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
+      sv.load(vbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
+    }
+    if (k0 >= kend_max_w) continue;
+
+    any_f32x16 S[2], dP[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; dP[blk][r] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < NKS; ks++) {
+        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Ks, blk * 32 + lo, ks, hi), qf[ks], S[blk], 0, 0, 0);   // :223-225
+        dP[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Vs, blk * 32 + lo, ks, hi), gf[ks], dP[blk], 0, 0, 0); // :228
+      }
+    }
+    const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
+                       (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+        float s;
+        if (plain) {
+          float add = 0.f;
+          if (bias_per_key) add = bias_ks[kk];
+          else if (mv.bias) {
+            add = mv.bias[ri.bias_off + mv.global_k(k0 + kk) * mv.bias_sk];
+            if (mv.any_mask) add = fminf(add, 0.f);
+          }
+          s = S[blk][r] / scale + add;
+        } else {
+          s = logit(mv, ri, S[blk][r], scale, k0 + kk, seg_ks[kk]);
+        }
+        const float p = __expf(s - m) * rden;                           // :226
+        // a pair whose tile does not run contributes nothing (:246-257)
+        S[blk][r] = (k0 + kk < ri.kend) ? (dP[blk][r] - delta) * p : 0.f;   // dS^T, :229
+      }
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int K = 0; K < 2; K++) {
+        const any_bf16x8 bop = any_bop(S[blk], K);
+        const uint16_t* rows16 = Ks + (blk * 32 + K * 16) * HD;
+#pragma unroll
+        for (int db = 0; db < NDB; db++)
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr.frag(rows16, db), bop, acc[db], 0, 0, 0);   // :230
+      }
+  }
+  if (valid) {
+    const int64_t off = (int64_t)h * HD + hi * 4;
+    float* dqp = a.dq + (int64_t)b * a.dq_sb + (int64_t)rrow * a.dq_ss + off;
+    uint16_t* op = (uint16_t*)a.dq_out + (int64_t)b * a.dqo_sb + (int64_t)rrow * a.dqo_ss + off;
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        any_f32x4 t4 = {0.f, 0.f, 0.f, 0.f};
+        if (!a.dq_initial) t4 = *(const any_f32x4*)(dqp + db * 32 + g * 8);
+#pragma unroll
+        for (int e = 0; e < 4; e++) t4[e] += acc[db][g * 4 + e] / scale;
+        if (a.dq_out) {                                                 // last call for these rows (:89)
+          uint2 pk = {f32x2_to_bf16x2(t4[0], t4[1]), f32x2_to_bf16x2(t4[2], t4[3])};
+          *(uint2*)(op + db * 32 + g * 8) = pk;
+        } else {
+          *(any_f32x4*)(dqp + db * 32 + g * 8) = t4;
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------ backward, dk or dv (a lane owns a key row)
+template <int HD, bool WANT_DK>
+__global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericArgs a) {
+  constexpr int NKS = HD / 16, NDB = HD / 32;
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Gs[ANY_TILE * HD];
+  __shared__ float r_m[ANY_TILE], r_rden[ANY_TILE], r_delta[ANY_TILE];
+  __shared__ RowInfo r_info[ANY_TILE];
+  __shared__ int r_kend_min;
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int first_key = blockIdx.x * ANY_ROWS;
+  const int kj = first_key + wave * 32 + lo;
+  const bool valid = kj < a.Skv;
+  const int rk = valid ? kj : a.Skv - 1;
+  const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)rk * a.kv_ss + (int64_t)h * HD;
+  const uint16_t* kp = (const uint16_t*)a.k + koff;
+  const uint16_t* vp = (const uint16_t*)a.v + koff;
+  const uint16_t* qbase = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)h * HD;
+  const uint16_t* gbase = (const uint16_t*)a.g + (int64_t)b * a.q_sb + (int64_t)h * HD;
+  const float scale = sqrtf((float)a.sdim);
+
+  any_bf16x8 kf[NKS], vf[WANT_DK ? NKS : 1];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ks++) kf[ks] = *(const any_bf16x8*)(kp + ks * 16 + hi * 8);
+  if (WANT_DK) {
+#pragma unroll
+    for (int ks = 0; ks < NKS; ks++) vf[ks] = *(const any_bf16x8*)(vp + ks * 16 + hi * 8);
+  }
+  any_f32x16 acc[NDB];                                                 // dK^T or dV^T
+#pragma unroll
+  for (int db = 0; db < NDB; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
+  const int seg_k = any_key_seg(mv, b, rk);
+  const int key_hi_w = first_key + wave * 32 + 32;                     // one past the wavefront's last key
+  const long long gkblk_max_w = any_key_block(mv, min(key_hi_w, a.Skv) - 1);
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0;
+  const bool elementwise_always = mv.seg || mv.keep || mv.kbits_k || (mv.bias && !bias_per_key);
+  float bias_k = 0.f;                                                  // a bias per key is a lane scalar here
+  if (bias_per_key) {
+    bias_k = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(rk) * mv.bias_sk];
+    if (mv.any_mask) bias_k = fminf(bias_k, 0.f);
+  }
+  const bool wave_valid = first_key + wave * 32 < a.Skv;               // some key of the wavefront exists
+  const bool all_valid = key_hi_w <= a.Skv;
+
+  AnyTr<HD> tr;
+  tr.init(lane);
+  AnyStage<HD> sq, sg;
+  // query tiles whose last row's run prefix ends before this block's first key hold nothing for it; the prefix grows
+  // with the query chunk, so the tiles that count are a suffix
+  int t_first = 0;
+  const int ntile = (a.Sq + ANY_TILE - 1) / ANY_TILE;
+  while (t_first < ntile &&
+         mv.run_prefix_keys((min((t_first + 1) * ANY_TILE, a.Sq) - 1) / mv.qc, a.Skv) <= first_key) t_first++;
+  if (t_first < ntile) {
+    sq.load(qbase, a.q_ss, t_first * ANY_TILE, a.Sq, tid);
+    sg.load(gbase, a.q_ss, t_first * ANY_TILE, a.Sq, tid);
+  }
+  for (int t = t_first; t < ntile; t++) {
+    const int q0 = t * ANY_TILE;
+    __syncthreads();
+    sq.store(Qs, tid);
+    sg.store(Gs, tid);
+    if (tid == 0) r_kend_min = 0x7fffffff;
+    __syncthreads();
+    if (tid < ANY_TILE) {
+      const int row = q0 + tid;
+      const bool rv = row < a.Sq;
+      const int rr = rv ? row : a.Sq - 1;
+      const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rr;
+      r_m[tid] = a.mx[st]; r_rden[tid] = 1.f / a.den[st]; r_delta[tid] = a.delta[st];
+      RowInfo ri = row_info(mv, b, h, rr, a.Skv);
+      if (!rv) ri.kend = 0;
+      r_info[tid] = ri;
+      atomicMin(&r_kend_min, ri.kend);
+    }
+    __syncthreads();
+    if (t + 1 < ntile) {
+      sq.load(qbase, a.q_ss, q0 + ANY_TILE, a.Sq, tid);
+      sg.load(gbase, a.q_ss, q0 + ANY_TILE, a.Sq, tid);
+    }
+    if (!wave_valid) continue;
+
+    any_f32x16 S[2], dP[2];                            // S, dP: the lane's key column; register 4 g + e = query 8 g + 4 hi + e
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; if (WANT_DK) dP[blk][r] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < NKS; ks++) {
+        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Qs, blk * 32 + lo, ks, hi), kf[ks], S[blk], 0, 0, 0);
+        if (WANT_DK)
+          dP[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Gs, blk * 32 + lo, ks, hi), vf[ks], dP[blk], 0, 0, 0);
+      }
+    }
+    // every pair of (tile rows, the wavefront's keys) runs and is unmasked
+    const bool plain = !elementwise_always && all_valid && key_hi_w <= r_kend_min &&
+                       (mv.cbs <= 0 || r_info[0].gq_blk >= gkblk_max_w);
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int qq = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+        float p;
+        if (plain) {
+          p = __expf(S[blk][r] / scale + bias_k - r_m[qq]) * r_rden[qq];
+        } else {
+          const RowInfo ri = r_info[qq];
+          const float s = logit(mv, ri, S[blk][r], scale, kj, seg_k);
+          p = (valid && kj < ri.kend) ? __expf(s - r_m[qq]) * r_rden[qq] : 0.f;     // :226; (:246-257)
+        }
+        S[blk][r] = WANT_DK ? (dP[blk][r] - r_delta[qq]) * p : p;       // dS (:229) or P
+      }
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+      for (int K = 0; K < 2; K++) {
+        const any_bf16x8 bop = any_bop(S[blk], K);
+        const uint16_t* rows16 = (WANT_DK ? Qs : Gs) + (blk * 32 + K * 16) * HD;
+#pragma unroll
+        for (int db = 0; db < NDB; db++)
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr.frag(rows16, db), bop, acc[db], 0, 0, 0);   // :231 / :232
+      }
+  }
+  if (valid) {
+    const int64_t off = (int64_t)h * HD + hi * 4;
+    float* outp = (WANT_DK ? a.dk : a.dv) + (int64_t)b * a.dkv_sb + (int64_t)rk * a.dkv_ss + off;
+    uint16_t* op = (uint16_t*)(WANT_DK ? a.dk_out : a.dv_out) + (int64_t)b * a.dkvo_sb + (int64_t)rk * a.dkvo_ss + off;
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        any_f32x4 t4 = {0.f, 0.f, 0.f, 0.f};
+        if (!a.dkv_initial) t4 = *(const any_f32x4*)(outp + db * 32 + g * 8);
+#pragma unroll
+        for (int e = 0; e < 4; e++) t4[e] += WANT_DK ? acc[db][g * 4 + e] / scale : acc[db][g * 4 + e];
+        if (a.dk_out) {                                                 // last call for these keys (:89)
+          uint2 pk = {f32x2_to_bf16x2(t4[0], t4[1]), f32x2_to_bf16x2(t4[2], t4[3])};
+          *(uint2*)(op + db * 32 + g * 8) = pk;
+        } else {
+          *(any_f32x4*)(outp + db * 32 + g * 8) = t4;
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------ host side
+static bool any_aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
+
+static bool any_mask_ok(const ra_mask& m) {
+  // attention dropout (its -inf bookkeeping, :321) and a boolean mask that exists in packed form only stay with the
+  // kernels built for them
+  return m.keep_mode != RA_KEEP_DROPOUT && !(m.keep_bits_k && !m.keep);
+}
+
+bool attn_fwd_any_supported(const ra_attn_fwd_params* p) {
+  return p->dtype == RA_BF16 && (p->D == 128 || p->D == 256) && any_mask_ok(p->mask) &&
+         p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 && p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 &&
+         any_aligned16(p->q) && any_aligned16(p->k) && any_aligned16(p->v) &&
+         (!p->numerator || (any_aligned16(p->numerator) && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0)) &&
+         (!p->out || (any_aligned16(p->out) && p->out_stride_s % 4 == 0 && p->out_stride_b % 4 == 0)) &&
+         any_aligned16(p->out_f32);
+}
+
+bool attn_bwd_any_supported(const ra_attn_bwd_params* p) {
+  return p->dtype == RA_BF16 && (p->D == 128 || p->D == 256) && any_mask_ok(p->mask) &&
+         p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 && p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 &&
+         any_aligned16(p->q) && any_aligned16(p->k) && any_aligned16(p->v) && any_aligned16(p->g) &&
+         (!p->dq || (any_aligned16(p->dq) && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0)) &&
+         (!p->dk || (any_aligned16(p->dk) && any_aligned16(p->dv) && p->dkv_stride_s % 4 == 0 && p->dkv_stride_b % 4 == 0)) &&
+         (!p->dq_out || (any_aligned16(p->dq_out) && p->dq_out_stride_s % 4 == 0 && p->dq_out_stride_b % 4 == 0)) &&
+         (!p->dk_out || (any_aligned16(p->dk_out) && any_aligned16(p->dv_out) && p->dkv_out_stride_s % 4 == 0 &&
+                         p->dkv_out_stride_b % 4 == 0));
+}
+
+int attn_fwd_any(const ra_attn_fwd_params* p, hipStream_t s) {
+  const GenericArgs a = make_args_fwd(p);
+  const dim3 grid((a.Sq + ANY_ROWS - 1) / ANY_ROWS, a.H, a.B), block(ANY_THREADS);
+  if (a.D == 128) attn_fwd_any_kernel<128><<<grid, block, 0, s>>>(a);
+  else attn_fwd_any_kernel<256><<<grid, block, 0, s>>>(a);
+  RA_CHECK_LAUNCH("attn_fwd_any");
+  return RA_OK;
+}
+
+template <int HD>
+static void launch_bwd_any(const GenericArgs& a, int parts, hipStream_t s) {
+  const dim3 block(ANY_THREADS);
+  const dim3 gq((a.Sq + ANY_ROWS - 1) / ANY_ROWS, a.H, a.B), gk((a.Skv + ANY_ROWS - 1) / ANY_ROWS, a.H, a.B);
+  if (parts & RA_BWD_PART_DQ) attn_bwd_dq_any_kernel<HD><<<gq, block, 0, s>>>(a);
+  if (parts & RA_BWD_PART_DKV) {
+    attn_bwd_dkv_any_kernel<HD, true><<<gk, block, 0, s>>>(a);
+    attn_bwd_dkv_any_kernel<HD, false><<<gk, block, 0, s>>>(a);
+  }
+}
+
+int attn_bwd_any(const ra_attn_bwd_params* p, int parts, hipStream_t s) {
+  const GenericArgs a = make_args_bwd(p);
+  if (a.D == 128) launch_bwd_any<128>(a, parts, s);
+  else launch_bwd_any<256>(a, parts, s);
+  RA_CHECK_LAUNCH("attn_bwd_any");
+  return RA_OK;
+}
+
+}  // namespace ra

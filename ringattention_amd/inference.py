@@ -164,7 +164,12 @@ def ring_attention_inference(q, k, v, attn_mask, axis_name, float32_logits=True)
     if padded is not None:
         return padded
     on_grid = q.shape[1] % (64 * n) == 0 and k.shape[1] % (64 * n) == 0 and D <= 128
-    to = (64 if D <= 64 else 128) if on_grid else next(s for s in (32, 64, 128, 256) if D <= s)
+    if on_grid:
+        to = 64 if D <= 64 else 128
+    elif q.dtype == torch.bfloat16:
+        to = 128 if D <= 128 else 256           # the matrix-core kernels that evaluate the mask element by element
+    else:
+        to = next(s for s in (32, 64, 128, 256) if D <= s)
     if to == D:
         return _RingAttentionInferenceFn.apply(q, k, v, attn_mask, axis_name, float32_logits)
     q, k, v = (torch.nn.functional.pad(t, (0, to - D)) for t in (q, k, v))

@@ -140,8 +140,8 @@ class _Config:
             self.seed = int(rng) & 0xFFFFFFFFFFFFFFFF
         self.dtype = _as_torch_dtype(kw.get("dtype", torch.float32))
         self.mask_min = float(torch.finfo(self.dtype).min)
-        self.impl = {"auto": L.RA_IMPL_AUTO, "generic": L.RA_IMPL_GENERIC, "mfma": L.RA_IMPL_MFMA}[
-            kw.get("impl", "auto")]
+        self.impl = {"auto": L.RA_IMPL_AUTO, "generic": L.RA_IMPL_GENERIC, "mfma": L.RA_IMPL_MFMA,
+                     "mfma_any": L.RA_IMPL_MFMA_ANY}[kw.get("impl", "auto")]
         # measurement hook: launch one of the two backward kernels alone (ra_attn_bwd_block_part)
         self.bwd_only = {None: 0, "dq": L.RA_BWD_PART_DQ, "dkv": L.RA_BWD_PART_DKV}[kw.get("bwd_only", None)]
         self.skip_masked_tiles = kw.get("skip_masked_tiles", None)
@@ -455,15 +455,17 @@ def _rows(t):
 
 
 # --------------------------------------------------------------------------- which kernels ran
-_FAMILY_NAMES = {L.RA_FAMILY_GENERIC: "generic", L.RA_FAMILY_MFMA_BF16: "mfma_bf16", L.RA_FAMILY_MFMA_F32: "mfma_f32"}
+_FAMILY_NAMES = {L.RA_FAMILY_GENERIC: "generic", L.RA_FAMILY_MFMA_BF16: "mfma_bf16", L.RA_FAMILY_MFMA_F32: "mfma_f32",
+                 L.RA_FAMILY_MFMA_BF16_ANY: "mfma_bf16_any"}
 _LAST_FAMILY = {"forward": None, "backward": None}
 _WARNED = set()
 _GENERIC_WARN_PAIRS = 1 << 28         # B * H * q_len * kv_len from which the vector-ALU kernels take seconds
 
 
 def kernel_family_of_last_call():
-    """{"forward": ..., "backward": ...}: the kernel family ("mfma_bf16", "mfma_f32", "generic") that the last
-    attention launch of each direction ran on - what blockwise_kwargs["impl"] = "auto" (the default) chose."""
+    """{"forward": ..., "backward": ...}: the kernel family ("mfma_bf16", "mfma_f32", "mfma_bf16_any" - the
+    matrix-core kernels that evaluate the mask element by element -, "generic") that the last attention launch of
+    each direction ran on - what blockwise_kwargs["impl"] = "auto" (the default) chose."""
     return dict(_LAST_FAMILY)
 
 
@@ -820,10 +822,13 @@ def _padded_head_size(cfg, mi, q):
     D = q.shape[3]
     if D > 256:
         raise NotImplementedError("head size %d: the kernels take head sizes up to 256" % D)
-    generic = (cfg.impl == L.RA_IMPL_GENERIC or D > 128 or q.dtype not in (torch.bfloat16, torch.float32)
+    generic = (cfg.impl in (L.RA_IMPL_GENERIC, L.RA_IMPL_MFMA_ANY) or D > 128
+               or q.dtype not in (torch.bfloat16, torch.float32)
                or cfg.qc % 128 or cfg.kc % 128 or (mi.bias is not None and mi.bias_strides[2] != 0)
                or (mi.keep is not None and mi.keep_packed is None))
-    if generic:
+    if generic and q.dtype == torch.bfloat16 and cfg.impl != L.RA_IMPL_GENERIC and cfg.pdrop == 0.0:
+        to = 128 if D <= 128 else 256       # the matrix-core kernels that evaluate the mask element by element
+    elif generic:
         to = next(s for s in (32, 64, 128, 256) if D <= s)
     else:
         to = 64 if D <= 64 else 128
@@ -840,7 +845,8 @@ def _fit_chunks_to_mfma_grid(cfg, mi, q, q_len, kv_len, q_total, kv_total, grid=
     long as its row has an unmasked key, which is what skip_masked_tiles already asks for; so both chunkings sum
     over the same pairs.  Without a causal block size every chunk pair runs.  The slices are not clamped when the
     segment ids cover every position, there is no dropout here, and a per-row bias takes the generic kernels."""
-    if cfg.impl == L.RA_IMPL_GENERIC or q.dtype not in (torch.bfloat16, torch.float32) or q.shape[3] > 128:
+    if cfg.impl in (L.RA_IMPL_GENERIC, L.RA_IMPL_MFMA_ANY) or q.dtype not in (torch.bfloat16, torch.float32) \
+            or q.shape[3] > 128:
         return
     if cfg.qc % grid == 0 and cfg.kc % grid == 0:
         return
@@ -881,7 +887,7 @@ def _ring_step_launches(cfg, mi, n):
     """Whether a scan step of all devices may go out as one launch per kernel (ra_attn_*_ring_step): a ring of 2 to
     64 devices, the MFMA kernels, no boolean / dropout mask, no cache_idx.  blockwise_kwargs["ring_launch"] =
     "device" keeps one launch per device."""
-    return (1 < n <= 64 and cfg.ring_launch != "device" and cfg.impl != L.RA_IMPL_GENERIC and cfg.pdrop == 0.0
+    return (1 < n <= 64 and cfg.ring_launch != "device" and cfg.impl in (L.RA_IMPL_AUTO, L.RA_IMPL_MFMA) and cfg.pdrop == 0.0
             and mi.keep is None and mi.keep_packed is None and mi.cache_idx_host is None and mi.cache_idx_dev is None)
 
 
@@ -1097,7 +1103,7 @@ def _pad_lengths_to_mfma_grid(q, k, v, attn_bias, segment_ids, cache_idx, n, axi
     B, S, H, D = q.shape
     if n != 1 or cache_idx is not None or k.shape[1] != S or S % grid == 0 or D > 128:
         return None
-    if q.dtype not in (torch.bfloat16, torch.float32) or kw.get("impl", "auto") == "generic":
+    if q.dtype not in (torch.bfloat16, torch.float32) or kw.get("impl", "auto") in ("generic", "mfma_any"):
         return None
     if kw.get("skip_masked_tiles", None) is False or kw.get("_padded", False):
         return None

@@ -190,14 +190,20 @@ def test_fit_chunks_to_mfma_grid_decisions(qc, kc, cbs, skip, expect):
     rh._fit_chunks_to_mfma_grid(cfg, _FakeMaskInputs(), q32, 768, 768, 768, 768)
     assert cfg.qc == expect
     on_grid = cfg.qc % 128 == 0 and cfg.kc % 128 == 0
-    # on the matrix-core grid 32 is padded to 64; a call that stays on the vector kernels keeps it (they tile 32)
-    assert rh._padded_head_size(cfg, _FakeMaskInputs(), q32) == (64 if on_grid else 0)
-    # 96 is tiled by neither family: 128 either way; 40 goes to 64 either way; above 128 only the vector kernels' 256
+    # on the matrix-core grid 32 is padded to 64; off it a bf16 call takes the matrix-core kernels that evaluate the
+    # mask element by element (head size 128 or 256), an fp32 call the vector kernels (they tile 32)
+    assert rh._padded_head_size(cfg, _FakeMaskInputs(), q32) == (64 if on_grid else 128)
+    assert rh._padded_head_size(cfg, _FakeMaskInputs(), q32.float()) == (64 if on_grid else 0)
+    # 96 is tiled by no family: 128 either way; above 128 the element-wise and the vector kernels' 256
     assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 96, dtype=torch.float32)) == 128
-    assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 40, dtype=torch.bfloat16)) == 64
+    assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 40, dtype=torch.bfloat16)) == (64 if on_grid else 128)
+    assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 40, dtype=torch.float32)) == 64
     assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 160, dtype=torch.bfloat16)) == 256
     assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 256, dtype=torch.bfloat16)) == 0
-    assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 16, dtype=torch.bfloat16)) == (64 if on_grid else 32)
+    assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 16, dtype=torch.float32)) == (64 if on_grid else 32)
+    # the vector kernels asked for by name, or attention dropout: their head sizes
+    cfg_g = rh._Config(dict(query_chunk_size=cfg.qc, key_chunk_size=cfg.kc, causal_block_size=cbs, impl="generic"))
+    assert rh._padded_head_size(cfg_g, _FakeMaskInputs(), q32) == 0
     with pytest.raises(NotImplementedError):
         rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 272, dtype=torch.bfloat16))
     assert rh._padded_head_size(cfg, _FakeMaskInputs(), torch.zeros(1, 1, 1, 128, dtype=torch.bfloat16)) == 0
