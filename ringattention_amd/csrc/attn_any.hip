@@ -12,7 +12,7 @@
 // are not masked skips the element-wise evaluation.
 //
 // Semantics follow ringattention_jax.py:130-145 (forward tile), :220-233 (backward tile), :272-322 (bias / mask)
-// and :324-331 (skip predicate), through the same row_info() / logit() the generic kernels use.
+// and :324-331 (skip predicate): row_info() of the generic kernels and their logit(), restated over per-tile tables.
 #include "generic_args.hpp"
 #include "../../include/ringattn_hip_measure.h"
 
@@ -50,20 +50,20 @@ __device__ __forceinline__ float any_sum_xor32(float x) {
 template <int HD>
 struct AnyStage {
   static constexpr int SLOTS = HD / 8, NCH = ANY_TILE * SLOTS / ANY_THREADS;
-  uint4 r[NCH];
+  any_u32x4 r[NCH];
   __device__ __forceinline__ void load(const uint16_t* base, int64_t stride, int row0, int limit, int tid) {
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       const int c = tid + ANY_THREADS * i, row = c / SLOTS, slot = c % SLOTS;
       const int gr = min(row0 + row, limit - 1);
-      r[i] = *(const uint4*)(base + (int64_t)gr * stride + slot * 8);
+      r[i] = *(const any_u32x4*)(base + (int64_t)gr * stride + slot * 8);
     }
   }
   __device__ __forceinline__ void store(uint16_t* lds, int tid) const {
 #pragma unroll
     for (int i = 0; i < NCH; i++) {
       const int c = tid + ANY_THREADS * i, row = c / SLOTS, slot = c % SLOTS;
-      *(uint4*)(lds + row * HD + ((slot ^ any_swz(row)) << 3)) = r[i];
+      *(any_u32x4*)(lds + row * HD + ((slot ^ any_swz(row)) << 3)) = r[i];
     }
   }
 };
@@ -121,16 +121,74 @@ __device__ __forceinline__ long long any_wave_min(long long v) {
   return v;
 }
 
-// segment id and additive bias of key kj (clamped into the shard) for the lanes' rows: what a tile keeps in LDS
+// segment id of key kj (already clamped into the shard)
 __device__ __forceinline__ int any_key_seg(const MaskView& mv, int b, int kj) {
   if (!mv.seg) return 0;
   const int ki = kj / mv.kc;
   const int idx = clamp_seg_index(((long long)mv.k_start + ki) * mv.kc, mv.kc, mv.seg_len, kj % mv.kc);
   return mv.seg[(int64_t)b * mv.seg_sb + idx];
 }
+// causal block (:326-331 compare query and key positions in units of causal_block_size) of local key kj
 __device__ __forceinline__ long long any_key_block(const MaskView& mv, int kj) {
   const long long gk = mv.global_k(kj);
   return mv.cbs > 1 ? gk / mv.cbs : gk;
+}
+// a block index relative to a tile's base, as an int that still orders correctly against offsets 0 .. 64
+__device__ __forceinline__ int any_rel(long long x) { return (int)(x < -2 ? -2 : (x > (1 << 20) ? (1 << 20) : x)); }
+
+// What a 64-key tile leaves in LDS for the element-wise evaluation by the lanes that own query rows: per key its
+// segment id, its bias (0 without a per-key bias; min(bias, 0) next to a mask, :299,:309) and its causal block
+// relative to the block of the tile's first key.
+struct AnyKeyTables {
+  int seg[ANY_TILE];
+  float bias[ANY_TILE];
+  int blk[ANY_TILE];
+  long long blk0;
+};
+__device__ __forceinline__ void any_stage_keys(AnyKeyTables& T, const MaskView& mv, int b, int h, int k0, int skv,
+                                               bool bias_per_key, int tid) {
+  if (tid < ANY_TILE) {
+    const int kj = min(k0 + tid, skv - 1);
+    T.seg[tid] = any_key_seg(mv, b, kj);
+    float add = 0.f;
+    if (bias_per_key) {
+      add = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(kj) * mv.bias_sk];
+      if (mv.any_mask) add = fminf(add, 0.f);
+    }
+    T.bias[tid] = add;
+    const long long b0 = any_key_block(mv, min(k0, skv - 1));
+    T.blk[tid] = mv.cbs > 0 ? (int)(any_key_block(mv, kj) - b0) : 0;
+    if (tid == 0) T.blk0 = b0;
+  }
+}
+
+// What a 64-row query tile leaves in LDS for the lanes that own key rows: the softmax statistics of every row and the
+// row's part of the mask (run prefix, segment id, causal block relative to the block of the tile's first row).
+struct AnyRowTables {
+  float m[ANY_TILE], rden[ANY_TILE], delta[ANY_TILE];
+  int kend[ANY_TILE], seg[ANY_TILE], blk[ANY_TILE];
+  int64_t bias_off[ANY_TILE], keep_off[ANY_TILE];
+  long long blk0;
+  int kend_min;
+};
+
+// logit of (this lane's row, key kk of the tile) from the raw dot product: logit() of the generic kernels with the
+// per-key parts read from the tile's tables.  drow: the row's causal block relative to the tile's base.
+__device__ __forceinline__ float any_logit_row(const MaskView& mv, const RowInfo& ri, const AnyKeyTables& T, float dot,
+                                               float rscale, int k0, int kk, int skv, int drow, bool bias_per_row) {
+  const int kj = k0 + kk;
+  float add = T.bias[kk];
+  bool masked = (mv.cbs > 0 && drow < T.blk[kk]) || (mv.seg && ri.seg != T.seg[kk]);
+  if (bias_per_row || mv.keep) {
+    const long long gk = mv.global_k(min(kj, skv - 1));
+    if (bias_per_row) {
+      add = mv.bias[ri.bias_off + gk * mv.bias_sk];
+      if (mv.any_mask) add = fminf(add, 0.f);                           // minimum(), :299,:309
+    }
+    if (mv.keep) masked = masked || !mv.keep[ri.keep_off + (gk - mv.keep_k0) * mv.keep_sk];   // ringattention_inference.py:24
+  }
+  const float s = masked ? mv.mask_min : fmaf(dot, rscale, add);        // :134-136 (a logit next to finfo.min is absorbed)
+  return kj < ri.kend ? s : RA_NEG_INF;                                 // the pair's chunks do not run (:158-164)
 }
 
 // ------------------------------------------------------------------ forward
@@ -139,8 +197,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
   constexpr int NKS = HD / 16, NDB = HD / 32;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[ANY_TILE * HD];
   __shared__ __attribute__((aligned(16))) uint16_t Vs[ANY_TILE * HD];
-  __shared__ int seg_ks[ANY_TILE];
-  __shared__ float bias_ks[ANY_TILE];
+  __shared__ __attribute__((aligned(16))) AnyKeyTables kt;
   __shared__ int kend_s[4];
   const MaskView mv = resolve_mask(a);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
@@ -187,8 +244,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
   __syncthreads();
   const int kend_wg = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
   const int ntile = (kend_wg + ANY_TILE - 1) / ANY_TILE;
-  const bool bias_per_key = mv.bias && mv.bias_sq == 0;
-  const bool elementwise_always = mv.seg || mv.keep || mv.kbits_k;
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
+  const bool elementwise_always = mv.seg || mv.keep || bias_per_row;
+  const float rscale = 1.f / scale;
 
   AnyTr<HD> tr;
   tr.init(lane);
@@ -197,21 +255,13 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
     sk.load(kbase, a.kv_ss, 0, a.Skv, tid);
     sv.load(vbase, a.kv_ss, 0, a.Skv, tid);
   }
+#pragma unroll 1
   for (int t = 0; t < ntile; t++) {
     const int k0 = t * ANY_TILE;
     __syncthreads();                                   // the tile before this one has been read by every wavefront
     sk.store(Ks, tid);
     sv.store(Vs, tid);
-    if (tid < ANY_TILE) {
-      const int kj = min(k0 + tid, a.Skv - 1);
-      seg_ks[tid] = any_key_seg(mv, b, kj);
-      float add = 0.f;
-      if (bias_per_key) {
-        add = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(kj) * mv.bias_sk];
-        if (mv.any_mask) add = fminf(add, 0.f);                         // minimum(), :299,:309
-      }
-      bias_ks[tid] = add;
-    }
+    any_stage_keys(kt, mv, b, h, k0, a.Skv, bias_per_key, tid);
     __syncthreads();
     if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
       sk.load(kbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
@@ -232,26 +282,31 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
                        (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
     float tmax = RA_NEG_INF;
+    if (plain) {
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++)
+      for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-        float s;
-        if (plain) {
-          float add = 0.f;
-          if (bias_per_key) add = bias_ks[kk];
-          else if (mv.bias) {
-            add = mv.bias[ri.bias_off + mv.global_k(k0 + kk) * mv.bias_sk];
-            if (mv.any_mask) add = fminf(add, 0.f);
+        for (int g = 0; g < 4; g++) {
+          const any_f32x4 b4 = *(const any_f32x4*)&kt.bias[blk * 32 + g * 8 + hi * 4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float s = fmaf(S[blk][g * 4 + e], rscale, b4[e]);     // :134-136
+            S[blk][g * 4 + e] = s;
+            tmax = fmaxf(tmax, s);
           }
-          s = S[blk][r] / scale + add;                                  // :134-136
-        } else {
-          s = logit(mv, ri, S[blk][r], scale, k0 + kk, seg_ks[kk]);
         }
-        S[blk][r] = s;
-        tmax = fmaxf(tmax, s);
-      }
+    } else {
+      const int drow = any_rel(ri.gq_blk - kt.blk0);
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+          const float s = any_logit_row(mv, ri, kt, S[blk][r], rscale, k0, kk, a.Skv, drow, bias_per_row);
+          S[blk][r] = s;
+          tmax = fmaxf(tmax, s);
+        }
+    }
     tmax = any_max_xor32(tmax);
     const float m_new = fmaxf(m, tmax);                                 // :138
     const float mm = m_new == RA_NEG_INF ? 0.f : m_new;                 // nothing ran for this row yet: every p is 0
@@ -315,8 +370,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
   constexpr int NKS = HD / 16, NDB = HD / 32;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[ANY_TILE * HD];
   __shared__ __attribute__((aligned(16))) uint16_t Vs[ANY_TILE * HD];
-  __shared__ int seg_ks[ANY_TILE];
-  __shared__ float bias_ks[ANY_TILE];
+  __shared__ __attribute__((aligned(16))) AnyKeyTables kt;
   __shared__ int kend_s[4];
   const MaskView mv = resolve_mask(a);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
@@ -353,8 +407,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
   __syncthreads();
   const int kend_wg = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
   const int ntile = (kend_wg + ANY_TILE - 1) / ANY_TILE;
-  const bool bias_per_key = mv.bias && mv.bias_sq == 0;
-  const bool elementwise_always = mv.seg || mv.keep || mv.kbits_k;
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
+  const bool elementwise_always = mv.seg || mv.keep || bias_per_row;
+  const float rscale = 1.f / scale;
 
   AnyTr<HD> tr;
   tr.init(lane);
@@ -363,21 +418,13 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
     sk.load(kbase, a.kv_ss, 0, a.Skv, tid);
     sv.load(vbase, a.kv_ss, 0, a.Skv, tid);
   }
+#pragma unroll 1
   for (int t = 0; t < ntile; t++) {
     const int k0 = t * ANY_TILE;
     __syncthreads();
     sk.store(Ks, tid);
     sv.store(Vs, tid);
-    if (tid < ANY_TILE) {
-      const int kj = min(k0 + tid, a.Skv - 1);
-      seg_ks[tid] = any_key_seg(mv, b, kj);
-      float add = 0.f;
-      if (bias_per_key) {
-        add = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(kj) * mv.bias_sk];
-        if (mv.any_mask) add = fminf(add, 0.f);
-      }
-      bias_ks[tid] = add;
-    }
+    any_stage_keys(kt, mv, b, h, k0, a.Skv, bias_per_key, tid);
     __syncthreads();
     if (t + 1 < ntile) {
       sk.load(kbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
@@ -398,27 +445,31 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
     }
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
                        (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
+    if (plain) {
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++)
+      for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-        float s;
-        if (plain) {
-          float add = 0.f;
-          if (bias_per_key) add = bias_ks[kk];
-          else if (mv.bias) {
-            add = mv.bias[ri.bias_off + mv.global_k(k0 + kk) * mv.bias_sk];
-            if (mv.any_mask) add = fminf(add, 0.f);
+        for (int g = 0; g < 4; g++) {
+          const any_f32x4 b4 = *(const any_f32x4*)&kt.bias[blk * 32 + g * 8 + hi * 4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p = __expf(fmaf(S[blk][g * 4 + e], rscale, b4[e]) - m) * rden;      // :226
+            S[blk][g * 4 + e] = (dP[blk][g * 4 + e] - delta) * p;                             // dS^T, :229
           }
-          s = S[blk][r] / scale + add;
-        } else {
-          s = logit(mv, ri, S[blk][r], scale, k0 + kk, seg_ks[kk]);
         }
-        const float p = __expf(s - m) * rden;                           // :226
-        // a pair whose tile does not run contributes nothing (:246-257)
-        S[blk][r] = (k0 + kk < ri.kend) ? (dP[blk][r] - delta) * p : 0.f;   // dS^T, :229
-      }
+    } else {
+      const int drow = any_rel(ri.gq_blk - kt.blk0);
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+          const float s = any_logit_row(mv, ri, kt, S[blk][r], rscale, k0, kk, a.Skv, drow, bias_per_row);
+          const float p = __expf(s - m) * rden;                         // :226
+          // a pair whose tile does not run contributes nothing (:246-257)
+          S[blk][r] = (k0 + kk < ri.kend) ? (dP[blk][r] - delta) * p : 0.f;   // dS^T, :229
+        }
+    }
 #pragma unroll
     for (int blk = 0; blk < 2; blk++)
 #pragma unroll
@@ -458,9 +509,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
   constexpr int NKS = HD / 16, NDB = HD / 32;
   __shared__ __attribute__((aligned(16))) uint16_t Qs[ANY_TILE * HD];
   __shared__ __attribute__((aligned(16))) uint16_t Gs[ANY_TILE * HD];
-  __shared__ float r_m[ANY_TILE], r_rden[ANY_TILE], r_delta[ANY_TILE];
-  __shared__ RowInfo r_info[ANY_TILE];
-  __shared__ int r_kend_min;
+  __shared__ __attribute__((aligned(16))) AnyRowTables rt;
   const MaskView mv = resolve_mask(a);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int b = blockIdx.z, h = blockIdx.y;
@@ -473,7 +522,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
   const uint16_t* vp = (const uint16_t*)a.v + koff;
   const uint16_t* qbase = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)h * HD;
   const uint16_t* gbase = (const uint16_t*)a.g + (int64_t)b * a.q_sb + (int64_t)h * HD;
-  const float scale = sqrtf((float)a.sdim);
+  const float scale = sqrtf((float)a.sdim), rscale = 1.f / scale;
 
   any_bf16x8 kf[NKS], vf[WANT_DK ? NKS : 1];
 #pragma unroll
@@ -488,13 +537,15 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[db][r] = 0.f;
   const int seg_k = any_key_seg(mv, b, rk);
+  const long long gk = mv.global_k(rk);
+  const long long kblk = any_key_block(mv, rk);                        // this lane's key
   const int key_hi_w = first_key + wave * 32 + 32;                     // one past the wavefront's last key
-  const long long gkblk_max_w = any_key_block(mv, min(key_hi_w, a.Skv) - 1);
-  const bool bias_per_key = mv.bias && mv.bias_sq == 0;
-  const bool elementwise_always = mv.seg || mv.keep || mv.kbits_k || (mv.bias && !bias_per_key);
+  const long long kblk_max_w = any_key_block(mv, min(key_hi_w, a.Skv) - 1);
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
+  const bool elementwise_always = mv.seg || mv.keep || bias_per_row;
   float bias_k = 0.f;                                                  // a bias per key is a lane scalar here
   if (bias_per_key) {
-    bias_k = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(rk) * mv.bias_sk];
+    bias_k = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + gk * mv.bias_sk];
     if (mv.any_mask) bias_k = fminf(bias_k, 0.f);
   }
   const bool wave_valid = first_key + wave * 32 < a.Skv;               // some key of the wavefront exists
@@ -513,23 +564,27 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
     sq.load(qbase, a.q_ss, t_first * ANY_TILE, a.Sq, tid);
     sg.load(gbase, a.q_ss, t_first * ANY_TILE, a.Sq, tid);
   }
+#pragma unroll 1
   for (int t = t_first; t < ntile; t++) {
     const int q0 = t * ANY_TILE;
     __syncthreads();
     sq.store(Qs, tid);
     sg.store(Gs, tid);
-    if (tid == 0) r_kend_min = 0x7fffffff;
+    if (tid == 0) rt.kend_min = 0x7fffffff;
     __syncthreads();
     if (tid < ANY_TILE) {
       const int row = q0 + tid;
       const bool rv = row < a.Sq;
       const int rr = rv ? row : a.Sq - 1;
       const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rr;
-      r_m[tid] = a.mx[st]; r_rden[tid] = 1.f / a.den[st]; r_delta[tid] = a.delta[st];
-      RowInfo ri = row_info(mv, b, h, rr, a.Skv);
-      if (!rv) ri.kend = 0;
-      r_info[tid] = ri;
-      atomicMin(&r_kend_min, ri.kend);
+      rt.m[tid] = a.mx[st]; rt.rden[tid] = 1.f / a.den[st]; rt.delta[tid] = a.delta[st];
+      const RowInfo ri = row_info(mv, b, h, rr, a.Skv);
+      const RowInfo r0 = row_info(mv, b, h, q0, a.Skv);
+      const int kend = rv ? ri.kend : 0;
+      rt.kend[tid] = kend; rt.seg[tid] = ri.seg; rt.blk[tid] = mv.cbs > 0 ? (int)(ri.gq_blk - r0.gq_blk) : 0;
+      rt.bias_off[tid] = ri.bias_off; rt.keep_off[tid] = ri.keep_off;
+      if (tid == 0) rt.blk0 = r0.gq_blk;
+      atomicMin(&rt.kend_min, kend);
     }
     __syncthreads();
     if (t + 1 < ntile) {
@@ -551,23 +606,41 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
       }
     }
     // every pair of (tile rows, the wavefront's keys) runs and is unmasked
-    const bool plain = !elementwise_always && all_valid && key_hi_w <= r_kend_min &&
-                       (mv.cbs <= 0 || r_info[0].gq_blk >= gkblk_max_w);
+    const bool plain = !elementwise_always && all_valid && key_hi_w <= rt.kend_min &&
+                       (mv.cbs <= 0 || rt.blk0 >= kblk_max_w);
+    if (plain) {
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++)
+      for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int qq = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-        float p;
-        if (plain) {
-          p = __expf(S[blk][r] / scale + bias_k - r_m[qq]) * r_rden[qq];
-        } else {
-          const RowInfo ri = r_info[qq];
-          const float s = logit(mv, ri, S[blk][r], scale, kj, seg_k);
-          p = (valid && kj < ri.kend) ? __expf(s - r_m[qq]) * r_rden[qq] : 0.f;     // :226; (:246-257)
+        for (int g = 0; g < 4; g++) {
+          const int q4 = blk * 32 + g * 8 + hi * 4;
+          const any_f32x4 m4 = *(const any_f32x4*)&rt.m[q4], d4 = *(const any_f32x4*)&rt.rden[q4];
+          const any_f32x4 e4 = *(const any_f32x4*)&rt.delta[q4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p = __expf(fmaf(S[blk][g * 4 + e], rscale, bias_k) - m4[e]) * d4[e];          // :226
+            S[blk][g * 4 + e] = WANT_DK ? (dP[blk][g * 4 + e] - e4[e]) * p : p;                        // dS (:229) or P
+          }
         }
-        S[blk][r] = WANT_DK ? (dP[blk][r] - r_delta[qq]) * p : p;       // dS (:229) or P
-      }
+    } else {
+      const int dkey = any_rel(kblk - rt.blk0);        // this key's causal block relative to the tile's first row's
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int qq = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+          float add = bias_k;
+          bool masked = (mv.cbs > 0 && rt.blk[qq] < dkey) || (mv.seg && rt.seg[qq] != seg_k);
+          if (bias_per_row) {
+            add = mv.bias[rt.bias_off[qq] + gk * mv.bias_sk];
+            if (mv.any_mask) add = fminf(add, 0.f);                     // minimum(), :299,:309
+          }
+          if (mv.keep) masked = masked || !mv.keep[rt.keep_off[qq] + (gk - mv.keep_k0) * mv.keep_sk];
+          const float s = masked ? mv.mask_min : fmaf(S[blk][r], rscale, add);
+          const float p = (valid && kj < rt.kend[qq]) ? __expf(s - rt.m[qq]) * rt.rden[qq] : 0.f;     // :226; (:246-257)
+          S[blk][r] = WANT_DK ? (dP[blk][r] - rt.delta[qq]) * p : p;    // dS (:229) or P
+        }
+    }
 #pragma unroll
     for (int blk = 0; blk < 2; blk++)
 #pragma unroll

@@ -638,10 +638,11 @@ def test_other_head_sizes_run_on_the_mfma_kernels(D, dtype, n, use_seg):
 
 def test_a_large_call_on_the_generic_kernels_warns_once():
     """RA_IMPL_AUTO falls back to the vector-ALU kernels silently for small problems; from 2^28 (query, key) pairs
-    on it says so, once per cause, and kernel_family_of_last_call tells which family ran."""
+    on it says so, once per cause, and kernel_family_of_last_call tells which family ran.  (fp32 inputs with a bias
+    row per query: bf16 ones take the matrix-core kernels that evaluate the mask element by element, silently.)"""
     import warnings
     B, S, H, D, qc = 1, 8192, 4, 64, 128
-    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=1, scale=D ** -0.25)
+    q, k, v, _ = make_qkv(B, S, H, D, dtype=torch.float32, seed=1, scale=D ** -0.25)
     bias = torch.randn(1, 1, qc, S, generator=torch.Generator().manual_seed(2))       # one bias row per query of a chunk
     kw = kwargs(qc, qc, 1)
     qd, kd, vd, bd = (t.to(DEV) for t in (q, k, v, bias))
@@ -660,6 +661,13 @@ def test_a_large_call_on_the_generic_kernels_warns_once():
         warnings.simplefilter("always")
         ra.ringattention(qd[:, :256], kd[:, :256], vd[:, :256], bd[..., :256], None, None, axis_name=None,
                          float32_logits=True, blockwise_kwargs=kw)
+    assert not [w for w in seen if "generic vector-ALU kernels" in str(w.message)]
+    # the same large call in bf16
+    with torch.no_grad(), warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        ra.ringattention(qd.bfloat16(), kd.bfloat16(), vd.bfloat16(), bd, None, None, axis_name=None, float32_logits=True,
+                         blockwise_kwargs=kw)
+    assert ra.kernel_family_of_last_call()["forward"] == "mfma_bf16_any"
     assert not [w for w in seen if "generic vector-ALU kernels" in str(w.message)]
 
 
