@@ -5,11 +5,13 @@
 // of attn_mfma.hip do not take; attention dropout stays with the generic kernels.
 //
 // A workgroup of four wavefronts keeps 128 rows of one operand in registers (32 per wavefront: a lane owns one of
-// them, so that row's softmax statistics are lane scalars) and streams 64-row tiles of the others through LDS, a
-// tile ahead in registers.  Products are formed transposed, S^T = K Q^T, so the C layout hands every lane its own
-// row's logits; P^T (dS^T) goes back in as a B operand from the same registers after one exchange with the partner
-// lane, and the second operand of O^T += V^T P^T comes from LDS transpose reads.  A tile whose pairs all run and
-// are not masked skips the element-wise evaluation.
+// them, so that row's softmax statistics are lane scalars) and streams 64-row tiles of the others through two LDS
+// buffers, loaded straight from global memory a tile ahead (buffer_load ... lds), one barrier per tile.  Products are
+// formed transposed, S^T = K Q^T, so the C layout hands every lane its own row's logits; P^T (dS^T) goes back in as a
+// B operand from the same registers after one exchange with the partner lane, and the second operand of
+// O^T += V^T P^T comes from LDS transpose reads.  With one wavefront per SIMD nothing hides a wait, so the LDS reads
+// of a group of eight products are issued among the MFMAs of the group before.  A tile whose pairs all run and are
+// not masked skips the element-wise evaluation.
 //
 // Semantics follow ringattention_jax.py:130-145 (forward tile), :220-233 (backward tile), :272-322 (bias / mask)
 // and :324-331 (skip predicate): row_info() of the generic kernels and their logit(), restated over per-tile tables.
@@ -45,28 +47,27 @@ __device__ __forceinline__ float any_sum_xor32(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// One 64-row tile of a (B, S, H, D) operand on its way to LDS: 16-byte chunks, a row's chunks on consecutive lanes.
-// Rows past `limit` repeat the last row (finite data that the mask logic never lets through).
+// One 64-row tile of a (B, S, H, D) operand straight into an LDS buffer: a wavefront's load instruction fills 1024
+// consecutive bytes (lane l the 16 bytes at 16 l), that is rows (4 i + wave) * RPL .. + RPL - 1 of the tile; the lane
+// fetches the logical slot that belongs at its place (the swizzle is applied on the global side).  `base` is the
+// tile's first row; rows past rows_avail repeat the last one (finite data that the mask logic never lets through).
+// The loads are asynchronous: any_tile_barrier() before the buffer is read.
+typedef __attribute__((address_space(3))) void* any_lds_ptr;
 template <int HD>
-struct AnyStage {
-  static constexpr int SLOTS = HD / 8, NCH = ANY_TILE * SLOTS / ANY_THREADS;
-  any_u32x4 r[NCH];
-  __device__ __forceinline__ void load(const uint16_t* base, int64_t stride, int row0, int limit, int tid) {
+__device__ __forceinline__ void any_tile_to_lds(uint16_t* lds_tile, const uint16_t* base, int64_t stride, int rows_avail,
+                                                int wave, int lane) {
+  constexpr int SLOTS = HD / 8, RPL = 64 / SLOTS, NL = ANY_TILE / RPL / 4;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7fffffff, 0x00020000);
 #pragma unroll
-    for (int i = 0; i < NCH; i++) {
-      const int c = tid + ANY_THREADS * i, row = c / SLOTS, slot = c % SLOTS;
-      const int gr = min(row0 + row, limit - 1);
-      r[i] = *(const any_u32x4*)(base + (int64_t)gr * stride + slot * 8);
-    }
+  for (int i = 0; i < NL; i++) {
+    const int r = (4 * i + wave) * RPL + lane / SLOTS, c = (lane % SLOTS) ^ any_swz(r);
+    const uint32_t voff = 2u * (uint32_t)(min(r, rows_avail - 1) * (int)stride + c * 8);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (any_lds_ptr)(lds_tile + (4 * i + wave) * 512), 16, voff, 0, 0, 0);
   }
-  __device__ __forceinline__ void store(uint16_t* lds, int tid) const {
-#pragma unroll
-    for (int i = 0; i < NCH; i++) {
-      const int c = tid + ANY_THREADS * i, row = c / SLOTS, slot = c % SLOTS;
-      *(any_u32x4*)(lds + row * HD + ((slot ^ any_swz(row)) << 3)) = r[i];
-    }
-  }
-};
+}
+// every load and LDS write of this wavefront has landed, then the workgroup meets: the tile loaded before is complete
+// in LDS and nobody reads the buffer the next loads will fill
+__device__ __forceinline__ void any_tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // A operand of contraction step ks (16 head dimensions): row `row` of an LDS tile, this lane's eight elements
 template <int HD>
@@ -106,6 +107,64 @@ __device__ __forceinline__ any_bf16x8 any_bop(const any_f32x16& c, int K) {
   const any_u32x2 b = __builtin_amdgcn_permlane32_swap(x1, y1, false, false);
   const any_u32x4 v = {a[0], b[0], a[1], b[1]};
   return __builtin_bit_cast(any_bf16x8, v);
+}
+
+// C[blk] += (rows 32 blk .. 32 blk + 31 of an LDS tile) x (the lane's resident operand), blk = 0, 1: the LDS reads of
+// a group of eight contraction steps are issued among the MFMAs of the group before.
+template <int HD>
+__device__ __forceinline__ void any_products(const uint16_t* tile, const any_bf16x8 (&bq)[HD / 16], any_f32x16 (&C)[2],
+                                             int lo, int hi) {
+  constexpr int G = 8, GPB = HD / 16 / G, NG = 2 * GPB;                 // groups per 32-row block, groups in all
+  any_bf16x8 F[2][G];
+#pragma unroll
+  for (int i = 0; i < G; i++) F[0][i] = any_row_frag<HD>(tile, lo, i, hi);
+  __builtin_amdgcn_sched_barrier(0);                   // all of the first group's reads go out before its first MFMA
+#pragma unroll
+  for (int g = 0; g < NG; g++) {
+    if (g + 1 < NG) {
+#pragma unroll
+      for (int i = 0; i < G; i++)
+        F[(g + 1) & 1][i] = any_row_frag<HD>(tile, ((g + 1) / GPB) * 32 + lo, ((g + 1) % GPB) * G + i, hi);
+    }
+#pragma unroll
+    for (int i = 0; i < G; i++)
+      C[g / GPB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[g & 1][i], bq[(g % GPB) * G + i], C[g / GPB], 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
+// acc^T (head dimensions x the lanes' rows) += tile^T P^T for the 64 tile rows, P in the C layout of any_products:
+// four steps of 16 tile rows, the transpose reads of a step issued among the MFMAs of the step before.
+template <int HD>
+__device__ __forceinline__ void any_accumulate(const uint16_t* tile, const AnyTr<HD>& tr, const any_f32x16 (&P)[2],
+                                               any_f32x16 (&acc)[HD / 32]) {
+  constexpr int NDB = HD / 32;
+  any_bf16x8 F[2][NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; db++) F[0][db] = tr.frag(tile, db);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < 4; s++) {
+    if (s + 1 < 4) {
+#pragma unroll
+      for (int db = 0; db < NDB; db++) F[(s + 1) & 1][db] = tr.frag(tile + (s + 1) * 16 * HD, db);
+    }
+    const any_bf16x8 bop = any_bop(P[s >> 1], s & 1);
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[s & 1][db], bop, acc[db], 0, 0, 0);
+#pragma unroll
+    for (int db = 0; db < NDB; db++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (s + 1 < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
 }
 
 __device__ __forceinline__ int any_wave_max(int v) {
@@ -172,6 +231,26 @@ struct AnyRowTables {
   int kend_min;
 };
 
+__device__ __forceinline__ void any_stage_rows(AnyRowTables& T, const GenericArgs& a, const MaskView& mv, int b, int h,
+                                               int q0, int tid) {
+  if (tid < ANY_TILE) {
+    const int row = q0 + tid;
+    const bool rv = row < a.Sq;
+    const int rr = rv ? row : a.Sq - 1;
+    const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rr;
+    T.m[tid] = a.mx[st]; T.rden[tid] = 1.f / a.den[st]; T.delta[tid] = a.delta[st];
+    const RowInfo ri = row_info(mv, b, h, rr, a.Skv);
+    const RowInfo r0 = row_info(mv, b, h, q0, a.Skv);
+    const int kend = rv ? ri.kend : 0;
+    T.kend[tid] = kend; T.seg[tid] = ri.seg; T.blk[tid] = mv.cbs > 0 ? (int)(ri.gq_blk - r0.gq_blk) : 0;
+    T.bias_off[tid] = ri.bias_off; T.keep_off[tid] = ri.keep_off;
+    if (tid == 0) T.blk0 = r0.gq_blk;
+    // the smallest run prefix of the tile's rows: rows are in order and the prefix grows with the row's chunk, so it
+    // is the first row's, or 0 when a row past the end sits in the tile
+    if (tid == 0) T.kend_min = (q0 + ANY_TILE <= a.Sq) ? kend : 0;
+  }
+}
+
 // logit of (this lane's row, key kk of the tile) from the raw dot product: logit() of the generic kernels with the
 // per-key parts read from the tile's tables.  drow: the row's causal block relative to the tile's base.
 __device__ __forceinline__ float any_logit_row(const MaskView& mv, const RowInfo& ri, const AnyKeyTables& T, float dot,
@@ -195,9 +274,9 @@ __device__ __forceinline__ float any_logit_row(const MaskView& mv, const RowInfo
 template <int HD>
 __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[ANY_TILE * HD];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[ANY_TILE * HD];
-  __shared__ __attribute__((aligned(16))) AnyKeyTables kt;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) AnyKeyTables kts[2];
   __shared__ int kend_s[4];
   const MaskView mv = resolve_mask(a);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
@@ -250,34 +329,32 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
 
   AnyTr<HD> tr;
   tr.init(lane);
-  AnyStage<HD> sk, sv;
   if (ntile > 0) {
-    sk.load(kbase, a.kv_ss, 0, a.Skv, tid);
-    sv.load(vbase, a.kv_ss, 0, a.Skv, tid);
+    any_tile_to_lds<HD>(Ks[0], kbase, a.kv_ss, a.Skv, wave, lane);
+    any_tile_to_lds<HD>(Vs[0], vbase, a.kv_ss, a.Skv, wave, lane);
+    any_stage_keys(kts[0], mv, b, h, 0, a.Skv, bias_per_key, tid);
   }
 #pragma unroll 1
   for (int t = 0; t < ntile; t++) {
     const int k0 = t * ANY_TILE;
-    __syncthreads();                                   // the tile before this one has been read by every wavefront
-    sk.store(Ks, tid);
-    sv.store(Vs, tid);
-    any_stage_keys(kt, mv, b, h, k0, a.Skv, bias_per_key, tid);
-    __syncthreads();
+    any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
     if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
-      sk.load(kbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
-      sv.load(vbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
+      const int k1 = k0 + ANY_TILE;
+      any_tile_to_lds<HD>(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
+      any_tile_to_lds<HD>(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
+      any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
     }
     if (k0 >= kend_max_w) continue;                    // no row of this wavefront runs against these keys
+    const uint16_t* Kt = Ks[t & 1];
+    const uint16_t* Vt = Vs[t & 1];
+    const AnyKeyTables& kt = kts[t & 1];
 
     any_f32x16 S[2];                                   // S^T, two blocks of 32 keys: register 4 g + e = key 8 g + 4 hi + e
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
+    for (int blk = 0; blk < 2; blk++)
 #pragma unroll
       for (int r = 0; r < 16; r++) S[blk][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < NKS; ks++)
-        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Ks, blk * 32 + lo, ks, hi), qf[ks], S[blk], 0, 0, 0);   // :134
-    }
+    any_products<HD>(Kt, qf, S, lo, hi);               // :134
     // every pair of the tile runs and is unmasked for every row of the wavefront: logit = dot / scale + bias
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
                        (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
@@ -328,16 +405,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[db][r] *= corr;                // :143
     }
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int K = 0; K < 2; K++) {
-        const any_bf16x8 bop = any_bop(S[blk], K);
-        const uint16_t* rows16 = Vs + (blk * 32 + K * 16) * HD;
-#pragma unroll
-        for (int db = 0; db < NDB; db++)
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr.frag(rows16, db), bop, acc[db], 0, 0, 0);   // :141
-      }
+    any_accumulate<HD>(Vt, tr, S, acc);                // :141
   }
   if (valid) {
     const float den = any_sum_xor32(l);
@@ -368,9 +436,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
 template <int HD>
 __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[ANY_TILE * HD];
-  __shared__ __attribute__((aligned(16))) uint16_t Vs[ANY_TILE * HD];
-  __shared__ __attribute__((aligned(16))) AnyKeyTables kt;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Vs[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) AnyKeyTables kts[2];
   __shared__ int kend_s[4];
   const MaskView mv = resolve_mask(a);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
@@ -413,36 +481,33 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
 
   AnyTr<HD> tr;
   tr.init(lane);
-  AnyStage<HD> sk, sv;
   if (ntile > 0) {
-    sk.load(kbase, a.kv_ss, 0, a.Skv, tid);
-    sv.load(vbase, a.kv_ss, 0, a.Skv, tid);
+    any_tile_to_lds<HD>(Ks[0], kbase, a.kv_ss, a.Skv, wave, lane);
+    any_tile_to_lds<HD>(Vs[0], vbase, a.kv_ss, a.Skv, wave, lane);
+    any_stage_keys(kts[0], mv, b, h, 0, a.Skv, bias_per_key, tid);
   }
 #pragma unroll 1
   for (int t = 0; t < ntile; t++) {
     const int k0 = t * ANY_TILE;
-    __syncthreads();
-    sk.store(Ks, tid);
-    sv.store(Vs, tid);
-    any_stage_keys(kt, mv, b, h, k0, a.Skv, bias_per_key, tid);
-    __syncthreads();
-    if (t + 1 < ntile) {
-      sk.load(kbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
-      sv.load(vbase, a.kv_ss, k0 + ANY_TILE, a.Skv, tid);
+    any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
+    if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
+      const int k1 = k0 + ANY_TILE;
+      any_tile_to_lds<HD>(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
+      any_tile_to_lds<HD>(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
+      any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
     }
     if (k0 >= kend_max_w) continue;
+    const uint16_t* Kt = Ks[t & 1];
+    const uint16_t* Vt = Vs[t & 1];
+    const AnyKeyTables& kt = kts[t & 1];
 
     any_f32x16 S[2], dP[2];
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
+    for (int blk = 0; blk < 2; blk++)
 #pragma unroll
       for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; dP[blk][r] = 0.f; }
-#pragma unroll
-      for (int ks = 0; ks < NKS; ks++) {
-        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Ks, blk * 32 + lo, ks, hi), qf[ks], S[blk], 0, 0, 0);   // :223-225
-        dP[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Vs, blk * 32 + lo, ks, hi), gf[ks], dP[blk], 0, 0, 0); // :228
-      }
-    }
+    any_products<HD>(Kt, qf, S, lo, hi);               // :223-225
+    any_products<HD>(Vt, gf, dP, lo, hi);              // :228
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
                        (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
     if (plain) {
@@ -470,16 +535,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
           S[blk][r] = (k0 + kk < ri.kend) ? (dP[blk][r] - delta) * p : 0.f;   // dS^T, :229
         }
     }
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int K = 0; K < 2; K++) {
-        const any_bf16x8 bop = any_bop(S[blk], K);
-        const uint16_t* rows16 = Ks + (blk * 32 + K * 16) * HD;
-#pragma unroll
-        for (int db = 0; db < NDB; db++)
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr.frag(rows16, db), bop, acc[db], 0, 0, 0);   // :230
-      }
+    any_accumulate<HD>(Kt, tr, S, acc);                // :230
   }
   if (valid) {
     const int64_t off = (int64_t)h * HD + hi * 4;
@@ -507,9 +563,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
 template <int HD, bool WANT_DK>
 __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
-  __shared__ __attribute__((aligned(16))) uint16_t Qs[ANY_TILE * HD];
-  __shared__ __attribute__((aligned(16))) uint16_t Gs[ANY_TILE * HD];
-  __shared__ __attribute__((aligned(16))) AnyRowTables rt;
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Gs[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) AnyRowTables rts[2];
   const MaskView mv = resolve_mask(a);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
   const int b = blockIdx.z, h = blockIdx.y;
@@ -524,7 +580,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
   const uint16_t* gbase = (const uint16_t*)a.g + (int64_t)b * a.q_sb + (int64_t)h * HD;
   const float scale = sqrtf((float)a.sdim), rscale = 1.f / scale;
 
-  any_bf16x8 kf[NKS], vf[WANT_DK ? NKS : 1];
+  any_bf16x8 kf[NKS], vf[NKS];
 #pragma unroll
   for (int ks = 0; ks < NKS; ks++) kf[ks] = *(const any_bf16x8*)(kp + ks * 16 + hi * 8);
   if (WANT_DK) {
@@ -553,7 +609,6 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
 
   AnyTr<HD> tr;
   tr.init(lane);
-  AnyStage<HD> sq, sg;
   // query tiles whose last row's run prefix ends before this block's first key hold nothing for it; the prefix grows
   // with the query chunk, so the tiles that count are a suffix
   int t_first = 0;
@@ -561,50 +616,33 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
   while (t_first < ntile &&
          mv.run_prefix_keys((min((t_first + 1) * ANY_TILE, a.Sq) - 1) / mv.qc, a.Skv) <= first_key) t_first++;
   if (t_first < ntile) {
-    sq.load(qbase, a.q_ss, t_first * ANY_TILE, a.Sq, tid);
-    sg.load(gbase, a.q_ss, t_first * ANY_TILE, a.Sq, tid);
+    const int q0 = t_first * ANY_TILE;
+    any_tile_to_lds<HD>(Qs[t_first & 1], qbase + (int64_t)q0 * a.q_ss, a.q_ss, a.Sq - q0, wave, lane);
+    any_tile_to_lds<HD>(Gs[t_first & 1], gbase + (int64_t)q0 * a.q_ss, a.q_ss, a.Sq - q0, wave, lane);
+    any_stage_rows(rts[t_first & 1], a, mv, b, h, q0, tid);
   }
 #pragma unroll 1
   for (int t = t_first; t < ntile; t++) {
     const int q0 = t * ANY_TILE;
-    __syncthreads();
-    sq.store(Qs, tid);
-    sg.store(Gs, tid);
-    if (tid == 0) rt.kend_min = 0x7fffffff;
-    __syncthreads();
-    if (tid < ANY_TILE) {
-      const int row = q0 + tid;
-      const bool rv = row < a.Sq;
-      const int rr = rv ? row : a.Sq - 1;
-      const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rr;
-      rt.m[tid] = a.mx[st]; rt.rden[tid] = 1.f / a.den[st]; rt.delta[tid] = a.delta[st];
-      const RowInfo ri = row_info(mv, b, h, rr, a.Skv);
-      const RowInfo r0 = row_info(mv, b, h, q0, a.Skv);
-      const int kend = rv ? ri.kend : 0;
-      rt.kend[tid] = kend; rt.seg[tid] = ri.seg; rt.blk[tid] = mv.cbs > 0 ? (int)(ri.gq_blk - r0.gq_blk) : 0;
-      rt.bias_off[tid] = ri.bias_off; rt.keep_off[tid] = ri.keep_off;
-      if (tid == 0) rt.blk0 = r0.gq_blk;
-      atomicMin(&rt.kend_min, kend);
-    }
-    __syncthreads();
+    any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
     if (t + 1 < ntile) {
-      sq.load(qbase, a.q_ss, q0 + ANY_TILE, a.Sq, tid);
-      sg.load(gbase, a.q_ss, q0 + ANY_TILE, a.Sq, tid);
+      const int q1 = q0 + ANY_TILE;
+      any_tile_to_lds<HD>(Qs[(t + 1) & 1], qbase + (int64_t)q1 * a.q_ss, a.q_ss, a.Sq - q1, wave, lane);
+      any_tile_to_lds<HD>(Gs[(t + 1) & 1], gbase + (int64_t)q1 * a.q_ss, a.q_ss, a.Sq - q1, wave, lane);
+      any_stage_rows(rts[(t + 1) & 1], a, mv, b, h, q1, tid);
     }
     if (!wave_valid) continue;
+    const uint16_t* Qt = Qs[t & 1];
+    const uint16_t* Gt = Gs[t & 1];
+    const AnyRowTables& rt = rts[t & 1];
 
     any_f32x16 S[2], dP[2];                            // S, dP: the lane's key column; register 4 g + e = query 8 g + 4 hi + e
 #pragma unroll
-    for (int blk = 0; blk < 2; blk++) {
+    for (int blk = 0; blk < 2; blk++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; if (WANT_DK) dP[blk][r] = 0.f; }
-#pragma unroll
-      for (int ks = 0; ks < NKS; ks++) {
-        S[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Qs, blk * 32 + lo, ks, hi), kf[ks], S[blk], 0, 0, 0);
-        if (WANT_DK)
-          dP[blk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(any_row_frag<HD>(Gs, blk * 32 + lo, ks, hi), vf[ks], dP[blk], 0, 0, 0);
-      }
-    }
+      for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; dP[blk][r] = 0.f; }
+    any_products<HD>(Qt, kf, S, lo, hi);
+    if (WANT_DK) any_products<HD>(Gt, vf, dP, lo, hi);
     // every pair of (tile rows, the wavefront's keys) runs and is unmasked
     const bool plain = !elementwise_always && all_valid && key_hi_w <= rt.kend_min &&
                        (mv.cbs <= 0 || rt.blk0 >= kblk_max_w);
@@ -641,16 +679,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
           S[blk][r] = WANT_DK ? (dP[blk][r] - rt.delta[qq]) * p : p;    // dS (:229) or P
         }
     }
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int K = 0; K < 2; K++) {
-        const any_bf16x8 bop = any_bop(S[blk], K);
-        const uint16_t* rows16 = (WANT_DK ? Qs : Gs) + (blk * 32 + K * 16) * HD;
-#pragma unroll
-        for (int db = 0; db < NDB; db++)
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tr.frag(rows16, db), bop, acc[db], 0, 0, 0);   // :231 / :232
-      }
+    any_accumulate<HD>(WANT_DK ? Qt : Gt, tr, S, acc);           // :231 / :232
   }
   if (valid) {
     const int64_t off = (int64_t)h * HD + hi * 4;
