@@ -54,17 +54,34 @@ __device__ __forceinline__ float any_sum_xor32(float x) {
 // The loads are asynchronous: any_tile_barrier() before the buffer is read.
 typedef __attribute__((address_space(3))) void* any_lds_ptr;
 template <int HD>
-__device__ __forceinline__ void any_tile_to_lds(uint16_t* lds_tile, const uint16_t* base, int64_t stride, int rows_avail,
-                                                int wave, int lane) {
-  constexpr int SLOTS = HD / 8, RPL = 64 / SLOTS, NL = ANY_TILE / RPL / 4;
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7fffffff, 0x00020000);
+struct AnyTileLoader {
+  static constexpr int SLOTS = HD / 8, RPL = 64 / SLOTS, NL = ANY_TILE / RPL / 4;
+  uint32_t voff[NL];                                   // byte offset of this lane's chunk of load i from the tile's first row
+  int row0, stride, wave;
+  __device__ __forceinline__ void init(int64_t stride_, int wave_, int lane) {
+    stride = (int)stride_; wave = wave_; row0 = lane / SLOTS;
 #pragma unroll
-  for (int i = 0; i < NL; i++) {
-    const int r = (4 * i + wave) * RPL + lane / SLOTS, c = (lane % SLOTS) ^ any_swz(r);
-    const uint32_t voff = 2u * (uint32_t)(min(r, rows_avail - 1) * (int)stride + c * 8);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (any_lds_ptr)(lds_tile + (4 * i + wave) * 512), 16, voff, 0, 0, 0);
+    for (int i = 0; i < NL; i++) {
+      const int r = (4 * i + wave) * RPL + row0, c = (lane % SLOTS) ^ any_swz(r);
+      voff[i] = 2u * (uint32_t)(r * stride + c * 8);
+    }
   }
-}
+  __device__ __forceinline__ void load(uint16_t* lds_tile, const uint16_t* base, int rows_avail) const {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, 0x7fffffff, 0x00020000);
+    if (rows_avail >= ANY_TILE) {
+#pragma unroll
+      for (int i = 0; i < NL; i++)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (any_lds_ptr)(lds_tile + (4 * i + wave) * 512), 16, voff[i], 0, 0, 0);
+    } else {                                           // the last tile of a length that is no multiple of 64
+#pragma unroll
+      for (int i = 0; i < NL; i++) {
+        const int r = (4 * i + wave) * RPL + row0;
+        const uint32_t v = voff[i] - 2u * (uint32_t)((r - min(r, rows_avail - 1)) * stride);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (any_lds_ptr)(lds_tile + (4 * i + wave) * 512), 16, v, 0, 0, 0);
+      }
+    }
+  }
+};
 // every load and LDS write of this wavefront has landed, then the workgroup meets: the tile loaded before is complete
 // in LDS and nobody reads the buffer the next loads will fill
 __device__ __forceinline__ void any_tile_barrier() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -202,8 +219,11 @@ struct AnyKeyTables {
   int seg[ANY_TILE];
   float bias[ANY_TILE];
   int blk[ANY_TILE];
-  long long blk0;
 };
+// what the tables hold when no tile writes them (no segment ids, no per-key bias, causal block size 1 or none)
+__device__ __forceinline__ void any_init_keys(AnyKeyTables& T, int tid) {
+  if (tid < ANY_TILE) { T.seg[tid] = 0; T.bias[tid] = 0.f; T.blk[tid] = tid; }
+}
 __device__ __forceinline__ void any_stage_keys(AnyKeyTables& T, const MaskView& mv, int b, int h, int k0, int skv,
                                                bool bias_per_key, int tid) {
   if (tid < ANY_TILE) {
@@ -215,9 +235,7 @@ __device__ __forceinline__ void any_stage_keys(AnyKeyTables& T, const MaskView& 
       if (mv.any_mask) add = fminf(add, 0.f);
     }
     T.bias[tid] = add;
-    const long long b0 = any_key_block(mv, min(k0, skv - 1));
-    T.blk[tid] = mv.cbs > 0 ? (int)(any_key_block(mv, kj) - b0) : 0;
-    if (tid == 0) T.blk0 = b0;
+    T.blk[tid] = mv.cbs > 1 ? (int)(any_key_block(mv, kj) - any_key_block(mv, min(k0, skv - 1))) : tid;
   }
 }
 
@@ -240,11 +258,11 @@ __device__ __forceinline__ void any_stage_rows(AnyRowTables& T, const GenericArg
     const int64_t st = (int64_t)b * a.st_sb + (int64_t)h * a.st_sh + rr;
     T.m[tid] = a.mx[st]; T.rden[tid] = 1.f / a.den[st]; T.delta[tid] = a.delta[st];
     const RowInfo ri = row_info(mv, b, h, rr, a.Skv);
-    const RowInfo r0 = row_info(mv, b, h, q0, a.Skv);
+    const long long g0 = mv.global_q(q0), b0 = mv.cbs > 1 ? g0 / mv.cbs : (mv.cbs == 1 ? g0 : 0);   // the first row's block
     const int kend = rv ? ri.kend : 0;
-    T.kend[tid] = kend; T.seg[tid] = ri.seg; T.blk[tid] = mv.cbs > 0 ? (int)(ri.gq_blk - r0.gq_blk) : 0;
+    T.kend[tid] = kend; T.seg[tid] = ri.seg; T.blk[tid] = mv.cbs > 0 ? (int)(ri.gq_blk - b0) : 0;
     T.bias_off[tid] = ri.bias_off; T.keep_off[tid] = ri.keep_off;
-    if (tid == 0) T.blk0 = r0.gq_blk;
+    if (tid == 0) T.blk0 = b0;
     // the smallest run prefix of the tile's rows: rows are in order and the prefix grows with the row's chunk, so it
     // is the first row's, or 0 when a row past the end sits in the tile
     if (tid == 0) T.kend_min = (q0 + ANY_TILE <= a.Sq) ? kend : 0;
@@ -329,10 +347,16 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
 
   AnyTr<HD> tr;
   tr.init(lane);
+  AnyTileLoader<HD> ld;
+  ld.init(a.kv_ss, wave, lane);
+  const bool key_tables = mv.seg || bias_per_key || mv.cbs > 1;        // else: no ids, no bias, key i of a tile in block i
+  any_init_keys(kts[0], tid);
+  any_init_keys(kts[1], tid);
+  __syncthreads();
   if (ntile > 0) {
-    any_tile_to_lds<HD>(Ks[0], kbase, a.kv_ss, a.Skv, wave, lane);
-    any_tile_to_lds<HD>(Vs[0], vbase, a.kv_ss, a.Skv, wave, lane);
-    any_stage_keys(kts[0], mv, b, h, 0, a.Skv, bias_per_key, tid);
+    ld.load(Ks[0], kbase, a.Skv);
+    ld.load(Vs[0], vbase, a.Skv);
+    if (key_tables) any_stage_keys(kts[0], mv, b, h, 0, a.Skv, bias_per_key, tid);
   }
 #pragma unroll 1
   for (int t = 0; t < ntile; t++) {
@@ -340,9 +364,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
     any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
     if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
       const int k1 = k0 + ANY_TILE;
-      any_tile_to_lds<HD>(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
-      any_tile_to_lds<HD>(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
-      any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
+      ld.load(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.Skv - k1);
+      ld.load(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.Skv - k1);
+      if (key_tables) any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
     }
     if (k0 >= kend_max_w) continue;                    // no row of this wavefront runs against these keys
     const uint16_t* Kt = Ks[t & 1];
@@ -373,7 +397,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
           }
         }
     } else {
-      const int drow = any_rel(ri.gq_blk - kt.blk0);
+      const int drow = any_rel(ri.gq_blk - any_key_block(mv, min(k0, a.Skv - 1)));
 #pragma unroll
       for (int blk = 0; blk < 2; blk++)
 #pragma unroll
@@ -481,10 +505,16 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
 
   AnyTr<HD> tr;
   tr.init(lane);
+  AnyTileLoader<HD> ld;
+  ld.init(a.kv_ss, wave, lane);
+  const bool key_tables = mv.seg || bias_per_key || mv.cbs > 1;        // else: no ids, no bias, key i of a tile in block i
+  any_init_keys(kts[0], tid);
+  any_init_keys(kts[1], tid);
+  __syncthreads();
   if (ntile > 0) {
-    any_tile_to_lds<HD>(Ks[0], kbase, a.kv_ss, a.Skv, wave, lane);
-    any_tile_to_lds<HD>(Vs[0], vbase, a.kv_ss, a.Skv, wave, lane);
-    any_stage_keys(kts[0], mv, b, h, 0, a.Skv, bias_per_key, tid);
+    ld.load(Ks[0], kbase, a.Skv);
+    ld.load(Vs[0], vbase, a.Skv);
+    if (key_tables) any_stage_keys(kts[0], mv, b, h, 0, a.Skv, bias_per_key, tid);
   }
 #pragma unroll 1
   for (int t = 0; t < ntile; t++) {
@@ -492,9 +522,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
     any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
     if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
       const int k1 = k0 + ANY_TILE;
-      any_tile_to_lds<HD>(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
-      any_tile_to_lds<HD>(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.kv_ss, a.Skv - k1, wave, lane);
-      any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
+      ld.load(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.Skv - k1);
+      ld.load(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.Skv - k1);
+      if (key_tables) any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
     }
     if (k0 >= kend_max_w) continue;
     const uint16_t* Kt = Ks[t & 1];
@@ -523,7 +553,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
           }
         }
     } else {
-      const int drow = any_rel(ri.gq_blk - kt.blk0);
+      const int drow = any_rel(ri.gq_blk - any_key_block(mv, min(k0, a.Skv - 1)));
 #pragma unroll
       for (int blk = 0; blk < 2; blk++)
 #pragma unroll
@@ -615,10 +645,12 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
   const int ntile = (a.Sq + ANY_TILE - 1) / ANY_TILE;
   while (t_first < ntile &&
          mv.run_prefix_keys((min((t_first + 1) * ANY_TILE, a.Sq) - 1) / mv.qc, a.Skv) <= first_key) t_first++;
+  AnyTileLoader<HD> ld;
+  ld.init(a.q_ss, wave, lane);
   if (t_first < ntile) {
     const int q0 = t_first * ANY_TILE;
-    any_tile_to_lds<HD>(Qs[t_first & 1], qbase + (int64_t)q0 * a.q_ss, a.q_ss, a.Sq - q0, wave, lane);
-    any_tile_to_lds<HD>(Gs[t_first & 1], gbase + (int64_t)q0 * a.q_ss, a.q_ss, a.Sq - q0, wave, lane);
+    ld.load(Qs[t_first & 1], qbase + (int64_t)q0 * a.q_ss, a.Sq - q0);
+    ld.load(Gs[t_first & 1], gbase + (int64_t)q0 * a.q_ss, a.Sq - q0);
     any_stage_rows(rts[t_first & 1], a, mv, b, h, q0, tid);
   }
 #pragma unroll 1
@@ -627,8 +659,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
     any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
     if (t + 1 < ntile) {
       const int q1 = q0 + ANY_TILE;
-      any_tile_to_lds<HD>(Qs[(t + 1) & 1], qbase + (int64_t)q1 * a.q_ss, a.q_ss, a.Sq - q1, wave, lane);
-      any_tile_to_lds<HD>(Gs[(t + 1) & 1], gbase + (int64_t)q1 * a.q_ss, a.q_ss, a.Sq - q1, wave, lane);
+      ld.load(Qs[(t + 1) & 1], qbase + (int64_t)q1 * a.q_ss, a.Sq - q1);
+      ld.load(Gs[(t + 1) & 1], gbase + (int64_t)q1 * a.q_ss, a.Sq - q1);
       any_stage_rows(rts[(t + 1) & 1], a, mv, b, h, q1, tid);
     }
     if (!wave_valid) continue;
@@ -702,6 +734,17 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
       }
   }
 }
+
+// every kernel is instantiated by name: left to the launches below (some of them inside a function template) the host
+// pass of the compiler has been seen to reference a kernel's launch stub without emitting it
+template __global__ void attn_fwd_any_kernel<128>(GenericArgs);
+template __global__ void attn_fwd_any_kernel<256>(GenericArgs);
+template __global__ void attn_bwd_dq_any_kernel<128>(GenericArgs);
+template __global__ void attn_bwd_dq_any_kernel<256>(GenericArgs);
+template __global__ void attn_bwd_dkv_any_kernel<128, true>(GenericArgs);
+template __global__ void attn_bwd_dkv_any_kernel<128, false>(GenericArgs);
+template __global__ void attn_bwd_dkv_any_kernel<256, true>(GenericArgs);
+template __global__ void attn_bwd_dkv_any_kernel<256, false>(GenericArgs);
 
 // ------------------------------------------------------------------ host side
 static bool any_aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
