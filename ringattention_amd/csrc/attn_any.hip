@@ -219,16 +219,21 @@ struct AnyKeyTables {
   int seg[ANY_TILE];
   float bias[ANY_TILE];
   int blk[ANY_TILE];
+  int segmin, segmax;                                  // range of the tile's segment ids
 };
 // what the tables hold when no tile writes them (no segment ids, no per-key bias, causal block size 1 or none)
 __device__ __forceinline__ void any_init_keys(AnyKeyTables& T, int tid) {
   if (tid < ANY_TILE) { T.seg[tid] = 0; T.bias[tid] = 0.f; T.blk[tid] = tid; }
+  if (tid == 0) { T.segmin = 0; T.segmax = 0; }
 }
 __device__ __forceinline__ void any_stage_keys(AnyKeyTables& T, const MaskView& mv, int b, int h, int k0, int skv,
                                                bool bias_per_key, int tid) {
   if (tid < ANY_TILE) {
     const int kj = min(k0 + tid, skv - 1);
-    T.seg[tid] = any_key_seg(mv, b, kj);
+    const int sg = any_key_seg(mv, b, kj);
+    T.seg[tid] = sg;
+    const int sgmin = any_wave_min(sg), sgmax = any_wave_max(sg);       // the staging threads are one wavefront
+    if (tid == 0) { T.segmin = sgmin; T.segmax = sgmax; }
     float add = 0.f;
     if (bias_per_key) {
       add = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + mv.global_k(kj) * mv.bias_sk];
@@ -247,6 +252,7 @@ struct AnyRowTables {
   int64_t bias_off[ANY_TILE], keep_off[ANY_TILE];
   long long blk0;
   int kend_min;
+  int segmin, segmax;                                  // range of the tile's rows' segment ids
 };
 
 __device__ __forceinline__ void any_stage_rows(AnyRowTables& T, const GenericArgs& a, const MaskView& mv, int b, int h,
@@ -261,6 +267,8 @@ __device__ __forceinline__ void any_stage_rows(AnyRowTables& T, const GenericArg
     const long long g0 = mv.global_q(q0), b0 = mv.cbs > 1 ? g0 / mv.cbs : (mv.cbs == 1 ? g0 : 0);   // the first row's block
     const int kend = rv ? ri.kend : 0;
     T.kend[tid] = kend; T.seg[tid] = ri.seg; T.blk[tid] = mv.cbs > 0 ? (int)(ri.gq_blk - b0) : 0;
+    const int sgmin = any_wave_min(ri.seg), sgmax = any_wave_max(ri.seg);       // the staging threads are one wavefront
+    if (tid == 0) { T.segmin = sgmin; T.segmax = sgmax; }
     T.bias_off[tid] = ri.bias_off; T.keep_off[tid] = ri.keep_off;
     if (tid == 0) T.blk0 = b0;
     // the smallest run prefix of the tile's rows: rows are in order and the prefix grows with the row's chunk, so it
@@ -342,7 +350,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
   const int kend_wg = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
   const int ntile = (kend_wg + ANY_TILE - 1) / ANY_TILE;
   const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
-  const bool elementwise_always = mv.seg || mv.keep || bias_per_row;
+  const bool elementwise_always = mv.keep || bias_per_row;
+  const int rseg_min_w = any_wave_min(ri.seg), rseg_max_w = any_wave_max(ri.seg);
   const float rscale = 1.f / scale;
 
   AnyTr<HD> tr;
@@ -372,6 +381,9 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
     const uint16_t* Kt = Ks[t & 1];
     const uint16_t* Vt = Vs[t & 1];
     const AnyKeyTables& kt = kts[t & 1];
+    // no key of the tile shares a segment id with a row of the wavefront: every pair is masked, and where the caller
+    // vouches that every row has a key of its own (skip_masked_tiles) such a tile weighs exactly nothing
+    if (mv.seg && mv.skip_tiles && (kt.segmax < rseg_min_w || kt.segmin > rseg_max_w)) continue;
 
     any_f32x16 S[2];                                   // S^T, two blocks of 32 keys: register 4 g + e = key 8 g + 4 hi + e
 #pragma unroll
@@ -381,7 +393,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
     any_products<HD>(Kt, qf, S, lo, hi);               // :134
     // every pair of the tile runs and is unmasked for every row of the wavefront: logit = dot / scale + bias
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
-                       (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
+                       (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1)) &&
+                       (!mv.seg || (kt.segmin == kt.segmax && rseg_min_w == rseg_max_w && kt.segmin == rseg_min_w));
     float tmax = RA_NEG_INF;
     if (plain) {
 #pragma unroll
@@ -500,7 +513,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
   const int kend_wg = max(max(kend_s[0], kend_s[1]), max(kend_s[2], kend_s[3]));
   const int ntile = (kend_wg + ANY_TILE - 1) / ANY_TILE;
   const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
-  const bool elementwise_always = mv.seg || mv.keep || bias_per_row;
+  const bool elementwise_always = mv.keep || bias_per_row;
+  const int rseg_min_w = any_wave_min(ri.seg), rseg_max_w = any_wave_max(ri.seg);
   const float rscale = 1.f / scale;
 
   AnyTr<HD> tr;
@@ -530,6 +544,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
     const uint16_t* Kt = Ks[t & 1];
     const uint16_t* Vt = Vs[t & 1];
     const AnyKeyTables& kt = kts[t & 1];
+    if (mv.seg && mv.skip_tiles && (kt.segmax < rseg_min_w || kt.segmin > rseg_max_w)) continue;   // as in the forward kernel
 
     any_f32x16 S[2], dP[2];
 #pragma unroll
@@ -539,7 +554,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
     any_products<HD>(Kt, qf, S, lo, hi);               // :223-225
     any_products<HD>(Vt, gf, dP, lo, hi);              // :228
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
-                       (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1));
+                       (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1)) &&
+                       (!mv.seg || (kt.segmin == kt.segmax && rseg_min_w == rseg_max_w && kt.segmin == rseg_min_w));
     if (plain) {
 #pragma unroll
       for (int blk = 0; blk < 2; blk++)
@@ -628,7 +644,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
   const int key_hi_w = first_key + wave * 32 + 32;                     // one past the wavefront's last key
   const long long kblk_max_w = any_key_block(mv, min(key_hi_w, a.Skv) - 1);
   const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
-  const bool elementwise_always = mv.seg || mv.keep || bias_per_row;
+  const bool elementwise_always = mv.keep || bias_per_row;
+  const int kseg_min_w = any_wave_min(seg_k), kseg_max_w = any_wave_max(seg_k);
   float bias_k = 0.f;                                                  // a bias per key is a lane scalar here
   if (bias_per_key) {
     bias_k = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + gk * mv.bias_sk];
@@ -667,6 +684,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
     const uint16_t* Qt = Qs[t & 1];
     const uint16_t* Gt = Gs[t & 1];
     const AnyRowTables& rt = rts[t & 1];
+    // no row of the tile shares a segment id with a key of the wavefront (see the forward kernel)
+    if (mv.seg && mv.skip_tiles && (rt.segmax < kseg_min_w || rt.segmin > kseg_max_w)) continue;
 
     any_f32x16 S[2], dP[2];                            // S, dP: the lane's key column; register 4 g + e = query 8 g + 4 hi + e
 #pragma unroll
@@ -677,7 +696,8 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericAr
     if (WANT_DK) any_products<HD>(Gt, vf, dP, lo, hi);
     // every pair of (tile rows, the wavefront's keys) runs and is unmasked
     const bool plain = !elementwise_always && all_valid && key_hi_w <= rt.kend_min &&
-                       (mv.cbs <= 0 || rt.blk0 >= kblk_max_w);
+                       (mv.cbs <= 0 || rt.blk0 >= kblk_max_w) &&
+                       (!mv.seg || (rt.segmin == rt.segmax && kseg_min_w == kseg_max_w && rt.segmin == kseg_min_w));
     if (plain) {
 #pragma unroll
       for (int blk = 0; blk < 2; blk++)
