@@ -49,3 +49,92 @@ def test_random_configuration_on_the_elementwise_matrix_core_kernels(seed):
     assert_close_scaled(out, ref_out, torch.bfloat16, "out")
     for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
         assert_close_scaled(a, b, torch.bfloat16, name)
+
+
+def _qkv(B, S, H, D, seed, Skv=None):
+    return make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=seed, Skv=Skv, scale=D ** -0.25)
+
+
+@pytest.mark.parametrize("D", [160, 192, 256])
+@pytest.mark.parametrize("n", [1, 4])
+def test_head_sizes_above_128_take_the_elementwise_matrix_core_kernels(D, n):
+    """bf16 calls with a head size above 128 (zero-padded to 256) are dispatched to these kernels by themselves, with
+    documents and a bias, on one device and on a ring; fp32 inputs of the same shape stay on the vector kernels."""
+    B, S, H = 1, 1024, 2
+    q, k, v, do = _qkv(B, S, H, D, 3)
+    seg = packed_segment_ids(B, S, 300, seed=5)
+    bias = torch.randn(1, 1, 1, S, generator=torch.Generator().manual_seed(6))
+    kw = kwargs(128, 128, 1)
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    assert ra.kernel_family_of_last_call() == {"forward": "mfma_bf16_any", "backward": "mfma_bf16_any"}
+    assert_close_scaled(out, ref_out, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close_scaled(a, b, torch.bfloat16, name)
+    if n == 1:
+        run_hip(q.float(), k.float(), v.float(), do.float(), bias, seg, None, n, kw)
+        assert ra.kernel_family_of_last_call() == {"forward": "generic", "backward": "generic"}
+
+
+def test_attention_dropout_stays_off_the_elementwise_matrix_core_kernels():
+    """Attention dropout at a head size above 128: the vector kernels (they hold the -inf bookkeeping of
+    ringattention_jax.py:321); asking for the element-wise matrix-core kernels by name is refused."""
+    B, S, H, D = 1, 256, 1, 160
+    q, k, v, do = _qkv(B, S, H, D, 4)
+    kw = kwargs(64, 64, 1, deterministic=False, attn_pdrop=0.1, dropout_rng=3)
+    run_hip(q, k, v, do, None, None, None, 1, kw)
+    assert ra.kernel_family_of_last_call() == {"forward": "generic", "backward": "generic"}
+    with pytest.raises(NotImplementedError):
+        run_hip(q, k, v, do, None, None, None, 1, dict(kw, impl="mfma_any"))
+
+
+@pytest.mark.parametrize("D,S,Sk,n", [(256, 512, 512, 1), (128, 200, 328, 1), (192, 384, 384, 2), (64, 1000, 1000, 1)])
+def test_boolean_mask_ring_on_the_elementwise_matrix_core_kernels(D, S, Sk, n):
+    """ring_attention_inference with a mask that leaves some rows without a key (so the lengths are not padded) or a
+    head size above 128: the mask is read as bytes, element by element, and a row that attends to nothing averages
+    over all keys (ringattention_inference.py:22-24)."""
+    from oracle import ringattention_oracle as O
+    from tests.test_gpu_inference import _run
+    B, H = 2, 2
+    g = torch.Generator().manual_seed(S + D)
+    q = (torch.randn(B, S, H, D, generator=g) * D ** -0.25).to(torch.bfloat16)
+    k = (torch.randn(B, Sk, H, D, generator=g) * D ** -0.25).to(torch.bfloat16)
+    v = torch.randn(B, Sk, H, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16)
+    mask = torch.rand(B, H, S, Sk, generator=g) < 0.5
+    mask[:, :, 5] = False                                   # a row that attends to nothing
+    out, grads = _run(q, k, v, do, mask, n)
+    fam = ra.kernel_family_of_last_call()
+    assert fam == {"forward": "mfma_bf16_any", "backward": "mfma_bf16_any"}, fam
+    ref_out, res = O.ring_attention_inference_fwd(q, k, v, mask, n, True)
+    ref_grads = O.ring_attention_inference_bwd(n, res, do)
+    assert_close_scaled(out, ref_out, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close_scaled(a, b, torch.bfloat16, name)
+
+
+def test_carry_of_a_ring_step_moves_between_the_kernel_families():
+    """A device's carry (numerator, denominator, max) written by the tiled matrix-core kernels and continued by the
+    element-wise ones, and the other way round, ends where one family alone ends (ringattention_jax.py:38-46)."""
+    B, S, H, D = 1, 512, 2, 128
+    q, k, v, _ = _qkv(B, S, H, D, 8)
+    kw = kwargs(128, 128, 1)
+    qd, kd, vd = (t.to("cuda") for t in (q, k, v))
+
+    def two_steps(first, second):
+        num = torch.zeros(B, 256, H, D, device="cuda")
+        den = torch.zeros(B, H, 256, device="cuda")
+        mx = torch.full((B, H, 256), float("-inf"), device="cuda")
+        carry = (num, den, mx)
+        # device 1 of a ring of two: its own shard, then shard 0
+        ra._blockwise_attention_fwd(qd[:, 256:], kd[:, 256:], vd[:, 256:], carry, 2, 2, None, None, impl=first, **kw)
+        ra._blockwise_attention_fwd(qd[:, 256:], kd[:, :256], vd[:, :256], carry, 2, 0, None, None, impl=second, **kw)
+        torch.cuda.synchronize()
+        return carry
+
+    base = two_steps("mfma", "mfma")
+    for first, second in (("mfma", "mfma_any"), ("mfma_any", "mfma"), ("mfma_any", "mfma_any")):
+        got = two_steps(first, second)
+        out_b, out_g = base[0] / base[1].transpose(1, 2)[..., None], got[0] / got[1].transpose(1, 2)[..., None]
+        assert float((out_b - out_g).abs().max()) < 2e-2, (first, second)
+        assert float((base[2] - got[2]).abs().max()) < 1e-3, (first, second)
