@@ -233,7 +233,8 @@ def bench_attention(args, ring, dropout=False, c1=False):
     fp32 = getattr(args, "dtype", "bf16") == "fp32"
     tdt = torch.float32 if fp32 else torch.bfloat16
     peak = PEAK_F32_TFLOPS if fp32 else PEAK_BF16_TFLOPS
-    sfx = "_f32_kernel" if fp32 else "_ws_kernel"
+    # (a head size above 128: the matrix-core kernels that evaluate the mask element by element)
+    sfx = "_f32_kernel" if fp32 else ("_any_kernel" if D > 128 else "_ws_kernel")
     mk = lambda sc: (torch.randn(B, S, H, D, device=dev, generator=g) * sc).to(tdt)
     q, k, v = mk(qk_scale).requires_grad_(True), mk(qk_scale).requires_grad_(True), mk(v_scale).requires_grad_(True)
     do = torch.randn(B, S, H, D, device=dev, generator=g).to(tdt)
@@ -881,7 +882,7 @@ def main():
                                                               "dropout32k", "c1", "mfma_probe", "vendor_sdpa"])
     ap.add_argument("--seq-len", type=int, default=0, help="override the sequence / cache / token length")
     ap.add_argument("--batch", type=int, default=0, help="attention workloads: batch rows (the configurations have 1)")
-    ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128],
+    ap.add_argument("--head-dim", type=int, default=0, choices=[0, 64, 128, 256],
                     help="attention workloads: head size (the number of heads follows, H * D = 4096)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"],
                     help="attention workloads: dtype of q, k, v (fp32 runs on v_mfma_f32_32x32x2_f32; its roofline is the "
