@@ -138,3 +138,38 @@ def test_carry_of_a_ring_step_moves_between_the_kernel_families():
         out_b, out_g = base[0] / base[1].transpose(1, 2)[..., None], got[0] / got[1].transpose(1, 2)[..., None]
         assert float((out_b - out_g).abs().max()) < 2e-2, (first, second)
         assert float((base[2] - got[2]).abs().max()) < 1e-3, (first, second)
+
+
+def test_head_size_256_at_16k_ring4_matches_oracle():
+    """B1 H2 S16384 D256 bf16 as a ring of four shards of 4096 with packed documents and a bias, chunks 512 / 512:
+    the size class the family's throughput is quoted on, against the CPU oracle's ring loop, forward and backward."""
+    import time
+    B, S, H, D, n = 1, 16384, 2, 256, 4
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=41, scale=D ** -0.25)
+    seg = packed_segment_ids(B, S, 3000, seed=42)
+    bias = torch.randn(1, 1, 1, S, generator=torch.Generator().manual_seed(43))
+    kw = kwargs(512, 512, 1)
+    t0 = time.time()
+    ref_out, ref_grads = oracle_fwd_bwd(q, k, v, do, bias, seg, None, n, kw)
+    print("oracle %.1f s" % (time.time() - t0), flush=True)
+    out, grads = run_hip(q, k, v, do, bias, seg, None, n, kw)
+    assert ra.kernel_family_of_last_call() == {"forward": "mfma_bf16_any", "backward": "mfma_bf16_any"}
+    assert_close_scaled(out, ref_out, torch.bfloat16, "out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads, ref_grads):
+        assert_close_scaled(a, b, torch.bfloat16, name)
+
+
+def test_families_agree_at_8k_on_the_tiled_kernels_shape():
+    """The same bf16 call (8192 positions, documents, a bias, head size 128) on the tiled matrix-core kernels and on
+    the element-wise ones: two independent implementations within the bf16 bar of each other."""
+    B, S, H, D = 1, 8192, 2, 128
+    q, k, v, do = make_qkv(B, S, H, D, dtype=torch.bfloat16, seed=44, scale=D ** -0.25)
+    seg = packed_segment_ids(B, S, 1500, seed=45)
+    bias = torch.randn(1, 1, 1, S, generator=torch.Generator().manual_seed(46))
+    a_out, a_grads = run_hip(q, k, v, do, bias, seg, None, 1, kwargs(512, 512, 1, impl="mfma"))
+    assert ra.kernel_family_of_last_call()["forward"] == "mfma_bf16"
+    b_out, b_grads = run_hip(q, k, v, do, bias, seg, None, 1, kwargs(512, 512, 1, impl="mfma_any"))
+    assert ra.kernel_family_of_last_call()["forward"] == "mfma_bf16_any"
+    assert_close_scaled(b_out, a_out.float().cpu(), torch.bfloat16, "out")
+    for name, x, y in zip(("dq", "dk", "dv"), b_grads, a_grads):
+        assert_close_scaled(x, y.float().cpu(), torch.bfloat16, name)
