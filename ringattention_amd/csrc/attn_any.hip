@@ -96,19 +96,18 @@ __device__ __forceinline__ any_bf16x8 any_row_frag(const uint16_t* tile, int row
 // operand "32 head dimensions of block db x those 16 rows": lane half hi takes rows 8 hi .. 8 hi + 7.
 template <int HD>
 struct AnyTr {
-  int off[HD / 32][2];
+  int a0, a1, x;                 // off[db][j] = aj + ((db ^ x) << 5): the swizzle flips the 32-dimension block by the row's low bits
   __device__ __forceinline__ void init(int lane) {
     const int hi = lane >> 5, i = lane & 15, rr = (i >> 2) + 8 * hi;
     const int c0 = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), half = lane & 1;
-#pragma unroll
-    for (int db = 0; db < HD / 32; db++) {
-      off[db][0] = rr * HD + (((4 * db + c0) ^ any_swz(rr)) << 3) + half * 4;
-      off[db][1] = (rr + 4) * HD + (((4 * db + c0) ^ any_swz(rr + 4)) << 3) + half * 4;
-    }
+    x = rr & 3;
+    a0 = rr * HD + ((c0 ^ ((rr >> 2) & 3)) << 3) + half * 4;
+    a1 = (rr + 4) * HD + ((c0 ^ (((rr + 4) >> 2) & 3)) << 3) + half * 4;
   }
   __device__ __forceinline__ any_bf16x8 frag(const uint16_t* rows16, int db) const {
-    const any_s16x4 x0 = any_read_tr(rows16 + off[db][0]);
-    const any_s16x4 x1 = any_read_tr(rows16 + off[db][1]);
+    const int o = (db ^ x) << 5;
+    const any_s16x4 x0 = any_read_tr(rows16 + a0 + o);
+    const any_s16x4 x1 = any_read_tr(rows16 + a1 + o);
     return __builtin_bit_cast(any_bf16x8, __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7));
   }
 };
@@ -131,7 +130,7 @@ __device__ __forceinline__ any_bf16x8 any_bop(const any_f32x16& c, int K) {
 template <int HD>
 __device__ __forceinline__ void any_products(const uint16_t* tile, const any_bf16x8 (&bq)[HD / 16], any_f32x16 (&C)[2],
                                              int lo, int hi) {
-  constexpr int G = 8, GPB = HD / 16 / G, NG = 2 * GPB;                 // groups per 32-row block, groups in all
+  constexpr int G = HD > 128 ? 4 : 8, GPB = HD / 16 / G, NG = 2 * GPB;  // groups per 32-row block, groups in all (fewer registers at 256)
   any_bf16x8 F[2][G];
 #pragma unroll
   for (int i = 0; i < G; i++) F[0][i] = any_row_frag<HD>(tile, lo, i, hi);
