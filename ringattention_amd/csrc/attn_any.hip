@@ -9,8 +9,9 @@
 // buffers, loaded straight from global memory a tile ahead (buffer_load ... lds), one barrier per tile.  Products are
 // formed transposed, S^T = K Q^T, so the C layout hands every lane its own row's logits; P^T (dS^T) goes back in as a
 // B operand from the same registers after one exchange with the partner lane, and the second operand of
-// O^T += V^T P^T comes from LDS transpose reads.  With one wavefront per SIMD nothing hides a wait, so the LDS reads
-// of a group of eight products are issued among the MFMAs of the group before.  A tile whose pairs all run and are
+// O^T += V^T P^T comes from LDS transpose reads.  At head size 256 the registers leave one wavefront per SIMD and
+// nothing hides a wait, so the LDS reads of a group of four products are issued among the MFMAs of the group before;
+// at head size 128 the kernels are bounded to 256 registers, so that two workgroups share a CU.  A tile whose pairs all run and are
 // not masked skips the element-wise evaluation.
 //
 // Semantics follow ringattention_jax.py:130-145 (forward tile), :220-233 (backward tile), :272-322 (bias / mask)
@@ -126,11 +127,11 @@ __device__ __forceinline__ any_bf16x8 any_bop(const any_f32x16& c, int K) {
 }
 
 // C[blk] += (rows 32 blk .. 32 blk + 31 of an LDS tile) x (the lane's resident operand), blk = 0, 1: the LDS reads of
-// a group of eight contraction steps are issued among the MFMAs of the group before.
+// a group of four contraction steps are issued among the MFMAs of the group before.
 template <int HD>
 __device__ __forceinline__ void any_products(const uint16_t* tile, const any_bf16x8 (&bq)[HD / 16], any_f32x16 (&C)[2],
                                              int lo, int hi) {
-  constexpr int G = HD > 128 ? 4 : 8, GPB = HD / 16 / G, NG = 2 * GPB;  // groups per 32-row block, groups in all (fewer registers at 256)
+  constexpr int G = 4, GPB = HD / 16 / G, NG = 2 * GPB;                 // groups per 32-row block, groups in all
   any_bf16x8 F[2][G];
 #pragma unroll
   for (int i = 0; i < G; i++) F[0][i] = any_row_frag<HD>(tile, lo, i, hi);
@@ -297,7 +298,7 @@ __device__ __forceinline__ float any_logit_row(const MaskView& mv, const RowInfo
 
 // ------------------------------------------------------------------ forward
 template <int HD>
-__global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a) {
+__global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_fwd_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][ANY_TILE * HD];
   __shared__ __attribute__((aligned(16))) uint16_t Vs[2][ANY_TILE * HD];
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_fwd_any_kernel(GenericArgs a
 
 // ------------------------------------------------------------------ backward, dq (a lane owns a query row)
 template <int HD>
-__global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArgs a) {
+__global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dq_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][ANY_TILE * HD];
   __shared__ __attribute__((aligned(16))) uint16_t Vs[2][ANY_TILE * HD];
@@ -606,7 +607,7 @@ __global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dq_any_kernel(GenericArg
 
 // ------------------------------------------------------------------ backward, dk or dv (a lane owns a key row)
 template <int HD, bool WANT_DK>
-__global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_any_kernel(GenericArgs a) {
+__global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dkv_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
   __shared__ __attribute__((aligned(16))) uint16_t Qs[2][ANY_TILE * HD];
   __shared__ __attribute__((aligned(16))) uint16_t Gs[2][ANY_TILE * HD];
