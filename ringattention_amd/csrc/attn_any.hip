@@ -155,6 +155,32 @@ __device__ __forceinline__ void any_products(const uint16_t* tile, const any_bf1
   }
 }
 
+// One 32-row block of any_products: C += (rows row0 .. row0 + 31 of an LDS tile) x (the lane's resident operand).
+template <int HD>
+__device__ __forceinline__ void any_products_block(const uint16_t* tile, int row0, const any_bf16x8 (&bq)[HD / 16],
+                                                   any_f32x16& C, int lo, int hi) {
+  constexpr int G = 4, NG = HD / 16 / G;
+  any_bf16x8 F[2][G];
+#pragma unroll
+  for (int i = 0; i < G; i++) F[0][i] = any_row_frag<HD>(tile, row0 + lo, i, hi);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int g = 0; g < NG; g++) {
+    if (g + 1 < NG) {
+#pragma unroll
+      for (int i = 0; i < G; i++) F[(g + 1) & 1][i] = any_row_frag<HD>(tile, row0 + lo, (g + 1) * G + i, hi);
+    }
+#pragma unroll
+    for (int i = 0; i < G; i++) C = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[g & 1][i], bq[g * G + i], C, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (g + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 // acc^T (head dimensions x the lanes' rows) += tile^T P^T for the 64 tile rows, P in the C layout of any_products:
 // four steps of 16 tile rows, the transpose reads of a step issued among the MFMAs of the step before.
 template <int HD>
@@ -606,6 +632,7 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dq_any
 }
 
 // ------------------------------------------------------------------ backward, dk or dv (a lane owns a key row)
+// Head size 128: one launch for each of the two (S is formed twice); head size 256 takes the kernel after this one.
 template <int HD, bool WANT_DK>
 __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dkv_any_kernel(GenericArgs a) {
   constexpr int NKS = HD / 16, NDB = HD / 32;
@@ -755,6 +782,210 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dkv_an
   }
 }
 
+// ------------------------------------------------------------------ backward, dk and dv at head size 256
+// Both accumulators of a 256-wide head do not fit one wavefront next to its operands, so two wavefronts share 32 keys:
+// each forms S and dP for one half of a query tile's rows (all 256 head dimensions), leaves P and dS, rounded to
+// bf16, in LDS as [key][query], and after a barrier accumulates one half of the head dimensions of dK^T and dV^T over
+// all 64 rows.  Every product is formed once (8 D per pair).  A workgroup of four wavefronts serves 64 keys.
+constexpr int ANY_PSTR = ANY_TILE + 8;                 // row of the P / dS exchange buffers: 64 queries and padding
+template <int HD>
+__global__ __launch_bounds__(ANY_THREADS) void attn_bwd_dkv_pair_any_kernel(GenericArgs a) {
+  constexpr int NKS = HD / 16, NDB = HD / 64;          // head-dimension blocks of 32 per wavefront: half of the head
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Gs[2][ANY_TILE * HD];
+  __shared__ __attribute__((aligned(16))) uint16_t Pt[2][32 * ANY_PSTR];      // [key group][key][query]
+  __shared__ __attribute__((aligned(16))) uint16_t Dt[2][32 * ANY_PSTR];
+  __shared__ __attribute__((aligned(16))) AnyRowTables rts[2];
+  const MaskView mv = resolve_mask(a);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, lo = lane & 31, hi = lane >> 5;
+  const int kg = wave >> 1, half = wave & 1;           // key group; half of the tile's rows, and of the head dimensions
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int first_key = blockIdx.x * 64;
+  const int kj = first_key + kg * 32 + lo;
+  const bool valid = kj < a.Skv;
+  const int rk = valid ? kj : a.Skv - 1;
+  const int64_t koff = (int64_t)b * a.kv_sb + (int64_t)rk * a.kv_ss + (int64_t)h * HD;
+  const uint16_t* kp = (const uint16_t*)a.k + koff;
+  const uint16_t* vp = (const uint16_t*)a.v + koff;
+  const uint16_t* qbase = (const uint16_t*)a.q + (int64_t)b * a.q_sb + (int64_t)h * HD;
+  const uint16_t* gbase = (const uint16_t*)a.g + (int64_t)b * a.q_sb + (int64_t)h * HD;
+  const float scale = sqrtf((float)a.sdim), rscale = 1.f / scale;
+
+  any_bf16x8 kf[NKS], vf[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ks++) {
+    kf[ks] = *(const any_bf16x8*)(kp + ks * 16 + hi * 8);
+    vf[ks] = *(const any_bf16x8*)(vp + ks * 16 + hi * 8);
+  }
+  any_f32x16 acc_k[NDB], acc_v[NDB];                   // dK^T, dV^T: head dimensions 128 half + 32 db + ...
+#pragma unroll
+  for (int db = 0; db < NDB; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { acc_k[db][r] = 0.f; acc_v[db][r] = 0.f; }
+  const int seg_k = any_key_seg(mv, b, rk);
+  const long long gk = mv.global_k(rk);
+  const long long kblk = any_key_block(mv, rk);
+  const int key_hi_w = first_key + kg * 32 + 32;
+  const long long kblk_max_w = any_key_block(mv, min(key_hi_w, a.Skv) - 1);
+  const bool bias_per_key = mv.bias && mv.bias_sq == 0, bias_per_row = mv.bias && mv.bias_sq != 0;
+  const bool elementwise_always = mv.keep || bias_per_row;
+  const int kseg_min_w = any_wave_min(seg_k), kseg_max_w = any_wave_max(seg_k);
+  float bias_k = 0.f;
+  if (bias_per_key) {
+    bias_k = mv.bias[(int64_t)b * mv.bias_sb + (int64_t)h * mv.bias_sh + gk * mv.bias_sk];
+    if (mv.any_mask) bias_k = fminf(bias_k, 0.f);
+  }
+  const bool wave_valid = first_key + kg * 32 < a.Skv;
+  const bool all_valid = key_hi_w <= a.Skv;
+
+  AnyTr<HD> tr;
+  tr.init(lane);
+  int t_first = 0;
+  const int ntile = (a.Sq + ANY_TILE - 1) / ANY_TILE;
+  while (t_first < ntile &&
+         mv.run_prefix_keys((min((t_first + 1) * ANY_TILE, a.Sq) - 1) / mv.qc, a.Skv) <= first_key) t_first++;
+  AnyTileLoader<HD> ld;
+  ld.init(a.q_ss, wave, lane);
+  if (t_first < ntile) {
+    const int q0 = t_first * ANY_TILE;
+    ld.load(Qs[t_first & 1], qbase + (int64_t)q0 * a.q_ss, a.Sq - q0);
+    ld.load(Gs[t_first & 1], gbase + (int64_t)q0 * a.q_ss, a.Sq - q0);
+    any_stage_rows(rts[t_first & 1], a, mv, b, h, q0, tid);
+  }
+  uint16_t* const pw = Pt[kg] + lo * ANY_PSTR + half * 32 + hi * 4;    // this lane's key, its half of the rows
+  uint16_t* const dw = Dt[kg] + lo * ANY_PSTR + half * 32 + hi * 4;
+  const uint16_t* const pr = Pt[kg] + lo * ANY_PSTR + hi * 8;          // B operands: key lo, eight queries per step
+  const uint16_t* const dr = Dt[kg] + lo * ANY_PSTR + hi * 8;
+#pragma unroll 1
+  for (int t = t_first; t < ntile; t++) {
+    const int q0 = t * ANY_TILE;
+    any_tile_barrier();                                // tile t is in LDS; the other buffers have been read by everyone
+    if (t + 1 < ntile) {
+      const int q1 = q0 + ANY_TILE;
+      ld.load(Qs[(t + 1) & 1], qbase + (int64_t)q1 * a.q_ss, a.Sq - q1);
+      ld.load(Gs[(t + 1) & 1], gbase + (int64_t)q1 * a.q_ss, a.Sq - q1);
+      any_stage_rows(rts[(t + 1) & 1], a, mv, b, h, q1, tid);
+    }
+    const uint16_t* Qt = Qs[t & 1];
+    const uint16_t* Gt = Gs[t & 1];
+    const AnyRowTables& rt = rts[t & 1];
+    // the two wavefronts of a key group decide alike: no key of the group exists, or no row of the tile shares a
+    // segment id with one of them (see the forward kernel)
+    const bool active = wave_valid && !(mv.seg && mv.skip_tiles && (rt.segmax < kseg_min_w || rt.segmin > kseg_max_w));
+    if (active) {
+      any_f32x16 S, dP;                                // rows 32 half .. + 31 of the tile x this lane's key
+#pragma unroll
+      for (int r = 0; r < 16; r++) { S[r] = 0.f; dP[r] = 0.f; }
+      any_products_block<HD>(Qt, half * 32, kf, S, lo, hi);
+      any_products_block<HD>(Gt, half * 32, vf, dP, lo, hi);
+      const bool plain = !elementwise_always && all_valid && key_hi_w <= rt.kend_min &&
+                         (mv.cbs <= 0 || rt.blk0 >= kblk_max_w) &&
+                         (!mv.seg || (rt.segmin == rt.segmax && kseg_min_w == kseg_max_w && rt.segmin == kseg_min_w));
+      if (plain) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          const int q4 = half * 32 + g * 8 + hi * 4;
+          const any_f32x4 m4 = *(const any_f32x4*)&rt.m[q4], d4 = *(const any_f32x4*)&rt.rden[q4];
+          const any_f32x4 e4 = *(const any_f32x4*)&rt.delta[q4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p = __expf(fmaf(S[g * 4 + e], rscale, bias_k) - m4[e]) * d4[e];                // :226
+            S[g * 4 + e] = p;
+            dP[g * 4 + e] = (dP[g * 4 + e] - e4[e]) * p;                                                 // :229
+          }
+        }
+      } else {
+        const int dkey = any_rel(kblk - rt.blk0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int qq = half * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
+          float add = bias_k;
+          bool masked = (mv.cbs > 0 && rt.blk[qq] < dkey) || (mv.seg && rt.seg[qq] != seg_k);
+          if (bias_per_row) {
+            add = mv.bias[rt.bias_off[qq] + gk * mv.bias_sk];
+            if (mv.any_mask) add = fminf(add, 0.f);                     // minimum(), :299,:309
+          }
+          if (mv.keep) masked = masked || !mv.keep[rt.keep_off[qq] + (gk - mv.keep_k0) * mv.keep_sk];
+          const float s = masked ? mv.mask_min : fmaf(S[r], rscale, add);
+          const float p = (valid && kj < rt.kend[qq]) ? __expf(s - rt.m[qq]) * rt.rden[qq] : 0.f;     // :226; (:246-257)
+          S[r] = p;
+          dP[r] = (dP[r] - rt.delta[qq]) * p;                           // :229
+          if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < 4; g++) {                    // queries 32 half + 8 g + 4 hi + e of this lane's key
+        const uint2 p2 = {f32x2_to_bf16x2(S[g * 4], S[g * 4 + 1]), f32x2_to_bf16x2(S[g * 4 + 2], S[g * 4 + 3])};
+        const uint2 d2 = {f32x2_to_bf16x2(dP[g * 4], dP[g * 4 + 1]), f32x2_to_bf16x2(dP[g * 4 + 2], dP[g * 4 + 3])};
+        *(uint2*)(pw + g * 8) = p2;
+        *(uint2*)(dw + g * 8) = d2;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // P and dS of all 64 rows are in LDS
+    if (active) {
+      // four steps of 16 rows: dV^T += dO^T P (:232) and dK^T += Q^T dS (:231) over this wavefront's half of the head
+      any_bf16x8 FG[2][NDB], FQ[2][NDB];
+#pragma unroll
+      for (int db = 0; db < NDB; db++) {
+        FG[0][db] = tr.frag(Gt, half * NDB + db);
+        FQ[0][db] = tr.frag(Qt, half * NDB + db);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int st = 0; st < 4; st++) {
+        if (st + 1 < 4) {
+#pragma unroll
+          for (int db = 0; db < NDB; db++) {
+            FG[(st + 1) & 1][db] = tr.frag(Gt + (st + 1) * 16 * HD, half * NDB + db);
+            FQ[(st + 1) & 1][db] = tr.frag(Qt + (st + 1) * 16 * HD, half * NDB + db);
+          }
+        }
+        const any_bf16x8 bp = *(const any_bf16x8*)(pr + st * 16);
+        const any_bf16x8 bd = *(const any_bf16x8*)(dr + st * 16);
+#pragma unroll
+        for (int db = 0; db < NDB; db++) {
+          acc_v[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FG[st & 1][db], bp, acc_v[db], 0, 0, 0);
+          acc_k[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(FQ[st & 1][db], bd, acc_k[db], 0, 0, 0);
+        }
+#pragma unroll
+        for (int db = 0; db < 2 * NDB; db++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (st + 1 < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  if (valid) {
+    const int64_t off = (int64_t)h * HD + half * (HD / 2) + hi * 4;
+    float* dkp = a.dk + (int64_t)b * a.dkv_sb + (int64_t)rk * a.dkv_ss + off;
+    float* dvp = a.dv + (int64_t)b * a.dkv_sb + (int64_t)rk * a.dkv_ss + off;
+    uint16_t* okp = (uint16_t*)a.dk_out + (int64_t)b * a.dkvo_sb + (int64_t)rk * a.dkvo_ss + off;
+    uint16_t* ovp = (uint16_t*)a.dv_out + (int64_t)b * a.dkvo_sb + (int64_t)rk * a.dkvo_ss + off;
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        any_f32x4 k4 = {0.f, 0.f, 0.f, 0.f}, v4 = {0.f, 0.f, 0.f, 0.f};
+        if (!a.dkv_initial) {
+          k4 = *(const any_f32x4*)(dkp + db * 32 + g * 8);
+          v4 = *(const any_f32x4*)(dvp + db * 32 + g * 8);
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) { k4[e] += acc_k[db][g * 4 + e] / scale; v4[e] += acc_v[db][g * 4 + e]; }
+        if (a.dk_out) {                                                 // last call for these keys (:89)
+          const uint2 pk = {f32x2_to_bf16x2(k4[0], k4[1]), f32x2_to_bf16x2(k4[2], k4[3])};
+          const uint2 pv = {f32x2_to_bf16x2(v4[0], v4[1]), f32x2_to_bf16x2(v4[2], v4[3])};
+          *(uint2*)(okp + db * 32 + g * 8) = pk;
+          *(uint2*)(ovp + db * 32 + g * 8) = pv;
+        } else {
+          *(any_f32x4*)(dkp + db * 32 + g * 8) = k4;
+          *(any_f32x4*)(dvp + db * 32 + g * 8) = v4;
+        }
+      }
+  }
+}
+
 // every kernel is instantiated by name: left to the launches below (some of them inside a function template) the host
 // pass of the compiler has been seen to reference a kernel's launch stub without emitting it
 template __global__ void attn_fwd_any_kernel<128>(GenericArgs);
@@ -765,6 +996,7 @@ template __global__ void attn_bwd_dkv_any_kernel<128, true>(GenericArgs);
 template __global__ void attn_bwd_dkv_any_kernel<128, false>(GenericArgs);
 template __global__ void attn_bwd_dkv_any_kernel<256, true>(GenericArgs);
 template __global__ void attn_bwd_dkv_any_kernel<256, false>(GenericArgs);
+template __global__ void attn_bwd_dkv_pair_any_kernel<256>(GenericArgs);
 
 // ------------------------------------------------------------------ host side
 static bool any_aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
@@ -810,8 +1042,13 @@ static void launch_bwd_any(const GenericArgs& a, int parts, hipStream_t s) {
   const dim3 gq((a.Sq + ANY_ROWS - 1) / ANY_ROWS, a.H, a.B), gk((a.Skv + ANY_ROWS - 1) / ANY_ROWS, a.H, a.B);
   if (parts & RA_BWD_PART_DQ) attn_bwd_dq_any_kernel<HD><<<gq, block, 0, s>>>(a);
   if (parts & RA_BWD_PART_DKV) {
-    attn_bwd_dkv_any_kernel<HD, true><<<gk, block, 0, s>>>(a);
-    attn_bwd_dkv_any_kernel<HD, false><<<gk, block, 0, s>>>(a);
+    if (HD == 256) {                                   // both gradients in one pass, a pair of wavefronts per 32 keys
+      const dim3 gk2((a.Skv + 63) / 64, a.H, a.B);
+      attn_bwd_dkv_pair_any_kernel<256><<<gk2, block, 0, s>>>(a);
+    } else {
+      attn_bwd_dkv_any_kernel<HD, true><<<gk, block, 0, s>>>(a);
+      attn_bwd_dkv_any_kernel<HD, false><<<gk, block, 0, s>>>(a);
+    }
   }
 }
 
