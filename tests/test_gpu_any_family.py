@@ -173,3 +173,32 @@ def test_families_agree_at_8k_on_the_tiled_kernels_shape():
     assert_close_scaled(b_out, a_out.float().cpu(), torch.bfloat16, "out")
     for name, x, y in zip(("dq", "dk", "dv"), b_grads, a_grads):
         assert_close_scaled(x, y.float().cpu(), torch.bfloat16, name)
+
+
+@pytest.mark.parametrize("D", [128, 256])
+def test_elementwise_kernels_repeat_their_bits_and_isolate_masked_keys(D):
+    """Two runs of one call give the same bits (every output element has one owner, no atomics); keys behind a row under
+    the causal mask, or in another document, have bitwise no effect on it, and get exactly zero gradient from rows whose
+    cotangent is zero."""
+    B, S, H = 1, 640, 2
+    q, k, v, do = _qkv(B, S, H, D, 12)
+    seg = torch.cat((torch.zeros(1, 400, dtype=torch.int32), torch.ones(1, 240, dtype=torch.int32)), dim=1)
+    kw = kwargs(40, 40, 1, impl="mfma_any")
+    a, ga = run_hip(q, k, v, do, None, seg, None, 1, kw)
+    b, gb = run_hip(q, k, v, do, None, seg, None, 1, kw)
+    assert torch.equal(a, b) and all(torch.equal(x, y) for x, y in zip(ga, gb))
+    k2, v2 = k.clone(), v.clone()
+    k2[:, 400:] += 50.0                                  # the second document's keys: invisible to rows < 400
+    v2[:, 400:] -= 20.0
+    c, _ = run_hip(q, k2, v2, do, None, seg, None, 1, kw)
+    assert torch.equal(a[:, :400], c[:, :400])
+    k3, v3 = k.clone(), v.clone()
+    k3[:, 300:400] += 50.0                               # keys behind row 299 under the causal mask
+    v3[:, 300:400] -= 20.0
+    d, _ = run_hip(q, k3, v3, do, None, seg, None, 1, kw)
+    assert torch.equal(a[:, :300], d[:, :300])
+    do2 = do.clone()
+    do2[:, 400:] = 0.0                                   # no cotangent on the second document's rows
+    _, g2 = run_hip(q, k, v, do2, None, seg, None, 1, kw)
+    assert float(g2[1][:, 400:].abs().max()) == 0.0 and float(g2[2][:, 400:].abs().max()) == 0.0
+    assert float(g2[0][:, 400:].abs().max()) == 0.0
