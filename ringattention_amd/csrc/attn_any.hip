@@ -397,26 +397,34 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_fwd_any_ke
   for (int t = 0; t < ntile; t++) {
     const int k0 = t * ANY_TILE;
     any_tile_barrier();                                // tile t is in LDS; the other buffer has been read by everyone
-    if (t + 1 < ntile) {                               // the next tile travels while this one is worked on
+    const uint16_t* Kt = Ks[t & 1];
+    const uint16_t* Vt = Vs[t & 1];
+    const AnyKeyTables& kt = kts[t & 1];
+    // no row of this wavefront runs against these keys; or no key of the tile shares a segment id with a row of the
+    // wavefront: every pair is masked, and where the caller vouches that every row has a key of its own
+    // (skip_masked_tiles) such a tile weighs exactly nothing
+    const bool active = k0 < kend_max_w &&
+                        !(mv.seg && mv.skip_tiles && (kt.segmax < rseg_min_w || kt.segmin > rseg_max_w));
+    any_f32x16 S[2];                                   // S^T, two blocks of 32 keys: register 4 g + e = key 8 g + 4 hi + e
+    if (active) {
+#pragma unroll
+      for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) S[blk][r] = 0.f;
+      any_products<HD>(Kt, qf, S, lo, hi);             // :134
+    }
+    // The next tile travels while this one is worked on.  Here its loads go out behind the first batch of products:
+    // they share a counter with every other memory access of the wavefront, and the registers that the compiler keeps
+    // in scratch memory at head size 256 are reloaded for those products - behind the loads they would wait for them
+    // too (measured: 10-25 % of the forward kernel; the backward kernels measured better with the loads first).
+    if (t + 1 < ntile) {
       const int k1 = k0 + ANY_TILE;
       ld.load(Ks[(t + 1) & 1], kbase + (int64_t)k1 * a.kv_ss, a.Skv - k1);
       ld.load(Vs[(t + 1) & 1], vbase + (int64_t)k1 * a.kv_ss, a.Skv - k1);
       if (key_tables) any_stage_keys(kts[(t + 1) & 1], mv, b, h, k1, a.Skv, bias_per_key, tid);
     }
-    if (k0 >= kend_max_w) continue;                    // no row of this wavefront runs against these keys
-    const uint16_t* Kt = Ks[t & 1];
-    const uint16_t* Vt = Vs[t & 1];
-    const AnyKeyTables& kt = kts[t & 1];
-    // no key of the tile shares a segment id with a row of the wavefront: every pair is masked, and where the caller
-    // vouches that every row has a key of its own (skip_masked_tiles) such a tile weighs exactly nothing
-    if (mv.seg && mv.skip_tiles && (kt.segmax < rseg_min_w || kt.segmin > rseg_max_w)) continue;
+    if (!active) continue;
 
-    any_f32x16 S[2];                                   // S^T, two blocks of 32 keys: register 4 g + e = key 8 g + 4 hi + e
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) S[blk][r] = 0.f;
-    any_products<HD>(Kt, qf, S, lo, hi);               // :134
     // every pair of the tile runs and is unmasked for every row of the wavefront: logit = dot / scale + bias
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
                        (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1)) &&
