@@ -1015,8 +1015,12 @@ static bool any_mask_ok(const ra_mask& m) {
   return m.keep_mode != RA_KEEP_DROPOUT && !(m.keep_bits_k && !m.keep);
 }
 
+// (the tile loader keeps a lane's byte offset within a tile of 64 rows in 32 bits)
+static bool any_strides_ok(int64_t q_ss, int64_t kv_ss) { return q_ss > 0 && kv_ss > 0 && q_ss < (1 << 24) && kv_ss < (1 << 24); }
+
 bool attn_fwd_any_supported(const ra_attn_fwd_params* p) {
   return p->dtype == RA_BF16 && (p->D == 128 || p->D == 256) && any_mask_ok(p->mask) &&
+         any_strides_ok(p->q_stride_s, p->kv_stride_s) &&
          p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 && p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 &&
          any_aligned16(p->q) && any_aligned16(p->k) && any_aligned16(p->v) &&
          (!p->numerator || (any_aligned16(p->numerator) && p->num_stride_s % 4 == 0 && p->num_stride_b % 4 == 0)) &&
@@ -1026,6 +1030,7 @@ bool attn_fwd_any_supported(const ra_attn_fwd_params* p) {
 
 bool attn_bwd_any_supported(const ra_attn_bwd_params* p) {
   return p->dtype == RA_BF16 && (p->D == 128 || p->D == 256) && any_mask_ok(p->mask) &&
+         any_strides_ok(p->q_stride_s, p->kv_stride_s) &&
          p->q_stride_s % 8 == 0 && p->kv_stride_s % 8 == 0 && p->q_stride_b % 8 == 0 && p->kv_stride_b % 8 == 0 &&
          any_aligned16(p->q) && any_aligned16(p->k) && any_aligned16(p->v) && any_aligned16(p->g) &&
          (!p->dq || (any_aligned16(p->dq) && p->dq_stride_s % 4 == 0 && p->dq_stride_b % 4 == 0)) &&
