@@ -210,6 +210,33 @@ __device__ __forceinline__ void any_accumulate(const uint16_t* tile, const AnyTr
   }
 }
 
+// any_accumulate with the four B operands (16 tile rows each) already built
+template <int HD>
+__device__ __forceinline__ void any_accumulate_bops(const uint16_t* tile, const AnyTr<HD>& tr, const any_bf16x8 (&bops)[4],
+                                                    any_f32x16 (&acc)[HD / 32]) {
+  constexpr int NDB = HD / 32;
+  any_bf16x8 F[2][NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; db++) F[0][db] = tr.frag(tile, db);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int s = 0; s < 4; s++) {
+    if (s + 1 < 4) {
+#pragma unroll
+      for (int db = 0; db < NDB; db++) F[(s + 1) & 1][db] = tr.frag(tile + (s + 1) * 16 * HD, db);
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; db++)
+      acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F[s & 1][db], bops[s], acc[db], 0, 0, 0);
+#pragma unroll
+    for (int db = 0; db < NDB; db++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (s + 1 < 4) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 __device__ __forceinline__ int any_wave_max(int v) {
   for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off));
   return v;
@@ -580,42 +607,45 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dq_any
     const AnyKeyTables& kt = kts[t & 1];
     if (mv.seg && mv.skip_tiles && (kt.segmax < rseg_min_w || kt.segmin > rseg_max_w)) continue;   // as in the forward kernel
 
-    any_f32x16 S[2], dP[2];
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; dP[blk][r] = 0.f; }
-    any_products<HD>(Kt, qf, S, lo, hi);               // :223-225
-    any_products<HD>(Vt, gf, dP, lo, hi);              // :228
     const bool plain = !elementwise_always && k0 + ANY_TILE <= kend_min_w &&
                        (mv.cbs <= 0 || gqblk_min_w >= any_key_block(mv, k0 + ANY_TILE - 1)) &&
                        (!mv.seg || (kt.segmin == kt.segmax && rseg_min_w == rseg_max_w && kt.segmin == rseg_min_w));
-    if (plain) {
+    const int drow = any_rel(ri.gq_blk - any_key_block(mv, min(k0, a.Skv - 1)));
+    // one block of 32 keys at a time: S^T and dP^T of a block are turned into dS^T and packed before the next block's
+    // products start, which keeps 32 registers fewer alive than both blocks at once
+    any_bf16x8 bops[4];
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+    for (int blk = 0; blk < 2; blk++) {
+      any_f32x16 S, dP;
+#pragma unroll
+      for (int r = 0; r < 16; r++) { S[r] = 0.f; dP[r] = 0.f; }
+      any_products_block<HD>(Kt, blk * 32, qf, S, lo, hi);             // :223-225
+      any_products_block<HD>(Vt, blk * 32, gf, dP, lo, hi);            // :228
+      if (plain) {
 #pragma unroll
         for (int g = 0; g < 4; g++) {
           const any_f32x4 b4 = *(const any_f32x4*)&kt.bias[blk * 32 + g * 8 + hi * 4];
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            const float p = __expf(fmaf(S[blk][g * 4 + e], rscale, b4[e]) - m) * rden;      // :226
-            S[blk][g * 4 + e] = (dP[blk][g * 4 + e] - delta) * p;                             // dS^T, :229
+            const float p = __expf(fmaf(S[g * 4 + e], rscale, b4[e]) - m) * rden;           // :226
+            S[g * 4 + e] = (dP[g * 4 + e] - delta) * p;                                       // dS^T, :229
           }
         }
-    } else {
-      const int drow = any_rel(ri.gq_blk - any_key_block(mv, min(k0, a.Skv - 1)));
-#pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+      } else {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int kk = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
-          const float s = any_logit_row(mv, ri, kt, S[blk][r], rscale, k0, kk, a.Skv, drow, bias_per_row);
+          const float s = any_logit_row(mv, ri, kt, S[r], rscale, k0, kk, a.Skv, drow, bias_per_row);
           const float p = __expf(s - m) * rden;                         // :226
           // a pair whose tile does not run contributes nothing (:246-257)
-          S[blk][r] = (k0 + kk < ri.kend) ? (dP[blk][r] - delta) * p : 0.f;   // dS^T, :229
+          S[r] = (k0 + kk < ri.kend) ? (dP[r] - delta) * p : 0.f;       // dS^T, :229
+          if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
         }
+      }
+      bops[2 * blk] = any_bop(S, 0);
+      bops[2 * blk + 1] = any_bop(S, 1);
     }
-    any_accumulate<HD>(Kt, tr, S, acc);                // :230
+    any_accumulate_bops<HD>(Kt, tr, bops, acc);        // :230
   }
   if (valid) {
     const int64_t off = (int64_t)h * HD + hi * 4;
