@@ -752,20 +752,22 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dkv_an
     // no row of the tile shares a segment id with a key of the wavefront (see the forward kernel)
     if (mv.seg && mv.skip_tiles && (rt.segmax < kseg_min_w || rt.segmin > kseg_max_w)) continue;
 
-    any_f32x16 S[2], dP[2];                            // S, dP: the lane's key column; register 4 g + e = query 8 g + 4 hi + e
-#pragma unroll
-    for (int blk = 0; blk < 2; blk++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) { S[blk][r] = 0.f; dP[blk][r] = 0.f; }
-    any_products<HD>(Qt, kf, S, lo, hi);
-    if (WANT_DK) any_products<HD>(Gt, vf, dP, lo, hi);
     // every pair of (tile rows, the wavefront's keys) runs and is unmasked
     const bool plain = !elementwise_always && all_valid && key_hi_w <= rt.kend_min &&
                        (mv.cbs <= 0 || rt.blk0 >= kblk_max_w) &&
                        (!mv.seg || (rt.segmin == rt.segmax && kseg_min_w == kseg_max_w && rt.segmin == kseg_min_w));
-    if (plain) {
+    const int dkey = any_rel(kblk - rt.blk0);          // this key's causal block relative to the tile's first row's
+    // one block of 32 query rows at a time (S, dP: the lane's key column; register 4 g + e = query 8 g + 4 hi + e), turned
+    // into P or dS and packed before the next block's products start
+    any_bf16x8 bops[4];
 #pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+    for (int blk = 0; blk < 2; blk++) {
+      any_f32x16 S, dP;
+#pragma unroll
+      for (int r = 0; r < 16; r++) { S[r] = 0.f; dP[r] = 0.f; }
+      any_products_block<HD>(Qt, blk * 32, kf, S, lo, hi);
+      if (WANT_DK) any_products_block<HD>(Gt, blk * 32, vf, dP, lo, hi);
+      if (plain) {
 #pragma unroll
         for (int g = 0; g < 4; g++) {
           const int q4 = blk * 32 + g * 8 + hi * 4;
@@ -773,14 +775,11 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dkv_an
           const any_f32x4 e4 = *(const any_f32x4*)&rt.delta[q4];
 #pragma unroll
           for (int e = 0; e < 4; e++) {
-            const float p = __expf(fmaf(S[blk][g * 4 + e], rscale, bias_k) - m4[e]) * d4[e];          // :226
-            S[blk][g * 4 + e] = WANT_DK ? (dP[blk][g * 4 + e] - e4[e]) * p : p;                        // dS (:229) or P
+            const float p = __expf(fmaf(S[g * 4 + e], rscale, bias_k) - m4[e]) * d4[e];               // :226
+            S[g * 4 + e] = WANT_DK ? (dP[g * 4 + e] - e4[e]) * p : p;                                   // dS (:229) or P
           }
         }
-    } else {
-      const int dkey = any_rel(kblk - rt.blk0);        // this key's causal block relative to the tile's first row's
-#pragma unroll
-      for (int blk = 0; blk < 2; blk++)
+      } else {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const int qq = blk * 32 + (r >> 2) * 8 + hi * 4 + (r & 3);
@@ -791,12 +790,16 @@ __global__ __launch_bounds__(ANY_THREADS, HD > 128 ? 1 : 2) void attn_bwd_dkv_an
             if (mv.any_mask) add = fminf(add, 0.f);                     // minimum(), :299,:309
           }
           if (mv.keep) masked = masked || !mv.keep[rt.keep_off[qq] + (gk - mv.keep_k0) * mv.keep_sk];
-          const float s = masked ? mv.mask_min : fmaf(S[blk][r], rscale, add);
+          const float s = masked ? mv.mask_min : fmaf(S[r], rscale, add);
           const float p = (valid && kj < rt.kend[qq]) ? __expf(s - rt.m[qq]) * rt.rden[qq] : 0.f;     // :226; (:246-257)
-          S[blk][r] = WANT_DK ? (dP[blk][r] - rt.delta[qq]) * p : p;    // dS (:229) or P
+          S[r] = WANT_DK ? (dP[r] - rt.delta[qq]) * p : p;              // dS (:229) or P
+          if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
         }
+      }
+      bops[2 * blk] = any_bop(S, 0);
+      bops[2 * blk + 1] = any_bop(S, 1);
     }
-    any_accumulate<HD>(WANT_DK ? Qt : Gt, tr, S, acc);           // :231 / :232
+    any_accumulate_bops<HD>(WANT_DK ? Qt : Gt, tr, bops, acc);   // :231 / :232
   }
   if (valid) {
     const int64_t off = (int64_t)h * HD + hi * 4;
