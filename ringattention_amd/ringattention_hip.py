@@ -815,10 +815,11 @@ def _ring_attention_fwd(q, k, v, attn_bias, segment_ids, cache_idx, axis_name, f
 
 def _padded_head_size(cfg, mi, q):
     """The head size to zero-pad q, k, v to (the products are those of the un-padded rows; the logits keep the scale
-    of the original head size), or 0 when the kernels take the head size as it is.  The matrix-core kernels tile 64
-    and 128, the generic ones 32, 64, 128 and 256: a call that stays on the generic kernels anyway (they were asked
-    for, chunk sizes off the 128-grid, a per-row bias, an unpacked boolean mask, a head size above 128) is padded to
-    the next of those, any other to 64 or 128."""
+    of the original head size), or 0 when the kernels take the head size as it is.  The tiled matrix-core kernels take
+    64 and 128; a bf16 call that leaves their grid (chunk sizes off the 128-grid, a per-row bias, an unpacked boolean
+    mask, a head size above 128) goes to the matrix-core kernels that evaluate the mask element by element, which
+    take 128 and 256; what is left - fp32 inputs off the grid, attention dropout there, the generic kernels asked for
+    by name - runs on the generic kernels, which take 32, 64, 128 and 256."""
     D = q.shape[3]
     if D > 256:
         raise NotImplementedError("head size %d: the kernels take head sizes up to 256" % D)
